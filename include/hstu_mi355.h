@@ -1,0 +1,134 @@
+/*
+ * hstu_mi355.h -- C ABI of the MI355X (gfx950) HSTU jagged attention forward library.
+ *
+ * This is the native boundary underneath the torch adapter.  It replaces the two-phase
+ * C API the reference's adapter binds for this path:
+ *
+ *   aclnnHstuJaggedForwardGetWorkspaceSize(q, k, v, mask, attnBias, seqOffsetQ, seqOffsetK,
+ *        numContext, numTarget, maskType, maxSeqLenQ, maxSeqLenK, siluScale, targetGroupSize,
+ *        alpha, deterministic, attnOutput, &workspaceSize, &executor)
+ *   aclnnHstuJaggedForward(workspace, workspaceSize, executor, stream)
+ *
+ *   documented at  ascendc/attention/hstu_v1/hstu_forward_v1/docs/aclnn_hstu_forward.md:50-62
+ *   called from    ascendc/attention/hstu_v1/torch_extension/hstu_jagged_plugin.cpp:63-65
+ *   C usage        ascendc/attention/hstu_v1/hstu_forward_v1/examples/aclnn/test_aclnn_hstu_forward_jagged.cpp:97-110
+ *
+ * Conventions kept from that API: C linkage, status-int returns (0 = success), caller owns
+ * every buffer including the workspace, optional inputs are NULL, the launch is enqueued on the
+ * caller's stream and returns before completion.  Differences: tensors are described by one
+ * plain struct of device pointers and sizes instead of opaque handles, and there is no executor
+ * object (the library keeps no per-call state).
+ *
+ * The library never allocates or frees device memory and never synchronises the device.
+ */
+#ifndef HSTU_MI355_H
+#define HSTU_MI355_H
+
+#include <stdint.h>
+
+#if defined(__GNUC__)
+#define HSTU_API __attribute__((visibility("default")))
+#else
+#define HSTU_API
+#endif
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* status codes; the two 1610xx values are the ones the reference documents
+ * (aclnn_hstu_forward.md:109-114: 161001 null pointer, 161002 invalid parameter) */
+#define HSTU_OK 0
+#define HSTU_ERR_NULLPTR 161001
+#define HSTU_ERR_INVALID 161002
+#define HSTU_ERR_UNSUPPORTED 161003 /* valid for the reference, not (yet) built here */
+#define HSTU_ERR_WORKSPACE 161004   /* workspace missing or too small */
+#define HSTU_ERR_RUNTIME 561000     /* the HIP runtime reported an error at launch */
+
+/* element types of q/k/v (and of mask / attn_bias, which follow q) */
+#define HSTU_DT_BF16 0
+#define HSTU_DT_FP16 1
+#define HSTU_DT_FP32 2
+#define HSTU_DT_FP8_E4M3 3 /* OCP e4m3fn */
+
+/* element type of seq_offset_q / seq_offset_k / num_context / num_target */
+#define HSTU_IDX_I32 0
+#define HSTU_IDX_I64 1
+
+/* mask_type values (ascendc/attention/hstu_v1/torch_extension/hstu_common.h:47-50) */
+#define HSTU_MASK_TRIL 0
+#define HSTU_MASK_TRIU 1 /* rejected, as in the reference */
+#define HSTU_MASK_NONE 2
+#define HSTU_MASK_CUSTOM 3
+
+/* limits (hstu_common.h:31-45, op_host/tiling_policy.cpp:68-93) */
+#define HSTU_MAX_BATCH 2048
+#define HSTU_MAX_SEQ_LEN 20480
+#define HSTU_MAX_HEADS 16
+#define HSTU_MAX_HEAD_DIM 512
+
+typedef struct hstu_jagged_fwd_params {
+    uint32_t struct_size; /* sizeof(hstu_jagged_fwd_params), checked by the library */
+    int32_t dtype;        /* HSTU_DT_* of q, k, v, mask, attn_bias */
+    int32_t out_dtype;    /* HSTU_DT_* of out: same as dtype; fp8 input -> HSTU_DT_FP16 (reference) or HSTU_DT_BF16 */
+    int32_t index_dtype;  /* HSTU_IDX_* */
+
+    const void* q;            /* [total_q, num_heads_q, head_dim_qk], contiguous, device */
+    const void* k;            /* [total_k, num_heads_k, head_dim_qk] */
+    const void* v;            /* [total_k, num_heads_k, head_dim_v] */
+    const void* mask;         /* NULL or [batch, num_heads_q, max_seq_len_q, max_seq_len_k]; read iff mask_type == 3 */
+    const void* attn_bias;    /* NULL or [batch, num_heads_q, max_seq_len_q, max_seq_len_k] */
+    const void* seq_offset_q; /* [n_offsets], non-decreasing, first element 0 */
+    const void* seq_offset_k; /* [n_offsets]; may equal seq_offset_q */
+    const void* num_context;  /* NULL (= zeros) or [n_offsets - 1] */
+    const void* num_target;   /* NULL (= zeros) or [n_offsets - 1] */
+    void* out;                /* [total_q, num_heads_q, head_dim_v]; every row is written (rows past the last
+                                 offset are zero-filled), so the caller need not clear it */
+
+    int64_t total_q;
+    int64_t total_k;
+    int64_t num_heads_q;
+    int64_t num_heads_k;
+    int64_t head_dim_qk;
+    int64_t head_dim_v;
+    int64_t n_offsets; /* batch + 1 */
+
+    int64_t mask_type;
+    int64_t max_seq_len_q;
+    int64_t max_seq_len_k;
+    int64_t target_group_size;
+    double silu_scale; /* already resolved by the caller (0.0 is treated as 1 / max_seq_len_q here too) */
+    double alpha;
+    int32_t deterministic; /* accepted for signature parity; results are bitwise reproducible either way */
+    int32_t reserved0;
+
+    /* extension for quantised inputs (no counterpart in the reference, whose fp8 path is unscaled):
+     * per-head dequantisation scales, device pointers, NULL = 1.0.  Ignored unless dtype is fp8. */
+    const float* q_descale; /* [num_heads_q] */
+    const float* k_descale; /* [num_heads_k] */
+    const float* v_descale; /* [num_heads_k] */
+} hstu_jagged_fwd_params;
+
+/* replaces aclnnHstuJaggedForwardGetWorkspaceSize: validates the description and reports the scratch
+ * size (may be 0).  No device work. */
+HSTU_API int hstu_jagged_fwd_workspace_size(const hstu_jagged_fwd_params* params, uint64_t* workspace_bytes);
+
+/* replaces aclnnHstuJaggedForward: enqueues the forward on `stream` (a hipStream_t passed as void*;
+ * NULL = the default stream) and returns without waiting for it. */
+HSTU_API int hstu_jagged_fwd(const hstu_jagged_fwd_params* params, void* workspace, uint64_t workspace_bytes, void* stream);
+
+/* replaces aclGetRecentErrMsg (ascendc/common/torch_plugin/pytorch_npu_helper.hpp:649,662):
+ * text of the calling thread's most recent failure; never NULL. */
+HSTU_API const char* hstu_last_error(void);
+
+/* library version, (major << 16) | minor */
+HSTU_API int hstu_version(void);
+
+/* name of the kernel variant hstu_jagged_fwd would launch for `params` (for profiles and logs),
+ * or NULL after an error.  The string is static. */
+HSTU_API const char* hstu_jagged_fwd_kernel_name(const hstu_jagged_fwd_params* params);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HSTU_MI355_H */

@@ -1,0 +1,257 @@
+// C ABI of the MI355X HSTU jagged attention forward library: argument validation, variant
+// selection and launch.  Host-side counterpart of the reference's adapter checks
+// (ascendc/attention/hstu_v1/torch_extension/hstu_jagged_plugin.cpp:29-51,
+//  ascendc/attention/hstu_v1/torch_extension/hstu_common.h:68-82) and of its host tiling
+// (ascendc/attention/hstu_v1/hstu_forward_v1/op_host/tiling_policy_jagged.cpp:103-203,
+//  ascendc/attention/hstu_v1/hstu_forward_v1/op_host/tiling_policy.cpp:68-93).
+#include "../../include/hstu_mi355.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "hstu_fwd_kernel.hip.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+struct Variant {
+    const char* name;
+    void (*kernel)(const hstu::FwdArgs);
+    int d_pad;
+};
+
+#define HSTU_VARIANT(tag, tagname, D, BN, RAB, MINW)                                                   \
+    {"hstu_fwd_" tagname "_d" #D "_bn" #BN "_rab" #RAB, hstu::hstu_fwd_kernel<hstu::tag, D, BN, RAB, MINW>, D}
+
+// [dtype: bf16, f16][rab: 0, 1][dim slot: 32, 64, 128, 256]
+const Variant kVariants[2][2][4] = {
+    {{HSTU_VARIANT(bf16_tag, "bf16", 32, 64, false, 2), HSTU_VARIANT(bf16_tag, "bf16", 64, 64, false, 2),
+      HSTU_VARIANT(bf16_tag, "bf16", 128, 64, false, 2), HSTU_VARIANT(bf16_tag, "bf16", 256, 32, false, 1)},
+     {HSTU_VARIANT(bf16_tag, "bf16", 32, 64, true, 2), HSTU_VARIANT(bf16_tag, "bf16", 64, 64, true, 2),
+      HSTU_VARIANT(bf16_tag, "bf16", 128, 64, true, 2), HSTU_VARIANT(bf16_tag, "bf16", 256, 32, true, 1)}},
+    {{HSTU_VARIANT(f16_tag, "f16", 32, 64, false, 2), HSTU_VARIANT(f16_tag, "f16", 64, 64, false, 2),
+      HSTU_VARIANT(f16_tag, "f16", 128, 64, false, 2), HSTU_VARIANT(f16_tag, "f16", 256, 32, false, 1)},
+     {HSTU_VARIANT(f16_tag, "f16", 32, 64, true, 2), HSTU_VARIANT(f16_tag, "f16", 64, 64, true, 2),
+      HSTU_VARIANT(f16_tag, "f16", 128, 64, true, 2), HSTU_VARIANT(f16_tag, "f16", 256, 32, true, 1)}},
+};
+
+int validate(const hstu_jagged_fwd_params* p)
+{
+    if (p == nullptr) {
+        return fail(HSTU_ERR_NULLPTR, "params is NULL");
+    }
+    if (p->struct_size != sizeof(hstu_jagged_fwd_params)) {
+        return fail(HSTU_ERR_INVALID, "struct_size %u does not match this library (%zu)", p->struct_size,
+                    sizeof(hstu_jagged_fwd_params));
+    }
+    if (p->n_offsets < 2) {
+        return fail(HSTU_ERR_INVALID, "seq_offset params error should have at least two element.");
+    }
+    const int64_t batch = p->n_offsets - 1;
+    if (batch > HSTU_MAX_BATCH) {
+        return fail(HSTU_ERR_INVALID, "batchSize limit (0, %d], but get %lld", HSTU_MAX_BATCH, (long long)batch);
+    }
+    if (p->max_seq_len_q < 1 || p->max_seq_len_q > HSTU_MAX_SEQ_LEN) {
+        return fail(HSTU_ERR_INVALID, "maxSeqLen expect in [1, 20480], but value is %lld",
+                    (long long)p->max_seq_len_q);
+    }
+    if (p->max_seq_len_k < 1 || p->max_seq_len_k > HSTU_MAX_SEQ_LEN) {
+        return fail(HSTU_ERR_INVALID, "maxSeqLenK expect in [1, 20480], but value is %lld",
+                    (long long)p->max_seq_len_k);
+    }
+    if (p->mask_type < HSTU_MASK_TRIL || p->mask_type > HSTU_MASK_CUSTOM) {
+        return fail(HSTU_ERR_INVALID, "maskType expect in [0, 3], but value is %lld", (long long)p->mask_type);
+    }
+    if (p->mask_type == HSTU_MASK_TRIU) {
+        return fail(HSTU_ERR_INVALID, "maskType current not support triu now, pls use custome mask");
+    }
+    if (p->mask_type == HSTU_MASK_CUSTOM && p->mask == nullptr) {
+        return fail(HSTU_ERR_INVALID, "use custome mask must have valide mask tensor");
+    }
+    if (p->total_q < 0 || p->total_k < 0) {
+        return fail(HSTU_ERR_INVALID, "negative row count");
+    }
+    if (p->num_heads_q < 1 || p->num_heads_q > HSTU_MAX_HEADS || p->num_heads_k < 1 ||
+        p->num_heads_k > HSTU_MAX_HEADS) {
+        return fail(HSTU_ERR_INVALID, "head num expect in [1, %d], but q has %lld and k has %lld", HSTU_MAX_HEADS,
+                    (long long)p->num_heads_q, (long long)p->num_heads_k);
+    }
+    if (p->num_heads_q % p->num_heads_k != 0) {
+        return fail(HSTU_ERR_INVALID, "For GQA, headNumQ must be divisible by headNumK");
+    }
+    if (p->head_dim_qk < 1 || p->head_dim_qk > HSTU_MAX_HEAD_DIM) {
+        return fail(HSTU_ERR_INVALID, "dim size expect in [1, 512], but q/k head dim is %lld",
+                    (long long)p->head_dim_qk);
+    }
+    if (p->head_dim_v < 16 || p->head_dim_v > HSTU_MAX_HEAD_DIM || p->head_dim_v % 16 != 0) {
+        return fail(HSTU_ERR_INVALID, "dim size expect in [16, 512] step 16, but v head dim is %lld",
+                    (long long)p->head_dim_v);
+    }
+    if (p->target_group_size < 0) {
+        return fail(HSTU_ERR_INVALID, "targetGroupSize must be >= 0");
+    }
+    if (p->index_dtype != HSTU_IDX_I32 && p->index_dtype != HSTU_IDX_I64) {
+        return fail(HSTU_ERR_INVALID, "index_dtype must be int32 or int64");
+    }
+    if (p->dtype < HSTU_DT_BF16 || p->dtype > HSTU_DT_FP8_E4M3) {
+        return fail(HSTU_ERR_INVALID, "unknown dtype %d", p->dtype);
+    }
+    const bool empty = (p->total_q == 0);
+    if (!empty && (p->q == nullptr || p->out == nullptr)) {
+        return fail(HSTU_ERR_NULLPTR, "q / out must not be NULL");
+    }
+    if (p->total_k > 0 && (p->k == nullptr || p->v == nullptr)) {
+        return fail(HSTU_ERR_NULLPTR, "k / v must not be NULL");
+    }
+    if (p->seq_offset_q == nullptr || p->seq_offset_k == nullptr) {
+        return fail(HSTU_ERR_NULLPTR, "seq_offset_q / seq_offset_k must not be NULL");
+    }
+    return HSTU_OK;
+}
+
+// picks the kernel variant; returns nullptr (and sets the error) when the combination is not built
+const Variant* select(const hstu_jagged_fwd_params* p)
+{
+    if (p->dtype != HSTU_DT_BF16 && p->dtype != HSTU_DT_FP16) {
+        fail(HSTU_ERR_UNSUPPORTED, "dtype %d is not built in this library version (bf16 and fp16 are)", p->dtype);
+        return nullptr;
+    }
+    if (p->out_dtype != p->dtype) {
+        fail(HSTU_ERR_UNSUPPORTED, "out_dtype must equal dtype for bf16 / fp16 inputs");
+        return nullptr;
+    }
+    if (p->head_dim_qk % 8 != 0) {
+        fail(HSTU_ERR_UNSUPPORTED, "q/k head dim %lld is not a multiple of 8", (long long)p->head_dim_qk);
+        return nullptr;
+    }
+    const int64_t dmax = p->head_dim_qk > p->head_dim_v ? p->head_dim_qk : p->head_dim_v;
+    int slot;
+    if (dmax <= 32) {
+        slot = 0;
+    } else if (dmax <= 64) {
+        slot = 1;
+    } else if (dmax <= 128) {
+        slot = 2;
+    } else if (dmax <= 256) {
+        slot = 3;
+    } else {
+        fail(HSTU_ERR_UNSUPPORTED, "head dims above 256 are not built in this library version (got %lld)",
+             (long long)dmax);
+        return nullptr;
+    }
+    return &kVariants[p->dtype == HSTU_DT_BF16 ? 0 : 1][p->attn_bias != nullptr ? 1 : 0][slot];
+}
+
+}  // namespace
+
+extern "C" {
+
+HSTU_API int hstu_version(void) { return (0 << 16) | 1; }
+
+HSTU_API const char* hstu_last_error(void) { return g_err; }
+
+HSTU_API int hstu_jagged_fwd_workspace_size(const hstu_jagged_fwd_params* params, uint64_t* workspace_bytes)
+{
+    if (workspace_bytes == nullptr) {
+        return fail(HSTU_ERR_NULLPTR, "workspace_bytes is NULL");
+    }
+    *workspace_bytes = 0;
+    const int rc = validate(params);
+    if (rc != HSTU_OK) {
+        return rc;
+    }
+    if (select(params) == nullptr) {
+        return HSTU_ERR_UNSUPPORTED;
+    }
+    // the tile schedule is derived inside the kernel from seq_offset, no scratch is needed
+    *workspace_bytes = 0;
+    return HSTU_OK;
+}
+
+HSTU_API const char* hstu_jagged_fwd_kernel_name(const hstu_jagged_fwd_params* params)
+{
+    if (validate(params) != HSTU_OK) {
+        return nullptr;
+    }
+    const Variant* v = select(params);
+    return v ? v->name : nullptr;
+}
+
+HSTU_API int hstu_jagged_fwd(const hstu_jagged_fwd_params* p, void* workspace, uint64_t workspace_bytes, void* stream)
+{
+    (void)workspace;
+    (void)workspace_bytes;
+    const int rc = validate(p);
+    if (rc != HSTU_OK) {
+        return rc;
+    }
+    const Variant* var = select(p);
+    if (var == nullptr) {
+        return HSTU_ERR_UNSUPPORTED;
+    }
+    if (p->total_q == 0) {
+        return HSTU_OK;
+    }
+
+    hstu::FwdArgs a;
+    memset(&a, 0, sizeof(a));
+    a.q = p->q;
+    a.k = p->k;
+    a.v = p->v;
+    a.rab = p->attn_bias;
+    a.mask = (p->mask_type == HSTU_MASK_CUSTOM) ? p->mask : nullptr;
+    a.out = p->out;
+    a.offs_q = p->seq_offset_q;
+    a.offs_k = p->seq_offset_k;
+    a.num_ctx = p->num_context;
+    a.num_tgt = p->num_target;
+    a.total_q = p->total_q;
+    a.total_k = p->total_k;
+    a.n_batch = static_cast<int>(p->n_offsets - 1);
+    a.n_heads_q = static_cast<int>(p->num_heads_q);
+    a.n_heads_k = static_cast<int>(p->num_heads_k);
+    a.head_ratio = a.n_heads_q / a.n_heads_k;
+    a.d_qk = static_cast<int>(p->head_dim_qk);
+    a.d_v = static_cast<int>(p->head_dim_v);
+    a.max_q = static_cast<int>(p->max_seq_len_q);
+    a.max_k = static_cast<int>(p->max_seq_len_k);
+    a.mask_type = static_cast<int>(p->mask_type);
+    a.target_group = static_cast<int>(p->target_group_size);
+    a.idx64 = (p->index_dtype == HSTU_IDX_I64) ? 1 : 0;
+    a.n_qtiles = (a.max_q + hstu::kBlockM - 1) / hstu::kBlockM;
+    a.bh = a.n_batch * a.n_heads_q;
+    const bool bias_aligned = (reinterpret_cast<uintptr_t>(p->attn_bias) % 8 == 0) &&
+                              (reinterpret_cast<uintptr_t>(p->mask) % 8 == 0) && (p->max_seq_len_k % 4 == 0);
+    a.rab_vec_ok = bias_aligned ? 1 : 0;
+    const double scale = (p->silu_scale == 0.0) ? 1.0 / static_cast<double>(p->max_seq_len_q) : p->silu_scale;
+    a.c_exp = static_cast<float>(-p->alpha * 1.4426950408889634);
+    a.c_out = static_cast<float>(p->alpha * scale);
+
+    const int64_t n_blocks = static_cast<int64_t>(a.n_qtiles) * a.bh;
+    if (n_blocks <= 0 || n_blocks > 0x7fffffffLL) {
+        return fail(HSTU_ERR_INVALID, "grid of %lld workgroups is out of range", (long long)n_blocks);
+    }
+    hipLaunchKernelGGL(var->kernel, dim3(static_cast<unsigned>(n_blocks)), dim3(hstu::kThreads), 0,
+                       static_cast<hipStream_t>(stream), a);
+    const hipError_t err = hipGetLastError();
+    if (err != hipSuccess) {
+        return fail(HSTU_ERR_RUNTIME, "launch of %s failed: %s", var->name, hipGetErrorString(err));
+    }
+    return HSTU_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,107 @@
+"""ctypes binding of the C ABI declared in ``include/hstu_mi355.h``.
+
+The library is loaded from ``ops_rec/_lib``; if it is missing the import fails loudly on
+first use -- there is no CPU or eager fallback for the operator.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import os
+from typing import Optional
+
+from . import _build
+
+HSTU_OK = 0
+DT_BF16, DT_FP16, DT_FP32, DT_FP8_E4M3 = 0, 1, 2, 3
+IDX_I32, IDX_I64 = 0, 1
+
+EXPORTED_SYMBOLS = (
+    "hstu_jagged_fwd_workspace_size",
+    "hstu_jagged_fwd",
+    "hstu_last_error",
+    "hstu_version",
+    "hstu_jagged_fwd_kernel_name",
+)
+
+
+class FwdParams(ctypes.Structure):
+    """Mirror of ``hstu_jagged_fwd_params``."""
+
+    _fields_ = [
+        ("struct_size", ctypes.c_uint32),
+        ("dtype", ctypes.c_int32),
+        ("out_dtype", ctypes.c_int32),
+        ("index_dtype", ctypes.c_int32),
+        ("q", ctypes.c_void_p),
+        ("k", ctypes.c_void_p),
+        ("v", ctypes.c_void_p),
+        ("mask", ctypes.c_void_p),
+        ("attn_bias", ctypes.c_void_p),
+        ("seq_offset_q", ctypes.c_void_p),
+        ("seq_offset_k", ctypes.c_void_p),
+        ("num_context", ctypes.c_void_p),
+        ("num_target", ctypes.c_void_p),
+        ("out", ctypes.c_void_p),
+        ("total_q", ctypes.c_int64),
+        ("total_k", ctypes.c_int64),
+        ("num_heads_q", ctypes.c_int64),
+        ("num_heads_k", ctypes.c_int64),
+        ("head_dim_qk", ctypes.c_int64),
+        ("head_dim_v", ctypes.c_int64),
+        ("n_offsets", ctypes.c_int64),
+        ("mask_type", ctypes.c_int64),
+        ("max_seq_len_q", ctypes.c_int64),
+        ("max_seq_len_k", ctypes.c_int64),
+        ("target_group_size", ctypes.c_int64),
+        ("silu_scale", ctypes.c_double),
+        ("alpha", ctypes.c_double),
+        ("deterministic", ctypes.c_int32),
+        ("reserved0", ctypes.c_int32),
+        ("q_descale", ctypes.c_void_p),
+        ("k_descale", ctypes.c_void_p),
+        ("v_descale", ctypes.c_void_p),
+    ]
+
+
+_lib: Optional[ctypes.CDLL] = None
+
+
+def library_path() -> str:
+    return _build.LIB_PATH
+
+
+def load() -> ctypes.CDLL:
+    """Load the HIP library; raises if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    path = library_path()
+    if not os.path.exists(path):
+        raise RuntimeError(
+            f"HIP library not found at {path}. Build it first (python -c 'import __graft_entry__ as g; g.build()' "
+            "or ops_rec._build.build()); the operator has no fallback path."
+        )
+    lib = ctypes.CDLL(path)
+    lib.hstu_jagged_fwd_workspace_size.restype = ctypes.c_int
+    lib.hstu_jagged_fwd_workspace_size.argtypes = [ctypes.POINTER(FwdParams), ctypes.POINTER(ctypes.c_uint64)]
+    lib.hstu_jagged_fwd.restype = ctypes.c_int
+    lib.hstu_jagged_fwd.argtypes = [ctypes.POINTER(FwdParams), ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]
+    lib.hstu_last_error.restype = ctypes.c_char_p
+    lib.hstu_last_error.argtypes = []
+    lib.hstu_version.restype = ctypes.c_int
+    lib.hstu_version.argtypes = []
+    lib.hstu_jagged_fwd_kernel_name.restype = ctypes.c_char_p
+    lib.hstu_jagged_fwd_kernel_name.argtypes = [ctypes.POINTER(FwdParams)]
+    _lib = lib
+    return lib
+
+
+def last_error() -> str:
+    return load().hstu_last_error().decode("utf-8", "replace")
+
+
+def new_params() -> FwdParams:
+    p = FwdParams()
+    p.struct_size = ctypes.sizeof(FwdParams)
+    return p

@@ -1,0 +1,350 @@
+"""Operator registration for ``torch.ops.ops_rec.hstu_jagged[_backward]``.
+
+Mirrors the reference adapter for this path
+(ascendc/attention/hstu_v1/torch_extension/hstu_jagged_plugin.cpp):
+
+* the four schema strings are the reference's (``:188-247``) -- they are the calling contract;
+* ``_forward_impl`` does the argument normalisation and checks of
+  ``hstu_deltaq_forward_impl_npu`` (``:22-67``) and then calls the C ABI of the HIP library
+  where the reference calls ``aclnnHstuJaggedForward`` (``:63-65``);
+* device tensors dispatch on the ``CUDA`` key (PyTorch-ROCm's key for HIP tensors), shape
+  inference for ``torch.compile`` on ``Meta`` (``:269-351``); autograd is attached from Python
+  (``ops_rec/autograd/hstu_v1_autograd.py``), not here (``:258-263``).
+
+There is no CPU implementation: calling the op on CPU tensors raises, as it does in the
+reference (which registers only the NPU and Meta keys).
+"""
+
+from __future__ import annotations
+
+import ctypes
+from typing import Optional, Tuple
+
+import torch
+
+from . import _native
+
+_MAX_SEQ_LEN = 20480
+
+_SCHEMAS = (
+    "hstu_jagged.equal(Tensor q, Tensor k, Tensor v, Tensor? mask=None, Tensor? attn_bias=None, int mask_type=0, "
+    "int max_seq_len=0, float silu_scale=0.0, Tensor seq_offset=None, Tensor? num_context=None, "
+    "Tensor? num_target=None, int? target_group_size=0, float? alpha=1.0, bool deterministic=False) -> Tensor",
+    "hstu_jagged_backward.equal(Tensor grad, Tensor q, Tensor k, Tensor v, Tensor? mask=None, "
+    "Tensor? attn_bias=None, int mask_type=0, int max_seq_len=0, float silu_scale=0.0, Tensor seq_offset=None, "
+    "Tensor? num_context=None, Tensor? num_target=None, int? target_group_size=0, float? alpha=1.0) "
+    "-> (Tensor, Tensor, Tensor, Tensor)",
+    "hstu_jagged.delta(Tensor q, Tensor k, Tensor v, Tensor? mask=None, Tensor? attn_bias=None, int mask_type=0, "
+    "int max_seq_len=0, int max_seq_len_k=0, float silu_scale=0.0, Tensor seq_offset=None, "
+    "Tensor seq_offset_k=None, Tensor? num_context=None, Tensor? num_target=None, int? target_group_size=0, "
+    "float? alpha=1.0, bool deterministic=False) -> Tensor",
+    "hstu_jagged_backward.delta(Tensor grad, Tensor q, Tensor k, Tensor v, Tensor? mask=None, "
+    "Tensor? attn_bias=None, int mask_type=0, int max_seq_len=0, int max_seq_len_k=0, float silu_scale=0.0, "
+    "Tensor seq_offset=None, Tensor seq_offset_k=None, Tensor? num_context=None, Tensor? num_target=None, "
+    "int? target_group_size=0, float? alpha=1.0) -> (Tensor, Tensor, Tensor, Tensor)",
+)
+
+_lib_def = torch.library.Library("ops_rec", "DEF")
+for _s in _SCHEMAS:
+    _lib_def.define(_s)
+_lib_cuda = torch.library.Library("ops_rec", "IMPL", "CUDA")
+_lib_meta = torch.library.Library("ops_rec", "IMPL", "Meta")
+
+_DTYPE_CODE = {
+    torch.bfloat16: _native.DT_BF16,
+    torch.float16: _native.DT_FP16,
+    torch.float32: _native.DT_FP32,
+    torch.float8_e4m3fn: _native.DT_FP8_E4M3,
+}
+
+
+def _check(cond: bool, msg: str) -> None:
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _max_seq_len_check(value: int, what: str) -> None:
+    _check(1 <= value <= _MAX_SEQ_LEN, f"{what} check failed: maxSeqLen expect in [1, 20480], but value is {value}")
+
+
+def _mask_check(mask_type: int, mask_defined: bool) -> None:
+    _check(0 <= mask_type <= 3, f"maskType expect in [0, 3], but value is {mask_type}")
+    _check(mask_type != 1, "maskType current not support triu now, pls use custome mask")
+    _check(not (mask_type == 3 and not mask_defined), "use custome mask must have valide mask tensor")
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    if t is None or t.numel() == 0:
+        return None
+    return t.data_ptr()
+
+
+def _out_dtype(q: torch.Tensor) -> torch.dtype:
+    return torch.float16 if q.dtype == torch.float8_e4m3fn else q.dtype
+
+
+def _forward_impl(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    mask: Optional[torch.Tensor],
+    attn_bias: Optional[torch.Tensor],
+    mask_type: int,
+    max_seq_len_q: int,
+    max_seq_len_k: int,
+    silu_scale: float,
+    seq_offset: torch.Tensor,
+    seq_offset_k: torch.Tensor,
+    num_context: Optional[torch.Tensor],
+    num_target: Optional[torch.Tensor],
+    target_group_size: Optional[int],
+    alpha: Optional[float],
+    deterministic: bool = False,
+) -> torch.Tensor:
+    _check(q.dim() == 3, "The q should be 3D in jagged layout")
+    _check(seq_offset is not None and seq_offset_k is not None, "seq_offset is required")
+    _check(seq_offset.dim() == 1 and seq_offset.size(0) >= 2,
+           "acSeqOffset params error should have at least two element.")  # fmt: skip
+    _check(seq_offset_k.dim() == 1 and seq_offset_k.size(0) >= 2,
+           "acSeqOffsetK params error should have at least two element.")  # fmt: skip
+    _check(seq_offset.dtype in (torch.int32, torch.int64), "seq_offset must be int32 or int64")
+    _check(k.dim() == 3 and v.dim() == 3, "The k and v should be 3D in jagged layout")
+    _check(q.dtype == k.dtype == v.dtype, "q, k, v must share one dtype")
+    _check(q.dtype in _DTYPE_CODE, f"unsupported dtype {q.dtype}")
+
+    idx_dtype = seq_offset.dtype
+    offs_q = seq_offset.contiguous()
+    offs_k = offs_q if seq_offset_k is seq_offset else seq_offset_k.to(idx_dtype).contiguous()
+    q_c, k_c, v_c = q.contiguous(), k.contiguous(), v.contiguous()
+    batch = offs_q.size(0) - 1
+    ctx = num_context.to(idx_dtype).contiguous() if num_context is not None else None
+    tgt = num_target.to(idx_dtype).contiguous() if num_target is not None else None
+    group = 0 if target_group_size is None else int(target_group_size)
+    real_alpha = 1.0 if alpha is None else float(alpha)
+
+    _max_seq_len_check(int(max_seq_len_q), "maxSeqLen")
+    _max_seq_len_check(int(max_seq_len_k), "maxSeqLenK")
+    _mask_check(int(mask_type), mask is not None)
+    _check(offs_k.size(0) == offs_q.size(0), "seq_offset and seq_offset_k must have the same length")
+    _check(k_c.size(0) == v_c.size(0), "K, V seqLens mismatch")
+    _check(k_c.size(1) == v_c.size(1), "K, V headNum mismatch")
+    _check(q_c.size(2) == k_c.size(2), "Q, K, V headDIM Shape Check failed")
+    if ctx is not None:
+        _check(ctx.dim() == 1 and ctx.size(0) == batch, f"The length of num_context expect {batch}")
+    if tgt is not None:
+        _check(tgt.dim() == 1 and tgt.size(0) == batch, f"The length of num_target expect {batch}")
+    bias_shape = (batch, q_c.size(1), int(max_seq_len_q), int(max_seq_len_k))
+    bias = None
+    if attn_bias is not None:
+        _check(attn_bias.dtype == q.dtype, "attn_bias must have the dtype of q")
+        _check(tuple(attn_bias.shape) == bias_shape, f"attn_bias must have shape {bias_shape}")
+        bias = attn_bias.contiguous()
+    mask_c = None
+    if mask is not None and int(mask_type) == 3:
+        _check(mask.dtype == q.dtype, "mask must have the dtype of q")
+        _check(tuple(mask.shape) == bias_shape, f"mask must have shape {bias_shape}")
+        mask_c = mask.contiguous()
+
+    out_dtype = _out_dtype(q_c)
+    # every row is written by the kernel (rows past the last offset are zero-filled there),
+    # so the zero-fill of the reference adapter (:56-59) is not repeated here
+    out = torch.empty((q_c.size(0), q_c.size(1), v_c.size(2)), dtype=out_dtype, device=q_c.device)
+    if out.numel() == 0:
+        return out
+
+    real_scale = (1.0 / float(max_seq_len_q)) if float(silu_scale) == 0.0 else float(silu_scale)
+
+    lib = _native.load()
+    p = _native.new_params()
+    p.dtype = _DTYPE_CODE[q_c.dtype]
+    p.out_dtype = _DTYPE_CODE[out_dtype]
+    p.index_dtype = _native.IDX_I64 if idx_dtype == torch.int64 else _native.IDX_I32
+    p.q, p.k, p.v = _ptr(q_c), _ptr(k_c), _ptr(v_c)
+    p.mask, p.attn_bias = _ptr(mask_c), _ptr(bias)
+    p.seq_offset_q, p.seq_offset_k = _ptr(offs_q), _ptr(offs_k)
+    p.num_context, p.num_target = _ptr(ctx), _ptr(tgt)
+    p.out = _ptr(out)
+    p.total_q, p.total_k = q_c.size(0), k_c.size(0)
+    p.num_heads_q, p.num_heads_k = q_c.size(1), k_c.size(1)
+    p.head_dim_qk, p.head_dim_v = q_c.size(2), v_c.size(2)
+    p.n_offsets = offs_q.size(0)
+    p.mask_type = int(mask_type)
+    p.max_seq_len_q, p.max_seq_len_k = int(max_seq_len_q), int(max_seq_len_k)
+    p.target_group_size = group
+    p.silu_scale = real_scale
+    p.alpha = real_alpha
+    p.deterministic = 1 if deterministic else 0
+
+    with torch.cuda.device(q_c.device):
+        ws_bytes = ctypes.c_uint64(0)
+        rc = lib.hstu_jagged_fwd_workspace_size(ctypes.byref(p), ctypes.byref(ws_bytes))
+        if rc != _native.HSTU_OK:
+            raise RuntimeError(f"hstu_jagged_fwd_workspace_size failed ({rc}): {_native.last_error()}")
+        ws = None
+        if ws_bytes.value:
+            ws = torch.empty(ws_bytes.value, dtype=torch.uint8, device=q_c.device)
+        stream = torch.cuda.current_stream(q_c.device).cuda_stream
+        rc = lib.hstu_jagged_fwd(ctypes.byref(p), _ptr(ws), ws_bytes.value, ctypes.c_void_p(stream))
+        if rc != _native.HSTU_OK:
+            raise RuntimeError(f"hstu_jagged_fwd failed ({rc}): {_native.last_error()}")
+    return out
+
+
+# Python kernels receive only the arguments the caller passed, so the schema defaults are
+# repeated in the signatures below.
+
+
+def hstu_jagged_equal(q, k, v, mask=None, attn_bias=None, mask_type=0, max_seq_len=0, silu_scale=0.0,
+                      seq_offset=None, num_context=None, num_target=None, target_group_size=0, alpha=1.0,
+                      deterministic=False):  # fmt: skip
+    return _forward_impl(q, k, v, mask, attn_bias, mask_type, max_seq_len, max_seq_len, silu_scale, seq_offset,
+                         seq_offset, num_context, num_target, target_group_size, alpha, deterministic)  # fmt: skip
+
+
+def hstu_jagged_delta(q, k, v, mask=None, attn_bias=None, mask_type=0, max_seq_len=0, max_seq_len_k=0,
+                      silu_scale=0.0, seq_offset=None, seq_offset_k=None, num_context=None, num_target=None,
+                      target_group_size=0, alpha=1.0, deterministic=False):  # fmt: skip
+    return _forward_impl(q, k, v, mask, attn_bias, mask_type, max_seq_len, max_seq_len_k, silu_scale, seq_offset,
+                         seq_offset_k, num_context, num_target, target_group_size, alpha, deterministic)  # fmt: skip
+
+
+def _forward_meta(q, v):
+    _check(q.dim() == 3, "The q should be 3D in jagged layout")
+    return q.new_empty((q.shape[0], q.shape[1], v.shape[2]), dtype=_out_dtype(q))
+
+
+def hstu_jagged_equal_meta(q, k, v, mask=None, attn_bias=None, mask_type=0, max_seq_len=0, silu_scale=0.0,
+                           seq_offset=None, num_context=None, num_target=None, target_group_size=0, alpha=1.0,
+                           deterministic=False):  # fmt: skip
+    return _forward_meta(q, v)
+
+
+def hstu_jagged_delta_meta(q, k, v, mask=None, attn_bias=None, mask_type=0, max_seq_len=0, max_seq_len_k=0,
+                           silu_scale=0.0, seq_offset=None, seq_offset_k=None, num_context=None, num_target=None,
+                           target_group_size=0, alpha=1.0, deterministic=False):  # fmt: skip
+    return _forward_meta(q, v)
+
+
+# ----------------------------------------------------------------------------------------------
+# backward op: device-side composite (torch ops on the GPU, per sequence, fp32).  It exists so that
+# the autograd wrapper of the forward is complete; it is not a tuned kernel.
+#   X = alpha (S + rab),  sig = sigmoid(X),  P = X sig scale M
+#   dV = P^T dO,  dX = (dO V^T) scale M sig (1 + X (1 - sig)),  dS = dRab = alpha dX,  dQ = dS K,  dK = dS^T Q
+# (ascendc/attention/hstu_v1/hstu_backward_v1/op_kernel/vector_score.h:159-205)
+# ----------------------------------------------------------------------------------------------
+
+
+def _device_builtin_mask(s_q, s_k, ctx, tgt, group, device):
+    rows = torch.arange(s_q, device=device)[:, None]
+    cols = torch.arange(s_k, device=device)[None, :]
+    m = cols <= rows + (s_k - s_q)
+    if ctx > 0:
+        m = m | ((rows < ctx) & (cols < s_k - tgt))
+    if tgt > 0 and group > 0:
+        ti = rows - (s_q - tgt)
+        tj = cols - (s_k - tgt)
+        inside = (ti >= 0) & (tj >= 0)
+        blk = (tj <= ti) & (torch.div(ti, group, rounding_mode="floor") == torch.div(tj, group, rounding_mode="floor"))
+        m = torch.where(inside, blk, m)
+    return m
+
+
+def _backward_impl(grad, q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max_seq_len_k, silu_scale, seq_offset,
+                   seq_offset_k, num_context, num_target, target_group_size, alpha):  # fmt: skip
+    _check(seq_offset.size(0) >= 2, "seqOffsetQ params error should have at least two element.")
+    _check(seq_offset_k.size(0) >= 2, "seqOffsetK params error should have at least two element.")
+    _max_seq_len_check(int(max_seq_len_q), "maxSeqLenQ")
+    _max_seq_len_check(int(max_seq_len_k), "maxSeqLenK")
+    if num_context is not None or num_target is not None:
+        _check(num_context is not None, "numContext is required when numTarget or targetGroupSize is not None")
+        _check(num_target is not None, "numTarget is required when numContext or targetGroupSize is not None")
+    group = 0 if target_group_size is None else int(target_group_size)
+    a = 1.0 if alpha is None else float(alpha)
+    scale = (1.0 / float(max_seq_len_q)) if float(silu_scale) == 0.0 else float(silu_scale)
+    offs_q = seq_offset.tolist()
+    offs_k = seq_offset_k.tolist()
+    ctx = num_context.tolist() if num_context is not None else None
+    tgt = num_target.tolist() if num_target is not None else None
+    n_q, n_k = q.shape[1], k.shape[1]
+    ratio = n_q // n_k
+    f32 = torch.float32
+    dq = torch.zeros(q.shape, dtype=f32, device=q.device)
+    dk = torch.zeros(k.shape, dtype=f32, device=q.device)
+    dv = torch.zeros(v.shape, dtype=f32, device=q.device)
+    dbias = torch.zeros(attn_bias.shape, dtype=f32, device=q.device) if attn_bias is not None else None
+    last = offs_q[-1]
+    batch = offs_q.index(last)
+    for b in range(batch):
+        q0, q1, k0, k1 = offs_q[b], offs_q[b + 1], offs_k[b], offs_k[b + 1]
+        s_q, s_k = q1 - q0, k1 - k0
+        if s_q <= 0 or s_k <= 0:
+            continue
+        qb = q[q0:q1].to(f32).transpose(0, 1)  # [n_q, s_q, d]
+        kb = k[k0:k1].to(f32).transpose(0, 1).repeat_interleave(ratio, dim=0)
+        vb = v[k0:k1].to(f32).transpose(0, 1).repeat_interleave(ratio, dim=0)
+        go = grad[q0:q1].to(f32).transpose(0, 1)  # [n_q, s_q, d_v]
+        s = qb @ kb.transpose(1, 2)
+        if attn_bias is not None:
+            s = s + attn_bias[b, :, :s_q, :s_k].to(f32)
+        x = s * a
+        sig = torch.sigmoid(x)
+        if mask_type == 3:
+            m = mask[b, :, :s_q, :s_k].to(f32)
+        elif mask_type == 0:
+            m = _device_builtin_mask(s_q, s_k, ctx[b] if ctx else 0, tgt[b] if tgt else 0, group, q.device).to(f32)[None]
+        else:
+            m = torch.ones((), dtype=f32, device=q.device)
+        p = x * sig * scale * m
+        dvb = p.transpose(1, 2) @ go  # [n_q, s_k, d_v]
+        dx = (go @ vb.transpose(1, 2)) * scale * m * (sig * (1.0 + x * (1.0 - sig)))
+        ds = dx * a
+        dq[q0:q1] = (ds @ kb).transpose(0, 1)
+        dkb = ds.transpose(1, 2) @ qb  # [n_q, s_k, d]
+        dk[k0:k1] = dkb.reshape(n_k, ratio, s_k, -1).sum(1).transpose(0, 1)
+        dv[k0:k1] = dvb.reshape(n_k, ratio, s_k, -1).sum(1).transpose(0, 1)
+        if dbias is not None:
+            dbias[b, :, :s_q, :s_k] = ds
+    out_bias = dbias.to(attn_bias.dtype) if dbias is not None else None
+    return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype), out_bias
+
+
+def hstu_jagged_backward_equal(grad, q, k, v, mask=None, attn_bias=None, mask_type=0, max_seq_len=0, silu_scale=0.0,
+                               seq_offset=None, num_context=None, num_target=None, target_group_size=0,
+                               alpha=1.0):  # fmt: skip
+    return _backward_impl(grad, q, k, v, mask, attn_bias, mask_type, max_seq_len, max_seq_len, silu_scale,
+                          seq_offset, seq_offset, num_context, num_target, target_group_size, alpha)  # fmt: skip
+
+
+def hstu_jagged_backward_delta(grad, q, k, v, mask=None, attn_bias=None, mask_type=0, max_seq_len=0,
+                               max_seq_len_k=0, silu_scale=0.0, seq_offset=None, seq_offset_k=None,
+                               num_context=None, num_target=None, target_group_size=0, alpha=1.0):  # fmt: skip
+    return _backward_impl(grad, q, k, v, mask, attn_bias, mask_type, max_seq_len, max_seq_len_k, silu_scale,
+                          seq_offset, seq_offset_k, num_context, num_target, target_group_size, alpha)  # fmt: skip
+
+
+def _backward_meta(grad, q, k, v, attn_bias) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor, Optional[torch.Tensor]]:
+    _check(grad.dim() == 3, "The grad should be 3D in jagged layout")
+    dbias = torch.empty_like(attn_bias) if attn_bias is not None else None
+    return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), dbias
+
+
+def hstu_jagged_backward_equal_meta(grad, q, k, v, mask=None, attn_bias=None, mask_type=0, max_seq_len=0,
+                                    silu_scale=0.0, seq_offset=None, num_context=None, num_target=None,
+                                    target_group_size=0, alpha=1.0):  # fmt: skip
+    return _backward_meta(grad, q, k, v, attn_bias)
+
+
+def hstu_jagged_backward_delta_meta(grad, q, k, v, mask=None, attn_bias=None, mask_type=0, max_seq_len=0,
+                                    max_seq_len_k=0, silu_scale=0.0, seq_offset=None, seq_offset_k=None,
+                                    num_context=None, num_target=None, target_group_size=0, alpha=1.0):  # fmt: skip
+    return _backward_meta(grad, q, k, v, attn_bias)
+
+
+_lib_cuda.impl("hstu_jagged.equal", hstu_jagged_equal)
+_lib_cuda.impl("hstu_jagged.delta", hstu_jagged_delta)
+_lib_cuda.impl("hstu_jagged_backward.equal", hstu_jagged_backward_equal)
+_lib_cuda.impl("hstu_jagged_backward.delta", hstu_jagged_backward_delta)
+_lib_meta.impl("hstu_jagged.equal", hstu_jagged_equal_meta)
+_lib_meta.impl("hstu_jagged.delta", hstu_jagged_delta_meta)
+_lib_meta.impl("hstu_jagged_backward.equal", hstu_jagged_backward_equal_meta)
+_lib_meta.impl("hstu_jagged_backward.delta", hstu_jagged_backward_delta_meta)

@@ -1,0 +1,5 @@
+"""Operator groups, named as in the reference (``ops_rec.ascendc.<group>.<op>``)."""
+
+from . import attention  # noqa: F401
+
+__all__ = ["attention"]
