@@ -1,0 +1,214 @@
+#!/usr/bin/env python3
+"""Benchmark of the HSTU jagged attention forward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2|C3|C4] [--no-cpu]
+
+A "step" is one forward over one synthetic jagged batch whose inputs already sit in HBM.
+The default workload is the configuration the headline metric is quoted on (C2: bf16, batch 32,
+heads 4, head dim 128, lengths uniform in [256, 1024], max_seq_len 1024, alpha 128^-0.5,
+silu_scale 1/1024, causal, no rab).
+
+Prints ONE JSON line.  ``value`` is causal-effective TFLOP/s of the whole job
+(FLOPs = 2 (d_qk + d_v) N_q sum_b nnz(mask_b); SiLU / bias / mask work is not counted);
+``ms_per_step`` is the ms/batch half of the metric.  Launches go through the C ABI
+(``hstu_jagged_fwd``, the drop-in boundary) back-to-back on torch's current stream and are
+timed with events on that same stream; the cost of one call through the Python entry point
+(``ops_rec.ascendc.attention.hstu_jagged``) is reported next to it as ``ms_per_step_python_entry``.
+
+``roofline``     -- dominant (only) kernel against the bf16 dense MFMA peak; ``hbm_*`` fields give the
+                    same launch against the HBM bound on compulsory bytes.
+``cpu_baseline`` -- the oracle's dense-padded fp32 restatement of the reference's PyTorch golden path,
+                    timed on this host's cores on the same batch (a reported baseline, not a target).
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+_ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(_ROOT, "ops-rec_amd"))
+sys.path.insert(0, _ROOT)
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA peak (published)
+PEAK_HBM_GBS = 8000.0  # MI355X HBM3E bandwidth (published)
+
+# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), scaled by the same
+# counters' reading of a plain copy kernel of known size; see profiles/.  None = not measured yet.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def algorithmic_bytes(w) -> int:
+    """Compulsory HBM traffic: Q, K, V read once, O written once, visible rab elements read once."""
+    es = w.q.element_size()
+    n = w.q.numel() * es + w.k.numel() * es + w.v.numel() * es
+    n += w.q.shape[0] * w.q.shape[1] * w.v.shape[2] * es
+    n += w.seq_offset.numel() * w.seq_offset.element_size()
+    return n
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="C2", choices=["C2", "C3", "C4"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(
+            "bench.py: this build runs on one GPU only (sequences and heads are independent, so the "
+            "path shards with no communication; nothing here uses a second GPU). Use --gpus 1.",
+            file=sys.stderr,
+        )
+        return 2
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the operator has no CPU path", file=sys.stderr)
+        return 1
+
+    import ops_rec
+    from ops_rec import _ops, workloads
+    from oracle import hstu_oracle as oracle  # FLOP model + cpu_baseline leg only
+
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    heavy = args.workload != "C2"
+    w_cpu = None if heavy else workloads.config(args.workload)
+    w = workloads.config(args.workload, device=dev) if heavy else w_cpu.to(dev)
+    n_q, d_qk, d_v = w.q.shape[1], w.q.shape[2], w.v.shape[2]
+    ctx = None if w.num_context is None else w.num_context.cpu()
+    tgt = None if w.num_target is None else w.num_target.cpu()
+    flops = oracle.causal_effective_flops(w.seq_offset.cpu(), None, n_q, d_qk, d_v, w.mask_type, ctx, tgt,
+                                          w.target_group_size)  # fmt: skip
+    nnz = flops // (2 * (d_qk + d_v) * n_q)
+    alg_bytes = algorithmic_bytes(w)
+    rab_bytes = 0
+    if w.attn_bias is not None:
+        rab_bytes = nnz * n_q * w.attn_bias.element_size()
+    alg_bytes += rab_bytes
+
+    prepared = _ops.prepare_forward(
+        w.q, w.k, w.v, w.mask, w.attn_bias, w.mask_type, w.max_seq_len, w.max_seq_len, w.silu_scale, w.seq_offset,
+        w.seq_offset, w.num_context, w.num_target, w.target_group_size, w.alpha,
+    )  # fmt: skip
+    kernel_name = prepared.kernel_name()
+    stream = torch.cuda.current_stream(dev)
+    raw_stream = stream.cuda_stream
+
+    # ---- GPU: K launches through the C ABI, events on the launch stream ----
+    for _ in range(args.warmup):
+        prepared.launch(raw_stream)
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record(stream)
+    for _ in range(args.steps):
+        prepared.launch(raw_stream)
+    e1.record(stream)
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    ev_ms = e0.elapsed_time(e1) / args.steps
+    ms_per_step = max(wall_ms, ev_ms)  # the slower clock: host-bound launches cannot hide
+
+    # ---- the same through the Python entry point ----
+    op = ops_rec.ascendc.attention.hstu_jagged
+    op_args = w.op_args()
+    for _ in range(5):
+        op(*op_args)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    n_py = max(10, args.steps // 4)
+    for _ in range(n_py):
+        op(*op_args)
+    torch.cuda.synchronize()
+    py_ms = (time.perf_counter() - t0) * 1e3 / n_py
+
+    tflops = flops / (ms_per_step * 1e-3) / 1e12
+    kernel_tflops = flops / (ev_ms * 1e-3) / 1e12
+    result = {
+        "metric": "HSTU attn fwd ms/batch + causal TFLOPS (% MFMA peak), B32 H4 d128 L1024 bf16",
+        "value": round(tflops, 3),
+        "unit": "TFLOP/s (causal-effective)",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{args.workload}: jagged causal HSTU attention fwd, B{len(w.lengths)} H{n_q} d{d_qk}, "
+            f"lengths {min(w.lengths)}..{max(w.lengths)} (T={sum(w.lengths)}), max_seq_len {w.max_seq_len}, "
+            f"rab={'yes' if w.attn_bias is not None else 'no'}, seed 0",
+            "flops_per_step": flops,
+            "algorithmic_bytes_per_step": alg_bytes,
+            "launch_path": "C ABI hstu_jagged_fwd, back-to-back on one stream",
+        },
+        "pct_of_bf16_mfma_peak": round(100.0 * tflops / PEAK_BF16_TFLOPS, 2),
+        "ms_per_step_events": round(ev_ms, 6),
+        "ms_per_step_wall": round(wall_ms, 6),
+        "ms_per_step_python_entry": round(py_ms, 6),
+        "roofline": {
+            "bound": "mfma",
+            "kernel": kernel_name,
+            "achieved": round(kernel_tflops, 3),
+            "peak": PEAK_BF16_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(kernel_tflops / PEAK_BF16_TFLOPS, 4),
+            "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
+            "avg_launch_us": round(ev_ms * 1e3, 3),
+            "hbm_achieved_GBs": round(alg_bytes / (ev_ms * 1e-3) / 1e9, 1),
+            "hbm_peak_GBs": PEAK_HBM_GBS,
+            "hbm_frac": round(alg_bytes / (ev_ms * 1e-3) / 1e9 / PEAK_HBM_GBS, 4),
+            "rab_read_GBs": round(rab_bytes / (ev_ms * 1e-3) / 1e9, 1) if rab_bytes else None,
+        },
+    }
+
+    # ---- CPU baseline: dense-padded fp32 golden path on this host's cores ----
+    if not args.no_cpu and w_cpu is not None:
+        cores = os.cpu_count() or 1
+        try:
+            cores = len(os.sched_getaffinity(0))
+        except AttributeError:
+            pass
+        cores = min(cores, 16)
+        torch.set_num_threads(cores)
+        kw = w_cpu.oracle_kwargs()
+        args_cpu = (w_cpu.q.float(), w_cpu.k.float(), w_cpu.v.float())
+        oracle.hstu_jagged_forward_dense(*args_cpu, **kw)  # warm-up
+        times = []
+        budget_end = time.perf_counter() + 25.0
+        while len(times) < 5 and time.perf_counter() < budget_end:
+            t0 = time.perf_counter()
+            oracle.hstu_jagged_forward_dense(*args_cpu, **kw)
+            times.append(time.perf_counter() - t0)
+        times.sort()
+        med = times[len(times) // 2]
+        t0 = time.perf_counter()
+        oracle.hstu_jagged_forward(*args_cpu, **kw)
+        per_seq = time.perf_counter() - t0
+        result["cpu_baseline"] = {
+            "value": round(flops / med / 1e12, 5),
+            "unit": "TFLOP/s (causal-effective)",
+            "cores": cores,
+            "kind": "port",
+            "sample": f"the full {args.workload} batch, dense-padded fp32 torch path, median of {len(times)} runs "
+            "after 1 warm-up",
+            "ms_per_batch": round(med * 1e3, 2),
+            "ms_per_batch_per_sequence_variant": round(per_seq * 1e3, 2),
+        }
+    print(json.dumps(result))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

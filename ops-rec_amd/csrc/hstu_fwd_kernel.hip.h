@@ -1,17 +1,26 @@
 // HSTU jagged attention forward for gfx950 (MI355X): device code.
 //
-// One workgroup (4 wavefronts) owns a 128-row query tile of one (sequence, head); each wavefront
-// owns 32 of those rows.  The wavefront keeps its Q rows in registers for the whole key sweep,
-// K and V tiles are staged in LDS (double-buffered), and
+// One workgroup owns a 128-row query tile of one (sequence, head).  Its wavefronts form a
+// 4 x NKH grid: four row groups of 32 query rows, times NKH "key lanes" that split the 32-key
+// sub-tiles of every K/V tile between them (NKH = 2: eight wavefronts, two per SIMD, which halves
+// the longest serial chain of a causal tile; their partial outputs are summed through LDS at the
+// end, in a fixed order).  A wavefront keeps its Q rows in registers for the whole key sweep,
+// K and V tiles are streamed global -> LDS by buffer loads that write LDS directly (no register
+// staging), double-buffered, and
 //
 //     S^T = K . Q^T                 v_mfma_f32_32x32x16  (A = K tile from LDS, B = Q from registers)
-//     P^T = silu(alpha * (S^T + rab^T)) * scale * mask, rounded to the input type
+//     P^T = silu(alpha * (S^T + rab^T)) * mask, rounded to the input type
 //     O^T += V^T . P^T              v_mfma_f32_32x32x16  (A = V^T via ds_read_b64_tr_b16, B = P^T)
+//     O    = (alpha * silu_scale) * O^T^T, rounded once on store
 //
 // Computing the transposed score means the accumulator layout of S^T (lane = query row, registers
 // = 4 consecutive keys) is exactly the B-operand layout the second product needs, so P never
 // leaves registers.  There is no row reduction (no softmax), every output row is produced by
-// exactly one wavefront and stored once: no atomics, bitwise deterministic.
+// one workgroup and stored once: no atomics, bitwise deterministic.
+//
+// Out-of-range rows (past the end of a sequence) are never branched on: all global accesses go
+// through buffer descriptors sized to the sequence, whose out-of-range reads return zero and
+// whose out-of-range writes are dropped.
 //
 // What this replaces in the reference (Ascend C):
 //   ascendc/attention/hstu_v1/hstu_forward_v1/op_kernel/atlas950/hstu_jagged_forward.cpp:36-62      (entry)
@@ -22,6 +31,8 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+
+#include <type_traits>
 
 namespace hstu {
 
@@ -37,7 +48,23 @@ struct f16_tag {};
 
 constexpr int kBlockM = 128;  // query rows per workgroup
 constexpr int kWaveM = 32;    // query rows per wavefront
-constexpr int kThreads = 256;
+constexpr uint32_t kBufferFlags = 0x00020000u;  // raw buffer, 32-bit data format (gfx9 family)
+constexpr uint32_t kOutOfRange = 0x80000000u;   // byte offset no descriptor here can contain
+
+// Optional per-wavefront timeline for kernel development (compile with -DHSTU_TIMELINE and pass a
+// buffer of 64 x uint64 per wavefront in FwdArgs::timeline); compiled out of the shipped library.
+#ifdef HSTU_TIMELINE
+#define HSTU_STAMP(slot)                                                                              \
+    do {                                                                                              \
+        if (a.timeline && lane == 0 && (slot) < 64)                                                   \
+            a.timeline[(static_cast<int64_t>(blockIdx.x) * NWAVES + wave) * 64 + (slot)] =            \
+                __builtin_amdgcn_s_memtime();                                                         \
+    } while (0)
+#else
+#define HSTU_STAMP(slot) \
+    do {                 \
+    } while (0)
+#endif
 
 struct FwdArgs {
     const void* q;
@@ -56,7 +83,7 @@ struct FwdArgs {
     int n_heads_q;
     int n_heads_k;
     int head_ratio;  // n_heads_q / n_heads_k
-    int d_qk;        // real head dims (<= the padded template dims)
+    int d_qk;        // real head dims (<= the padded template dim)
     int d_v;
     int max_q;
     int max_k;
@@ -65,14 +92,24 @@ struct FwdArgs {
     int idx64;       // offsets / context / target are int64
     int n_qtiles;    // ceil(max_q / kBlockM)
     int bh;          // n_batch * n_heads_q
-    int rab_vec_ok;  // rab / mask rows may be read 4 elements (8 bytes) at a time
+    int bias_vec_ok; // rab / mask rows may be read 4 elements (8 bytes) at a time
     float c_exp;     // -alpha * log2(e)
     float c_out;     // alpha * silu_scale
+#ifdef HSTU_TIMELINE
+    unsigned long long* timeline;
+#endif
 };
 
 __device__ __forceinline__ int64_t load_index(const void* p, int64_t i, int idx64)
 {
     return idx64 ? static_cast<const int64_t*>(p)[i] : static_cast<int64_t>(static_cast<const int32_t*>(p)[i]);
+}
+
+__device__ __forceinline__ int uniform(int x) { return __builtin_amdgcn_readfirstlane(x); }
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, uint32_t bytes)
+{
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(bytes), kBufferFlags);
 }
 
 // ---- type helpers -------------------------------------------------------------------------
@@ -115,16 +152,28 @@ __device__ __forceinline__ uint32_t pack2<f16_tag>(float lo, float hi)
 }
 
 template <typename Tag>
-__device__ __forceinline__ float to_float(uint16_t bits);
+__device__ __forceinline__ float lo_to_float(uint32_t packed);  // element in bits 0..15
+template <typename Tag>
+__device__ __forceinline__ float hi_to_float(uint32_t packed);  // element in bits 16..31
 template <>
-__device__ __forceinline__ float to_float<bf16_tag>(uint16_t bits)
+__device__ __forceinline__ float lo_to_float<bf16_tag>(uint32_t packed)
 {
-    return __builtin_bit_cast(float, static_cast<uint32_t>(bits) << 16);
+    return __builtin_bit_cast(float, packed << 16);
 }
 template <>
-__device__ __forceinline__ float to_float<f16_tag>(uint16_t bits)
+__device__ __forceinline__ float hi_to_float<bf16_tag>(uint32_t packed)
 {
-    return static_cast<float>(__builtin_bit_cast(_Float16, bits));
+    return __builtin_bit_cast(float, packed & 0xffff0000u);
+}
+template <>
+__device__ __forceinline__ float lo_to_float<f16_tag>(uint32_t packed)
+{
+    return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(packed & 0xffffu)));
+}
+template <>
+__device__ __forceinline__ float hi_to_float<f16_tag>(uint32_t packed)
+{
+    return static_cast<float>(__builtin_bit_cast(_Float16, static_cast<uint16_t>(packed >> 16)));
 }
 
 // ---- LDS layout ---------------------------------------------------------------------------
@@ -163,28 +212,45 @@ __device__ __forceinline__ u32x2_t lds_read_tr16_b64(const uint16_t* p)
     return __builtin_bit_cast(u32x2_t, r);
 }
 
+__device__ __forceinline__ void load_to_lds_b128(__amdgpu_buffer_rsrc_t rsrc, uint16_t* lds_wave_base, uint32_t voffset)
+{
+    // each lane's 16 bytes land at lds_wave_base + lane * 16; out-of-range sources write zeros
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rsrc, (__attribute__((address_space(3))) void*)lds_wave_base, 16,
+                                             static_cast<int>(voffset), 0, 0, 0);
+}
+
 // ---- the kernel ---------------------------------------------------------------------------
 // Tag      : bf16_tag / f16_tag
 // D        : padded head dim used for both QK and V (32, 64, 128 or 256); real dims come from args
-// BN       : keys per LDS tile (multiple of 32)
+// BN       : keys per LDS tile (multiple of 32 * NKH)
+// NKH      : key lanes (1 or 2); the workgroup has 4 * NKH wavefronts
 // HAS_RAB  : attn_bias present
-template <typename Tag, int D, int BN, bool HAS_RAB, int MIN_WAVES>
-__global__ __launch_bounds__(kThreads, MIN_WAVES) void hstu_fwd_kernel(const FwdArgs a)
+// HAS_MASK : mask_type 3 (dense custom mask multiplied in)
+template <typename Tag, int D, int BN, int NKH, bool HAS_RAB, bool HAS_MASK>
+__global__ __launch_bounds__(256 * NKH, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const FwdArgs a)
 {
-    constexpr int CPR = D / 8;                        // 16-byte chunks per row
-    constexpr int TILE_CHUNKS = BN * CPR;             // chunks per K (or V) tile
-    constexpr int LD_PER_THREAD = TILE_CHUNKS / kThreads;
-    static_assert(TILE_CHUNKS % kThreads == 0, "tile must split evenly over the workgroup");
-    constexpr int KSTEPS = D / 16;   // MFMA steps over the head dim (QK product)
-    constexpr int MTILES = D / 32;   // 32-wide output tiles over the head dim (PV product)
-    constexpr int NSUB = BN / 32;    // 32-key sub-tiles per LDS tile
+    constexpr int kThreads = 256 * NKH;
+    constexpr int NWAVES = 4 * NKH;
+    constexpr int CPR = D / 8;                       // 16-byte chunks per row
+    constexpr int TILE_ELEMS = BN * D;
+    constexpr int LOADS = TILE_ELEMS / 512 / NWAVES;  // 1 KiB load instructions per wavefront per tile
+    static_assert(TILE_ELEMS % (512 * NWAVES) == 0, "tile must split evenly over the wavefronts");
+    constexpr int KSTEPS = D / 16;  // MFMA steps over the head dim (QK product)
+    constexpr int MTILES = D / 32;  // 32-wide output tiles over the head dim (PV product)
+    constexpr int NSUB = BN / 32;   // 32-key sub-tiles per LDS tile
+    constexpr int MYSUB = NSUB / NKH;  // sub-tiles per tile handled by one wavefront (ms = kh, kh + NKH, ...)
+    static_assert(NSUB % NKH == 0 && MYSUB >= 1, "sub-tiles must split evenly over the key lanes");
 
-    __shared__ __attribute__((aligned(16))) uint16_t s_k[2][BN * D];
-    __shared__ __attribute__((aligned(16))) uint16_t s_v[2][BN * D];
+    // four separate arrays (not one block) so that the compiler can tell the buffer being filled by
+    // the asynchronous loads from the buffer being read, and does not wait for the loads early
+    __shared__ __attribute__((aligned(1024))) uint16_t s_k0[TILE_ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_k1[TILE_ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_v0[TILE_ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_v1[TILE_ELEMS];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = tid >> 6;
+    const int wave = uniform(tid >> 6);
     const int ln = lane & 31;
     const int lh = lane >> 5;
 
@@ -207,8 +273,8 @@ __global__ __launch_bounds__(kThreads, MIN_WAVES) void hstu_fwd_kernel(const Fwd
     k0 = k0 < 0 ? 0 : k0;
     int sq = static_cast<int>(q1 > q0 ? q1 - q0 : 0);
     int sk = static_cast<int>(k1 > k0 ? k1 - k0 : 0);
-    sq = sq < a.max_q ? sq : a.max_q;
-    sk = sk < a.max_k ? sk : a.max_k;
+    sq = uniform(sq < a.max_q ? sq : a.max_q);
+    sk = uniform(sk < a.max_k ? sk : a.max_k);
 
     uint16_t* const out16 = static_cast<uint16_t*>(a.out);
 
@@ -229,8 +295,11 @@ __global__ __launch_bounds__(kThreads, MIN_WAVES) void hstu_fwd_kernel(const Fwd
     if (r0 >= sq) {
         return;
     }
-    const int wr0 = r0 + wave * kWaveM;
-    const bool wave_active = wr0 < sq;  // inactive wavefronts still help with loads and barriers
+    HSTU_STAMP(0);
+    const int row_group = wave & 3;
+    const int kh = wave >> 2;  // key lane
+    const int wr0 = r0 + row_group * kWaveM;
+    const bool wave_active = wr0 < sq;  // inactive wavefronts still take part in loads and barriers
 
     int n_ctx = 0;
     int n_tgt = 0;
@@ -241,8 +310,8 @@ __global__ __launch_bounds__(kThreads, MIN_WAVES) void hstu_fwd_kernel(const Fwd
         if (a.num_tgt) {
             n_tgt = static_cast<int>(load_index(a.num_tgt, b, a.idx64));
         }
-        n_ctx = n_ctx < 0 ? 0 : n_ctx;
-        n_tgt = n_tgt < 0 ? 0 : (n_tgt > sk ? sk : n_tgt);
+        n_ctx = uniform(n_ctx < 0 ? 0 : n_ctx);
+        n_tgt = uniform(n_tgt < 0 ? 0 : (n_tgt > sk ? sk : n_tgt));
     }
     const int delta = sk - sq;
     const int hist_k = sk - n_tgt;  // keys before the target block
@@ -250,7 +319,6 @@ __global__ __launch_bounds__(kThreads, MIN_WAVES) void hstu_fwd_kernel(const Fwd
     // ---- per-row visibility constants (row = this lane's query row, clamped into the sequence) ----
     //   visible(j) = j < lim  &&  !(hole_lo <= j < hole_hi)
     int row = wr0 + ln;
-    const bool row_valid = row < sq;
     {
         const int last_row = sq - 1;
         row = row < last_row ? row : last_row;
@@ -287,6 +355,9 @@ __global__ __launch_bounds__(kThreads, MIN_WAVES) void hstu_fwd_kernel(const Fwd
         lim_max = o_max > lim_max ? o_max : lim_max;
         hole_hi_max = o_hh > hole_hi_max ? o_hh : hole_hi_max;
     }
+    lim_min = uniform(lim_min);
+    lim_max = uniform(wave_active ? lim_max : 0);
+    hole_hi_max = uniform(hole_hi_max);
     const bool any_hole = hole_hi_max > hist_k && n_tgt > 0 && a.target_group > 0;
 
     // ---- keys needed by this workgroup ----
@@ -301,23 +372,94 @@ __global__ __launch_bounds__(kThreads, MIN_WAVES) void hstu_fwd_kernel(const Fwd
     } else {
         kmax = sk;
     }
-    const int n_kt = (kmax + BN - 1) / BN;
+    const int n_kt = uniform((kmax + BN - 1) / BN);
+
+    // ---- buffer descriptors sized to this sequence / head ----
+    const uint32_t q_stride = static_cast<uint32_t>(a.n_heads_q) * a.d_qk * 2u;  // bytes per row
+    const uint32_t k_stride = static_cast<uint32_t>(a.n_heads_k) * a.d_qk * 2u;
+    const uint32_t v_stride = static_cast<uint32_t>(a.n_heads_k) * a.d_v * 2u;
+    const uint32_t o_stride = static_cast<uint32_t>(a.n_heads_q) * a.d_v * 2u;
+    const __amdgpu_buffer_rsrc_t q_rsrc =
+        make_rsrc(static_cast<const uint16_t*>(a.q) + (q0 * a.n_heads_q + h) * static_cast<int64_t>(a.d_qk),
+                  static_cast<uint32_t>(sq - 1) * q_stride + a.d_qk * 2u);
+    const __amdgpu_buffer_rsrc_t k_rsrc =
+        make_rsrc(static_cast<const uint16_t*>(a.k) + (k0 * a.n_heads_k + hk) * static_cast<int64_t>(a.d_qk),
+                  sk > 0 ? static_cast<uint32_t>(sk - 1) * k_stride + a.d_qk * 2u : 0u);
+    const __amdgpu_buffer_rsrc_t v_rsrc =
+        make_rsrc(static_cast<const uint16_t*>(a.v) + (k0 * a.n_heads_k + hk) * static_cast<int64_t>(a.d_v),
+                  sk > 0 ? static_cast<uint32_t>(sk - 1) * v_stride + a.d_v * 2u : 0u);
+    const __amdgpu_buffer_rsrc_t o_rsrc =
+        make_rsrc(out16 + (q0 * a.n_heads_q + h) * static_cast<int64_t>(a.d_v),
+                  static_cast<uint32_t>(sq - 1) * o_stride + a.d_v * 2u);
 
     // ---- Q fragment: lane (ln, lh) holds Q[row][16*js + 8*lh .. +7] for js = 0..KSTEPS-1 ----
     u32x4_t qf[KSTEPS];
     {
-        const uint16_t* qrow = static_cast<const uint16_t*>(a.q) +
-                               ((q0 + wr0 + ln) * a.n_heads_q + h) * static_cast<int64_t>(a.d_qk);
+        const uint32_t row_off = static_cast<uint32_t>(wr0 + ln) * q_stride;
 #pragma unroll
         for (int js = 0; js < KSTEPS; ++js) {
             const int d0 = 16 * js + 8 * lh;
-            u32x4_t val = {0u, 0u, 0u, 0u};
-            if (row_valid && d0 < a.d_qk) {
-                val = *reinterpret_cast<const u32x4_t*>(qrow + d0);
-            }
-            qf[js] = val;
+            const uint32_t off = (d0 < a.d_qk) ? row_off + d0 * 2u : kOutOfRange;
+            qf[js] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, static_cast<int>(off), 0, 0);
         }
     }
+
+    // ---- K / V tile streaming: per-lane source offsets are fixed, only the tile base moves ----
+    // load instruction i of this wavefront fills LDS bytes [(wave * LOADS + i) * 1024, +1024)
+    uint32_t k_src[LOADS];
+    uint32_t v_src[LOADS];
+#pragma unroll
+    for (int i = 0; i < LOADS; ++i) {
+        const int slot = (wave * LOADS + i) * 64 + lane;  // 16-byte slot within the tile
+        const int r = slot / CPR;
+        const int pc = slot - r * CPR;
+        const int kc = k_chunk_swizzle<D>(r, pc);  // XOR swizzles are their own inverse
+        const int vc = v_chunk_swizzle<D>(r, pc);
+        k_src[i] = (kc * 8 < a.d_qk) ? static_cast<uint32_t>(r) * k_stride + kc * 16u : kOutOfRange;
+        v_src[i] = (vc * 8 < a.d_v) ? static_cast<uint32_t>(r) * v_stride + vc * 16u : kOutOfRange;
+    }
+    auto issue_tile = [&](int kt, uint16_t* dst_k, uint16_t* dst_v) {
+        const uint32_t kb = static_cast<uint32_t>(kt * BN) * k_stride;
+        const uint32_t vb = static_cast<uint32_t>(kt * BN) * v_stride;
+#pragma unroll
+        for (int i = 0; i < LOADS; ++i) {
+            uint16_t* wk = dst_k + (wave * LOADS + i) * 512;
+            uint16_t* wv = dst_v + (wave * LOADS + i) * 512;
+            // kOutOfRange + tile base stays out of range: tile bases are far below 2^31
+            load_to_lds_b128(k_rsrc, wk, k_src[i] + kb);
+            load_to_lds_b128(v_rsrc, wv, v_src[i] + vb);
+        }
+    };
+
+    // ---- rab / custom mask: per (sequence, head) descriptor, rows indexed by the local (i, j) ----
+    const uint32_t bias_bytes = static_cast<uint32_t>(a.max_q) * static_cast<uint32_t>(a.max_k) * 2u;
+    const int64_t bias_plane = (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k);
+    const __amdgpu_buffer_rsrc_t rab_rsrc =
+        make_rsrc(HAS_RAB ? static_cast<const uint16_t*>(a.rab) + bias_plane : nullptr, HAS_RAB ? bias_bytes : 0u);
+    const __amdgpu_buffer_rsrc_t mask_rsrc =
+        make_rsrc(HAS_MASK ? static_cast<const uint16_t*>(a.mask) + bias_plane : nullptr, HAS_MASK ? bias_bytes : 0u);
+    const uint32_t bias_row_off = static_cast<uint32_t>(wr0 + ln) * static_cast<uint32_t>(a.max_k) * 2u;
+    const bool bias_vec = a.bias_vec_ok != 0;
+
+    // loads the 16 bias (or mask) values of one 32-key sub-tile in accumulator order, as 8 packed words
+    auto load_bias = [&](__amdgpu_buffer_rsrc_t rsrc, int c0, uint32_t (&w)[8]) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const uint32_t off = bias_row_off + static_cast<uint32_t>(c0 + 8 * g + 4 * lh) * 2u;
+            if (bias_vec) {
+                const u32x2_t t = __builtin_amdgcn_raw_buffer_load_b64(rsrc, static_cast<int>(off), 0, 0);
+                w[2 * g + 0] = t[0];
+                w[2 * g + 1] = t[1];
+            } else {
+                const uint32_t e0 = __builtin_amdgcn_raw_buffer_load_b16(rsrc, static_cast<int>(off), 0, 0);
+                const uint32_t e1 = __builtin_amdgcn_raw_buffer_load_b16(rsrc, static_cast<int>(off + 2u), 0, 0);
+                const uint32_t e2 = __builtin_amdgcn_raw_buffer_load_b16(rsrc, static_cast<int>(off + 4u), 0, 0);
+                const uint32_t e3 = __builtin_amdgcn_raw_buffer_load_b16(rsrc, static_cast<int>(off + 6u), 0, 0);
+                w[2 * g + 0] = (e0 & 0xffffu) | (e1 << 16);
+                w[2 * g + 1] = (e2 & 0xffffu) | (e3 << 16);
+            }
+        }
+    };
 
     f32x16_t o_acc[MTILES];
 #pragma unroll
@@ -328,197 +470,351 @@ __global__ __launch_bounds__(kThreads, MIN_WAVES) void hstu_fwd_kernel(const Fwd
         }
     }
 
-    // ---- K/V tile movement: global -> registers -> LDS ----
-    const uint16_t* const kbase = static_cast<const uint16_t*>(a.k);
-    const uint16_t* const vbase = static_cast<const uint16_t*>(a.v);
-    const int64_t k_row_stride = static_cast<int64_t>(a.n_heads_k) * a.d_qk;
-    const int64_t v_row_stride = static_cast<int64_t>(a.n_heads_k) * a.d_v;
-    u32x4_t k_stage[LD_PER_THREAD];
-    u32x4_t v_stage[LD_PER_THREAD];
+    const float c_exp = a.c_exp;
 
-    auto load_tile = [&](int kt) {
+    // ---- per-lane LDS read offsets (in elements, relative to a tile), fixed for the whole kernel;
+    //      sub-tile / MFMA-step / buffer displacements are compile-time constants on top of them
+    //      (the swizzles only look at row bits that such displacements leave unchanged) ----
+    int k_lane_off[KSTEPS];
 #pragma unroll
-        for (int i = 0; i < LD_PER_THREAD; ++i) {
-            const int idx = tid + i * kThreads;
-            const int r = idx / CPR;
-            const int c = idx - r * CPR;
-            const int key = kt * BN + r;
-            u32x4_t kv = {0u, 0u, 0u, 0u};
-            u32x4_t vv = {0u, 0u, 0u, 0u};
-            if (key < sk) {
-                if (c * 8 < a.d_qk) {
-                    kv = *reinterpret_cast<const u32x4_t*>(kbase + (k0 + key) * k_row_stride +
-                                                           static_cast<int64_t>(hk) * a.d_qk + c * 8);
-                }
-                if (c * 8 < a.d_v) {
-                    vv = *reinterpret_cast<const u32x4_t*>(vbase + (k0 + key) * v_row_stride +
-                                                           static_cast<int64_t>(hk) * a.d_v + c * 8);
-                }
-            }
-            k_stage[i] = kv;
-            v_stage[i] = vv;
-        }
-    };
-    auto store_tile = [&](int buf) {
-#pragma unroll
-        for (int i = 0; i < LD_PER_THREAD; ++i) {
-            const int idx = tid + i * kThreads;
-            const int r = idx / CPR;
-            const int c = idx - r * CPR;
-            *reinterpret_cast<u32x4_t*>(&s_k[buf][r * D + k_chunk_swizzle<D>(r, c) * 8]) = k_stage[i];
-            *reinterpret_cast<u32x4_t*>(&s_v[buf][r * D + v_chunk_swizzle<D>(r, c) * 8]) = v_stage[i];
-        }
-    };
-
-    const uint16_t* const rab16 = static_cast<const uint16_t*>(a.rab);
-    const uint16_t* const mask16 = static_cast<const uint16_t*>(a.mask);
-    const int64_t bias_row =
-        ((static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q + (wr0 + ln)) * static_cast<int64_t>(a.max_k);
-    const bool use_custom_mask = (a.mask_type == 3);
-
-    if (n_kt > 0) {
-        load_tile(0);
-        store_tile(0);
+    for (int js = 0; js < KSTEPS; ++js) {
+        k_lane_off[js] = ln * D + k_chunk_swizzle<D>(ln, 2 * js + lh) * 8;
     }
-    __syncthreads();
-
-    for (int kt = 0; kt < n_kt; ++kt) {
-        const int buf = kt & 1;
-        const bool has_next = kt + 1 < n_kt;
-        if (has_next) {
-            load_tile(kt + 1);
+    int v_lane_off[MTILES];
+    {
+        const int vr0 = 4 * lh + ((lane & 15) >> 2);
+#pragma unroll
+        for (int mt = 0; mt < MTILES; ++mt) {
+            const int col = 32 * mt + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+            v_lane_off[mt] = vr0 * D + v_chunk_swizzle<D>(vr0, col >> 3) * 8 + (col & 7);
         }
+    }
 
-        if (wave_active) {
+    // one MFMA step of S^T for sub-tile ms
+    auto qk_step = [&](const uint16_t* k_tile, int ms, int js, f32x16_t acc) -> f32x16_t {
+        const u32x4_t ka = *reinterpret_cast<const u32x4_t*>(k_tile + k_lane_off[js] + ms * 32 * D);
+        return mfma32<Tag>(ka, qf[js], acc);
+    };
+    // one MFMA of O^T += V^T . P^T : keys 16*j2 .. 16*j2+15 of sub-tile ms, output dims 32*mt .. +31
+    auto pv_step = [&](const uint16_t* v_tile, int ms, int j2, int mt, const uint32_t (&pk)[8]) {
+        const u32x4_t pb = {pk[4 * j2 + 0], pk[4 * j2 + 1], pk[4 * j2 + 2], pk[4 * j2 + 3]};
+        const uint16_t* p = v_tile + v_lane_off[mt] + (ms * 32 + 16 * j2) * D;
+        const u32x2_t lo = lds_read_tr16_b64(p);
+        const u32x2_t hi = lds_read_tr16_b64(p + 8 * D);
+        const u32x4_t va = {lo[0], lo[1], hi[0], hi[1]};
+        o_acc[mt] = mfma32<Tag>(va, pb, o_acc[mt]);
+    };
+    // unscaled P^T = S^T * sigmoid(alpha * S^T) for keys 8g + 4lh + 0..3 of this lane's row, packed
+    auto silu_group = [&](const f32x16_t& s, int g, uint32_t (&pk)[8]) {
+        float p[4];
 #pragma unroll
-            for (int ms = 0; ms < NSUB; ++ms) {
-                const int c0 = kt * BN + ms * 32;  // first key of this 32-key sub-tile
-                if (c0 >= lim_max) {
-                    continue;  // no row of this wavefront sees any of these keys
-                }
-                // ---- S^T = K . Q^T (+ rab^T) ----
-                f32x16_t s_acc;
-                if constexpr (HAS_RAB) {
+        for (int e = 0; e < 4; ++e) {
+            const float sv = s[4 * g + e];
+            const float ex = __builtin_amdgcn_exp2f(sv * c_exp);
+            p[e] = sv * __builtin_amdgcn_rcpf(1.0f + ex);
+        }
+        pk[2 * g + 0] = pack2<Tag>(p[0], p[1]);
+        pk[2 * g + 1] = pack2<Tag>(p[2], p[3]);
+    };
+    auto init_scores = [&](int c0, f32x16_t& s) {
+        if constexpr (HAS_RAB) {
+            uint32_t w[8];
+            load_bias(rab_rsrc, c0, w);
 #pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        const int j = c0 + 8 * g + 4 * lh;
-                        float b0 = 0.f, b1 = 0.f, b2 = 0.f, b3 = 0.f;
-                        if (row_valid) {
-                            const uint16_t* p = rab16 + bias_row + j;
-                            if (a.rab_vec_ok && j + 3 < sk) {
-                                const u32x2_t w = *reinterpret_cast<const u32x2_t*>(p);
-                                b0 = to_float<Tag>(static_cast<uint16_t>(w[0] & 0xffffu));
-                                b1 = to_float<Tag>(static_cast<uint16_t>(w[0] >> 16));
-                                b2 = to_float<Tag>(static_cast<uint16_t>(w[1] & 0xffffu));
-                                b3 = to_float<Tag>(static_cast<uint16_t>(w[1] >> 16));
-                            } else {
-                                if (j + 0 < sk) b0 = to_float<Tag>(p[0]);
-                                if (j + 1 < sk) b1 = to_float<Tag>(p[1]);
-                                if (j + 2 < sk) b2 = to_float<Tag>(p[2]);
-                                if (j + 3 < sk) b3 = to_float<Tag>(p[3]);
-                            }
-                        }
-                        s_acc[4 * g + 0] = b0;
-                        s_acc[4 * g + 1] = b1;
-                        s_acc[4 * g + 2] = b2;
-                        s_acc[4 * g + 3] = b3;
+            for (int i = 0; i < 8; ++i) {
+                s[2 * i + 0] = lo_to_float<Tag>(w[i]);
+                s[2 * i + 1] = hi_to_float<Tag>(w[i]);
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                s[i] = 0.f;
+            }
+        }
+    };
+
+    // one LDS tile, for this wavefront: its sub-tiles are ms = kh, kh + NKH, ...
+    auto compute_tile = [&](auto buf_const, int kt) {
+        constexpr int BUF = decltype(buf_const)::value;
+        const uint16_t* const k_tile = BUF ? s_k1 : s_k0;
+        const uint16_t* const v_tile = BUF ? s_v1 : s_v0;
+        const int cbeg = kt * BN;
+        if (cbeg + kh * 32 >= lim_max) {
+            return;  // no row of this wavefront sees any key of its sub-tiles
+        }
+        const bool tile_full = !HAS_MASK && (cbeg + BN <= lim_min) &&
+                               !(any_hole && cbeg + BN > hist_k && cbeg < hole_hi_max);
+        if (tile_full) {
+            // Fast path: every element of every sub-tile is visible.
+            if constexpr (MYSUB == 2) {
+                // Two sub-tiles (a, b) per wavefront, issued as four stages of NCH chunks.  A chunk is
+                // one MFMA plus the LDS operand reads of a later chunk plus a slice of SiLU work, and
+                // chunks are fenced so that the order below is the order issued:
+                //   A: QK(a)            + reads K(b)
+                //   B: QK(b) + silu(a)  + reads V(a)
+                //   C: PV(a) + silu(b)  + reads V(b)
+                //   D: PV(b)
+                // so the matrix pipe always has an MFMA in flight while the SiLU arithmetic runs.
+                static_assert(KSTEPS == 2 * MTILES, "QK and PV stages must have the same number of MFMAs");
+                constexpr int NCH = KSTEPS;        // chunks (= MFMAs) per stage
+                constexpr int EPC = 16 / NCH;      // score elements handled per chunk
+                static_assert(NCH * EPC == 16 && EPC % 2 == 0, "chunks must cover packed pairs");
+                const int ms_a = kh;
+                const int ms_b = kh + NKH;
+                f32x16_t s_a, s_b;
+                init_scores(cbeg + ms_a * 32, s_a);
+                init_scores(cbeg + ms_b * 32, s_b);
+                uint32_t pk_a[8], pk_b[8];
+                auto read_k = [&](int ms, int js) -> u32x4_t {
+                    return *reinterpret_cast<const u32x4_t*>(k_tile + k_lane_off[js] + ms * 32 * D);
+                };
+                auto read_v = [&](int ms, int t) -> u32x4_t {
+                    const int j2 = t / MTILES, mt = t % MTILES;
+                    const uint16_t* p = v_tile + v_lane_off[mt] + (ms * 32 + 16 * j2) * D;
+                    const u32x2_t lo = lds_read_tr16_b64(p);
+                    const u32x2_t hi = lds_read_tr16_b64(p + 8 * D);
+                    const u32x4_t r = {lo[0], lo[1], hi[0], hi[1]};
+                    return r;
+                };
+                // LDS operand of chunk c (0 .. 4 * NCH - 1), read LOOKAHEAD chunks before its MFMA
+                auto read_operand = [&](int c) -> u32x4_t {
+                    const int stage = c / NCH, i = c % NCH;
+                    return stage == 0 ? read_k(ms_a, i)
+                           : stage == 1 ? read_k(ms_b, i)
+                           : stage == 2 ? read_v(ms_a, i)
+                                        : read_v(ms_b, i);
+                };
+                auto silu_chunk = [&](const f32x16_t& sc, int i, uint32_t (&pk)[8]) {
+                    float t[EPC], p[EPC];
+#pragma unroll
+                    for (int e = 0; e < EPC; ++e) {
+                        t[e] = sc[i * EPC + e] * c_exp;
                     }
-                } else {
 #pragma unroll
-                    for (int i = 0; i < 16; ++i) {
-                        s_acc[i] = 0.f;
+                    for (int e = 0; e < EPC; ++e) {
+                        t[e] = __builtin_amdgcn_exp2f(t[e]);
                     }
+#pragma unroll
+                    for (int e = 0; e < EPC; ++e) {
+                        t[e] = 1.0f + t[e];
+                    }
+#pragma unroll
+                    for (int e = 0; e < EPC; ++e) {
+                        t[e] = __builtin_amdgcn_rcpf(t[e]);
+                    }
+#pragma unroll
+                    for (int e = 0; e < EPC; ++e) {
+                        p[e] = sc[i * EPC + e] * t[e];
+                    }
+#pragma unroll
+                    for (int e = 0; e < EPC; e += 2) {
+                        pk[(i * EPC + e) / 2] = pack2<Tag>(p[e], p[e + 1]);
+                    }
+                };
+                constexpr int LOOKAHEAD = 3;
+                u32x4_t opnd[4 * NCH];
+#pragma unroll
+                for (int c = 0; c < LOOKAHEAD; ++c) {
+                    opnd[c] = read_operand(c);
                 }
-                {
-                    const int kr = ms * 32 + ln;
-                    const uint16_t* krow = &s_k[buf][kr * D];
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int c = 0; c < 4 * NCH; ++c) {
+                    const int stage = c / NCH, i = c % NCH;
+                    const int j2 = i / MTILES, mt = i % MTILES;
+                    if (stage == 0) {
+                        s_a = mfma32<Tag>(opnd[c], qf[i], s_a);
+                    } else if (stage == 1) {
+                        s_b = mfma32<Tag>(opnd[c], qf[i], s_b);
+                    } else if (stage == 2) {
+                        const u32x4_t pb = {pk_a[4 * j2 + 0], pk_a[4 * j2 + 1], pk_a[4 * j2 + 2], pk_a[4 * j2 + 3]};
+                        o_acc[mt] = mfma32<Tag>(opnd[c], pb, o_acc[mt]);
+                    } else {
+                        const u32x4_t pb = {pk_b[4 * j2 + 0], pk_b[4 * j2 + 1], pk_b[4 * j2 + 2], pk_b[4 * j2 + 3]};
+                        o_acc[mt] = mfma32<Tag>(opnd[c], pb, o_acc[mt]);
+                    }
+                    if (c + LOOKAHEAD < 4 * NCH) {
+                        opnd[c + LOOKAHEAD] = read_operand(c + LOOKAHEAD);
+                    }
+                    if (stage == 1) {
+                        silu_chunk(s_a, i, pk_a);
+                    } else if (stage == 2) {
+                        silu_chunk(s_b, i, pk_b);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else {
+                f32x16_t s[MYSUB];
+                uint32_t pk[MYSUB][8];
+#pragma unroll
+                for (int u = 0; u < MYSUB; ++u) {
+                    init_scores(cbeg + (kh + u * NKH) * 32, s[u]);
+                }
+#pragma unroll
+                for (int u = 0; u < MYSUB; ++u) {
 #pragma unroll
                     for (int js = 0; js < KSTEPS; ++js) {
-                        const u32x4_t ka =
-                            *reinterpret_cast<const u32x4_t*>(krow + k_chunk_swizzle<D>(kr, 2 * js + lh) * 8);
-                        s_acc = mfma32<Tag>(ka, qf[js], s_acc);
+                        s[u] = qk_step(k_tile, kh + u * NKH, js, s[u]);
                     }
                 }
-                // ---- P^T = silu(alpha * S^T) * scale, masked, rounded to the input type ----
-                const bool full = (c0 + 32 <= lim_min) && !(any_hole && c0 + 32 > hist_k && c0 < hole_hi_max) &&
-                                  !use_custom_mask;
-                uint32_t pk[8];
 #pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    float p[4];
+                for (int u = 0; u < MYSUB; ++u) {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const float s = s_acc[4 * g + e];
-                        const float ex = __builtin_amdgcn_exp2f(s * a.c_exp);
-                        p[e] = (s * a.c_out) * __builtin_amdgcn_rcpf(1.0f + ex);
+                    for (int g = 0; g < 4; ++g) {
+                        silu_group(s[u], g, pk[u]);
                     }
-                    if (!full) {
-                        const int j = c0 + 8 * g + 4 * lh;
 #pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            const int jj = j + e;
-                            const bool vis = (jj < lim) && !(jj >= hole_lo && jj < hole_hi);
-                            p[e] = vis ? p[e] : 0.f;
-                        }
-                        if (use_custom_mask) {
-#pragma unroll
-                            for (int e = 0; e < 4; ++e) {
-                                const int jj = j + e;
-                                float m = 0.f;
-                                if (row_valid && jj < sk) {
-                                    m = to_float<Tag>(mask16[bias_row + jj]);
-                                }
-                                p[e] *= m;
-                            }
-                        }
-                    }
-                    pk[2 * g + 0] = pack2<Tag>(p[0], p[1]);
-                    pk[2 * g + 1] = pack2<Tag>(p[2], p[3]);
-                }
-                // ---- O^T += V^T . P^T ----
-#pragma unroll
-                for (int j2 = 0; j2 < 2; ++j2) {
-                    const u32x4_t pb = {pk[4 * j2 + 0], pk[4 * j2 + 1], pk[4 * j2 + 2], pk[4 * j2 + 3]};
-                    const int vr = ms * 32 + 16 * j2 + 4 * lh + ((lane & 15) >> 2);
-#pragma unroll
-                    for (int mt = 0; mt < MTILES; ++mt) {
-                        const int col = 32 * mt + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-                        const int ch = col >> 3;
-                        const int within = col & 7;
-                        const u32x2_t lo = lds_read_tr16_b64(
-                            &s_v[buf][vr * D + v_chunk_swizzle<D>(vr, ch) * 8 + within]);
-                        const u32x2_t hi = lds_read_tr16_b64(
-                            &s_v[buf][(vr + 8) * D + v_chunk_swizzle<D>(vr + 8, ch) * 8 + within]);
-                        const u32x4_t va = {lo[0], lo[1], hi[0], hi[1]};
-                        o_acc[mt] = mfma32<Tag>(va, pb, o_acc[mt]);
+                    for (int t = 0; t < 2 * MTILES; ++t) {
+                        pv_step(v_tile, kh + u * NKH, t / MTILES, t % MTILES, pk[u]);
                     }
                 }
             }
+            return;
         }
+        // general path: per sub-tile skip / mask
+        for (int ms = kh; ms < NSUB; ms += NKH) {
+            const int c0 = cbeg + ms * 32;
+            if (c0 >= lim_max) {
+                break;
+            }
+            f32x16_t s;
+            init_scores(c0, s);
+            uint32_t mw[8];
+            if constexpr (HAS_MASK) {
+                load_bias(mask_rsrc, c0, mw);
+            }
+#pragma unroll
+            for (int js = 0; js < KSTEPS; ++js) {
+                s = qk_step(k_tile, ms, js, s);
+            }
+            uint32_t pk[8];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                float p[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float sv = s[4 * g + e];
+                    const float ex = __builtin_amdgcn_exp2f(sv * c_exp);
+                    p[e] = sv * __builtin_amdgcn_rcpf(1.0f + ex);
+                }
+                const int j = c0 + 8 * g + 4 * lh;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int jj = j + e;
+                    const bool vis = (jj < lim) && !(jj >= hole_lo && jj < hole_hi);
+                    p[e] = vis ? p[e] : 0.f;
+                }
+                if constexpr (HAS_MASK) {
+                    p[0] *= lo_to_float<Tag>(mw[2 * g + 0]);
+                    p[1] *= hi_to_float<Tag>(mw[2 * g + 0]);
+                    p[2] *= lo_to_float<Tag>(mw[2 * g + 1]);
+                    p[3] *= hi_to_float<Tag>(mw[2 * g + 1]);
+                    // a masked-out element must stay exactly zero even if the mask word is garbage
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        p[e] = (j + e < lim) ? p[e] : 0.f;
+                    }
+                }
+                pk[2 * g + 0] = pack2<Tag>(p[0], p[1]);
+                pk[2 * g + 1] = pack2<Tag>(p[2], p[3]);
+            }
+#pragma unroll
+            for (int t = 0; t < 2 * MTILES; ++t) {
+                pv_step(v_tile, ms, t / MTILES, t % MTILES, pk);
+            }
+        }
+    };
 
-        if (has_next) {
-            store_tile(buf ^ 1);
+    // ---- main loop, two tiles per trip so that the LDS buffer of each half is a constant ----
+    typedef std::integral_constant<int, 0> buf0_t;
+    typedef std::integral_constant<int, 1> buf1_t;
+    HSTU_STAMP(1);
+    if (n_kt > 0) {
+        issue_tile(0, s_k0, s_v0);
+    }
+    __builtin_amdgcn_s_waitcnt(0);
+    HSTU_STAMP(2);
+    __syncthreads();
+    HSTU_STAMP(3);
+    for (int kt = 0; kt < n_kt; kt += 2) {
+        if (kt + 1 < n_kt) {
+            issue_tile(kt + 1, s_k1, s_v1);
+        }
+        compute_tile(buf0_t{}, kt);
+        HSTU_STAMP(4 + 3 * kt);
+        __builtin_amdgcn_s_waitcnt(0);
+        HSTU_STAMP(5 + 3 * kt);
+        __syncthreads();
+        HSTU_STAMP(6 + 3 * kt);
+        if (kt + 1 >= n_kt) {
+            break;
+        }
+        if (kt + 2 < n_kt) {
+            issue_tile(kt + 2, s_k0, s_v0);
+        }
+        compute_tile(buf1_t{}, kt + 1);
+        HSTU_STAMP(7 + 3 * kt);
+        __builtin_amdgcn_s_waitcnt(0);
+        HSTU_STAMP(8 + 3 * kt);
+        __syncthreads();
+        HSTU_STAMP(9 + 3 * kt);
+    }
+
+    // ---- sum the partial outputs of the key lanes: lane kh = 1 hands its accumulators to lane 0
+    //      through LDS (the K/V buffers are free now), always added in the same order ----
+    if constexpr (NKH == 2) {
+        // slot (row group, i) holds one float4 per lane: conflict-free 16-byte accesses;
+        // row groups 0, 1 exchange through the first K buffer, 2, 3 through the second
+        static_assert(2 * MTILES * 4 * 64 * 16 <= TILE_ELEMS * 2, "exchange area too small");
+        float* xch = reinterpret_cast<float*>(row_group < 2 ? s_k0 : s_k1);
+        if (kh == 1) {
+#pragma unroll
+            for (int mt = 0; mt < MTILES; ++mt) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int slot = ((row_group & 1) * MTILES + mt) * 4 + g;
+                    float4 t = make_float4(o_acc[mt][4 * g + 0], o_acc[mt][4 * g + 1], o_acc[mt][4 * g + 2],
+                                           o_acc[mt][4 * g + 3]);
+                    *reinterpret_cast<float4*>(xch + (slot * 64 + lane) * 4) = t;
+                }
+            }
         }
         __syncthreads();
+        if (kh == 1) {
+            return;
+        }
+#pragma unroll
+        for (int mt = 0; mt < MTILES; ++mt) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int slot = ((row_group & 1) * MTILES + mt) * 4 + g;
+                const float4 t = *reinterpret_cast<const float4*>(xch + (slot * 64 + lane) * 4);
+                o_acc[mt][4 * g + 0] += t.x;
+                o_acc[mt][4 * g + 1] += t.y;
+                o_acc[mt][4 * g + 2] += t.z;
+                o_acc[mt][4 * g + 3] += t.w;
+            }
+        }
     }
 
     // ---- store O: lane holds query row (wr0 + ln), dims 32*mt + 8*g + 4*lh + 0..3 ----
-    if (row_valid) {
-        uint16_t* orow = out16 + ((q0 + wr0 + ln) * a.n_heads_q + h) * static_cast<int64_t>(a.d_v);
+    {
+        const float c_out = a.c_out;
+        const uint32_t row_off = static_cast<uint32_t>(wr0 + ln) * o_stride;
 #pragma unroll
         for (int mt = 0; mt < MTILES; ++mt) {
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 const int d0 = 32 * mt + 8 * g + 4 * lh;
-                if (d0 < a.d_v) {
-                    u32x2_t w;
-                    w[0] = pack2<Tag>(o_acc[mt][4 * g + 0], o_acc[mt][4 * g + 1]);
-                    w[1] = pack2<Tag>(o_acc[mt][4 * g + 2], o_acc[mt][4 * g + 3]);
-                    *reinterpret_cast<u32x2_t*>(orow + d0) = w;
-                }
+                const uint32_t off = (d0 < a.d_v) ? row_off + d0 * 2u : kOutOfRange;
+                u32x2_t w;
+                w[0] = pack2<Tag>(o_acc[mt][4 * g + 0] * c_out, o_acc[mt][4 * g + 1] * c_out);
+                w[1] = pack2<Tag>(o_acc[mt][4 * g + 2] * c_out, o_acc[mt][4 * g + 3] * c_out);
+                __builtin_amdgcn_raw_buffer_store_b64(w, o_rsrc, static_cast<int>(off), 0, 0);
             }
         }
     }
+    HSTU_STAMP(63);
 }
 
 }  // namespace hstu

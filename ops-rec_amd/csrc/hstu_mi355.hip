@@ -32,21 +32,22 @@ struct Variant {
     const char* name;
     void (*kernel)(const hstu::FwdArgs);
     int d_pad;
+    int threads;
 };
 
-#define HSTU_VARIANT(tag, tagname, D, BN, RAB, MINW)                                                   \
-    {"hstu_fwd_" tagname "_d" #D "_bn" #BN "_rab" #RAB, hstu::hstu_fwd_kernel<hstu::tag, D, BN, RAB, MINW>, D}
+#define HSTU_VARIANT(tag, tagname, D, BN, NKH, RAB, MASK)                                             \
+    {"hstu_fwd_" tagname "_d" #D "_bn" #BN "_kl" #NKH "_rab" #RAB "_mask" #MASK,                       \
+     hstu::hstu_fwd_kernel<hstu::tag, D, BN, NKH, RAB, MASK>, D, 256 * NKH}
+#define HSTU_DIMS(tag, tagname, RAB, MASK)                                                               \
+    {HSTU_VARIANT(tag, tagname, 32, 64, 1, RAB, MASK), HSTU_VARIANT(tag, tagname, 64, 64, 1, RAB, MASK), \
+     HSTU_VARIANT(tag, tagname, 128, 64, 1, RAB, MASK), HSTU_VARIANT(tag, tagname, 256, 32, 1, RAB, MASK)}
 
-// [dtype: bf16, f16][rab: 0, 1][dim slot: 32, 64, 128, 256]
-const Variant kVariants[2][2][4] = {
-    {{HSTU_VARIANT(bf16_tag, "bf16", 32, 64, false, 2), HSTU_VARIANT(bf16_tag, "bf16", 64, 64, false, 2),
-      HSTU_VARIANT(bf16_tag, "bf16", 128, 64, false, 2), HSTU_VARIANT(bf16_tag, "bf16", 256, 32, false, 1)},
-     {HSTU_VARIANT(bf16_tag, "bf16", 32, 64, true, 2), HSTU_VARIANT(bf16_tag, "bf16", 64, 64, true, 2),
-      HSTU_VARIANT(bf16_tag, "bf16", 128, 64, true, 2), HSTU_VARIANT(bf16_tag, "bf16", 256, 32, true, 1)}},
-    {{HSTU_VARIANT(f16_tag, "f16", 32, 64, false, 2), HSTU_VARIANT(f16_tag, "f16", 64, 64, false, 2),
-      HSTU_VARIANT(f16_tag, "f16", 128, 64, false, 2), HSTU_VARIANT(f16_tag, "f16", 256, 32, false, 1)},
-     {HSTU_VARIANT(f16_tag, "f16", 32, 64, true, 2), HSTU_VARIANT(f16_tag, "f16", 64, 64, true, 2),
-      HSTU_VARIANT(f16_tag, "f16", 128, 64, true, 2), HSTU_VARIANT(f16_tag, "f16", 256, 32, true, 1)}},
+// [dtype: bf16, f16][rab: 0, 1][custom mask: 0, 1][dim slot: 32, 64, 128, 256]
+const Variant kVariants[2][2][2][4] = {
+    {{HSTU_DIMS(bf16_tag, "bf16", false, false), HSTU_DIMS(bf16_tag, "bf16", false, true)},
+     {HSTU_DIMS(bf16_tag, "bf16", true, false), HSTU_DIMS(bf16_tag, "bf16", true, true)}},
+    {{HSTU_DIMS(f16_tag, "f16", false, false), HSTU_DIMS(f16_tag, "f16", false, true)},
+     {HSTU_DIMS(f16_tag, "f16", true, false), HSTU_DIMS(f16_tag, "f16", true, true)}},
 };
 
 int validate(const hstu_jagged_fwd_params* p)
@@ -153,7 +154,8 @@ const Variant* select(const hstu_jagged_fwd_params* p)
              (long long)dmax);
         return nullptr;
     }
-    return &kVariants[p->dtype == HSTU_DT_BF16 ? 0 : 1][p->attn_bias != nullptr ? 1 : 0][slot];
+    return &kVariants[p->dtype == HSTU_DT_BF16 ? 0 : 1][p->attn_bias != nullptr ? 1 : 0]
+                     [p->mask_type == HSTU_MASK_CUSTOM ? 1 : 0][slot];
 }
 
 }  // namespace
@@ -236,16 +238,19 @@ HSTU_API int hstu_jagged_fwd(const hstu_jagged_fwd_params* p, void* workspace, u
     a.bh = a.n_batch * a.n_heads_q;
     const bool bias_aligned = (reinterpret_cast<uintptr_t>(p->attn_bias) % 8 == 0) &&
                               (reinterpret_cast<uintptr_t>(p->mask) % 8 == 0) && (p->max_seq_len_k % 4 == 0);
-    a.rab_vec_ok = bias_aligned ? 1 : 0;
+    a.bias_vec_ok = bias_aligned ? 1 : 0;
     const double scale = (p->silu_scale == 0.0) ? 1.0 / static_cast<double>(p->max_seq_len_q) : p->silu_scale;
     a.c_exp = static_cast<float>(-p->alpha * 1.4426950408889634);
     a.c_out = static_cast<float>(p->alpha * scale);
 
+#ifdef HSTU_TIMELINE
+    a.timeline = static_cast<unsigned long long*>(workspace);  // development builds only
+#endif
     const int64_t n_blocks = static_cast<int64_t>(a.n_qtiles) * a.bh;
     if (n_blocks <= 0 || n_blocks > 0x7fffffffLL) {
         return fail(HSTU_ERR_INVALID, "grid of %lld workgroups is out of range", (long long)n_blocks);
     }
-    hipLaunchKernelGGL(var->kernel, dim3(static_cast<unsigned>(n_blocks)), dim3(hstu::kThreads), 0,
+    hipLaunchKernelGGL(var->kernel, dim3(static_cast<unsigned>(n_blocks)), dim3(static_cast<unsigned>(var->threads)), 0,
                        static_cast<hipStream_t>(stream), a);
     const hipError_t err = hipGetLastError();
     if (err != hipSuccess) {

@@ -83,7 +83,39 @@ def _out_dtype(q: torch.Tensor) -> torch.dtype:
     return torch.float16 if q.dtype == torch.float8_e4m3fn else q.dtype
 
 
-def _forward_impl(
+class PreparedForward:
+    """A validated forward call: the filled C-ABI parameter block, its output tensor and the
+    tensors it points into.  ``launch()`` enqueues it on the current stream; it may be launched
+    repeatedly (benchmarks, steady-state serving with static shapes)."""
+
+    __slots__ = ("params", "out", "workspace", "workspace_bytes", "device", "_keep")
+
+    def __init__(self, params, out, workspace, workspace_bytes, device, keep):
+        self.params = params
+        self.out = out
+        self.workspace = workspace
+        self.workspace_bytes = workspace_bytes
+        self.device = device
+        self._keep = keep
+
+    def launch(self, stream: Optional[int] = None) -> torch.Tensor:
+        if self.out.numel() == 0:
+            return self.out
+        lib = _native.load()
+        if stream is None:
+            stream = torch.cuda.current_stream(self.device).cuda_stream
+        rc = lib.hstu_jagged_fwd(ctypes.byref(self.params), _ptr(self.workspace), self.workspace_bytes,
+                                 ctypes.c_void_p(stream))  # fmt: skip
+        if rc != _native.HSTU_OK:
+            raise RuntimeError(f"hstu_jagged_fwd failed ({rc}): {_native.last_error()}")
+        return self.out
+
+    def kernel_name(self) -> str:
+        name = _native.load().hstu_jagged_fwd_kernel_name(ctypes.byref(self.params))
+        return name.decode() if name else ""
+
+
+def prepare_forward(
     q: torch.Tensor,
     k: torch.Tensor,
     v: torch.Tensor,
@@ -100,7 +132,9 @@ def _forward_impl(
     target_group_size: Optional[int],
     alpha: Optional[float],
     deterministic: bool = False,
-) -> torch.Tensor:
+) -> PreparedForward:
+    """Argument normalisation and checks of the reference adapter
+    (torch_extension/hstu_jagged_plugin.cpp:22-67), ending in a filled parameter block."""
     _check(q.dim() == 3, "The q should be 3D in jagged layout")
     _check(seq_offset is not None and seq_offset_k is not None, "seq_offset is required")
     _check(seq_offset.dim() == 1 and seq_offset.size(0) >= 2,
@@ -149,13 +183,14 @@ def _forward_impl(
     # every row is written by the kernel (rows past the last offset are zero-filled there),
     # so the zero-fill of the reference adapter (:56-59) is not repeated here
     out = torch.empty((q_c.size(0), q_c.size(1), v_c.size(2)), dtype=out_dtype, device=q_c.device)
+    keep = (q_c, k_c, v_c, mask_c, bias, offs_q, offs_k, ctx, tgt)
+    p = _native.new_params()
     if out.numel() == 0:
-        return out
+        return PreparedForward(p, out, None, 0, q_c.device, keep)
 
     real_scale = (1.0 / float(max_seq_len_q)) if float(silu_scale) == 0.0 else float(silu_scale)
 
     lib = _native.load()
-    p = _native.new_params()
     p.dtype = _DTYPE_CODE[q_c.dtype]
     p.out_dtype = _DTYPE_CODE[out_dtype]
     p.index_dtype = _native.IDX_I64 if idx_dtype == torch.int64 else _native.IDX_I32
@@ -175,19 +210,23 @@ def _forward_impl(
     p.alpha = real_alpha
     p.deterministic = 1 if deterministic else 0
 
-    with torch.cuda.device(q_c.device):
-        ws_bytes = ctypes.c_uint64(0)
-        rc = lib.hstu_jagged_fwd_workspace_size(ctypes.byref(p), ctypes.byref(ws_bytes))
-        if rc != _native.HSTU_OK:
-            raise RuntimeError(f"hstu_jagged_fwd_workspace_size failed ({rc}): {_native.last_error()}")
-        ws = None
-        if ws_bytes.value:
-            ws = torch.empty(ws_bytes.value, dtype=torch.uint8, device=q_c.device)
-        stream = torch.cuda.current_stream(q_c.device).cuda_stream
-        rc = lib.hstu_jagged_fwd(ctypes.byref(p), _ptr(ws), ws_bytes.value, ctypes.c_void_p(stream))
-        if rc != _native.HSTU_OK:
-            raise RuntimeError(f"hstu_jagged_fwd failed ({rc}): {_native.last_error()}")
-    return out
+    ws_bytes = ctypes.c_uint64(0)
+    rc = lib.hstu_jagged_fwd_workspace_size(ctypes.byref(p), ctypes.byref(ws_bytes))
+    if rc != _native.HSTU_OK:
+        raise RuntimeError(f"hstu_jagged_fwd_workspace_size failed ({rc}): {_native.last_error()}")
+    ws = None
+    if ws_bytes.value:
+        ws = torch.empty(ws_bytes.value, dtype=torch.uint8, device=q_c.device)
+    return PreparedForward(p, out, ws, ws_bytes.value, q_c.device, keep)
+
+
+def _forward_impl(q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max_seq_len_k, silu_scale, seq_offset,
+                  seq_offset_k, num_context, num_target, target_group_size, alpha, deterministic=False):  # fmt: skip
+    prepared = prepare_forward(q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max_seq_len_k, silu_scale,
+                               seq_offset, seq_offset_k, num_context, num_target, target_group_size, alpha,
+                               deterministic)  # fmt: skip
+    with torch.cuda.device(prepared.device):
+        return prepared.launch()
 
 
 # Python kernels receive only the arguments the caller passed, so the schema defaults are
