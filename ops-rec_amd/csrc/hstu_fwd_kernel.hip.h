@@ -54,11 +54,16 @@ constexpr uint32_t kOutOfRange = 0x80000000u;   // byte offset no descriptor her
 // Optional per-wavefront timeline for kernel development (compile with -DHSTU_TIMELINE and pass a
 // buffer of 64 x uint64 per wavefront in FwdArgs::timeline); compiled out of the shipped library.
 #ifdef HSTU_TIMELINE
+#ifdef HSTU_TIMELINE_REALTIME
+#define HSTU_CLOCK() __builtin_amdgcn_s_memrealtime() /* 100 MHz, same base on every XCD */
+#else
+#define HSTU_CLOCK() __builtin_amdgcn_s_memtime() /* core clock, per-XCD base */
+#endif
 #define HSTU_STAMP(slot)                                                                              \
     do {                                                                                              \
         if (a.timeline && lane == 0 && (slot) < 64)                                                   \
             a.timeline[(static_cast<int64_t>(blockIdx.x) * NWAVES + wave) * 64 + (slot)] =            \
-                __builtin_amdgcn_s_memtime();                                                         \
+                HSTU_CLOCK();                                                         \
     } while (0)
 #else
 #define HSTU_STAMP(slot) \

@@ -1,0 +1,261 @@
+"""CPU-only checks of the host side: schemas and overload resolution, argument checks, Meta shape
+inference, the proxy module, the autograd wrapper's plumbing, and the C ABI (symbols, struct,
+status codes) -- no kernel is launched here."""
+
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+import ops_rec
+from ops_rec import _native, _ops
+from ops_rec.autograd import hstu_v1_autograd as ag
+
+_ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _meta_inputs(total=10, heads=4, dim=32, dim_v=None, dtype=torch.bfloat16):
+    q = torch.empty(total, heads, dim, device="meta", dtype=dtype)
+    v = torch.empty(total, heads, dim_v or dim, device="meta", dtype=dtype)
+    offs = torch.empty(3, device="meta", dtype=torch.int32)
+    return q, q, v, offs
+
+
+# ---------------------------------------------------------------- schemas / dispatch ----
+
+
+def test_ops_are_registered_with_both_overloads():
+    pkt = torch.ops.ops_rec.hstu_jagged
+    assert set(pkt.overloads()) == {"equal", "delta"}
+    assert set(torch.ops.ops_rec.hstu_jagged_backward.overloads()) == {"equal", "delta"}
+    eq = pkt.equal._schema
+    assert [a.name for a in eq.arguments] == [
+        "q", "k", "v", "mask", "attn_bias", "mask_type", "max_seq_len", "silu_scale", "seq_offset", "num_context",
+        "num_target", "target_group_size", "alpha", "deterministic",
+    ]  # fmt: skip
+    de = pkt.delta._schema
+    assert [a.name for a in de.arguments][6:11] == ["max_seq_len", "max_seq_len_k", "silu_scale", "seq_offset",
+                                                    "seq_offset_k"]  # fmt: skip
+
+
+def test_packet_resolves_equal_and_delta_by_argument_types():
+    q, k, v, offs = _meta_inputs()
+    op = ops_rec.ascendc.attention.hstu_jagged
+    # 9 positional (equal), keyword form (equal), 11 positional (delta): the reference's examples
+    assert op(q, k, v, None, None, 0, 6, 1.0 / 6, offs).shape == (10, 4, 32)
+    assert op(q, k, v, mask=None, attn_bias=None, mask_type=0, max_seq_len=6, silu_scale=0.0, seq_offset=offs).shape == (10, 4, 32)
+    assert op(q, k, v, None, None, 0, 6, 8, 1.0 / 6, offs, offs).shape == (10, 4, 32)
+    assert op.equal(q, k, v, None, None, 0, 6, 0, offs).shape == (10, 4, 32)  # int accepted for silu_scale
+
+
+def test_meta_shape_and_dtype_inference():
+    q, k, v, offs = _meta_inputs(dim=64, dim_v=32)
+    out = torch.ops.ops_rec.hstu_jagged.equal(q, k, v, None, None, 0, 6, 0.0, offs)
+    assert out.shape == (10, 4, 32) and out.dtype == torch.bfloat16 and out.device.type == "meta"
+    q8 = torch.empty(10, 4, 64, device="meta", dtype=torch.float8_e4m3fn)
+    out8 = torch.ops.ops_rec.hstu_jagged.equal(q8, q8, q8, None, None, 0, 6, 0.0, offs)
+    assert out8.dtype == torch.float16  # fp8 inputs produce half outputs, as in the reference adapter
+    with pytest.raises(RuntimeError, match="3D"):
+        torch.ops.ops_rec.hstu_jagged.equal(q[0], k, v, None, None, 0, 6, 0.0, offs)
+    dq, dk, dv, db = torch.ops.ops_rec.hstu_jagged_backward.equal(out, q, k, v, None, None, 0, 6, 0.0, offs)
+    assert dq.shape == q.shape and dk.shape == k.shape and dv.shape == v.shape and db is None
+
+
+def test_no_cpu_implementation():
+    q = torch.zeros(4, 2, 32, dtype=torch.bfloat16)
+    offs = torch.tensor([0, 4], dtype=torch.int32)
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        torch.ops.ops_rec.hstu_jagged.equal(q, q, q, None, None, 0, 4, 0.0, offs)
+
+
+def test_proxy_module_surface():
+    att = ops_rec.ascendc.attention
+    assert att.hstu_jagged is torch.ops.ops_rec.hstu_jagged
+    from ops_rec.ascendc.attention import hstu_jagged, hstu_jagged_backward  # noqa: F401
+
+    assert "hstu_jagged" in dir(att)
+    with pytest.raises(AttributeError, match="Available ops"):
+        att.no_such_operator
+
+
+# ---------------------------------------------------------------- argument checks ----
+
+
+def _cpu_args(**over):
+    q = torch.zeros(10, 4, 32, dtype=torch.bfloat16)
+    offs = torch.tensor([0, 4, 10], dtype=torch.int32)
+    a = dict(q=q, k=q, v=q, mask=None, attn_bias=None, mask_type=0, max_seq_len_q=6, max_seq_len_k=6, silu_scale=0.0,
+             seq_offset=offs, seq_offset_k=offs, num_context=None, num_target=None, target_group_size=0, alpha=1.0)  # fmt: skip
+    a.update(over)
+    return a
+
+
+@pytest.mark.parametrize(
+    "over,msg",
+    [
+        (dict(q=torch.zeros(10, 32, dtype=torch.bfloat16)), "3D in jagged layout"),
+        (dict(seq_offset=torch.tensor([0], dtype=torch.int32)), "at least two element"),
+        (dict(seq_offset_k=torch.tensor([0], dtype=torch.int32)), "at least two element"),
+        (dict(max_seq_len_q=0), r"expect in \[1, 20480\]"),
+        (dict(max_seq_len_q=20481), r"expect in \[1, 20480\]"),
+        (dict(max_seq_len_k=0), r"expect in \[1, 20480\]"),
+        (dict(mask_type=4), r"maskType expect in \[0, 3\]"),
+        (dict(mask_type=-1), r"maskType expect in \[0, 3\]"),
+        (dict(mask_type=1), "not support triu"),
+        (dict(mask_type=3), "must have valide mask tensor"),
+        (dict(v=torch.zeros(9, 4, 32, dtype=torch.bfloat16)), "K, V seqLens mismatch"),
+        (dict(v=torch.zeros(10, 2, 32, dtype=torch.bfloat16)), "K, V headNum mismatch"),
+        (dict(k=torch.zeros(10, 4, 16, dtype=torch.bfloat16)), "headDIM"),
+        (dict(num_context=torch.zeros(3, dtype=torch.int32)), "num_context"),
+        (dict(num_target=torch.zeros(1, dtype=torch.int32)), "num_target"),
+        (dict(attn_bias=torch.zeros(2, 4, 6, 5, dtype=torch.bfloat16)), "attn_bias must have shape"),
+        (dict(attn_bias=torch.zeros(2, 4, 6, 6, dtype=torch.float16)), "attn_bias must have the dtype"),
+    ],
+)
+def test_adapter_rejects_bad_arguments(over, msg):
+    # same trigger conditions as the reference adapter's TORCH_CHECKs; raised before any device work
+    with pytest.raises(RuntimeError, match=msg):
+        _ops.prepare_forward(**_cpu_args(**over))
+
+
+def test_empty_input_returns_empty_output_without_touching_the_library():
+    q = torch.zeros(0, 4, 32, dtype=torch.bfloat16)
+    p = _ops.prepare_forward(**_cpu_args(q=q, k=q, v=q, seq_offset=torch.tensor([0, 0], dtype=torch.int32),
+                                         seq_offset_k=torch.tensor([0, 0], dtype=torch.int32)))  # fmt: skip
+    assert p.launch().shape == (0, 4, 32)
+
+
+# ---------------------------------------------------------------- autograd wrapper ----
+
+
+def test_autograd_formulas_are_registered_once():
+    assert ag._registered and ag._registration_errors == {}
+    ag.register_autograd()  # idempotent
+    assert "hstu_v1_autograd" in ops_rec.autograd.__all__
+
+
+def test_unpack_fills_schema_defaults():
+    vals = ag._unpack(("q", "k", "v"), ag._EQUAL_DEFAULTS)
+    assert len(vals) == 14 and vals[5] == 0 and vals[7] == 0.0 and vals[12] == 1.0 and vals[13] is False
+    vals = ag._unpack(tuple(range(16)), ag._DELTA_DEFAULTS)
+    assert vals == tuple(range(16))
+
+
+def test_fit_grads_pads_and_cuts():
+    class Ctx:
+        needs_input_grad = (True,) * 9
+
+    assert ag._fit_grads((1, 2, 3, None, 5), Ctx) == (1, 2, 3, None, 5, None, None, None, None)
+    Ctx.needs_input_grad = (True,) * 3
+    assert ag._fit_grads((1, 2, 3, None, 5), Ctx) == (1, 2, 3)
+
+
+def test_mask_requiring_grad_is_rejected():
+    m = torch.zeros(2, 2, requires_grad=True)
+    with pytest.raises(NotImplementedError, match="non-differentiable"):
+        ag._reject_mask_grad(m, "hstu_jagged.equal")
+    ag._reject_mask_grad(None, "x")
+    ag._reject_mask_grad(torch.zeros(2), "x")
+
+
+# ---------------------------------------------------------------- C ABI ----
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(_ROOT, "include", "hstu_mi355.h")).read()
+    declared = set(re.findall(r"HSTU_API\s+[\w\s\*]+?\b(hstu_\w+)\s*\(", header))
+    assert declared == set(_native.EXPORTED_SYMBOLS)
+    lib = _native.load()
+    for sym in declared:
+        assert getattr(lib, sym) is not None
+    assert lib.hstu_version() >= 1
+
+
+def test_struct_mirror_matches_library():
+    # the library checks struct_size itself: a correct mirror gets past that check
+    lib = _native.load()
+    p = _native.new_params()
+    ws = ctypes.c_uint64(123)
+    rc = lib.hstu_jagged_fwd_workspace_size(ctypes.byref(p), ctypes.byref(ws))
+    assert rc == 161002 and "at least two element" in _native.last_error()
+    p.struct_size = 8
+    rc = lib.hstu_jagged_fwd_workspace_size(ctypes.byref(p), ctypes.byref(ws))
+    assert rc == 161002 and "struct_size" in _native.last_error()
+
+
+def _valid_params():
+    p = _native.new_params()
+    p.dtype = p.out_dtype = _native.DT_BF16
+    p.index_dtype = _native.IDX_I32
+    fake = 0x1000  # never dereferenced: only validation runs
+    p.q = p.k = p.v = p.out = p.seq_offset_q = p.seq_offset_k = fake
+    p.total_q = p.total_k = 10
+    p.num_heads_q = p.num_heads_k = 4
+    p.head_dim_qk = p.head_dim_v = 128
+    p.n_offsets = 3
+    p.max_seq_len_q = p.max_seq_len_k = 6
+    p.silu_scale, p.alpha = 0.0, 1.0
+    return p
+
+
+def test_c_abi_validation_codes():
+    lib = _native.load()
+    ws = ctypes.c_uint64(7)
+
+    def rc(p):
+        return lib.hstu_jagged_fwd_workspace_size(ctypes.byref(p), ctypes.byref(ws))
+
+    p = _valid_params()
+    assert rc(p) == 0 and ws.value == 0
+    assert lib.hstu_jagged_fwd_kernel_name(ctypes.byref(p)).decode().startswith("hstu_fwd_bf16_d128")
+    assert lib.hstu_jagged_fwd_workspace_size(None, ctypes.byref(ws)) == 161001
+    assert lib.hstu_jagged_fwd_workspace_size(ctypes.byref(p), None) == 161001
+    for field, value, code, text in [
+        ("q", None, 161001, "must not be NULL"),
+        ("seq_offset_q", None, 161001, "must not be NULL"),
+        ("mask_type", 1, 161002, "triu"),
+        ("mask_type", 3, 161002, "valide mask"),
+        ("mask_type", 9, 161002, r"\[0, 3\]"),
+        ("max_seq_len_q", 0, 161002, "20480"),
+        ("max_seq_len_k", 30000, 161002, "20480"),
+        ("n_offsets", 2050, 161002, "batchSize"),
+        ("num_heads_q", 17, 161002, "head num"),
+        ("num_heads_k", 3, 161002, "divisible"),
+        ("head_dim_v", 24, 161002, "step 16"),
+        ("head_dim_qk", 513, 161002, "512"),
+        ("index_dtype", 5, 161002, "index_dtype"),
+        ("dtype", 9, 161002, "unknown dtype"),
+        ("head_dim_qk", 12, 161003, "multiple of 8"),
+    ]:
+        p = _valid_params()
+        setattr(p, field, value)
+        if field == "head_dim_qk" and value == 12:
+            p.head_dim_v = 16
+        got = rc(p)
+        assert got == code, (field, value, got, _native.last_error())
+        assert re.search(text, _native.last_error()), (field, _native.last_error())
+    # launching with an invalid description is refused before any device call
+    p = _valid_params()
+    p.mask_type = 1
+    assert lib.hstu_jagged_fwd(ctypes.byref(p), None, 0, None) == 161002
+
+
+def test_kernel_variant_selection():
+    lib = _native.load()
+
+    def name(**kw):
+        p = _valid_params()
+        for k, v in kw.items():
+            setattr(p, k, v)
+        n = lib.hstu_jagged_fwd_kernel_name(ctypes.byref(p))
+        return n.decode() if n else None
+
+    assert "_d32_" in name(head_dim_qk=16, head_dim_v=16)
+    assert "_d64_" in name(head_dim_qk=64, head_dim_v=48)
+    assert "_d128_" in name(head_dim_qk=64, head_dim_v=128)
+    assert "_d256_" in name(head_dim_qk=256, head_dim_v=256)
+    assert "rabtrue" in name(attn_bias=0x2000)
+    assert "masktrue" in name(mask=0x2000, mask_type=3)
+    assert "f16" in name(dtype=_native.DT_FP16, out_dtype=_native.DT_FP16)
