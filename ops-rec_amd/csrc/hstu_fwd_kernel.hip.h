@@ -117,6 +117,66 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, ui
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(bytes), kBufferFlags);
 }
 
+// Visibility bounds shared by the 32 query rows [wr0, min(wr0 + 32, sq)) of one wavefront under the
+// built-in mask, in closed form (no cross-lane traffic).  A key j is visible to row i iff
+//   j < lim(i)  &&  !(hist_k <= j < hole_hi(i))
+// with lim(i) = clamp(i < n_ctx ? max(i + delta + 1, hist_k) : i + delta + 1, 0, sk), delta = sk - sq,
+// hist_k = sk - n_tgt, and hole_hi(i) = hist_k + ((i - (sq - n_tgt)) / g) * g for target rows
+// (.../op_kernel/atlas950/hstu_dense_causal_mask.h:186-260).  A 32-key tile starting at c0 is
+//   skipped    when c0 >= lim_max,
+//   unmasked   when c0 + 32 <= lim_min and it does not touch [hist_k, hole_hi_max).
+struct WaveBounds {
+    int lim_min;
+    int lim_max;
+    int hole_hi_max;
+    bool any_hole;
+};
+
+__device__ __forceinline__ WaveBounds wave_bounds(int mask_type, int wr0, int sq, int sk, int n_ctx, int n_tgt,
+                                                  int group, bool active)
+{
+    WaveBounds w;
+    w.hole_hi_max = 0;
+    w.any_hole = false;
+    if (!active) {
+        w.lim_min = 0;
+        w.lim_max = 0;
+        return w;
+    }
+    if (mask_type != 0) {
+        w.lim_min = sk;
+        w.lim_max = sk;
+        return w;
+    }
+    const int wr1 = (wr0 + kWaveM < sq) ? wr0 + kWaveM : sq;
+    const int delta = sk - sq;
+    const int hist_k = sk - n_tgt;
+    int hi = wr1 + delta;  // lim of the last row
+    if (wr0 < n_ctx) {
+        hi = hi > hist_k ? hi : hist_k;
+    }
+    int lo = 0x7fffffff;
+    if (wr0 < n_ctx) {  // first context row
+        const int c = wr0 + delta + 1;
+        lo = c > hist_k ? c : hist_k;
+    }
+    const int rn = wr0 > n_ctx ? wr0 : n_ctx;  // first row that is not a context row
+    if (rn < wr1) {
+        const int c = rn + delta + 1;
+        lo = c < lo ? c : lo;
+    }
+    w.lim_max = hi < 0 ? 0 : (hi > sk ? sk : hi);
+    w.lim_min = lo < 0 ? 0 : (lo > sk ? sk : lo);
+    if (n_tgt > 0 && group > 0) {
+        const int ti = (wr1 - 1) - (sq - n_tgt);
+        if (ti >= 0) {
+            w.hole_hi_max = hist_k + (ti / group) * group;
+            w.any_hole = w.hole_hi_max > hist_k;
+        }
+    }
+    return w;
+}
+
 // ---- type helpers -------------------------------------------------------------------------
 
 template <typename Tag>
@@ -456,10 +516,15 @@ __global__ __launch_bounds__(256 * NKH, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel
                 w[2 * g + 0] = t[0];
                 w[2 * g + 1] = t[1];
             } else {
-                const uint32_t e0 = __builtin_amdgcn_raw_buffer_load_b16(rsrc, static_cast<int>(off), 0, 0);
-                const uint32_t e1 = __builtin_amdgcn_raw_buffer_load_b16(rsrc, static_cast<int>(off + 2u), 0, 0);
-                const uint32_t e2 = __builtin_amdgcn_raw_buffer_load_b16(rsrc, static_cast<int>(off + 4u), 0, 0);
-                const uint32_t e3 = __builtin_amdgcn_raw_buffer_load_b16(rsrc, static_cast<int>(off + 6u), 0, 0);
+                // the offset is laundered through an empty asm so that the optimiser cannot relate these
+                // element loads to the vector load of the other branch (it otherwise folds the two and
+                // replicates the first element)
+                uint32_t eoff = off;
+                asm volatile("" : "+v"(eoff));
+                const uint32_t e0 = __builtin_amdgcn_raw_buffer_load_b16(rsrc, static_cast<int>(eoff), 0, 0);
+                const uint32_t e1 = __builtin_amdgcn_raw_buffer_load_b16(rsrc, static_cast<int>(eoff + 2u), 0, 0);
+                const uint32_t e2 = __builtin_amdgcn_raw_buffer_load_b16(rsrc, static_cast<int>(eoff + 4u), 0, 0);
+                const uint32_t e3 = __builtin_amdgcn_raw_buffer_load_b16(rsrc, static_cast<int>(eoff + 6u), 0, 0);
                 w[2 * g + 0] = (e0 & 0xffffu) | (e1 << 16);
                 w[2 * g + 1] = (e2 & 0xffffu) | (e3 << 16);
             }

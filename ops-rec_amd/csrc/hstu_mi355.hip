@@ -13,6 +13,7 @@
 #include <cstdio>
 #include <cstring>
 
+#include "hstu_fwd_f32_kernel.hip.h"
 #include "hstu_fwd_kernel.hip.h"
 
 namespace {
@@ -49,6 +50,15 @@ const Variant kVariants[2][2][2][4] = {
     {{HSTU_DIMS(f16_tag, "f16", false, false), HSTU_DIMS(f16_tag, "f16", false, true)},
      {HSTU_DIMS(f16_tag, "f16", true, false), HSTU_DIMS(f16_tag, "f16", true, true)}},
 };
+
+#define HSTU_F32_VARIANT(D, RAB, MASK) \
+    {"hstu_fwd_f32_d" #D "_rab" #RAB "_mask" #MASK, hstu::hstu_fwd_f32_kernel<D, RAB, MASK>, D, 256}
+#define HSTU_F32_DIMS(RAB, MASK) \
+    {HSTU_F32_VARIANT(32, RAB, MASK), HSTU_F32_VARIANT(64, RAB, MASK), HSTU_F32_VARIANT(128, RAB, MASK), \
+     HSTU_F32_VARIANT(256, RAB, MASK)}
+// fp32 inputs: [rab][custom mask][dim slot]
+const Variant kVariantsF32[2][2][4] = {{HSTU_F32_DIMS(false, false), HSTU_F32_DIMS(false, true)},
+                                       {HSTU_F32_DIMS(true, false), HSTU_F32_DIMS(true, true)}};
 
 int validate(const hstu_jagged_fwd_params* p)
 {
@@ -127,12 +137,13 @@ int validate(const hstu_jagged_fwd_params* p)
 // picks the kernel variant; returns nullptr (and sets the error) when the combination is not built
 const Variant* select(const hstu_jagged_fwd_params* p)
 {
-    if (p->dtype != HSTU_DT_BF16 && p->dtype != HSTU_DT_FP16) {
-        fail(HSTU_ERR_UNSUPPORTED, "dtype %d is not built in this library version (bf16 and fp16 are)", p->dtype);
+    if (p->dtype != HSTU_DT_BF16 && p->dtype != HSTU_DT_FP16 && p->dtype != HSTU_DT_FP32) {
+        fail(HSTU_ERR_UNSUPPORTED, "dtype %d is not built in this library version (bf16, fp16 and fp32 are)",
+             p->dtype);
         return nullptr;
     }
     if (p->out_dtype != p->dtype) {
-        fail(HSTU_ERR_UNSUPPORTED, "out_dtype must equal dtype for bf16 / fp16 inputs");
+        fail(HSTU_ERR_UNSUPPORTED, "out_dtype must equal dtype for bf16 / fp16 / fp32 inputs");
         return nullptr;
     }
     if (p->head_dim_qk % 8 != 0) {
@@ -153,6 +164,9 @@ const Variant* select(const hstu_jagged_fwd_params* p)
         fail(HSTU_ERR_UNSUPPORTED, "head dims above 256 are not built in this library version (got %lld)",
              (long long)dmax);
         return nullptr;
+    }
+    if (p->dtype == HSTU_DT_FP32) {
+        return &kVariantsF32[p->attn_bias != nullptr ? 1 : 0][p->mask_type == HSTU_MASK_CUSTOM ? 1 : 0][slot];
     }
     return &kVariants[p->dtype == HSTU_DT_BF16 ? 0 : 1][p->attn_bias != nullptr ? 1 : 0]
                      [p->mask_type == HSTU_MASK_CUSTOM ? 1 : 0][slot];
@@ -236,8 +250,9 @@ HSTU_API int hstu_jagged_fwd(const hstu_jagged_fwd_params* p, void* workspace, u
     a.idx64 = (p->index_dtype == HSTU_IDX_I64) ? 1 : 0;
     a.n_qtiles = (a.max_q + hstu::kBlockM - 1) / hstu::kBlockM;
     a.bh = a.n_batch * a.n_heads_q;
-    const bool bias_aligned = (reinterpret_cast<uintptr_t>(p->attn_bias) % 8 == 0) &&
-                              (reinterpret_cast<uintptr_t>(p->mask) % 8 == 0) && (p->max_seq_len_k % 4 == 0);
+    const uintptr_t vec_bytes = (p->dtype == HSTU_DT_FP32) ? 16 : 8;  // four elements
+    const bool bias_aligned = (reinterpret_cast<uintptr_t>(p->attn_bias) % vec_bytes == 0) &&
+                              (reinterpret_cast<uintptr_t>(p->mask) % vec_bytes == 0) && (p->max_seq_len_k % 4 == 0);
     a.bias_vec_ok = bias_aligned ? 1 : 0;
     const double scale = (p->silu_scale == 0.0) ? 1.0 / static_cast<double>(p->max_seq_len_q) : p->silu_scale;
     a.c_exp = static_cast<float>(-p->alpha * 1.4426950408889634);
