@@ -38,7 +38,7 @@ PEAK_HBM_GBS = 8000.0  # MI355X HBM3E bandwidth (published)
 
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), scaled by the same
 # counters' reading of a plain copy kernel of known size; see profiles/.  None = not measured yet.
-MEASURED_TRAFFIC_BYTES = {}
+MEASURED_TRAFFIC_BYTES = {"C2": 99_300_000}  # profiles/hstu_fwd_bf16_d128_C2_counters.md
 
 
 def algorithmic_bytes(w) -> int:
@@ -57,6 +57,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="C2", choices=["C2", "C3", "C4"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--calibration-copy-mib", type=int, default=0,
+                    help="after the timed steps also run 5 plain device-to-device copies of this many MiB, so that a "
+                    "counter run (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) can be scaled by a kernel of known traffic")  # fmt: skip
     args = ap.parse_args()
     if args.gpus != 1:
         print(
@@ -116,6 +119,14 @@ def main() -> int:
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
     ev_ms = e0.elapsed_time(e1) / args.steps
     ms_per_step = max(wall_ms, ev_ms)  # the slower clock: host-bound launches cannot hide
+
+    if args.calibration_copy_mib > 0:
+        src = torch.empty(args.calibration_copy_mib << 20, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     # ---- the same through the Python entry point ----
     op = ops_rec.ascendc.attention.hstu_jagged
