@@ -1,12 +1,15 @@
 // HSTU jagged attention forward for gfx950 (MI355X): device code.
 //
-// One workgroup owns a 128-row query tile of one (sequence, head).  Its wavefronts form a
-// 4 x NKH grid: four row groups of 32 query rows, times NKH "key lanes" that split the 32-key
-// sub-tiles of every K/V tile between them (NKH = 2: eight wavefronts, two per SIMD, which halves
-// the longest serial chain of a causal tile; their partial outputs are summed through LDS at the
-// end, in a fixed order).  A wavefront keeps its Q rows in registers for the whole key sweep,
-// K and V tiles are streamed global -> LDS by buffer loads that write LDS directly (no register
-// staging), double-buffered, and
+// Work item = one 128-row query tile of one (sequence, head): four wavefronts of 32 query rows each.
+// The kernel is persistent: a fixed number of workgroups (two per CU) is launched, each builds the
+// work list in its own LDS from seq_offset (sequences bucketed by their number of query tiles,
+// heaviest tiles first, tiles past the end of a sequence never listed) and then pulls item after
+// item from a device-side counter, so that the jagged, causal mix of long and short items is
+// balanced dynamically and the launch / set-up cost of a workgroup is paid once, not per tile.
+//
+// Per wavefront: its Q rows stay in registers for the whole key sweep of an item, K and V tiles
+// are streamed global -> LDS by buffer loads that write LDS directly (no register staging),
+// double-buffered, and
 //
 //     S^T = K . Q^T                 v_mfma_f32_32x32x16  (A = K tile from LDS, B = Q from registers)
 //     P^T = silu(alpha * (S^T + rab^T)) * mask, rounded to the input type
@@ -16,7 +19,8 @@
 // Computing the transposed score means the accumulator layout of S^T (lane = query row, registers
 // = 4 consecutive keys) is exactly the B-operand layout the second product needs, so P never
 // leaves registers.  There is no row reduction (no softmax), every output row is produced by
-// one workgroup and stored once: no atomics, bitwise deterministic.
+// one wavefront and stored once: no atomics on data, bitwise deterministic whatever workgroup
+// happens to pull an item.
 //
 // Out-of-range rows (past the end of a sequence) are never branched on: all global accesses go
 // through buffer descriptors sized to the sequence, whose out-of-range reads return zero and
@@ -62,8 +66,7 @@ constexpr uint32_t kOutOfRange = 0x80000000u;   // byte offset no descriptor her
 #define HSTU_STAMP(slot)                                                                              \
     do {                                                                                              \
         if (a.timeline && lane == 0 && (slot) < 64)                                                   \
-            a.timeline[(static_cast<int64_t>(blockIdx.x) * NWAVES + wave) * 64 + (slot)] =            \
-                HSTU_CLOCK();                                                         \
+            a.timeline[(static_cast<int64_t>(blockIdx.x) * 4 + wave) * 64 + (slot)] = HSTU_CLOCK();   \
     } while (0)
 #else
 #define HSTU_STAMP(slot) \
@@ -100,6 +103,7 @@ struct FwdArgs {
     int bias_vec_ok; // rab / mask rows may be read 4 elements (8 bytes) at a time
     float c_exp;     // -alpha * log2(e)
     float c_out;     // alpha * silu_scale
+    int counter_slot;  // which pair of device-side work counters this launch uses
 #ifdef HSTU_TIMELINE
     unsigned long long* timeline;
 #endif
@@ -284,27 +288,49 @@ __device__ __forceinline__ void load_to_lds_b128(__amdgpu_buffer_rsrc_t rsrc, ui
                                              static_cast<int>(voffset), 0, 0, 0);
 }
 
+// ---- device-side work counters ---------------------------------------------------------------
+// One (work, done) pair per slot; a launch is given a slot by the host (round robin), so launches
+// that overlap on one GPU do not share a pair unless more than kCounterSlots of them are in flight.
+// Zero at module load; the last workgroup of a launch to leave puts its pair back to zero.
+constexpr int kCounterSlots = 64;
+static __device__ unsigned int g_work_counter[kCounterSlots];
+static __device__ unsigned int g_done_counter[kCounterSlots];
+
+constexpr int kMaxBatchSlots = 2048;  // sequences per call (the reference's limit)
+constexpr int kMaxLevels = 160;       // ceil(20480 / 128) query-tile levels
+
+// scalar (uniform-address) load of an offset / count
+__device__ __forceinline__ int64_t load_index_uniform(const void* p, int64_t i, int idx64)
+{
+    typedef const __attribute__((address_space(4))) int64_t* cptr64_t;
+    typedef const __attribute__((address_space(4))) int32_t* cptr32_t;
+    if (idx64) {
+        return ((cptr64_t)(reinterpret_cast<uintptr_t>(p)))[i];
+    }
+    return static_cast<int64_t>(((cptr32_t)(reinterpret_cast<uintptr_t>(p)))[i]);
+}
+
+struct U32Pair {
+    uint32_t v[2];
+};
+
 // ---- the kernel ---------------------------------------------------------------------------
 // Tag      : bf16_tag / f16_tag
 // D        : padded head dim used for both QK and V (32, 64, 128 or 256); real dims come from args
-// BN       : keys per LDS tile (multiple of 32 * NKH)
-// NKH      : key lanes (1 or 2); the workgroup has 4 * NKH wavefronts
+// BN       : keys per LDS tile (multiple of 32)
 // HAS_RAB  : attn_bias present
 // HAS_MASK : mask_type 3 (dense custom mask multiplied in)
-template <typename Tag, int D, int BN, int NKH, bool HAS_RAB, bool HAS_MASK>
-__global__ __launch_bounds__(256 * NKH, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const FwdArgs a)
+template <typename Tag, int D, int BN, bool HAS_RAB, bool HAS_MASK>
+__global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const FwdArgs a)
 {
-    constexpr int kThreads = 256 * NKH;
-    constexpr int NWAVES = 4 * NKH;
-    constexpr int CPR = D / 8;                       // 16-byte chunks per row
+    constexpr int kThreads = 256;
+    constexpr int CPR = D / 8;                  // 16-byte chunks per row
     constexpr int TILE_ELEMS = BN * D;
-    constexpr int LOADS = TILE_ELEMS / 512 / NWAVES;  // 1 KiB load instructions per wavefront per tile
-    static_assert(TILE_ELEMS % (512 * NWAVES) == 0, "tile must split evenly over the wavefronts");
+    constexpr int LOADS = TILE_ELEMS / 512 / 4;  // 1 KiB load instructions per wavefront per tile
+    static_assert(TILE_ELEMS % 2048 == 0, "tile must split evenly over the four wavefronts");
     constexpr int KSTEPS = D / 16;  // MFMA steps over the head dim (QK product)
     constexpr int MTILES = D / 32;  // 32-wide output tiles over the head dim (PV product)
     constexpr int NSUB = BN / 32;   // 32-key sub-tiles per LDS tile
-    constexpr int MYSUB = NSUB / NKH;  // sub-tiles per tile handled by one wavefront (ms = kh, kh + NKH, ...)
-    static_assert(NSUB % NKH == 0 && MYSUB >= 1, "sub-tiles must split evenly over the key lanes");
 
     // four separate arrays (not one block) so that the compiler can tell the buffer being filled by
     // the asynchronous loads from the buffer being read, and does not wait for the loads early
@@ -312,6 +338,12 @@ __global__ __launch_bounds__(256 * NKH, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel
     __shared__ __attribute__((aligned(1024))) uint16_t s_k1[TILE_ELEMS];
     __shared__ __attribute__((aligned(1024))) uint16_t s_v0[TILE_ELEMS];
     __shared__ __attribute__((aligned(1024))) uint16_t s_v1[TILE_ELEMS];
+    // work list
+    __shared__ uint8_t s_ntiles[kMaxBatchSlots];          // query tiles of each sequence
+    __shared__ uint16_t s_order[kMaxBatchSlots];          // sequences, most query tiles first
+    __shared__ uint32_t s_bucket[kMaxLevels + 2];         // histogram, then scatter cursors
+    __shared__ uint32_t s_level_start[kMaxLevels + 2];    // first item of each level (level = tiles from the top)
+    __shared__ uint32_t s_next;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -319,158 +351,94 @@ __global__ __launch_bounds__(256 * NKH, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel
     const int ln = lane & 31;
     const int lh = lane >> 5;
 
-    // ---- which (q-tile, sequence, head): heaviest q-tiles are dispatched first ----
-    const int lvl = blockIdx.x / a.bh;
-    const int bhid = blockIdx.x - lvl * a.bh;
-    const int qt = a.n_qtiles - 1 - lvl;
-    const int b = bhid / a.n_heads_q;
-    const int h = bhid - b * a.n_heads_q;
-    const int hk = h / a.head_ratio;
-
-    int64_t q0 = load_index(a.offs_q, b, a.idx64);
-    int64_t q1 = load_index(a.offs_q, b + 1, a.idx64);
-    int64_t k0 = load_index(a.offs_k, b, a.idx64);
-    int64_t k1 = load_index(a.offs_k, b + 1, a.idx64);
-    // defensive clamps: malformed offsets must not turn into out-of-bounds addresses
-    q1 = q1 < a.total_q ? q1 : a.total_q;
-    k1 = k1 < a.total_k ? k1 : a.total_k;
-    q0 = q0 < 0 ? 0 : q0;
-    k0 = k0 < 0 ? 0 : k0;
-    int sq = static_cast<int>(q1 > q0 ? q1 - q0 : 0);
-    int sk = static_cast<int>(k1 > k0 ? k1 - k0 : 0);
-    sq = uniform(sq < a.max_q ? sq : a.max_q);
-    sk = uniform(sk < a.max_k ? sk : a.max_k);
-
     uint16_t* const out16 = static_cast<uint16_t*>(a.out);
+    const int n_levels = a.n_qtiles;
+    const int n_heads = a.n_heads_q;
 
-    // rows past the last offset belong to no sequence: the lightest level zero-fills them
-    if (qt == 0) {
-        const int64_t last = load_index(a.offs_q, a.n_batch, a.idx64);
-        const int64_t first_tail = last < 0 ? 0 : last;
-        const int64_t row_elems = static_cast<int64_t>(a.n_heads_q) * a.d_v;
-        const int64_t n_tail = (a.total_q > first_tail ? a.total_q - first_tail : 0) * row_elems;
+    // ---- rows past the last offset belong to no sequence: zero-fill them (all workgroups share the job) ----
+    {
+        const int64_t last = load_index_uniform(a.offs_q, a.n_batch, a.idx64);
+        const int64_t first_tail = last < 0 ? 0 : (last < a.total_q ? last : a.total_q);
+        const int64_t row_elems = static_cast<int64_t>(n_heads) * a.d_v;
+        const int64_t n_tail = (a.total_q - first_tail) * row_elems;
         uint16_t* tail = out16 + first_tail * row_elems;
-        for (int64_t e = static_cast<int64_t>(bhid) * kThreads + tid; e < n_tail;
-             e += static_cast<int64_t>(a.bh) * kThreads) {
+        for (int64_t e = static_cast<int64_t>(blockIdx.x) * kThreads + tid; e < n_tail;
+             e += static_cast<int64_t>(gridDim.x) * kThreads) {
             tail[e] = 0;
         }
     }
 
-    const int r0 = qt * kBlockM;
-    if (r0 >= sq) {
-        return;
+    // ---- work list: bucket the sequences by their number of query tiles ----
+    for (int i = tid; i <= n_levels; i += kThreads) {
+        s_bucket[i] = 0;
     }
-    HSTU_STAMP(0);
-    const int row_group = wave & 3;
-    const int kh = wave >> 2;  // key lane
-    const int wr0 = r0 + row_group * kWaveM;
-    const bool wave_active = wr0 < sq;  // inactive wavefronts still take part in loads and barriers
-
-    int n_ctx = 0;
-    int n_tgt = 0;
-    if (a.mask_type == 0) {
-        if (a.num_ctx) {
-            n_ctx = static_cast<int>(load_index(a.num_ctx, b, a.idx64));
-        }
-        if (a.num_tgt) {
-            n_tgt = static_cast<int>(load_index(a.num_tgt, b, a.idx64));
-        }
-        n_ctx = uniform(n_ctx < 0 ? 0 : n_ctx);
-        n_tgt = uniform(n_tgt < 0 ? 0 : (n_tgt > sk ? sk : n_tgt));
+    __syncthreads();
+    for (int b = tid; b < a.n_batch; b += kThreads) {
+        int64_t q0 = load_index(a.offs_q, b, a.idx64);
+        int64_t q1 = load_index(a.offs_q, b + 1, a.idx64);
+        q1 = q1 < a.total_q ? q1 : a.total_q;
+        q0 = q0 < 0 ? 0 : q0;
+        int sq = static_cast<int>(q1 > q0 ? q1 - q0 : 0);
+        sq = sq < a.max_q ? sq : a.max_q;
+        const int nt = (sq + kBlockM - 1) / kBlockM;  // 0 .. n_levels
+        s_ntiles[b] = static_cast<uint8_t>(nt);
+        atomicAdd(&s_bucket[nt], 1u);
     }
-    const int delta = sk - sq;
-    const int hist_k = sk - n_tgt;  // keys before the target block
-
-    // ---- per-row visibility constants (row = this lane's query row, clamped into the sequence) ----
-    //   visible(j) = j < lim  &&  !(hole_lo <= j < hole_hi)
-    int row = wr0 + ln;
-    {
-        const int last_row = sq - 1;
-        row = row < last_row ? row : last_row;
-    }
-    int lim;
-    int hole_lo = 0;
-    int hole_hi = 0;
-    if (a.mask_type == 0) {
-        lim = row + delta + 1;
-        if (row < n_ctx) {
-            lim = lim > hist_k ? lim : hist_k;
+    __syncthreads();
+    if (tid == 0) {
+        // bucket start in "most tiles first" order = number of sequences with more tiles
+        uint32_t run = 0;
+        for (int nt = n_levels; nt >= 0; --nt) {
+            const uint32_t c = s_bucket[nt];
+            s_bucket[nt] = run;
+            run += c;
         }
-        lim = lim < 0 ? 0 : (lim > sk ? sk : lim);
-        if (n_tgt > 0 && a.target_group > 0) {
-            const int ti = row - (sq - n_tgt);
-            if (ti >= 0) {
-                hole_lo = hist_k;
-                hole_hi = hist_k + (ti / a.target_group) * a.target_group;
+        // level l holds query tile qt = n_levels - 1 - l of every sequence that has more than qt tiles,
+        // for every head: s_bucket[qt] sequences (the start of bucket qt counts exactly those)
+        uint32_t acc = 0;
+        for (int l = 0; l < n_levels; ++l) {
+            s_level_start[l] = acc;
+            acc += s_bucket[n_levels - 1 - l] * static_cast<uint32_t>(n_heads);
+        }
+        s_level_start[n_levels] = acc;
+    }
+    __syncthreads();
+    // Stable scatter (sequences of one bucket stay in index order) by wavefront 0 alone: every workgroup
+    // must arrive at the very same list, which an order-of-arrival scatter over four wavefronts would
+    // not give.  64 sequences per trip; lanes holding the same tile count are ranked with a ballot.
+    if (wave == 0) {
+        for (int base = 0; base < a.n_batch; base += 64) {
+            const int b = base + lane;
+            const bool valid = b < a.n_batch;
+            const int key = valid ? static_cast<int>(s_ntiles[valid ? b : 0]) : -1;
+            uint64_t todo = __builtin_amdgcn_ballot_w64(valid);
+            while (todo != 0) {
+                const int leader = __builtin_ctzll(todo);
+                const int k0 = __builtin_amdgcn_readlane(key, leader);
+                const bool mine = valid && key == k0;
+                const uint64_t same = __builtin_amdgcn_ballot_w64(mine);
+                const uint32_t start = s_bucket[k0];
+                if (mine) {
+                    const uint32_t before = __builtin_popcountll(same & ((1ull << lane) - 1ull));
+                    s_order[start + before] = static_cast<uint16_t>(b);
+                }
+                if (lane == leader) {
+                    s_bucket[k0] = start + static_cast<uint32_t>(__builtin_popcountll(same));
+                }
+                todo &= ~same;
             }
         }
-    } else {
-        lim = sk;
     }
-    // wavefront-uniform bounds for tile classification
-    int lim_min = lim;
-    int lim_max = lim;
-    int hole_hi_max = hole_hi;
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) {
-        const int o_min = __shfl_xor(lim_min, off);
-        const int o_max = __shfl_xor(lim_max, off);
-        const int o_hh = __shfl_xor(hole_hi_max, off);
-        lim_min = o_min < lim_min ? o_min : lim_min;
-        lim_max = o_max > lim_max ? o_max : lim_max;
-        hole_hi_max = o_hh > hole_hi_max ? o_hh : hole_hi_max;
-    }
-    lim_min = uniform(lim_min);
-    lim_max = uniform(wave_active ? lim_max : 0);
-    hole_hi_max = uniform(hole_hi_max);
-    const bool any_hole = hole_hi_max > hist_k && n_tgt > 0 && a.target_group > 0;
+    __syncthreads();
+    const uint32_t n_items = s_level_start[n_levels];
 
-    // ---- keys needed by this workgroup ----
-    int kmax;
-    if (a.mask_type == 0) {
-        const int r1 = (r0 + kBlockM < sq) ? r0 + kBlockM : sq;
-        kmax = r1 + delta;
-        if (r0 < n_ctx) {
-            kmax = kmax > hist_k ? kmax : hist_k;
-        }
-        kmax = kmax < 0 ? 0 : (kmax > sk ? sk : kmax);
-    } else {
-        kmax = sk;
-    }
-    const int n_kt = uniform((kmax + BN - 1) / BN);
-
-    // ---- buffer descriptors sized to this sequence / head ----
+    // ---- per-lane constants that do not depend on the item ----
     const uint32_t q_stride = static_cast<uint32_t>(a.n_heads_q) * a.d_qk * 2u;  // bytes per row
     const uint32_t k_stride = static_cast<uint32_t>(a.n_heads_k) * a.d_qk * 2u;
     const uint32_t v_stride = static_cast<uint32_t>(a.n_heads_k) * a.d_v * 2u;
     const uint32_t o_stride = static_cast<uint32_t>(a.n_heads_q) * a.d_v * 2u;
-    const __amdgpu_buffer_rsrc_t q_rsrc =
-        make_rsrc(static_cast<const uint16_t*>(a.q) + (q0 * a.n_heads_q + h) * static_cast<int64_t>(a.d_qk),
-                  static_cast<uint32_t>(sq - 1) * q_stride + a.d_qk * 2u);
-    const __amdgpu_buffer_rsrc_t k_rsrc =
-        make_rsrc(static_cast<const uint16_t*>(a.k) + (k0 * a.n_heads_k + hk) * static_cast<int64_t>(a.d_qk),
-                  sk > 0 ? static_cast<uint32_t>(sk - 1) * k_stride + a.d_qk * 2u : 0u);
-    const __amdgpu_buffer_rsrc_t v_rsrc =
-        make_rsrc(static_cast<const uint16_t*>(a.v) + (k0 * a.n_heads_k + hk) * static_cast<int64_t>(a.d_v),
-                  sk > 0 ? static_cast<uint32_t>(sk - 1) * v_stride + a.d_v * 2u : 0u);
-    const __amdgpu_buffer_rsrc_t o_rsrc =
-        make_rsrc(out16 + (q0 * a.n_heads_q + h) * static_cast<int64_t>(a.d_v),
-                  static_cast<uint32_t>(sq - 1) * o_stride + a.d_v * 2u);
-
-    // ---- Q fragment: lane (ln, lh) holds Q[row][16*js + 8*lh .. +7] for js = 0..KSTEPS-1 ----
-    u32x4_t qf[KSTEPS];
-    {
-        const uint32_t row_off = static_cast<uint32_t>(wr0 + ln) * q_stride;
-#pragma unroll
-        for (int js = 0; js < KSTEPS; ++js) {
-            const int d0 = 16 * js + 8 * lh;
-            const uint32_t off = (d0 < a.d_qk) ? row_off + d0 * 2u : kOutOfRange;
-            qf[js] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, static_cast<int>(off), 0, 0);
-        }
-    }
-
-    // ---- K / V tile streaming: per-lane source offsets are fixed, only the tile base moves ----
-    // load instruction i of this wavefront fills LDS bytes [(wave * LOADS + i) * 1024, +1024)
+    // K / V tile streaming: load instruction i of this wavefront fills LDS bytes
+    // [(wave * LOADS + i) * 1024, +1024); per-lane source offsets are fixed, only the tile base moves
     uint32_t k_src[LOADS];
     uint32_t v_src[LOADS];
 #pragma unroll
@@ -483,68 +451,8 @@ __global__ __launch_bounds__(256 * NKH, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel
         k_src[i] = (kc * 8 < a.d_qk) ? static_cast<uint32_t>(r) * k_stride + kc * 16u : kOutOfRange;
         v_src[i] = (vc * 8 < a.d_v) ? static_cast<uint32_t>(r) * v_stride + vc * 16u : kOutOfRange;
     }
-    auto issue_tile = [&](int kt, uint16_t* dst_k, uint16_t* dst_v) {
-        const uint32_t kb = static_cast<uint32_t>(kt * BN) * k_stride;
-        const uint32_t vb = static_cast<uint32_t>(kt * BN) * v_stride;
-#pragma unroll
-        for (int i = 0; i < LOADS; ++i) {
-            uint16_t* wk = dst_k + (wave * LOADS + i) * 512;
-            uint16_t* wv = dst_v + (wave * LOADS + i) * 512;
-            // kOutOfRange + tile base stays out of range: tile bases are far below 2^31
-            load_to_lds_b128(k_rsrc, wk, k_src[i] + kb);
-            load_to_lds_b128(v_rsrc, wv, v_src[i] + vb);
-        }
-    };
-
-    // ---- rab / custom mask: per (sequence, head) descriptor, rows indexed by the local (i, j) ----
-    const uint32_t bias_bytes = static_cast<uint32_t>(a.max_q) * static_cast<uint32_t>(a.max_k) * 2u;
-    const int64_t bias_plane = (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k);
-    const __amdgpu_buffer_rsrc_t rab_rsrc =
-        make_rsrc(HAS_RAB ? static_cast<const uint16_t*>(a.rab) + bias_plane : nullptr, HAS_RAB ? bias_bytes : 0u);
-    const __amdgpu_buffer_rsrc_t mask_rsrc =
-        make_rsrc(HAS_MASK ? static_cast<const uint16_t*>(a.mask) + bias_plane : nullptr, HAS_MASK ? bias_bytes : 0u);
-    const uint32_t bias_row_off = static_cast<uint32_t>(wr0 + ln) * static_cast<uint32_t>(a.max_k) * 2u;
-    const bool bias_vec = a.bias_vec_ok != 0;
-
-    // loads the 16 bias (or mask) values of one 32-key sub-tile in accumulator order, as 8 packed words
-    auto load_bias = [&](__amdgpu_buffer_rsrc_t rsrc, int c0, uint32_t (&w)[8]) {
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const uint32_t off = bias_row_off + static_cast<uint32_t>(c0 + 8 * g + 4 * lh) * 2u;
-            if (bias_vec) {
-                const u32x2_t t = __builtin_amdgcn_raw_buffer_load_b64(rsrc, static_cast<int>(off), 0, 0);
-                w[2 * g + 0] = t[0];
-                w[2 * g + 1] = t[1];
-            } else {
-                // the offset is laundered through an empty asm so that the optimiser cannot relate these
-                // element loads to the vector load of the other branch (it otherwise folds the two and
-                // replicates the first element)
-                uint32_t eoff = off;
-                asm volatile("" : "+v"(eoff));
-                const uint32_t e0 = __builtin_amdgcn_raw_buffer_load_b16(rsrc, static_cast<int>(eoff), 0, 0);
-                const uint32_t e1 = __builtin_amdgcn_raw_buffer_load_b16(rsrc, static_cast<int>(eoff + 2u), 0, 0);
-                const uint32_t e2 = __builtin_amdgcn_raw_buffer_load_b16(rsrc, static_cast<int>(eoff + 4u), 0, 0);
-                const uint32_t e3 = __builtin_amdgcn_raw_buffer_load_b16(rsrc, static_cast<int>(eoff + 6u), 0, 0);
-                w[2 * g + 0] = (e0 & 0xffffu) | (e1 << 16);
-                w[2 * g + 1] = (e2 & 0xffffu) | (e3 << 16);
-            }
-        }
-    };
-
-    f32x16_t o_acc[MTILES];
-#pragma unroll
-    for (int mt = 0; mt < MTILES; ++mt) {
-#pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            o_acc[mt][i] = 0.f;
-        }
-    }
-
-    const float c_exp = a.c_exp;
-
-    // ---- per-lane LDS read offsets (in elements, relative to a tile), fixed for the whole kernel;
-    //      sub-tile / MFMA-step / buffer displacements are compile-time constants on top of them
-    //      (the swizzles only look at row bits that such displacements leave unchanged) ----
+    // LDS read offsets (in elements, relative to a tile); sub-tile / MFMA-step / buffer displacements are
+    // compile-time constants on top of them (the swizzles only look at row bits such displacements keep)
     int k_lane_off[KSTEPS];
 #pragma unroll
     for (int js = 0; js < KSTEPS; ++js) {
@@ -559,329 +467,509 @@ __global__ __launch_bounds__(256 * NKH, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel
             v_lane_off[mt] = vr0 * D + v_chunk_swizzle<D>(vr0, col >> 3) * 8 + (col & 7);
         }
     }
+    const float c_exp = a.c_exp;
+    const float c_out = a.c_out;
+    const bool bias_vec = a.bias_vec_ok != 0;
 
-    // one MFMA step of S^T for sub-tile ms
-    auto qk_step = [&](const uint16_t* k_tile, int ms, int js, f32x16_t acc) -> f32x16_t {
-        const u32x4_t ka = *reinterpret_cast<const u32x4_t*>(k_tile + k_lane_off[js] + ms * 32 * D);
-        return mfma32<Tag>(ka, qf[js], acc);
-    };
-    // one MFMA of O^T += V^T . P^T : keys 16*j2 .. 16*j2+15 of sub-tile ms, output dims 32*mt .. +31
-    auto pv_step = [&](const uint16_t* v_tile, int ms, int j2, int mt, const uint32_t (&pk)[8]) {
-        const u32x4_t pb = {pk[4 * j2 + 0], pk[4 * j2 + 1], pk[4 * j2 + 2], pk[4 * j2 + 3]};
-        const uint16_t* p = v_tile + v_lane_off[mt] + (ms * 32 + 16 * j2) * D;
-        const u32x2_t lo = lds_read_tr16_b64(p);
-        const u32x2_t hi = lds_read_tr16_b64(p + 8 * D);
-        const u32x4_t va = {lo[0], lo[1], hi[0], hi[1]};
-        o_acc[mt] = mfma32<Tag>(va, pb, o_acc[mt]);
-    };
-    // unscaled P^T = S^T * sigmoid(alpha * S^T) for keys 8g + 4lh + 0..3 of this lane's row, packed
-    auto silu_group = [&](const f32x16_t& s, int g, uint32_t (&pk)[8]) {
-        float p[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            const float sv = s[4 * g + e];
-            const float ex = __builtin_amdgcn_exp2f(sv * c_exp);
-            p[e] = sv * __builtin_amdgcn_rcpf(1.0f + ex);
+    // =============================== item loop ===============================
+    uint32_t idx = blockIdx.x;
+    int lvl = 0;
+    while (idx < n_items) {
+        while (idx >= s_level_start[lvl + 1]) {
+            ++lvl;
         }
-        pk[2 * g + 0] = pack2<Tag>(p[0], p[1]);
-        pk[2 * g + 1] = pack2<Tag>(p[2], p[3]);
-    };
-    auto init_scores = [&](int c0, f32x16_t& s) {
-        if constexpr (HAS_RAB) {
-            uint32_t w[8];
-            load_bias(rab_rsrc, c0, w);
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                s[2 * i + 0] = lo_to_float<Tag>(w[i]);
-                s[2 * i + 1] = hi_to_float<Tag>(w[i]);
+        const int qt = n_levels - 1 - lvl;
+        const int in_level = static_cast<int>(idx - s_level_start[lvl]);
+        const int rank = in_level / n_heads;
+        const int h = in_level - rank * n_heads;
+        const int b = uniform(static_cast<int>(s_order[rank]));
+        const int hk = h / a.head_ratio;
+#ifdef HSTU_TIMELINE
+        int log_slot = 0;
+        if (a.timeline && lane == 0) {
+            unsigned long long* row = a.timeline + (static_cast<int64_t>(blockIdx.x) * 4 + wave) * 64;
+            log_slot = static_cast<int>(row[0]);
+            if (log_slot < 15) {
+                row[1 + 4 * log_slot + 0] = idx;
+                row[1 + 4 * log_slot + 1] = HSTU_CLOCK();
             }
+        }
+#endif
+
+        int64_t q0 = load_index_uniform(a.offs_q, b, a.idx64);
+        int64_t q1 = load_index_uniform(a.offs_q, b + 1, a.idx64);
+        int64_t k0 = load_index_uniform(a.offs_k, b, a.idx64);
+        int64_t k1 = load_index_uniform(a.offs_k, b + 1, a.idx64);
+        // defensive clamps: malformed offsets must not turn into out-of-bounds addresses
+        q1 = q1 < a.total_q ? q1 : a.total_q;
+        k1 = k1 < a.total_k ? k1 : a.total_k;
+        q0 = q0 < 0 ? 0 : q0;
+        k0 = k0 < 0 ? 0 : k0;
+        int sq = static_cast<int>(q1 > q0 ? q1 - q0 : 0);
+        int sk = static_cast<int>(k1 > k0 ? k1 - k0 : 0);
+        sq = sq < a.max_q ? sq : a.max_q;
+        sk = sk < a.max_k ? sk : a.max_k;
+
+        const int r0 = qt * kBlockM;  // < sq by construction of the work list
+        const int wr0 = r0 + wave * kWaveM;
+        const bool wave_active = wr0 < sq;  // inactive wavefronts still take part in loads and barriers
+
+        int n_ctx = 0;
+        int n_tgt = 0;
+        if (a.mask_type == 0) {
+            if (a.num_ctx) {
+                n_ctx = static_cast<int>(load_index_uniform(a.num_ctx, b, a.idx64));
+            }
+            if (a.num_tgt) {
+                n_tgt = static_cast<int>(load_index_uniform(a.num_tgt, b, a.idx64));
+            }
+            n_ctx = n_ctx < 0 ? 0 : n_ctx;
+            n_tgt = n_tgt < 0 ? 0 : (n_tgt > sk ? sk : n_tgt);
+        }
+        const int delta = sk - sq;
+        const int hist_k = sk - n_tgt;  // keys before the target block
+
+        // ---- buffer descriptors sized to this sequence / head ----
+        const __amdgpu_buffer_rsrc_t q_rsrc =
+            make_rsrc(static_cast<const uint16_t*>(a.q) + (q0 * a.n_heads_q + h) * static_cast<int64_t>(a.d_qk),
+                      static_cast<uint32_t>(sq - 1) * q_stride + a.d_qk * 2u);
+        const __amdgpu_buffer_rsrc_t k_rsrc =
+            make_rsrc(static_cast<const uint16_t*>(a.k) + (k0 * a.n_heads_k + hk) * static_cast<int64_t>(a.d_qk),
+                      sk > 0 ? static_cast<uint32_t>(sk - 1) * k_stride + a.d_qk * 2u : 0u);
+        const __amdgpu_buffer_rsrc_t v_rsrc =
+            make_rsrc(static_cast<const uint16_t*>(a.v) + (k0 * a.n_heads_k + hk) * static_cast<int64_t>(a.d_v),
+                      sk > 0 ? static_cast<uint32_t>(sk - 1) * v_stride + a.d_v * 2u : 0u);
+        const __amdgpu_buffer_rsrc_t o_rsrc =
+            make_rsrc(out16 + (q0 * a.n_heads_q + h) * static_cast<int64_t>(a.d_v),
+                      static_cast<uint32_t>(sq - 1) * o_stride + a.d_v * 2u);
+
+        // ---- keys needed by this item ----
+        int kmax;
+        if (a.mask_type == 0) {
+            const int r1 = (r0 + kBlockM < sq) ? r0 + kBlockM : sq;
+            kmax = r1 + delta;
+            if (r0 < n_ctx) {
+                kmax = kmax > hist_k ? kmax : hist_k;
+            }
+            kmax = kmax < 0 ? 0 : (kmax > sk ? sk : kmax);
         } else {
-#pragma unroll
-            for (int i = 0; i < 16; ++i) {
-                s[i] = 0.f;
-            }
+            kmax = sk;
         }
-    };
+        const int n_kt = (kmax + BN - 1) / BN;
 
-    // one LDS tile, for this wavefront: its sub-tiles are ms = kh, kh + NKH, ...
-    auto compute_tile = [&](auto buf_const, int kt) {
-        constexpr int BUF = decltype(buf_const)::value;
-        const uint16_t* const k_tile = BUF ? s_k1 : s_k0;
-        const uint16_t* const v_tile = BUF ? s_v1 : s_v0;
-        const int cbeg = kt * BN;
-        if (cbeg + kh * 32 >= lim_max) {
-            return;  // no row of this wavefront sees any key of its sub-tiles
+        auto issue_tile = [&](int kt, uint16_t* dst_k, uint16_t* dst_v) {
+            const uint32_t kb = static_cast<uint32_t>(kt * BN) * k_stride;
+            const uint32_t vb = static_cast<uint32_t>(kt * BN) * v_stride;
+#pragma unroll
+            for (int i = 0; i < LOADS; ++i) {
+                uint16_t* wk = dst_k + (wave * LOADS + i) * 512;
+                uint16_t* wv = dst_v + (wave * LOADS + i) * 512;
+                // kOutOfRange + tile base stays out of range: tile bases are far below 2^31
+                load_to_lds_b128(k_rsrc, wk, k_src[i] + kb);
+                load_to_lds_b128(v_rsrc, wv, v_src[i] + vb);
+            }
+        };
+
+        // first K/V tile and the Q fragment are requested before the mask set-up arithmetic
+        if (n_kt > 0) {
+            issue_tile(0, s_k0, s_v0);
         }
-        const bool tile_full = !HAS_MASK && (cbeg + BN <= lim_min) &&
-                               !(any_hole && cbeg + BN > hist_k && cbeg < hole_hi_max);
-        if (tile_full) {
-            // Fast path: every element of every sub-tile is visible.
-            if constexpr (MYSUB == 2) {
-                // Two sub-tiles (a, b) per wavefront, issued as four stages of NCH chunks.  A chunk is
-                // one MFMA plus the LDS operand reads of a later chunk plus a slice of SiLU work, and
-                // chunks are fenced so that the order below is the order issued:
-                //   A: QK(a)            + reads K(b)
-                //   B: QK(b) + silu(a)  + reads V(a)
-                //   C: PV(a) + silu(b)  + reads V(b)
-                //   D: PV(b)
-                // so the matrix pipe always has an MFMA in flight while the SiLU arithmetic runs.
-                static_assert(KSTEPS == 2 * MTILES, "QK and PV stages must have the same number of MFMAs");
-                constexpr int NCH = KSTEPS;        // chunks (= MFMAs) per stage
-                constexpr int EPC = 16 / NCH;      // score elements handled per chunk
-                static_assert(NCH * EPC == 16 && EPC % 2 == 0, "chunks must cover packed pairs");
-                const int ms_a = kh;
-                const int ms_b = kh + NKH;
-                f32x16_t s_a, s_b;
-                init_scores(cbeg + ms_a * 32, s_a);
-                init_scores(cbeg + ms_b * 32, s_b);
-                uint32_t pk_a[8], pk_b[8];
-                auto read_k = [&](int ms, int js) -> u32x4_t {
-                    return *reinterpret_cast<const u32x4_t*>(k_tile + k_lane_off[js] + ms * 32 * D);
-                };
-                auto read_v = [&](int ms, int t) -> u32x4_t {
-                    const int j2 = t / MTILES, mt = t % MTILES;
-                    const uint16_t* p = v_tile + v_lane_off[mt] + (ms * 32 + 16 * j2) * D;
-                    const u32x2_t lo = lds_read_tr16_b64(p);
-                    const u32x2_t hi = lds_read_tr16_b64(p + 8 * D);
-                    const u32x4_t r = {lo[0], lo[1], hi[0], hi[1]};
-                    return r;
-                };
-                // LDS operand of chunk c (0 .. 4 * NCH - 1), read LOOKAHEAD chunks before its MFMA
-                auto read_operand = [&](int c) -> u32x4_t {
-                    const int stage = c / NCH, i = c % NCH;
-                    return stage == 0 ? read_k(ms_a, i)
-                           : stage == 1 ? read_k(ms_b, i)
-                           : stage == 2 ? read_v(ms_a, i)
-                                        : read_v(ms_b, i);
-                };
-                auto silu_chunk = [&](const f32x16_t& sc, int i, uint32_t (&pk)[8]) {
-                    float t[EPC], p[EPC];
-#pragma unroll
-                    for (int e = 0; e < EPC; ++e) {
-                        t[e] = sc[i * EPC + e] * c_exp;
-                    }
-#pragma unroll
-                    for (int e = 0; e < EPC; ++e) {
-                        t[e] = __builtin_amdgcn_exp2f(t[e]);
-                    }
-#pragma unroll
-                    for (int e = 0; e < EPC; ++e) {
-                        t[e] = 1.0f + t[e];
-                    }
-#pragma unroll
-                    for (int e = 0; e < EPC; ++e) {
-                        t[e] = __builtin_amdgcn_rcpf(t[e]);
-                    }
-#pragma unroll
-                    for (int e = 0; e < EPC; ++e) {
-                        p[e] = sc[i * EPC + e] * t[e];
-                    }
-#pragma unroll
-                    for (int e = 0; e < EPC; e += 2) {
-                        pk[(i * EPC + e) / 2] = pack2<Tag>(p[e], p[e + 1]);
-                    }
-                };
-                constexpr int LOOKAHEAD = 3;
-                u32x4_t opnd[4 * NCH];
-#pragma unroll
-                for (int c = 0; c < LOOKAHEAD; ++c) {
-                    opnd[c] = read_operand(c);
-                }
-                __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                for (int c = 0; c < 4 * NCH; ++c) {
-                    const int stage = c / NCH, i = c % NCH;
-                    const int j2 = i / MTILES, mt = i % MTILES;
-                    if (stage == 0) {
-                        s_a = mfma32<Tag>(opnd[c], qf[i], s_a);
-                    } else if (stage == 1) {
-                        s_b = mfma32<Tag>(opnd[c], qf[i], s_b);
-                    } else if (stage == 2) {
-                        const u32x4_t pb = {pk_a[4 * j2 + 0], pk_a[4 * j2 + 1], pk_a[4 * j2 + 2], pk_a[4 * j2 + 3]};
-                        o_acc[mt] = mfma32<Tag>(opnd[c], pb, o_acc[mt]);
-                    } else {
-                        const u32x4_t pb = {pk_b[4 * j2 + 0], pk_b[4 * j2 + 1], pk_b[4 * j2 + 2], pk_b[4 * j2 + 3]};
-                        o_acc[mt] = mfma32<Tag>(opnd[c], pb, o_acc[mt]);
-                    }
-                    if (c + LOOKAHEAD < 4 * NCH) {
-                        opnd[c + LOOKAHEAD] = read_operand(c + LOOKAHEAD);
-                    }
-                    if (stage == 1) {
-                        silu_chunk(s_a, i, pk_a);
-                    } else if (stage == 2) {
-                        silu_chunk(s_b, i, pk_b);
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
-                }
-            } else {
-                f32x16_t s[MYSUB];
-                uint32_t pk[MYSUB][8];
-#pragma unroll
-                for (int u = 0; u < MYSUB; ++u) {
-                    init_scores(cbeg + (kh + u * NKH) * 32, s[u]);
-                }
-#pragma unroll
-                for (int u = 0; u < MYSUB; ++u) {
-#pragma unroll
-                    for (int js = 0; js < KSTEPS; ++js) {
-                        s[u] = qk_step(k_tile, kh + u * NKH, js, s[u]);
-                    }
-                }
-#pragma unroll
-                for (int u = 0; u < MYSUB; ++u) {
-#pragma unroll
-                    for (int g = 0; g < 4; ++g) {
-                        silu_group(s[u], g, pk[u]);
-                    }
-#pragma unroll
-                    for (int t = 0; t < 2 * MTILES; ++t) {
-                        pv_step(v_tile, kh + u * NKH, t / MTILES, t % MTILES, pk[u]);
-                    }
-                }
-            }
-            return;
-        }
-        // general path: per sub-tile skip / mask
-        for (int ms = kh; ms < NSUB; ms += NKH) {
-            const int c0 = cbeg + ms * 32;
-            if (c0 >= lim_max) {
-                break;
-            }
-            f32x16_t s;
-            init_scores(c0, s);
-            uint32_t mw[8];
-            if constexpr (HAS_MASK) {
-                load_bias(mask_rsrc, c0, mw);
-            }
+        // Q fragment: lane (ln, lh) holds Q[row][16*js + 8*lh .. +7] for js = 0..KSTEPS-1
+        u32x4_t qf[KSTEPS];
+        {
+            const uint32_t row_off = static_cast<uint32_t>(wr0 + ln) * q_stride;
 #pragma unroll
             for (int js = 0; js < KSTEPS; ++js) {
-                s = qk_step(k_tile, ms, js, s);
+                const int d0 = 16 * js + 8 * lh;
+                const uint32_t off = (d0 < a.d_qk) ? row_off + d0 * 2u : kOutOfRange;
+                qf[js] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, static_cast<int>(off), 0, 0);
             }
-            uint32_t pk[8];
+        }
+
+        // ---- per-row visibility constants (row = this lane's query row, clamped into the sequence) ----
+        //   visible(j) = j < lim  &&  !(hole_lo <= j < hole_hi)
+        int row = wr0 + ln;
+        row = row < sq - 1 ? row : sq - 1;
+        int lim;
+        int hole_lo = 0;
+        int hole_hi = 0;
+        if (a.mask_type == 0) {
+            lim = row + delta + 1;
+            if (row < n_ctx) {
+                lim = lim > hist_k ? lim : hist_k;
+            }
+            lim = lim < 0 ? 0 : (lim > sk ? sk : lim);
+            if (n_tgt > 0 && a.target_group > 0) {
+                const int ti = row - (sq - n_tgt);
+                if (ti >= 0) {
+                    hole_lo = hist_k;
+                    hole_hi = hist_k + (ti / a.target_group) * a.target_group;
+                }
+            }
+        } else {
+            lim = sk;
+        }
+        const WaveBounds wb = wave_bounds(a.mask_type, wr0, sq, sk, n_ctx, n_tgt, a.target_group, wave_active);
+        const int lim_min = wb.lim_min;
+        const int lim_max = wb.lim_max;
+        const int hole_hi_max = wb.hole_hi_max;
+        const bool any_hole = wb.any_hole;
+
+        // ---- rab / custom mask: per (sequence, head) descriptor, rows indexed by the local (i, j) ----
+        const uint32_t bias_bytes = static_cast<uint32_t>(a.max_q) * static_cast<uint32_t>(a.max_k) * 2u;
+        const int64_t bias_plane =
+            (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k);
+        const __amdgpu_buffer_rsrc_t rab_rsrc =
+            make_rsrc(HAS_RAB ? static_cast<const uint16_t*>(a.rab) + bias_plane : nullptr, HAS_RAB ? bias_bytes : 0u);
+        const __amdgpu_buffer_rsrc_t mask_rsrc = make_rsrc(
+            HAS_MASK ? static_cast<const uint16_t*>(a.mask) + bias_plane : nullptr, HAS_MASK ? bias_bytes : 0u);
+        const uint32_t bias_row_off = static_cast<uint32_t>(wr0 + ln) * static_cast<uint32_t>(a.max_k) * 2u;
+
+        // loads the 16 bias (or mask) values of one 32-key sub-tile in accumulator order, as 8 packed words
+        auto load_bias = [&](__amdgpu_buffer_rsrc_t rsrc, int c0, uint32_t (&w)[8]) {
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                float p[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const float sv = s[4 * g + e];
-                    const float ex = __builtin_amdgcn_exp2f(sv * c_exp);
-                    p[e] = sv * __builtin_amdgcn_rcpf(1.0f + ex);
+                const uint32_t off = bias_row_off + static_cast<uint32_t>(c0 + 8 * g + 4 * lh) * 2u;
+                if (bias_vec) {
+                    // (reinterpreted as a struct before its words are taken: taking integer elements
+                    // straight from the builtin's vector result is narrowed to a one-element load by the
+                    // optimiser of this toolchain)
+                    const U32Pair t = __builtin_bit_cast(
+                        U32Pair, __builtin_amdgcn_raw_buffer_load_b64(rsrc, static_cast<int>(off), 0, 0));
+                    w[2 * g + 0] = t.v[0];
+                    w[2 * g + 1] = t.v[1];
+                } else {
+                    // the offset is laundered through an empty asm so that the optimiser cannot relate
+                    // these element loads to the vector load of the other branch
+                    uint32_t eoff = off;
+                    asm volatile("" : "+v"(eoff));
+                    const uint32_t e0 = __builtin_amdgcn_raw_buffer_load_b16(rsrc, static_cast<int>(eoff), 0, 0);
+                    const uint32_t e1 = __builtin_amdgcn_raw_buffer_load_b16(rsrc, static_cast<int>(eoff + 2u), 0, 0);
+                    const uint32_t e2 = __builtin_amdgcn_raw_buffer_load_b16(rsrc, static_cast<int>(eoff + 4u), 0, 0);
+                    const uint32_t e3 = __builtin_amdgcn_raw_buffer_load_b16(rsrc, static_cast<int>(eoff + 6u), 0, 0);
+                    w[2 * g + 0] = (e0 & 0xffffu) | (e1 << 16);
+                    w[2 * g + 1] = (e2 & 0xffffu) | (e3 << 16);
                 }
-                const int j = c0 + 8 * g + 4 * lh;
+            }
+        };
+
+        f32x16_t o_acc[MTILES];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    const int jj = j + e;
-                    const bool vis = (jj < lim) && !(jj >= hole_lo && jj < hole_hi);
-                    p[e] = vis ? p[e] : 0.f;
+        for (int mt = 0; mt < MTILES; ++mt) {
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                o_acc[mt][i] = 0.f;
+            }
+        }
+
+        // one MFMA step of S^T for sub-tile ms
+        auto qk_step = [&](const uint16_t* k_tile, int ms, int js, f32x16_t acc) -> f32x16_t {
+            const u32x4_t ka = *reinterpret_cast<const u32x4_t*>(k_tile + k_lane_off[js] + ms * 32 * D);
+            return mfma32<Tag>(ka, qf[js], acc);
+        };
+        // one MFMA of O^T += V^T . P^T : keys 16*j2 .. 16*j2+15 of sub-tile ms, output dims 32*mt .. +31
+        auto pv_step = [&](const uint16_t* v_tile, int ms, int j2, int mt, const uint32_t (&pk)[8]) {
+            const u32x4_t pb = {pk[4 * j2 + 0], pk[4 * j2 + 1], pk[4 * j2 + 2], pk[4 * j2 + 3]};
+            const uint16_t* p = v_tile + v_lane_off[mt] + (ms * 32 + 16 * j2) * D;
+            const u32x2_t lo = lds_read_tr16_b64(p);
+            const u32x2_t hi = lds_read_tr16_b64(p + 8 * D);
+            const u32x4_t va = {lo[0], lo[1], hi[0], hi[1]};
+            o_acc[mt] = mfma32<Tag>(va, pb, o_acc[mt]);
+        };
+        // unscaled P^T = S^T * sigmoid(alpha * S^T) for keys 8g + 4lh + 0..3 of this lane's row, packed
+        auto silu_group = [&](const f32x16_t& s, int g, uint32_t (&pk)[8]) {
+            float p[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float sv = s[4 * g + e];
+                const float ex = __builtin_amdgcn_exp2f(sv * c_exp);
+                p[e] = sv * __builtin_amdgcn_rcpf(1.0f + ex);
+            }
+            pk[2 * g + 0] = pack2<Tag>(p[0], p[1]);
+            pk[2 * g + 1] = pack2<Tag>(p[2], p[3]);
+        };
+        auto init_scores = [&](int c0, f32x16_t& s) {
+            if constexpr (HAS_RAB) {
+                uint32_t w[8];
+                load_bias(rab_rsrc, c0, w);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    s[2 * i + 0] = lo_to_float<Tag>(w[i]);
+                    s[2 * i + 1] = hi_to_float<Tag>(w[i]);
                 }
-                if constexpr (HAS_MASK) {
-                    p[0] *= lo_to_float<Tag>(mw[2 * g + 0]);
-                    p[1] *= hi_to_float<Tag>(mw[2 * g + 0]);
-                    p[2] *= lo_to_float<Tag>(mw[2 * g + 1]);
-                    p[3] *= hi_to_float<Tag>(mw[2 * g + 1]);
-                    // a masked-out element must stay exactly zero even if the mask word is garbage
+            } else {
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        p[e] = (j + e < lim) ? p[e] : 0.f;
+                for (int i = 0; i < 16; ++i) {
+                    s[i] = 0.f;
+                }
+            }
+        };
+
+        // one LDS tile, for this wavefront
+        auto compute_tile = [&](auto buf_const, int kt) {
+            constexpr int BUF = decltype(buf_const)::value;
+            const uint16_t* const k_tile = BUF ? s_k1 : s_k0;
+            const uint16_t* const v_tile = BUF ? s_v1 : s_v0;
+            const int cbeg = kt * BN;
+            if (cbeg >= lim_max) {
+                return;  // no row of this wavefront sees any key of this tile
+            }
+            const bool tile_full = !HAS_MASK && (cbeg + BN <= lim_min) &&
+                                   !(any_hole && cbeg + BN > hist_k && cbeg < hole_hi_max);
+            if (tile_full) {
+                // Fast path: every element of every sub-tile is visible.
+                if constexpr (NSUB == 2) {
+                    // Two sub-tiles (a, b), issued as four stages of NCH chunks.  A chunk is one MFMA plus
+                    // the LDS operand read of a later chunk plus a slice of SiLU work, and chunks are
+                    // fenced so that the order below is the order issued:
+                    //   A: QK(a)   B: QK(b) + silu(a)   C: PV(a) + silu(b)   D: PV(b)
+                    // so the matrix pipe has an MFMA in flight while the SiLU arithmetic runs.
+                    static_assert(KSTEPS == 2 * MTILES, "QK and PV stages must have the same number of MFMAs");
+                    constexpr int NCH = KSTEPS;    // chunks (= MFMAs) per stage
+                    constexpr int EPC = 16 / NCH;  // score elements handled per chunk
+                    static_assert(NCH * EPC == 16 && EPC % 2 == 0, "chunks must cover packed pairs");
+                    f32x16_t s_a, s_b;
+                    init_scores(cbeg, s_a);
+                    init_scores(cbeg + 32, s_b);
+                    uint32_t pk_a[8], pk_b[8];
+                    auto read_k = [&](int ms, int js) -> u32x4_t {
+                        return *reinterpret_cast<const u32x4_t*>(k_tile + k_lane_off[js] + ms * 32 * D);
+                    };
+                    auto read_v = [&](int ms, int t) -> u32x4_t {
+                        const int j2 = t / MTILES, mt = t % MTILES;
+                        const uint16_t* p = v_tile + v_lane_off[mt] + (ms * 32 + 16 * j2) * D;
+                        const u32x2_t lo = lds_read_tr16_b64(p);
+                        const u32x2_t hi = lds_read_tr16_b64(p + 8 * D);
+                        const u32x4_t r = {lo[0], lo[1], hi[0], hi[1]};
+                        return r;
+                    };
+                    // LDS operand of chunk c (0 .. 4 * NCH - 1), read LOOKAHEAD chunks before its MFMA
+                    auto read_operand = [&](int c) -> u32x4_t {
+                        const int stage = c / NCH, i = c % NCH;
+                        return stage == 0 ? read_k(0, i) : stage == 1 ? read_k(1, i) : stage == 2 ? read_v(0, i) : read_v(1, i);
+                    };
+                    auto silu_chunk = [&](const f32x16_t& sc, int i, uint32_t (&pk)[8]) {
+                        float t[EPC], p[EPC];
+#pragma unroll
+                        for (int e = 0; e < EPC; ++e) {
+                            t[e] = sc[i * EPC + e] * c_exp;
+                        }
+#pragma unroll
+                        for (int e = 0; e < EPC; ++e) {
+                            t[e] = __builtin_amdgcn_exp2f(t[e]);
+                        }
+#pragma unroll
+                        for (int e = 0; e < EPC; ++e) {
+                            t[e] = 1.0f + t[e];
+                        }
+#pragma unroll
+                        for (int e = 0; e < EPC; ++e) {
+                            t[e] = __builtin_amdgcn_rcpf(t[e]);
+                        }
+#pragma unroll
+                        for (int e = 0; e < EPC; ++e) {
+                            p[e] = sc[i * EPC + e] * t[e];
+                        }
+#pragma unroll
+                        for (int e = 0; e < EPC; e += 2) {
+                            pk[(i * EPC + e) / 2] = pack2<Tag>(p[e], p[e + 1]);
+                        }
+                    };
+                    constexpr int LOOKAHEAD = 3;
+                    u32x4_t opnd[4 * NCH];
+#pragma unroll
+                    for (int c = 0; c < LOOKAHEAD; ++c) {
+                        opnd[c] = read_operand(c);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int c = 0; c < 4 * NCH; ++c) {
+                        const int stage = c / NCH, i = c % NCH;
+                        const int j2 = i / MTILES, mt = i % MTILES;
+                        if (stage == 0) {
+                            s_a = mfma32<Tag>(opnd[c], qf[i], s_a);
+                        } else if (stage == 1) {
+                            s_b = mfma32<Tag>(opnd[c], qf[i], s_b);
+                        } else if (stage == 2) {
+                            const u32x4_t pb = {pk_a[4 * j2 + 0], pk_a[4 * j2 + 1], pk_a[4 * j2 + 2], pk_a[4 * j2 + 3]};
+                            o_acc[mt] = mfma32<Tag>(opnd[c], pb, o_acc[mt]);
+                        } else {
+                            const u32x4_t pb = {pk_b[4 * j2 + 0], pk_b[4 * j2 + 1], pk_b[4 * j2 + 2], pk_b[4 * j2 + 3]};
+                            o_acc[mt] = mfma32<Tag>(opnd[c], pb, o_acc[mt]);
+                        }
+                        if (c + LOOKAHEAD < 4 * NCH) {
+                            opnd[c + LOOKAHEAD] = read_operand(c + LOOKAHEAD);
+                        }
+                        if (stage == 1) {
+                            silu_chunk(s_a, i, pk_a);
+                        } else if (stage == 2) {
+                            silu_chunk(s_b, i, pk_b);
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                } else {
+                    f32x16_t s[NSUB];
+                    uint32_t pk[NSUB][8];
+#pragma unroll
+                    for (int u = 0; u < NSUB; ++u) {
+                        init_scores(cbeg + u * 32, s[u]);
+                    }
+#pragma unroll
+                    for (int u = 0; u < NSUB; ++u) {
+#pragma unroll
+                        for (int js = 0; js < KSTEPS; ++js) {
+                            s[u] = qk_step(k_tile, u, js, s[u]);
+                        }
+                    }
+#pragma unroll
+                    for (int u = 0; u < NSUB; ++u) {
+#pragma unroll
+                        for (int g = 0; g < 4; ++g) {
+                            silu_group(s[u], g, pk[u]);
+                        }
+#pragma unroll
+                        for (int t = 0; t < 2 * MTILES; ++t) {
+                            pv_step(v_tile, u, t / MTILES, t % MTILES, pk[u]);
+                        }
                     }
                 }
-                pk[2 * g + 0] = pack2<Tag>(p[0], p[1]);
-                pk[2 * g + 1] = pack2<Tag>(p[2], p[3]);
+                return;
             }
+            // general path: per sub-tile skip / mask
+            for (int ms = 0; ms < NSUB; ++ms) {
+                const int c0 = cbeg + ms * 32;
+                if (c0 >= lim_max) {
+                    break;
+                }
+                f32x16_t s;
+                init_scores(c0, s);
+                uint32_t mw[8];
+                if constexpr (HAS_MASK) {
+                    load_bias(mask_rsrc, c0, mw);
+                }
 #pragma unroll
-            for (int t = 0; t < 2 * MTILES; ++t) {
-                pv_step(v_tile, ms, t / MTILES, t % MTILES, pk);
+                for (int js = 0; js < KSTEPS; ++js) {
+                    s = qk_step(k_tile, ms, js, s);
+                }
+                uint32_t pk[8];
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    float p[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float sv = s[4 * g + e];
+                        const float ex = __builtin_amdgcn_exp2f(sv * c_exp);
+                        p[e] = sv * __builtin_amdgcn_rcpf(1.0f + ex);
+                    }
+                    const int j = c0 + 8 * g + 4 * lh;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const int jj = j + e;
+                        const bool vis = (jj < lim) && !(jj >= hole_lo && jj < hole_hi);
+                        p[e] = vis ? p[e] : 0.f;
+                    }
+                    if constexpr (HAS_MASK) {
+                        p[0] *= lo_to_float<Tag>(mw[2 * g + 0]);
+                        p[1] *= hi_to_float<Tag>(mw[2 * g + 0]);
+                        p[2] *= lo_to_float<Tag>(mw[2 * g + 1]);
+                        p[3] *= hi_to_float<Tag>(mw[2 * g + 1]);
+                        // a masked-out element must stay exactly zero even if the mask word is garbage
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            p[e] = (j + e < lim) ? p[e] : 0.f;
+                        }
+                    }
+                    pk[2 * g + 0] = pack2<Tag>(p[0], p[1]);
+                    pk[2 * g + 1] = pack2<Tag>(p[2], p[3]);
+                }
+#pragma unroll
+                for (int t = 0; t < 2 * MTILES; ++t) {
+                    pv_step(v_tile, ms, t / MTILES, t % MTILES, pk);
+                }
             }
-        }
-    };
+        };
 
-    // ---- main loop, two tiles per trip so that the LDS buffer of each half is a constant ----
-    typedef std::integral_constant<int, 0> buf0_t;
-    typedef std::integral_constant<int, 1> buf1_t;
-    HSTU_STAMP(1);
-    if (n_kt > 0) {
-        issue_tile(0, s_k0, s_v0);
-    }
-    __builtin_amdgcn_s_waitcnt(0);
-    HSTU_STAMP(2);
-    __syncthreads();
-    HSTU_STAMP(3);
-    for (int kt = 0; kt < n_kt; kt += 2) {
-        if (kt + 1 < n_kt) {
-            issue_tile(kt + 1, s_k1, s_v1);
-        }
-        compute_tile(buf0_t{}, kt);
-        HSTU_STAMP(4 + 3 * kt);
+        // ---- key sweep, two tiles per trip so that the LDS buffer of each half is a constant ----
+        typedef std::integral_constant<int, 0> buf0_t;
+        typedef std::integral_constant<int, 1> buf1_t;
         __builtin_amdgcn_s_waitcnt(0);
-        HSTU_STAMP(5 + 3 * kt);
         __syncthreads();
-        HSTU_STAMP(6 + 3 * kt);
-        if (kt + 1 >= n_kt) {
-            break;
+#ifdef HSTU_TIMELINE
+        if (a.timeline && lane == 0 && log_slot < 15) {
+            a.timeline[(static_cast<int64_t>(blockIdx.x) * 4 + wave) * 64 + 1 + 4 * log_slot + 2] = HSTU_CLOCK();
         }
-        if (kt + 2 < n_kt) {
-            issue_tile(kt + 2, s_k0, s_v0);
+#endif
+#ifdef HSTU_PROBE_NOSYNC
+        // development probe: same arithmetic, no tile loads and no barriers inside the sweep (results are
+        // meaningless); isolates the issue-bound cost of the inner loop
+        for (int kt = 0; kt < n_kt; kt += 2) {
+            compute_tile(buf0_t{}, kt);
+            if (kt + 1 >= n_kt) {
+                break;
+            }
+            compute_tile(buf1_t{}, kt + 1);
         }
-        compute_tile(buf1_t{}, kt + 1);
-        HSTU_STAMP(7 + 3 * kt);
-        __builtin_amdgcn_s_waitcnt(0);
-        HSTU_STAMP(8 + 3 * kt);
         __syncthreads();
-        HSTU_STAMP(9 + 3 * kt);
-    }
+#else
+        for (int kt = 0; kt < n_kt; kt += 2) {
+            if (kt + 1 < n_kt) {
+                issue_tile(kt + 1, s_k1, s_v1);
+            }
+            compute_tile(buf0_t{}, kt);
+            __builtin_amdgcn_s_waitcnt(0);
+            __syncthreads();
+            if (kt + 1 >= n_kt) {
+                break;
+            }
+            if (kt + 2 < n_kt) {
+                issue_tile(kt + 2, s_k0, s_v0);
+            }
+            compute_tile(buf1_t{}, kt + 1);
+            __builtin_amdgcn_s_waitcnt(0);
+            __syncthreads();
+        }
 
-    // ---- sum the partial outputs of the key lanes: lane kh = 1 hands its accumulators to lane 0
-    //      through LDS (the K/V buffers are free now), always added in the same order ----
-    if constexpr (NKH == 2) {
-        // slot (row group, i) holds one float4 per lane: conflict-free 16-byte accesses;
-        // row groups 0, 1 exchange through the first K buffer, 2, 3 through the second
-        static_assert(2 * MTILES * 4 * 64 * 16 <= TILE_ELEMS * 2, "exchange area too small");
-        float* xch = reinterpret_cast<float*>(row_group < 2 ? s_k0 : s_k1);
-        if (kh == 1) {
+#endif
+        // ---- store O: lane holds query row (wr0 + ln), dims 32*mt + 8*g + 4*lh + 0..3 ----
+        {
+            const uint32_t row_off = static_cast<uint32_t>(wr0 + ln) * o_stride;
 #pragma unroll
             for (int mt = 0; mt < MTILES; ++mt) {
 #pragma unroll
                 for (int g = 0; g < 4; ++g) {
-                    const int slot = ((row_group & 1) * MTILES + mt) * 4 + g;
-                    float4 t = make_float4(o_acc[mt][4 * g + 0], o_acc[mt][4 * g + 1], o_acc[mt][4 * g + 2],
-                                           o_acc[mt][4 * g + 3]);
-                    *reinterpret_cast<float4*>(xch + (slot * 64 + lane) * 4) = t;
+                    const int d0 = 32 * mt + 8 * g + 4 * lh;
+                    const uint32_t off = (d0 < a.d_v) ? row_off + d0 * 2u : kOutOfRange;
+                    u32x2_t w;
+                    w[0] = pack2<Tag>(o_acc[mt][4 * g + 0] * c_out, o_acc[mt][4 * g + 1] * c_out);
+                    w[1] = pack2<Tag>(o_acc[mt][4 * g + 2] * c_out, o_acc[mt][4 * g + 3] * c_out);
+                    __builtin_amdgcn_raw_buffer_store_b64(w, o_rsrc, static_cast<int>(off), 0, 0);
                 }
             }
         }
+#ifdef HSTU_TIMELINE
+        if (a.timeline && lane == 0 && log_slot < 15) {
+            unsigned long long* row = a.timeline + (static_cast<int64_t>(blockIdx.x) * 4 + wave) * 64;
+            row[1 + 4 * log_slot + 3] = HSTU_CLOCK();
+            row[0] = log_slot + 1;
+        }
+#endif
+
+        // ---- pull the next item ----
+        if (tid == 0) {
+            s_next = gridDim.x + atomicAdd(&g_work_counter[a.counter_slot], 1u);
+        }
         __syncthreads();
-        if (kh == 1) {
-            return;
-        }
-#pragma unroll
-        for (int mt = 0; mt < MTILES; ++mt) {
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int slot = ((row_group & 1) * MTILES + mt) * 4 + g;
-                const float4 t = *reinterpret_cast<const float4*>(xch + (slot * 64 + lane) * 4);
-                o_acc[mt][4 * g + 0] += t.x;
-                o_acc[mt][4 * g + 1] += t.y;
-                o_acc[mt][4 * g + 2] += t.z;
-                o_acc[mt][4 * g + 3] += t.w;
-            }
-        }
+        idx = s_next;
+        __syncthreads();  // everyone has read s_next before thread 0 may overwrite it again
     }
 
-    // ---- store O: lane holds query row (wr0 + ln), dims 32*mt + 8*g + 4*lh + 0..3 ----
-    {
-        const float c_out = a.c_out;
-        const uint32_t row_off = static_cast<uint32_t>(wr0 + ln) * o_stride;
-#pragma unroll
-        for (int mt = 0; mt < MTILES; ++mt) {
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int d0 = 32 * mt + 8 * g + 4 * lh;
-                const uint32_t off = (d0 < a.d_v) ? row_off + d0 * 2u : kOutOfRange;
-                u32x2_t w;
-                w[0] = pack2<Tag>(o_acc[mt][4 * g + 0] * c_out, o_acc[mt][4 * g + 1] * c_out);
-                w[1] = pack2<Tag>(o_acc[mt][4 * g + 2] * c_out, o_acc[mt][4 * g + 3] * c_out);
-                __builtin_amdgcn_raw_buffer_store_b64(w, o_rsrc, static_cast<int>(off), 0, 0);
-            }
+    // ---- leave: the last workgroup out puts the counters of this slot back to zero ----
+    if (tid == 0) {
+        const unsigned int left = atomicAdd(&g_done_counter[a.counter_slot], 1u);
+        if (left == gridDim.x - 1) {
+            g_work_counter[a.counter_slot] = 0;
+            __threadfence();
+            g_done_counter[a.counter_slot] = 0;
         }
     }
     HSTU_STAMP(63);

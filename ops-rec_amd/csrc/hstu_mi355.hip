@@ -8,6 +8,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -34,14 +35,41 @@ struct Variant {
     void (*kernel)(const hstu::FwdArgs);
     int d_pad;
     int threads;
+    int persistent_wgs_per_cu;  // > 0: persistent kernel, this many workgroups per CU; 0: one workgroup per tile
 };
 
-#define HSTU_VARIANT(tag, tagname, D, BN, NKH, RAB, MASK)                                             \
-    {"hstu_fwd_" tagname "_d" #D "_bn" #BN "_kl" #NKH "_rab" #RAB "_mask" #MASK,                       \
-     hstu::hstu_fwd_kernel<hstu::tag, D, BN, NKH, RAB, MASK>, D, 256 * NKH}
-#define HSTU_DIMS(tag, tagname, RAB, MASK)                                                               \
-    {HSTU_VARIANT(tag, tagname, 32, 64, 1, RAB, MASK), HSTU_VARIANT(tag, tagname, 64, 64, 1, RAB, MASK), \
-     HSTU_VARIANT(tag, tagname, 128, 64, 1, RAB, MASK), HSTU_VARIANT(tag, tagname, 256, 32, 1, RAB, MASK)}
+// compute units of each device, looked up once
+int compute_units(int* out)
+{
+    static int cached[64] = {0};
+    int dev = 0;
+    hipError_t err = hipGetDevice(&dev);
+    if (err != hipSuccess) {
+        return fail(HSTU_ERR_RUNTIME, "hipGetDevice failed: %s", hipGetErrorString(err));
+    }
+    if (dev < 0 || dev >= 64) {
+        dev = 0;
+    }
+    if (cached[dev] == 0) {
+        int n = 0;
+        err = hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev);
+        if (err != hipSuccess || n <= 0) {
+            return fail(HSTU_ERR_RUNTIME, "cannot read the number of compute units: %s", hipGetErrorString(err));
+        }
+        cached[dev] = n;
+    }
+    *out = cached[dev];
+    return HSTU_OK;
+}
+
+std::atomic<unsigned> g_next_counter_slot{0};
+
+#define HSTU_VARIANT(tag, tagname, D, BN, RAB, MASK, WGS)                                           \
+    {"hstu_fwd_" tagname "_d" #D "_bn" #BN "_rab" #RAB "_mask" #MASK,                              \
+     hstu::hstu_fwd_kernel<hstu::tag, D, BN, RAB, MASK>, D, 256, WGS}
+#define HSTU_DIMS(tag, tagname, RAB, MASK)                                                           \
+    {HSTU_VARIANT(tag, tagname, 32, 64, RAB, MASK, 2), HSTU_VARIANT(tag, tagname, 64, 64, RAB, MASK, 2), \
+     HSTU_VARIANT(tag, tagname, 128, 64, RAB, MASK, 2), HSTU_VARIANT(tag, tagname, 256, 32, RAB, MASK, 1)}
 
 // [dtype: bf16, f16][rab: 0, 1][custom mask: 0, 1][dim slot: 32, 64, 128, 256]
 const Variant kVariants[2][2][2][4] = {
@@ -52,7 +80,7 @@ const Variant kVariants[2][2][2][4] = {
 };
 
 #define HSTU_F32_VARIANT(D, RAB, MASK) \
-    {"hstu_fwd_f32_d" #D "_rab" #RAB "_mask" #MASK, hstu::hstu_fwd_f32_kernel<D, RAB, MASK>, D, 256}
+    {"hstu_fwd_f32_d" #D "_rab" #RAB "_mask" #MASK, hstu::hstu_fwd_f32_kernel<D, RAB, MASK>, D, 256, 0}
 #define HSTU_F32_DIMS(RAB, MASK) \
     {HSTU_F32_VARIANT(32, RAB, MASK), HSTU_F32_VARIANT(64, RAB, MASK), HSTU_F32_VARIANT(128, RAB, MASK), \
      HSTU_F32_VARIANT(256, RAB, MASK)}
@@ -261,9 +289,20 @@ HSTU_API int hstu_jagged_fwd(const hstu_jagged_fwd_params* p, void* workspace, u
 #ifdef HSTU_TIMELINE
     a.timeline = static_cast<unsigned long long*>(workspace);  // development builds only
 #endif
-    const int64_t n_blocks = static_cast<int64_t>(a.n_qtiles) * a.bh;
+    int64_t n_blocks = static_cast<int64_t>(a.n_qtiles) * a.bh;  // one per (query tile, sequence, head) slot
     if (n_blocks <= 0 || n_blocks > 0x7fffffffLL) {
         return fail(HSTU_ERR_INVALID, "grid of %lld workgroups is out of range", (long long)n_blocks);
+    }
+    if (var->persistent_wgs_per_cu > 0) {
+        // persistent kernel: a fixed number of workgroups pulls the (at most n_blocks) work items
+        int cus = 0;
+        const int rc_cu = compute_units(&cus);
+        if (rc_cu != HSTU_OK) {
+            return rc_cu;
+        }
+        const int64_t resident = static_cast<int64_t>(cus) * var->persistent_wgs_per_cu;
+        n_blocks = n_blocks < resident ? n_blocks : resident;
+        a.counter_slot = static_cast<int>(g_next_counter_slot.fetch_add(1) % hstu::kCounterSlots);
     }
     hipLaunchKernelGGL(var->kernel, dim3(static_cast<unsigned>(n_blocks)), dim3(static_cast<unsigned>(var->threads)), 0,
                        static_cast<hipStream_t>(stream), a);
