@@ -317,27 +317,53 @@ struct U32Pair {
 // ---- the kernel ---------------------------------------------------------------------------
 // Tag      : bf16_tag / f16_tag
 // D        : padded head dim used for both QK and V (32, 64, 128 or 256); real dims come from args
-// BN       : keys per LDS tile (multiple of 32)
 // HAS_RAB  : attn_bias present
 // HAS_MASK : mask_type 3 (dense custom mask multiplied in)
-template <typename Tag, int D, int BN, bool HAS_RAB, bool HAS_MASK>
+//
+// Key sweep of one item.  Keys are taken 32 at a time ("sub-tile" x = 0, 1, ...); K and V sub-tiles live
+// in two rings of four LDS slots each (sub-tile x in slot x mod 4).  One wavefront runs a three-deep
+// rolling pipeline: at time t it issues, interleaved instruction by instruction,
+//
+//     QK(t+1)   S^T(t+1) = K(t+1) . Q^T            MFMA, accumulates in one register block
+//     silu(t)   P^T(t)   = silu(S^T(t)) * mask     VALU + transcendental unit
+//     PV(t-1)   O^T     += V^T(t-1) . P^T(t-1)     MFMA, different accumulators
+//
+// so that neither the matrix pipe nor the vector ALU waits for the other and the two MFMA streams are
+// never back-to-back dependent.  Register blocks for S and P alternate with the parity of the sub-tile;
+// the loop over t is unrolled four times so that LDS slots and register blocks are compile-time.
+//
+// Ring protocol (all wavefronts of the workgroup, whether or not their rows need the sub-tile):
+//   start of time t : K slot of K(t) and V slot of V(t-2) are free -> request K(t+4) and V(t+2)
+//                     (requests past the last sub-tile are sent with an out-of-range offset: they move
+//                     no data but keep the number of requests per time step constant)
+//   end of time t   : wait until the requests made at time t-2 have landed (they are needed at t+1):
+//                     at most the requests of times t-1 and t may be outstanding; then one barrier.
+template <typename Tag, int D, bool HAS_RAB, bool HAS_MASK>
 __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const FwdArgs a)
 {
     constexpr int kThreads = 256;
-    constexpr int CPR = D / 8;                  // 16-byte chunks per row
-    constexpr int TILE_ELEMS = BN * D;
-    constexpr int LOADS = TILE_ELEMS / 512 / 4;  // 1 KiB load instructions per wavefront per tile
-    static_assert(TILE_ELEMS % 2048 == 0, "tile must split evenly over the four wavefronts");
-    constexpr int KSTEPS = D / 16;  // MFMA steps over the head dim (QK product)
-    constexpr int MTILES = D / 32;  // 32-wide output tiles over the head dim (PV product)
-    constexpr int NSUB = BN / 32;   // 32-key sub-tiles per LDS tile
+    constexpr int CPR = D / 8;                   // 16-byte chunks per row
+    constexpr int SUB_ELEMS = 32 * D;            // one 32-key sub-tile
+    constexpr int LPW = D >= 64 ? D / 64 : 1;    // 1 KiB load instructions per loading wavefront per sub-tile
+    constexpr int NLW = D >= 64 ? 4 : D / 16;    // wavefronts that take part in filling a sub-tile
+    constexpr int KSTEPS = D / 16;               // MFMA steps over the head dim (QK product)
+    constexpr int MTILES = D / 32;               // 32-wide output tiles over the head dim (PV product)
+    constexpr int NCH = KSTEPS;                  // chunks per time step: one QK MFMA + one PV MFMA each
+    static_assert(2 * MTILES == NCH, "QK and PV products must have the same number of MFMAs");
+    constexpr int VM_OUTSTANDING = 2 * 2 * LPW;  // tile requests of two time steps
+    constexpr int kWaitTiles = (VM_OUTSTANDING & 15) | (7 << 4) | (15 << 8) | ((VM_OUTSTANDING >> 4) << 14);
+    constexpr uint32_t kPastEnd = 0x40000000u;   // added to a source offset: leaves every descriptor
 
-    // four separate arrays (not one block) so that the compiler can tell the buffer being filled by
-    // the asynchronous loads from the buffer being read, and does not wait for the loads early
-    __shared__ __attribute__((aligned(1024))) uint16_t s_k0[TILE_ELEMS];
-    __shared__ __attribute__((aligned(1024))) uint16_t s_k1[TILE_ELEMS];
-    __shared__ __attribute__((aligned(1024))) uint16_t s_v0[TILE_ELEMS];
-    __shared__ __attribute__((aligned(1024))) uint16_t s_v1[TILE_ELEMS];
+    // eight separate arrays (not one block) so that the compiler can tell the slot being filled by the
+    // asynchronous loads from the slot being read, and does not wait for the loads early
+    __shared__ __attribute__((aligned(1024))) uint16_t s_k0[SUB_ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_k1[SUB_ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_k2[SUB_ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_k3[SUB_ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_v0[SUB_ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_v1[SUB_ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_v2[SUB_ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_v3[SUB_ELEMS];
     // work list
     __shared__ uint8_t s_ntiles[kMaxBatchSlots];          // query tiles of each sequence
     __shared__ uint16_t s_order[kMaxBatchSlots];          // sequences, most query tiles first
@@ -437,22 +463,21 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
     const uint32_t k_stride = static_cast<uint32_t>(a.n_heads_k) * a.d_qk * 2u;
     const uint32_t v_stride = static_cast<uint32_t>(a.n_heads_k) * a.d_v * 2u;
     const uint32_t o_stride = static_cast<uint32_t>(a.n_heads_q) * a.d_v * 2u;
-    // K / V tile streaming: load instruction i of this wavefront fills LDS bytes
-    // [(wave * LOADS + i) * 1024, +1024); per-lane source offsets are fixed, only the tile base moves
-    uint32_t k_src[LOADS];
-    uint32_t v_src[LOADS];
+    // K / V sub-tile streaming: load instruction i of this wavefront fills LDS bytes
+    // [(wave * LPW + i) * 1024, +1024) of a slot; per-lane source offsets are fixed, only the base moves
+    uint32_t k_src[LPW];
+    uint32_t v_src[LPW];
 #pragma unroll
-    for (int i = 0; i < LOADS; ++i) {
-        const int slot = (wave * LOADS + i) * 64 + lane;  // 16-byte slot within the tile
-        const int r = slot / CPR;
-        const int pc = slot - r * CPR;
+    for (int i = 0; i < LPW; ++i) {
+        const int slot = (wave * LPW + i) * 64 + lane;  // 16-byte slot within the sub-tile
+        const int r = (slot / CPR) & 31;
+        const int pc = slot % CPR;
         const int kc = k_chunk_swizzle<D>(r, pc);  // XOR swizzles are their own inverse
         const int vc = v_chunk_swizzle<D>(r, pc);
         k_src[i] = (kc * 8 < a.d_qk) ? static_cast<uint32_t>(r) * k_stride + kc * 16u : kOutOfRange;
         v_src[i] = (vc * 8 < a.d_v) ? static_cast<uint32_t>(r) * v_stride + vc * 16u : kOutOfRange;
     }
-    // LDS read offsets (in elements, relative to a tile); sub-tile / MFMA-step / buffer displacements are
-    // compile-time constants on top of them (the swizzles only look at row bits such displacements keep)
+    // LDS read offsets (in elements, relative to a sub-tile)
     int k_lane_off[KSTEPS];
 #pragma unroll
     for (int js = 0; js < KSTEPS; ++js) {
@@ -470,6 +495,31 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
     const float c_exp = a.c_exp;
     const float c_out = a.c_out;
     const bool bias_vec = a.bias_vec_ok != 0;
+
+    auto k_slot = [&](auto ic) -> uint16_t* {
+        constexpr int I = decltype(ic)::value & 3;
+        if constexpr (I == 0) {
+            return s_k0;
+        } else if constexpr (I == 1) {
+            return s_k1;
+        } else if constexpr (I == 2) {
+            return s_k2;
+        } else {
+            return s_k3;
+        }
+    };
+    auto v_slot = [&](auto ic) -> uint16_t* {
+        constexpr int I = decltype(ic)::value & 3;
+        if constexpr (I == 0) {
+            return s_v0;
+        } else if constexpr (I == 1) {
+            return s_v1;
+        } else if constexpr (I == 2) {
+            return s_v2;
+        } else {
+            return s_v3;
+        }
+    };
 
     // =============================== item loop ===============================
     uint32_t idx = blockIdx.x;
@@ -555,25 +605,39 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         } else {
             kmax = sk;
         }
-        const int n_kt = (kmax + BN - 1) / BN;
+        const int n_sub = (kmax + 31) / 32;  // sub-tiles swept by the workgroup
 
-        auto issue_tile = [&](int kt, uint16_t* dst_k, uint16_t* dst_v) {
-            const uint32_t kb = static_cast<uint32_t>(kt * BN) * k_stride;
-            const uint32_t vb = static_cast<uint32_t>(kt * BN) * v_stride;
+        // requests for K sub-tile xk into K slot KS and V sub-tile xv into V slot VS
+        auto request_k = [&](auto ks, int xk) {
+            if (NLW == 4 || wave < NLW) {
+                const uint32_t kb = (xk < n_sub) ? static_cast<uint32_t>(xk * 32) * k_stride : kPastEnd;
+                uint16_t* const dst = k_slot(ks);
 #pragma unroll
-            for (int i = 0; i < LOADS; ++i) {
-                uint16_t* wk = dst_k + (wave * LOADS + i) * 512;
-                uint16_t* wv = dst_v + (wave * LOADS + i) * 512;
-                // kOutOfRange + tile base stays out of range: tile bases are far below 2^31
-                load_to_lds_b128(k_rsrc, wk, k_src[i] + kb);
-                load_to_lds_b128(v_rsrc, wv, v_src[i] + vb);
+                for (int i = 0; i < LPW; ++i) {
+                    load_to_lds_b128(k_rsrc, dst + (wave * LPW + i) * 512, k_src[i] + kb);
+                }
             }
         };
+        auto request_v = [&](auto vs, int xv) {
+            if (NLW == 4 || wave < NLW) {
+                const uint32_t vb = (xv < n_sub) ? static_cast<uint32_t>(xv * 32) * v_stride : kPastEnd;
+                uint16_t* const dst = v_slot(vs);
+#pragma unroll
+                for (int i = 0; i < LPW; ++i) {
+                    load_to_lds_b128(v_rsrc, dst + (wave * LPW + i) * 512, v_src[i] + vb);
+                }
+            }
+        };
+        typedef std::integral_constant<int, 0> ic0_t;
+        typedef std::integral_constant<int, 1> ic1_t;
+        typedef std::integral_constant<int, 2> ic2_t;
+        typedef std::integral_constant<int, 3> ic3_t;
 
-        // first K/V tile and the Q fragment are requested before the mask set-up arithmetic
-        if (n_kt > 0) {
-            issue_tile(0, s_k0, s_v0);
-        }
+        // ---- start-up: what the times before the first would have requested, and the Q fragment ----
+        request_k(ic0_t{}, 0);
+        request_v(ic0_t{}, 0);
+        request_k(ic1_t{}, 1);
+        request_k(ic2_t{}, 2);
         // Q fragment: lane (ln, lh) holds Q[row][16*js + 8*lh .. +7] for js = 0..KSTEPS-1
         u32x4_t qf[KSTEPS];
         {
@@ -611,9 +675,13 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         }
         const WaveBounds wb = wave_bounds(a.mask_type, wr0, sq, sk, n_ctx, n_tgt, a.target_group, wave_active);
         const int lim_min = wb.lim_min;
-        const int lim_max = wb.lim_max;
         const int hole_hi_max = wb.hole_hi_max;
         const bool any_hole = wb.any_hole;
+        const int nx_w = (wb.lim_max + 31) / 32;  // sub-tiles this wavefront's rows can see (<= n_sub)
+        // per-lane bounds relative to the lane's first key of a sub-tile (key = c0 + 4*lh + kk)
+        const int lim_lane = lim - 4 * lh;
+        const int hole_lo_lane = hole_lo - 4 * lh;
+        const int hole_hi_lane = hole_hi - 4 * lh;
 
         // ---- rab / custom mask: per (sequence, head) descriptor, rows indexed by the local (i, j) ----
         const uint32_t bias_bytes = static_cast<uint32_t>(a.max_q) * static_cast<uint32_t>(a.max_k) * 2u;
@@ -661,237 +729,217 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                 o_acc[mt][i] = 0.f;
             }
         }
-
-        // one MFMA step of S^T for sub-tile ms
-        auto qk_step = [&](const uint16_t* k_tile, int ms, int js, f32x16_t acc) -> f32x16_t {
-            const u32x4_t ka = *reinterpret_cast<const u32x4_t*>(k_tile + k_lane_off[js] + ms * 32 * D);
-            return mfma32<Tag>(ka, qf[js], acc);
-        };
-        // one MFMA of O^T += V^T . P^T : keys 16*j2 .. 16*j2+15 of sub-tile ms, output dims 32*mt .. +31
-        auto pv_step = [&](const uint16_t* v_tile, int ms, int j2, int mt, const uint32_t (&pk)[8]) {
-            const u32x4_t pb = {pk[4 * j2 + 0], pk[4 * j2 + 1], pk[4 * j2 + 2], pk[4 * j2 + 3]};
-            const uint16_t* p = v_tile + v_lane_off[mt] + (ms * 32 + 16 * j2) * D;
-            const u32x2_t lo = lds_read_tr16_b64(p);
-            const u32x2_t hi = lds_read_tr16_b64(p + 8 * D);
-            const u32x4_t va = {lo[0], lo[1], hi[0], hi[1]};
-            o_acc[mt] = mfma32<Tag>(va, pb, o_acc[mt]);
-        };
-        // unscaled P^T = S^T * sigmoid(alpha * S^T) for keys 8g + 4lh + 0..3 of this lane's row, packed
-        auto silu_group = [&](const f32x16_t& s, int g, uint32_t (&pk)[8]) {
-            float p[4];
+        // register blocks of the rolling pipeline: sub-tile x uses block x & 1
+        f32x16_t s_blk0, s_blk1;     // S^T
+        uint32_t p_blk0[8], p_blk1[8];  // P^T, packed pairs
+        uint32_t rabw0[8], rabw1[8];  // rab words of sub-tile x in block x & 1
+        uint32_t mw0[8], mw1[8];      // custom mask words of sub-tile x in block x & 1
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                const float sv = s[4 * g + e];
-                const float ex = __builtin_amdgcn_exp2f(sv * c_exp);
-                p[e] = sv * __builtin_amdgcn_rcpf(1.0f + ex);
+        for (int i = 0; i < 16; ++i) {
+            s_blk0[i] = 0.f;
+            s_blk1[i] = 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            p_blk0[i] = 0;
+            p_blk1[i] = 0;
+            rabw0[i] = 0;
+            rabw1[i] = 0;
+            mw0[i] = 0;
+            mw1[i] = 0;
+        }
+        if constexpr (HAS_RAB) {
+            if (nx_w > 0) {
+                load_bias(rab_rsrc, 0, rabw0);
             }
-            pk[2 * g + 0] = pack2<Tag>(p[0], p[1]);
-            pk[2 * g + 1] = pack2<Tag>(p[2], p[3]);
-        };
-        auto init_scores = [&](int c0, f32x16_t& s) {
+
+        }
+
+        // one time step, for this wavefront; S = t mod 4
+        auto time_step = [&](auto sc, const int t) {
+            constexpr int S = decltype(sc)::value;
+            constexpr int PAR = S & 1;  // parity of t
+            const f32x16_t& s_cur = PAR ? s_blk1 : s_blk0;  // S^T(t), transformed in this step
+            f32x16_t& s_nxt = PAR ? s_blk0 : s_blk1;        // S^T(t+1), accumulated in this step
+            uint32_t(&pk_cur)[8] = PAR ? p_blk1 : p_blk0;         // P^T(t), written
+            const uint32_t(&pk_prev)[8] = PAR ? p_blk0 : p_blk1;  // P^T(t-1), consumed
+            const uint32_t(&mw_cur)[8] = PAR ? mw1 : mw0;         // custom mask words of sub-tile t
+            uint32_t(&mw_nxt)[8] = PAR ? mw0 : mw1;
+            uint32_t(&rab_far)[8] = PAR ? rabw1 : rabw0;          // receives rab(t+2)
+            const uint32_t(&rab_nxt)[8] = PAR ? rabw0 : rabw1;    // rab(t+1)
+            const uint16_t* const kt = k_slot(std::integral_constant<int, (S + 1) & 3>{});  // K(t+1)
+            const uint16_t* const vt = v_slot(std::integral_constant<int, (S + 3) & 3>{});  // V(t-1)
+            const int c0 = t * 32;
+
+            const bool do_qk = t + 1 < nx_w;
+            const bool do_silu = t >= 0 && t < nx_w;
+            const bool do_pv = t >= 1 && t <= nx_w;
+            const bool full = (c0 + 32 <= lim_min) && !(any_hole && c0 + 32 > hist_k && c0 < hole_hi_max);
+
+            // (1) bias / mask requests for later steps; they go out before the tile requests of this step so
+            //     that waiting for them never waits for a younger tile
             if constexpr (HAS_RAB) {
-                uint32_t w[8];
-                load_bias(rab_rsrc, c0, w);
+                if (t + 2 < nx_w) {
+                    load_bias(rab_rsrc, c0 + 64, rab_far);
+                }
+            }
+            if constexpr (HAS_MASK) {
+                if (t + 1 >= 0 && t + 1 < nx_w) {
+                    load_bias(mask_rsrc, c0 + 32, mw_nxt);
+                }
+            }
+            // (2) tile requests of this time step
+#if !defined(HSTU_PROBE) || HSTU_PROBE >= 2
+            request_k(sc, t + 4);
+            request_v(std::integral_constant<int, (S + 2) & 3>{}, t + 2);
+#endif
+
+            // (3) arithmetic.  Two straight-line blocks, each entered on one wavefront-uniform flag:
+            //       block A (sub-tile t-1 exists):  PV(t-1) MFMAs with the first half of silu(t) between them
+            //       block B (sub-tile t+1 exists):  QK(t+1) MFMAs with the second half of silu(t) between them
+            //     Every accumulator is updated at exactly one place in the code.  Inside a block nothing is
+            //     conditional: at the two ends of a sweep the SiLU half of a block may work on a score block
+            //     that holds no sub-tile; what it writes is never consumed.  Visibility is applied afterwards,
+            //     to the packed P^T, and only in the steps whose sub-tile is not fully visible.
+            auto read_k = [&](int js) -> u32x4_t { return *reinterpret_cast<const u32x4_t*>(kt + k_lane_off[js]); };
+            auto read_v = [&](int c) -> u32x4_t {
+                const int j2 = c / MTILES, mt = c % MTILES;
+                const uint16_t* p = vt + v_lane_off[mt] + 16 * j2 * D;
+                const u32x2_t lo = lds_read_tr16_b64(p);
+                const u32x2_t hi = lds_read_tr16_b64(p + 8 * D);
+                const u32x4_t r = {lo[0], lo[1], hi[0], hi[1]};
+                return r;
+            };
+            // unmasked P^T pair i (score elements 2i, 2i+1)
+            auto silu_pair = [&](int i) {
+                float tt[2], p[2];
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    tt[e] = s_cur[2 * i + e] * c_exp;
+                }
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    tt[e] = __builtin_amdgcn_exp2f(tt[e]);
+                }
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    tt[e] = 1.0f + tt[e];
+                }
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    tt[e] = __builtin_amdgcn_rcpf(tt[e]);
+                }
+#pragma unroll
+                for (int e = 0; e < 2; ++e) {
+                    p[e] = s_cur[2 * i + e] * tt[e];
+                }
+                if constexpr (HAS_MASK) {
+                    p[0] *= lo_to_float<Tag>(mw_cur[i]);
+                    p[1] *= hi_to_float<Tag>(mw_cur[i]);
+                }
+                pk_cur[i] = pack2<Tag>(p[0], p[1]);
+            };
+            // the pairs of one half (first = 0 or 4) that chunk c of a block takes care of
+            auto silu_chunk = [&](int first, int c) {
+#pragma unroll
+                for (int i = c * 4 / NCH; i < (c + 1) * 4 / NCH; ++i) {
+                    silu_pair(first + i);
+                }
+            };
+            constexpr int LOOKAHEAD = NCH >= 4 ? 2 : 1;
+
+            if (do_pv) {
+                u32x4_t vop[NCH];
+#pragma unroll
+                for (int c = 0; c < LOOKAHEAD; ++c) {
+                    vop[c] = read_v(c);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int c = 0; c < NCH; ++c) {
+                    const int j2 = c / MTILES, mt = c % MTILES;
+                    const u32x4_t pb = {pk_prev[4 * j2 + 0], pk_prev[4 * j2 + 1], pk_prev[4 * j2 + 2], pk_prev[4 * j2 + 3]};
+                    o_acc[mt] = mfma32<Tag>(vop[c], pb, o_acc[mt]);
+                    if (c + LOOKAHEAD < NCH) {
+                        vop[c + LOOKAHEAD] = read_v(c + LOOKAHEAD);
+                    }
+                    silu_chunk(0, c);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else if (do_silu) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    silu_pair(i);
+                }
+            }
+            if (do_qk) {
+                u32x4_t kop[NCH];
+#pragma unroll
+                for (int c = 0; c < LOOKAHEAD; ++c) {
+                    kop[c] = read_k(c);
+                }
+                if constexpr (HAS_RAB) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        s_nxt[2 * i + 0] = lo_to_float<Tag>(rab_nxt[i]);
+                        s_nxt[2 * i + 1] = hi_to_float<Tag>(rab_nxt[i]);
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                for (int c = 0; c < NCH; ++c) {
+                    if (c == 0 && !HAS_RAB) {
+                        f32x16_t zero;
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) {
+                            zero[i] = 0.f;
+                        }
+                        s_nxt = mfma32<Tag>(kop[c], qf[c], zero);
+                    } else {
+                        s_nxt = mfma32<Tag>(kop[c], qf[c], s_nxt);
+                    }
+                    if (c + LOOKAHEAD < NCH) {
+                        kop[c + LOOKAHEAD] = read_k(c + LOOKAHEAD);
+                    }
+                    silu_chunk(4, c);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            } else if (do_silu) {
+#pragma unroll
+                for (int i = 4; i < 8; ++i) {
+                    silu_pair(i);
+                }
+            }
+            // visibility: key c0 + 8*(e/4) + 4*lh + e%4 of element e is hidden at or past lim and inside the hole
+            if (do_silu && !full) {
 #pragma unroll
                 for (int i = 0; i < 8; ++i) {
-                    s[2 * i + 0] = lo_to_float<Tag>(w[i]);
-                    s[2 * i + 1] = hi_to_float<Tag>(w[i]);
-                }
-            } else {
+                    uint32_t keep = 0;
 #pragma unroll
-                for (int i = 0; i < 16; ++i) {
-                    s[i] = 0.f;
+                    for (int e = 0; e < 2; ++e) {
+                        const int el = 2 * i + e;
+                        const int kk = c0 + 8 * (el / 4) + (el % 4);  // + 4*lh is folded into the *_lane bounds
+                        const bool vis = (kk < lim_lane) && !(kk >= hole_lo_lane && kk < hole_hi_lane);
+                        keep |= vis ? (e ? 0xffff0000u : 0x0000ffffu) : 0u;
+                    }
+                    pk_cur[i] &= keep;
                 }
             }
+
+            // (4) the requests made two time steps ago have landed (mine), then everybody's
+            __builtin_amdgcn_sched_barrier(0);
+#if !defined(HSTU_PROBE)
+            __builtin_amdgcn_s_waitcnt(kWaitTiles);
+            __builtin_amdgcn_s_barrier();
+#elif HSTU_PROBE == 2 /* requests and barrier, but nobody waits for data */
+            __builtin_amdgcn_s_barrier();
+#elif HSTU_PROBE == 3 /* requests and wait, no barrier */
+            __builtin_amdgcn_s_waitcnt(kWaitTiles);
+#endif
+            __builtin_amdgcn_sched_barrier(0);
         };
 
-        // one LDS tile, for this wavefront
-        auto compute_tile = [&](auto buf_const, int kt) {
-            constexpr int BUF = decltype(buf_const)::value;
-            const uint16_t* const k_tile = BUF ? s_k1 : s_k0;
-            const uint16_t* const v_tile = BUF ? s_v1 : s_v0;
-            const int cbeg = kt * BN;
-            if (cbeg >= lim_max) {
-                return;  // no row of this wavefront sees any key of this tile
-            }
-            const bool tile_full = !HAS_MASK && (cbeg + BN <= lim_min) &&
-                                   !(any_hole && cbeg + BN > hist_k && cbeg < hole_hi_max);
-            if (tile_full) {
-                // Fast path: every element of every sub-tile is visible.
-                if constexpr (NSUB == 2) {
-                    // Two sub-tiles (a, b), issued as four stages of NCH chunks.  A chunk is one MFMA plus
-                    // the LDS operand read of a later chunk plus a slice of SiLU work, and chunks are
-                    // fenced so that the order below is the order issued:
-                    //   A: QK(a)   B: QK(b) + silu(a)   C: PV(a) + silu(b)   D: PV(b)
-                    // so the matrix pipe has an MFMA in flight while the SiLU arithmetic runs.
-                    static_assert(KSTEPS == 2 * MTILES, "QK and PV stages must have the same number of MFMAs");
-                    constexpr int NCH = KSTEPS;    // chunks (= MFMAs) per stage
-                    constexpr int EPC = 16 / NCH;  // score elements handled per chunk
-                    static_assert(NCH * EPC == 16 && EPC % 2 == 0, "chunks must cover packed pairs");
-                    f32x16_t s_a, s_b;
-                    init_scores(cbeg, s_a);
-                    init_scores(cbeg + 32, s_b);
-                    uint32_t pk_a[8], pk_b[8];
-                    auto read_k = [&](int ms, int js) -> u32x4_t {
-                        return *reinterpret_cast<const u32x4_t*>(k_tile + k_lane_off[js] + ms * 32 * D);
-                    };
-                    auto read_v = [&](int ms, int t) -> u32x4_t {
-                        const int j2 = t / MTILES, mt = t % MTILES;
-                        const uint16_t* p = v_tile + v_lane_off[mt] + (ms * 32 + 16 * j2) * D;
-                        const u32x2_t lo = lds_read_tr16_b64(p);
-                        const u32x2_t hi = lds_read_tr16_b64(p + 8 * D);
-                        const u32x4_t r = {lo[0], lo[1], hi[0], hi[1]};
-                        return r;
-                    };
-                    // LDS operand of chunk c (0 .. 4 * NCH - 1), read LOOKAHEAD chunks before its MFMA
-                    auto read_operand = [&](int c) -> u32x4_t {
-                        const int stage = c / NCH, i = c % NCH;
-                        return stage == 0 ? read_k(0, i) : stage == 1 ? read_k(1, i) : stage == 2 ? read_v(0, i) : read_v(1, i);
-                    };
-                    auto silu_chunk = [&](const f32x16_t& sc, int i, uint32_t (&pk)[8]) {
-                        float t[EPC], p[EPC];
-#pragma unroll
-                        for (int e = 0; e < EPC; ++e) {
-                            t[e] = sc[i * EPC + e] * c_exp;
-                        }
-#pragma unroll
-                        for (int e = 0; e < EPC; ++e) {
-                            t[e] = __builtin_amdgcn_exp2f(t[e]);
-                        }
-#pragma unroll
-                        for (int e = 0; e < EPC; ++e) {
-                            t[e] = 1.0f + t[e];
-                        }
-#pragma unroll
-                        for (int e = 0; e < EPC; ++e) {
-                            t[e] = __builtin_amdgcn_rcpf(t[e]);
-                        }
-#pragma unroll
-                        for (int e = 0; e < EPC; ++e) {
-                            p[e] = sc[i * EPC + e] * t[e];
-                        }
-#pragma unroll
-                        for (int e = 0; e < EPC; e += 2) {
-                            pk[(i * EPC + e) / 2] = pack2<Tag>(p[e], p[e + 1]);
-                        }
-                    };
-                    constexpr int LOOKAHEAD = 3;
-                    u32x4_t opnd[4 * NCH];
-#pragma unroll
-                    for (int c = 0; c < LOOKAHEAD; ++c) {
-                        opnd[c] = read_operand(c);
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                    for (int c = 0; c < 4 * NCH; ++c) {
-                        const int stage = c / NCH, i = c % NCH;
-                        const int j2 = i / MTILES, mt = i % MTILES;
-                        if (stage == 0) {
-                            s_a = mfma32<Tag>(opnd[c], qf[i], s_a);
-                        } else if (stage == 1) {
-                            s_b = mfma32<Tag>(opnd[c], qf[i], s_b);
-                        } else if (stage == 2) {
-                            const u32x4_t pb = {pk_a[4 * j2 + 0], pk_a[4 * j2 + 1], pk_a[4 * j2 + 2], pk_a[4 * j2 + 3]};
-                            o_acc[mt] = mfma32<Tag>(opnd[c], pb, o_acc[mt]);
-                        } else {
-                            const u32x4_t pb = {pk_b[4 * j2 + 0], pk_b[4 * j2 + 1], pk_b[4 * j2 + 2], pk_b[4 * j2 + 3]};
-                            o_acc[mt] = mfma32<Tag>(opnd[c], pb, o_acc[mt]);
-                        }
-                        if (c + LOOKAHEAD < 4 * NCH) {
-                            opnd[c + LOOKAHEAD] = read_operand(c + LOOKAHEAD);
-                        }
-                        if (stage == 1) {
-                            silu_chunk(s_a, i, pk_a);
-                        } else if (stage == 2) {
-                            silu_chunk(s_b, i, pk_b);
-                        }
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-                } else {
-                    f32x16_t s[NSUB];
-                    uint32_t pk[NSUB][8];
-#pragma unroll
-                    for (int u = 0; u < NSUB; ++u) {
-                        init_scores(cbeg + u * 32, s[u]);
-                    }
-#pragma unroll
-                    for (int u = 0; u < NSUB; ++u) {
-#pragma unroll
-                        for (int js = 0; js < KSTEPS; ++js) {
-                            s[u] = qk_step(k_tile, u, js, s[u]);
-                        }
-                    }
-#pragma unroll
-                    for (int u = 0; u < NSUB; ++u) {
-#pragma unroll
-                        for (int g = 0; g < 4; ++g) {
-                            silu_group(s[u], g, pk[u]);
-                        }
-#pragma unroll
-                        for (int t = 0; t < 2 * MTILES; ++t) {
-                            pv_step(v_tile, u, t / MTILES, t % MTILES, pk[u]);
-                        }
-                    }
-                }
-                return;
-            }
-            // general path: per sub-tile skip / mask
-            for (int ms = 0; ms < NSUB; ++ms) {
-                const int c0 = cbeg + ms * 32;
-                if (c0 >= lim_max) {
-                    break;
-                }
-                f32x16_t s;
-                init_scores(c0, s);
-                uint32_t mw[8];
-                if constexpr (HAS_MASK) {
-                    load_bias(mask_rsrc, c0, mw);
-                }
-#pragma unroll
-                for (int js = 0; js < KSTEPS; ++js) {
-                    s = qk_step(k_tile, ms, js, s);
-                }
-                uint32_t pk[8];
-#pragma unroll
-                for (int g = 0; g < 4; ++g) {
-                    float p[4];
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const float sv = s[4 * g + e];
-                        const float ex = __builtin_amdgcn_exp2f(sv * c_exp);
-                        p[e] = sv * __builtin_amdgcn_rcpf(1.0f + ex);
-                    }
-                    const int j = c0 + 8 * g + 4 * lh;
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const int jj = j + e;
-                        const bool vis = (jj < lim) && !(jj >= hole_lo && jj < hole_hi);
-                        p[e] = vis ? p[e] : 0.f;
-                    }
-                    if constexpr (HAS_MASK) {
-                        p[0] *= lo_to_float<Tag>(mw[2 * g + 0]);
-                        p[1] *= hi_to_float<Tag>(mw[2 * g + 0]);
-                        p[2] *= lo_to_float<Tag>(mw[2 * g + 1]);
-                        p[3] *= hi_to_float<Tag>(mw[2 * g + 1]);
-                        // a masked-out element must stay exactly zero even if the mask word is garbage
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            p[e] = (j + e < lim) ? p[e] : 0.f;
-                        }
-                    }
-                    pk[2 * g + 0] = pack2<Tag>(p[0], p[1]);
-                    pk[2 * g + 1] = pack2<Tag>(p[2], p[3]);
-                }
-#pragma unroll
-                for (int t = 0; t < 2 * MTILES; ++t) {
-                    pv_step(v_tile, ms, t / MTILES, t % MTILES, pk);
-                }
-            }
-        };
-
-        // ---- key sweep, two tiles per trip so that the LDS buffer of each half is a constant ----
-        typedef std::integral_constant<int, 0> buf0_t;
-        typedef std::integral_constant<int, 1> buf1_t;
+        // ---- key sweep ----
         __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
 #ifdef HSTU_TIMELINE
@@ -899,37 +947,28 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             a.timeline[(static_cast<int64_t>(blockIdx.x) * 4 + wave) * 64 + 1 + 4 * log_slot + 2] = HSTU_CLOCK();
         }
 #endif
-#ifdef HSTU_PROBE_NOSYNC
-        // development probe: same arithmetic, no tile loads and no barriers inside the sweep (results are
-        // meaningless); isolates the issue-bound cost of the inner loop
-        for (int kt = 0; kt < n_kt; kt += 2) {
-            compute_tile(buf0_t{}, kt);
-            if (kt + 1 >= n_kt) {
-                break;
+        if (n_sub > 0) {
+            int t = -1;
+            while (true) {
+                time_step(ic3_t{}, t);
+                if (++t > n_sub) {
+                    break;
+                }
+                time_step(ic0_t{}, t);
+                if (++t > n_sub) {
+                    break;
+                }
+                time_step(ic1_t{}, t);
+                if (++t > n_sub) {
+                    break;
+                }
+                time_step(ic2_t{}, t);
+                if (++t > n_sub) {
+                    break;
+                }
             }
-            compute_tile(buf1_t{}, kt + 1);
-        }
-        __syncthreads();
-#else
-        for (int kt = 0; kt < n_kt; kt += 2) {
-            if (kt + 1 < n_kt) {
-                issue_tile(kt + 1, s_k1, s_v1);
-            }
-            compute_tile(buf0_t{}, kt);
-            __builtin_amdgcn_s_waitcnt(0);
-            __syncthreads();
-            if (kt + 1 >= n_kt) {
-                break;
-            }
-            if (kt + 2 < n_kt) {
-                issue_tile(kt + 2, s_k0, s_v0);
-            }
-            compute_tile(buf1_t{}, kt + 1);
-            __builtin_amdgcn_s_waitcnt(0);
-            __syncthreads();
         }
 
-#endif
         // ---- store O: lane holds query row (wr0 + ln), dims 32*mt + 8*g + 4*lh + 0..3 ----
         {
             const uint32_t row_off = static_cast<uint32_t>(wr0 + ln) * o_stride;

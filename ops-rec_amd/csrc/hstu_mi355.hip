@@ -64,12 +64,12 @@ int compute_units(int* out)
 
 std::atomic<unsigned> g_next_counter_slot{0};
 
-#define HSTU_VARIANT(tag, tagname, D, BN, RAB, MASK, WGS)                                           \
-    {"hstu_fwd_" tagname "_d" #D "_bn" #BN "_rab" #RAB "_mask" #MASK,                              \
-     hstu::hstu_fwd_kernel<hstu::tag, D, BN, RAB, MASK>, D, 256, WGS}
+#define HSTU_VARIANT(tag, tagname, D, RAB, MASK, WGS)                                               \
+    {"hstu_fwd_" tagname "_d" #D "_rab" #RAB "_mask" #MASK,                                        \
+     hstu::hstu_fwd_kernel<hstu::tag, D, RAB, MASK>, D, 256, WGS}
 #define HSTU_DIMS(tag, tagname, RAB, MASK)                                                           \
-    {HSTU_VARIANT(tag, tagname, 32, 64, RAB, MASK, 2), HSTU_VARIANT(tag, tagname, 64, 64, RAB, MASK, 2), \
-     HSTU_VARIANT(tag, tagname, 128, 64, RAB, MASK, 2), HSTU_VARIANT(tag, tagname, 256, 32, RAB, MASK, 1)}
+    {HSTU_VARIANT(tag, tagname, 32, RAB, MASK, 2), HSTU_VARIANT(tag, tagname, 64, RAB, MASK, 2), \
+     HSTU_VARIANT(tag, tagname, 128, RAB, MASK, 2), HSTU_VARIANT(tag, tagname, 256, RAB, MASK, 1)}
 
 // [dtype: bf16, f16][rab: 0, 1][custom mask: 0, 1][dim slot: 32, 64, 128, 256]
 const Variant kVariants[2][2][2][4] = {
@@ -192,6 +192,19 @@ const Variant* select(const hstu_jagged_fwd_params* p)
         fail(HSTU_ERR_UNSUPPORTED, "head dims above 256 are not built in this library version (got %lld)",
              (long long)dmax);
         return nullptr;
+    }
+    {
+        // one sequence of one head group is addressed through a 32-bit buffer descriptor, with room above it
+        // for the offsets that mark a request as out of range
+        const int64_t esize = p->dtype == HSTU_DT_FP32 ? 4 : 2;
+        const int64_t span_q = p->max_seq_len_q * p->num_heads_q * dmax * esize;
+        const int64_t span_k = p->max_seq_len_k * p->num_heads_k * dmax * esize;
+        const int64_t span_b = p->max_seq_len_q * p->max_seq_len_k * esize;
+        if (span_q >= (1LL << 30) || span_k >= (1LL << 30) ||
+            ((p->attn_bias != nullptr || p->mask_type == HSTU_MASK_CUSTOM) && span_b >= (1LL << 31))) {
+            fail(HSTU_ERR_UNSUPPORTED, "max_seq_len x heads x head dim spans 1 GiB or more per sequence");
+            return nullptr;
+        }
     }
     if (p->dtype == HSTU_DT_FP32) {
         return &kVariantsF32[p->attn_bias != nullptr ? 1 : 0][p->mask_type == HSTU_MASK_CUSTOM ? 1 : 0][slot];
