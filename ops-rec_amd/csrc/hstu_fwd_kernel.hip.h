@@ -7,14 +7,17 @@
 // item from a device-side counter, so that the jagged, causal mix of long and short items is
 // balanced dynamically and the launch / set-up cost of a workgroup is paid once, not per tile.
 //
-// Per wavefront: its Q rows stay in registers for the whole key sweep of an item, K and V tiles
-// are streamed global -> LDS by buffer loads that write LDS directly (no register staging),
-// double-buffered, and
+// Per wavefront: its Q rows stay in registers for the whole key sweep of an item; K and V are
+// streamed global -> LDS, 32 keys at a time, by buffer loads that write LDS directly (no register
+// staging) into two four-slot rings, and
 //
-//     S^T = K . Q^T                 v_mfma_f32_32x32x16  (A = K tile from LDS, B = Q from registers)
+//     S^T = K . Q^T                 v_mfma_f32_32x32x16  (A = K sub-tile from LDS, B = Q from registers)
 //     P^T = silu(alpha * (S^T + rab^T)) * mask, rounded to the input type
 //     O^T += V^T . P^T              v_mfma_f32_32x32x16  (A = V^T via ds_read_b64_tr_b16, B = P^T)
 //     O    = (alpha * silu_scale) * O^T^T, rounded once on store
+//
+// run as a three-deep rolling pipeline (QK of the next sub-tile, SiLU of the current one, PV of the
+// previous one in the same time step), so that the matrix pipe and the vector ALU work side by side.
 //
 // Computing the transposed score means the accumulator layout of S^T (lane = query row, registers
 // = 4 consecutive keys) is exactly the B-operand layout the second product needs, so P never
@@ -789,10 +792,8 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                 }
             }
             // (2) tile requests of this time step
-#if !defined(HSTU_PROBE) || HSTU_PROBE >= 2
             request_k(sc, t + 4);
             request_v(std::integral_constant<int, (S + 2) & 3>{}, t + 2);
-#endif
 
             // (3) arithmetic.  Two straight-line blocks, each entered on one wavefront-uniform flag:
             //       block A (sub-tile t-1 exists):  PV(t-1) MFMAs with the first half of silu(t) between them
@@ -928,14 +929,8 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
 
             // (4) the requests made two time steps ago have landed (mine), then everybody's
             __builtin_amdgcn_sched_barrier(0);
-#if !defined(HSTU_PROBE)
             __builtin_amdgcn_s_waitcnt(kWaitTiles);
             __builtin_amdgcn_s_barrier();
-#elif HSTU_PROBE == 2 /* requests and barrier, but nobody waits for data */
-            __builtin_amdgcn_s_barrier();
-#elif HSTU_PROBE == 3 /* requests and wait, no barrier */
-            __builtin_amdgcn_s_waitcnt(kWaitTiles);
-#endif
             __builtin_amdgcn_sched_barrier(0);
         };
 
