@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the HSTU jagged attention forward on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2|C3|C4] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2|C3|C4|C5] [--no-cpu]
 
 A "step" is one forward over one synthetic jagged batch whose inputs already sit in HBM.
 The default workload is the configuration the headline metric is quoted on (C2: bf16, batch 32,
@@ -34,6 +34,7 @@ sys.path.insert(0, os.path.join(_ROOT, "ops-rec_amd"))
 sys.path.insert(0, _ROOT)
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA peak (published)
+PEAK_FP8_TFLOPS = 5000.0  # MI355X dense fp8 MFMA peak (published)
 PEAK_HBM_GBS = 8000.0  # MI355X HBM3E bandwidth (published)
 
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), scaled by the same
@@ -41,11 +42,11 @@ PEAK_HBM_GBS = 8000.0  # MI355X HBM3E bandwidth (published)
 MEASURED_TRAFFIC_BYTES = {"C2": 113_700_000}  # profiles/hstu_fwd_bf16_d128_C2_counters.md
 
 
-def algorithmic_bytes(w) -> int:
+def algorithmic_bytes(w, out_element_size: int) -> int:
     """Compulsory HBM traffic: Q, K, V read once, O written once, visible rab elements read once."""
     es = w.q.element_size()
     n = w.q.numel() * es + w.k.numel() * es + w.v.numel() * es
-    n += w.q.shape[0] * w.q.shape[1] * w.v.shape[2] * es
+    n += w.q.shape[0] * w.q.shape[1] * w.v.shape[2] * out_element_size
     n += w.seq_offset.numel() * w.seq_offset.element_size()
     return n
 
@@ -55,7 +56,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="C2", choices=["C2", "C3", "C4"])
+    ap.add_argument("--workload", default="C2", choices=["C2", "C3", "C4", "C5"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="after the timed steps also run 5 plain device-to-device copies of this many MiB, so that a "
@@ -90,16 +91,21 @@ def main() -> int:
     flops = oracle.causal_effective_flops(w.seq_offset.cpu(), None, n_q, d_qk, d_v, w.mask_type, ctx, tgt,
                                           w.target_group_size)  # fmt: skip
     nnz = flops // (2 * (d_qk + d_v) * n_q)
-    alg_bytes = algorithmic_bytes(w)
+    fp8 = args.workload == "C5"  # fp8-e4m3 inputs with per-head scales, bf16 output
+    extra = {}
+    if fp8:
+        (q8, qs), (k8, ks), (v8, vs) = (workloads.quantize_fp8(t) for t in (w.q, w.k, w.v))
+        w.q, w.k, w.v = q8, k8, v8
+        extra = dict(out_dtype=torch.bfloat16, q_descale=qs, k_descale=ks, v_descale=vs)
+    prepared = _ops.prepare_forward(
+        w.q, w.k, w.v, w.mask, w.attn_bias, w.mask_type, w.max_seq_len, w.max_seq_len, w.silu_scale, w.seq_offset,
+        w.seq_offset, w.num_context, w.num_target, w.target_group_size, w.alpha, **extra,
+    )  # fmt: skip
+    alg_bytes = algorithmic_bytes(w, prepared.out.element_size())
     rab_bytes = 0
     if w.attn_bias is not None:
         rab_bytes = nnz * n_q * w.attn_bias.element_size()
     alg_bytes += rab_bytes
-
-    prepared = _ops.prepare_forward(
-        w.q, w.k, w.v, w.mask, w.attn_bias, w.mask_type, w.max_seq_len, w.max_seq_len, w.silu_scale, w.seq_offset,
-        w.seq_offset, w.num_context, w.num_target, w.target_group_size, w.alpha,
-    )  # fmt: skip
     kernel_name = prepared.kernel_name()
     stream = torch.cuda.current_stream(dev)
     raw_stream = stream.cuda_stream
@@ -129,8 +135,14 @@ def main() -> int:
         del src, dst
 
     # ---- the same through the Python entry point ----
-    op = ops_rec.ascendc.attention.hstu_jagged
-    op_args = w.op_args()
+    if fp8:
+        def op(*_):
+            return ops_rec.hstu_jagged_fp8(w.q, w.k, w.v, qs, ks, vs, mask_type=w.mask_type, max_seq_len=w.max_seq_len,
+                                           silu_scale=w.silu_scale, seq_offset=w.seq_offset, alpha=w.alpha)  # fmt: skip
+        op_args = ()
+    else:
+        op = ops_rec.ascendc.attention.hstu_jagged
+        op_args = w.op_args()
     for _ in range(5):
         op(*op_args)
     torch.cuda.synchronize()
@@ -141,6 +153,7 @@ def main() -> int:
     torch.cuda.synchronize()
     py_ms = (time.perf_counter() - t0) * 1e3 / n_py
 
+    peak = PEAK_FP8_TFLOPS if fp8 else PEAK_BF16_TFLOPS
     tflops = flops / (ms_per_step * 1e-3) / 1e12
     kernel_tflops = flops / (ev_ms * 1e-3) / 1e12
     result = {
@@ -154,7 +167,7 @@ def main() -> int:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "bf16",
+        "dtype": "fp8_e4m3" if fp8 else "bf16",
         "data": "synthetic",
         "config": {
             "workload": f"{args.workload}: jagged causal HSTU attention fwd, B{len(w.lengths)} H{n_q} d{d_qk}, "
@@ -164,7 +177,7 @@ def main() -> int:
             "algorithmic_bytes_per_step": alg_bytes,
             "launch_path": "C ABI hstu_jagged_fwd, back-to-back on one stream",
         },
-        "pct_of_bf16_mfma_peak": round(100.0 * tflops / PEAK_BF16_TFLOPS, 2),
+        ("pct_of_fp8_mfma_peak" if fp8 else "pct_of_bf16_mfma_peak"): round(100.0 * tflops / peak, 2),
         "ms_per_step_events": round(ev_ms, 6),
         "ms_per_step_wall": round(wall_ms, 6),
         "ms_per_step_python_entry": round(py_ms, 6),
@@ -172,9 +185,9 @@ def main() -> int:
             "bound": "mfma",
             "kernel": kernel_name,
             "achieved": round(kernel_tflops, 3),
-            "peak": PEAK_BF16_TFLOPS,
+            "peak": peak,
             "unit": "TFLOP/s",
-            "frac": round(kernel_tflops / PEAK_BF16_TFLOPS, 4),
+            "frac": round(kernel_tflops / peak, 4),
             "traffic": MEASURED_TRAFFIC_BYTES.get(args.workload),
             "avg_launch_us": round(ev_ms * 1e3, 3),
             "hbm_achieved_GBs": round(alg_bytes / (ev_ms * 1e-3) / 1e9, 1),

@@ -102,8 +102,15 @@ typedef struct hstu_jagged_fwd_params {
     int32_t deterministic; /* accepted for signature parity; results are bitwise reproducible either way */
     int32_t reserved0;
 
-    /* extension for quantised inputs (no counterpart in the reference, whose fp8 path is unscaled):
-     * per-head dequantisation scales, device pointers, NULL = 1.0.  Ignored unless dtype is fp8. */
+    /* fp8 inputs (dtype HSTU_DT_FP8_E4M3, OCP e4m3fn; the reference takes them on its 950 target,
+     * op_host/atlas950/op_def_arch.h:23-24): S is kept in fp32, P is clamped to +-448 and re-quantised to
+     * e4m3 (round to nearest even), P.V accumulates in fp32, the output is fp16 (the reference's choice,
+     * torch_extension/hstu_jagged_plugin.cpp:53-54) or bf16.  P is quantised BEFORE silu_scale is applied
+     * (the reference quantises silu(X) * silu_scale, which for the default 1 / max_seq_len falls below
+     * e4m3's normal range); with silu_scale = 1 the two coincide.  No attn_bias / custom mask; head_dim_qk
+     * must be a multiple of 16.
+     * Extension with no counterpart in the reference (its fp8 path is unscaled): per-head dequantisation
+     * scales, x = x8 * descale[head]; device pointers, NULL = 1.0.  Ignored unless dtype is fp8. */
     const float* q_descale; /* [num_heads_q] */
     const float* k_descale; /* [num_heads_k] */
     const float* v_descale; /* [num_heads_k] */

@@ -52,6 +52,18 @@ typedef __attribute__((ext_vector_type(2))) uint32_t u32x2_t;
 
 struct bf16_tag {};
 struct f16_tag {};
+struct f8_tag {};  // OCP e4m3fn inputs; P is re-quantised to e4m3, the products run on the fp8 MFMA
+
+template <typename Tag>
+struct elem_traits {
+    static constexpr int kBytes = 2;
+    static constexpr bool kF8 = false;
+};
+template <>
+struct elem_traits<f8_tag> {
+    static constexpr int kBytes = 1;
+    static constexpr bool kF8 = true;
+};
 
 constexpr int kBlockM = 128;  // query rows per workgroup
 constexpr int kWaveM = 32;    // query rows per wavefront
@@ -106,6 +118,11 @@ struct FwdArgs {
     int bias_vec_ok; // rab / mask rows may be read 4 elements (8 bytes) at a time
     float c_exp;     // -alpha * log2(e)
     float c_out;     // alpha * silu_scale
+    float alpha;     // fp8 inputs only: the kernel folds the per-head scales in itself
+    float silu_scale;
+    const float* q_descale;  // fp8 inputs only; per head, nullptr = 1
+    const float* k_descale;
+    const float* v_descale;
     int counter_slot;  // which pair of device-side work counters this launch uses
 #ifdef HSTU_TIMELINE
     unsigned long long* timeline;
@@ -223,6 +240,21 @@ __device__ __forceinline__ uint32_t pack2<f16_tag>(float lo, float hi)
     return __builtin_bit_cast(uint32_t, r);
 }
 
+// fp8: 8 e4m3 values per operand and lane (same row / column / k mapping as the 16-bit 32x32x16 form)
+__device__ __forceinline__ f32x16_t mfma32_f8(u32x2_t a, u32x2_t b, f32x16_t c)
+{
+    return __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(__builtin_bit_cast(long, a), __builtin_bit_cast(long, b), c, 0, 0, 0);
+}
+// two floats -> two e4m3 bytes in the low (hi = false) or high half of `old`; round to nearest even.
+// The conversion turns magnitudes above 464 into NaN, so the values are clamped to the format's range first.
+template <bool HI>
+__device__ __forceinline__ uint32_t pack2_f8(float a, float b, uint32_t old)
+{
+    a = __builtin_amdgcn_fmed3f(a, -448.0f, 448.0f);
+    b = __builtin_amdgcn_fmed3f(b, -448.0f, 448.0f);
+    return static_cast<uint32_t>(__builtin_amdgcn_cvt_pk_fp8_f32(a, b, static_cast<int>(old), HI));
+}
+
 template <typename Tag>
 __device__ __forceinline__ float lo_to_float(uint32_t packed);  // element in bits 0..15
 template <typename Tag>
@@ -251,6 +283,16 @@ __device__ __forceinline__ float hi_to_float<f16_tag>(uint32_t packed)
 // ---- LDS layout ---------------------------------------------------------------------------
 // K tile: [rows][D] elements, 16-byte chunks XOR-swizzled by row so that the 32x32x16 A-operand
 // read (32 lanes = 32 consecutive rows, same logical chunk) spreads over the banks.
+template <int CPR>  // CPR = 16-byte chunks per row
+__device__ __forceinline__ int chunk_swizzle(int row, int chunk)
+{
+    if constexpr (CPR >= 16) {
+        return chunk ^ (row & 15);
+    } else {
+        constexpr int RPG = 16 / CPR;  // rows per 256 bytes
+        return chunk ^ ((row / RPG) & (CPR - 1));
+    }
+}
 template <int D>
 __device__ __forceinline__ int k_chunk_swizzle(int row, int chunk)
 {
@@ -275,6 +317,16 @@ __device__ __forceinline__ int v_chunk_swizzle(int row, int chunk)
     } else {
         return chunk;
     }
+}
+
+// 8-bit transposed read.  In each group of 16 lanes, lane s supplies the address of 8 bytes M[s][0..7];
+// lane i < 8 receives M[0][i], M[2][i], ..., M[14][i] and lane 8 + i receives M[1][i], M[3][i], ..., M[15][i].
+__device__ __forceinline__ u32x2_t lds_read_tr8_b64(const uint8_t* p)
+{
+    typedef __attribute__((ext_vector_type(2))) int i32x2_t;
+    typedef i32x2_t __attribute__((address_space(3))) * lds_ptr_t;
+    i32x2_t r = __builtin_amdgcn_ds_read_tr8_b64_v2i32((lds_ptr_t)(p));
+    return __builtin_bit_cast(u32x2_t, r);
 }
 
 __device__ __forceinline__ u32x2_t lds_read_tr16_b64(const uint16_t* p)
@@ -341,14 +393,27 @@ struct U32Pair {
 //                     no data but keep the number of requests per time step constant)
 //   end of time t   : wait until the requests made at time t-2 have landed (they are needed at t+1):
 //                     at most the requests of times t-1 and t may be outstanding; then one barrier.
-template <typename Tag, int D, bool HAS_RAB, bool HAS_MASK>
+//
+// fp8 inputs (Tag = f8_tag; OutTag picks the 16-bit output type): same structure with one-byte elements.  The
+// score is brought to its real scale (alpha x per-head dequantisation scales) before SiLU, P^T is clamped to
+// +-448 and re-quantised to e4m3 (round to nearest even) BEFORE silu_scale is applied, silu_scale and the V
+// scale are applied to the fp32 output.  K is read 16 bytes per lane for two MFMA steps at a time (k index
+// (half, byte) of step 2p / 2p+1 = dim 16 (2p + half) + byte / + 8 + byte), V^T by one 8-bit transposed read
+// per MFMA.  rab and custom masks are not available for fp8 inputs.
+template <typename Tag, typename OutTag, int D, bool HAS_RAB, bool HAS_MASK>
 __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const FwdArgs a)
 {
     constexpr int kThreads = 256;
-    constexpr int CPR = D / 8;                   // 16-byte chunks per row
-    constexpr int SUB_ELEMS = 32 * D;            // one 32-key sub-tile
-    constexpr int LPW = D >= 64 ? D / 64 : 1;    // 1 KiB load instructions per loading wavefront per sub-tile
-    constexpr int NLW = D >= 64 ? 4 : D / 16;    // wavefronts that take part in filling a sub-tile
+    constexpr bool F8 = elem_traits<Tag>::kF8;
+    constexpr uint32_t ES = elem_traits<Tag>::kBytes;  // bytes per input element
+    static_assert(!F8 || (!HAS_RAB && !HAS_MASK), "no rab / custom mask with fp8 inputs");
+    static_assert(!F8 || D >= 64, "fp8 rows are at least 64 bytes");
+    constexpr int CPR = D * ES / 16;             // 16-byte chunks per row
+    constexpr int EPC16 = 16 / ES;               // elements per 16-byte chunk
+    constexpr int SUB_ELEMS = 32 * D * ES / 2;   // one 32-key sub-tile, in 16-bit units
+    constexpr int SUB_KIB = 32 * D * ES / 1024;  // 1 KiB load instructions per sub-tile
+    constexpr int LPW = SUB_KIB >= 4 ? SUB_KIB / 4 : 1;  // ... per loading wavefront
+    constexpr int NLW = SUB_KIB >= 4 ? 4 : SUB_KIB;      // wavefronts that take part in filling a sub-tile
     constexpr int KSTEPS = D / 16;               // MFMA steps over the head dim (QK product)
     constexpr int MTILES = D / 32;               // 32-wide output tiles over the head dim (PV product)
     constexpr int NCH = KSTEPS;                  // chunks per time step: one QK MFMA + one PV MFMA each
@@ -462,10 +527,10 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
     const uint32_t n_items = s_level_start[n_levels];
 
     // ---- per-lane constants that do not depend on the item ----
-    const uint32_t q_stride = static_cast<uint32_t>(a.n_heads_q) * a.d_qk * 2u;  // bytes per row
-    const uint32_t k_stride = static_cast<uint32_t>(a.n_heads_k) * a.d_qk * 2u;
-    const uint32_t v_stride = static_cast<uint32_t>(a.n_heads_k) * a.d_v * 2u;
-    const uint32_t o_stride = static_cast<uint32_t>(a.n_heads_q) * a.d_v * 2u;
+    const uint32_t q_stride = static_cast<uint32_t>(a.n_heads_q) * a.d_qk * ES;  // bytes per row
+    const uint32_t k_stride = static_cast<uint32_t>(a.n_heads_k) * a.d_qk * ES;
+    const uint32_t v_stride = static_cast<uint32_t>(a.n_heads_k) * a.d_v * ES;
+    const uint32_t o_stride = static_cast<uint32_t>(a.n_heads_q) * a.d_v * 2u;  // the output is 16-bit
     // K / V sub-tile streaming: load instruction i of this wavefront fills LDS bytes
     // [(wave * LPW + i) * 1024, +1024) of a slot; per-lane source offsets are fixed, only the base moves
     uint32_t k_src[LPW];
@@ -475,19 +540,36 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         const int slot = (wave * LPW + i) * 64 + lane;  // 16-byte slot within the sub-tile
         const int r = (slot / CPR) & 31;
         const int pc = slot % CPR;
-        const int kc = k_chunk_swizzle<D>(r, pc);  // XOR swizzles are their own inverse
-        const int vc = v_chunk_swizzle<D>(r, pc);
-        k_src[i] = (kc * 8 < a.d_qk) ? static_cast<uint32_t>(r) * k_stride + kc * 16u : kOutOfRange;
-        v_src[i] = (vc * 8 < a.d_v) ? static_cast<uint32_t>(r) * v_stride + vc * 16u : kOutOfRange;
+        const int kc = F8 ? chunk_swizzle<CPR>(r, pc) : k_chunk_swizzle<D>(r, pc);  // XOR swizzles are their own inverse
+        const int vc = F8 ? chunk_swizzle<CPR>(r, pc) : v_chunk_swizzle<D>(r, pc);
+        k_src[i] = (kc * EPC16 < a.d_qk) ? static_cast<uint32_t>(r) * k_stride + kc * 16u : kOutOfRange;
+        v_src[i] = (vc * EPC16 < a.d_v) ? static_cast<uint32_t>(r) * v_stride + vc * 16u : kOutOfRange;
     }
-    // LDS read offsets (in elements, relative to a sub-tile)
-    int k_lane_off[KSTEPS];
-#pragma unroll
-    for (int js = 0; js < KSTEPS; ++js) {
-        k_lane_off[js] = ln * D + k_chunk_swizzle<D>(ln, 2 * js + lh) * 8;
-    }
+    // LDS read offsets relative to a sub-tile (16-bit inputs: in elements; fp8: in bytes)
+    constexpr int KREADS = F8 ? KSTEPS / 2 : KSTEPS;  // fp8: one 16-byte read feeds two MFMA steps
+    int k_lane_off[KREADS];
     int v_lane_off[MTILES];
-    {
+    if constexpr (F8) {
+#pragma unroll
+        for (int jp = 0; jp < KREADS; ++jp) {
+            k_lane_off[jp] = ln * D + chunk_swizzle<CPR>(ln, 2 * jp + lh) * 16;
+        }
+        // transposed read of 16 keys x 32 dims: source lane s of a 16-lane group g supplies 8 dims of one key,
+        //   key  = 8 * ((s / 2) / 4) + 4 * (g / 2) + (s / 2) % 4   (so that byte j of k-half g / 2 is the key P^T holds there)
+        //   dims = 32 * mt + 16 * (g % 2) + 8 * (s % 2) .. + 7
+        const int s16 = lane & 15;
+        const int g16 = lane >> 4;
+        const int key = 8 * ((s16 >> 1) >> 2) + 4 * (g16 >> 1) + ((s16 >> 1) & 3);
+#pragma unroll
+        for (int mt = 0; mt < MTILES; ++mt) {
+            const int col = 32 * mt + 16 * (g16 & 1) + 8 * (s16 & 1);
+            v_lane_off[mt] = key * D + chunk_swizzle<CPR>(key, col >> 4) * 16 + (col & 15);
+        }
+    } else {
+#pragma unroll
+        for (int js = 0; js < KREADS; ++js) {
+            k_lane_off[js] = ln * D + k_chunk_swizzle<D>(ln, 2 * js + lh) * 8;
+        }
         const int vr0 = 4 * lh + ((lane & 15) >> 2);
 #pragma unroll
         for (int mt = 0; mt < MTILES; ++mt) {
@@ -495,8 +577,9 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             v_lane_off[mt] = vr0 * D + v_chunk_swizzle<D>(vr0, col >> 3) * 8 + (col & 7);
         }
     }
-    const float c_exp = a.c_exp;
-    const float c_out = a.c_out;
+    float c_exp = a.c_exp;
+    float c_out = a.c_out;
+    float c_x = 1.0f;  // fp8 only: raw score -> alpha * (dequantised score)
     const bool bias_vec = a.bias_vec_ok != 0;
 
     auto k_slot = [&](auto ic) -> uint16_t* {
@@ -584,17 +667,28 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
 
         // ---- buffer descriptors sized to this sequence / head ----
         const __amdgpu_buffer_rsrc_t q_rsrc =
-            make_rsrc(static_cast<const uint16_t*>(a.q) + (q0 * a.n_heads_q + h) * static_cast<int64_t>(a.d_qk),
-                      static_cast<uint32_t>(sq - 1) * q_stride + a.d_qk * 2u);
+            make_rsrc(static_cast<const uint8_t*>(a.q) + (q0 * a.n_heads_q + h) * static_cast<int64_t>(a.d_qk) * ES,
+                      static_cast<uint32_t>(sq - 1) * q_stride + a.d_qk * ES);
         const __amdgpu_buffer_rsrc_t k_rsrc =
-            make_rsrc(static_cast<const uint16_t*>(a.k) + (k0 * a.n_heads_k + hk) * static_cast<int64_t>(a.d_qk),
-                      sk > 0 ? static_cast<uint32_t>(sk - 1) * k_stride + a.d_qk * 2u : 0u);
+            make_rsrc(static_cast<const uint8_t*>(a.k) + (k0 * a.n_heads_k + hk) * static_cast<int64_t>(a.d_qk) * ES,
+                      sk > 0 ? static_cast<uint32_t>(sk - 1) * k_stride + a.d_qk * ES : 0u);
         const __amdgpu_buffer_rsrc_t v_rsrc =
-            make_rsrc(static_cast<const uint16_t*>(a.v) + (k0 * a.n_heads_k + hk) * static_cast<int64_t>(a.d_v),
-                      sk > 0 ? static_cast<uint32_t>(sk - 1) * v_stride + a.d_v * 2u : 0u);
+            make_rsrc(static_cast<const uint8_t*>(a.v) + (k0 * a.n_heads_k + hk) * static_cast<int64_t>(a.d_v) * ES,
+                      sk > 0 ? static_cast<uint32_t>(sk - 1) * v_stride + a.d_v * ES : 0u);
         const __amdgpu_buffer_rsrc_t o_rsrc =
             make_rsrc(out16 + (q0 * a.n_heads_q + h) * static_cast<int64_t>(a.d_v),
                       static_cast<uint32_t>(sq - 1) * o_stride + a.d_v * 2u);
+
+        if constexpr (F8) {
+            // per-head dequantisation scales: score scale alpha * qs * ks, output scale silu_scale * vs
+            typedef const __attribute__((address_space(4))) float* cfloat_t;
+            const float qs = a.q_descale ? ((cfloat_t)(reinterpret_cast<uintptr_t>(a.q_descale)))[h] : 1.0f;
+            const float ks = a.k_descale ? ((cfloat_t)(reinterpret_cast<uintptr_t>(a.k_descale)))[hk] : 1.0f;
+            const float vs = a.v_descale ? ((cfloat_t)(reinterpret_cast<uintptr_t>(a.v_descale)))[hk] : 1.0f;
+            c_x = a.alpha * qs * ks;
+            c_exp = -1.4426950408889634f * c_x;
+            c_out = a.silu_scale * vs;
+        }
 
         // ---- keys needed by this item ----
         int kmax;
@@ -642,13 +736,14 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         request_k(ic1_t{}, 1);
         request_k(ic2_t{}, 2);
         // Q fragment: lane (ln, lh) holds Q[row][16*js + 8*lh .. +7] for js = 0..KSTEPS-1
-        u32x4_t qf[KSTEPS];
+        // (fp8: 16 bytes per pair of steps, dims 16 * (2 * jp + lh) .. + 15, low half for step 2 jp)
+        u32x4_t qf[KREADS];
         {
             const uint32_t row_off = static_cast<uint32_t>(wr0 + ln) * q_stride;
 #pragma unroll
-            for (int js = 0; js < KSTEPS; ++js) {
-                const int d0 = 16 * js + 8 * lh;
-                const uint32_t off = (d0 < a.d_qk) ? row_off + d0 * 2u : kOutOfRange;
+            for (int js = 0; js < KREADS; ++js) {
+                const int d0 = F8 ? 32 * js + 16 * lh : 16 * js + 8 * lh;
+                const uint32_t off = (d0 < a.d_qk) ? row_off + d0 * ES : kOutOfRange;
                 qf[js] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, static_cast<int>(off), 0, 0);
             }
         }
@@ -802,14 +897,27 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             //     conditional: at the two ends of a sweep the SiLU half of a block may work on a score block
             //     that holds no sub-tile; what it writes is never consumed.  Visibility is applied afterwards,
             //     to the packed P^T, and only in the steps whose sub-tile is not fully visible.
-            auto read_k = [&](int js) -> u32x4_t { return *reinterpret_cast<const u32x4_t*>(kt + k_lane_off[js]); };
+            // K operand read r (16-bit inputs: MFMA step r; fp8: steps 2r and 2r+1) and V^T operand of chunk c
+            auto read_k = [&](int r) -> u32x4_t {
+                if constexpr (F8) {
+                    return *reinterpret_cast<const u32x4_t*>(reinterpret_cast<const uint8_t*>(kt) + k_lane_off[r]);
+                } else {
+                    return *reinterpret_cast<const u32x4_t*>(kt + k_lane_off[r]);
+                }
+            };
             auto read_v = [&](int c) -> u32x4_t {
                 const int j2 = c / MTILES, mt = c % MTILES;
-                const uint16_t* p = vt + v_lane_off[mt] + 16 * j2 * D;
-                const u32x2_t lo = lds_read_tr16_b64(p);
-                const u32x2_t hi = lds_read_tr16_b64(p + 8 * D);
-                const u32x4_t r = {lo[0], lo[1], hi[0], hi[1]};
-                return r;
+                if constexpr (F8) {
+                    const u32x2_t t8 = lds_read_tr8_b64(reinterpret_cast<const uint8_t*>(vt) + v_lane_off[mt] + 16 * j2 * D);
+                    const u32x4_t r = {t8[0], t8[1], 0u, 0u};
+                    return r;
+                } else {
+                    const uint16_t* p = vt + v_lane_off[mt] + 16 * j2 * D;
+                    const u32x2_t lo = lds_read_tr16_b64(p);
+                    const u32x2_t hi = lds_read_tr16_b64(p + 8 * D);
+                    const u32x4_t r = {lo[0], lo[1], hi[0], hi[1]};
+                    return r;
+                }
             };
             // unmasked P^T pair i (score elements 2i, 2i+1)
             auto silu_pair = [&](int i) {
@@ -838,7 +946,16 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                     p[0] *= lo_to_float<Tag>(mw_cur[i]);
                     p[1] *= hi_to_float<Tag>(mw_cur[i]);
                 }
-                pk_cur[i] = pack2<Tag>(p[0], p[1]);
+                if constexpr (F8) {
+                    // bring P^T to its real scale before it is quantised; pair i = bytes 2 (i % 2), +1 of word i / 2
+                    if (i & 1) {
+                        pk_cur[i / 2] = pack2_f8<true>(p[0] * c_x, p[1] * c_x, pk_cur[i / 2]);
+                    } else {
+                        pk_cur[i / 2] = pack2_f8<false>(p[0] * c_x, p[1] * c_x, pk_cur[i / 2]);
+                    }
+                } else {
+                    pk_cur[i] = pack2<Tag>(p[0], p[1]);
+                }
             };
             // the pairs of one half (first = 0 or 4) that chunk c of a block takes care of
             auto silu_chunk = [&](int first, int c) {
@@ -859,8 +976,14 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
 #pragma unroll
                 for (int c = 0; c < NCH; ++c) {
                     const int j2 = c / MTILES, mt = c % MTILES;
-                    const u32x4_t pb = {pk_prev[4 * j2 + 0], pk_prev[4 * j2 + 1], pk_prev[4 * j2 + 2], pk_prev[4 * j2 + 3]};
-                    o_acc[mt] = mfma32<Tag>(vop[c], pb, o_acc[mt]);
+                    if constexpr (F8) {
+                        const u32x2_t va = {vop[c][0], vop[c][1]};
+                        const u32x2_t pb = {pk_prev[2 * j2 + 0], pk_prev[2 * j2 + 1]};
+                        o_acc[mt] = mfma32_f8(va, pb, o_acc[mt]);
+                    } else {
+                        const u32x4_t pb = {pk_prev[4 * j2 + 0], pk_prev[4 * j2 + 1], pk_prev[4 * j2 + 2], pk_prev[4 * j2 + 3]};
+                        o_acc[mt] = mfma32<Tag>(vop[c], pb, o_acc[mt]);
+                    }
                     if (c + LOOKAHEAD < NCH) {
                         vop[c + LOOKAHEAD] = read_v(c + LOOKAHEAD);
                     }
@@ -873,7 +996,39 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                     silu_pair(i);
                 }
             }
-            if (do_qk) {
+            if constexpr (F8) {
+                if (do_qk) {
+                    u32x4_t kop[KREADS];
+                    kop[0] = read_k(0);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int c = 0; c < NCH; ++c) {
+                        const int r = c / 2;
+                        const u32x2_t ka = (c & 1) ? u32x2_t{kop[r][2], kop[r][3]} : u32x2_t{kop[r][0], kop[r][1]};
+                        const u32x2_t qb = (c & 1) ? u32x2_t{qf[r][2], qf[r][3]} : u32x2_t{qf[r][0], qf[r][1]};
+                        if (c == 0) {
+                            f32x16_t zero;
+#pragma unroll
+                            for (int i = 0; i < 16; ++i) {
+                                zero[i] = 0.f;
+                            }
+                            s_nxt = mfma32_f8(ka, qb, zero);
+                        } else {
+                            s_nxt = mfma32_f8(ka, qb, s_nxt);
+                        }
+                        if (!(c & 1) && r + 1 < KREADS) {
+                            kop[r + 1] = read_k(r + 1);
+                        }
+                        silu_chunk(4, c);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                } else if (do_silu) {
+#pragma unroll
+                    for (int i = 4; i < 8; ++i) {
+                        silu_pair(i);
+                    }
+                }
+            } else if (do_qk) {
                 u32x4_t kop[NCH];
 #pragma unroll
                 for (int c = 0; c < LOOKAHEAD; ++c) {
@@ -913,17 +1068,19 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             }
             // visibility: key c0 + 8*(e/4) + 4*lh + e%4 of element e is hidden at or past lim and inside the hole
             if (do_silu && !full) {
+                constexpr int EPW = F8 ? 4 : 2;  // packed elements per word
 #pragma unroll
-                for (int i = 0; i < 8; ++i) {
+                for (int w = 0; w < 16 / EPW; ++w) {
                     uint32_t keep = 0;
 #pragma unroll
-                    for (int e = 0; e < 2; ++e) {
-                        const int el = 2 * i + e;
+                    for (int e = 0; e < EPW; ++e) {
+                        const int el = EPW * w + e;
                         const int kk = c0 + 8 * (el / 4) + (el % 4);  // + 4*lh is folded into the *_lane bounds
                         const bool vis = (kk < lim_lane) && !(kk >= hole_lo_lane && kk < hole_hi_lane);
-                        keep |= vis ? (e ? 0xffff0000u : 0x0000ffffu) : 0u;
+                        const uint32_t bits = (F8 ? 0xffu : 0xffffu) << ((32 / EPW) * e);
+                        keep |= vis ? bits : 0u;
                     }
-                    pk_cur[i] &= keep;
+                    pk_cur[w] &= keep;
                 }
             }
 
@@ -974,8 +1131,8 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                     const int d0 = 32 * mt + 8 * g + 4 * lh;
                     const uint32_t off = (d0 < a.d_v) ? row_off + d0 * 2u : kOutOfRange;
                     u32x2_t w;
-                    w[0] = pack2<Tag>(o_acc[mt][4 * g + 0] * c_out, o_acc[mt][4 * g + 1] * c_out);
-                    w[1] = pack2<Tag>(o_acc[mt][4 * g + 2] * c_out, o_acc[mt][4 * g + 3] * c_out);
+                    w[0] = pack2<OutTag>(o_acc[mt][4 * g + 0] * c_out, o_acc[mt][4 * g + 1] * c_out);
+                    w[1] = pack2<OutTag>(o_acc[mt][4 * g + 2] * c_out, o_acc[mt][4 * g + 3] * c_out);
                     __builtin_amdgcn_raw_buffer_store_b64(w, o_rsrc, static_cast<int>(off), 0, 0);
                 }
             }

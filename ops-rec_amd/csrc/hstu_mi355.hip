@@ -66,7 +66,7 @@ std::atomic<unsigned> g_next_counter_slot{0};
 
 #define HSTU_VARIANT(tag, tagname, D, RAB, MASK, WGS)                                               \
     {"hstu_fwd_" tagname "_d" #D "_rab" #RAB "_mask" #MASK,                                        \
-     hstu::hstu_fwd_kernel<hstu::tag, D, RAB, MASK>, D, 256, WGS}
+     hstu::hstu_fwd_kernel<hstu::tag, hstu::tag, D, RAB, MASK>, D, 256, WGS}
 #define HSTU_DIMS(tag, tagname, RAB, MASK)                                                           \
     {HSTU_VARIANT(tag, tagname, 32, RAB, MASK, 2), HSTU_VARIANT(tag, tagname, 64, RAB, MASK, 2), \
      HSTU_VARIANT(tag, tagname, 128, RAB, MASK, 2), HSTU_VARIANT(tag, tagname, 256, RAB, MASK, 1)}
@@ -85,6 +85,15 @@ const Variant kVariants[2][2][2][4] = {
     {HSTU_F32_VARIANT(32, RAB, MASK), HSTU_F32_VARIANT(64, RAB, MASK), HSTU_F32_VARIANT(128, RAB, MASK), \
      HSTU_F32_VARIANT(256, RAB, MASK)}
 // fp32 inputs: [rab][custom mask][dim slot]
+// fp8-e4m3 inputs: [output: fp16, bf16][dim slot: 64, 128, 256] (no rab, no custom mask)
+#define HSTU_F8_VARIANT(otag, oname, D, WGS)                                                         \
+    {"hstu_fwd_f8e4m3_" oname "_d" #D, hstu::hstu_fwd_kernel<hstu::f8_tag, hstu::otag, D, false, false>, D, 256, WGS}
+const Variant kVariantsF8[2][3] = {
+    {HSTU_F8_VARIANT(f16_tag, "f16", 64, 2), HSTU_F8_VARIANT(f16_tag, "f16", 128, 2), HSTU_F8_VARIANT(f16_tag, "f16", 256, 1)},
+    {HSTU_F8_VARIANT(bf16_tag, "bf16", 64, 2), HSTU_F8_VARIANT(bf16_tag, "bf16", 128, 2),
+     HSTU_F8_VARIANT(bf16_tag, "bf16", 256, 1)},
+};
+
 const Variant kVariantsF32[2][2][4] = {{HSTU_F32_DIMS(false, false), HSTU_F32_DIMS(false, true)},
                                        {HSTU_F32_DIMS(true, false), HSTU_F32_DIMS(true, true)}};
 
@@ -165,12 +174,20 @@ int validate(const hstu_jagged_fwd_params* p)
 // picks the kernel variant; returns nullptr (and sets the error) when the combination is not built
 const Variant* select(const hstu_jagged_fwd_params* p)
 {
-    if (p->dtype != HSTU_DT_BF16 && p->dtype != HSTU_DT_FP16 && p->dtype != HSTU_DT_FP32) {
-        fail(HSTU_ERR_UNSUPPORTED, "dtype %d is not built in this library version (bf16, fp16 and fp32 are)",
-             p->dtype);
-        return nullptr;
-    }
-    if (p->out_dtype != p->dtype) {
+    if (p->dtype == HSTU_DT_FP8_E4M3) {
+        if (p->out_dtype != HSTU_DT_FP16 && p->out_dtype != HSTU_DT_BF16) {
+            fail(HSTU_ERR_UNSUPPORTED, "fp8 inputs produce fp16 (the reference's choice) or bf16 output");
+            return nullptr;
+        }
+        if (p->attn_bias != nullptr || p->mask_type == HSTU_MASK_CUSTOM) {
+            fail(HSTU_ERR_UNSUPPORTED, "attn_bias and custom masks are not built for fp8 inputs");
+            return nullptr;
+        }
+        if (p->head_dim_qk % 16 != 0) {
+            fail(HSTU_ERR_UNSUPPORTED, "fp8 q/k head dim %lld is not a multiple of 16", (long long)p->head_dim_qk);
+            return nullptr;
+        }
+    } else if (p->out_dtype != p->dtype) {
         fail(HSTU_ERR_UNSUPPORTED, "out_dtype must equal dtype for bf16 / fp16 / fp32 inputs");
         return nullptr;
     }
@@ -205,6 +222,9 @@ const Variant* select(const hstu_jagged_fwd_params* p)
             fail(HSTU_ERR_UNSUPPORTED, "max_seq_len x heads x head dim spans 1 GiB or more per sequence");
             return nullptr;
         }
+    }
+    if (p->dtype == HSTU_DT_FP8_E4M3) {
+        return &kVariantsF8[p->out_dtype == HSTU_DT_FP16 ? 0 : 1][slot <= 1 ? 0 : slot - 1];
     }
     if (p->dtype == HSTU_DT_FP32) {
         return &kVariantsF32[p->attn_bias != nullptr ? 1 : 0][p->mask_type == HSTU_MASK_CUSTOM ? 1 : 0][slot];
@@ -298,6 +318,11 @@ HSTU_API int hstu_jagged_fwd(const hstu_jagged_fwd_params* p, void* workspace, u
     const double scale = (p->silu_scale == 0.0) ? 1.0 / static_cast<double>(p->max_seq_len_q) : p->silu_scale;
     a.c_exp = static_cast<float>(-p->alpha * 1.4426950408889634);
     a.c_out = static_cast<float>(p->alpha * scale);
+    a.alpha = static_cast<float>(p->alpha);
+    a.silu_scale = static_cast<float>(scale);
+    a.q_descale = p->q_descale;
+    a.k_descale = p->k_descale;
+    a.v_descale = p->v_descale;
 
 #ifdef HSTU_TIMELINE
     a.timeline = static_cast<unsigned long long*>(workspace);  // development builds only

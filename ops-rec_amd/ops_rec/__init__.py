@@ -16,8 +16,9 @@ import logging
 from . import _ops  # noqa: F401  (defines the operators)
 from . import ascendc  # noqa: F401
 from . import autograd  # noqa: F401  (registers the autograd formulas)
+from ._ops import hstu_jagged_fp8  # noqa: F401  (extension: fp8 inputs with per-head scales)
 
 logger = logging.getLogger(__name__)
 
 __version__ = "0.1.0"
-__all__ = ["ascendc", "autograd", "__version__"]
+__all__ = ["ascendc", "autograd", "hstu_jagged_fp8", "__version__"]

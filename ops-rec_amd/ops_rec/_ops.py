@@ -132,9 +132,17 @@ def prepare_forward(
     target_group_size: Optional[int],
     alpha: Optional[float],
     deterministic: bool = False,
+    *,
+    out_dtype: Optional[torch.dtype] = None,
+    q_descale: Optional[torch.Tensor] = None,
+    k_descale: Optional[torch.Tensor] = None,
+    v_descale: Optional[torch.Tensor] = None,
 ) -> PreparedForward:
     """Argument normalisation and checks of the reference adapter
-    (torch_extension/hstu_jagged_plugin.cpp:22-67), ending in a filled parameter block."""
+    (torch_extension/hstu_jagged_plugin.cpp:22-67), ending in a filled parameter block.
+
+    The keyword-only arguments belong to the fp8 extension (``hstu_jagged_fp8``): output type
+    (fp16 as in the reference, or bf16) and per-head fp32 dequantisation scales."""
     _check(q.dim() == 3, "The q should be 3D in jagged layout")
     _check(seq_offset is not None and seq_offset_k is not None, "seq_offset is required")
     _check(seq_offset.dim() == 1 and seq_offset.size(0) >= 2,
@@ -179,11 +187,24 @@ def prepare_forward(
         _check(tuple(mask.shape) == bias_shape, f"mask must have shape {bias_shape}")
         mask_c = mask.contiguous()
 
-    out_dtype = _out_dtype(q_c)
+    is_fp8 = q_c.dtype == torch.float8_e4m3fn
+    _check(is_fp8 or (out_dtype is None and q_descale is None and k_descale is None and v_descale is None),
+           "out_dtype and descales are only taken with fp8 inputs")  # fmt: skip
+    if out_dtype is None:
+        out_dtype = _out_dtype(q_c)
+    _check(not is_fp8 or out_dtype in (torch.float16, torch.bfloat16), "fp8 inputs produce fp16 or bf16 output")
+    scales = []
+    for name, t, heads in (("q_descale", q_descale, q_c.size(1)), ("k_descale", k_descale, k_c.size(1)),
+                           ("v_descale", v_descale, k_c.size(1))):  # fmt: skip
+        if t is not None:
+            _check(t.dtype == torch.float32 and t.dim() == 1 and t.size(0) == heads and t.device == q_c.device,
+                   f"{name} must be a float32 tensor of {heads} per-head scales on the device of q")  # fmt: skip
+            t = t.contiguous()
+        scales.append(t)
     # every row is written by the kernel (rows past the last offset are zero-filled there),
     # so the zero-fill of the reference adapter (:56-59) is not repeated here
     out = torch.empty((q_c.size(0), q_c.size(1), v_c.size(2)), dtype=out_dtype, device=q_c.device)
-    keep = (q_c, k_c, v_c, mask_c, bias, offs_q, offs_k, ctx, tgt)
+    keep = (q_c, k_c, v_c, mask_c, bias, offs_q, offs_k, ctx, tgt, *scales)
     p = _native.new_params()
     if out.numel() == 0:
         return PreparedForward(p, out, None, 0, q_c.device, keep)
@@ -209,6 +230,7 @@ def prepare_forward(
     p.silu_scale = real_scale
     p.alpha = real_alpha
     p.deterministic = 1 if deterministic else 0
+    p.q_descale, p.k_descale, p.v_descale = (_ptr(t) for t in scales)
 
     ws_bytes = ctypes.c_uint64(0)
     rc = lib.hstu_jagged_fwd_workspace_size(ctypes.byref(p), ctypes.byref(ws_bytes))
@@ -225,6 +247,25 @@ def _forward_impl(q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max_seq_le
     prepared = prepare_forward(q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max_seq_len_k, silu_scale,
                                seq_offset, seq_offset_k, num_context, num_target, target_group_size, alpha,
                                deterministic)  # fmt: skip
+    with torch.cuda.device(prepared.device):
+        return prepared.launch()
+
+
+def hstu_jagged_fp8(q, k, v, q_descale=None, k_descale=None, v_descale=None, *, mask_type=0, max_seq_len=0,
+                    max_seq_len_k=None, silu_scale=0.0, seq_offset=None, seq_offset_k=None, num_context=None,
+                    num_target=None, target_group_size=0, alpha=1.0, out_dtype=torch.bfloat16):  # fmt: skip
+    """Forward on fp8-e4m3 (``torch.float8_e4m3fn``) Q / K / V with per-head fp32 dequantisation scales.
+
+    An extension: the reference's fp8 path (``hstu_jagged`` called with e4m3 tensors, which this
+    package serves too) has no scales and a half output.  Here ``x = x8 * descale[head]`` for each of
+    q, k, v (``None`` = 1), P is re-quantised to e4m3 before ``silu_scale`` is applied, and the
+    output is ``out_dtype`` (bf16 or fp16).  No attn_bias, no custom mask."""
+    _check(q.dtype == torch.float8_e4m3fn, "hstu_jagged_fp8 takes float8_e4m3fn tensors")
+    offs_k = seq_offset if seq_offset_k is None else seq_offset_k
+    max_k = max_seq_len if max_seq_len_k is None else max_seq_len_k
+    prepared = prepare_forward(q, k, v, None, None, mask_type, max_seq_len, max_k, silu_scale, seq_offset, offs_k,
+                               num_context, num_target, target_group_size, alpha, False, out_dtype=out_dtype,
+                               q_descale=q_descale, k_descale=k_descale, v_descale=v_descale)  # fmt: skip
     with torch.cuda.device(prepared.device):
         return prepared.launch()
 

@@ -1,8 +1,9 @@
 """Synthetic jagged batches for the named HSTU attention configurations.
 
 Used by the benchmark and by the parity tests so that both run the same seeded inputs.
-Everything is generated on the CPU with a seeded ``torch.Generator`` (so the CPU oracle and the
-GPU operator see identical bits) and moved to a device by the caller.
+Lengths always come from a seeded CPU generator; the tensors are drawn with a seeded
+``torch.Generator`` on the device asked for (the CPU by default, so that the CPU oracle and the
+GPU operator see identical bits; the large configurations are drawn on the GPU directly).
 
 Configurations (lengths are per sequence, drawn uniformly unless stated):
 
@@ -132,6 +133,18 @@ def make(
         silu_scale=silu_scale, alpha=(dim**-0.5 if alpha is None else alpha), attn_bias=bias,
         num_context=ctx, num_target=tgt, target_group_size=target_group_size, lengths=list(lengths),
     )  # fmt: skip
+
+
+E4M3_MAX = 448.0
+
+
+def quantize_fp8(x: torch.Tensor):
+    """``x[T, H, d]`` -> (``float8_e4m3fn`` tensor, ``descale[H]`` float32) with one scale per head,
+    ``descale = absmax / 448``: the quantisation configuration C5 is defined with."""
+    absmax = x.abs().amax(dim=(0, 2)).clamp_min(1e-12).float()
+    descale = absmax / E4M3_MAX
+    x8 = (x.float() / descale[None, :, None]).clamp(-E4M3_MAX, E4M3_MAX).to(torch.float8_e4m3fn)
+    return x8, descale
 
 
 def zipf_lengths(batch: int, s: float = 1.2, lo: int = 32, hi: int = 8192, seed: int = 0) -> list:

@@ -201,6 +201,7 @@ def hstu_jagged_forward(
     compute_dtype: torch.dtype = torch.float32,
     emulate_lowp: Optional[torch.dtype] = None,
     out_dtype: Optional[torch.dtype] = None,
+    _p_hook=None,
 ) -> torch.Tensor:
     """Per-sequence restatement of the jagged forward (CPU).
 
@@ -265,7 +266,79 @@ def hstu_jagged_forward(
         elif mask_type != MASK_NONE:
             raise ValueError(f"unsupported mask_type {mask_type}")
         p = _round_to(p, emulate_lowp)
+        if _p_hook is not None:  # the fp8 definition re-quantises P here
+            p = _p_hook(p).to(cd)
         out[q0:q1] = torch.einsum("hnm,mhd->nhd", p, vb)
+    return out.to(out_dtype)
+
+
+# --------------------------------------------------------------------------- #
+# forward with fp8-e4m3 inputs and per-head scales
+# --------------------------------------------------------------------------- #
+
+E4M3_MAX = 448.0
+
+
+def quantize_e4m3(x: torch.Tensor) -> torch.Tensor:
+    """Round to nearest even onto OCP e4m3fn after clamping to +-448 (the format has no infinity)."""
+    return x.clamp(-E4M3_MAX, E4M3_MAX).to(torch.float8_e4m3fn)
+
+
+def quantize_per_head(x: torch.Tensor):
+    """``x[T, H, d]`` -> (e4m3 tensor, ``descale[H]``) with ``descale = absmax / 448`` per head, the
+    quantisation the fp8 workload is defined with."""
+    absmax = x.abs().amax(dim=(0, 2)).clamp_min(1e-12).float()
+    descale = absmax / E4M3_MAX
+    return quantize_e4m3(x.float() / descale[None, :, None]), descale
+
+
+def hstu_jagged_forward_fp8(
+    q8: torch.Tensor,
+    k8: torch.Tensor,
+    v8: torch.Tensor,
+    q_descale: Optional[torch.Tensor],
+    k_descale: Optional[torch.Tensor],
+    v_descale: Optional[torch.Tensor],
+    *,
+    quantize_p: bool = True,
+    out_dtype: torch.dtype = torch.float16,
+    **kwargs,
+) -> torch.Tensor:
+    """fp8 forward as this build defines it, on CPU in fp32.
+
+    The reference's fp8 path takes raw e4m3 Q / K / V, keeps S in fp32, re-quantises P to e4m3
+    (round to nearest) and accumulates P.V in fp32 into a half output
+    (.../hstu_dense_forward_kernel_patten_bsnd.h:76, 279, 453-459, 643-646;
+    torch_extension/hstu_jagged_plugin.cpp:53-54).  Two things are added here: per-head
+    dequantisation scales (``x = x8 * descale[head]``; ``None`` = 1) and the place of the
+    re-quantisation, which is BEFORE ``silu_scale`` is applied: the reference quantises
+    ``silu(X) * silu_scale``, which with the default ``silu_scale = 1 / max_seq_len`` lies below
+    e4m3's smallest normal number.  With ``silu_scale = 1`` and no scales the two definitions
+    coincide.  ``quantize_p=False`` gives the unrounded result on the de-quantised inputs.
+
+    Not pinned by any reference artefact (the reference's fp8 tests are disabled,
+    .../test_hstu_jagged.py:687-689): parity unpinned beyond the fp32 formula it shares with
+    ``hstu_jagged_forward``, which the checks of that function cover.
+    """
+    n_q, n_k = q8.shape[1], k8.shape[1]
+    one_q, one_k = torch.ones(n_q), torch.ones(n_k)
+    qs = one_q if q_descale is None else q_descale.float().cpu()
+    ks = one_k if k_descale is None else k_descale.float().cpu()
+    vs = one_k if v_descale is None else v_descale.float().cpu()
+    qf = q8.float() * qs[None, :, None]
+    kf = k8.float() * ks[None, :, None]
+    scale = resolve_silu_scale(kwargs.get("silu_scale", 0.0), kwargs["max_seq_len"])
+    kw = dict(kwargs)
+    kw["silu_scale"] = 1.0  # P is formed (and rounded) unscaled
+    if kw.get("attn_bias") is not None or kw.get("mask_type", 0) == MASK_CUSTOM:
+        raise ValueError("the fp8 path takes no attn_bias / custom mask")
+    # V enters unscaled so that P (e4m3) x V (e4m3) is what is accumulated; its scale goes on the output
+    out = hstu_jagged_forward(
+        qf, kf, v8.float(), compute_dtype=torch.float32,
+        emulate_lowp=None, out_dtype=torch.float32, _p_hook=(quantize_e4m3 if quantize_p else None), **kw,
+    )  # fmt: skip
+    ratio = n_q // n_k
+    out = out * (scale * vs.repeat_interleave(ratio))[None, :, None]
     return out.to(out_dtype)
 
 

@@ -259,3 +259,29 @@ def test_kernel_variant_selection():
     assert "rabtrue" in name(attn_bias=0x2000)
     assert "masktrue" in name(mask=0x2000, mask_type=3)
     assert "f16" in name(dtype=_native.DT_FP16, out_dtype=_native.DT_FP16)
+
+
+def test_fp8_variant_selection_and_limits():
+    lib = _native.load()
+
+    def name(**kw):
+        p = _valid_params()
+        p.dtype = _native.DT_FP8_E4M3
+        p.out_dtype = _native.DT_FP16
+        for k, v in kw.items():
+            setattr(p, k, v)
+        n = lib.hstu_jagged_fwd_kernel_name(ctypes.byref(p))
+        return n.decode() if n else None
+
+    assert name() == "hstu_fwd_f8e4m3_f16_d128"
+    assert name(out_dtype=_native.DT_BF16) == "hstu_fwd_f8e4m3_bf16_d128"
+    assert name(head_dim_qk=32, head_dim_v=48).endswith("_d64")  # fp8 rows are padded to at least 64 bytes
+    assert name(head_dim_qk=256, head_dim_v=256).endswith("_d256")
+    for kw, text in [
+        (dict(out_dtype=_native.DT_FP32), "fp16 .* or bf16"),
+        (dict(attn_bias=0x2000), "not built for fp8"),
+        (dict(mask=0x2000, mask_type=3), "not built for fp8"),
+        (dict(head_dim_qk=24, head_dim_v=16), "multiple of 16"),
+    ]:
+        assert name(**kw) is None
+        assert re.search(text, _native.last_error()), (kw, _native.last_error())

@@ -202,3 +202,70 @@ def test_flop_model():
     offs = [0, 10, 10, 35]
     assert O.causal_effective_flops(offs, None, 4, 128, 128) == 2 * 256 * 4 * (55 + 325)
     assert O.causal_effective_flops(offs, None, 2, 64, 32, mask_type=2) == 2 * 96 * 2 * (100 + 625)
+
+
+# --------------------------------------------------------------------------- #
+# fp8 definition (inputs e4m3 with per-head scales, P re-quantised before silu_scale)
+# --------------------------------------------------------------------------- #
+
+
+def test_e4m3_quantiser_known_values():
+    x = torch.tensor([0.0, 1.0, -1.0, 0.3, 17.0, 18.0, 19.0, 447.0, 449.0, 1000.0, -1000.0, 0.0625, 0.001])
+    got = O.quantize_e4m3(x).float()
+    # 3 mantissa bits: spacing 2 between 16 and 32 (ties to even), 0.03125 between 0.25 and 0.5; no infinity: clamp to 448
+    want = torch.tensor([0.0, 1.0, -1.0, 0.3125, 16.0, 18.0, 20.0, 448.0, 448.0, 448.0, -448.0, 0.0625, 0.001953125])
+    assert torch.equal(got, want)
+
+
+def _fp8_case(seed=0, heads=4, heads_k=2, d=32, dv=16):
+    g = torch.Generator().manual_seed(seed)
+    lengths = [7, 33, 1, 20]
+    total = sum(lengths)
+    offs = torch.tensor([0] + list(torch.tensor(lengths).cumsum(0)), dtype=torch.int32)
+    q8, qs = O.quantize_per_head(torch.randn(total, heads, d, generator=g))
+    k8, ks = O.quantize_per_head(torch.randn(total, heads_k, d, generator=g))
+    v8, vs = O.quantize_per_head(torch.randn(total, heads_k, dv, generator=g))
+    kw = dict(mask_type=0, max_seq_len=40, silu_scale=0.0, seq_offset=offs, alpha=d**-0.5)
+    return (q8, k8, v8), (qs, ks, vs), kw
+
+
+def test_fp8_unrounded_equals_generic_forward_on_dequantised_inputs():
+    (q8, k8, v8), (qs, ks, vs), kw = _fp8_case()
+    got = O.hstu_jagged_forward_fp8(q8, k8, v8, qs, ks, vs, quantize_p=False, out_dtype=torch.float32, **kw)
+    deq = lambda x8, s: x8.float() * s[None, :, None]  # noqa: E731
+    want = O.hstu_jagged_forward(deq(q8, qs), deq(k8, ks), deq(v8, vs), out_dtype=torch.float32, **kw)
+    torch.testing.assert_close(got, want, atol=1e-6, rtol=1e-5)
+
+
+def test_fp8_scale_algebra():
+    (q8, k8, v8), (qs, ks, vs), kw = _fp8_case(seed=3)
+    base = O.hstu_jagged_forward_fp8(q8, k8, v8, qs, ks, vs, out_dtype=torch.float32, **kw)
+    # the V scale is applied to the fp32 output: a power of two passes through exactly
+    twice = O.hstu_jagged_forward_fp8(q8, k8, v8, qs, ks, vs * 2, out_dtype=torch.float32, **kw)
+    assert torch.equal(twice, base * 2)
+    # a uniform q scale is the same as a factor on alpha (powers of two: exact)
+    kw2 = dict(kw, alpha=kw["alpha"] * 4.0)
+    moved = O.hstu_jagged_forward_fp8(q8, k8, v8, qs / 4, ks, vs, out_dtype=torch.float32, **kw2)
+    assert torch.equal(moved, base)
+    # P is rounded before silu_scale: changing silu_scale by a power of two only scales the result
+    kw3 = dict(kw, silu_scale=1.0 / 8)
+    kw4 = dict(kw, silu_scale=1.0 / 64)
+    a = O.hstu_jagged_forward_fp8(q8, k8, v8, qs, ks, vs, out_dtype=torch.float32, **kw3)
+    b = O.hstu_jagged_forward_fp8(q8, k8, v8, qs, ks, vs, out_dtype=torch.float32, **kw4)
+    assert torch.equal(a, b * 8)
+
+
+def test_fp8_reduces_to_the_reference_definition_without_scales_and_silu_scale_one():
+    # reference: P = rint_e4m3(silu(X) * silu_scale * M), S and the accumulation in fp32, half output
+    (q8, k8, v8), _, kw = _fp8_case(seed=5)
+    kw = dict(kw, silu_scale=1.0)
+    got = O.hstu_jagged_forward_fp8(q8, k8, v8, None, None, None, out_dtype=torch.float16, **kw)
+    want = O.hstu_jagged_forward(q8.float(), k8.float(), v8.float(), out_dtype=torch.float16,
+                                 _p_hook=O.quantize_e4m3, **kw)  # fmt: skip
+    assert torch.equal(got, want)
+
+
+def test_fp8_rejects_bias_and_custom_mask():
+    (q8, k8, v8), (qs, ks, vs), kw = _fp8_case()
+    with pytest.raises(ValueError):
+        O.hstu_jagged_forward_fp8(q8, k8, v8, qs, ks, vs, **dict(kw, mask_type=3, mask=torch.ones(4, 4, 40, 40)))
