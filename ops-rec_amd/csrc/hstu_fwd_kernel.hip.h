@@ -283,11 +283,18 @@ __device__ __forceinline__ float hi_to_float<f16_tag>(uint32_t packed)
 // ---- LDS layout ---------------------------------------------------------------------------
 // K tile: [rows][D] elements, 16-byte chunks XOR-swizzled by row so that the 32x32x16 A-operand
 // read (32 lanes = 32 consecutive rows, same logical chunk) spreads over the banks.
-template <int CPR>  // CPR = 16-byte chunks per row
+// fp8 tiles (rows of CPR 16-byte chunks), one layout for K and V.  Two read patterns must both be free of
+// bank conflicts: the K operand read (16 consecutive rows, one chunk) and the 8-bit transposed V read
+// (rows {0,1,2,3,8,9,10,11} + 4 * half, two neighbouring chunks).  The XOR term is therefore a bijection
+// of the row bits above the rows-per-256-bytes bits in which row bit 2 (the k-half of the transposed read,
+// constant within one of its groups) is moved to the lowest place, so that the other bits separate chunk pairs.
+template <int CPR>
 __device__ __forceinline__ int chunk_swizzle(int row, int chunk)
 {
     if constexpr (CPR >= 16) {
-        return chunk ^ (row & 15);
+        return chunk ^ ((((row >> 3) & 1) << 3) | (((row >> 1) & 1) << 2) | ((row & 1) << 1) | ((row >> 2) & 1));
+    } else if constexpr (CPR == 8) {
+        return chunk ^ ((((row >> 3) & 1) << 2) | (((row >> 1) & 1) << 1) | ((row >> 2) & 1));
     } else {
         constexpr int RPG = 16 / CPR;  // rows per 256 bytes
         return chunk ^ ((row / RPG) & (CPR - 1));
