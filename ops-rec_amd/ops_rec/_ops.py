@@ -42,6 +42,9 @@ _SCHEMAS = (
     "Tensor? attn_bias=None, int mask_type=0, int max_seq_len=0, int max_seq_len_k=0, float silu_scale=0.0, "
     "Tensor seq_offset=None, Tensor seq_offset_k=None, Tensor? num_context=None, Tensor? num_target=None, "
     "int? target_group_size=0, float? alpha=1.0) -> (Tensor, Tensor, Tensor, Tensor)",
+    # dense [B, S, N, D] layout (torch_extension/hstu_dense_plugin.cpp:156-163): forward only here
+    "hstu_dense(Tensor q, Tensor k, Tensor v, Tensor? mask=None, Tensor? attn_bias=None, int mask_type=0, "
+    "int max_seq_len=0, float silu_scale=0.0) -> Tensor",
 )
 
 _lib_def = torch.library.Library("ops_rec", "DEF")
@@ -420,6 +423,36 @@ def hstu_jagged_backward_delta_meta(grad, q, k, v, mask=None, attn_bias=None, ma
     return _backward_meta(grad, q, k, v, attn_bias)
 
 
+def hstu_dense(q, k, v, mask=None, attn_bias=None, mask_type=0, max_seq_len=0, silu_scale=0.0):
+    """Dense ``[B, S, N, D]`` forward (torch_extension/hstu_dense_plugin.cpp:19-40): every sequence has the full
+    length S, no alpha (1.0), no context / target arguments.  Served by the jagged kernel on a view
+    ``[B * S, N, D]`` with offsets ``0, S, 2S, ...``; output ``empty_like(q)`` as in the reference."""
+    _check(q.dim() == 4, "The q should be 4D in dense layout")
+    _check(k.dim() == 4 and v.dim() == 4, "The k and v should be 4D in dense layout")
+    _max_seq_len_check(int(max_seq_len), "maxSeqLen")
+    _mask_check(int(mask_type), mask is not None)
+    batch, s_q, s_k = q.size(0), q.size(1), k.size(1)
+    _check(k.size(0) == batch and v.size(0) == batch and v.size(1) == s_k, "Q, K, V batch / sequence shapes mismatch")
+    real_scale = (1.0 / float(max_seq_len)) if float(silu_scale) == 0.0 else float(silu_scale)
+    qc, kc, vc = q.contiguous(), k.contiguous(), v.contiguous()
+    dev = qc.device
+    offs_q = torch.arange(0, (batch + 1) * s_q, max(s_q, 1), dtype=torch.int32, device=dev)[: batch + 1]
+    offs_k = offs_q if s_k == s_q else torch.arange(0, (batch + 1) * s_k, max(s_k, 1), dtype=torch.int32, device=dev)[: batch + 1]
+    if batch == 0 or s_q == 0:
+        return torch.empty((batch, s_q, q.size(2), v.size(3)), dtype=_out_dtype(qc), device=dev)
+    out = _forward_impl(qc.view(batch * s_q, q.size(2), q.size(3)), kc.view(batch * s_k, k.size(2), k.size(3)),
+                        vc.view(batch * s_k, v.size(2), v.size(3)), mask, attn_bias, mask_type, max(s_q, 1), max(s_k, 1),
+                        real_scale, offs_q, offs_k, None, None, 0, 1.0)  # fmt: skip
+    return out.view(batch, s_q, q.size(2), v.size(3))
+
+
+def hstu_dense_meta(q, k, v, mask=None, attn_bias=None, mask_type=0, max_seq_len=0, silu_scale=0.0):
+    _check(q.dim() == 4, "The q should be 4D in dense layout")
+    return torch.empty((q.size(0), q.size(1), q.size(2), v.size(3)), dtype=_out_dtype(q), device=q.device)
+
+
+_lib_cuda.impl("hstu_dense", hstu_dense)
+_lib_meta.impl("hstu_dense", hstu_dense_meta)
 _lib_cuda.impl("hstu_jagged.equal", hstu_jagged_equal)
 _lib_cuda.impl("hstu_jagged.delta", hstu_jagged_delta)
 _lib_cuda.impl("hstu_jagged_backward.equal", hstu_jagged_backward_equal)

@@ -246,3 +246,23 @@ def test_kernel_errors_surface_as_runtime_error():
     q = torch.zeros(8, 2, 32, dtype=torch.float64, device=DEV)
     with pytest.raises(RuntimeError, match="unsupported dtype"):
         ops_rec.ascendc.attention.hstu_jagged(q, q, q, None, None, 0, 8, 0.0, offs)
+
+
+@pytest.mark.parametrize("mask_type", [0, 2, 3])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("batch,seq,heads,dim,enable_bias", [(3, 40, 2, 64, False), (2, 130, 4, 128, True), (1, 300, 1, 32, True)])
+def test_dense_layout_entry_point(batch, seq, heads, dim, enable_bias, dtype, mask_type):
+    # hstu_dense: [B, S, N, D] tensors, alpha 1, every sequence of full length
+    # (torch_extension/hstu_dense_plugin.cpp:19-40; formula hstu_forward_v1/README.md:61-75)
+    g = torch.Generator().manual_seed(seq)
+    q, k, v = ((torch.randn(batch, seq, heads, dim, generator=g) * 0.3).to(dtype) for _ in range(3))
+    bias = (torch.randn(batch, heads, seq, seq, generator=g) * 0.1).to(dtype) if enable_bias else None
+    mask = (torch.rand(batch, heads, seq, seq, generator=g) > 0.3).to(dtype) if mask_type == 3 else None
+    d = lambda t: None if t is None else t.to(DEV)  # noqa: E731
+    out = ops_rec.ascendc.attention.hstu_dense(d(q), d(k), d(v), d(mask), d(bias), mask_type, seq, 0.0)
+    assert tuple(out.shape) == (batch, seq, heads, dim) and out.dtype == dtype
+    offs = torch.arange(0, (batch + 1) * seq, seq, dtype=torch.int32)
+    ref = O.hstu_jagged_forward(q.reshape(-1, heads, dim), k.reshape(-1, heads, dim), v.reshape(-1, heads, dim),
+                                mask=mask, attn_bias=bias, mask_type=mask_type, max_seq_len=seq, silu_scale=0.0,
+                                seq_offset=offs, alpha=1.0, out_dtype=torch.float32)  # fmt: skip
+    torch.testing.assert_close(out.float().cpu().reshape(-1, heads, dim), ref, atol=1e-2, rtol=1e-2)

@@ -285,3 +285,13 @@ def test_fp8_variant_selection_and_limits():
     ]:
         assert name(**kw) is None
         assert re.search(text, _native.last_error()), (kw, _native.last_error())
+
+
+def test_dense_op_is_registered_with_meta_inference():
+    op = ops_rec.ascendc.attention.hstu_dense
+    q = torch.empty(3, 40, 2, 64, device="meta", dtype=torch.bfloat16)
+    v = torch.empty(3, 40, 2, 32, device="meta", dtype=torch.bfloat16)
+    out = op(q, q, v, None, None, 0, 40, 0.0)
+    assert out.shape == (3, 40, 2, 32) and out.dtype == torch.bfloat16
+    with pytest.raises(RuntimeError, match="4D in dense layout"):
+        op(q[0], q[0], v[0], None, None, 0, 40, 0.0)
