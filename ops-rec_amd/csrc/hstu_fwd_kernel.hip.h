@@ -351,11 +351,14 @@ __device__ __forceinline__ void load_to_lds_b128(__amdgpu_buffer_rsrc_t rsrc, ui
 }
 
 // ---- device-side work counters ---------------------------------------------------------------
-// One (work, done) pair per slot; a launch is given a slot by the host (round robin), so launches
-// that overlap on one GPU do not share a pair unless more than kCounterSlots of them are in flight.
-// Zero at module load; the last workgroup of a launch to leave puts its pair back to zero.
+// One set of (work x kQueues, done) counters per slot; a launch is given a slot by the host (round
+// robin), so launches that overlap on one GPU do not share a set unless more than kCounterSlots of
+// them are in flight.  Zero at module load; the last workgroup of a launch to leave puts its set
+// back to zero.
 constexpr int kCounterSlots = 64;
-static __device__ unsigned int g_work_counter[kCounterSlots];
+constexpr int kQueues = 8;          // one work queue per XCD (MI355X: 8 XCDs; workgroup w runs on XCD w mod 8)
+constexpr int kCounterStride = 32;  // counters of different queues sit in different 128-byte lines
+static __device__ unsigned int g_work_counter[kCounterSlots][kQueues * kCounterStride];
 static __device__ unsigned int g_done_counter[kCounterSlots];
 
 constexpr int kMaxBatchSlots = 2048;  // sequences per call (the reference's limit)
@@ -374,6 +377,9 @@ __device__ __forceinline__ int64_t load_index_uniform(const void* p, int64_t i, 
 
 struct U32Pair {
     uint32_t v[2];
+};
+struct U32Quad {
+    uint32_t v[4];
 };
 
 // ---- the kernel ---------------------------------------------------------------------------
@@ -407,7 +413,11 @@ struct U32Pair {
 // scale are applied to the fp32 output.  K is read 16 bytes per lane for two MFMA steps at a time (k index
 // (half, byte) of step 2p / 2p+1 = dim 16 (2p + half) + byte / + 8 + byte), V^T by one 8-bit transposed read
 // per MFMA.  rab and custom masks are not available for fp8 inputs.
-template <typename Tag, typename OutTag, int D, bool HAS_RAB, bool HAS_MASK>
+//
+// QUEUES: build the per-XCD queue machinery (see "Work queues" below).  It pays on long, jagged batches with many
+// items per workgroup; its code is on the path of every item, so launches that cannot profit (the host decides by
+// an upper bound on the number of items) use the variant without it.
+template <typename Tag, typename OutTag, int D, bool HAS_RAB, bool HAS_MASK, bool QUEUES = false>
 __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const FwdArgs a)
 {
     constexpr int kThreads = 256;
@@ -443,8 +453,9 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
     __shared__ uint8_t s_ntiles[kMaxBatchSlots];          // query tiles of each sequence
     __shared__ uint16_t s_order[kMaxBatchSlots];          // sequences, most query tiles first
     __shared__ uint32_t s_bucket[kMaxLevels + 2];         // histogram, then scatter cursors
-    __shared__ uint32_t s_level_start[kMaxLevels + 2];    // first item of each level (level = tiles from the top)
-    __shared__ uint32_t s_next;
+    __shared__ uint32_t s_rank_start[kMaxLevels + 2];     // [nt]: number of sequences with more than nt query tiles
+    __shared__ uint32_t s_queue_start[QUEUES ? kQueues : 1][kMaxLevels + 2];  // per queue: first item of each level / bucket
+    __shared__ uint32_t s_item[8];  // [0..3]: the item handed to the workgroup (valid, query tile, sequence, head); [4]: queue order
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -494,14 +505,68 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             s_bucket[nt] = run;
             run += c;
         }
-        // level l holds query tile qt = n_levels - 1 - l of every sequence that has more than qt tiles,
-        // for every head: s_bucket[qt] sequences (the start of bucket qt counts exactly those)
+        for (int nt = 0; nt <= n_levels; ++nt) {
+            s_rank_start[nt] = s_bucket[nt];
+        }
+    }
+    if constexpr (QUEUES) {
+        __syncthreads();  // (without queues, thread 0 alone goes on to build the one table)
+    }
+    // Work queues.  A "pair" is one (sequence, K/V head): its K / V rows are read by every query tile of every
+    // query head that shares the K/V head.  Pairs are numbered p = sorted position * n_heads_k + kv head; pair p
+    // belongs to queue p mod 8, and a queue is served first by the workgroups of one XCD, so that the rows of a
+    // pair are fetched into one L2 instead of eight.  Two orders inside a queue:
+    //   by tile  - the heaviest (highest) query tile of all its pairs first, then the next tile down, ...: longest
+    //              items first.  With a handful of items per workgroup and item lengths between 1 and
+    //              max_seq_len / 32 steps this is what keeps the end of the launch short.  Level l of the queue =
+    //              query tile n_levels - 1 - l of its pairs that have it (the sequences at sorted positions
+    //              [0, s_rank_start[qt]) have more than qt tiles).
+    //   by pair  - pair after pair (most tiles first), the tiles of a pair together, heaviest first: the
+    //              workgroups of the XCD sweep the K / V rows of few pairs at a time, and each row is fetched
+    //              from HBM about once instead of once per query tile.  Bucket l of the queue = its pairs with
+    //              nt = n_levels - l tiles (sorted positions [s_rank_start[nt], s_rank_start[nt - 1])).
+    // "By pair" starts the heavy tiles of late pairs late; that is harmless when there are many items per
+    // workgroup and the late pairs are short (a jagged batch), and costly when all sequences are equally long.
+    // It is chosen when the list has at least 4 items per workgroup and the mean tile count of the sequences is
+    // at most 0.7 of the largest.
+    // "By tile" runs as ONE queue shared by all workgroups (the order that matters there is global), "by pair" as
+    // one queue per XCD.
+    if (tid < (QUEUES ? kQueues : 1)) {
+        bool by_pair = false;
+        if constexpr (QUEUES) {
+            // total tiles = sum over nt of nt * (sequences with nt tiles); sequences with nt tiles =
+            // s_rank_start[nt-1] - s_rank_start[nt]  (every builder thread works the order out for itself)
+            uint32_t tiles = 0, seqs = 0;
+            int nt_max = 0;
+            for (int nt = 1; nt <= n_levels; ++nt) {
+                const uint32_t c = s_rank_start[nt - 1] - s_rank_start[nt];
+                tiles += c * static_cast<uint32_t>(nt);
+                seqs += c;
+                nt_max = c != 0 ? nt : nt_max;
+            }
+            by_pair = tiles * static_cast<uint32_t>(n_heads) >= 4u * gridDim.x &&
+                      10u * tiles <= 7u * seqs * static_cast<uint32_t>(nt_max);
+        }
+        if (tid == 0) {
+            s_item[4] = by_pair ? 1u : 0u;
+        }
+        const int ratio = a.head_ratio;
+        const int n_heads_k = a.n_heads_k;
         uint32_t acc = 0;
         for (int l = 0; l < n_levels; ++l) {
-            s_level_start[l] = acc;
-            acc += s_bucket[n_levels - 1 - l] * static_cast<uint32_t>(n_heads);
+            s_queue_start[tid][l] = acc;
+            if (by_pair) {
+                const int nt = n_levels - l;
+                const uint32_t p0 = s_rank_start[nt] * static_cast<uint32_t>(n_heads_k);
+                const uint32_t p1 = s_rank_start[nt - 1] * static_cast<uint32_t>(n_heads_k);
+                // pairs p in [p0, p1) with p mod 8 == tid
+                const uint32_t mine = (p1 + kQueues - 1 - tid) / kQueues - (p0 + kQueues - 1 - tid) / kQueues;
+                acc += mine * static_cast<uint32_t>(nt * ratio);
+            } else if (tid == 0) {
+                acc += s_rank_start[n_levels - 1 - l] * static_cast<uint32_t>(n_heads);  // every pair that has this tile
+            }
         }
-        s_level_start[n_levels] = acc;
+        s_queue_start[tid][n_levels] = acc;
     }
     __syncthreads();
     // Stable scatter (sequences of one bucket stay in index order) by wavefront 0 alone: every workgroup
@@ -531,7 +596,6 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         }
     }
     __syncthreads();
-    const uint32_t n_items = s_level_start[n_levels];
 
     // ---- per-lane constants that do not depend on the item ----
     const uint32_t q_stride = static_cast<uint32_t>(a.n_heads_q) * a.d_qk * ES;  // bytes per row
@@ -587,7 +651,23 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
     float c_exp = a.c_exp;
     float c_out = a.c_out;
     float c_x = 1.0f;  // fp8 only: raw score -> alpha * (dequantised score)
-    const bool bias_vec = a.bias_vec_ok != 0;
+    // rab is added to S^T by the matrix pipe: S^T += E_j . R_j (j = 0, 1), where R_j holds, per lane (query row,
+    // half lh), the 8 consecutive rab values of keys 16 lh + 8 j .. + 7 exactly as they lie in memory (B operand)
+    // and E_j is the constant 0/1 matrix that routes k-slot (lh, e) to key row 16 lh + 8 j + e (A operand).
+    // This costs two MFMAs per sub-tile and no conversion, lane exchange or add on the vector ALU.
+    u32x4_t rab_route[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
+    if constexpr (HAS_RAB) {
+        const uint32_t one = std::is_same<Tag, bf16_tag>::value ? 0x3f80u : 0x3c00u;  // 1.0 in the input type
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int d = ln - 16 * lh - 8 * j;  // the element of this lane's row that is 1, if in 0..7
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                rab_route[j][i] = (d == 2 * i) ? one : (d == 2 * i + 1) ? (one << 16) : 0u;
+            }
+        }
+    }
+    const int bias_mode = a.bias_vec_ok;  // 0: element loads, 1: 8-byte loads, 2: 16-byte loads + lane exchange
 
     auto k_slot = [&](auto ic) -> uint16_t* {
         constexpr int I = decltype(ic)::value & 3;
@@ -615,25 +695,126 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
     };
 
     // =============================== item loop ===============================
-    uint32_t idx = blockIdx.x;
-    int lvl = 0;
-    while (idx < n_items) {
-        while (idx >= s_level_start[lvl + 1]) {
+    // The first item of a workgroup is fixed (workgroup w: item w / nq of queue w mod nq, nq = number of queues);
+    // later ones are pulled from the queue's counter.  With the pull, the position of the next non-empty queue is
+    // read as well: a workgroup whose queue is drained moves on to that queue if it still has items (and so on
+    // around the ring), otherwise it leaves.  Every queue keeps the workgroups of its own XCD until it is empty,
+    // so moving on only ever adds help.  One lane does this bookkeeping and the decoding of the item and hands
+    // the result to the workgroup through LDS.
+    int fq_queue = 0;           // lane 0 only: the queue this workgroup pulls from
+    uint32_t fq_idx = 0;        //              the item index it holds in that queue
+    bool fq_first = true;       //              nothing pulled yet
+    auto fetch_item = [&]() {   // executed by thread 0
+        const bool by_pair = QUEUES && s_item[4] != 0;
+        const int nq = by_pair ? kQueues : 1;
+        const int nq_shift = by_pair ? 3 : 0;
+        const int ratio = a.head_ratio;
+        const int n_heads_k = a.n_heads_k;
+        unsigned int* const counters = &g_work_counter[a.counter_slot][0];
+        auto fixed_items = [&](int qu) -> uint32_t {  // workgroups qu, qu + nq, ... took the first items of queue qu
+            return gridDim.x > static_cast<uint32_t>(qu) ? (gridDim.x - qu + nq - 1) >> nq_shift : 0u;
+        };
+        auto next_queue = [&](int qu) -> int {  // the next queue after qu that has items at all (qu itself if there is none)
+            for (int i = 1; i < nq; ++i) {
+                const int cand = (qu + i) & (nq - 1);
+                if (s_queue_start[cand][n_levels] != 0) {
+                    return cand;
+                }
+            }
+            return qu;
+        };
+        uint32_t other_next = 0;  // where the next non-empty queue stands, as far as known
+        bool other_known = false;
+        if (fq_first) {
+            fq_first = false;
+            fq_queue = static_cast<int>(blockIdx.x) & (nq - 1);
+            fq_idx = blockIdx.x >> nq_shift;
+        } else {
+            const int other = next_queue(fq_queue);
+            const uint32_t got = atomicAdd(&counters[fq_queue * kCounterStride], 1u);
+            if (other != fq_queue) {
+                other_next = fixed_items(other) + __hip_atomic_load(&counters[other * kCounterStride], __ATOMIC_RELAXED,
+                                                                    __HIP_MEMORY_SCOPE_AGENT);
+                other_known = true;
+            }
+            fq_idx = fixed_items(fq_queue) + got;
+        }
+        while (fq_idx >= s_queue_start[fq_queue][n_levels]) {
+            // this queue is drained (or empty from the start): help the next one if it has work left
+            const int other = next_queue(fq_queue);
+            if (other == fq_queue) {
+                s_item[0] = 0;
+                return;
+            }
+            if (!other_known) {
+                other_next = fixed_items(other);  // optimistic: nothing pulled there yet
+            }
+            if (other_next >= s_queue_start[other][n_levels]) {
+                s_item[0] = 0;
+                return;
+            }
+            fq_queue = other;
+            const int after = next_queue(other);
+            const uint32_t got = atomicAdd(&counters[other * kCounterStride], 1u);
+            other_known = after != other;
+            if (other_known) {
+                other_next = fixed_items(after) + __hip_atomic_load(&counters[after * kCounterStride], __ATOMIC_RELAXED,
+                                                                    __HIP_MEMORY_SCOPE_AGENT);
+            }
+            fq_idx = fixed_items(other) + got;
+        }
+        int lvl = 0;
+        while (fq_idx >= s_queue_start[fq_queue][lvl + 1]) {
             ++lvl;
         }
-        const int qt = n_levels - 1 - lvl;
-        const int in_level = static_cast<int>(idx - s_level_start[lvl]);
-        const int rank = in_level / n_heads;
-        const int h = in_level - rank * n_heads;
-        const int b = uniform(static_cast<int>(s_order[rank]));
-        const int hk = h / a.head_ratio;
+        const int j_item = static_cast<int>(fq_idx - s_queue_start[fq_queue][lvl]);
+        int qt, p_item, r_item;
+        if (by_pair) {
+            // item j of bucket lvl (pairs with nt tiles) = pair j / (nt * ratio) of this queue there, query tile
+            // nt - 1 - (j % (nt * ratio)) / ratio, query head (kv head) * ratio + j % ratio
+            const int nt_item = n_levels - lvl;
+            const int per_pair = nt_item * ratio;
+            const int m_item = j_item / per_pair;
+            const int rem_item = j_item - m_item * per_pair;
+            const int t_item = rem_item / ratio;
+            qt = nt_item - 1 - t_item;
+            r_item = rem_item - t_item * ratio;
+            const int p_first = static_cast<int>(s_rank_start[nt_item]) * n_heads_k;
+            p_item = p_first + ((fq_queue + kQueues - (p_first & (kQueues - 1))) & (kQueues - 1)) + m_item * kQueues;
+        } else {
+            // item j of level lvl (query tile qt) = pair j / ratio, query head (kv head) * ratio + j % ratio
+            qt = n_levels - 1 - lvl;
+            p_item = j_item / ratio;
+            r_item = j_item - p_item * ratio;
+        }
+        const int rank = p_item / n_heads_k;
+        const int hk_item = p_item - rank * n_heads_k;
+        s_item[0] = 1;
+        s_item[1] = static_cast<uint32_t>(qt);
+        s_item[2] = static_cast<uint32_t>(s_order[rank]);
+        s_item[3] = static_cast<uint32_t>(hk_item * ratio + r_item);
+        s_item[5] = (static_cast<uint32_t>(fq_queue) << 28) | fq_idx;  // (for the development item log)
+        s_item[6] = static_cast<uint32_t>(hk_item);
+    };
+    for (;;) {
+        if (tid == 0) {
+            fetch_item();
+        }
+        __syncthreads();
+        if (s_item[0] == 0) {
+            break;
+        }
+        const int qt = uniform(static_cast<int>(s_item[1]));
+        const int b = uniform(static_cast<int>(s_item[2]));
+        const int h = uniform(static_cast<int>(s_item[3]));
+        const int hk = uniform(static_cast<int>(s_item[6]));
 #ifdef HSTU_TIMELINE
         int log_slot = 0;
         if (a.timeline && lane == 0) {
             unsigned long long* row = a.timeline + (static_cast<int64_t>(blockIdx.x) * 4 + wave) * 64;
             log_slot = static_cast<int>(row[0]);
             if (log_slot < 15) {
-                row[1 + 4 * log_slot + 0] = idx;
+                row[1 + 4 * log_slot + 0] = s_item[5];
                 row[1 + 4 * log_slot + 1] = HSTU_CLOCK();
             }
         }
@@ -798,12 +979,59 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             HAS_MASK ? static_cast<const uint16_t*>(a.mask) + bias_plane : nullptr, HAS_MASK ? bias_bytes : 0u);
         const uint32_t bias_row_off = static_cast<uint32_t>(wr0 + ln) * static_cast<uint32_t>(a.max_k) * 2u;
 
-        // loads the 16 bias (or mask) values of one 32-key sub-tile in accumulator order, as 8 packed words
+        // Requests the rab values of keys c0 + 16 lh .. + 15 of this lane's row, 8 packed words in memory order
+        // (what the routing MFMAs above take as their B operands).
+        auto load_rab = [&](int c0, uint32_t (&w)[8]) {
+            const uint32_t off = bias_row_off + static_cast<uint32_t>(c0 + 16 * lh) * 2u;
+            if (bias_mode == 2) {
+                const U32Quad t0 = __builtin_bit_cast(U32Quad, __builtin_amdgcn_raw_buffer_load_b128(rab_rsrc, static_cast<int>(off), 0, 0));
+                const U32Quad t1 = __builtin_bit_cast(U32Quad, __builtin_amdgcn_raw_buffer_load_b128(rab_rsrc, static_cast<int>(off + 16u), 0, 0));
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    w[i] = t0.v[i];
+                    w[4 + i] = t1.v[i];
+                }
+            } else if (bias_mode == 1) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const U32Pair t = __builtin_bit_cast(
+                        U32Pair, __builtin_amdgcn_raw_buffer_load_b64(rab_rsrc, static_cast<int>(off + 8u * i), 0, 0));
+                    w[2 * i + 0] = t.v[0];
+                    w[2 * i + 1] = t.v[1];
+                }
+            } else {
+                uint32_t eoff = off;
+                asm volatile("" : "+v"(eoff));  // (keeps the optimiser from relating these to the vector loads above)
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const uint32_t e0 = __builtin_amdgcn_raw_buffer_load_b16(rab_rsrc, static_cast<int>(eoff + 4u * i), 0, 0);
+                    const uint32_t e1 = __builtin_amdgcn_raw_buffer_load_b16(rab_rsrc, static_cast<int>(eoff + 4u * i + 2u), 0, 0);
+                    w[i] = (e0 & 0xffffu) | (e1 << 16);
+                }
+            }
+        };
+        // Requests the 16 bias (or mask) values of one 32-key sub-tile as 8 packed words; order_bias() must be
+        // applied to the words once they are about to be used.
+        // Mode 2 (rows 16-byte aligned): the two lanes of a row (lh = 0, 1) read 32 contiguous bytes each (keys
+        // 16 lh .. 16 lh + 15), i.e. the row's 64 bytes in two 16-byte loads per lane instead of four 8-byte
+        // loads; the accumulator layout wants keys 8g + 4 lh + 0..3 per lane, so the lanes exchange half of
+        // what they read (v_permlane32_swap, in order_bias).
         auto load_bias = [&](__amdgpu_buffer_rsrc_t rsrc, int c0, uint32_t (&w)[8]) {
+            if (bias_mode == 2) {
+                const uint32_t off = bias_row_off + static_cast<uint32_t>(c0 + 16 * lh) * 2u;
+                const U32Quad t0 = __builtin_bit_cast(U32Quad, __builtin_amdgcn_raw_buffer_load_b128(rsrc, static_cast<int>(off), 0, 0));
+                const U32Quad t1 = __builtin_bit_cast(U32Quad, __builtin_amdgcn_raw_buffer_load_b128(rsrc, static_cast<int>(off + 16u), 0, 0));
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    w[i] = t0.v[i];
+                    w[4 + i] = t1.v[i];
+                }
+                return;
+            }
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 const uint32_t off = bias_row_off + static_cast<uint32_t>(c0 + 8 * g + 4 * lh) * 2u;
-                if (bias_vec) {
+                if (bias_mode == 1) {
                     // (reinterpreted as a struct before its words are taken: taking integer elements
                     // straight from the builtin's vector result is narrowed to a one-element load by the
                     // optimiser of this toolchain)
@@ -823,6 +1051,31 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                     w[2 * g + 0] = (e0 & 0xffffu) | (e1 << 16);
                     w[2 * g + 1] = (e2 & 0xffffu) | (e3 << 16);
                 }
+            }
+        };
+
+        // brings requested words into accumulator order (word 2g, 2g+1 = keys 8g + 4 lh + 0..3)
+        auto order_bias = [&](uint32_t (&w)[8]) {
+            if (bias_mode == 2) {
+                // lane (row, 0) holds words d0..d7 (keys 0..15), lane (row, 1) d8..d15; lh = 0 wants d0 d1 d4 d5 d8 d9
+                // d12 d13, lh = 1 wants d2 d3 d6 d7 d10 d11 d14 d15: words 2, 3, 6, 7 of the lower half-wave trade
+                // places with words 0, 1, 4, 5 of the upper one
+                typedef __attribute__((ext_vector_type(2))) unsigned u2_t;
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+#pragma unroll
+                    for (int j = 0; j < 2; ++j) {
+                        const u2_t r = __builtin_amdgcn_permlane32_swap(w[4 * i + j], w[4 * i + 2 + j], false, false);
+                        w[4 * i + j] = r[0];
+                        w[4 * i + 2 + j] = r[1];
+                    }
+                }
+                // now {w0 w1 | w2 w3 | w4 w5 | w6 w7} = groups g = {0 | 2 | 1 | 3}
+                const uint32_t t2 = w[2], t3 = w[3];
+                w[2] = w[4];
+                w[3] = w[5];
+                w[4] = t2;
+                w[5] = t3;
             }
         };
 
@@ -855,7 +1108,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         }
         if constexpr (HAS_RAB) {
             if (nx_w > 0) {
-                load_bias(rab_rsrc, 0, rabw0);
+                load_rab(0, rabw0);
             }
 
         }
@@ -868,10 +1121,10 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             f32x16_t& s_nxt = PAR ? s_blk0 : s_blk1;        // S^T(t+1), accumulated in this step
             uint32_t(&pk_cur)[8] = PAR ? p_blk1 : p_blk0;         // P^T(t), written
             const uint32_t(&pk_prev)[8] = PAR ? p_blk0 : p_blk1;  // P^T(t-1), consumed
-            const uint32_t(&mw_cur)[8] = PAR ? mw1 : mw0;         // custom mask words of sub-tile t
+            uint32_t(&mw_cur)[8] = PAR ? mw1 : mw0;               // custom mask words of sub-tile t
             uint32_t(&mw_nxt)[8] = PAR ? mw0 : mw1;
             uint32_t(&rab_far)[8] = PAR ? rabw1 : rabw0;          // receives rab(t+2)
-            const uint32_t(&rab_nxt)[8] = PAR ? rabw0 : rabw1;    // rab(t+1)
+            uint32_t(&rab_nxt)[8] = PAR ? rabw0 : rabw1;          // rab(t+1)
             const uint16_t* const kt = k_slot(std::integral_constant<int, (S + 1) & 3>{});  // K(t+1)
             const uint16_t* const vt = v_slot(std::integral_constant<int, (S + 3) & 3>{});  // V(t-1)
             const int c0 = t * 32;
@@ -885,7 +1138,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             //     that waiting for them never waits for a younger tile
             if constexpr (HAS_RAB) {
                 if (t + 2 < nx_w) {
-                    load_bias(rab_rsrc, c0 + 64, rab_far);
+                    load_rab(c0 + 64, rab_far);
                 }
             }
             if constexpr (HAS_MASK) {
@@ -973,6 +1226,11 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             };
             constexpr int LOOKAHEAD = NCH >= 4 ? 2 : 1;
 
+            if constexpr (HAS_MASK) {
+                if (do_silu) {
+                    order_bias(mw_cur);
+                }
+            }
             if (do_pv) {
                 u32x4_t vop[NCH];
 #pragma unroll
@@ -1041,17 +1299,10 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                 for (int c = 0; c < LOOKAHEAD; ++c) {
                     kop[c] = read_k(c);
                 }
-                if constexpr (HAS_RAB) {
-#pragma unroll
-                    for (int i = 0; i < 8; ++i) {
-                        s_nxt[2 * i + 0] = lo_to_float<Tag>(rab_nxt[i]);
-                        s_nxt[2 * i + 1] = hi_to_float<Tag>(rab_nxt[i]);
-                    }
-                }
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int c = 0; c < NCH; ++c) {
-                    if (c == 0 && !HAS_RAB) {
+                    if (c == 0) {
                         f32x16_t zero;
 #pragma unroll
                         for (int i = 0; i < 16; ++i) {
@@ -1066,6 +1317,13 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                     }
                     silu_chunk(4, c);
                     __builtin_amdgcn_sched_barrier(0);
+                }
+                if constexpr (HAS_RAB) {
+                    // S^T(t+1) += rab^T, last so that the rab request has had the whole block to land
+                    const u32x4_t r0 = {rab_nxt[0], rab_nxt[1], rab_nxt[2], rab_nxt[3]};
+                    const u32x4_t r1 = {rab_nxt[4], rab_nxt[5], rab_nxt[6], rab_nxt[7]};
+                    s_nxt = mfma32<Tag>(rab_route[0], r0, s_nxt);
+                    s_nxt = mfma32<Tag>(rab_route[1], r1, s_nxt);
                 }
             } else if (do_silu) {
 #pragma unroll
@@ -1152,20 +1410,16 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         }
 #endif
 
-        // ---- pull the next item ----
-        if (tid == 0) {
-            s_next = gridDim.x + atomicAdd(&g_work_counter[a.counter_slot], 1u);
-        }
-        __syncthreads();
-        idx = s_next;
-        __syncthreads();  // everyone has read s_next before thread 0 may overwrite it again
+        // (the barriers of the sweep separate this item's reads of s_item from the next fetch)
     }
 
     // ---- leave: the last workgroup out puts the counters of this slot back to zero ----
     if (tid == 0) {
         const unsigned int left = atomicAdd(&g_done_counter[a.counter_slot], 1u);
         if (left == gridDim.x - 1) {
-            g_work_counter[a.counter_slot] = 0;
+            for (int qu = 0; qu < kQueues; ++qu) {
+                g_work_counter[a.counter_slot][qu * kCounterStride] = 0;
+            }
             __threadfence();
             g_done_counter[a.counter_slot] = 0;
         }

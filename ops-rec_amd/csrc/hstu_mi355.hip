@@ -30,9 +30,11 @@ int fail(int code, const char* fmt, ...)
     return code;
 }
 
+// kernel variants with the per-XCD work queues exist for the head-dim slots 64 and 128 (nullptr elsewhere)
 struct Variant {
     const char* name;
     void (*kernel)(const hstu::FwdArgs);
+    void (*kernel_queues)(const hstu::FwdArgs);  // the same with per-XCD work queues, for long lists; may be nullptr
     int d_pad;
     int threads;
     int persistent_wgs_per_cu;  // > 0: persistent kernel, this many workgroups per CU; 0: one workgroup per tile
@@ -64,9 +66,20 @@ int compute_units(int* out)
 
 std::atomic<unsigned> g_next_counter_slot{0};
 
+template <typename Tag, typename OutTag, int D, bool RAB, bool MASK>
+constexpr auto queues_kernel() -> void (*)(const hstu::FwdArgs)
+{
+    if constexpr (D == 64 || D == 128) {
+        return hstu::hstu_fwd_kernel<Tag, OutTag, D, RAB, MASK, true>;
+    } else {
+        return nullptr;
+    }
+}
+
 #define HSTU_VARIANT(tag, tagname, D, RAB, MASK, WGS)                                               \
     {"hstu_fwd_" tagname "_d" #D "_rab" #RAB "_mask" #MASK,                                        \
-     hstu::hstu_fwd_kernel<hstu::tag, hstu::tag, D, RAB, MASK>, D, 256, WGS}
+     hstu::hstu_fwd_kernel<hstu::tag, hstu::tag, D, RAB, MASK>,                                     \
+     queues_kernel<hstu::tag, hstu::tag, D, RAB, MASK>(), D, 256, WGS}
 #define HSTU_DIMS(tag, tagname, RAB, MASK)                                                           \
     {HSTU_VARIANT(tag, tagname, 32, RAB, MASK, 2), HSTU_VARIANT(tag, tagname, 64, RAB, MASK, 2), \
      HSTU_VARIANT(tag, tagname, 128, RAB, MASK, 2), HSTU_VARIANT(tag, tagname, 256, RAB, MASK, 1)}
@@ -80,14 +93,15 @@ const Variant kVariants[2][2][2][4] = {
 };
 
 #define HSTU_F32_VARIANT(D, RAB, MASK) \
-    {"hstu_fwd_f32_d" #D "_rab" #RAB "_mask" #MASK, hstu::hstu_fwd_f32_kernel<D, RAB, MASK>, D, 256, 0}
+    {"hstu_fwd_f32_d" #D "_rab" #RAB "_mask" #MASK, hstu::hstu_fwd_f32_kernel<D, RAB, MASK>, nullptr, D, 256, 0}
 #define HSTU_F32_DIMS(RAB, MASK) \
     {HSTU_F32_VARIANT(32, RAB, MASK), HSTU_F32_VARIANT(64, RAB, MASK), HSTU_F32_VARIANT(128, RAB, MASK), \
      HSTU_F32_VARIANT(256, RAB, MASK)}
 // fp32 inputs: [rab][custom mask][dim slot]
 // fp8-e4m3 inputs: [output: fp16, bf16][dim slot: 64, 128, 256] (no rab, no custom mask)
 #define HSTU_F8_VARIANT(otag, oname, D, WGS)                                                         \
-    {"hstu_fwd_f8e4m3_" oname "_d" #D, hstu::hstu_fwd_kernel<hstu::f8_tag, hstu::otag, D, false, false>, D, 256, WGS}
+    {"hstu_fwd_f8e4m3_" oname "_d" #D, hstu::hstu_fwd_kernel<hstu::f8_tag, hstu::otag, D, false, false>,     \
+     queues_kernel<hstu::f8_tag, hstu::otag, D, false, false>(), D, 256, WGS}
 const Variant kVariantsF8[2][3] = {
     {HSTU_F8_VARIANT(f16_tag, "f16", 64, 2), HSTU_F8_VARIANT(f16_tag, "f16", 128, 2), HSTU_F8_VARIANT(f16_tag, "f16", 256, 1)},
     {HSTU_F8_VARIANT(bf16_tag, "bf16", 64, 2), HSTU_F8_VARIANT(bf16_tag, "bf16", 128, 2),
@@ -315,6 +329,10 @@ HSTU_API int hstu_jagged_fwd(const hstu_jagged_fwd_params* p, void* workspace, u
     const bool bias_aligned = (reinterpret_cast<uintptr_t>(p->attn_bias) % vec_bytes == 0) &&
                               (reinterpret_cast<uintptr_t>(p->mask) % vec_bytes == 0) && (p->max_seq_len_k % 4 == 0);
     a.bias_vec_ok = bias_aligned ? 1 : 0;
+    if (bias_aligned && p->dtype != HSTU_DT_FP32 && reinterpret_cast<uintptr_t>(p->attn_bias) % 16 == 0 &&
+        reinterpret_cast<uintptr_t>(p->mask) % 16 == 0 && p->max_seq_len_k % 8 == 0) {
+        a.bias_vec_ok = 2;  // 16-byte row alignment: the 16-bit kernels read rab / mask rows 32 bytes per lane
+    }
     const double scale = (p->silu_scale == 0.0) ? 1.0 / static_cast<double>(p->max_seq_len_q) : p->silu_scale;
     a.c_exp = static_cast<float>(-p->alpha * 1.4426950408889634);
     a.c_out = static_cast<float>(p->alpha * scale);
@@ -331,6 +349,7 @@ HSTU_API int hstu_jagged_fwd(const hstu_jagged_fwd_params* p, void* workspace, u
     if (n_blocks <= 0 || n_blocks > 0x7fffffffLL) {
         return fail(HSTU_ERR_INVALID, "grid of %lld workgroups is out of range", (long long)n_blocks);
     }
+    void (*kernel)(const hstu::FwdArgs) = var->kernel;
     if (var->persistent_wgs_per_cu > 0) {
         // persistent kernel: a fixed number of workgroups pulls the (at most n_blocks) work items
         int cus = 0;
@@ -339,10 +358,14 @@ HSTU_API int hstu_jagged_fwd(const hstu_jagged_fwd_params* p, void* workspace, u
             return rc_cu;
         }
         const int64_t resident = static_cast<int64_t>(cus) * var->persistent_wgs_per_cu;
+        // the variant with per-XCD queues can only pay when the list may hold several items per workgroup
+        if (var->kernel_queues != nullptr && n_blocks >= 4 * resident) {
+            kernel = var->kernel_queues;
+        }
         n_blocks = n_blocks < resident ? n_blocks : resident;
         a.counter_slot = static_cast<int>(g_next_counter_slot.fetch_add(1) % hstu::kCounterSlots);
     }
-    hipLaunchKernelGGL(var->kernel, dim3(static_cast<unsigned>(n_blocks)), dim3(static_cast<unsigned>(var->threads)), 0,
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(n_blocks)), dim3(static_cast<unsigned>(var->threads)), 0,
                        static_cast<hipStream_t>(stream), a);
     const hipError_t err = hipGetLastError();
     if (err != hipSuccess) {
