@@ -33,6 +33,7 @@ int fail(int code, const char* fmt, ...)
 // kernel variants with the per-XCD work queues exist for the head-dim slots 64 and 128 (nullptr elsewhere)
 struct Variant {
     const char* name;
+    const char* name_queues;
     void (*kernel)(const hstu::FwdArgs);
     void (*kernel_queues)(const hstu::FwdArgs);  // the same with per-XCD work queues, for long lists; may be nullptr
     int d_pad;
@@ -78,6 +79,7 @@ constexpr auto queues_kernel() -> void (*)(const hstu::FwdArgs)
 
 #define HSTU_VARIANT(tag, tagname, D, RAB, MASK, WGS)                                               \
     {"hstu_fwd_" tagname "_d" #D "_rab" #RAB "_mask" #MASK,                                        \
+     "hstu_fwd_" tagname "_d" #D "_rab" #RAB "_mask" #MASK "_queues",                               \
      hstu::hstu_fwd_kernel<hstu::tag, hstu::tag, D, RAB, MASK>,                                     \
      queues_kernel<hstu::tag, hstu::tag, D, RAB, MASK>(), D, 256, WGS}
 #define HSTU_DIMS(tag, tagname, RAB, MASK)                                                           \
@@ -93,14 +95,15 @@ const Variant kVariants[2][2][2][4] = {
 };
 
 #define HSTU_F32_VARIANT(D, RAB, MASK) \
-    {"hstu_fwd_f32_d" #D "_rab" #RAB "_mask" #MASK, hstu::hstu_fwd_f32_kernel<D, RAB, MASK>, nullptr, D, 256, 0}
+    {"hstu_fwd_f32_d" #D "_rab" #RAB "_mask" #MASK, nullptr, hstu::hstu_fwd_f32_kernel<D, RAB, MASK>, nullptr, D, 256, 0}
 #define HSTU_F32_DIMS(RAB, MASK) \
     {HSTU_F32_VARIANT(32, RAB, MASK), HSTU_F32_VARIANT(64, RAB, MASK), HSTU_F32_VARIANT(128, RAB, MASK), \
      HSTU_F32_VARIANT(256, RAB, MASK)}
 // fp32 inputs: [rab][custom mask][dim slot]
 // fp8-e4m3 inputs: [output: fp16, bf16][dim slot: 64, 128, 256] (no rab, no custom mask)
 #define HSTU_F8_VARIANT(otag, oname, D, WGS)                                                         \
-    {"hstu_fwd_f8e4m3_" oname "_d" #D, hstu::hstu_fwd_kernel<hstu::f8_tag, hstu::otag, D, false, false>,     \
+    {"hstu_fwd_f8e4m3_" oname "_d" #D, "hstu_fwd_f8e4m3_" oname "_d" #D "_queues",                              \
+     hstu::hstu_fwd_kernel<hstu::f8_tag, hstu::otag, D, false, false>,                                         \
      queues_kernel<hstu::f8_tag, hstu::otag, D, false, false>(), D, 256, WGS}
 const Variant kVariantsF8[2][3] = {
     {HSTU_F8_VARIANT(f16_tag, "f16", 64, 2), HSTU_F8_VARIANT(f16_tag, "f16", 128, 2), HSTU_F8_VARIANT(f16_tag, "f16", 256, 1)},
@@ -247,6 +250,26 @@ const Variant* select(const hstu_jagged_fwd_params* p)
                      [p->mask_type == HSTU_MASK_CUSTOM ? 1 : 0][slot];
 }
 
+// whether the launch described by p takes the variant with per-XCD work queues: only when the list may hold
+// several items per resident workgroup.  *resident_out (optional) receives the resident grid.
+bool takes_queue_variant(const Variant* var, const hstu_jagged_fwd_params* p, int64_t* resident_out)
+{
+    if (var->persistent_wgs_per_cu <= 0) {
+        return false;
+    }
+    int cus = 0;
+    if (compute_units(&cus) != HSTU_OK) {
+        return false;
+    }
+    const int64_t resident = static_cast<int64_t>(cus) * var->persistent_wgs_per_cu;
+    if (resident_out != nullptr) {
+        *resident_out = resident;
+    }
+    const int64_t n_qtiles = (p->max_seq_len_q + hstu::kBlockM - 1) / hstu::kBlockM;
+    const int64_t n_blocks = n_qtiles * (p->n_offsets - 1) * p->num_heads_q;
+    return var->kernel_queues != nullptr && n_blocks >= 4 * resident;
+}
+
 }  // namespace
 
 extern "C" {
@@ -279,7 +302,11 @@ HSTU_API const char* hstu_jagged_fwd_kernel_name(const hstu_jagged_fwd_params* p
         return nullptr;
     }
     const Variant* v = select(params);
-    return v ? v->name : nullptr;
+    if (v == nullptr) {
+        return nullptr;
+    }
+    // (without a usable device the plain name is reported)
+    return takes_queue_variant(v, params, nullptr) ? v->name_queues : v->name;
 }
 
 HSTU_API int hstu_jagged_fwd(const hstu_jagged_fwd_params* p, void* workspace, uint64_t workspace_bytes, void* stream)
@@ -357,9 +384,8 @@ HSTU_API int hstu_jagged_fwd(const hstu_jagged_fwd_params* p, void* workspace, u
         if (rc_cu != HSTU_OK) {
             return rc_cu;
         }
-        const int64_t resident = static_cast<int64_t>(cus) * var->persistent_wgs_per_cu;
-        // the variant with per-XCD queues can only pay when the list may hold several items per workgroup
-        if (var->kernel_queues != nullptr && n_blocks >= 4 * resident) {
+        int64_t resident = static_cast<int64_t>(cus) * var->persistent_wgs_per_cu;
+        if (takes_queue_variant(var, p, &resident)) {
             kernel = var->kernel_queues;
         }
         n_blocks = n_blocks < resident ? n_blocks : resident;
