@@ -117,7 +117,14 @@ typedef struct hstu_jagged_fwd_params {
 } hstu_jagged_fwd_params;
 
 /* replaces aclnnHstuJaggedForwardGetWorkspaceSize: validates the description and reports the scratch
- * size (may be 0).  No device work. */
+ * size (may be 0).  No device work.
+ * Scratch is asked for by calls whose work list may be shorter than the machine (few, long sequences): the
+ * kernel then cuts the key range of long items into parts that run on different workgroups and adds their
+ * fp32 partial outputs, in a fixed order, through the workspace (contents undefined before and after; 16-byte
+ * aligned).  A caller that passes less than asked for, or nothing, gets the same results computed without
+ * that split.  Because a split changes the order of the fp32 sums, the last bit of an output element may then
+ * depend on what else is in the batch; HSTU_MI355_SPLIT=0 in the environment turns the split off (the size
+ * reported is then 0). */
 HSTU_API int hstu_jagged_fwd_workspace_size(const hstu_jagged_fwd_params* params, uint64_t* workspace_bytes);
 
 /* replaces aclnnHstuJaggedForward: enqueues the forward on `stream` (a hipStream_t passed as void*;

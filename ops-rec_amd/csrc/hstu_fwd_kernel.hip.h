@@ -124,6 +124,8 @@ struct FwdArgs {
     const float* k_descale;
     const float* v_descale;
     int counter_slot;  // which pair of device-side work counters this launch uses
+    float* ws;           // split variant: room for ws_parts partial outputs of kBlockM x D floats each (may be null)
+    uint32_t ws_parts;
 #ifdef HSTU_TIMELINE
     unsigned long long* timeline;
 #endif
@@ -361,6 +363,12 @@ constexpr int kCounterStride = 32;  // counters of different queues sit in diffe
 static __device__ unsigned int g_work_counter[kCounterSlots][kQueues * kCounterStride];
 static __device__ unsigned int g_done_counter[kCounterSlots];
 
+// Split items (see "Splitting long items" in the kernel): one arrival counter per split item, same life cycle
+// as the work counters (zero at load; the workgroup that completes an item puts its counter back to zero).
+constexpr int kMaxSplitItems = 2048;
+constexpr int kMaxParts = 8;
+static __device__ unsigned int g_split_arrived[kCounterSlots][kMaxSplitItems];
+
 constexpr int kMaxBatchSlots = 2048;  // sequences per call (the reference's limit)
 constexpr int kMaxLevels = 160;       // ceil(20480 / 128) query-tile levels
 
@@ -417,7 +425,12 @@ struct U32Quad {
 // QUEUES: build the per-XCD queue machinery (see "Work queues" below).  It pays on long, jagged batches with many
 // items per workgroup; its code is on the path of every item, so launches that cannot profit (the host decides by
 // an upper bound on the number of items) use the variant without it.
-template <typename Tag, typename OutTag, int D, bool HAS_RAB, bool HAS_MASK, bool QUEUES = false>
+//
+// SPLIT: a list with fewer items than workgroups leaves compute units idle while its longest item runs.  This
+// variant cuts the key range of the long items into up to kMaxParts parts that are separate entries of the work
+// list ("Splitting long items" below); the host uses it when the list is short and a workspace is supplied.  It
+// excludes QUEUES.
+template <typename Tag, typename OutTag, int D, bool HAS_RAB, bool HAS_MASK, bool QUEUES = false, bool SPLIT = false>
 __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const FwdArgs a)
 {
     constexpr int kThreads = 256;
@@ -425,6 +438,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
     constexpr uint32_t ES = elem_traits<Tag>::kBytes;  // bytes per input element
     static_assert(!F8 || (!HAS_RAB && !HAS_MASK), "no rab / custom mask with fp8 inputs");
     static_assert(!F8 || D >= 64, "fp8 rows are at least 64 bytes");
+    static_assert(!(QUEUES && SPLIT), "one list policy per variant");
     constexpr int CPR = D * ES / 16;             // 16-byte chunks per row
     constexpr int EPC16 = 16 / ES;               // elements per 16-byte chunk
     constexpr int SUB_ELEMS = 32 * D * ES / 2;   // one 32-key sub-tile, in 16-bit units
@@ -455,7 +469,11 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
     __shared__ uint32_t s_bucket[kMaxLevels + 2];         // histogram, then scatter cursors
     __shared__ uint32_t s_rank_start[kMaxLevels + 2];     // [nt]: number of sequences with more than nt query tiles
     __shared__ uint32_t s_queue_start[QUEUES ? kQueues : 1][kMaxLevels + 2];  // per queue: first item of each level / bucket
-    __shared__ uint32_t s_item[8];  // [0..3]: the item handed to the workgroup (valid, query tile, sequence, head); [4]: queue order
+    __shared__ uint32_t s_item[12];  // [0..3]: the item handed to the workgroup (valid, query tile, sequence, head); [4]: queue order
+                                     // [7]: part | parts << 8, [8]: arrival counter, [9]: first partial buffer, [10]: arrivals before
+    __shared__ uint8_t s_parts[SPLIT ? kMaxLevels + 2 : 1];         // parts per item of each level
+    __shared__ uint32_t s_split_first[SPLIT ? kMaxLevels + 2 : 1];  // first arrival counter of each split level
+    __shared__ uint32_t s_ws_first[SPLIT ? kMaxLevels + 2 : 1];     // first partial buffer of each split level
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -552,9 +570,62 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         }
         const int ratio = a.head_ratio;
         const int n_heads_k = a.n_heads_k;
+        // Splitting long items.  Level l holds the items of query tile qt = n_levels - 1 - l; under the built-in
+        // mask such an item sweeps about 4 (qt + 1) sub-tiles, otherwise all of max_seq_len_k.  With `target` = the
+        // mean number of time steps per workgroup (3 steps of start-up per item included, never below 8), the items
+        // of a level whose nominal length exceeds it are listed as m = ceil(nominal / target) entries (at most
+        // kMaxParts), one per part of the key range, next to each other in the list.  Part i sweeps the sub-tiles
+        // [i * len, (i + 1) * len) of the item's real range, len a multiple of 4; it writes its fp32 accumulators
+        // to its own buffer in the workspace and counts itself in; the part that finds all others counted in adds
+        // the m buffers in part order (so the sum does not depend on who came last) and stores the rows.
+        // A level is split only while arrival counters and workspace buffers last, and nothing is split when the
+        // list has an item for every workgroup anyway: measured on MI355X, a part costs about 2 us on top of its
+        // sweep (its own start-up, the hand-over of its accumulators), which a list of 1.4 items per workgroup
+        // (batch 32 x 4 heads, lengths 256..1024) no longer earns back, while a list that leaves workgroups idle
+        // (one 20480-row sequence, or 4 sequences x 2 heads up to 3000 rows) finishes in 0.5 - 0.65 of the time.
+        uint32_t split_target = 0;
+        uint32_t split_items = 0, split_bufs = 0;
+        auto nominal_steps = [&](int qt) -> uint32_t {
+            const int all = (a.max_k + 31) / 32;
+            if (a.mask_type != 0) {
+                return static_cast<uint32_t>(all);
+            }
+            const int causal = 4 * (qt + 1) + (a.max_k > a.max_q ? (a.max_k - a.max_q) / 32 : 0);
+            return static_cast<uint32_t>(causal < all ? causal : all);
+        };
+        if constexpr (SPLIT) {
+            uint32_t steps = 0, items = 0;
+            for (int l = 0; l < n_levels; ++l) {
+                const uint32_t cnt = s_rank_start[n_levels - 1 - l] * static_cast<uint32_t>(n_heads);
+                steps += cnt * (nominal_steps(n_levels - 1 - l) + 3u);
+                items += cnt;
+            }
+            split_target = steps / gridDim.x;
+            split_target = split_target < 8u ? 8u : split_target;
+            if (a.ws == nullptr || items >= gridDim.x) {
+                split_target = 0x7fffffffu;  // nothing is split
+            }
+        }
         uint32_t acc = 0;
         for (int l = 0; l < n_levels; ++l) {
             s_queue_start[tid][l] = acc;
+            if constexpr (SPLIT) {
+                const uint32_t cnt = s_rank_start[n_levels - 1 - l] * static_cast<uint32_t>(n_heads);
+                uint32_t m = (nominal_steps(n_levels - 1 - l) + split_target - 1u) / split_target;
+                m = m > static_cast<uint32_t>(kMaxParts) ? static_cast<uint32_t>(kMaxParts) : m;
+                if (m > 1u && (split_items + cnt > static_cast<uint32_t>(kMaxSplitItems) || split_bufs + cnt * m > a.ws_parts)) {
+                    m = 1u;
+                }
+                s_parts[l] = static_cast<uint8_t>(m);
+                s_split_first[l] = split_items;
+                s_ws_first[l] = split_bufs;
+                if (m > 1u) {
+                    split_items += cnt;
+                    split_bufs += cnt * m;
+                }
+                acc += cnt * m;
+                continue;
+            }
             if (by_pair) {
                 const int nt = n_levels - l;
                 const uint32_t p0 = s_rank_start[nt] * static_cast<uint32_t>(n_heads_k);
@@ -784,8 +855,17 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         } else {
             // item j of level lvl (query tile qt) = pair j / ratio, query head (kv head) * ratio + j % ratio
             qt = n_levels - 1 - lvl;
-            p_item = j_item / ratio;
-            r_item = j_item - p_item * ratio;
+            int j_whole = j_item;
+            if constexpr (SPLIT) {
+                // entry j of a split level = part j % m of item j / m
+                const int m = s_parts[lvl];
+                j_whole = j_item / m;
+                s_item[7] = static_cast<uint32_t>(j_item - j_whole * m) | (static_cast<uint32_t>(m) << 8);
+                s_item[8] = s_split_first[lvl] + static_cast<uint32_t>(j_whole);
+                s_item[9] = s_ws_first[lvl] + static_cast<uint32_t>(j_whole * m);
+            }
+            p_item = j_whole / ratio;
+            r_item = j_whole - p_item * ratio;
         }
         const int rank = p_item / n_heads_k;
         const int hk_item = p_item - rank * n_heads_k;
@@ -813,9 +893,9 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         if (a.timeline && lane == 0) {
             unsigned long long* row = a.timeline + (static_cast<int64_t>(blockIdx.x) * 4 + wave) * 64;
             log_slot = static_cast<int>(row[0]);
-            if (log_slot < 15) {
-                row[1 + 4 * log_slot + 0] = s_item[5];
-                row[1 + 4 * log_slot + 1] = HSTU_CLOCK();
+            if (log_slot < 12) {
+                row[1 + 5 * log_slot + 0] = s_item[5] | (static_cast<unsigned long long>(SPLIT ? s_item[7] : 0u) << 32);
+                row[1 + 5 * log_slot + 1] = HSTU_CLOCK();
             }
         }
 #endif
@@ -890,12 +970,27 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         } else {
             kmax = sk;
         }
-        const int n_sub = (kmax + 31) / 32;  // sub-tiles swept by the workgroup
+        const int n_sub = (kmax + 31) / 32;  // sub-tiles swept for the item
+        // the part of them this entry of the list stands for
+        int x_begin = 0;
+        int x_end = n_sub;
+        int part = 0;
+        int n_parts = 1;
+        if constexpr (SPLIT) {
+            part = uniform(static_cast<int>(s_item[7] & 0xffu));
+            n_parts = uniform(static_cast<int>(s_item[7] >> 8));
+            if (n_parts > 1) {
+                const int len = ((n_sub + n_parts - 1) / n_parts + 3) & ~3;
+                x_begin = part * len;
+                x_begin = x_begin < n_sub ? x_begin : n_sub;
+                x_end = x_begin + len < n_sub ? x_begin + len : n_sub;
+            }
+        }
 
         // requests for K sub-tile xk into K slot KS and V sub-tile xv into V slot VS
         auto request_k = [&](auto ks, int xk) {
             if (NLW == 4 || wave < NLW) {
-                const uint32_t kb = (xk < n_sub) ? static_cast<uint32_t>(xk * 32) * k_stride : kPastEnd;
+                const uint32_t kb = (xk < x_end) ? static_cast<uint32_t>(xk * 32) * k_stride : kPastEnd;
                 uint16_t* const dst = k_slot(ks);
 #pragma unroll
                 for (int i = 0; i < LPW; ++i) {
@@ -905,7 +1000,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         };
         auto request_v = [&](auto vs, int xv) {
             if (NLW == 4 || wave < NLW) {
-                const uint32_t vb = (xv < n_sub) ? static_cast<uint32_t>(xv * 32) * v_stride : kPastEnd;
+                const uint32_t vb = (xv < x_end) ? static_cast<uint32_t>(xv * 32) * v_stride : kPastEnd;
                 uint16_t* const dst = v_slot(vs);
 #pragma unroll
                 for (int i = 0; i < LPW; ++i) {
@@ -919,10 +1014,11 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         typedef std::integral_constant<int, 3> ic3_t;
 
         // ---- start-up: what the times before the first would have requested, and the Q fragment ----
-        request_k(ic0_t{}, 0);
-        request_v(ic0_t{}, 0);
-        request_k(ic1_t{}, 1);
-        request_k(ic2_t{}, 2);
+        // (x_begin is a multiple of 4: sub-tile x_begin + i belongs in slot i)
+        request_k(ic0_t{}, x_begin);
+        request_v(ic0_t{}, x_begin);
+        request_k(ic1_t{}, x_begin + 1);
+        request_k(ic2_t{}, x_begin + 2);
         // Q fragment: lane (ln, lh) holds Q[row][16*js + 8*lh .. +7] for js = 0..KSTEPS-1
         // (fp8: 16 bytes per pair of steps, dims 16 * (2 * jp + lh) .. + 15, low half for step 2 jp)
         u32x4_t qf[KREADS];
@@ -963,7 +1059,8 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         const int lim_min = wb.lim_min;
         const int hole_hi_max = wb.hole_hi_max;
         const bool any_hole = wb.any_hole;
-        const int nx_w = (wb.lim_max + 31) / 32;  // sub-tiles this wavefront's rows can see (<= n_sub)
+        const int nx_all = (wb.lim_max + 31) / 32;  // sub-tiles this wavefront's rows can see (<= n_sub)
+        const int nx_w = (SPLIT && x_end < nx_all) ? x_end : nx_all;  // ... and the end of what it works on in this part
         // per-lane bounds relative to the lane's first key of a sub-tile (key = c0 + 4*lh + kk)
         const int lim_lane = lim - 4 * lh;
         const int hole_lo_lane = hole_lo - 4 * lh;
@@ -1107,8 +1204,8 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             mw1[i] = 0;
         }
         if constexpr (HAS_RAB) {
-            if (nx_w > 0) {
-                load_rab(0, rabw0);
+            if (nx_w > x_begin) {
+                load_rab(x_begin * 32, rabw0);
             }
 
         }
@@ -1130,8 +1227,8 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             const int c0 = t * 32;
 
             const bool do_qk = t + 1 < nx_w;
-            const bool do_silu = t >= 0 && t < nx_w;
-            const bool do_pv = t >= 1 && t <= nx_w;
+            const bool do_silu = t >= x_begin && t < nx_w;
+            const bool do_pv = t >= x_begin + 1 && t <= nx_w;
             const bool full = (c0 + 32 <= lim_min) && !(any_hole && c0 + 32 > hist_k && c0 < hole_hi_max);
 
             // (1) bias / mask requests for later steps; they go out before the tile requests of this step so
@@ -1142,7 +1239,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                 }
             }
             if constexpr (HAS_MASK) {
-                if (t + 1 >= 0 && t + 1 < nx_w) {
+                if (t + 1 < nx_w) {
                     load_bias(mask_rsrc, c0 + 32, mw_nxt);
                 }
             }
@@ -1360,34 +1457,111 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
 #ifdef HSTU_TIMELINE
-        if (a.timeline && lane == 0 && log_slot < 15) {
-            a.timeline[(static_cast<int64_t>(blockIdx.x) * 4 + wave) * 64 + 1 + 4 * log_slot + 2] = HSTU_CLOCK();
+        if (a.timeline && lane == 0 && log_slot < 12) {
+            a.timeline[(static_cast<int64_t>(blockIdx.x) * 4 + wave) * 64 + 1 + 5 * log_slot + 2] = HSTU_CLOCK();
         }
 #endif
-        if (n_sub > 0) {
-            int t = -1;
+        if (x_end > x_begin) {
+            int t = x_begin - 1;
             while (true) {
                 time_step(ic3_t{}, t);
-                if (++t > n_sub) {
+                if (++t > x_end) {
                     break;
                 }
                 time_step(ic0_t{}, t);
-                if (++t > n_sub) {
+                if (++t > x_end) {
                     break;
                 }
                 time_step(ic1_t{}, t);
-                if (++t > n_sub) {
+                if (++t > x_end) {
                     break;
                 }
                 time_step(ic2_t{}, t);
-                if (++t > n_sub) {
+                if (++t > x_end) {
                     break;
                 }
             }
         }
 
+#ifdef HSTU_TIMELINE
+        if (a.timeline && lane == 0 && log_slot < 12) {
+            a.timeline[(static_cast<int64_t>(blockIdx.x) * 4 + wave) * 64 + 1 + 5 * log_slot + 3] = HSTU_CLOCK();
+        }
+#endif
+        // ---- split item: hand in this part; the part that completes the item adds all of them up ----
+        bool store_rows = true;
+        if constexpr (SPLIT) {
+            if (n_parts > 1) {
+                // The partial outputs travel between workgroups on different XCDs, whose L2 caches do not see each
+                // other's lines: they are written and read with device-scope accesses (through to memory / from
+                // memory), which costs nothing to anybody else, instead of writing back and invalidating whole caches
+                // around the counter.  Order: stores complete (the wait the barrier brings) -> barrier -> count in.
+                constexpr int kDeviceScope = 1 | 16;  // cache policy bits sc0 | sc1 of gfx94x / gfx950 buffer accesses
+                constexpr int kQuads = MTILES * 4;                       // 16-byte pieces of a lane's accumulators
+                constexpr uint32_t kPartBytes = kBlockM * D * 4u;        // one partial output
+                const int ws_index = uniform(static_cast<int>(s_item[9]));
+                const __amdgpu_buffer_rsrc_t ws_rsrc =
+                    make_rsrc(reinterpret_cast<const uint8_t*>(a.ws) + static_cast<int64_t>(ws_index) * kPartBytes,
+                              static_cast<uint32_t>(n_parts) * kPartBytes);
+                // piece q of (wavefront, lane) sits at ((wave * kQuads + q) * 64 + lane) * 16 bytes: each store
+                // instruction writes 1 KiB in a row
+                const uint32_t lane_off = static_cast<uint32_t>(wave * kQuads * 64 + lane) * 16u;
+                typedef __attribute__((ext_vector_type(4))) float f32x4_t;
+#pragma unroll
+                for (int q = 0; q < kQuads; ++q) {
+                    // (the four floats are reinterpreted as one vector: element-wise reinterpretation into an integer
+                    // vector is narrowed to the first element by the optimiser of this toolchain)
+                    const f32x4_t v4 = {o_acc[q / 4][4 * (q % 4) + 0], o_acc[q / 4][4 * (q % 4) + 1],
+                                        o_acc[q / 4][4 * (q % 4) + 2], o_acc[q / 4][4 * (q % 4) + 3]};
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, v4), ws_rsrc,
+                                                           static_cast<int>(part * kPartBytes + lane_off + q * 1024u), 0,
+                                                           kDeviceScope);
+                }
+                __builtin_amdgcn_s_waitcnt(0);
+                __syncthreads();  // every wavefront's stores have completed
+                unsigned int* const arrived = &g_split_arrived[a.counter_slot][s_item[8]];
+                if (tid == 0) {
+                    s_item[10] = __hip_atomic_fetch_add(arrived, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+                __syncthreads();
+                store_rows = s_item[10] == static_cast<uint32_t>(n_parts - 1);
+                if (store_rows) {
+                    if (tid == 0) {
+                        __hip_atomic_store(arrived, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    }
+                    // the m partial outputs, added in part order whoever arrived last; the loads of one part
+                    // are all in flight together
+                    f32x4_t tot[kQuads];
+#pragma unroll
+                    for (int q = 0; q < kQuads; ++q) {
+                        tot[q] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+                    }
+                    for (int pp = 0; pp < n_parts; ++pp) {
+                        u32x4_t got[kQuads];
+#pragma unroll
+                        for (int q = 0; q < kQuads; ++q) {
+                            got[q] = __builtin_amdgcn_raw_buffer_load_b128(
+                                ws_rsrc, static_cast<int>(pp * kPartBytes + lane_off + q * 1024u), 0, kDeviceScope);
+                        }
+#pragma unroll
+                        for (int q = 0; q < kQuads; ++q) {
+                            tot[q] += __builtin_bit_cast(f32x4_t, got[q]);
+                        }
+                    }
+#pragma unroll
+                    for (int q = 0; q < kQuads; ++q) {
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            o_acc[q / 4][4 * (q % 4) + e] = tot[q][e];
+                        }
+                    }
+                }
+                __syncthreads();  // s_item[10] has been read before the next fetch writes the item
+            }
+        }
+
         // ---- store O: lane holds query row (wr0 + ln), dims 32*mt + 8*g + 4*lh + 0..3 ----
-        {
+        if (store_rows) {
             const uint32_t row_off = static_cast<uint32_t>(wr0 + ln) * o_stride;
 #pragma unroll
             for (int mt = 0; mt < MTILES; ++mt) {
@@ -1403,9 +1577,9 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             }
         }
 #ifdef HSTU_TIMELINE
-        if (a.timeline && lane == 0 && log_slot < 15) {
+        if (a.timeline && lane == 0 && log_slot < 12) {
             unsigned long long* row = a.timeline + (static_cast<int64_t>(blockIdx.x) * 4 + wave) * 64;
-            row[1 + 4 * log_slot + 3] = HSTU_CLOCK();
+            row[1 + 5 * log_slot + 4] = HSTU_CLOCK();
             row[0] = log_slot + 1;
         }
 #endif

@@ -7,6 +7,7 @@
 #include "../../include/hstu_mi355.h"
 
 #include <hip/hip_runtime.h>
+#include <stdlib.h>
 
 #include <atomic>
 #include <cmath>
@@ -30,12 +31,15 @@ int fail(int code, const char* fmt, ...)
     return code;
 }
 
-// kernel variants with the per-XCD work queues exist for the head-dim slots 64 and 128 (nullptr elsewhere)
+// kernel variants with the per-XCD work queues, and with split items, exist for the head-dim slots 64 and 128
+// (nullptr elsewhere)
 struct Variant {
     const char* name;
     const char* name_queues;
+    const char* name_split;
     void (*kernel)(const hstu::FwdArgs);
     void (*kernel_queues)(const hstu::FwdArgs);  // the same with per-XCD work queues, for long lists; may be nullptr
+    void (*kernel_split)(const hstu::FwdArgs);   // the same with long items split over workgroups, for short lists
     int d_pad;
     int threads;
     int persistent_wgs_per_cu;  // > 0: persistent kernel, this many workgroups per CU; 0: one workgroup per tile
@@ -77,11 +81,23 @@ constexpr auto queues_kernel() -> void (*)(const hstu::FwdArgs)
     }
 }
 
+template <typename Tag, typename OutTag, int D, bool RAB, bool MASK>
+constexpr auto split_kernel() -> void (*)(const hstu::FwdArgs)
+{
+    if constexpr (D == 64 || D == 128) {
+        return hstu::hstu_fwd_kernel<Tag, OutTag, D, RAB, MASK, false, true>;
+    } else {
+        return nullptr;
+    }
+}
+
 #define HSTU_VARIANT(tag, tagname, D, RAB, MASK, WGS)                                               \
     {"hstu_fwd_" tagname "_d" #D "_rab" #RAB "_mask" #MASK,                                        \
      "hstu_fwd_" tagname "_d" #D "_rab" #RAB "_mask" #MASK "_queues",                               \
+     "hstu_fwd_" tagname "_d" #D "_rab" #RAB "_mask" #MASK "_split",                                \
      hstu::hstu_fwd_kernel<hstu::tag, hstu::tag, D, RAB, MASK>,                                     \
-     queues_kernel<hstu::tag, hstu::tag, D, RAB, MASK>(), D, 256, WGS}
+     queues_kernel<hstu::tag, hstu::tag, D, RAB, MASK>(),                                           \
+     split_kernel<hstu::tag, hstu::tag, D, RAB, MASK>(), D, 256, WGS}
 #define HSTU_DIMS(tag, tagname, RAB, MASK)                                                           \
     {HSTU_VARIANT(tag, tagname, 32, RAB, MASK, 2), HSTU_VARIANT(tag, tagname, 64, RAB, MASK, 2), \
      HSTU_VARIANT(tag, tagname, 128, RAB, MASK, 2), HSTU_VARIANT(tag, tagname, 256, RAB, MASK, 1)}
@@ -95,7 +111,7 @@ const Variant kVariants[2][2][2][4] = {
 };
 
 #define HSTU_F32_VARIANT(D, RAB, MASK) \
-    {"hstu_fwd_f32_d" #D "_rab" #RAB "_mask" #MASK, nullptr, hstu::hstu_fwd_f32_kernel<D, RAB, MASK>, nullptr, D, 256, 0}
+    {"hstu_fwd_f32_d" #D "_rab" #RAB "_mask" #MASK, nullptr, nullptr, hstu::hstu_fwd_f32_kernel<D, RAB, MASK>, nullptr, nullptr, D, 256, 0}
 #define HSTU_F32_DIMS(RAB, MASK) \
     {HSTU_F32_VARIANT(32, RAB, MASK), HSTU_F32_VARIANT(64, RAB, MASK), HSTU_F32_VARIANT(128, RAB, MASK), \
      HSTU_F32_VARIANT(256, RAB, MASK)}
@@ -103,8 +119,10 @@ const Variant kVariants[2][2][2][4] = {
 // fp8-e4m3 inputs: [output: fp16, bf16][dim slot: 64, 128, 256] (no rab, no custom mask)
 #define HSTU_F8_VARIANT(otag, oname, D, WGS)                                                         \
     {"hstu_fwd_f8e4m3_" oname "_d" #D, "hstu_fwd_f8e4m3_" oname "_d" #D "_queues",                              \
+     "hstu_fwd_f8e4m3_" oname "_d" #D "_split",                                                                  \
      hstu::hstu_fwd_kernel<hstu::f8_tag, hstu::otag, D, false, false>,                                         \
-     queues_kernel<hstu::f8_tag, hstu::otag, D, false, false>(), D, 256, WGS}
+     queues_kernel<hstu::f8_tag, hstu::otag, D, false, false>(),                                               \
+     split_kernel<hstu::f8_tag, hstu::otag, D, false, false>(), D, 256, WGS}
 const Variant kVariantsF8[2][3] = {
     {HSTU_F8_VARIANT(f16_tag, "f16", 64, 2), HSTU_F8_VARIANT(f16_tag, "f16", 128, 2), HSTU_F8_VARIANT(f16_tag, "f16", 256, 1)},
     {HSTU_F8_VARIANT(bf16_tag, "bf16", 64, 2), HSTU_F8_VARIANT(bf16_tag, "bf16", 128, 2),
@@ -270,6 +288,44 @@ bool takes_queue_variant(const Variant* var, const hstu_jagged_fwd_params* p, in
     return var->kernel_queues != nullptr && n_blocks >= 4 * resident;
 }
 
+// Split items: a list that cannot have two items per resident workgroup takes the variant that may cut long items
+// into parts (it does so when there are fewer items than workgroups), if the caller brings a workspace.  The workspace holds the fp32 partial outputs, kBlockM x d_pad
+// floats each; room for two per resident workgroup is asked for (the kernel splits only as far as the room goes).
+constexpr uint64_t kMaxWorkspaceBytes = 128ull << 20;
+uint64_t split_part_bytes(const Variant* var) { return static_cast<uint64_t>(hstu::kBlockM) * var->d_pad * sizeof(float); }
+bool may_take_split_variant(const Variant* var, const hstu_jagged_fwd_params* p, int64_t* resident_out)
+{
+    if (var->persistent_wgs_per_cu <= 0 || var->kernel_split == nullptr) {
+        return false;
+    }
+    // HSTU_MI355_SPLIT=0 in the environment (read at every call) turns splitting off: the rows of a sequence then
+    // come out bit for bit the same whatever else is in the batch (a split changes the order of the fp32 sums)
+    const char* const env = getenv("HSTU_MI355_SPLIT");
+    if (env != nullptr && env[0] == '0') {
+        return false;
+    }
+    int cus = 0;
+    if (compute_units(&cus) != HSTU_OK) {
+        return false;
+    }
+    const int64_t resident = static_cast<int64_t>(cus) * var->persistent_wgs_per_cu;
+    if (resident_out != nullptr) {
+        *resident_out = resident;
+    }
+    const int64_t n_qtiles = (p->max_seq_len_q + hstu::kBlockM - 1) / hstu::kBlockM;
+    const int64_t n_blocks = n_qtiles * (p->n_offsets - 1) * p->num_heads_q;
+    return n_blocks < 2 * resident;
+}
+uint64_t split_workspace_bytes(const Variant* var, const hstu_jagged_fwd_params* p)
+{
+    int64_t resident = 0;
+    if (!may_take_split_variant(var, p, &resident)) {
+        return 0;
+    }
+    const uint64_t bytes = 2ull * static_cast<uint64_t>(resident) * split_part_bytes(var);
+    return bytes < kMaxWorkspaceBytes ? bytes : kMaxWorkspaceBytes;
+}
+
 }  // namespace
 
 extern "C" {
@@ -288,11 +344,14 @@ HSTU_API int hstu_jagged_fwd_workspace_size(const hstu_jagged_fwd_params* params
     if (rc != HSTU_OK) {
         return rc;
     }
-    if (select(params) == nullptr) {
+    const Variant* v = select(params);
+    if (v == nullptr) {
         return HSTU_ERR_UNSUPPORTED;
     }
-    // the tile schedule is derived inside the kernel from seq_offset, no scratch is needed
-    *workspace_bytes = 0;
+    // The tile schedule is derived inside the kernel from seq_offset.  Scratch is asked for only by short lists
+    // (room for the partial outputs of split items, see split_workspace_bytes); a caller that brings less, or
+    // none, is served without splitting.  Without a usable device the answer is 0.
+    *workspace_bytes = split_workspace_bytes(v, params);
     return HSTU_OK;
 }
 
@@ -306,13 +365,14 @@ HSTU_API const char* hstu_jagged_fwd_kernel_name(const hstu_jagged_fwd_params* p
         return nullptr;
     }
     // (without a usable device the plain name is reported)
-    return takes_queue_variant(v, params, nullptr) ? v->name_queues : v->name;
+    if (takes_queue_variant(v, params, nullptr)) {
+        return v->name_queues;
+    }
+    return may_take_split_variant(v, params, nullptr) ? v->name_split : v->name;  // (given the workspace asked for)
 }
 
 HSTU_API int hstu_jagged_fwd(const hstu_jagged_fwd_params* p, void* workspace, uint64_t workspace_bytes, void* stream)
 {
-    (void)workspace;
-    (void)workspace_bytes;
     const int rc = validate(p);
     if (rc != HSTU_OK) {
         return rc;
@@ -370,7 +430,10 @@ HSTU_API int hstu_jagged_fwd(const hstu_jagged_fwd_params* p, void* workspace, u
     a.v_descale = p->v_descale;
 
 #ifdef HSTU_TIMELINE
-    a.timeline = static_cast<unsigned long long*>(workspace);  // development builds only
+    // development builds only: the first MiB of the workspace receives the timeline
+    a.timeline = static_cast<unsigned long long*>(workspace);
+    workspace = static_cast<char*>(workspace) + (1 << 20);
+    workspace_bytes = workspace_bytes > (1u << 20) ? workspace_bytes - (1 << 20) : 0;
 #endif
     int64_t n_blocks = static_cast<int64_t>(a.n_qtiles) * a.bh;  // one per (query tile, sequence, head) slot
     if (n_blocks <= 0 || n_blocks > 0x7fffffffLL) {
@@ -389,6 +452,15 @@ HSTU_API int hstu_jagged_fwd(const hstu_jagged_fwd_params* p, void* workspace, u
             kernel = var->kernel_queues;
         }
         n_blocks = n_blocks < resident ? n_blocks : resident;
+        const uint64_t part_bytes = split_part_bytes(var);
+        if (workspace != nullptr && workspace_bytes >= 2 * part_bytes && reinterpret_cast<uintptr_t>(workspace) % 16 == 0 &&
+            may_take_split_variant(var, p, nullptr)) {
+            kernel = var->kernel_split;
+            a.ws = static_cast<float*>(workspace);
+            const uint64_t parts = workspace_bytes / part_bytes;
+            a.ws_parts = static_cast<uint32_t>(parts < 0x7fffffffull ? parts : 0x7fffffffull);
+            n_blocks = resident;  // the list may have more entries than items: all resident workgroups take part
+        }
         a.counter_slot = static_cast<int>(g_next_counter_slot.fetch_add(1) % hstu::kCounterSlots);
     }
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(n_blocks)), dim3(static_cast<unsigned>(var->threads)), 0,

@@ -131,7 +131,8 @@ def test_c5_full_size_properties(c5):
     assert (out.float().abs().amax(dim=(1, 2)) > 0).all()  # every row of every sequence was written
 
 
-def test_c5_sub_batch_matches_oracle(c5):
+def test_c5_sub_batch_matches_oracle(c5, monkeypatch):
+    monkeypatch.setenv("HSTU_MI355_SPLIT", "0")  # (bit-identity with the full batch needs the same order of fp32 sums)
     w, x8, sc, kw, out = c5
     order = sorted(range(len(w.lengths)), key=lambda b: w.lengths[b])
     seqs = sorted(order[:3] + [order[len(order) * 3 // 4]])  # three shortest and one of a few hundred rows

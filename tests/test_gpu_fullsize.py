@@ -53,8 +53,11 @@ def config(request):
     torch.cuda.empty_cache()
 
 
-def test_subbatch_matches_oracle(config):
+def test_subbatch_matches_oracle(config, monkeypatch):
     name, w, out = config
+    # the cut-out sequences make a list shorter than the machine; with splitting on, the fp32 sums of their long
+    # items would be taken in another order than in the full batch
+    monkeypatch.setenv("HSTU_MI355_SPLIT", "0")
     order = sorted(range(len(w.lengths)), key=lambda b: w.lengths[b])
     seqs = sorted(order[:2] + order[-1:]) if name == "C2" else sorted(order[:2])
     sub, rows = sub_batch(w, seqs)
