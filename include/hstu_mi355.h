@@ -131,6 +131,37 @@ HSTU_API int hstu_jagged_fwd_workspace_size(const hstu_jagged_fwd_params* params
  * NULL = the default stream) and returns without waiting for it. */
 HSTU_API int hstu_jagged_fwd(const hstu_jagged_fwd_params* params, void* workspace, uint64_t workspace_bytes, void* stream);
 
+/* ---- backward ------------------------------------------------------------------------------------------
+ * Replaces the two-phase pair the reference's adapter binds for the backward of this path:
+ *
+ *   aclnnHstuJaggedBackwardGetWorkspaceSize(grad, q, k, v, mask, attnBias, seqOffsetQ, seqOffsetK, numContext,
+ *        numTarget, layout, maskType, maxSeqLenQ, maxSeqLenK, siluScale, targetGroupSize, alpha,
+ *        qGrad, kGrad, vGrad, attnBiasGrad, &workspaceSize, &executor)
+ *   aclnnHstuJaggedBackward(workspace, workspaceSize, executor, stream)
+ *
+ *   documented at  ascendc/attention/hstu_v1/hstu_backward_v1/docs/aclnn_hstu_jagged_backward.md:24-56
+ *   C usage        ascendc/attention/hstu_v1/hstu_backward_v1/examples/aclnn/test_aclnn_hstu_backward_v1_jagged.cpp:174-186
+ *
+ * `fwd` describes q, k, v, mask, attn_bias, the offsets and the scalars exactly as for the forward (fwd.out is
+ * not used and may be NULL).  Built for bf16 / fp16 with head dims up to 128 (q/k head dim a multiple of 8);
+ * other valid descriptions return HSTU_ERR_UNSUPPORTED.
+ * grad_q / grad_k / grad_v: every row inside a sequence is written; rows past the last offset are not (clear
+ * them beforehand if they are read).  grad_attn_bias (optional; requires attn_bias): only the elements inside a
+ * sequence's [S_q, S_k] corner that a query tile sweeps are written -- the caller clears the tensor beforehand. */
+typedef struct hstu_jagged_bwd_params {
+    uint32_t struct_size; /* sizeof(hstu_jagged_bwd_params) */
+    uint32_t reserved0;
+    hstu_jagged_fwd_params fwd;
+    const void* grad;     /* [total_q, num_heads_q, head_dim_v], dtype of q */
+    void* grad_q;         /* [total_q, num_heads_q, head_dim_qk] */
+    void* grad_k;         /* [total_k, num_heads_k, head_dim_qk] */
+    void* grad_v;         /* [total_k, num_heads_k, head_dim_v] */
+    void* grad_attn_bias; /* NULL or [batch, num_heads_q, max_seq_len_q, max_seq_len_k] */
+} hstu_jagged_bwd_params;
+
+HSTU_API int hstu_jagged_bwd_workspace_size(const hstu_jagged_bwd_params* params, uint64_t* workspace_bytes);
+HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* params, void* workspace, uint64_t workspace_bytes, void* stream);
+
 /* replaces aclGetRecentErrMsg (ascendc/common/torch_plugin/pytorch_npu_helper.hpp:649,662):
  * text of the calling thread's most recent failure; never NULL. */
 HSTU_API const char* hstu_last_error(void);

@@ -1,0 +1,739 @@
+// HSTU jagged attention backward for gfx950 (MI355X): device code.
+//
+//   X = alpha (Q K^T + rab),  sig = sigmoid(X),  P = X sig scale M
+//   dV = P^T dO,   dP = dO V^T,   dS = alpha scale M dP sig (1 + X (1 - sig)),   d rab = dS,
+//   dQ = dS K,     dK = dS^T Q
+// (ascendc/attention/hstu_v1/hstu_backward_v1/op_kernel/vector_score.h:159-205; golden
+//  ascendc/attention/hstu_v2/test/pytest/backend/ascend_native_backend.py:86-150)
+//
+// Two kernels, no atomics, every output row written by exactly one wavefront (bitwise reproducible):
+//
+//   hstu_bwd_dkv_kernel  one workgroup per 128-key tile of one (sequence, K/V head): each wavefront keeps the K
+//                        and V rows of its 32 keys in registers (B operands) and sweeps the query rows that can
+//                        see them, 32 at a time, for every query head of the group.  Q and dO sub-tiles stream
+//                        through LDS.  Per sub-tile:
+//                            S  = Q . K^T          (A = Q  from LDS,            B = K registers)
+//                            dP = dO . V^T         (A = dO from LDS,            B = V registers)
+//                            dV^T += dO^T . P      (A = dO^T, transposed read,  B = P  from the accumulators)
+//                            dK^T += Q^T . dS      (A = Q^T,  transposed read,  B = dS from the accumulators)
+//   hstu_bwd_dq_kernel   one workgroup per 128-row query tile of one (sequence, head), the forward's shape: Q and
+//                        dO rows in registers, K and V sub-tiles stream through LDS.  Per sub-tile:
+//                            S^T  = K . Q^T,   dP^T = V . dO^T,   dQ^T += K^T . dS^T
+//                        and d rab = dS is stored from the accumulators when asked for.
+//
+// As in the forward, the score block is computed with the streamed operand as rows, so that its accumulator layout
+// (lane = resident row, registers = streamed rows) is the B-operand layout of the products that consume it: P and
+// dS never leave registers.  A sub-tile that is read both plainly and transposed is kept in LDS twice, once in
+// each bank-conflict-free layout.  Recomputing S and dP in both kernels costs 7 products instead of 5 and buys
+// freedom from atomics and from a dQ workspace.
+#pragma once
+#include "hstu_fwd_kernel.hip.h"
+
+namespace hstu {
+
+struct BwdArgs {
+    const void* q;
+    const void* k;
+    const void* v;
+    const void* grad;  // dO
+    const void* rab;
+    const void* mask;
+    void* dq;
+    void* dk;
+    void* dv;
+    void* drab;  // may be null
+    const void* offs_q;
+    const void* offs_k;
+    const void* num_ctx;
+    const void* num_tgt;
+    int64_t total_q;
+    int64_t total_k;
+    int n_batch;
+    int n_heads_q;
+    int n_heads_k;
+    int head_ratio;
+    int d_qk;
+    int d_v;
+    int max_q;
+    int max_k;
+    int mask_type;
+    int target_group;
+    int idx64;
+    int n_qtiles;     // ceil(max_q / 128)
+    int n_ktiles;     // ceil(max_k / 128)
+    int bias_vec_ok;  // rab / mask / d rab rows may be accessed 4 elements (8 bytes) at a time
+    float alpha;
+    float scale;  // silu_scale, resolved
+};
+
+struct SeqInfo {
+    int64_t q0;
+    int64_t k0;
+    int sq;
+    int sk;
+    int n_ctx;
+    int n_tgt;
+    int delta;
+    int hist_k;
+};
+
+__device__ __forceinline__ SeqInfo load_seq(const BwdArgs& a, int b)
+{
+    SeqInfo s;
+    int64_t q0 = load_index_uniform(a.offs_q, b, a.idx64);
+    int64_t q1 = load_index_uniform(a.offs_q, b + 1, a.idx64);
+    int64_t k0 = load_index_uniform(a.offs_k, b, a.idx64);
+    int64_t k1 = load_index_uniform(a.offs_k, b + 1, a.idx64);
+    q1 = q1 < a.total_q ? q1 : a.total_q;
+    k1 = k1 < a.total_k ? k1 : a.total_k;
+    q0 = q0 < 0 ? 0 : q0;
+    k0 = k0 < 0 ? 0 : k0;
+    int sq = static_cast<int>(q1 > q0 ? q1 - q0 : 0);
+    int sk = static_cast<int>(k1 > k0 ? k1 - k0 : 0);
+    s.sq = sq < a.max_q ? sq : a.max_q;
+    s.sk = sk < a.max_k ? sk : a.max_k;
+    s.q0 = q0;
+    s.k0 = k0;
+    s.n_ctx = 0;
+    s.n_tgt = 0;
+    if (a.mask_type == 0) {
+        if (a.num_ctx) {
+            s.n_ctx = static_cast<int>(load_index_uniform(a.num_ctx, b, a.idx64));
+        }
+        if (a.num_tgt) {
+            s.n_tgt = static_cast<int>(load_index_uniform(a.num_tgt, b, a.idx64));
+        }
+        s.n_ctx = s.n_ctx < 0 ? 0 : s.n_ctx;
+        s.n_tgt = s.n_tgt < 0 ? 0 : (s.n_tgt > s.sk ? s.sk : s.n_tgt);
+    }
+    s.delta = s.sk - s.sq;
+    s.hist_k = s.sk - s.n_tgt;
+    return s;
+}
+
+// first key hidden from query row r by the causal / context rule, and the hole the grouped targets cut out
+__device__ __forceinline__ void row_bounds(const SeqInfo& s, int mask_type, int group, int r, int& lim, int& hole_lo,
+                                           int& hole_hi)
+{
+    hole_lo = 0;
+    hole_hi = 0;
+    if (mask_type != 0) {
+        lim = s.sk;
+        return;
+    }
+    lim = r + s.delta + 1;
+    if (r < s.n_ctx) {
+        lim = lim > s.hist_k ? lim : s.hist_k;
+    }
+    lim = lim < 0 ? 0 : (lim > s.sk ? s.sk : lim);
+    if (s.n_tgt > 0 && group > 0) {
+        const int ti = r - (s.sq - s.n_tgt);
+        if (ti >= 0) {
+            hole_lo = s.hist_k;
+            hole_hi = s.hist_k + (ti / group) * group;
+        }
+    }
+}
+
+// P (without mask) and dS (without mask) of one score element
+__device__ __forceinline__ void score_grad(float s, float dp, float alpha, float c_exp, float scale, float ascale,
+                                           float& p, float& ds)
+{
+    const float x = s * alpha;
+    const float e = __builtin_amdgcn_exp2f(s * c_exp);
+    const float sig = __builtin_amdgcn_rcpf(1.0f + e);
+    const float xs = x * sig;
+    p = xs * scale;
+    ds = ascale * dp * (sig + xs * (1.0f - sig));
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// shared pieces of the two kernels: the two LDS layouts of a 32-row sub-tile and their read patterns
+// ---------------------------------------------------------------------------------------------------------
+template <int D>
+struct SubTile {
+    static constexpr int CPR = D / 8;                 // 16-byte chunks per row
+    static constexpr int ELEMS = 32 * D;              // 16-bit elements
+    static constexpr int KIB = 32 * D * 2 / 1024;     // 1 KiB load instructions per sub-tile
+    static constexpr int LPW = KIB >= 4 ? KIB / 4 : 1;  // ... per loading wavefront
+    static constexpr int NLW = KIB >= 4 ? 4 : KIB;      // wavefronts that take part
+    static constexpr int KSTEPS = D / 16;
+    static constexpr int MTILES = D / 32;
+};
+
+// ---------------------------------------------------------------------------------------------------------
+// dQ (and d rab)
+// ---------------------------------------------------------------------------------------------------------
+template <typename Tag, int D, bool HAS_RAB, bool HAS_MASK, bool WANT_DRAB>
+__global__ __launch_bounds__(256, 2) void hstu_bwd_dq_kernel(const BwdArgs a)
+{
+    typedef SubTile<D> T;
+    constexpr int LPW = T::LPW, NLW = T::NLW, KSTEPS = T::KSTEPS, MTILES = T::MTILES, NCH = 2 * T::MTILES;
+    __shared__ __attribute__((aligned(1024))) uint16_t s_kn0[T::ELEMS];  // K, layout for plain reads
+    __shared__ __attribute__((aligned(1024))) uint16_t s_kn1[T::ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_kt0[T::ELEMS];  // K, layout for transposed reads
+    __shared__ __attribute__((aligned(1024))) uint16_t s_kt1[T::ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_vn0[T::ELEMS];  // V, layout for plain reads
+    __shared__ __attribute__((aligned(1024))) uint16_t s_vn1[T::ELEMS];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = uniform(tid >> 6);
+    const int ln = lane & 31;
+    const int lh = lane >> 5;
+
+    // heaviest (last) query tiles first
+    const int per_level = a.n_batch * a.n_heads_q;
+    const int lvl = static_cast<int>(blockIdx.x) / per_level;
+    const int rem = static_cast<int>(blockIdx.x) - lvl * per_level;
+    const int qt = a.n_qtiles - 1 - lvl;
+    const int b = rem / a.n_heads_q;
+    const int h = rem - b * a.n_heads_q;
+    const int hk = h / a.head_ratio;
+    const SeqInfo sq_info = load_seq(a, b);
+    const int sq = sq_info.sq, sk = sq_info.sk;
+    const int r0 = qt * kBlockM;
+    if (r0 >= sq) {
+        return;
+    }
+    const int wr0 = r0 + wave * kWaveM;
+
+    const uint32_t q_stride = static_cast<uint32_t>(a.n_heads_q) * a.d_qk * 2u;
+    const uint32_t g_stride = static_cast<uint32_t>(a.n_heads_q) * a.d_v * 2u;
+    const uint32_t k_stride = static_cast<uint32_t>(a.n_heads_k) * a.d_qk * 2u;
+    const uint32_t v_stride = static_cast<uint32_t>(a.n_heads_k) * a.d_v * 2u;
+    const __amdgpu_buffer_rsrc_t q_rsrc =
+        make_rsrc(static_cast<const uint8_t*>(a.q) + (sq_info.q0 * a.n_heads_q + h) * static_cast<int64_t>(a.d_qk) * 2,
+                  static_cast<uint32_t>(sq - 1) * q_stride + a.d_qk * 2u);
+    const __amdgpu_buffer_rsrc_t g_rsrc =
+        make_rsrc(static_cast<const uint8_t*>(a.grad) + (sq_info.q0 * a.n_heads_q + h) * static_cast<int64_t>(a.d_v) * 2,
+                  static_cast<uint32_t>(sq - 1) * g_stride + a.d_v * 2u);
+    const __amdgpu_buffer_rsrc_t dq_rsrc =
+        make_rsrc(static_cast<uint8_t*>(a.dq) + (sq_info.q0 * a.n_heads_q + h) * static_cast<int64_t>(a.d_qk) * 2,
+                  static_cast<uint32_t>(sq - 1) * q_stride + a.d_qk * 2u);
+    const __amdgpu_buffer_rsrc_t k_rsrc =
+        make_rsrc(static_cast<const uint8_t*>(a.k) + (sq_info.k0 * a.n_heads_k + hk) * static_cast<int64_t>(a.d_qk) * 2,
+                  sk > 0 ? static_cast<uint32_t>(sk - 1) * k_stride + a.d_qk * 2u : 0u);
+    const __amdgpu_buffer_rsrc_t v_rsrc =
+        make_rsrc(static_cast<const uint8_t*>(a.v) + (sq_info.k0 * a.n_heads_k + hk) * static_cast<int64_t>(a.d_v) * 2,
+                  sk > 0 ? static_cast<uint32_t>(sk - 1) * v_stride + a.d_v * 2u : 0u);
+
+    // per-lane source offsets of the sub-tile loads (see the forward kernel: 16-byte slot -> row, swizzled chunk)
+    uint32_t kn_src[LPW], kt_src[LPW], vn_src[LPW];
+#pragma unroll
+    for (int i = 0; i < LPW; ++i) {
+        const int slot = (wave * LPW + i) * 64 + lane;
+        const int r = (slot / T::CPR) & 31;
+        const int pc = slot % T::CPR;
+        const int cn = k_chunk_swizzle<D>(r, pc);
+        const int ct = v_chunk_swizzle<D>(r, pc);
+        kn_src[i] = (cn * 8 < a.d_qk) ? static_cast<uint32_t>(r) * k_stride + cn * 16u : kOutOfRange;
+        kt_src[i] = (ct * 8 < a.d_qk) ? static_cast<uint32_t>(r) * k_stride + ct * 16u : kOutOfRange;
+        vn_src[i] = (cn * 8 < a.d_v) ? static_cast<uint32_t>(r) * v_stride + cn * 16u : kOutOfRange;
+    }
+    int n_lane_off[KSTEPS];  // plain read of row ln, MFMA step js
+    int t_lane_off[MTILES];  // transposed read, output tile mt
+#pragma unroll
+    for (int js = 0; js < KSTEPS; ++js) {
+        n_lane_off[js] = ln * D + k_chunk_swizzle<D>(ln, 2 * js + lh) * 8;
+    }
+    {
+        const int vr0 = 4 * lh + ((lane & 15) >> 2);
+#pragma unroll
+        for (int mt = 0; mt < MTILES; ++mt) {
+            const int col = 32 * mt + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+            t_lane_off[mt] = vr0 * D + v_chunk_swizzle<D>(vr0, col >> 3) * 8 + (col & 7);
+        }
+    }
+
+    // keys needed by this tile (as in the forward)
+    int kmax;
+    if (a.mask_type == 0) {
+        const int r1 = (r0 + kBlockM < sq) ? r0 + kBlockM : sq;
+        kmax = r1 + sq_info.delta;
+        if (r0 < sq_info.n_ctx) {
+            kmax = kmax > sq_info.hist_k ? kmax : sq_info.hist_k;
+        }
+        kmax = kmax < 0 ? 0 : (kmax > sk ? sk : kmax);
+    } else {
+        kmax = sk;
+    }
+    const int n_sub = (kmax + 31) / 32;
+
+    // resident rows: Q and dO fragments (B operands: lane = row, 8 dims per MFMA step)
+    u32x4_t qf[KSTEPS], gf[KSTEPS];
+    {
+        const uint32_t q_off = static_cast<uint32_t>(wr0 + ln) * q_stride;
+        const uint32_t g_off = static_cast<uint32_t>(wr0 + ln) * g_stride;
+#pragma unroll
+        for (int js = 0; js < KSTEPS; ++js) {
+            const int d0 = 16 * js + 8 * lh;
+            qf[js] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, static_cast<int>(d0 < a.d_qk ? q_off + d0 * 2u : kOutOfRange), 0, 0);
+            gf[js] = __builtin_amdgcn_raw_buffer_load_b128(g_rsrc, static_cast<int>(d0 < a.d_v ? g_off + d0 * 2u : kOutOfRange), 0, 0);
+        }
+    }
+    int row = wr0 + ln;
+    row = row < sq - 1 ? row : sq - 1;
+    int lim, hole_lo, hole_hi;
+    row_bounds(sq_info, a.mask_type, a.target_group, row, lim, hole_lo, hole_hi);
+    const WaveBounds wb = wave_bounds(a.mask_type, wr0, sq, sk, sq_info.n_ctx, sq_info.n_tgt, a.target_group, wr0 < sq);
+    const int nx_w = (wb.lim_max + 31) / 32;
+
+    const uint32_t bias_bytes = static_cast<uint32_t>(a.max_q) * static_cast<uint32_t>(a.max_k) * 2u;
+    const int64_t bias_plane = (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k);
+    const __amdgpu_buffer_rsrc_t rab_rsrc =
+        make_rsrc(HAS_RAB ? static_cast<const uint16_t*>(a.rab) + bias_plane : nullptr, HAS_RAB ? bias_bytes : 0u);
+    const __amdgpu_buffer_rsrc_t mask_rsrc =
+        make_rsrc(HAS_MASK ? static_cast<const uint16_t*>(a.mask) + bias_plane : nullptr, HAS_MASK ? bias_bytes : 0u);
+    const __amdgpu_buffer_rsrc_t drab_rsrc =
+        make_rsrc(WANT_DRAB ? static_cast<uint16_t*>(a.drab) + bias_plane : nullptr, WANT_DRAB ? bias_bytes : 0u);
+    // rows past the sequence lie inside the plane but must stay untouched / unread: their offset leaves it
+    const uint32_t bias_row_off =
+        (wr0 + ln < sq) ? static_cast<uint32_t>(wr0 + ln) * static_cast<uint32_t>(a.max_k) * 2u : kOutOfRange;
+    const bool vec = a.bias_vec_ok != 0;
+
+    // words 2g, 2g+1 = the row's values at keys c0 + 8g + 4 lh + 0..3 (accumulator order)
+    auto load_words = [&](__amdgpu_buffer_rsrc_t rsrc, int c0, uint32_t (&w)[8]) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int key = c0 + 8 * g + 4 * lh;
+            const uint32_t off = bias_row_off + static_cast<uint32_t>(key) * 2u;
+            if (vec) {
+                const U32Pair t = __builtin_bit_cast(
+                    U32Pair, __builtin_amdgcn_raw_buffer_load_b64(rsrc, static_cast<int>(key < a.max_k ? off : kOutOfRange), 0, 0));
+                w[2 * g + 0] = t.v[0];
+                w[2 * g + 1] = t.v[1];
+            } else {
+                uint32_t e[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    uint32_t eoff = (key + i < a.max_k) ? off + 2u * i : kOutOfRange;
+                    asm volatile("" : "+v"(eoff));
+                    e[i] = __builtin_amdgcn_raw_buffer_load_b16(rsrc, static_cast<int>(eoff), 0, 0);
+                }
+                w[2 * g + 0] = (e[0] & 0xffffu) | (e[1] << 16);
+                w[2 * g + 1] = (e[2] & 0xffffu) | (e[3] << 16);
+            }
+        }
+    };
+
+    f32x16_t dq_acc[MTILES];
+#pragma unroll
+    for (int mt = 0; mt < MTILES; ++mt) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            dq_acc[mt][i] = 0.f;
+        }
+    }
+    const float c_exp = -a.alpha * 1.4426950408889634f;
+    const float ascale = a.alpha * a.scale;
+
+    auto request = [&](uint16_t* kn, uint16_t* kt, uint16_t* vn, int x) {
+        if (NLW == 4 || wave < NLW) {
+            const uint32_t kb = static_cast<uint32_t>(x * 32) * k_stride;
+            const uint32_t vb = static_cast<uint32_t>(x * 32) * v_stride;
+#pragma unroll
+            for (int i = 0; i < LPW; ++i) {
+                load_to_lds_b128(k_rsrc, kn + (wave * LPW + i) * 512, kn_src[i] + kb);
+                load_to_lds_b128(k_rsrc, kt + (wave * LPW + i) * 512, kt_src[i] + kb);
+                load_to_lds_b128(v_rsrc, vn + (wave * LPW + i) * 512, vn_src[i] + vb);
+            }
+        }
+    };
+    auto read_n = [&](const uint16_t* tile, int js) -> u32x4_t {
+        return *reinterpret_cast<const u32x4_t*>(tile + n_lane_off[js]);
+    };
+    auto read_t = [&](const uint16_t* tile, int c) -> u32x4_t {
+        const int j2 = c / MTILES, mt = c % MTILES;
+        const uint16_t* p = tile + t_lane_off[mt] + 16 * j2 * D;
+        const u32x2_t lo = lds_read_tr16_b64(p);
+        const u32x2_t hi = lds_read_tr16_b64(p + 8 * D);
+        const u32x4_t r = {lo[0], lo[1], hi[0], hi[1]};
+        return r;
+    };
+
+    auto step = [&](const uint16_t* kn, const uint16_t* kt, const uint16_t* vn, uint16_t* kn_o, uint16_t* kt_o,
+                    uint16_t* vn_o, int x) {
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();  // sub-tile x has landed for everybody, and nobody reads the other buffer any more
+        if (x + 1 < n_sub) {
+            request(kn_o, kt_o, vn_o, x + 1);
+        }
+        if (x >= nx_w) {
+            return;  // nothing of this sub-tile is visible to the rows of this wavefront
+        }
+        const int c0 = x * 32;
+        uint32_t rw[8], mw[8];
+        if constexpr (HAS_RAB) {
+            load_words(rab_rsrc, c0, rw);
+        }
+        if constexpr (HAS_MASK) {
+            load_words(mask_rsrc, c0, mw);
+        }
+        f32x16_t s, dp;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            s[i] = 0.f;
+            dp[i] = 0.f;
+        }
+#pragma unroll
+        for (int js = 0; js < KSTEPS; ++js) {
+            s = mfma32<Tag>(read_n(kn, js), qf[js], s);
+            dp = mfma32<Tag>(read_n(vn, js), gf[js], dp);
+        }
+        uint32_t pk[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float ds2[2];
+#pragma unroll
+            for (int e2 = 0; e2 < 2; ++e2) {
+                const int e = 2 * i + e2;
+                float sv = s[e];
+                if constexpr (HAS_RAB) {
+                    sv += e2 ? hi_to_float<Tag>(rw[i]) : lo_to_float<Tag>(rw[i]);
+                }
+                float p, ds;
+                score_grad(sv, dp[e], a.alpha, c_exp, a.scale, ascale, p, ds);
+                if constexpr (HAS_MASK) {
+                    ds *= e2 ? hi_to_float<Tag>(mw[i]) : lo_to_float<Tag>(mw[i]);
+                }
+                const int key = c0 + 8 * (e / 4) + 4 * lh + (e % 4);
+                const bool vis = (key < lim) && !(key >= hole_lo && key < hole_hi);
+                ds2[e2] = vis ? ds : 0.f;
+            }
+            pk[i] = pack2<Tag>(ds2[0], ds2[1]);
+        }
+        if constexpr (WANT_DRAB) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int key = c0 + 8 * g + 4 * lh;
+                const uint32_t off = bias_row_off + static_cast<uint32_t>(key) * 2u;
+                if (vec) {
+                    const u32x2_t w2 = {pk[2 * g], pk[2 * g + 1]};
+                    __builtin_amdgcn_raw_buffer_store_b64(w2, drab_rsrc, static_cast<int>(key < sk ? off : kOutOfRange), 0, 0);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const uint32_t word = pk[2 * g + i / 2];
+                        const uint16_t val = static_cast<uint16_t>((i & 1) ? (word >> 16) : (word & 0xffffu));
+                        __builtin_amdgcn_raw_buffer_store_b16(val, drab_rsrc,
+                                                              static_cast<int>(key + i < sk ? off + 2u * i : kOutOfRange), 0, 0);
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            const int j2 = c / MTILES, mt = c % MTILES;
+            const u32x4_t pb = {pk[4 * j2 + 0], pk[4 * j2 + 1], pk[4 * j2 + 2], pk[4 * j2 + 3]};
+            dq_acc[mt] = mfma32<Tag>(read_t(kt, c), pb, dq_acc[mt]);
+        }
+    };
+
+    if (n_sub > 0) {
+        request(s_kn0, s_kt0, s_vn0, 0);
+    }
+    for (int x = 0; x < n_sub; x += 2) {
+        step(s_kn0, s_kt0, s_vn0, s_kn1, s_kt1, s_vn1, x);
+        if (x + 1 < n_sub) {
+            step(s_kn1, s_kt1, s_vn1, s_kn0, s_kt0, s_vn0, x + 1);
+        }
+    }
+
+    // store dQ: lane holds query row (wr0 + ln), dims 32*mt + 8*g + 4*lh + 0..3
+    {
+        const uint32_t row_off = static_cast<uint32_t>(wr0 + ln) * q_stride;
+#pragma unroll
+        for (int mt = 0; mt < MTILES; ++mt) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int d0 = 32 * mt + 8 * g + 4 * lh;
+                const uint32_t off = (d0 < a.d_qk) ? row_off + d0 * 2u : kOutOfRange;
+                u32x2_t w;
+                w[0] = pack2<Tag>(dq_acc[mt][4 * g + 0], dq_acc[mt][4 * g + 1]);
+                w[1] = pack2<Tag>(dq_acc[mt][4 * g + 2], dq_acc[mt][4 * g + 3]);
+                __builtin_amdgcn_raw_buffer_store_b64(w, dq_rsrc, static_cast<int>(off), 0, 0);
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// dK, dV
+// ---------------------------------------------------------------------------------------------------------
+template <typename Tag, int D, bool HAS_RAB, bool HAS_MASK>
+__global__ __launch_bounds__(256, 1) void hstu_bwd_dkv_kernel(const BwdArgs a)
+{
+    typedef SubTile<D> T;
+    constexpr int LPW = T::LPW, NLW = T::NLW, KSTEPS = T::KSTEPS, MTILES = T::MTILES, NCH = 2 * T::MTILES;
+    __shared__ __attribute__((aligned(1024))) uint16_t s_qn0[T::ELEMS];  // Q, plain / transposed layouts
+    __shared__ __attribute__((aligned(1024))) uint16_t s_qn1[T::ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_qt0[T::ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_qt1[T::ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_gn0[T::ELEMS];  // dO, plain / transposed layouts
+    __shared__ __attribute__((aligned(1024))) uint16_t s_gn1[T::ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_gt0[T::ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_gt1[T::ELEMS];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = uniform(tid >> 6);
+    const int ln = lane & 31;
+    const int lh = lane >> 5;
+
+    // key tile 0 is seen by the most query rows: heaviest first
+    const int per_level = a.n_batch * a.n_heads_k;
+    const int kt_idx = static_cast<int>(blockIdx.x) / per_level;
+    const int rem = static_cast<int>(blockIdx.x) - kt_idx * per_level;
+    const int b = rem / a.n_heads_k;
+    const int hk = rem - b * a.n_heads_k;
+    const SeqInfo si = load_seq(a, b);
+    const int sq = si.sq, sk = si.sk;
+    const int c0 = kt_idx * kBlockM;
+    if (c0 >= sk) {
+        return;
+    }
+    const int cw0 = c0 + wave * 32;  // first key of this wavefront
+    const int key = cw0 + ln;        // this lane's key
+
+    const uint32_t q_stride = static_cast<uint32_t>(a.n_heads_q) * a.d_qk * 2u;
+    const uint32_t g_stride = static_cast<uint32_t>(a.n_heads_q) * a.d_v * 2u;
+    const uint32_t k_stride = static_cast<uint32_t>(a.n_heads_k) * a.d_qk * 2u;
+    const uint32_t v_stride = static_cast<uint32_t>(a.n_heads_k) * a.d_v * 2u;
+    const __amdgpu_buffer_rsrc_t k_rsrc =
+        make_rsrc(static_cast<const uint8_t*>(a.k) + (si.k0 * a.n_heads_k + hk) * static_cast<int64_t>(a.d_qk) * 2,
+                  static_cast<uint32_t>(sk - 1) * k_stride + a.d_qk * 2u);
+    const __amdgpu_buffer_rsrc_t v_rsrc =
+        make_rsrc(static_cast<const uint8_t*>(a.v) + (si.k0 * a.n_heads_k + hk) * static_cast<int64_t>(a.d_v) * 2,
+                  static_cast<uint32_t>(sk - 1) * v_stride + a.d_v * 2u);
+    const __amdgpu_buffer_rsrc_t dk_rsrc =
+        make_rsrc(static_cast<uint8_t*>(a.dk) + (si.k0 * a.n_heads_k + hk) * static_cast<int64_t>(a.d_qk) * 2,
+                  static_cast<uint32_t>(sk - 1) * k_stride + a.d_qk * 2u);
+    const __amdgpu_buffer_rsrc_t dv_rsrc =
+        make_rsrc(static_cast<uint8_t*>(a.dv) + (si.k0 * a.n_heads_k + hk) * static_cast<int64_t>(a.d_v) * 2,
+                  static_cast<uint32_t>(sk - 1) * v_stride + a.d_v * 2u);
+
+    uint32_t qn_src[LPW], qt_src[LPW], gn_src[LPW], gt_src[LPW];
+#pragma unroll
+    for (int i = 0; i < LPW; ++i) {
+        const int slot = (wave * LPW + i) * 64 + lane;
+        const int r = (slot / T::CPR) & 31;
+        const int pc = slot % T::CPR;
+        const int cn = k_chunk_swizzle<D>(r, pc);
+        const int ct = v_chunk_swizzle<D>(r, pc);
+        qn_src[i] = (cn * 8 < a.d_qk) ? static_cast<uint32_t>(r) * q_stride + cn * 16u : kOutOfRange;
+        qt_src[i] = (ct * 8 < a.d_qk) ? static_cast<uint32_t>(r) * q_stride + ct * 16u : kOutOfRange;
+        gn_src[i] = (cn * 8 < a.d_v) ? static_cast<uint32_t>(r) * g_stride + cn * 16u : kOutOfRange;
+        gt_src[i] = (ct * 8 < a.d_v) ? static_cast<uint32_t>(r) * g_stride + ct * 16u : kOutOfRange;
+    }
+    int n_lane_off[KSTEPS];
+    int t_lane_off[MTILES];
+#pragma unroll
+    for (int js = 0; js < KSTEPS; ++js) {
+        n_lane_off[js] = ln * D + k_chunk_swizzle<D>(ln, 2 * js + lh) * 8;
+    }
+    {
+        const int vr0 = 4 * lh + ((lane & 15) >> 2);
+#pragma unroll
+        for (int mt = 0; mt < MTILES; ++mt) {
+            const int col = 32 * mt + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+            t_lane_off[mt] = vr0 * D + v_chunk_swizzle<D>(vr0, col >> 3) * 8 + (col & 7);
+        }
+    }
+
+    // resident rows: K and V fragments of this lane's key
+    u32x4_t kf[KSTEPS], vf[KSTEPS];
+    {
+        const uint32_t k_off = static_cast<uint32_t>(key) * k_stride;
+        const uint32_t v_off = static_cast<uint32_t>(key) * v_stride;
+#pragma unroll
+        for (int js = 0; js < KSTEPS; ++js) {
+            const int d0 = 16 * js + 8 * lh;
+            kf[js] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, static_cast<int>(d0 < a.d_qk ? k_off + d0 * 2u : kOutOfRange), 0, 0);
+            vf[js] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, static_cast<int>(d0 < a.d_v ? v_off + d0 * 2u : kOutOfRange), 0, 0);
+        }
+    }
+
+    // query sub-tiles that can see a key of this tile
+    const int n_qsub = (sq + 31) / 32;
+    int x_first = 0;
+    if (a.mask_type == 0 && !(si.n_ctx > 0 && c0 < si.hist_k)) {
+        const int first_row = c0 - si.delta;  // the first row that sees key c0
+        x_first = first_row > 0 ? first_row / 32 : 0;
+    }
+    const int nx = n_qsub > x_first ? n_qsub - x_first : 0;
+    const int n_iter = nx * a.head_ratio;  // (query head of the group, query sub-tile), head-major
+
+    f32x16_t dk_acc[MTILES], dv_acc[MTILES];
+#pragma unroll
+    for (int mt = 0; mt < MTILES; ++mt) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            dk_acc[mt][i] = 0.f;
+            dv_acc[mt][i] = 0.f;
+        }
+    }
+    const float c_exp = -a.alpha * 1.4426950408889634f;
+    const float ascale = a.alpha * a.scale;
+    const uint32_t bias_bytes = static_cast<uint32_t>(a.max_q) * static_cast<uint32_t>(a.max_k) * 2u;
+    const bool targets = a.mask_type == 0 && si.n_tgt > 0 && a.target_group > 0;
+
+    auto head_of = [&](int it) -> int { return hk * a.head_ratio + it / nx; };
+    auto sub_of = [&](int it) -> int { return x_first + it % nx; };
+    auto request = [&](uint16_t* qn, uint16_t* qt, uint16_t* gn, uint16_t* gt, int it) {
+        if (NLW == 4 || wave < NLW) {
+            const int h = head_of(it);
+            const int x = sub_of(it);
+            const __amdgpu_buffer_rsrc_t q_rsrc =
+                make_rsrc(static_cast<const uint8_t*>(a.q) + (si.q0 * a.n_heads_q + h) * static_cast<int64_t>(a.d_qk) * 2,
+                          static_cast<uint32_t>(sq - 1) * q_stride + a.d_qk * 2u);
+            const __amdgpu_buffer_rsrc_t g_rsrc =
+                make_rsrc(static_cast<const uint8_t*>(a.grad) + (si.q0 * a.n_heads_q + h) * static_cast<int64_t>(a.d_v) * 2,
+                          static_cast<uint32_t>(sq - 1) * g_stride + a.d_v * 2u);
+            const uint32_t qb = static_cast<uint32_t>(x * 32) * q_stride;
+            const uint32_t gb = static_cast<uint32_t>(x * 32) * g_stride;
+#pragma unroll
+            for (int i = 0; i < LPW; ++i) {
+                load_to_lds_b128(q_rsrc, qn + (wave * LPW + i) * 512, qn_src[i] + qb);
+                load_to_lds_b128(q_rsrc, qt + (wave * LPW + i) * 512, qt_src[i] + qb);
+                load_to_lds_b128(g_rsrc, gn + (wave * LPW + i) * 512, gn_src[i] + gb);
+                load_to_lds_b128(g_rsrc, gt + (wave * LPW + i) * 512, gt_src[i] + gb);
+            }
+        }
+    };
+    auto read_n = [&](const uint16_t* tile, int js) -> u32x4_t {
+        return *reinterpret_cast<const u32x4_t*>(tile + n_lane_off[js]);
+    };
+    auto read_t = [&](const uint16_t* tile, int c) -> u32x4_t {
+        const int j2 = c / MTILES, mt = c % MTILES;
+        const uint16_t* p = tile + t_lane_off[mt] + 16 * j2 * D;
+        const u32x2_t lo = lds_read_tr16_b64(p);
+        const u32x2_t hi = lds_read_tr16_b64(p + 8 * D);
+        const u32x4_t r = {lo[0], lo[1], hi[0], hi[1]};
+        return r;
+    };
+
+    auto step = [&](const uint16_t* qn, const uint16_t* qt, const uint16_t* gn, const uint16_t* gt, uint16_t* qn_o,
+                    uint16_t* qt_o, uint16_t* gn_o, uint16_t* gt_o, int it) {
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        if (it + 1 < n_iter) {
+            request(qn_o, qt_o, gn_o, gt_o, it + 1);
+        }
+        const int h = head_of(it);
+        const int x = sub_of(it);
+        const int rq0 = x * 32;  // first query row of the sub-tile
+        // whole block hidden from the keys of this wavefront?  (rows rq0 .. rq0 + 31, keys cw0 .. cw0 + 31)
+        if (a.mask_type == 0) {
+            int lim_max = rq0 + 32 + si.delta;  // lim of the last row
+            if (rq0 < si.n_ctx) {
+                lim_max = lim_max > si.hist_k ? lim_max : si.hist_k;
+            }
+            if (cw0 >= lim_max) {
+                return;
+            }
+        }
+        if (cw0 >= sk) {
+            return;
+        }
+        f32x16_t s, dp;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            s[i] = 0.f;
+            dp[i] = 0.f;
+        }
+#pragma unroll
+        for (int js = 0; js < KSTEPS; ++js) {
+            s = mfma32<Tag>(read_n(qn, js), kf[js], s);
+            dp = mfma32<Tag>(read_n(gn, js), vf[js], dp);
+        }
+        // fully visible block: every row's lim is past the last key, no context / target effects
+        bool full = a.mask_type != 0;
+        if (a.mask_type == 0) {
+            full = (cw0 + 32 <= rq0 + si.delta + 1) && (cw0 + 32 <= sk) && (rq0 + 32 <= sq) &&
+                   !(targets && rq0 + 31 >= sq - si.n_tgt);
+        }
+        const __amdgpu_buffer_rsrc_t rab_rsrc = make_rsrc(
+            HAS_RAB ? static_cast<const uint16_t*>(a.rab) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k) : nullptr,
+            HAS_RAB ? bias_bytes : 0u);
+        const __amdgpu_buffer_rsrc_t mask_rsrc = make_rsrc(
+            HAS_MASK ? static_cast<const uint16_t*>(a.mask) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k) : nullptr,
+            HAS_MASK ? bias_bytes : 0u);
+        uint32_t p_pk[8], ds_pk[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float p2[2], ds2[2];
+#pragma unroll
+            for (int e2 = 0; e2 < 2; ++e2) {
+                const int e = 2 * i + e2;
+                const int r = rq0 + 8 * (e / 4) + 4 * lh + (e % 4);  // query row of this element
+                float sv = s[e];
+                const uint32_t boff = (r < sq && key < a.max_k)
+                                          ? (static_cast<uint32_t>(r) * static_cast<uint32_t>(a.max_k) + static_cast<uint32_t>(key)) * 2u
+                                          : kOutOfRange;
+                if constexpr (HAS_RAB) {
+                    const uint32_t raw = __builtin_amdgcn_raw_buffer_load_b16(rab_rsrc, static_cast<int>(boff), 0, 0);
+                    sv += lo_to_float<Tag>(raw & 0xffffu);
+                }
+                float p, ds;
+                score_grad(sv, dp[e], a.alpha, c_exp, a.scale, ascale, p, ds);
+                if constexpr (HAS_MASK) {
+                    const uint32_t raw = __builtin_amdgcn_raw_buffer_load_b16(mask_rsrc, static_cast<int>(boff), 0, 0);
+                    const float m = lo_to_float<Tag>(raw & 0xffffu);
+                    p *= m;
+                    ds *= m;
+                }
+                bool vis = true;
+                if (!full) {
+                    int lim, hole_lo, hole_hi;
+                    row_bounds(si, a.mask_type, a.target_group, r, lim, hole_lo, hole_hi);
+                    vis = (r < sq) && (key < lim) && !(key >= hole_lo && key < hole_hi);
+                }
+                p2[e2] = vis ? p : 0.f;
+                ds2[e2] = vis ? ds : 0.f;
+            }
+            p_pk[i] = pack2<Tag>(p2[0], p2[1]);
+            ds_pk[i] = pack2<Tag>(ds2[0], ds2[1]);
+        }
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            const int j2 = c / MTILES, mt = c % MTILES;
+            const u32x4_t pb = {p_pk[4 * j2 + 0], p_pk[4 * j2 + 1], p_pk[4 * j2 + 2], p_pk[4 * j2 + 3]};
+            const u32x4_t db = {ds_pk[4 * j2 + 0], ds_pk[4 * j2 + 1], ds_pk[4 * j2 + 2], ds_pk[4 * j2 + 3]};
+            dv_acc[mt] = mfma32<Tag>(read_t(gt, c), pb, dv_acc[mt]);
+            dk_acc[mt] = mfma32<Tag>(read_t(qt, c), db, dk_acc[mt]);
+        }
+    };
+
+    if (n_iter > 0) {
+        request(s_qn0, s_qt0, s_gn0, s_gt0, 0);
+    }
+    for (int it = 0; it < n_iter; it += 2) {
+        step(s_qn0, s_qt0, s_gn0, s_gt0, s_qn1, s_qt1, s_gn1, s_gt1, it);
+        if (it + 1 < n_iter) {
+            step(s_qn1, s_qt1, s_gn1, s_gt1, s_qn0, s_qt0, s_gn0, s_gt0, it + 1);
+        }
+    }
+
+    // store dK, dV: lane holds key (cw0 + ln), dims 32*mt + 8*g + 4*lh + 0..3
+    {
+        const uint32_t k_off = static_cast<uint32_t>(key) * k_stride;
+        const uint32_t v_off = static_cast<uint32_t>(key) * v_stride;
+#pragma unroll
+        for (int mt = 0; mt < MTILES; ++mt) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const int d0 = 32 * mt + 8 * g + 4 * lh;
+                u32x2_t w;
+                w[0] = pack2<Tag>(dk_acc[mt][4 * g + 0], dk_acc[mt][4 * g + 1]);
+                w[1] = pack2<Tag>(dk_acc[mt][4 * g + 2], dk_acc[mt][4 * g + 3]);
+                __builtin_amdgcn_raw_buffer_store_b64(w, dk_rsrc, static_cast<int>(d0 < a.d_qk ? k_off + d0 * 2u : kOutOfRange), 0, 0);
+                w[0] = pack2<Tag>(dv_acc[mt][4 * g + 0], dv_acc[mt][4 * g + 1]);
+                w[1] = pack2<Tag>(dv_acc[mt][4 * g + 2], dv_acc[mt][4 * g + 3]);
+                __builtin_amdgcn_raw_buffer_store_b64(w, dv_rsrc, static_cast<int>(d0 < a.d_v ? v_off + d0 * 2u : kOutOfRange), 0, 0);
+            }
+        }
+    }
+}
+
+}  // namespace hstu

@@ -16,6 +16,7 @@
 #include <cstring>
 
 #include "hstu_fwd_f32_kernel.hip.h"
+#include "hstu_bwd_kernel.hip.h"
 #include "hstu_fwd_kernel.hip.h"
 
 namespace {
@@ -132,7 +133,7 @@ const Variant kVariantsF8[2][3] = {
 const Variant kVariantsF32[2][2][4] = {{HSTU_F32_DIMS(false, false), HSTU_F32_DIMS(false, true)},
                                        {HSTU_F32_DIMS(true, false), HSTU_F32_DIMS(true, true)}};
 
-int validate(const hstu_jagged_fwd_params* p)
+int validate(const hstu_jagged_fwd_params* p, bool need_out = true)
 {
     if (p == nullptr) {
         return fail(HSTU_ERR_NULLPTR, "params is NULL");
@@ -194,7 +195,7 @@ int validate(const hstu_jagged_fwd_params* p)
         return fail(HSTU_ERR_INVALID, "unknown dtype %d", p->dtype);
     }
     const bool empty = (p->total_q == 0);
-    if (!empty && (p->q == nullptr || p->out == nullptr)) {
+    if (!empty && (p->q == nullptr || (need_out && p->out == nullptr))) {
         return fail(HSTU_ERR_NULLPTR, "q / out must not be NULL");
     }
     if (p->total_k > 0 && (p->k == nullptr || p->v == nullptr)) {
@@ -326,9 +327,175 @@ uint64_t split_workspace_bytes(const Variant* var, const hstu_jagged_fwd_params*
     return bytes < kMaxWorkspaceBytes ? bytes : kMaxWorkspaceBytes;
 }
 
+// ---- backward -------------------------------------------------------------------------------------------
+struct BwdVariant {
+    const char* name;
+    void (*dkv)(const hstu::BwdArgs);
+    void (*dq)(const hstu::BwdArgs);       // without d rab
+    void (*dq_drab)(const hstu::BwdArgs);  // with d rab (nullptr when the variant has no rab)
+};
+template <typename Tag, int D, bool RAB, bool MASK>
+constexpr auto dq_drab_kernel() -> void (*)(const hstu::BwdArgs)
+{
+    if constexpr (RAB) {
+        return hstu::hstu_bwd_dq_kernel<Tag, D, RAB, MASK, true>;
+    } else {
+        return nullptr;
+    }
+}
+#define HSTU_BWD_VARIANT(tag, tagname, D, RAB, MASK)                                             \
+    {"hstu_bwd_" tagname "_d" #D "_rab" #RAB "_mask" #MASK,                                      \
+     hstu::hstu_bwd_dkv_kernel<hstu::tag, D, RAB, MASK>,                                         \
+     hstu::hstu_bwd_dq_kernel<hstu::tag, D, RAB, MASK, false>, dq_drab_kernel<hstu::tag, D, RAB, MASK>()}
+#define HSTU_BWD_DIMS(tag, tagname, RAB, MASK) \
+    {HSTU_BWD_VARIANT(tag, tagname, 64, RAB, MASK), HSTU_BWD_VARIANT(tag, tagname, 128, RAB, MASK)}
+// [dtype: bf16, f16][rab][custom mask][dim slot: 64, 128]
+const BwdVariant kBwdVariants[2][2][2][2] = {
+    {{HSTU_BWD_DIMS(bf16_tag, "bf16", false, false), HSTU_BWD_DIMS(bf16_tag, "bf16", false, true)},
+     {HSTU_BWD_DIMS(bf16_tag, "bf16", true, false), HSTU_BWD_DIMS(bf16_tag, "bf16", true, true)}},
+    {{HSTU_BWD_DIMS(f16_tag, "f16", false, false), HSTU_BWD_DIMS(f16_tag, "f16", false, true)},
+     {HSTU_BWD_DIMS(f16_tag, "f16", true, false), HSTU_BWD_DIMS(f16_tag, "f16", true, true)}},
+};
+
+int validate_bwd(const hstu_jagged_bwd_params* p)
+{
+    if (p == nullptr) {
+        return fail(HSTU_ERR_NULLPTR, "params is NULL");
+    }
+    if (p->struct_size != sizeof(hstu_jagged_bwd_params)) {
+        return fail(HSTU_ERR_INVALID, "struct_size %u does not match this library (%zu)", p->struct_size,
+                    sizeof(hstu_jagged_bwd_params));
+    }
+    const int rc = validate(&p->fwd, false);
+    if (rc != HSTU_OK) {
+        return rc;
+    }
+    if (p->fwd.total_q > 0 && (p->grad == nullptr || p->grad_q == nullptr)) {
+        return fail(HSTU_ERR_NULLPTR, "grad / grad_q must not be NULL");
+    }
+    if (p->fwd.total_k > 0 && (p->grad_k == nullptr || p->grad_v == nullptr)) {
+        return fail(HSTU_ERR_NULLPTR, "grad_k / grad_v must not be NULL");
+    }
+    if (p->grad_attn_bias != nullptr && p->fwd.attn_bias == nullptr) {
+        return fail(HSTU_ERR_INVALID, "grad_attn_bias without attn_bias");
+    }
+    return HSTU_OK;
+}
+
+const BwdVariant* select_bwd(const hstu_jagged_bwd_params* p)
+{
+    const hstu_jagged_fwd_params* f = &p->fwd;
+    if (f->dtype != HSTU_DT_BF16 && f->dtype != HSTU_DT_FP16) {
+        fail(HSTU_ERR_UNSUPPORTED, "the backward is built for bf16 and fp16");
+        return nullptr;
+    }
+    const int64_t dmax = f->head_dim_qk > f->head_dim_v ? f->head_dim_qk : f->head_dim_v;
+    if (dmax > 128 || f->head_dim_qk % 8 != 0) {
+        fail(HSTU_ERR_UNSUPPORTED, "the backward is built for head dims up to 128, q/k head dim a multiple of 8 (got %lld / %lld)",
+             (long long)f->head_dim_qk, (long long)f->head_dim_v);
+        return nullptr;
+    }
+    const int64_t span_q = f->max_seq_len_q * f->num_heads_q * dmax * 2;
+    const int64_t span_k = f->max_seq_len_k * f->num_heads_k * dmax * 2;
+    const int64_t span_b = f->max_seq_len_q * f->max_seq_len_k * 2;
+    if (span_q >= (1LL << 30) || span_k >= (1LL << 30) ||
+        ((f->attn_bias != nullptr || f->mask_type == HSTU_MASK_CUSTOM) && span_b >= (1LL << 31))) {
+        fail(HSTU_ERR_UNSUPPORTED, "max_seq_len x heads x head dim spans 1 GiB or more per sequence");
+        return nullptr;
+    }
+    return &kBwdVariants[f->dtype == HSTU_DT_BF16 ? 0 : 1][f->attn_bias != nullptr ? 1 : 0]
+                        [f->mask_type == HSTU_MASK_CUSTOM ? 1 : 0][dmax <= 64 ? 0 : 1];
+}
+
 }  // namespace
 
 extern "C" {
+
+HSTU_API int hstu_jagged_bwd_workspace_size(const hstu_jagged_bwd_params* params, uint64_t* workspace_bytes)
+{
+    if (workspace_bytes == nullptr) {
+        return fail(HSTU_ERR_NULLPTR, "workspace_bytes is NULL");
+    }
+    *workspace_bytes = 0;
+    const int rc = validate_bwd(params);
+    if (rc != HSTU_OK) {
+        return rc;
+    }
+    return select_bwd(params) == nullptr ? HSTU_ERR_UNSUPPORTED : HSTU_OK;
+}
+
+HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, uint64_t workspace_bytes, void* stream)
+{
+    (void)workspace;
+    (void)workspace_bytes;
+    const int rc = validate_bwd(p);
+    if (rc != HSTU_OK) {
+        return rc;
+    }
+    const BwdVariant* var = select_bwd(p);
+    if (var == nullptr) {
+        return HSTU_ERR_UNSUPPORTED;
+    }
+    const hstu_jagged_fwd_params* f = &p->fwd;
+    if (f->total_q == 0 && f->total_k == 0) {
+        return HSTU_OK;
+    }
+    hstu::BwdArgs a;
+    memset(&a, 0, sizeof(a));
+    a.q = f->q;
+    a.k = f->k;
+    a.v = f->v;
+    a.grad = p->grad;
+    a.rab = f->attn_bias;
+    a.mask = (f->mask_type == HSTU_MASK_CUSTOM) ? f->mask : nullptr;
+    a.dq = p->grad_q;
+    a.dk = p->grad_k;
+    a.dv = p->grad_v;
+    a.drab = p->grad_attn_bias;
+    a.offs_q = f->seq_offset_q;
+    a.offs_k = f->seq_offset_k;
+    a.num_ctx = f->num_context;
+    a.num_tgt = f->num_target;
+    a.total_q = f->total_q;
+    a.total_k = f->total_k;
+    a.n_batch = static_cast<int>(f->n_offsets - 1);
+    a.n_heads_q = static_cast<int>(f->num_heads_q);
+    a.n_heads_k = static_cast<int>(f->num_heads_k);
+    a.head_ratio = a.n_heads_q / a.n_heads_k;
+    a.d_qk = static_cast<int>(f->head_dim_qk);
+    a.d_v = static_cast<int>(f->head_dim_v);
+    a.max_q = static_cast<int>(f->max_seq_len_q);
+    a.max_k = static_cast<int>(f->max_seq_len_k);
+    a.mask_type = static_cast<int>(f->mask_type);
+    a.target_group = static_cast<int>(f->target_group_size);
+    a.idx64 = (f->index_dtype == HSTU_IDX_I64) ? 1 : 0;
+    a.n_qtiles = (a.max_q + hstu::kBlockM - 1) / hstu::kBlockM;
+    a.n_ktiles = (a.max_k + hstu::kBlockM - 1) / hstu::kBlockM;
+    a.bias_vec_ok = (reinterpret_cast<uintptr_t>(f->attn_bias) % 8 == 0 && reinterpret_cast<uintptr_t>(f->mask) % 8 == 0 &&
+                     reinterpret_cast<uintptr_t>(p->grad_attn_bias) % 8 == 0 && f->max_seq_len_k % 4 == 0)
+                        ? 1
+                        : 0;
+    a.alpha = static_cast<float>(f->alpha);
+    a.scale = static_cast<float>((f->silu_scale == 0.0) ? 1.0 / static_cast<double>(f->max_seq_len_q) : f->silu_scale);
+
+    const int64_t grid_kv = static_cast<int64_t>(a.n_ktiles) * a.n_batch * a.n_heads_k;
+    const int64_t grid_q = static_cast<int64_t>(a.n_qtiles) * a.n_batch * a.n_heads_q;
+    if (grid_kv > 0x7fffffffLL || grid_q > 0x7fffffffLL) {
+        return fail(HSTU_ERR_INVALID, "grid out of range");
+    }
+    if (f->total_k > 0 && grid_kv > 0) {
+        hipLaunchKernelGGL(var->dkv, dim3(static_cast<unsigned>(grid_kv)), dim3(256), 0, static_cast<hipStream_t>(stream), a);
+    }
+    if (f->total_q > 0 && grid_q > 0) {
+        hipLaunchKernelGGL(p->grad_attn_bias != nullptr ? var->dq_drab : var->dq, dim3(static_cast<unsigned>(grid_q)), dim3(256),
+                           0, static_cast<hipStream_t>(stream), a);
+    }
+    const hipError_t err = hipGetLastError();
+    if (err != hipSuccess) {
+        return fail(HSTU_ERR_RUNTIME, "launch of %s failed: %s", var->name, hipGetErrorString(err));
+    }
+    return HSTU_OK;
+}
 
 HSTU_API int hstu_version(void) { return (0 << 16) | 1; }
 

@@ -22,6 +22,8 @@ EXPORTED_SYMBOLS = (
     "hstu_last_error",
     "hstu_version",
     "hstu_jagged_fwd_kernel_name",
+    "hstu_jagged_bwd_workspace_size",
+    "hstu_jagged_bwd",
 )
 
 
@@ -64,6 +66,21 @@ class FwdParams(ctypes.Structure):
     ]
 
 
+class BwdParams(ctypes.Structure):
+    """Mirror of ``hstu_jagged_bwd_params``."""
+
+    _fields_ = [
+        ("struct_size", ctypes.c_uint32),
+        ("reserved0", ctypes.c_uint32),
+        ("fwd", FwdParams),
+        ("grad", ctypes.c_void_p),
+        ("grad_q", ctypes.c_void_p),
+        ("grad_k", ctypes.c_void_p),
+        ("grad_v", ctypes.c_void_p),
+        ("grad_attn_bias", ctypes.c_void_p),
+    ]
+
+
 _lib: Optional[ctypes.CDLL] = None
 
 
@@ -93,6 +110,10 @@ def load() -> ctypes.CDLL:
     lib.hstu_version.argtypes = []
     lib.hstu_jagged_fwd_kernel_name.restype = ctypes.c_char_p
     lib.hstu_jagged_fwd_kernel_name.argtypes = [ctypes.POINTER(FwdParams)]
+    lib.hstu_jagged_bwd_workspace_size.restype = ctypes.c_int
+    lib.hstu_jagged_bwd_workspace_size.argtypes = [ctypes.POINTER(BwdParams), ctypes.POINTER(ctypes.c_uint64)]
+    lib.hstu_jagged_bwd.restype = ctypes.c_int
+    lib.hstu_jagged_bwd.argtypes = [ctypes.POINTER(BwdParams), ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]
     _lib = lib
     return lib
 
@@ -104,4 +125,11 @@ def last_error() -> str:
 def new_params() -> FwdParams:
     p = FwdParams()
     p.struct_size = ctypes.sizeof(FwdParams)
+    return p
+
+
+def new_bwd_params() -> BwdParams:
+    p = BwdParams()
+    p.struct_size = ctypes.sizeof(BwdParams)
+    p.fwd.struct_size = ctypes.sizeof(FwdParams)
     return p

@@ -18,6 +18,7 @@ reference (which registers only the NPU and Meta keys).
 from __future__ import annotations
 
 import ctypes
+import os
 from typing import Optional, Tuple
 
 import torch
@@ -309,8 +310,9 @@ def hstu_jagged_delta_meta(q, k, v, mask=None, attn_bias=None, mask_type=0, max_
 
 
 # ----------------------------------------------------------------------------------------------
-# backward op: device-side composite (torch ops on the GPU, per sequence, fp32).  It exists so that
-# the autograd wrapper of the forward is complete; it is not a tuned kernel.
+# backward op: HIP kernels through the C ABI for bf16 / fp16 with head dims up to 128 (_backward_hip); a
+# device-side composite (torch ops on the GPU, per sequence, fp32) for the rest (fp32 inputs, larger head
+# dims), which is also what HSTU_MI355_COMPOSITE_BACKWARD=1 selects for comparisons.
 #   X = alpha (S + rab),  sig = sigmoid(X),  P = X sig scale M
 #   dV = P^T dO,  dX = (dO V^T) scale M sig (1 + X (1 - sig)),  dS = dRab = alpha dX,  dQ = dS K,  dK = dS^T Q
 # (ascendc/attention/hstu_v1/hstu_backward_v1/op_kernel/vector_score.h:159-205)
@@ -332,6 +334,71 @@ def _device_builtin_mask(s_q, s_k, ctx, tgt, group, device):
     return m
 
 
+def hip_backward_available(q, k, v) -> bool:
+    """Whether the HIP backward kernels cover these tensors (bf16 / fp16, head dims up to 128, q/k head dim a
+    multiple of 8); everything else takes the composite below."""
+    return (q.dtype in (torch.bfloat16, torch.float16) and max(q.shape[2], v.shape[2]) <= 128 and q.shape[2] % 8 == 0
+            and v.shape[2] % 16 == 0)  # fmt: skip
+
+
+def _backward_hip(grad, q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max_seq_len_k, silu_scale, seq_offset,
+                  seq_offset_k, num_context, num_target, group, alpha):  # fmt: skip
+    """The backward through the C ABI (``hstu_jagged_bwd``): two kernels on the current stream."""
+    idx_dtype = seq_offset.dtype
+    offs_q = seq_offset.contiguous()
+    offs_k = offs_q if seq_offset_k is seq_offset else seq_offset_k.to(idx_dtype).contiguous()
+    q_c, k_c, v_c, g_c = q.contiguous(), k.contiguous(), v.contiguous(), grad.contiguous()
+    batch = offs_q.size(0) - 1
+    ctx = num_context.to(idx_dtype).contiguous() if num_context is not None else None
+    tgt = num_target.to(idx_dtype).contiguous() if num_target is not None else None
+    _check(g_c.dtype == q_c.dtype == k_c.dtype == v_c.dtype, "grad, q, k, v must share one dtype")
+    _check(tuple(g_c.shape) == (q_c.size(0), q_c.size(1), v_c.size(2)), "grad must have the shape of the forward output")
+    bias_shape = (batch, q_c.size(1), int(max_seq_len_q), int(max_seq_len_k))
+    bias = mask_c = None
+    if attn_bias is not None:
+        _check(attn_bias.dtype == q.dtype and tuple(attn_bias.shape) == bias_shape, f"attn_bias must be {bias_shape} of q's dtype")
+        bias = attn_bias.contiguous()
+    if int(mask_type) == 3:
+        _check(mask is not None and mask.dtype == q.dtype and tuple(mask.shape) == bias_shape,
+               f"mask must be {bias_shape} of q's dtype")  # fmt: skip
+        mask_c = mask.contiguous()
+    # rows past the last offset belong to no sequence and are not written by the kernels; the bias gradient is
+    # written only where a query tile sweeps
+    dq, dk, dv = torch.zeros_like(q_c), torch.zeros_like(k_c), torch.zeros_like(v_c)
+    dbias = torch.zeros_like(bias) if bias is not None else None
+    if q_c.numel() == 0 and k_c.numel() == 0:
+        return dq, dk, dv, dbias
+    p = _native.new_bwd_params()
+    f = p.fwd
+    f.dtype = f.out_dtype = _DTYPE_CODE[q_c.dtype]
+    f.index_dtype = _native.IDX_I64 if idx_dtype == torch.int64 else _native.IDX_I32
+    f.q, f.k, f.v = _ptr(q_c), _ptr(k_c), _ptr(v_c)
+    f.mask, f.attn_bias = _ptr(mask_c), _ptr(bias)
+    f.seq_offset_q, f.seq_offset_k = _ptr(offs_q), _ptr(offs_k)
+    f.num_context, f.num_target = _ptr(ctx), _ptr(tgt)
+    f.total_q, f.total_k = q_c.size(0), k_c.size(0)
+    f.num_heads_q, f.num_heads_k = q_c.size(1), k_c.size(1)
+    f.head_dim_qk, f.head_dim_v = q_c.size(2), v_c.size(2)
+    f.n_offsets = offs_q.size(0)
+    f.mask_type = int(mask_type)
+    f.max_seq_len_q, f.max_seq_len_k = int(max_seq_len_q), int(max_seq_len_k)
+    f.target_group_size = group
+    f.silu_scale = (1.0 / float(max_seq_len_q)) if float(silu_scale) == 0.0 else float(silu_scale)
+    f.alpha = alpha
+    p.grad, p.grad_q, p.grad_k, p.grad_v, p.grad_attn_bias = _ptr(g_c), _ptr(dq), _ptr(dk), _ptr(dv), _ptr(dbias)
+    lib = _native.load()
+    ws_bytes = ctypes.c_uint64(0)
+    rc = lib.hstu_jagged_bwd_workspace_size(ctypes.byref(p), ctypes.byref(ws_bytes))
+    if rc != _native.HSTU_OK:
+        raise RuntimeError(f"hstu_jagged_bwd_workspace_size failed ({rc}): {_native.last_error()}")
+    ws = torch.empty(ws_bytes.value, dtype=torch.uint8, device=q_c.device) if ws_bytes.value else None
+    stream = torch.cuda.current_stream(q_c.device).cuda_stream
+    rc = lib.hstu_jagged_bwd(ctypes.byref(p), _ptr(ws), ws_bytes.value, ctypes.c_void_p(stream))
+    if rc != _native.HSTU_OK:
+        raise RuntimeError(f"hstu_jagged_bwd failed ({rc}): {_native.last_error()}")
+    return dq, dk, dv, dbias
+
+
 def _backward_impl(grad, q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max_seq_len_k, silu_scale, seq_offset,
                    seq_offset_k, num_context, num_target, target_group_size, alpha):  # fmt: skip
     _check(seq_offset.size(0) >= 2, "seqOffsetQ params error should have at least two element.")
@@ -343,6 +410,10 @@ def _backward_impl(grad, q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max
         _check(num_target is not None, "numTarget is required when numContext or targetGroupSize is not None")
     group = 0 if target_group_size is None else int(target_group_size)
     a = 1.0 if alpha is None else float(alpha)
+    if hip_backward_available(q, k, v) and os.environ.get("HSTU_MI355_COMPOSITE_BACKWARD", "0") != "1":
+        _mask_check(int(mask_type), mask is not None)
+        return _backward_hip(grad, q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max_seq_len_k, silu_scale,
+                             seq_offset, seq_offset_k, num_context, num_target, group, a)  # fmt: skip
     scale = (1.0 / float(max_seq_len_q)) if float(silu_scale) == 0.0 else float(silu_scale)
     offs_q = seq_offset.tolist()
     offs_k = seq_offset_k.tolist()

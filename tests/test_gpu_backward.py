@@ -1,0 +1,153 @@
+"""The HIP backward kernels (``hstu_jagged_bwd`` of the C ABI, reached through ``hstu_jagged_backward`` and through
+``loss.backward()``) against torch autograd on the CPU oracle, on the same seeded inputs.
+
+Tolerance: the kernels round P and dS to the input type before the products that consume them (as the reference's
+backward does, hstu_backward_v1/op_kernel/vector_score.h:159-205), so a gradient element carries the rounding of a
+sum of up to S products: each gradient tensor must agree with the fp32 oracle within atol = 1e-2 x max|reference|
+and rtol = 1e-2 (bf16) / atol = 2e-3 x max|reference|, rtol = 2e-3 (fp16) -- the forward's 1e-2 bar relative to the
+tensor's scale -- and must not be further from it than 2 x the device-side fp32 composite's own rounding to the
+output type plus that bound.  The same cases run through the composite (HSTU_MI355_COMPOSITE_BACKWARD=1) pin that the
+two device paths agree.
+"""
+
+import dataclasses
+
+import pytest
+import torch
+
+import ops_rec
+from ops_rec import workloads
+from oracle import hstu_oracle as O
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def oracle_grads(w, grad_out):
+    c = w.to("cpu")
+    q, k, v = (t.float().clone().requires_grad_(True) for t in (c.q, c.k, c.v))
+    kw = c.oracle_kwargs()
+    bias = None
+    if c.attn_bias is not None:
+        bias = c.attn_bias.float().clone().requires_grad_(True)
+        kw["attn_bias"] = bias
+    out = O.hstu_jagged_forward(q, k, v, out_dtype=torch.float32, **kw)
+    out.backward(grad_out.float().cpu())
+    return q.grad, k.grad, v.grad, (bias.grad if bias is not None else None)
+
+
+def device_grads(w, grad_out):
+    k_offs = w.seq_offset if w.seq_offset_k is None else w.seq_offset_k
+    max_k = w.max_seq_len if w.max_seq_len_k is None else w.max_seq_len_k
+    ctx, tgt = w.num_context, w.num_target
+    if (ctx is None) != (tgt is None):  # the backward op wants both or neither (hstu_jagged_plugin.cpp:81-84)
+        zeros = torch.zeros_like(ctx if tgt is None else tgt)
+        ctx, tgt = (zeros if ctx is None else ctx), (zeros if tgt is None else tgt)
+    got = ops_rec.ascendc.attention.hstu_jagged_backward(
+        grad_out, w.q, w.k, w.v, w.mask, w.attn_bias, w.mask_type, w.max_seq_len, max_k, w.silu_scale, w.seq_offset,
+        k_offs, ctx, tgt, w.target_group_size, w.alpha)  # fmt: skip
+    torch.cuda.synchronize()
+    return got
+
+
+def check(w, monkeypatch, seed=5):
+    g = torch.Generator(device=DEV).manual_seed(seed)
+    grad_out = torch.randn(w.q.shape[0], w.q.shape[1], w.v.shape[2], generator=g, device=DEV).to(w.q.dtype)
+    monkeypatch.setenv("HSTU_MI355_COMPOSITE_BACKWARD", "0")
+    got = device_grads(w, grad_out)
+    assert torch.equal(device_grads(w, grad_out)[0], got[0])  # reproducible
+    monkeypatch.setenv("HSTU_MI355_COMPOSITE_BACKWARD", "1")
+    comp = device_grads(w, grad_out)
+    ref = oracle_grads(w, grad_out)
+    tol = 1e-2 if w.q.dtype == torch.bfloat16 else 2e-3
+    for name, a, c, r in zip(("dq", "dk", "dv", "dbias"), got, comp, ref):
+        if r is None:
+            assert a is None
+            continue
+        assert a.dtype == w.q.dtype and a.shape == r.shape, name
+        a, c = a.float().cpu(), c.float().cpu()
+        assert torch.isfinite(a).all(), name
+        scale = r.abs().max().item()
+        torch.testing.assert_close(a, r, atol=tol * scale, rtol=tol, msg=lambda m, n=name: f"{n} vs oracle: {m}")
+        torch.testing.assert_close(a, c, atol=tol * scale, rtol=tol, msg=lambda m, n=name: f"{n} vs composite: {m}")
+        assert (a - r).abs().max() <= 2 * (c - r).abs().max() + tol * scale, name
+
+
+def make(**kw):
+    kw.setdefault("dtype", torch.bfloat16)
+    kw.setdefault("std", 0.5)
+    kw.setdefault("silu_scale", 1.0)
+    return workloads.make("bwd", device=DEV, **kw)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("dim,dim_v", [(64, 64), (128, 128), (96, 64), (32, 16), (8, 128)])
+def test_plain_causal(dim, dim_v, dtype, monkeypatch):
+    check(make(batch=3, heads=2, dim=dim, dim_v=dim_v, lo=1, hi=300, seed=dim + dim_v, dtype=dtype), monkeypatch)
+
+
+@pytest.mark.parametrize("ctx,tgt,group", [(0, 30, 1), (0, 30, 3), (6, 0, 0), (6, 30, 3), (200, 40, 7)])
+@pytest.mark.parametrize("rab", [False, True], ids=["norab", "rab"])
+def test_context_targets_rab(ctx, tgt, group, rab, monkeypatch):
+    w = make(batch=3, heads=2, dim=64, lo=260, hi=420, max_seq_len=420, seed=ctx + tgt, num_context=ctx, max_target=tgt,
+             target_group_size=group, rab_std=0.5 if rab else None)  # fmt: skip
+    check(w, monkeypatch)
+
+
+@pytest.mark.parametrize("max_len", [300, 301, 303])  # rows of rab / mask / d rab 8-byte aligned or not
+def test_custom_mask_and_rab_alignment(max_len, monkeypatch):
+    w = make(batch=2, heads=2, dim=64, lo=150, hi=max_len, max_seq_len=max_len, seed=max_len, rab_std=0.5, dtype=torch.float16)
+    g = torch.Generator(device=DEV).manual_seed(1)
+    mask = (torch.rand(2, 2, max_len, max_len, generator=g, device=DEV) < 0.6).to(torch.float16)
+    check(dataclasses.replace(w, mask=mask, mask_type=3), monkeypatch)
+
+
+def test_no_mask(monkeypatch):
+    check(dataclasses.replace(make(batch=2, heads=2, dim=128, lo=100, hi=300, seed=9), mask_type=2), monkeypatch)
+
+
+@pytest.mark.parametrize("heads,heads_k", [(4, 2), (8, 1), (3, 3)])
+def test_grouped_heads(heads, heads_k, monkeypatch):
+    check(make(batch=3, heads=heads, heads_k=heads_k, dim=64, lo=50, hi=400, seed=heads, rab_std=0.3), monkeypatch)
+
+
+def test_more_keys_than_queries(monkeypatch):
+    lq, lk = [70, 200, 1], [370, 333, 129]
+    g = torch.Generator(device=DEV).manual_seed(8)
+    mk = lambda n, h, d: (torch.randn(n, h, d, generator=g, device=DEV) * 0.5).to(torch.bfloat16)  # noqa: E731
+    offs = lambda ls: torch.tensor([0] + list(torch.tensor(ls).cumsum(0)), dtype=torch.int64, device=DEV)  # noqa: E731
+    w = workloads.Workload(name="delta", q=mk(sum(lq), 2, 64), k=mk(sum(lk), 2, 64), v=mk(sum(lk), 2, 64),
+                           seq_offset=offs(lq), max_seq_len=200, silu_scale=1.0, alpha=0.125, seq_offset_k=offs(lk),
+                           max_seq_len_k=370, lengths=lq)  # fmt: skip
+    check(w, monkeypatch)
+
+
+def test_long_sequences_and_rows_past_the_last_offset(monkeypatch):
+    w = make(batch=2, heads=2, dim=128, lo=1500, hi=2500, seed=7, std=0.3)
+    # 40 rows that belong to no sequence: their gradients must come back as zeros
+    pad = lambda t: torch.cat([t, torch.ones(40, *t.shape[1:], dtype=t.dtype, device=DEV)])  # noqa: E731
+    w = dataclasses.replace(w, q=pad(w.q), k=pad(w.k), v=pad(w.v))
+    check(w, monkeypatch)
+    grad_out = torch.ones(w.q.shape[0], 2, 128, dtype=torch.bfloat16, device=DEV)
+    monkeypatch.setenv("HSTU_MI355_COMPOSITE_BACKWARD", "0")
+    dq, dk, dv, _ = device_grads(w, grad_out)
+    assert not dq[-40:].any() and not dk[-40:].any() and not dv[-40:].any()
+
+
+def test_empty_sequences_and_trailing_repeated_offset(monkeypatch):
+    w = make(batch=5, heads=2, dim=64, lo=0, hi=0, lengths=[0, 130, 0, 57, 0], seed=3)
+    check(w, monkeypatch)
+
+
+def test_loss_backward_uses_the_kernels(monkeypatch):
+    monkeypatch.setenv("HSTU_MI355_COMPOSITE_BACKWARD", "0")
+    w = make(batch=2, heads=2, dim=64, lo=100, hi=200, seed=11, rab_std=0.3)
+    q, k, v, bias = (t.clone().requires_grad_(True) for t in (w.q, w.k, w.v, w.attn_bias))
+    args = list(w.op_args())
+    args[0], args[1], args[2], args[4] = q, k, v, bias
+    out = ops_rec.ascendc.attention.hstu_jagged(*args)
+    grad_out = torch.randn(out.shape, device=DEV).to(out.dtype)
+    out.backward(grad_out)
+    direct = device_grads(w, grad_out)
+    for a, b in zip((q.grad, k.grad, v.grad, bias.grad), direct):
+        assert torch.equal(a, b)
