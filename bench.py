@@ -58,6 +58,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="C2", choices=["C2", "C3", "C4", "C5"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--backward", action="store_true",
+                    help="also time hstu_jagged_backward (the two HIP backward kernels) on the same workload and add a "
+                    "'backward' object to the line (bf16 workloads only)")  # fmt: skip
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="after the timed steps also run 5 plain device-to-device copies of this many MiB, so that a "
                     "counter run (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) can be scaled by a kernel of known traffic")  # fmt: skip
@@ -196,6 +199,35 @@ def main() -> int:
             "rab_read_GBs": round(rab_bytes / (ev_ms * 1e-3) / 1e9, 1) if rab_bytes else None,
         },
     }
+
+    # ---- backward (optional): d q, d k, d v (and d attn_bias) through the operator ----
+    if args.backward and not fp8:
+        grad = torch.randn(prepared.out.shape, device=dev).to(prepared.out.dtype)
+        zeros = None if w.num_context is None and w.num_target is None else torch.zeros(len(w.lengths), dtype=w.seq_offset.dtype, device=dev)
+        bwd_args = (grad, w.q, w.k, w.v, w.mask, w.attn_bias, w.mask_type, w.max_seq_len, w.silu_scale, w.seq_offset,
+                    w.num_context if w.num_context is not None else zeros, w.num_target if w.num_target is not None else zeros,
+                    w.target_group_size, w.alpha)  # fmt: skip
+        bwd = ops_rec.ascendc.attention.hstu_jagged_backward
+        n_bwd = max(5, args.steps // 10)
+        for _ in range(3):
+            bwd(*bwd_args)
+        torch.cuda.synchronize()
+        e0.record(stream)
+        for _ in range(n_bwd):
+            bwd(*bwd_args)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        bwd_ms = e0.elapsed_time(e1) / n_bwd
+        bwd_flops = flops * 5 // 2  # five products (S, dP, dV, dK, dQ) against the forward's two
+        result["backward"] = {
+            "ms_per_step": round(bwd_ms, 6),
+            "steps": n_bwd,
+            "flops_per_step": bwd_flops,
+            "tflops": round(bwd_flops / (bwd_ms * 1e-3) / 1e12, 3),
+            "pct_of_bf16_mfma_peak": round(100.0 * bwd_flops / (bwd_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 2),
+            "note": "through torch.ops.ops_rec.hstu_jagged_backward: zero-filled gradient tensors + hstu_bwd_dkv_kernel "
+            "+ hstu_bwd_dq_kernel per step; the kernels recompute S and dP (seven products issued)",
+        }
 
     # ---- CPU baseline: dense-padded fp32 golden path on this host's cores ----
     if not args.no_cpu and w_cpu is not None:

@@ -8,14 +8,15 @@
 //
 // Two kernels, no atomics, every output row written by exactly one wavefront (bitwise reproducible):
 //
-//   hstu_bwd_dkv_kernel  one workgroup per 128-key tile of one (sequence, K/V head): each wavefront keeps the K
-//                        and V rows of its 32 keys in registers (B operands) and sweeps the query rows that can
-//                        see them, 32 at a time, for every query head of the group.  Q and dO sub-tiles stream
-//                        through LDS.  Per sub-tile:
-//                            S  = Q . K^T          (A = Q  from LDS,            B = K registers)
-//                            dP = dO . V^T         (A = dO from LDS,            B = V registers)
-//                            dV^T += dO^T . P      (A = dO^T, transposed read,  B = P  from the accumulators)
-//                            dK^T += Q^T . dS      (A = Q^T,  transposed read,  B = dS from the accumulators)
+//   hstu_bwd_dkv_kernel  one workgroup (8 wavefronts) per 128-key tile of one (sequence, K/V head).  The key rows
+//                        stay in registers (B operands) while the query rows that can see them stream through
+//                        LDS, 32 at a time, for every query head of the group.  Two wavefronts share each set of
+//                        32 keys, one per output, so that either fits in 256 registers and a SIMD holds one of
+//                        each kind (their MFMA and VALU phases overlap):
+//                          dV wavefront:  S = Q . K^T,  P,            dV^T += dO^T . P
+//                          dK wavefront:  S = Q . K^T,  dP = dO . V^T,  dS,  dK^T += Q^T . dS
+//                        (A operands from LDS: Q, dO plain; dO^T, Q^T by transposed reads; B operands: K, V rows in
+//                        registers, P / dS straight from the accumulators)
 //   hstu_bwd_dq_kernel   one workgroup per 128-row query tile of one (sequence, head), the forward's shape: Q and
 //                        dO rows in registers, K and V sub-tiles stream through LDS.  Per sub-tile:
 //                            S^T  = K . Q^T,   dP^T = V . dO^T,   dQ^T += K^T . dS^T
@@ -23,9 +24,9 @@
 //
 // As in the forward, the score block is computed with the streamed operand as rows, so that its accumulator layout
 // (lane = resident row, registers = streamed rows) is the B-operand layout of the products that consume it: P and
-// dS never leave registers.  A sub-tile that is read both plainly and transposed is kept in LDS twice, once in
-// each bank-conflict-free layout.  Recomputing S and dP in both kernels costs 7 products instead of 5 and buys
-// freedom from atomics and from a dQ workspace.
+// dS never leave registers.  A sub-tile that is read both plainly and transposed is kept in LDS once, in a layout
+// that is free of bank conflicts for both reads.  Recomputing S and dP in both kernels costs 7 products instead of 5 and buys
+// freedom from atomics and from a dQ workspace (8 with the S computed by both wavefronts of a key set).
 #pragma once
 #include "hstu_fwd_kernel.hip.h"
 
@@ -150,6 +151,23 @@ __device__ __forceinline__ void score_grad(float s, float dp, float alpha, float
 // ---------------------------------------------------------------------------------------------------------
 // shared pieces of the two kernels: the two LDS layouts of a 32-row sub-tile and their read patterns
 // ---------------------------------------------------------------------------------------------------------
+// One LDS layout of a 32-row sub-tile that is free of bank conflicts for both ways it is read here: plainly (A
+// operand rows = tile rows: 16 consecutive rows, one 16-byte chunk each) and transposed (ds_read_b64_tr_b16: rows
+// 4 h .. 4 h + 3, 64 bytes each).  The XOR term is a bijection of the row bits that index the rows sharing 16 chunk
+// positions, with the two bits that tell rows 0..3 apart moved to the top, where they select the 64-byte group.
+// Adding 8 to the row flips bit 1 of the term, adding 16 leaves it alone.
+template <int D>
+__device__ __forceinline__ int both_ways_swizzle(int row, int chunk)
+{
+    static_assert(D == 64 || D == 128, "layouts exist for 64 and 128 elements per row");
+    if constexpr (D == 128) {
+        return chunk ^ (((row & 3) << 2) | ((row >> 2) & 3));
+    } else {
+        const int p = row >> 1;
+        return chunk ^ (((p & 1) << 2) | ((p >> 1) & 3));
+    }
+}
+
 template <int D>
 struct SubTile {
     static constexpr int CPR = D / 8;                 // 16-byte chunks per row
@@ -169,12 +187,20 @@ __global__ __launch_bounds__(256, 2) void hstu_bwd_dq_kernel(const BwdArgs a)
 {
     typedef SubTile<D> T;
     constexpr int LPW = T::LPW, NLW = T::NLW, KSTEPS = T::KSTEPS, MTILES = T::MTILES, NCH = 2 * T::MTILES;
-    __shared__ __attribute__((aligned(1024))) uint16_t s_kn0[T::ELEMS];  // K, layout for plain reads
-    __shared__ __attribute__((aligned(1024))) uint16_t s_kn1[T::ELEMS];
-    __shared__ __attribute__((aligned(1024))) uint16_t s_kt0[T::ELEMS];  // K, layout for transposed reads
-    __shared__ __attribute__((aligned(1024))) uint16_t s_kt1[T::ELEMS];
-    __shared__ __attribute__((aligned(1024))) uint16_t s_vn0[T::ELEMS];  // V, layout for plain reads
-    __shared__ __attribute__((aligned(1024))) uint16_t s_vn1[T::ELEMS];
+    // three stages of {K, V} sub-tiles; separate arrays so that the compiler can tell the stage being filled by
+    // the asynchronous loads from the one being read.  K is read plainly (S^T) and transposed (dQ^T) from one copy.
+    __shared__ __attribute__((aligned(1024))) uint16_t s_k0[T::ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_k1[T::ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_k2[T::ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_v0[T::ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_v1[T::ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_v2[T::ELEMS];
+    // The sub-tile of step x is requested two steps ahead; a wavefront may have the requests of one later step
+    // outstanding when it starts a step (requests past the last sub-tile are sent out of range, so that the count
+    // per step is constant).  Memory latency under load is longer than one step.
+    constexpr int kReqs = 2 * LPW;
+    constexpr int kWaitStage = (kReqs & 15) | (7 << 4) | (15 << 8) | ((kReqs >> 4) << 14);
+    constexpr uint32_t kPastEnd = 0x40000000u;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -219,30 +245,29 @@ __global__ __launch_bounds__(256, 2) void hstu_bwd_dq_kernel(const BwdArgs a)
                   sk > 0 ? static_cast<uint32_t>(sk - 1) * v_stride + a.d_v * 2u : 0u);
 
     // per-lane source offsets of the sub-tile loads (see the forward kernel: 16-byte slot -> row, swizzled chunk)
-    uint32_t kn_src[LPW], kt_src[LPW], vn_src[LPW];
+    uint32_t k_src[LPW], v_src[LPW];
 #pragma unroll
     for (int i = 0; i < LPW; ++i) {
         const int slot = (wave * LPW + i) * 64 + lane;
         const int r = (slot / T::CPR) & 31;
         const int pc = slot % T::CPR;
-        const int cn = k_chunk_swizzle<D>(r, pc);
-        const int ct = v_chunk_swizzle<D>(r, pc);
-        kn_src[i] = (cn * 8 < a.d_qk) ? static_cast<uint32_t>(r) * k_stride + cn * 16u : kOutOfRange;
-        kt_src[i] = (ct * 8 < a.d_qk) ? static_cast<uint32_t>(r) * k_stride + ct * 16u : kOutOfRange;
-        vn_src[i] = (cn * 8 < a.d_v) ? static_cast<uint32_t>(r) * v_stride + cn * 16u : kOutOfRange;
+        const int cs = both_ways_swizzle<D>(r, pc);  // (its own inverse)
+        k_src[i] = (cs * 8 < a.d_qk) ? static_cast<uint32_t>(r) * k_stride + cs * 16u : kOutOfRange;
+        v_src[i] = (cs * 8 < a.d_v) ? static_cast<uint32_t>(r) * v_stride + cs * 16u : kOutOfRange;
     }
     int n_lane_off[KSTEPS];  // plain read of row ln, MFMA step js
-    int t_lane_off[MTILES];  // transposed read, output tile mt
+    int t_lane_off[MTILES][2];  // transposed read, output tile mt: rows vr0 (+ 16 j2) and vr0 + 8 (+ 16 j2)
 #pragma unroll
     for (int js = 0; js < KSTEPS; ++js) {
-        n_lane_off[js] = ln * D + k_chunk_swizzle<D>(ln, 2 * js + lh) * 8;
+        n_lane_off[js] = ln * D + both_ways_swizzle<D>(ln, 2 * js + lh) * 8;
     }
     {
         const int vr0 = 4 * lh + ((lane & 15) >> 2);
 #pragma unroll
         for (int mt = 0; mt < MTILES; ++mt) {
             const int col = 32 * mt + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-            t_lane_off[mt] = vr0 * D + v_chunk_swizzle<D>(vr0, col >> 3) * 8 + (col & 7);
+            t_lane_off[mt][0] = vr0 * D + both_ways_swizzle<D>(vr0, col >> 3) * 8 + (col & 7);
+            t_lane_off[mt][1] = (vr0 + 8) * D + both_ways_swizzle<D>(vr0 + 8, col >> 3) * 8 + (col & 7);
         }
     }
 
@@ -328,15 +353,15 @@ __global__ __launch_bounds__(256, 2) void hstu_bwd_dq_kernel(const BwdArgs a)
     const float c_exp = -a.alpha * 1.4426950408889634f;
     const float ascale = a.alpha * a.scale;
 
-    auto request = [&](uint16_t* kn, uint16_t* kt, uint16_t* vn, int x) {
-        if (NLW == 4 || wave < NLW) {
-            const uint32_t kb = static_cast<uint32_t>(x * 32) * k_stride;
-            const uint32_t vb = static_cast<uint32_t>(x * 32) * v_stride;
+    static_assert(NLW == 4, "every wavefront takes part in the loads");
+    auto request = [&](uint16_t* kd, uint16_t* vd, int x) {
+        {
+            const uint32_t kb = x < n_sub ? static_cast<uint32_t>(x * 32) * k_stride : kPastEnd;
+            const uint32_t vb = x < n_sub ? static_cast<uint32_t>(x * 32) * v_stride : kPastEnd;
 #pragma unroll
             for (int i = 0; i < LPW; ++i) {
-                load_to_lds_b128(k_rsrc, kn + (wave * LPW + i) * 512, kn_src[i] + kb);
-                load_to_lds_b128(k_rsrc, kt + (wave * LPW + i) * 512, kt_src[i] + kb);
-                load_to_lds_b128(v_rsrc, vn + (wave * LPW + i) * 512, vn_src[i] + vb);
+                load_to_lds_b128(k_rsrc, kd + (wave * LPW + i) * 512, k_src[i] + kb);
+                load_to_lds_b128(v_rsrc, vd + (wave * LPW + i) * 512, v_src[i] + vb);
             }
         }
     };
@@ -345,20 +370,21 @@ __global__ __launch_bounds__(256, 2) void hstu_bwd_dq_kernel(const BwdArgs a)
     };
     auto read_t = [&](const uint16_t* tile, int c) -> u32x4_t {
         const int j2 = c / MTILES, mt = c % MTILES;
-        const uint16_t* p = tile + t_lane_off[mt] + 16 * j2 * D;
-        const u32x2_t lo = lds_read_tr16_b64(p);
-        const u32x2_t hi = lds_read_tr16_b64(p + 8 * D);
+        const u32x2_t lo = lds_read_tr16_b64(tile + t_lane_off[mt][0] + 16 * j2 * D);
+        const u32x2_t hi = lds_read_tr16_b64(tile + t_lane_off[mt][1] + 16 * j2 * D);
         const u32x4_t r = {lo[0], lo[1], hi[0], hi[1]};
         return r;
     };
 
-    auto step = [&](const uint16_t* kn, const uint16_t* kt, const uint16_t* vn, uint16_t* kn_o, uint16_t* kt_o,
-                    uint16_t* vn_o, int x) {
-        __builtin_amdgcn_s_waitcnt(0);
-        __syncthreads();  // sub-tile x has landed for everybody, and nobody reads the other buffer any more
-        if (x + 1 < n_sub) {
-            request(kn_o, kt_o, vn_o, x + 1);
-        }
+    auto step = [&](const uint16_t* kn, const uint16_t* vn, uint16_t* kn_o, uint16_t* vn_o, int x) {
+        // sub-tile x has landed (mine, then everybody's), and nobody reads the stage of step x - 1 any more: all
+        // LDS reads of a step feed MFMAs that were issued before the barrier.  (A bare barrier: __syncthreads()
+        // would add a fence that waits for every outstanding request.)
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(kWaitStage);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        request(kn_o, vn_o, x + 2);
         if (x >= nx_w) {
             return;  // nothing of this sub-tile is visible to the rows of this wavefront
         }
@@ -426,17 +452,27 @@ __global__ __launch_bounds__(256, 2) void hstu_bwd_dq_kernel(const BwdArgs a)
         for (int c = 0; c < NCH; ++c) {
             const int j2 = c / MTILES, mt = c % MTILES;
             const u32x4_t pb = {pk[4 * j2 + 0], pk[4 * j2 + 1], pk[4 * j2 + 2], pk[4 * j2 + 3]};
-            dq_acc[mt] = mfma32<Tag>(read_t(kt, c), pb, dq_acc[mt]);
+            dq_acc[mt] = mfma32<Tag>(read_t(kn, c), pb, dq_acc[mt]);
         }
     };
 
     if (n_sub > 0) {
-        request(s_kn0, s_kt0, s_vn0, 0);
-    }
-    for (int x = 0; x < n_sub; x += 2) {
-        step(s_kn0, s_kt0, s_vn0, s_kn1, s_kt1, s_vn1, x);
-        if (x + 1 < n_sub) {
-            step(s_kn1, s_kt1, s_vn1, s_kn0, s_kt0, s_vn0, x + 1);
+        request(s_k0, s_v0, 0);
+        request(s_k1, s_v1, 1);
+        int x = 0;
+        while (true) {  // (step x reads stage x mod 3 and has stage (x + 2) mod 3 filled)
+            step(s_k0, s_v0, s_k2, s_v2, x);
+            if (++x >= n_sub) {
+                break;
+            }
+            step(s_k1, s_v1, s_k0, s_v0, x);
+            if (++x >= n_sub) {
+                break;
+            }
+            step(s_k2, s_v2, s_k1, s_v1, x);
+            if (++x >= n_sub) {
+                break;
+            }
         }
     }
 
@@ -461,23 +497,30 @@ __global__ __launch_bounds__(256, 2) void hstu_bwd_dq_kernel(const BwdArgs a)
 // ---------------------------------------------------------------------------------------------------------
 // dK, dV
 // ---------------------------------------------------------------------------------------------------------
+constexpr int kDkvThreads = 512;
+
 template <typename Tag, int D, bool HAS_RAB, bool HAS_MASK>
-__global__ __launch_bounds__(256, 1) void hstu_bwd_dkv_kernel(const BwdArgs a)
+__global__ __launch_bounds__(kDkvThreads, 1) void hstu_bwd_dkv_kernel(const BwdArgs a)
 {
     typedef SubTile<D> T;
     constexpr int LPW = T::LPW, NLW = T::NLW, KSTEPS = T::KSTEPS, MTILES = T::MTILES, NCH = 2 * T::MTILES;
-    __shared__ __attribute__((aligned(1024))) uint16_t s_qn0[T::ELEMS];  // Q, plain / transposed layouts
-    __shared__ __attribute__((aligned(1024))) uint16_t s_qn1[T::ELEMS];
-    __shared__ __attribute__((aligned(1024))) uint16_t s_qt0[T::ELEMS];
-    __shared__ __attribute__((aligned(1024))) uint16_t s_qt1[T::ELEMS];
-    __shared__ __attribute__((aligned(1024))) uint16_t s_gn0[T::ELEMS];  // dO, plain / transposed layouts
-    __shared__ __attribute__((aligned(1024))) uint16_t s_gn1[T::ELEMS];
-    __shared__ __attribute__((aligned(1024))) uint16_t s_gt0[T::ELEMS];
-    __shared__ __attribute__((aligned(1024))) uint16_t s_gt1[T::ELEMS];
+    // four stages, each the Q sub-tile followed by the dO sub-tile (separate arrays per stage, see the dQ kernel;
+    // Q and dO of a stage share an array so that a wavefront can address "the tile of my role" by an offset)
+    __shared__ __attribute__((aligned(1024))) uint16_t s_st0[2 * T::ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_st1[2 * T::ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_st2[2 * T::ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_st3[2 * T::ELEMS];
+    // a sub-tile is requested three steps ahead: the requests of two later steps may be outstanding at a step's start
+    constexpr int kReqs = 2 * LPW;
+    constexpr int kWaitStage = (kReqs & 15) | (7 << 4) | (15 << 8) | ((kReqs >> 4) << 14);
+    constexpr uint32_t kPastEnd = 0x40000000u;
+    static_assert(NLW == 4, "every wavefront takes part in the loads");
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave = uniform(tid >> 6);
+    const int wave8 = uniform(tid >> 6);
+    const bool dk_role = wave8 >= 4;  // wavefronts 0..3 produce dV, 4..7 dK; w and w + 4 share keys (and a SIMD)
+    const int wave = wave8 & 3;
     const int ln = lane & 31;
     const int lh = lane >> 5;
 
@@ -506,42 +549,46 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dkv_kernel(const BwdArgs a)
     const __amdgpu_buffer_rsrc_t v_rsrc =
         make_rsrc(static_cast<const uint8_t*>(a.v) + (si.k0 * a.n_heads_k + hk) * static_cast<int64_t>(a.d_v) * 2,
                   static_cast<uint32_t>(sk - 1) * v_stride + a.d_v * 2u);
-    const __amdgpu_buffer_rsrc_t dk_rsrc =
-        make_rsrc(static_cast<uint8_t*>(a.dk) + (si.k0 * a.n_heads_k + hk) * static_cast<int64_t>(a.d_qk) * 2,
-                  static_cast<uint32_t>(sk - 1) * k_stride + a.d_qk * 2u);
-    const __amdgpu_buffer_rsrc_t dv_rsrc =
-        make_rsrc(static_cast<uint8_t*>(a.dv) + (si.k0 * a.n_heads_k + hk) * static_cast<int64_t>(a.d_v) * 2,
-                  static_cast<uint32_t>(sk - 1) * v_stride + a.d_v * 2u);
+    // the output of this wavefront's role
+    const uint32_t out_stride = dk_role ? k_stride : v_stride;
+    const int out_dim = dk_role ? a.d_qk : a.d_v;
+    const __amdgpu_buffer_rsrc_t out_rsrc =
+        make_rsrc(static_cast<uint8_t*>(dk_role ? a.dk : a.dv) + (si.k0 * a.n_heads_k + hk) * static_cast<int64_t>(out_dim) * 2,
+                  static_cast<uint32_t>(sk - 1) * out_stride + static_cast<uint32_t>(out_dim) * 2u);
 
-    uint32_t qn_src[LPW], qt_src[LPW], gn_src[LPW], gt_src[LPW];
+    // the dV wavefronts fill the Q half of a stage, the dK wavefronts the dO half: one set of per-lane source
+    // offsets per wavefront, for the tensor it loads
+    const uint32_t ld_stride = dk_role ? g_stride : q_stride;
+    const int ld_dim = dk_role ? a.d_v : a.d_qk;
+    const int ld_half = dk_role ? T::ELEMS : 0;
+    uint32_t ld_src[LPW];
 #pragma unroll
     for (int i = 0; i < LPW; ++i) {
         const int slot = (wave * LPW + i) * 64 + lane;
         const int r = (slot / T::CPR) & 31;
         const int pc = slot % T::CPR;
-        const int cn = k_chunk_swizzle<D>(r, pc);
-        const int ct = v_chunk_swizzle<D>(r, pc);
-        qn_src[i] = (cn * 8 < a.d_qk) ? static_cast<uint32_t>(r) * q_stride + cn * 16u : kOutOfRange;
-        qt_src[i] = (ct * 8 < a.d_qk) ? static_cast<uint32_t>(r) * q_stride + ct * 16u : kOutOfRange;
-        gn_src[i] = (cn * 8 < a.d_v) ? static_cast<uint32_t>(r) * g_stride + cn * 16u : kOutOfRange;
-        gt_src[i] = (ct * 8 < a.d_v) ? static_cast<uint32_t>(r) * g_stride + ct * 16u : kOutOfRange;
+        const int cs = both_ways_swizzle<D>(r, pc);
+        ld_src[i] = (cs * 8 < ld_dim) ? static_cast<uint32_t>(r) * ld_stride + cs * 16u : kOutOfRange;
     }
     int n_lane_off[KSTEPS];
-    int t_lane_off[MTILES];
+    int t_lane_off[MTILES][2];
 #pragma unroll
     for (int js = 0; js < KSTEPS; ++js) {
-        n_lane_off[js] = ln * D + k_chunk_swizzle<D>(ln, 2 * js + lh) * 8;
+        n_lane_off[js] = ln * D + both_ways_swizzle<D>(ln, 2 * js + lh) * 8;
     }
     {
         const int vr0 = 4 * lh + ((lane & 15) >> 2);
+        // the transposed operand of this role: Q^T (first half of a stage) for dK, dO^T (second half) for dV
+        const int role_half = dk_role ? 0 : T::ELEMS;
 #pragma unroll
         for (int mt = 0; mt < MTILES; ++mt) {
             const int col = 32 * mt + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-            t_lane_off[mt] = vr0 * D + v_chunk_swizzle<D>(vr0, col >> 3) * 8 + (col & 7);
+            t_lane_off[mt][0] = role_half + vr0 * D + both_ways_swizzle<D>(vr0, col >> 3) * 8 + (col & 7);
+            t_lane_off[mt][1] = role_half + (vr0 + 8) * D + both_ways_swizzle<D>(vr0 + 8, col >> 3) * 8 + (col & 7);
         }
     }
 
-    // resident rows: K and V fragments of this lane's key
+    // resident rows: K (both roles) and V (dK role) fragments of this lane's key
     u32x4_t kf[KSTEPS], vf[KSTEPS];
     {
         const uint32_t k_off = static_cast<uint32_t>(key) * k_stride;
@@ -550,7 +597,7 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dkv_kernel(const BwdArgs a)
         for (int js = 0; js < KSTEPS; ++js) {
             const int d0 = 16 * js + 8 * lh;
             kf[js] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, static_cast<int>(d0 < a.d_qk ? k_off + d0 * 2u : kOutOfRange), 0, 0);
-            vf[js] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, static_cast<int>(d0 < a.d_v ? v_off + d0 * 2u : kOutOfRange), 0, 0);
+            vf[js] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, static_cast<int>(dk_role && d0 < a.d_v ? v_off + d0 * 2u : kOutOfRange), 0, 0);
         }
     }
 
@@ -564,13 +611,12 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dkv_kernel(const BwdArgs a)
     const int nx = n_qsub > x_first ? n_qsub - x_first : 0;
     const int n_iter = nx * a.head_ratio;  // (query head of the group, query sub-tile), head-major
 
-    f32x16_t dk_acc[MTILES], dv_acc[MTILES];
+    f32x16_t acc[MTILES];  // dK^T or dV^T of this wavefront's keys, by role
 #pragma unroll
     for (int mt = 0; mt < MTILES; ++mt) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
-            dk_acc[mt][i] = 0.f;
-            dv_acc[mt][i] = 0.f;
+            acc[mt][i] = 0.f;
         }
     }
     const float c_exp = -a.alpha * 1.4426950408889634f;
@@ -578,159 +624,187 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_dkv_kernel(const BwdArgs a)
     const uint32_t bias_bytes = static_cast<uint32_t>(a.max_q) * static_cast<uint32_t>(a.max_k) * 2u;
     const bool targets = a.mask_type == 0 && si.n_tgt > 0 && a.target_group > 0;
 
-    auto head_of = [&](int it) -> int { return hk * a.head_ratio + it / nx; };
-    auto sub_of = [&](int it) -> int { return x_first + it % nx; };
-    auto request = [&](uint16_t* qn, uint16_t* qt, uint16_t* gn, uint16_t* gt, int it) {
-        if (NLW == 4 || wave < NLW) {
-            const int h = head_of(it);
-            const int x = sub_of(it);
-            const __amdgpu_buffer_rsrc_t q_rsrc =
-                make_rsrc(static_cast<const uint8_t*>(a.q) + (si.q0 * a.n_heads_q + h) * static_cast<int64_t>(a.d_qk) * 2,
-                          static_cast<uint32_t>(sq - 1) * q_stride + a.d_qk * 2u);
-            const __amdgpu_buffer_rsrc_t g_rsrc =
-                make_rsrc(static_cast<const uint8_t*>(a.grad) + (si.q0 * a.n_heads_q + h) * static_cast<int64_t>(a.d_v) * 2,
-                          static_cast<uint32_t>(sq - 1) * g_stride + a.d_v * 2u);
-            const uint32_t qb = static_cast<uint32_t>(x * 32) * q_stride;
-            const uint32_t gb = static_cast<uint32_t>(x * 32) * g_stride;
+    // head and sub-tile of iteration it, kept incrementally (no division in the loop)
+    int req_h = hk * a.head_ratio, req_x = x_first, req_it = 0;  // next request
+    int cur_h = hk * a.head_ratio, cur_x = x_first;              // current step
+    auto request = [&](uint16_t* stage) {
+        const bool past = req_it >= n_iter;  // (sent out of range: moves no data, keeps the count per step constant)
+        const uint8_t* const ld_base = static_cast<const uint8_t*>(dk_role ? a.grad : a.q);
+        const __amdgpu_buffer_rsrc_t ld_rsrc =
+            make_rsrc(ld_base + (si.q0 * a.n_heads_q + req_h) * static_cast<int64_t>(ld_dim) * 2,
+                      static_cast<uint32_t>(sq - 1) * ld_stride + static_cast<uint32_t>(ld_dim) * 2u);
+        const uint32_t base = past ? kPastEnd : static_cast<uint32_t>(req_x * 32) * ld_stride;
 #pragma unroll
-            for (int i = 0; i < LPW; ++i) {
-                load_to_lds_b128(q_rsrc, qn + (wave * LPW + i) * 512, qn_src[i] + qb);
-                load_to_lds_b128(q_rsrc, qt + (wave * LPW + i) * 512, qt_src[i] + qb);
-                load_to_lds_b128(g_rsrc, gn + (wave * LPW + i) * 512, gn_src[i] + gb);
-                load_to_lds_b128(g_rsrc, gt + (wave * LPW + i) * 512, gt_src[i] + gb);
+        for (int i = 0; i < LPW; ++i) {
+            load_to_lds_b128(ld_rsrc, stage + ld_half + (wave * LPW + i) * 512, ld_src[i] + base);
+        }
+        ++req_it;
+        if (++req_x >= n_qsub) {
+            req_x = x_first;
+            if (!past && req_it < n_iter) {
+                ++req_h;
             }
         }
     };
     auto read_n = [&](const uint16_t* tile, int js) -> u32x4_t {
         return *reinterpret_cast<const u32x4_t*>(tile + n_lane_off[js]);
     };
-    auto read_t = [&](const uint16_t* tile, int c) -> u32x4_t {
+    auto read_t = [&](const uint16_t* stage, int c) -> u32x4_t {
         const int j2 = c / MTILES, mt = c % MTILES;
-        const uint16_t* p = tile + t_lane_off[mt] + 16 * j2 * D;
-        const u32x2_t lo = lds_read_tr16_b64(p);
-        const u32x2_t hi = lds_read_tr16_b64(p + 8 * D);
+        const u32x2_t lo = lds_read_tr16_b64(stage + t_lane_off[mt][0] + 16 * j2 * D);
+        const u32x2_t hi = lds_read_tr16_b64(stage + t_lane_off[mt][1] + 16 * j2 * D);
         const u32x4_t r = {lo[0], lo[1], hi[0], hi[1]};
         return r;
     };
 
-    auto step = [&](const uint16_t* qn, const uint16_t* qt, const uint16_t* gn, const uint16_t* gt, uint16_t* qn_o,
-                    uint16_t* qt_o, uint16_t* gn_o, uint16_t* gt_o, int it) {
-        __builtin_amdgcn_s_waitcnt(0);
-        __syncthreads();
-        if (it + 1 < n_iter) {
-            request(qn_o, qt_o, gn_o, gt_o, it + 1);
+    auto step = [&](const uint16_t* stage, uint16_t* stage_o) {
+        // this step's sub-tile has landed for everybody; the stage of the previous step is free (see the dQ kernel)
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(kWaitStage);
+        __builtin_amdgcn_s_barrier();
+        __builtin_amdgcn_sched_barrier(0);
+        request(stage_o);
+        const int h = cur_h;
+        const int rq0 = cur_x * 32;  // first query row of the sub-tile
+        if (++cur_x >= n_qsub) {
+            cur_x = x_first;
+            ++cur_h;
         }
-        const int h = head_of(it);
-        const int x = sub_of(it);
-        const int rq0 = x * 32;  // first query row of the sub-tile
         // whole block hidden from the keys of this wavefront?  (rows rq0 .. rq0 + 31, keys cw0 .. cw0 + 31)
+        bool active = cw0 < sk;
         if (a.mask_type == 0) {
             int lim_max = rq0 + 32 + si.delta;  // lim of the last row
             if (rq0 < si.n_ctx) {
                 lim_max = lim_max > si.hist_k ? lim_max : si.hist_k;
             }
-            if (cw0 >= lim_max) {
-                return;
+            active = active && cw0 < lim_max;
+        }
+        if (active) {
+            f32x16_t s, dp;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                s[i] = 0.f;
+                dp[i] = 0.f;
             }
-        }
-        if (cw0 >= sk) {
-            return;
-        }
-        f32x16_t s, dp;
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            s[i] = 0.f;
-            dp[i] = 0.f;
-        }
+            for (int js = 0; js < KSTEPS; ++js) {
+                s = mfma32<Tag>(read_n(stage, js), kf[js], s);
+            }
+            if (dk_role) {
 #pragma unroll
-        for (int js = 0; js < KSTEPS; ++js) {
-            s = mfma32<Tag>(read_n(qn, js), kf[js], s);
-            dp = mfma32<Tag>(read_n(gn, js), vf[js], dp);
-        }
-        // fully visible block: every row's lim is past the last key, no context / target effects
-        bool full = a.mask_type != 0;
-        if (a.mask_type == 0) {
-            full = (cw0 + 32 <= rq0 + si.delta + 1) && (cw0 + 32 <= sk) && (rq0 + 32 <= sq) &&
-                   !(targets && rq0 + 31 >= sq - si.n_tgt);
-        }
-        const __amdgpu_buffer_rsrc_t rab_rsrc = make_rsrc(
-            HAS_RAB ? static_cast<const uint16_t*>(a.rab) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k) : nullptr,
-            HAS_RAB ? bias_bytes : 0u);
-        const __amdgpu_buffer_rsrc_t mask_rsrc = make_rsrc(
-            HAS_MASK ? static_cast<const uint16_t*>(a.mask) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k) : nullptr,
-            HAS_MASK ? bias_bytes : 0u);
-        uint32_t p_pk[8], ds_pk[8];
+                for (int js = 0; js < KSTEPS; ++js) {
+                    dp = mfma32<Tag>(read_n(stage + T::ELEMS, js), vf[js], dp);
+                }
+            }
+            // fully visible block: every row's lim is past the last key, no context / target effects, all in range
+            bool full = (cw0 + 32 <= sk) && (rq0 + 32 <= sq);
+            if (a.mask_type == 0) {
+                full = full && (cw0 + 32 <= rq0 + si.delta + 1) && !(targets && rq0 + 31 >= sq - si.n_tgt);
+            }
+            const __amdgpu_buffer_rsrc_t rab_rsrc = make_rsrc(
+                HAS_RAB ? static_cast<const uint16_t*>(a.rab) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k) : nullptr,
+                HAS_RAB ? bias_bytes : 0u);
+            const __amdgpu_buffer_rsrc_t mask_rsrc = make_rsrc(
+                HAS_MASK ? static_cast<const uint16_t*>(a.mask) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k) : nullptr,
+                HAS_MASK ? bias_bytes : 0u);
+            // X and the custom mask value of every element, then the role's own function of it
+            float xs[16], ms[16];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            float p2[2], ds2[2];
-#pragma unroll
-            for (int e2 = 0; e2 < 2; ++e2) {
-                const int e = 2 * i + e2;
+            for (int e = 0; e < 16; ++e) {
                 const int r = rq0 + 8 * (e / 4) + 4 * lh + (e % 4);  // query row of this element
-                float sv = s[e];
-                const uint32_t boff = (r < sq && key < a.max_k)
-                                          ? (static_cast<uint32_t>(r) * static_cast<uint32_t>(a.max_k) + static_cast<uint32_t>(key)) * 2u
-                                          : kOutOfRange;
-                if constexpr (HAS_RAB) {
-                    const uint32_t raw = __builtin_amdgcn_raw_buffer_load_b16(rab_rsrc, static_cast<int>(boff), 0, 0);
-                    sv += lo_to_float<Tag>(raw & 0xffffu);
+                xs[e] = s[e];
+                ms[e] = 1.0f;
+                if constexpr (HAS_RAB || HAS_MASK) {
+                    const uint32_t boff = (r < sq && key < a.max_k)
+                                              ? (static_cast<uint32_t>(r) * static_cast<uint32_t>(a.max_k) + static_cast<uint32_t>(key)) * 2u
+                                              : kOutOfRange;
+                    if constexpr (HAS_RAB) {
+                        const uint32_t raw = __builtin_amdgcn_raw_buffer_load_b16(rab_rsrc, static_cast<int>(boff), 0, 0);
+                        xs[e] += lo_to_float<Tag>(raw & 0xffffu);
+                    }
+                    if constexpr (HAS_MASK) {
+                        const uint32_t raw = __builtin_amdgcn_raw_buffer_load_b16(mask_rsrc, static_cast<int>(boff), 0, 0);
+                        ms[e] = lo_to_float<Tag>(raw & 0xffffu);
+                    }
                 }
-                float p, ds;
-                score_grad(sv, dp[e], a.alpha, c_exp, a.scale, ascale, p, ds);
-                if constexpr (HAS_MASK) {
-                    const uint32_t raw = __builtin_amdgcn_raw_buffer_load_b16(mask_rsrc, static_cast<int>(boff), 0, 0);
-                    const float m = lo_to_float<Tag>(raw & 0xffffu);
-                    p *= m;
-                    ds *= m;
+            }
+            float o[16];
+            if (dk_role) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    float p, ds;
+                    score_grad(xs[e], dp[e], a.alpha, c_exp, a.scale, ascale, p, ds);
+                    o[e] = ds * ms[e];
                 }
-                bool vis = true;
-                if (!full) {
+            } else {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const float sig = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(xs[e] * c_exp));
+                    o[e] = xs[e] * sig * ascale * ms[e];  // P = X sig scale, X = alpha (S + rab)
+                }
+            }
+            if (!full) {
+#pragma unroll
+                for (int e = 0; e < 16; ++e) {
+                    const int r = rq0 + 8 * (e / 4) + 4 * lh + (e % 4);
                     int lim, hole_lo, hole_hi;
                     row_bounds(si, a.mask_type, a.target_group, r, lim, hole_lo, hole_hi);
-                    vis = (r < sq) && (key < lim) && !(key >= hole_lo && key < hole_hi);
+                    const bool vis = (r < sq) && (key < lim) && !(key >= hole_lo && key < hole_hi);
+                    o[e] = vis ? o[e] : 0.f;
                 }
-                p2[e2] = vis ? p : 0.f;
-                ds2[e2] = vis ? ds : 0.f;
             }
-            p_pk[i] = pack2<Tag>(p2[0], p2[1]);
-            ds_pk[i] = pack2<Tag>(ds2[0], ds2[1]);
-        }
+            uint32_t pk[8];  // P (dV role) or dS (dK role), B operand of the output product
 #pragma unroll
-        for (int c = 0; c < NCH; ++c) {
-            const int j2 = c / MTILES, mt = c % MTILES;
-            const u32x4_t pb = {p_pk[4 * j2 + 0], p_pk[4 * j2 + 1], p_pk[4 * j2 + 2], p_pk[4 * j2 + 3]};
-            const u32x4_t db = {ds_pk[4 * j2 + 0], ds_pk[4 * j2 + 1], ds_pk[4 * j2 + 2], ds_pk[4 * j2 + 3]};
-            dv_acc[mt] = mfma32<Tag>(read_t(gt, c), pb, dv_acc[mt]);
-            dk_acc[mt] = mfma32<Tag>(read_t(qt, c), db, dk_acc[mt]);
+            for (int i = 0; i < 8; ++i) {
+                pk[i] = pack2<Tag>(o[2 * i], o[2 * i + 1]);
+            }
+            // dK^T += Q^T . dS  or  dV^T += dO^T . P: the transposed operand sits in the role's half of the stage
+#pragma unroll
+            for (int c = 0; c < NCH; ++c) {
+                const int j2 = c / MTILES, mt = c % MTILES;
+                const u32x4_t pb = {pk[4 * j2 + 0], pk[4 * j2 + 1], pk[4 * j2 + 2], pk[4 * j2 + 3]};
+                acc[mt] = mfma32<Tag>(read_t(stage, c), pb, acc[mt]);
+            }
         }
     };
 
     if (n_iter > 0) {
-        request(s_qn0, s_qt0, s_gn0, s_gt0, 0);
-    }
-    for (int it = 0; it < n_iter; it += 2) {
-        step(s_qn0, s_qt0, s_gn0, s_gt0, s_qn1, s_qt1, s_gn1, s_gt1, it);
-        if (it + 1 < n_iter) {
-            step(s_qn1, s_qt1, s_gn1, s_gt1, s_qn0, s_qt0, s_gn0, s_gt0, it + 1);
+        request(s_st0);
+        request(s_st1);
+        request(s_st2);
+        int it = 0;
+        while (true) {  // (step it reads stage it mod 4 and has stage (it + 3) mod 4 filled)
+            step(s_st0, s_st3);
+            if (++it >= n_iter) {
+                break;
+            }
+            step(s_st1, s_st0);
+            if (++it >= n_iter) {
+                break;
+            }
+            step(s_st2, s_st1);
+            if (++it >= n_iter) {
+                break;
+            }
+            step(s_st3, s_st2);
+            if (++it >= n_iter) {
+                break;
+            }
         }
     }
 
-    // store dK, dV: lane holds key (cw0 + ln), dims 32*mt + 8*g + 4*lh + 0..3
+    // store dK or dV: lane holds key (cw0 + ln), dims 32*mt + 8*g + 4*lh + 0..3
     {
-        const uint32_t k_off = static_cast<uint32_t>(key) * k_stride;
-        const uint32_t v_off = static_cast<uint32_t>(key) * v_stride;
+        const uint32_t row_off = static_cast<uint32_t>(key) * out_stride;
 #pragma unroll
         for (int mt = 0; mt < MTILES; ++mt) {
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 const int d0 = 32 * mt + 8 * g + 4 * lh;
                 u32x2_t w;
-                w[0] = pack2<Tag>(dk_acc[mt][4 * g + 0], dk_acc[mt][4 * g + 1]);
-                w[1] = pack2<Tag>(dk_acc[mt][4 * g + 2], dk_acc[mt][4 * g + 3]);
-                __builtin_amdgcn_raw_buffer_store_b64(w, dk_rsrc, static_cast<int>(d0 < a.d_qk ? k_off + d0 * 2u : kOutOfRange), 0, 0);
-                w[0] = pack2<Tag>(dv_acc[mt][4 * g + 0], dv_acc[mt][4 * g + 1]);
-                w[1] = pack2<Tag>(dv_acc[mt][4 * g + 2], dv_acc[mt][4 * g + 3]);
-                __builtin_amdgcn_raw_buffer_store_b64(w, dv_rsrc, static_cast<int>(d0 < a.d_v ? v_off + d0 * 2u : kOutOfRange), 0, 0);
+                w[0] = pack2<Tag>(acc[mt][4 * g + 0], acc[mt][4 * g + 1]);
+                w[1] = pack2<Tag>(acc[mt][4 * g + 2], acc[mt][4 * g + 3]);
+                __builtin_amdgcn_raw_buffer_store_b64(w, out_rsrc, static_cast<int>(d0 < out_dim ? row_off + d0 * 2u : kOutOfRange), 0, 0);
             }
         }
     }

@@ -484,7 +484,8 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
         return fail(HSTU_ERR_INVALID, "grid out of range");
     }
     if (f->total_k > 0 && grid_kv > 0) {
-        hipLaunchKernelGGL(var->dkv, dim3(static_cast<unsigned>(grid_kv)), dim3(256), 0, static_cast<hipStream_t>(stream), a);
+        hipLaunchKernelGGL(var->dkv, dim3(static_cast<unsigned>(grid_kv)), dim3(hstu::kDkvThreads), 0,
+                           static_cast<hipStream_t>(stream), a);
     }
     if (f->total_q > 0 && grid_q > 0) {
         hipLaunchKernelGGL(p->grad_attn_bias != nullptr ? var->dq_drab : var->dq, dim3(static_cast<unsigned>(grid_q)), dim3(256),
