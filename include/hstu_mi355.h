@@ -145,8 +145,8 @@ HSTU_API int hstu_jagged_fwd(const hstu_jagged_fwd_params* params, void* workspa
  * `fwd` describes q, k, v, mask, attn_bias, the offsets and the scalars exactly as for the forward (fwd.out is
  * not used and may be NULL).  Built for bf16 / fp16 with head dims up to 128 (q/k head dim a multiple of 8);
  * other valid descriptions return HSTU_ERR_UNSUPPORTED.
- * grad_q / grad_k / grad_v: every row inside a sequence is written; rows past the last offset are not (clear
- * them beforehand if they are read).  grad_attn_bias (optional; requires attn_bias): only the elements inside a
+ * grad_q / grad_k / grad_v: every row is written (rows past the last offset are zero-filled), so the caller
+ * need not clear them.  grad_attn_bias (optional; requires attn_bias): only the elements inside a
  * sequence's [S_q, S_k] corner that a query tile sweeps are written -- the caller clears the tensor beforehand. */
 typedef struct hstu_jagged_bwd_params {
     uint32_t struct_size; /* sizeof(hstu_jagged_bwd_params) */

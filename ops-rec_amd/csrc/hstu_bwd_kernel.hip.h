@@ -112,6 +112,20 @@ __device__ __forceinline__ SeqInfo load_seq(const BwdArgs& a, int b)
     return s;
 }
 
+// rows past the last offset belong to no sequence: zero-fill them (all workgroups of a launch share the job)
+__device__ __forceinline__ void zero_tail_rows(void* out, const void* offs, int n_batch, int idx64, int64_t total,
+                                               int64_t row_elems, int threads)
+{
+    const int64_t last = load_index_uniform(offs, n_batch, idx64);
+    const int64_t first_tail = last < 0 ? 0 : (last < total ? last : total);
+    const int64_t n_tail = (total - first_tail) * row_elems;
+    uint16_t* const tail = static_cast<uint16_t*>(out) + first_tail * row_elems;
+    for (int64_t e = static_cast<int64_t>(blockIdx.x) * threads + threadIdx.x; e < n_tail;
+         e += static_cast<int64_t>(gridDim.x) * threads) {
+        tail[e] = 0;
+    }
+}
+
 // first key hidden from query row r by the causal / context rule, and the hole the grouped targets cut out
 __device__ __forceinline__ void row_bounds(const SeqInfo& s, int mask_type, int group, int r, int& lim, int& hole_lo,
                                            int& hole_hi)
@@ -216,6 +230,7 @@ __global__ __launch_bounds__(256, 2) void hstu_bwd_dq_kernel(const BwdArgs a)
     const int b = rem / a.n_heads_q;
     const int h = rem - b * a.n_heads_q;
     const int hk = h / a.head_ratio;
+    zero_tail_rows(a.dq, a.offs_q, a.n_batch, a.idx64, a.total_q, static_cast<int64_t>(a.n_heads_q) * a.d_qk, 256);
     const SeqInfo sq_info = load_seq(a, b);
     const int sq = sq_info.sq, sk = sq_info.sk;
     const int r0 = qt * kBlockM;
@@ -530,6 +545,8 @@ __global__ __launch_bounds__(kDkvThreads, 1) void hstu_bwd_dkv_kernel(const BwdA
     const int rem = static_cast<int>(blockIdx.x) - kt_idx * per_level;
     const int b = rem / a.n_heads_k;
     const int hk = rem - b * a.n_heads_k;
+    zero_tail_rows(a.dk, a.offs_k, a.n_batch, a.idx64, a.total_k, static_cast<int64_t>(a.n_heads_k) * a.d_qk, kDkvThreads);
+    zero_tail_rows(a.dv, a.offs_k, a.n_batch, a.idx64, a.total_k, static_cast<int64_t>(a.n_heads_k) * a.d_v, kDkvThreads);
     const SeqInfo si = load_seq(a, b);
     const int sq = si.sq, sk = si.sk;
     const int c0 = kt_idx * kBlockM;

@@ -362,9 +362,9 @@ def _backward_hip(grad, q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max_
         _check(mask is not None and mask.dtype == q.dtype and tuple(mask.shape) == bias_shape,
                f"mask must be {bias_shape} of q's dtype")  # fmt: skip
         mask_c = mask.contiguous()
-    # rows past the last offset belong to no sequence and are not written by the kernels; the bias gradient is
-    # written only where a query tile sweeps
-    dq, dk, dv = torch.zeros_like(q_c), torch.zeros_like(k_c), torch.zeros_like(v_c)
+    # every row of dq / dk / dv is written by the kernels (rows past the last offset are zero-filled there); the
+    # bias gradient is written only where a query tile sweeps
+    dq, dk, dv = torch.empty_like(q_c), torch.empty_like(k_c), torch.empty_like(v_c)
     dbias = torch.zeros_like(bias) if bias is not None else None
     if q_c.numel() == 0 and k_c.numel() == 0:
         return dq, dk, dv, dbias
