@@ -162,6 +162,41 @@ typedef struct hstu_jagged_bwd_params {
 HSTU_API int hstu_jagged_bwd_workspace_size(const hstu_jagged_bwd_params* params, uint64_t* workspace_bytes);
 HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* params, void* workspace, uint64_t workspace_bytes, void* stream);
 
+/* ---- paged K/V ---------------------------------------------------------------------------------------
+ * Replaces the pair the reference's adapter binds for hstu_paged (inference with a paged KV cache):
+ *
+ *   aclnnHstuPagedForward[GetWorkspaceSize](q, k, v, mask, attnBias, seqOffset, seqOffsetK, seqOffsetT, kvCache,
+ *        pageOffsets, pageIds, lastPageLen, numContext, numTarget, maskType, maxSeqLen, maxSeqLenK, siluScale,
+ *        targetGroupSize, alpha, deterministic, attnOutput)
+ *   called from  ascendc/attention/hstu_v1/torch_extension/hstu_paged_plugin.cpp:66-69
+ *
+ * The keys / values of sequence b are its cached rows -- the pages page_ids[page_offsets[b] .. page_offsets[b+1])
+ * of kv_cache [num_pages, 2 (K, V), page_size, num_heads_k, head_dim], in order -- followed by the rows of its
+ * num_target[b] new target tokens, which are the LAST num_target[b] rows of its segment [seq_offset_q[b],
+ * seq_offset_q[b+1]) of the k / v inputs (the other rows of k / v are not read).  fwd.seq_offset_k gives the
+ * resulting key ranges (cached + targets per sequence) and fwd.total_k an upper bound on their end
+ * (page_ids count x page_size + total_q is always enough); fwd.k / fwd.v are the inputs with total_q rows;
+ * fwd.num_context is ignored (zeros, as in the reference adapter); everything else as in the forward.
+ * Implementation: the library gathers the rows into the workspace (one copy kernel), then runs the jagged forward
+ * on them, so the workspace is 2 x total_k rows (plus what the forward asks for).  last_page_len and seq_offset_t
+ * are taken for signature parity; the number of cached rows of a sequence is its key count minus its targets. */
+typedef struct hstu_paged_fwd_params {
+    uint32_t struct_size; /* sizeof(hstu_paged_fwd_params) */
+    uint32_t reserved0;
+    hstu_jagged_fwd_params fwd;
+    const void* kv_cache;      /* dtype of q */
+    const void* page_offsets;  /* [n_offsets], index dtype */
+    const void* page_ids;      /* [n_page_ids] */
+    const void* last_page_len; /* [n_offsets - 1]; may be NULL */
+    const void* seq_offset_t;  /* [n_offsets]; may be NULL */
+    int64_t num_pages;
+    int64_t page_size;
+    int64_t n_page_ids;
+} hstu_paged_fwd_params;
+
+HSTU_API int hstu_paged_fwd_workspace_size(const hstu_paged_fwd_params* params, uint64_t* workspace_bytes);
+HSTU_API int hstu_paged_fwd(const hstu_paged_fwd_params* params, void* workspace, uint64_t workspace_bytes, void* stream);
+
 /* replaces aclGetRecentErrMsg (ascendc/common/torch_plugin/pytorch_npu_helper.hpp:649,662):
  * text of the calling thread's most recent failure; never NULL. */
 HSTU_API const char* hstu_last_error(void);

@@ -18,6 +18,7 @@
 #include "hstu_fwd_f32_kernel.hip.h"
 #include "hstu_bwd_kernel.hip.h"
 #include "hstu_fwd_kernel.hip.h"
+#include "hstu_paged_gather.hip.h"
 
 namespace {
 
@@ -407,9 +408,127 @@ const BwdVariant* select_bwd(const hstu_jagged_bwd_params* p)
                         [f->mask_type == HSTU_MASK_CUSTOM ? 1 : 0][dmax <= 64 ? 0 : 1];
 }
 
+// ---- paged K/V --------------------------------------------------------------------------------------------
+uint64_t round_up_256(uint64_t x) { return (x + 255u) & ~static_cast<uint64_t>(255u); }
+
+int validate_paged(const hstu_paged_fwd_params* p, hstu_jagged_fwd_params* gathered, uint64_t* region_bytes)
+{
+    if (p == nullptr) {
+        return fail(HSTU_ERR_NULLPTR, "params is NULL");
+    }
+    if (p->struct_size != sizeof(hstu_paged_fwd_params)) {
+        return fail(HSTU_ERR_INVALID, "struct_size %u does not match this library (%zu)", p->struct_size,
+                    sizeof(hstu_paged_fwd_params));
+    }
+    const int rc = validate(&p->fwd);
+    if (rc != HSTU_OK) {
+        return rc;
+    }
+    if (p->kv_cache == nullptr || p->page_offsets == nullptr || p->page_ids == nullptr) {
+        return fail(HSTU_ERR_NULLPTR, "kv_cache / page_offsets / page_ids must not be NULL");
+    }
+    if (p->page_size != 32 && p->page_size != 64 && p->page_size != 128 && p->page_size != 256) {
+        return fail(HSTU_ERR_INVALID, "page_size must be 32, 64, 128 or 256, but value is %lld", (long long)p->page_size);
+    }
+    if (p->num_pages < 1 || p->n_page_ids < 1) {
+        return fail(HSTU_ERR_INVALID, "kv_cache and page_ids must not be empty");
+    }
+    if (p->fwd.dtype == HSTU_DT_FP8_E4M3) {
+        fail(HSTU_ERR_UNSUPPORTED, "paged K/V is not built for fp8 inputs");
+        return HSTU_ERR_UNSUPPORTED;
+    }
+    if (p->fwd.head_dim_qk != p->fwd.head_dim_v) {
+        return fail(HSTU_ERR_INVALID, "the cache holds K and V rows of one head dim, but q/k has %lld and v has %lld",
+                    (long long)p->fwd.head_dim_qk, (long long)p->fwd.head_dim_v);
+    }
+    const uint64_t esize = p->fwd.dtype == HSTU_DT_FP32 ? 4 : 2;
+    const uint64_t row_bytes = static_cast<uint64_t>(p->fwd.num_heads_k) * p->fwd.head_dim_qk * esize;
+    if (row_bytes % 16 != 0) {
+        fail(HSTU_ERR_UNSUPPORTED, "a K/V row of %llu bytes is not a multiple of 16", (unsigned long long)row_bytes);
+        return HSTU_ERR_UNSUPPORTED;
+    }
+    *region_bytes = round_up_256(static_cast<uint64_t>(p->fwd.total_k) * row_bytes);
+    *gathered = p->fwd;
+    gathered->num_context = nullptr;
+    return HSTU_OK;
+}
+
 }  // namespace
 
 extern "C" {
+
+HSTU_API int hstu_paged_fwd_workspace_size(const hstu_paged_fwd_params* params, uint64_t* workspace_bytes)
+{
+    if (workspace_bytes == nullptr) {
+        return fail(HSTU_ERR_NULLPTR, "workspace_bytes is NULL");
+    }
+    *workspace_bytes = 0;
+    hstu_jagged_fwd_params g;
+    uint64_t region = 0;
+    const int rc = validate_paged(params, &g, &region);
+    if (rc != HSTU_OK) {
+        return rc;
+    }
+    uint64_t inner = 0;
+    const int rc2 = hstu_jagged_fwd_workspace_size(&g, &inner);
+    if (rc2 != HSTU_OK) {
+        return rc2;
+    }
+    *workspace_bytes = 2 * region + inner;
+    return HSTU_OK;
+}
+
+HSTU_API int hstu_paged_fwd(const hstu_paged_fwd_params* p, void* workspace, uint64_t workspace_bytes, void* stream)
+{
+    hstu_jagged_fwd_params g;
+    uint64_t region = 0;
+    const int rc = validate_paged(p, &g, &region);
+    if (rc != HSTU_OK) {
+        return rc;
+    }
+    if (p->fwd.total_q == 0) {
+        return HSTU_OK;
+    }
+    if (p->fwd.total_k > 0) {
+        if (workspace == nullptr || workspace_bytes < 2 * region || reinterpret_cast<uintptr_t>(workspace) % 16 != 0) {
+            return fail(HSTU_ERR_WORKSPACE, "the paged forward needs a 16-byte aligned workspace of at least %llu bytes",
+                        (unsigned long long)(2 * region));
+        }
+        if (p->fwd.total_k > 0x7fffffffLL) {
+            return fail(HSTU_ERR_INVALID, "too many key rows");
+        }
+        hstu::PagedGatherArgs a;
+        memset(&a, 0, sizeof(a));
+        a.k = p->fwd.k;
+        a.v = p->fwd.v;
+        a.kv_cache = p->kv_cache;
+        a.k_out = workspace;
+        a.v_out = static_cast<char*>(workspace) + region;
+        a.offs_q = p->fwd.seq_offset_q;
+        a.offs_k = p->fwd.seq_offset_k;
+        a.page_offsets = p->page_offsets;
+        a.page_ids = p->page_ids;
+        a.num_tgt = p->fwd.num_target;
+        a.total_q = p->fwd.total_q;
+        a.total_k = p->fwd.total_k;
+        a.num_pages = p->num_pages;
+        a.n_page_ids = p->n_page_ids;
+        a.n_batch = static_cast<int>(p->fwd.n_offsets - 1);
+        a.page_size = static_cast<int>(p->page_size);
+        a.row_bytes = static_cast<int>(p->fwd.num_heads_k * p->fwd.head_dim_qk * (p->fwd.dtype == HSTU_DT_FP32 ? 4 : 2));
+        a.idx64 = (p->fwd.index_dtype == HSTU_IDX_I64) ? 1 : 0;
+        hipLaunchKernelGGL(hstu::hstu_paged_gather_kernel, dim3(static_cast<unsigned>(p->fwd.total_k)),
+                           dim3(hstu::kGatherThreads), 0, static_cast<hipStream_t>(stream), a);
+        const hipError_t err = hipGetLastError();
+        if (err != hipSuccess) {
+            return fail(HSTU_ERR_RUNTIME, "launch of the paged gather failed: %s", hipGetErrorString(err));
+        }
+        g.k = workspace;
+        g.v = static_cast<char*>(workspace) + region;
+    }
+    const uint64_t used = p->fwd.total_k > 0 ? 2 * region : 0;
+    return hstu_jagged_fwd(&g, static_cast<char*>(workspace) + used, workspace_bytes > used ? workspace_bytes - used : 0, stream);
+}
 
 HSTU_API int hstu_jagged_bwd_workspace_size(const hstu_jagged_bwd_params* params, uint64_t* workspace_bytes)
 {

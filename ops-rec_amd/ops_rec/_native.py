@@ -24,6 +24,8 @@ EXPORTED_SYMBOLS = (
     "hstu_jagged_fwd_kernel_name",
     "hstu_jagged_bwd_workspace_size",
     "hstu_jagged_bwd",
+    "hstu_paged_fwd_workspace_size",
+    "hstu_paged_fwd",
 )
 
 
@@ -81,6 +83,24 @@ class BwdParams(ctypes.Structure):
     ]
 
 
+class PagedParams(ctypes.Structure):
+    """Mirror of ``hstu_paged_fwd_params``."""
+
+    _fields_ = [
+        ("struct_size", ctypes.c_uint32),
+        ("reserved0", ctypes.c_uint32),
+        ("fwd", FwdParams),
+        ("kv_cache", ctypes.c_void_p),
+        ("page_offsets", ctypes.c_void_p),
+        ("page_ids", ctypes.c_void_p),
+        ("last_page_len", ctypes.c_void_p),
+        ("seq_offset_t", ctypes.c_void_p),
+        ("num_pages", ctypes.c_int64),
+        ("page_size", ctypes.c_int64),
+        ("n_page_ids", ctypes.c_int64),
+    ]
+
+
 _lib: Optional[ctypes.CDLL] = None
 
 
@@ -114,6 +134,10 @@ def load() -> ctypes.CDLL:
     lib.hstu_jagged_bwd_workspace_size.argtypes = [ctypes.POINTER(BwdParams), ctypes.POINTER(ctypes.c_uint64)]
     lib.hstu_jagged_bwd.restype = ctypes.c_int
     lib.hstu_jagged_bwd.argtypes = [ctypes.POINTER(BwdParams), ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]
+    lib.hstu_paged_fwd_workspace_size.restype = ctypes.c_int
+    lib.hstu_paged_fwd_workspace_size.argtypes = [ctypes.POINTER(PagedParams), ctypes.POINTER(ctypes.c_uint64)]
+    lib.hstu_paged_fwd.restype = ctypes.c_int
+    lib.hstu_paged_fwd.argtypes = [ctypes.POINTER(PagedParams), ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]
     _lib = lib
     return lib
 

@@ -46,6 +46,12 @@ _SCHEMAS = (
     # dense [B, S, N, D] layout (torch_extension/hstu_dense_plugin.cpp:156-163): forward only here
     "hstu_dense(Tensor q, Tensor k, Tensor v, Tensor? mask=None, Tensor? attn_bias=None, int mask_type=0, "
     "int max_seq_len=0, float silu_scale=0.0) -> Tensor",
+    # paged KV cache (torch_extension/hstu_paged_plugin.cpp:71-92)
+    "hstu_paged(Tensor q, Tensor k, Tensor v, Tensor kv_cache=None, Tensor? mask=None, Tensor? attn_bias=None, "
+    "int mask_type=0, int max_seq_len=0, int max_seq_len_k=0, float silu_scale=0.0, Tensor seq_offset=None, "
+    "Tensor seq_offset_k=None, Tensor seq_offset_t=None, Tensor page_offsets=None, Tensor page_ids=None, "
+    "Tensor last_page_len=None, Tensor num_target=None, int target_group_size=0, float? alpha=1.0, "
+    "bool deterministic=False) -> Tensor",
 )
 
 _lib_def = torch.library.Library("ops_rec", "DEF")
@@ -522,6 +528,68 @@ def hstu_dense_meta(q, k, v, mask=None, attn_bias=None, mask_type=0, max_seq_len
     return torch.empty((q.size(0), q.size(1), q.size(2), v.size(3)), dtype=_out_dtype(q), device=q.device)
 
 
+def hstu_paged(q, k, v, kv_cache=None, mask=None, attn_bias=None, mask_type=0, max_seq_len=0, max_seq_len_k=0,
+               silu_scale=0.0, seq_offset=None, seq_offset_k=None, seq_offset_t=None, page_offsets=None, page_ids=None,
+               last_page_len=None, num_target=None, target_group_size=0, alpha=1.0, deterministic=False):  # fmt: skip
+    """Forward with a paged KV cache (torch_extension/hstu_paged_plugin.cpp:21-69): the keys / values of a sequence
+    are its cached rows (pages of ``kv_cache`` [num_pages, 2, page_size, N_k, D]) followed by the rows of its
+    ``num_target`` new tokens, taken from the end of its segment of ``k`` / ``v``.  ``seq_offset_k`` describes the
+    resulting key ranges.  Same checks and argument normalisation as the reference adapter; output like ``q``."""
+    for name, t in (("kv_cache", kv_cache), ("page_ids", page_ids), ("last_page_len", last_page_len)):
+        _check(t is not None and t.numel() > 0, f"{name} must be a non-empty tensor")
+    _check(seq_offset is not None and seq_offset_k is not None and seq_offset_t is not None and page_offsets is not None,
+           "seq_offset, seq_offset_k, seq_offset_t and page_offsets are required")  # fmt: skip
+    _check(q.dim() == 3, "The q should be 3D in jagged layout")
+    for name, t in (("acSeqOffsetq", seq_offset), ("acSeqOffsetK", seq_offset_k), ("acSeqOffsetT", seq_offset_t)):
+        _check(t.dim() == 1 and t.size(0) >= 2, f"{name} params error should have at least two element.")
+    _check(num_target is None or int(target_group_size) > 0,
+           "targetGroupSize must be greater than 0 when numTarget is defined")  # fmt: skip
+    _check(kv_cache.dim() == 5 and kv_cache.size(1) == 2, "kv_cache must be [num_pages, 2, page_size, heads, dim]")
+    _check(kv_cache.dtype == q.dtype, "kv_cache must have the dtype of q")
+    _check(kv_cache.size(3) == k.size(1) and kv_cache.size(4) == k.size(2) and v.size(2) == k.size(2),
+           "kv_cache rows must have the heads and head dim of k and v")  # fmt: skip
+    idx_dtype = seq_offset.dtype
+    cache = kv_cache.contiguous()
+    p_offs = page_offsets.to(idx_dtype).contiguous()
+    p_ids = page_ids.to(idx_dtype).contiguous()
+    last_len = last_page_len.to(idx_dtype).contiguous()
+    offs_t = seq_offset_t.to(idx_dtype).contiguous()
+    _check(p_offs.dim() == 1 and p_offs.size(0) == seq_offset.size(0), "page_offsets must have the length of seq_offset")
+    prepared = prepare_forward(q, k, v, mask, attn_bias, mask_type, max_seq_len, max_seq_len_k, silu_scale, seq_offset,
+                               seq_offset_k, None, num_target, target_group_size, alpha, deterministic)  # fmt: skip
+    if prepared.out.numel() == 0:
+        return prepared.out
+    pp = _native.PagedParams()
+    pp.struct_size = ctypes.sizeof(_native.PagedParams)
+    pp.fwd = prepared.params
+    # an upper bound on the end of the key ranges that needs no device read: every page full plus every input row
+    pp.fwd.total_k = p_ids.numel() * cache.size(2) + q.size(0)
+    pp.kv_cache, pp.page_offsets, pp.page_ids = _ptr(cache), _ptr(p_offs), _ptr(p_ids)
+    pp.last_page_len, pp.seq_offset_t = _ptr(last_len), _ptr(offs_t)
+    pp.num_pages, pp.page_size, pp.n_page_ids = cache.size(0), cache.size(2), p_ids.numel()
+    lib = _native.load()
+    ws_bytes = ctypes.c_uint64(0)
+    rc = lib.hstu_paged_fwd_workspace_size(ctypes.byref(pp), ctypes.byref(ws_bytes))
+    if rc != _native.HSTU_OK:
+        raise RuntimeError(f"hstu_paged_fwd_workspace_size failed ({rc}): {_native.last_error()}")
+    ws = torch.empty(max(ws_bytes.value, 1), dtype=torch.uint8, device=q.device)
+    stream = torch.cuda.current_stream(q.device).cuda_stream
+    rc = lib.hstu_paged_fwd(ctypes.byref(pp), _ptr(ws), ws_bytes.value, ctypes.c_void_p(stream))
+    if rc != _native.HSTU_OK:
+        raise RuntimeError(f"hstu_paged_fwd failed ({rc}): {_native.last_error()}")
+    return prepared.out
+
+
+def hstu_paged_meta(q, k, v, kv_cache=None, mask=None, attn_bias=None, mask_type=0, max_seq_len=0, max_seq_len_k=0,
+                    silu_scale=0.0, seq_offset=None, seq_offset_k=None, seq_offset_t=None, page_offsets=None,
+                    page_ids=None, last_page_len=None, num_target=None, target_group_size=0, alpha=1.0,
+                    deterministic=False):  # fmt: skip
+    _check(q.dim() == 3, "The q should be 3D in jagged layout")
+    return torch.empty_like(q)
+
+
+_lib_cuda.impl("hstu_paged", hstu_paged)
+_lib_meta.impl("hstu_paged", hstu_paged_meta)
 _lib_cuda.impl("hstu_dense", hstu_dense)
 _lib_meta.impl("hstu_dense", hstu_dense_meta)
 _lib_cuda.impl("hstu_jagged.equal", hstu_jagged_equal)

@@ -36,6 +36,11 @@ How each function is pinned (none of them by retyping its own formula):
   (see the function); it is only used to apply the reference's own
   "double benchmark" acceptance rule, never as the primary check.
 
+* ``paged_keys_values`` / ``hstu_paged_forward`` -- against a scalar restatement of the
+  paged golden's own mask sentence (history columns: lower triangle; target columns:
+  identity) written with explicit loops over pages and rows, and against invariance
+  under a renumbering of the physical pages (``tests/test_oracle_paged.py``).
+
 The reference holds no stored golden vectors for this path (its tests compare an
 NPU run with a golden computed on the fly), so there is nothing to load.
 """
@@ -426,6 +431,51 @@ def hstu_jagged_forward_dense(
 # --------------------------------------------------------------------------- #
 # acceptance rules
 # --------------------------------------------------------------------------- #
+
+
+# --------------------------------------------------------------------------- #
+# paged KV cache
+# --------------------------------------------------------------------------- #
+
+
+def paged_keys_values(k, v, kv_cache, seq_offset, seq_offset_k, page_offsets, page_ids, last_page_len, num_target):
+    """The key / value rows the paged operator attends to, laid out by ``seq_offset_k``.
+
+    Per sequence: its pages ``page_ids[page_offsets[b] : page_offsets[b + 1]]`` of ``kv_cache``
+    [num_pages, 2, page_size, N_k, D] in order, the last one cut at ``last_page_len[b]``, followed by the last
+    ``num_target[b]`` rows of its segment of ``k`` / ``v``
+    (hstu_forward_v1/test/pytest/test_hstu_paged.py:234-262; common.py:270-285)."""
+    offs_q, offs_k = _as_list(seq_offset), _as_list(seq_offset_k)
+    p_offs, p_ids, last = _as_list(page_offsets), _as_list(page_ids), _as_list(last_page_len)
+    tgt = _as_list(num_target)
+    ks, vs = [], []
+    for b in range(len(offs_q) - 1):
+        q1 = offs_q[b + 1]
+        n_pages = p_offs[b + 1] - p_offs[b]
+        for j in range(n_pages):
+            pid = p_ids[p_offs[b] + j]
+            n = last[b] if j == n_pages - 1 else kv_cache.shape[2]
+            ks.append(kv_cache[pid, 0, :n])
+            vs.append(kv_cache[pid, 1, :n])
+        ks.append(k[q1 - tgt[b] : q1])
+        vs.append(v[q1 - tgt[b] : q1])
+        got = sum(t.shape[0] for t in ks)
+        assert got == offs_k[b + 1], f"sequence {b}: {got} key rows, seq_offset_k says {offs_k[b + 1]}"
+    return torch.cat(ks, dim=0), torch.cat(vs, dim=0)
+
+
+def hstu_paged_forward(q, k, v, kv_cache, *, seq_offset, seq_offset_k, page_offsets, page_ids, last_page_len,
+                       num_target, target_group_size=1, max_seq_len, max_seq_len_k=None, silu_scale=0.0, alpha=1.0,
+                       mask=None, attn_bias=None, mask_type=0, out_dtype=None, emulate_lowp=None):  # fmt: skip
+    """Paged forward = the jagged forward on the gathered keys / values, no context rows, grouped targets
+    (torch_extension/hstu_paged_plugin.cpp:62-69 passes zeros for num_context; golden common.py:255-300)."""
+    k_all, v_all = paged_keys_values(k, v, kv_cache, seq_offset, seq_offset_k, page_offsets, page_ids, last_page_len,
+                                     num_target)  # fmt: skip
+    return hstu_jagged_forward(q, k_all, v_all, mask=mask, attn_bias=attn_bias, mask_type=mask_type,
+                               max_seq_len=max_seq_len, max_seq_len_k=max_seq_len_k, silu_scale=silu_scale,
+                               seq_offset=seq_offset, seq_offset_k=seq_offset_k, num_context=None,
+                               num_target=num_target, target_group_size=target_group_size, alpha=alpha,
+                               out_dtype=out_dtype, emulate_lowp=emulate_lowp)  # fmt: skip
 
 
 def mismatch_fraction(actual: torch.Tensor, golden: torch.Tensor, atol: float) -> float:

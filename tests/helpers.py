@@ -2,6 +2,7 @@
 
 from __future__ import annotations
 
+import numpy as np
 import torch
 
 from ops_rec import workloads
@@ -84,4 +85,34 @@ def reference_style_case(batch, heads, max_len, dim, dtype, *, enable_bias=False
         num_target=n_tgt, target_group_size=group,
         seq_offset_k=(torch.tensor(ok, dtype=index_dtype) if delta else None), max_seq_len_k=(max_k if delta else None),
         lengths=lq,
+    )  # fmt: skip
+
+
+def paged_case(hist, prev, targets, page_size, heads=2, heads_k=None, dim=32, dtype=torch.float32, std=1.0, seed=0,
+               index_dtype=torch.int32, shuffle_pages=True, spare_pages=2):
+    """Inputs of ``hstu_paged`` in the way the reference's test builds them
+    (hstu_forward_v1/test/pytest/test_hstu_paged.py:274-330): per sequence ``hist[b]`` new history tokens and
+    ``targets[b]`` target tokens are the query rows; the cache holds ``prev[b] + hist[b]`` rows in pages of
+    ``page_size``; physical pages are numbered in a shuffled order with unused spare pages in between."""
+    g = torch.Generator().manual_seed(seed)
+    heads_k = heads_k or heads
+    batch = len(hist)
+    q_lens = [h + t for h, t in zip(hist, targets)]
+    k_lens = [p + h + t for p, h, t in zip(prev, hist, targets)]
+    total = sum(q_lens)
+    rnd = lambda *shape: (torch.randn(*shape, generator=g) * std).to(dtype)  # noqa: E731
+    q, k, v = rnd(total, heads, dim), rnd(total, heads_k, dim), rnd(total, heads_k, dim)
+    cached = [p + h for p, h in zip(prev, hist)]
+    pages_per_seq = [(c + page_size - 1) // page_size for c in cached]
+    n_pages = sum(pages_per_seq) + spare_pages
+    order = torch.randperm(n_pages, generator=g).tolist() if shuffle_pages else list(range(n_pages))
+    kv_cache = rnd(n_pages, 2, page_size, heads_k, dim)
+    page_ids = order[: sum(pages_per_seq)]
+    offs = lambda ls: torch.tensor([0] + list(np.cumsum(ls)), dtype=index_dtype)  # noqa: E731
+    last = [c % page_size if c % page_size else (page_size if c else 0) for c in cached]
+    return dict(
+        q=q, k=k, v=v, kv_cache=kv_cache, seq_offset=offs(q_lens), seq_offset_k=offs(k_lens),
+        seq_offset_t=offs(targets), page_offsets=offs(pages_per_seq), page_ids=torch.tensor(page_ids, dtype=index_dtype),
+        last_page_len=torch.tensor(last, dtype=index_dtype), num_target=torch.tensor(targets, dtype=index_dtype),
+        max_seq_len=max(q_lens), max_seq_len_k=max(k_lens),
     )  # fmt: skip
