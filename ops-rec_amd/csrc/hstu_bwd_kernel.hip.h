@@ -8,13 +8,14 @@
 //
 // Two kernels, no atomics, every output row written by exactly one wavefront (bitwise reproducible):
 //
-//   hstu_bwd_dkv_kernel  one workgroup (8 wavefronts) per 128-key tile of one (sequence, K/V head).  The key rows
+//   hstu_bwd_dkv_kernel  two workgroups per 128-key tile of one (sequence, K/V head), one per output.  The key rows
 //                        stay in registers (B operands) while the query rows that can see them stream through
-//                        LDS, 32 at a time, for every query head of the group.  Two wavefronts share each set of
-//                        32 keys, one per output, so that either fits in 256 registers and a SIMD holds one of
-//                        each kind (their MFMA and VALU phases overlap):
-//                          dV wavefront:  S = Q . K^T,  P,            dV^T += dO^T . P
-//                          dK wavefront:  S = Q . K^T,  dP = dO . V^T,  dS,  dK^T += Q^T . dS
+//                        LDS, 32 at a time, for every query head of the group.  Both outputs in one wavefront
+//                        would need 328 registers (one wavefront per SIMD, which cannot overlap its own MFMA and
+//                        VALU phases); as two workgroups either fits in 256 and two of them share a CU without
+//                        sharing a barrier, so that their phases drift apart and overlap:
+//                          dV workgroup:  S = Q . K^T,  P,            dV^T += dO^T . P
+//                          dK workgroup:  S = Q . K^T,  dP = dO . V^T,  dS,  dK^T += Q^T . dS
 //                        (A operands from LDS: Q, dO plain; dO^T, Q^T by transposed reads; B operands: K, V rows in
 //                        registers, P / dS straight from the accumulators)
 //   hstu_bwd_dq_kernel   one workgroup per 128-row query tile of one (sequence, head), the forward's shape: Q and
@@ -512,10 +513,10 @@ __global__ __launch_bounds__(256, 2) void hstu_bwd_dq_kernel(const BwdArgs a)
 // ---------------------------------------------------------------------------------------------------------
 // dK, dV
 // ---------------------------------------------------------------------------------------------------------
-constexpr int kDkvThreads = 512;
+constexpr int kDkvThreads = 256;
 
 template <typename Tag, int D, bool HAS_RAB, bool HAS_MASK>
-__global__ __launch_bounds__(kDkvThreads, 1) void hstu_bwd_dkv_kernel(const BwdArgs a)
+__global__ __launch_bounds__(kDkvThreads, 2) void hstu_bwd_dkv_kernel(const BwdArgs a)
 {
     typedef SubTile<D> T;
     constexpr int LPW = T::LPW, NLW = T::NLW, KSTEPS = T::KSTEPS, MTILES = T::MTILES, NCH = 2 * T::MTILES;
@@ -526,23 +527,25 @@ __global__ __launch_bounds__(kDkvThreads, 1) void hstu_bwd_dkv_kernel(const BwdA
     __shared__ __attribute__((aligned(1024))) uint16_t s_st2[2 * T::ELEMS];
     __shared__ __attribute__((aligned(1024))) uint16_t s_st3[2 * T::ELEMS];
     // a sub-tile is requested three steps ahead: the requests of two later steps may be outstanding at a step's start
-    constexpr int kReqs = 2 * LPW;
+    constexpr int kReqs = 2 * 2 * LPW;
     constexpr int kWaitStage = (kReqs & 15) | (7 << 4) | (15 << 8) | ((kReqs >> 4) << 14);
     constexpr uint32_t kPastEnd = 0x40000000u;
     static_assert(NLW == 4, "every wavefront takes part in the loads");
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
-    const int wave8 = uniform(tid >> 6);
-    const bool dk_role = wave8 >= 4;  // wavefronts 0..3 produce dV, 4..7 dK; w and w + 4 share keys (and a SIMD)
-    const int wave = wave8 & 3;
+    const int wave = uniform(tid >> 6);
+    // even workgroups produce dV, odd ones dK of the same key tile (neighbours in the grid, so that they tend to
+    // run side by side and find each other's Q / dO rows in the L2)
+    const bool dk_role = (blockIdx.x & 1) != 0;
     const int ln = lane & 31;
     const int lh = lane >> 5;
 
     // key tile 0 is seen by the most query rows: heaviest first
     const int per_level = a.n_batch * a.n_heads_k;
-    const int kt_idx = static_cast<int>(blockIdx.x) / per_level;
-    const int rem = static_cast<int>(blockIdx.x) - kt_idx * per_level;
+    const int tile_slot = static_cast<int>(blockIdx.x >> 1);
+    const int kt_idx = tile_slot / per_level;
+    const int rem = tile_slot - kt_idx * per_level;
     const int b = rem / a.n_heads_k;
     const int hk = rem - b * a.n_heads_k;
     zero_tail_rows(a.dk, a.offs_k, a.n_batch, a.idx64, a.total_k, static_cast<int64_t>(a.n_heads_k) * a.d_qk, kDkvThreads);
@@ -573,19 +576,16 @@ __global__ __launch_bounds__(kDkvThreads, 1) void hstu_bwd_dkv_kernel(const BwdA
         make_rsrc(static_cast<uint8_t*>(dk_role ? a.dk : a.dv) + (si.k0 * a.n_heads_k + hk) * static_cast<int64_t>(out_dim) * 2,
                   static_cast<uint32_t>(sk - 1) * out_stride + static_cast<uint32_t>(out_dim) * 2u);
 
-    // the dV wavefronts fill the Q half of a stage, the dK wavefronts the dO half: one set of per-lane source
-    // offsets per wavefront, for the tensor it loads
-    const uint32_t ld_stride = dk_role ? g_stride : q_stride;
-    const int ld_dim = dk_role ? a.d_v : a.d_qk;
-    const int ld_half = dk_role ? T::ELEMS : 0;
-    uint32_t ld_src[LPW];
+    // per-lane source offsets of the sub-tile loads (Q into the first half of a stage, dO into the second)
+    uint32_t q_src[LPW], g_src[LPW];
 #pragma unroll
     for (int i = 0; i < LPW; ++i) {
         const int slot = (wave * LPW + i) * 64 + lane;
         const int r = (slot / T::CPR) & 31;
         const int pc = slot % T::CPR;
         const int cs = both_ways_swizzle<D>(r, pc);
-        ld_src[i] = (cs * 8 < ld_dim) ? static_cast<uint32_t>(r) * ld_stride + cs * 16u : kOutOfRange;
+        q_src[i] = (cs * 8 < a.d_qk) ? static_cast<uint32_t>(r) * q_stride + cs * 16u : kOutOfRange;
+        g_src[i] = (cs * 8 < a.d_v) ? static_cast<uint32_t>(r) * g_stride + cs * 16u : kOutOfRange;
     }
     int n_lane_off[KSTEPS];
     int t_lane_off[MTILES][2];
@@ -646,14 +646,18 @@ __global__ __launch_bounds__(kDkvThreads, 1) void hstu_bwd_dkv_kernel(const BwdA
     int cur_h = hk * a.head_ratio, cur_x = x_first;              // current step
     auto request = [&](uint16_t* stage) {
         const bool past = req_it >= n_iter;  // (sent out of range: moves no data, keeps the count per step constant)
-        const uint8_t* const ld_base = static_cast<const uint8_t*>(dk_role ? a.grad : a.q);
-        const __amdgpu_buffer_rsrc_t ld_rsrc =
-            make_rsrc(ld_base + (si.q0 * a.n_heads_q + req_h) * static_cast<int64_t>(ld_dim) * 2,
-                      static_cast<uint32_t>(sq - 1) * ld_stride + static_cast<uint32_t>(ld_dim) * 2u);
-        const uint32_t base = past ? kPastEnd : static_cast<uint32_t>(req_x * 32) * ld_stride;
+        const __amdgpu_buffer_rsrc_t q_rsrc =
+            make_rsrc(static_cast<const uint8_t*>(a.q) + (si.q0 * a.n_heads_q + req_h) * static_cast<int64_t>(a.d_qk) * 2,
+                      static_cast<uint32_t>(sq - 1) * q_stride + a.d_qk * 2u);
+        const __amdgpu_buffer_rsrc_t g_rsrc =
+            make_rsrc(static_cast<const uint8_t*>(a.grad) + (si.q0 * a.n_heads_q + req_h) * static_cast<int64_t>(a.d_v) * 2,
+                      static_cast<uint32_t>(sq - 1) * g_stride + a.d_v * 2u);
+        const uint32_t qb = past ? kPastEnd : static_cast<uint32_t>(req_x * 32) * q_stride;
+        const uint32_t gb = past ? kPastEnd : static_cast<uint32_t>(req_x * 32) * g_stride;
 #pragma unroll
         for (int i = 0; i < LPW; ++i) {
-            load_to_lds_b128(ld_rsrc, stage + ld_half + (wave * LPW + i) * 512, ld_src[i] + base);
+            load_to_lds_b128(q_rsrc, stage + (wave * LPW + i) * 512, q_src[i] + qb);
+            load_to_lds_b128(g_rsrc, stage + T::ELEMS + (wave * LPW + i) * 512, g_src[i] + gb);
         }
         ++req_it;
         if (++req_x >= n_qsub) {
@@ -703,14 +707,23 @@ __global__ __launch_bounds__(kDkvThreads, 1) void hstu_bwd_dkv_kernel(const BwdA
                 s[i] = 0.f;
                 dp[i] = 0.f;
             }
-#pragma unroll
-            for (int js = 0; js < KSTEPS; ++js) {
-                s = mfma32<Tag>(read_n(stage, js), kf[js], s);
-            }
+            // two independent accumulation chains per wavefront, so that an MFMA never waits for the one before it:
+            // S and dP for the dK role; the even and the odd steps of S for the dV role (dp then holds half of S)
             if (dk_role) {
 #pragma unroll
                 for (int js = 0; js < KSTEPS; ++js) {
+                    s = mfma32<Tag>(read_n(stage, js), kf[js], s);
                     dp = mfma32<Tag>(read_n(stage + T::ELEMS, js), vf[js], dp);
+                }
+            } else {
+#pragma unroll
+                for (int js = 0; js < KSTEPS; js += 2) {
+                    s = mfma32<Tag>(read_n(stage, js), kf[js], s);
+                    dp = mfma32<Tag>(read_n(stage, js + 1), kf[js + 1], dp);
+                }
+#pragma unroll
+                for (int i = 0; i < 16; ++i) {
+                    s[i] += dp[i];
                 }
             }
             // fully visible block: every row's lim is past the last key, no context / target effects, all in range

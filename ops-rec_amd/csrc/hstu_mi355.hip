@@ -597,7 +597,7 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
     a.alpha = static_cast<float>(f->alpha);
     a.scale = static_cast<float>((f->silu_scale == 0.0) ? 1.0 / static_cast<double>(f->max_seq_len_q) : f->silu_scale);
 
-    const int64_t grid_kv = static_cast<int64_t>(a.n_ktiles) * a.n_batch * a.n_heads_k;
+    const int64_t grid_kv = 2 * static_cast<int64_t>(a.n_ktiles) * a.n_batch * a.n_heads_k;  // a dV and a dK workgroup per tile
     const int64_t grid_q = static_cast<int64_t>(a.n_qtiles) * a.n_batch * a.n_heads_q;
     if (grid_kv > 0x7fffffffLL || grid_q > 0x7fffffffLL) {
         return fail(HSTU_ERR_INVALID, "grid out of range");
