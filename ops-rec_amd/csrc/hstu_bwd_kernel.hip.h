@@ -63,7 +63,7 @@ struct BwdArgs {
     int idx64;
     int n_qtiles;     // ceil(max_q / 128)
     int n_ktiles;     // ceil(max_k / 128)
-    int bias_vec_ok;  // rab / mask / d rab rows may be accessed 4 elements (8 bytes) at a time
+    int bias_vec_ok;  // rab / mask / d rab rows may be accessed 4 elements (8 bytes) at a time (1), 16 bytes (2)
     float alpha;
     float scale;  // silu_scale, resolved
 };
@@ -400,17 +400,23 @@ __global__ __launch_bounds__(256, 2) void hstu_bwd_dq_kernel(const BwdArgs a)
         __builtin_amdgcn_s_waitcnt(kWaitStage);
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
-        request(kn_o, vn_o, x + 2);
-        if (x >= nx_w) {
-            return;  // nothing of this sub-tile is visible to the rows of this wavefront
-        }
+        // rab / mask values of this step go out before the tile requests: loads return in order, so waiting for
+        // them then only waits for requests of earlier steps, not for the ones made now
         const int c0 = x * 32;
         uint32_t rw[8], mw[8];
-        if constexpr (HAS_RAB) {
-            load_words(rab_rsrc, c0, rw);
+        if (x < nx_w) {
+            if constexpr (HAS_RAB) {
+                load_words(rab_rsrc, c0, rw);
+            }
+            if constexpr (HAS_MASK) {
+                load_words(mask_rsrc, c0, mw);
+            }
         }
-        if constexpr (HAS_MASK) {
-            load_words(mask_rsrc, c0, mw);
+        __builtin_amdgcn_sched_barrier(0);
+        request(kn_o, vn_o, x + 2);
+        __builtin_amdgcn_sched_barrier(0);
+        if (x >= nx_w) {
+            return;  // nothing of this sub-tile is visible to the rows of this wavefront
         }
         f32x16_t s, dp;
 #pragma unroll
@@ -640,6 +646,24 @@ __global__ __launch_bounds__(kDkvThreads, 2) void hstu_bwd_dkv_kernel(const BwdA
     const float ascale = a.alpha * a.scale;
     const uint32_t bias_bytes = static_cast<uint32_t>(a.max_q) * static_cast<uint32_t>(a.max_k) * 2u;
     const bool targets = a.mask_type == 0 && si.n_tgt > 0 && a.target_group > 0;
+    // rab / custom mask tiles are wanted with lane = key and registers = query rows, but lie in memory with the
+    // keys of a query row side by side.  With 16-byte aligned rows they are read the way they lie (lane = query
+    // row, 8 consecutive keys per 16-byte load) as the A operand of two MFMAs whose B operand is a constant 0/1
+    // matrix that routes k-slot (half lh, element e) of MFMA j to key column 16 j + 8 lh + e: the matrix pipe does
+    // the transposition (exactly: every product is a value times 1 or 0), and rab lands in the S accumulators.
+    const bool vec16 = a.bias_vec_ok == 2;
+    u32x4_t route[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
+    if constexpr (HAS_RAB || HAS_MASK) {
+        const uint32_t one = std::is_same<Tag, bf16_tag>::value ? 0x3f80u : 0x3c00u;  // 1.0 in the input type
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int d = ln - 16 * j - 8 * lh;  // the element of this lane's k-slots that is 1, if in 0..7
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                route[j][i] = (d == 2 * i) ? one : (d == 2 * i + 1) ? (one << 16) : 0u;
+            }
+        }
+    }
 
     // head and sub-tile of iteration it, kept incrementally (no division in the loop)
     int req_h = hk * a.head_ratio, req_x = x_first, req_it = 0;  // next request
@@ -684,7 +708,6 @@ __global__ __launch_bounds__(kDkvThreads, 2) void hstu_bwd_dkv_kernel(const BwdA
         __builtin_amdgcn_s_waitcnt(kWaitStage);
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
-        request(stage_o);
         const int h = cur_h;
         const int rq0 = cur_x * 32;  // first query row of the sub-tile
         if (++cur_x >= n_qsub) {
@@ -700,6 +723,37 @@ __global__ __launch_bounds__(kDkvThreads, 2) void hstu_bwd_dkv_kernel(const BwdA
             }
             active = active && cw0 < lim_max;
         }
+        const __amdgpu_buffer_rsrc_t rab_rsrc = make_rsrc(
+            HAS_RAB ? static_cast<const uint16_t*>(a.rab) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k) : nullptr,
+            HAS_RAB ? bias_bytes : 0u);
+        const __amdgpu_buffer_rsrc_t mask_rsrc = make_rsrc(
+            HAS_MASK ? static_cast<const uint16_t*>(a.mask) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k) : nullptr,
+            HAS_MASK ? bias_bytes : 0u);
+        // rab / mask rows of this step (16-byte path) go out before the tile requests: loads return in order, so
+        // waiting for them then only waits for requests of earlier steps.  Lane (ln, lh) reads row rq0 + ln, keys
+        // cw0 + 16 j + 8 lh .. + 7 (whole chunks are in or out of the row: max_seq_len_k is a multiple of 8 here).
+        u32x4_t ra[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
+        u32x4_t ma[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
+        if constexpr (HAS_RAB || HAS_MASK) {
+            if (vec16 && active) {
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int key0 = cw0 + 16 * j + 8 * lh;
+                    const uint32_t off = (rq0 + ln < sq && key0 < a.max_k)
+                                             ? (static_cast<uint32_t>(rq0 + ln) * static_cast<uint32_t>(a.max_k) + static_cast<uint32_t>(key0)) * 2u
+                                             : kOutOfRange;
+                    if constexpr (HAS_RAB) {
+                        ra[j] = __builtin_amdgcn_raw_buffer_load_b128(rab_rsrc, static_cast<int>(off), 0, 0);
+                    }
+                    if constexpr (HAS_MASK) {
+                        ma[j] = __builtin_amdgcn_raw_buffer_load_b128(mask_rsrc, static_cast<int>(off), 0, 0);
+                    }
+                }
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        request(stage_o);
+        __builtin_amdgcn_sched_barrier(0);
         if (active) {
             f32x16_t s, dp;
 #pragma unroll
@@ -731,20 +785,37 @@ __global__ __launch_bounds__(kDkvThreads, 2) void hstu_bwd_dkv_kernel(const BwdA
             if (a.mask_type == 0) {
                 full = full && (cw0 + 32 <= rq0 + si.delta + 1) && !(targets && rq0 + 31 >= sq - si.n_tgt);
             }
-            const __amdgpu_buffer_rsrc_t rab_rsrc = make_rsrc(
-                HAS_RAB ? static_cast<const uint16_t*>(a.rab) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k) : nullptr,
-                HAS_RAB ? bias_bytes : 0u);
-            const __amdgpu_buffer_rsrc_t mask_rsrc = make_rsrc(
-                HAS_MASK ? static_cast<const uint16_t*>(a.mask) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k) : nullptr,
-                HAS_MASK ? bias_bytes : 0u);
             // X and the custom mask value of every element, then the role's own function of it
             float xs[16], ms[16];
+            f32x16_t mt16;  // custom mask tile, transposed by the matrix pipe
+            if constexpr (HAS_RAB || HAS_MASK) {
+                if (vec16) {
+                    if constexpr (HAS_RAB) {
+                        s = mfma32<Tag>(ra[0], route[0], s);
+                        s = mfma32<Tag>(ra[1], route[1], s);
+                    }
+                    if constexpr (HAS_MASK) {
+#pragma unroll
+                        for (int i = 0; i < 16; ++i) {
+                            mt16[i] = 0.f;
+                        }
+                        mt16 = mfma32<Tag>(ma[0], route[0], mt16);
+                        mt16 = mfma32<Tag>(ma[1], route[1], mt16);
+                    }
+                }
+            }
 #pragma unroll
             for (int e = 0; e < 16; ++e) {
                 const int r = rq0 + 8 * (e / 4) + 4 * lh + (e % 4);  // query row of this element
                 xs[e] = s[e];
                 ms[e] = 1.0f;
+                if constexpr (HAS_MASK) {
+                    if (vec16) {
+                        ms[e] = mt16[e];
+                    }
+                }
                 if constexpr (HAS_RAB || HAS_MASK) {
+                    if (!vec16) {
                     const uint32_t boff = (r < sq && key < a.max_k)
                                               ? (static_cast<uint32_t>(r) * static_cast<uint32_t>(a.max_k) + static_cast<uint32_t>(key)) * 2u
                                               : kOutOfRange;
@@ -755,6 +826,7 @@ __global__ __launch_bounds__(kDkvThreads, 2) void hstu_bwd_dkv_kernel(const BwdA
                     if constexpr (HAS_MASK) {
                         const uint32_t raw = __builtin_amdgcn_raw_buffer_load_b16(mask_rsrc, static_cast<int>(boff), 0, 0);
                         ms[e] = lo_to_float<Tag>(raw & 0xffffu);
+                    }
                     }
                 }
             }

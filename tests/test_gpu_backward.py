@@ -94,7 +94,7 @@ def test_context_targets_rab(ctx, tgt, group, rab, monkeypatch):
     check(w, monkeypatch)
 
 
-@pytest.mark.parametrize("max_len", [300, 301, 303])  # rows of rab / mask / d rab 8-byte aligned or not
+@pytest.mark.parametrize("max_len", [300, 301, 303, 304])  # rows of rab / mask / d rab 8-byte, 2-byte, 16-byte aligned
 def test_custom_mask_and_rab_alignment(max_len, monkeypatch):
     w = make(batch=2, heads=2, dim=64, lo=150, hi=max_len, max_seq_len=max_len, seed=max_len, rab_std=0.5, dtype=torch.float16)
     g = torch.Generator(device=DEV).manual_seed(1)
