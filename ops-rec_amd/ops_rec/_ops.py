@@ -43,9 +43,11 @@ _SCHEMAS = (
     "Tensor? attn_bias=None, int mask_type=0, int max_seq_len=0, int max_seq_len_k=0, float silu_scale=0.0, "
     "Tensor seq_offset=None, Tensor seq_offset_k=None, Tensor? num_context=None, Tensor? num_target=None, "
     "int? target_group_size=0, float? alpha=1.0) -> (Tensor, Tensor, Tensor, Tensor)",
-    # dense [B, S, N, D] layout (torch_extension/hstu_dense_plugin.cpp:156-163): forward only here
+    # dense [B, S, N, D] layout (torch_extension/hstu_dense_plugin.cpp:156-172)
     "hstu_dense(Tensor q, Tensor k, Tensor v, Tensor? mask=None, Tensor? attn_bias=None, int mask_type=0, "
     "int max_seq_len=0, float silu_scale=0.0) -> Tensor",
+    "hstu_dense_backward(Tensor grad, Tensor q, Tensor k, Tensor v, Tensor? mask, Tensor? attn_bias, int mask_type=0, "
+    "int max_seq_len=0, float silu_scale=0.0) -> (Tensor, Tensor, Tensor, Tensor)",
     # paged KV cache (torch_extension/hstu_paged_plugin.cpp:71-92)
     "hstu_paged(Tensor q, Tensor k, Tensor v, Tensor kv_cache=None, Tensor? mask=None, Tensor? attn_bias=None, "
     "int mask_type=0, int max_seq_len=0, int max_seq_len_k=0, float silu_scale=0.0, Tensor seq_offset=None, "
@@ -588,6 +590,54 @@ def hstu_paged_meta(q, k, v, kv_cache=None, mask=None, attn_bias=None, mask_type
     return torch.empty_like(q)
 
 
+def hstu_dense_backward(grad, q, k, v, mask, attn_bias, mask_type=0, max_seq_len=0, silu_scale=0.0):
+    """Gradients of ``hstu_dense`` (torch_extension/hstu_dense_plugin.cpp:41-151): equal shapes for grad, q, k, v
+    ([B, S, N, D], seqLen == maxSeqLen), alpha 1, served by the jagged backward on the [B * S, N, D] views.  When
+    there is no attn_bias the reference returns a zero placeholder with the sequence length rounded up to 256;
+    so does this."""
+    _check(grad.dim() == 4, "The grad should be 4D in normal layout")
+    for name, t in (("q", q), ("k", k), ("v", v)):
+        _check(t.dim() == 4, f"The {name} should be 4D in normal layout")
+        _check(t.shape == grad.shape, f"Q and {name.upper() if name != 'q' else 'grad'} batch size check failed")
+        _check(t.dtype == grad.dtype, f"grad dtype should be the same as {name} dtype, but got grad: {grad.dtype} and {name}: {t.dtype}")
+    _check(grad.dtype in (torch.float16, torch.float32, torch.bfloat16),
+           f"float16, float32 or bfloat16 tensor expected but got a tensor with dtype: {grad.dtype}")  # fmt: skip
+    batch, s_len, heads, dim = grad.shape
+    _check(1 <= batch <= 2048, f"batchSize expect in [1, 2048], but value is {batch}")
+    _check(1 <= s_len <= _MAX_SEQ_LEN, f"seqLen expect in [1, 20480], but value is {s_len}")
+    _check(1 <= heads <= 16, f"headNum expect in [1, 16], but value is {heads}")
+    _check(16 <= dim <= 512, f"headDim expect in [16, 512], but value is {dim}")
+    _max_seq_len_check(int(max_seq_len), "maxSeqLen")
+    _mask_check(int(mask_type), mask is not None)
+    plane = (batch, heads, s_len, s_len)
+    for name, t in (("mask", mask if int(mask_type) == 3 else None), ("attnBias", attn_bias)):
+        if t is not None:
+            _check(t.dim() == 4 and tuple(t.shape) == plane, f"The {name} should be {plane}")
+            _check(t.dtype == grad.dtype, f"{name} dtype should be the same as grad dtype, but got {name}: {t.dtype} and grad: {grad.dtype}")
+    _check(s_len == int(max_seq_len), "seqLen must be equal to maxSeqLen")
+    dev = grad.device
+    offs = torch.arange(0, (batch + 1) * s_len, s_len, dtype=torch.int32, device=dev)[: batch + 1]
+    flat = lambda t: t.contiguous().view(batch * s_len, heads, dim)  # noqa: E731
+    dq, dk, dv, dbias = _backward_impl(flat(grad), flat(q), flat(k), flat(v), mask, attn_bias, mask_type, s_len, s_len,
+                                       silu_scale, offs, offs, None, None, 0, 1.0)  # fmt: skip
+    if dbias is None:
+        padded = (s_len + 255) // 256 * 256
+        dbias = torch.zeros((batch, heads, padded, padded), dtype=grad.dtype, device=dev)
+    return dq.view(grad.shape), dk.view(grad.shape), dv.view(grad.shape), dbias
+
+
+def hstu_dense_backward_meta(grad, q, k, v, mask, attn_bias, mask_type=0, max_seq_len=0, silu_scale=0.0):
+    _check(grad.dim() == 4, "The grad should be 4D in normal layout")
+    if attn_bias is not None:
+        dbias = torch.empty_like(attn_bias)
+    else:
+        padded = (grad.size(1) + 255) // 256 * 256
+        dbias = grad.new_empty((grad.size(0), grad.size(2), padded, padded))
+    return torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), dbias
+
+
+_lib_cuda.impl("hstu_dense_backward", hstu_dense_backward)
+_lib_meta.impl("hstu_dense_backward", hstu_dense_backward_meta)
 _lib_cuda.impl("hstu_paged", hstu_paged)
 _lib_meta.impl("hstu_paged", hstu_paged_meta)
 _lib_cuda.impl("hstu_dense", hstu_dense)

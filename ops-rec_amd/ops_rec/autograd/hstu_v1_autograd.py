@@ -93,6 +93,29 @@ def _jagged_delta_backward(ctx, grad):
     return _fit_grads((dq, dk, dv, None, dbias if attn_bias is not None else None), ctx)
 
 
+# hstu_dense: (q, k, v, mask, attn_bias, mask_type, max_seq_len, silu_scale)
+# (torch_extension/hstu_v1_autograd.py:90-135 of the reference)
+_DENSE_DEFAULTS = (None, None, None, None, None, 0, 0, 0.0)
+
+
+def _dense_setup_context(ctx, inputs, output=None):
+    q, k, v, mask, attn_bias, mask_type, max_seq_len, silu_scale = _unpack(inputs, _DENSE_DEFAULTS)
+    _reject_mask_grad(mask, "hstu_dense")
+    ctx.save_for_backward(q, k, v, mask, attn_bias)
+    ctx.mask_type = mask_type
+    ctx.max_seq_len = max_seq_len
+    ctx.silu_scale = silu_scale
+
+
+def _dense_backward(ctx, grad):
+    q, k, v, mask, attn_bias = ctx.saved_tensors
+    dq, dk, dv, dbias = torch.ops.ops_rec.hstu_dense_backward(
+        grad, q, k, v, mask, attn_bias, ctx.mask_type, ctx.max_seq_len, ctx.silu_scale
+    )
+    # without attn_bias the op returns a 256-aligned placeholder: dropped
+    return _fit_grads((dq, dk, dv, None, dbias if attn_bias is not None else None, None, None, None), ctx)
+
+
 _registered = False
 _registration_errors = {}
 
@@ -119,6 +142,7 @@ def register_autograd():
                         _jagged_equal_setup_context)  # fmt: skip
     ok &= _register_one("hstu_jagged.delta", torch.ops.ops_rec.hstu_jagged.delta, _jagged_delta_backward,
                         _jagged_delta_setup_context)  # fmt: skip
+    ok &= _register_one("hstu_dense", torch.ops.ops_rec.hstu_dense.default, _dense_backward, _dense_setup_context)
     if not ok:
         warnings.warn(
             "ops_rec.autograd.hstu_v1: some autograd registrations failed, see "

@@ -151,3 +151,40 @@ def test_loss_backward_uses_the_kernels(monkeypatch):
     direct = device_grads(w, grad_out)
     for a, b in zip((q.grad, k.grad, v.grad, bias.grad), direct):
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("use_bias", [False, True], ids=["nobias", "bias"])
+@pytest.mark.parametrize("dtype,dim", [(torch.bfloat16, 64), (torch.float16, 128), (torch.float32, 32)])
+def test_dense_layout_backward(dtype, dim, use_bias, monkeypatch):
+    # hstu_dense / hstu_dense_backward: [B, S, N, D], alpha 1, every sequence of full length
+    # (torch_extension/hstu_dense_plugin.cpp:41-151); loss.backward() through the registered autograd as well
+    monkeypatch.setenv("HSTU_MI355_COMPOSITE_BACKWARD", "0")
+    batch, seq, heads = 3, 200, 2
+    g = torch.Generator().manual_seed(dim)
+    mk = lambda *shape, std=0.5: (torch.randn(*shape, generator=g) * std).to(dtype)  # noqa: E731
+    q, k, v, grad = (mk(batch, seq, heads, dim) for _ in range(4))
+    bias = mk(batch, heads, seq, seq, std=0.3) if use_bias else None
+    d = lambda t: None if t is None else t.to(DEV)  # noqa: E731
+    dq, dk, dv, db = ops_rec.ascendc.attention.hstu_dense_backward(d(grad), d(q), d(k), d(v), None, d(bias), 0, seq, 0.0)
+    assert dq.shape == q.shape and dk.shape == k.shape and dv.shape == v.shape
+    assert tuple(db.shape) == ((batch, heads, seq, seq) if use_bias else (batch, heads, 256, 256))
+    # oracle: the jagged forward on the flattened tensors with offsets 0, S, 2S, ...
+    qf, kf, vf = (t.float().view(batch * seq, heads, dim).clone().requires_grad_(True) for t in (q, k, v))
+    bf = bias.float().clone().requires_grad_(True) if use_bias else None
+    offs = torch.arange(0, (batch + 1) * seq, seq, dtype=torch.int32)
+    out = O.hstu_jagged_forward(qf, kf, vf, attn_bias=bf, mask_type=0, max_seq_len=seq, seq_offset=offs, alpha=1.0,
+                                out_dtype=torch.float32)  # fmt: skip
+    out.backward(grad.float().view(batch * seq, heads, dim))
+    tol = {torch.bfloat16: 1e-2, torch.float16: 2e-3, torch.float32: 1e-4}[dtype]
+    for name, a, r in (("dq", dq, qf.grad), ("dk", dk, kf.grad), ("dv", dv, vf.grad)):
+        r = r.view(batch, seq, heads, dim)
+        torch.testing.assert_close(a.float().cpu(), r, atol=tol * r.abs().max().item(), rtol=tol, msg=lambda m, n=name: f"{n}: {m}")
+    if use_bias:
+        torch.testing.assert_close(db.float().cpu(), bf.grad, atol=tol * bf.grad.abs().max().item(), rtol=tol)
+    else:
+        assert not db.any()
+    # the same through autograd
+    qd, kd, vd = (d(t).clone().requires_grad_(True) for t in (q, k, v))
+    y = ops_rec.ascendc.attention.hstu_dense(qd, kd, vd, None, d(bias), 0, seq, 0.0)
+    y.backward(d(grad))
+    assert torch.equal(qd.grad, dq) and torch.equal(kd.grad, dk) and torch.equal(vd.grad, dv)
