@@ -177,9 +177,12 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* params, void* workspa
  * resulting key ranges (cached + targets per sequence) and fwd.total_k an upper bound on their end
  * (page_ids count x page_size + total_q is always enough); fwd.k / fwd.v are the inputs with total_q rows;
  * fwd.num_context is ignored (zeros, as in the reference adapter); everything else as in the forward.
- * Implementation: the library gathers the rows into the workspace (one copy kernel), then runs the jagged forward
- * on them, so the workspace is 2 x total_k rows (plus what the forward asks for).  last_page_len and seq_offset_t
- * are taken for signature parity; the number of cached rows of a sequence is its key count minus its targets. */
+ * Implementation: for bf16 / fp16 with head dims up to 128 the forward kernel reads the pages itself (a page
+ * look-up per 32-key sub-tile, page_size being a multiple of 32), and the workspace is only the optional room for
+ * splitting long key ranges over workgroups, as in hstu_jagged_fwd.  Otherwise (fp32, larger head dims) the library
+ * first gathers the rows into the workspace (one copy kernel: 2 x total_k rows, required) and runs the jagged
+ * forward on them.  last_page_len and seq_offset_t are taken for signature parity; the number of cached rows of a
+ * sequence is its key count minus its targets. */
 typedef struct hstu_paged_fwd_params {
     uint32_t struct_size; /* sizeof(hstu_paged_fwd_params) */
     uint32_t reserved0;

@@ -126,6 +126,15 @@ struct FwdArgs {
     int counter_slot;  // which pair of device-side work counters this launch uses
     float* ws;           // split variant: room for ws_parts partial outputs of kBlockM x D floats each (may be null)
     uint32_t ws_parts;
+    // paged variant: the first (key count - num_target) key rows of a sequence live in pages of kv_cache
+    // [num_pages, 2 (K, V), page_size, n_heads_k, d]; k / v then hold the rows of ALL query tokens, of which the last
+    // num_target of each sequence are its remaining keys
+    const void* kv_cache;
+    const void* page_offsets;  // [n_batch + 1]
+    const void* page_ids;      // [n_page_ids]
+    int64_t num_pages;
+    int64_t n_page_ids;
+    int page_shift;  // log2(page_size); page_size is 32, 64, 128 or 256
 #ifdef HSTU_TIMELINE
     unsigned long long* timeline;
 #endif
@@ -430,7 +439,11 @@ struct U32Quad {
 // variant cuts the key range of the long items into up to kMaxParts parts that are separate entries of the work
 // list ("Splitting long items" below); the host uses it when the list is short and a workspace is supplied.  It
 // excludes QUEUES.
-template <typename Tag, typename OutTag, int D, bool HAS_RAB, bool HAS_MASK, bool QUEUES = false, bool SPLIT = false>
+//
+// PAGED: K / V rows come from a paged cache plus the tail of the k / v inputs (see "Paged keys" below); built on top
+// of the SPLIT variant, because its callers (inference: few query rows against a long cache) have short lists.
+template <typename Tag, typename OutTag, int D, bool HAS_RAB, bool HAS_MASK, bool QUEUES = false, bool SPLIT = false,
+          bool PAGED = false>
 __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const FwdArgs a)
 {
     constexpr int kThreads = 256;
@@ -439,6 +452,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
     static_assert(!F8 || (!HAS_RAB && !HAS_MASK), "no rab / custom mask with fp8 inputs");
     static_assert(!F8 || D >= 64, "fp8 rows are at least 64 bytes");
     static_assert(!(QUEUES && SPLIT), "one list policy per variant");
+    static_assert(!PAGED || (SPLIT && !F8), "the paged variant builds on the split variant, 16-bit inputs");
     constexpr int CPR = D * ES / 16;             // 16-byte chunks per row
     constexpr int EPC16 = 16 / ES;               // elements per 16-byte chunk
     constexpr int SUB_ELEMS = 32 * D * ES / 2;   // one 32-key sub-tile, in 16-bit units
@@ -677,10 +691,12 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
     // [(wave * LPW + i) * 1024, +1024) of a slot; per-lane source offsets are fixed, only the base moves
     uint32_t k_src[LPW];
     uint32_t v_src[LPW];
+    int ld_row[LPW];  // row of the sub-tile that load i of this lane fills (paged variant)
 #pragma unroll
     for (int i = 0; i < LPW; ++i) {
         const int slot = (wave * LPW + i) * 64 + lane;  // 16-byte slot within the sub-tile
         const int r = (slot / CPR) & 31;
+        ld_row[i] = r;
         const int pc = slot % CPR;
         const int kc = F8 ? chunk_swizzle<CPR>(r, pc) : k_chunk_swizzle<D>(r, pc);  // XOR swizzles are their own inverse
         const int vc = F8 ? chunk_swizzle<CPR>(r, pc) : v_chunk_swizzle<D>(r, pc);
@@ -933,16 +949,48 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         const int delta = sk - sq;
         const int hist_k = sk - n_tgt;  // keys before the target block
 
+        // Paged keys.  Key rows [0, n_cached) of the sequence are rows of its pages page_ids[page_first ..
+        // page_last), page_size rows each, in order; key rows [n_cached, sk) are the last n_new rows of its segment
+        // of the k / v inputs.  page_size is a multiple of 32, so a 32-key sub-tile lies in one page; the sub-tile
+        // that holds row n_cached takes its rows from both sources (two requests under complementary lane masks).
+        // The physical page of sub-tile x is kept in pid_ring[x mod 4]: it is looked up (a scalar load) one time
+        // step before the request for K(x) needs it and stays until the request for V(x), two steps later, is out.
+        int n_new = 0, n_cached = 0;
+        int64_t page_first = 0, page_last = 0;
+        int pid_ring[4] = {0, 0, 0, 0};
+        if constexpr (PAGED) {
+            if (a.num_tgt) {
+                n_new = static_cast<int>(load_index_uniform(a.num_tgt, b, a.idx64));
+            }
+            n_new = n_new < 0 ? 0 : (n_new > sk ? sk : n_new);
+            n_new = n_new > sq ? sq : n_new;
+            n_cached = sk - n_new;
+            page_first = load_index_uniform(a.page_offsets, b, a.idx64);
+            page_last = load_index_uniform(a.page_offsets, b + 1, a.idx64);
+        }
+        auto page_of = [&](int x) -> int {
+            int64_t idx = page_first + ((static_cast<int64_t>(x) * 32) >> a.page_shift);
+            idx = idx < page_last ? idx : page_last - 1;
+            idx = idx < a.n_page_ids ? idx : a.n_page_ids - 1;
+            idx = idx < 0 ? 0 : idx;
+            int64_t pid = load_index_uniform(a.page_ids, idx, a.idx64);
+            pid = pid < a.num_pages ? pid : a.num_pages - 1;
+            return static_cast<int>(pid < 0 ? 0 : pid);
+        };
+
         // ---- buffer descriptors sized to this sequence / head ----
         const __amdgpu_buffer_rsrc_t q_rsrc =
             make_rsrc(static_cast<const uint8_t*>(a.q) + (q0 * a.n_heads_q + h) * static_cast<int64_t>(a.d_qk) * ES,
                       static_cast<uint32_t>(sq - 1) * q_stride + a.d_qk * ES);
+        // (paged variant: the descriptors of the new rows, i.e. the last n_new rows of the segment of k / v)
+        const int64_t k_first_row = PAGED ? q1 - n_new : k0;
+        const int k_rows = PAGED ? n_new : sk;
         const __amdgpu_buffer_rsrc_t k_rsrc =
-            make_rsrc(static_cast<const uint8_t*>(a.k) + (k0 * a.n_heads_k + hk) * static_cast<int64_t>(a.d_qk) * ES,
-                      sk > 0 ? static_cast<uint32_t>(sk - 1) * k_stride + a.d_qk * ES : 0u);
+            make_rsrc(static_cast<const uint8_t*>(a.k) + (k_first_row * a.n_heads_k + hk) * static_cast<int64_t>(a.d_qk) * ES,
+                      k_rows > 0 ? static_cast<uint32_t>(k_rows - 1) * k_stride + a.d_qk * ES : 0u);
         const __amdgpu_buffer_rsrc_t v_rsrc =
-            make_rsrc(static_cast<const uint8_t*>(a.v) + (k0 * a.n_heads_k + hk) * static_cast<int64_t>(a.d_v) * ES,
-                      sk > 0 ? static_cast<uint32_t>(sk - 1) * v_stride + a.d_v * ES : 0u);
+            make_rsrc(static_cast<const uint8_t*>(a.v) + (k_first_row * a.n_heads_k + hk) * static_cast<int64_t>(a.d_v) * ES,
+                      k_rows > 0 ? static_cast<uint32_t>(k_rows - 1) * v_stride + a.d_v * ES : 0u);
         const __amdgpu_buffer_rsrc_t o_rsrc =
             make_rsrc(out16 + (q0 * a.n_heads_q + h) * static_cast<int64_t>(a.d_v),
                       static_cast<uint32_t>(sq - 1) * o_stride + a.d_v * 2u);
@@ -988,23 +1036,55 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         }
 
         // requests for K sub-tile xk into K slot KS and V sub-tile xv into V slot VS
+        // paged variant: sub-tile x of K (kv = 0) or V (kv = 1), physical page pid, into dst.  Rows below `bnd`
+        // come from the page, the others from the new rows; a request past the end moves nothing.
+        auto request_paged = [&](uint16_t* dst, const __amdgpu_buffer_rsrc_t new_rsrc, const uint32_t (&src)[LPW], int x,
+                                 int pid, int kv) {
+            const bool live = x < x_end;
+            const int bnd = live ? n_cached - x * 32 : 0;
+            const int rows_c = bnd < 0 ? 0 : (bnd > 32 ? 32 : bnd);
+            const int page_size = 1 << a.page_shift;
+            const int64_t row0 = (static_cast<int64_t>(pid) * 2 + kv) * page_size + ((x * 32) & (page_size - 1));
+            const __amdgpu_buffer_rsrc_t page_rsrc =
+                make_rsrc(static_cast<const uint8_t*>(a.kv_cache) + (row0 * a.n_heads_k + hk) * static_cast<int64_t>(a.d_qk) * ES,
+                          rows_c > 0 ? static_cast<uint32_t>(rows_c - 1) * k_stride + a.d_qk * ES : 0u);
+            // offset of sub-tile row 0 among the new rows (negative, as a wrapped unsigned, while bnd > 0: the
+            // lanes that use it have rows >= bnd, which brings the sum back into range)
+            const uint32_t new_base = live ? static_cast<uint32_t>(x * 32 - n_cached) * k_stride : kPastEnd;
+#pragma unroll
+            for (int i = 0; i < LPW; ++i) {
+                if (ld_row[i] < bnd) {
+                    load_to_lds_b128(page_rsrc, dst + (wave * LPW + i) * 512, src[i]);
+                } else {
+                    load_to_lds_b128(new_rsrc, dst + (wave * LPW + i) * 512, src[i] + new_base);
+                }
+            }
+        };
         auto request_k = [&](auto ks, int xk) {
             if (NLW == 4 || wave < NLW) {
-                const uint32_t kb = (xk < x_end) ? static_cast<uint32_t>(xk * 32) * k_stride : kPastEnd;
                 uint16_t* const dst = k_slot(ks);
+                if constexpr (PAGED) {
+                    request_paged(dst, k_rsrc, k_src, xk, pid_ring[decltype(ks)::value & 3], 0);
+                } else {
+                    const uint32_t kb = (xk < x_end) ? static_cast<uint32_t>(xk * 32) * k_stride : kPastEnd;
 #pragma unroll
-                for (int i = 0; i < LPW; ++i) {
-                    load_to_lds_b128(k_rsrc, dst + (wave * LPW + i) * 512, k_src[i] + kb);
+                    for (int i = 0; i < LPW; ++i) {
+                        load_to_lds_b128(k_rsrc, dst + (wave * LPW + i) * 512, k_src[i] + kb);
+                    }
                 }
             }
         };
         auto request_v = [&](auto vs, int xv) {
             if (NLW == 4 || wave < NLW) {
-                const uint32_t vb = (xv < x_end) ? static_cast<uint32_t>(xv * 32) * v_stride : kPastEnd;
                 uint16_t* const dst = v_slot(vs);
+                if constexpr (PAGED) {
+                    request_paged(dst, v_rsrc, v_src, xv, pid_ring[decltype(vs)::value & 3], 1);
+                } else {
+                    const uint32_t vb = (xv < x_end) ? static_cast<uint32_t>(xv * 32) * v_stride : kPastEnd;
 #pragma unroll
-                for (int i = 0; i < LPW; ++i) {
-                    load_to_lds_b128(v_rsrc, dst + (wave * LPW + i) * 512, v_src[i] + vb);
+                    for (int i = 0; i < LPW; ++i) {
+                        load_to_lds_b128(v_rsrc, dst + (wave * LPW + i) * 512, v_src[i] + vb);
+                    }
                 }
             }
         };
@@ -1015,6 +1095,12 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
 
         // ---- start-up: what the times before the first would have requested, and the Q fragment ----
         // (x_begin is a multiple of 4: sub-tile x_begin + i belongs in slot i)
+        if constexpr (PAGED) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                pid_ring[i] = page_of(x_begin + i);
+            }
+        }
         request_k(ic0_t{}, x_begin);
         request_v(ic0_t{}, x_begin);
         request_k(ic1_t{}, x_begin + 1);
@@ -1246,6 +1332,9 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             // (2) tile requests of this time step
             request_k(sc, t + 4);
             request_v(std::integral_constant<int, (S + 2) & 3>{}, t + 2);
+            if constexpr (PAGED) {
+                pid_ring[(S + 1) & 3] = page_of(t + 5);  // for the request of K(t + 5) in the next time step
+            }
 
             // (3) arithmetic.  Two straight-line blocks, each entered on one wavefront-uniform flag:
             //       block A (sub-tile t-1 exists):  PV(t-1) MFMAs with the first half of silu(t) between them

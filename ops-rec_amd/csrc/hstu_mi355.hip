@@ -42,6 +42,7 @@ struct Variant {
     void (*kernel)(const hstu::FwdArgs);
     void (*kernel_queues)(const hstu::FwdArgs);  // the same with per-XCD work queues, for long lists; may be nullptr
     void (*kernel_split)(const hstu::FwdArgs);   // the same with long items split over workgroups, for short lists
+    void (*kernel_paged)(const hstu::FwdArgs);   // split variant that reads K / V through a page table; may be nullptr
     int d_pad;
     int threads;
     int persistent_wgs_per_cu;  // > 0: persistent kernel, this many workgroups per CU; 0: one workgroup per tile
@@ -93,13 +94,23 @@ constexpr auto split_kernel() -> void (*)(const hstu::FwdArgs)
     }
 }
 
+template <typename Tag, typename OutTag, int D, bool RAB, bool MASK>
+constexpr auto paged_kernel() -> void (*)(const hstu::FwdArgs)
+{
+    if constexpr (D == 64 || D == 128) {
+        return hstu::hstu_fwd_kernel<Tag, OutTag, D, RAB, MASK, false, true, true>;
+    } else {
+        return nullptr;
+    }
+}
+
 #define HSTU_VARIANT(tag, tagname, D, RAB, MASK, WGS)                                               \
     {"hstu_fwd_" tagname "_d" #D "_rab" #RAB "_mask" #MASK,                                        \
      "hstu_fwd_" tagname "_d" #D "_rab" #RAB "_mask" #MASK "_queues",                               \
      "hstu_fwd_" tagname "_d" #D "_rab" #RAB "_mask" #MASK "_split",                                \
      hstu::hstu_fwd_kernel<hstu::tag, hstu::tag, D, RAB, MASK>,                                     \
      queues_kernel<hstu::tag, hstu::tag, D, RAB, MASK>(),                                           \
-     split_kernel<hstu::tag, hstu::tag, D, RAB, MASK>(), D, 256, WGS}
+     split_kernel<hstu::tag, hstu::tag, D, RAB, MASK>(), paged_kernel<hstu::tag, hstu::tag, D, RAB, MASK>(), D, 256, WGS}
 #define HSTU_DIMS(tag, tagname, RAB, MASK)                                                           \
     {HSTU_VARIANT(tag, tagname, 32, RAB, MASK, 2), HSTU_VARIANT(tag, tagname, 64, RAB, MASK, 2), \
      HSTU_VARIANT(tag, tagname, 128, RAB, MASK, 2), HSTU_VARIANT(tag, tagname, 256, RAB, MASK, 1)}
@@ -113,7 +124,7 @@ const Variant kVariants[2][2][2][4] = {
 };
 
 #define HSTU_F32_VARIANT(D, RAB, MASK) \
-    {"hstu_fwd_f32_d" #D "_rab" #RAB "_mask" #MASK, nullptr, nullptr, hstu::hstu_fwd_f32_kernel<D, RAB, MASK>, nullptr, nullptr, D, 256, 0}
+    {"hstu_fwd_f32_d" #D "_rab" #RAB "_mask" #MASK, nullptr, nullptr, hstu::hstu_fwd_f32_kernel<D, RAB, MASK>, nullptr, nullptr, nullptr, D, 256, 0}
 #define HSTU_F32_DIMS(RAB, MASK) \
     {HSTU_F32_VARIANT(32, RAB, MASK), HSTU_F32_VARIANT(64, RAB, MASK), HSTU_F32_VARIANT(128, RAB, MASK), \
      HSTU_F32_VARIANT(256, RAB, MASK)}
@@ -124,7 +135,7 @@ const Variant kVariants[2][2][2][4] = {
      "hstu_fwd_f8e4m3_" oname "_d" #D "_split",                                                                  \
      hstu::hstu_fwd_kernel<hstu::f8_tag, hstu::otag, D, false, false>,                                         \
      queues_kernel<hstu::f8_tag, hstu::otag, D, false, false>(),                                               \
-     split_kernel<hstu::f8_tag, hstu::otag, D, false, false>(), D, 256, WGS}
+     split_kernel<hstu::f8_tag, hstu::otag, D, false, false>(), nullptr, D, 256, WGS}
 const Variant kVariantsF8[2][3] = {
     {HSTU_F8_VARIANT(f16_tag, "f16", 64, 2), HSTU_F8_VARIANT(f16_tag, "f16", 128, 2), HSTU_F8_VARIANT(f16_tag, "f16", 256, 1)},
     {HSTU_F8_VARIANT(bf16_tag, "bf16", 64, 2), HSTU_F8_VARIANT(bf16_tag, "bf16", 128, 2),
@@ -409,6 +420,9 @@ const BwdVariant* select_bwd(const hstu_jagged_bwd_params* p)
 }
 
 // ---- paged K/V --------------------------------------------------------------------------------------------
+int launch_forward(const hstu_jagged_fwd_params* p, const hstu_paged_fwd_params* paged, void* workspace,
+                   uint64_t workspace_bytes, void* stream);
+
 uint64_t round_up_256(uint64_t x) { return (x + 255u) & ~static_cast<uint64_t>(255u); }
 
 int validate_paged(const hstu_paged_fwd_params* p, hstu_jagged_fwd_params* gathered, uint64_t* region_bytes)
@@ -469,6 +483,15 @@ HSTU_API int hstu_paged_fwd_workspace_size(const hstu_paged_fwd_params* params, 
     if (rc != HSTU_OK) {
         return rc;
     }
+    const Variant* var = select(&g);
+    if (var == nullptr) {
+        return HSTU_ERR_UNSUPPORTED;
+    }
+    if (var->kernel_paged != nullptr) {
+        // the kernel reads the pages itself; scratch only for splitting long items (optional, may be 0)
+        *workspace_bytes = split_workspace_bytes(var, &g);
+        return HSTU_OK;
+    }
     uint64_t inner = 0;
     const int rc2 = hstu_jagged_fwd_workspace_size(&g, &inner);
     if (rc2 != HSTU_OK) {
@@ -489,6 +512,14 @@ HSTU_API int hstu_paged_fwd(const hstu_paged_fwd_params* p, void* workspace, uin
     if (p->fwd.total_q == 0) {
         return HSTU_OK;
     }
+    const Variant* var = select(&g);
+    if (var == nullptr) {
+        return HSTU_ERR_UNSUPPORTED;
+    }
+    if (var->kernel_paged != nullptr) {
+        return launch_forward(&g, p, workspace, workspace_bytes, stream);
+    }
+    // no paged kernel for this combination (fp32, head dims above 128): gather the rows, then the plain forward
     if (p->fwd.total_k > 0) {
         if (workspace == nullptr || workspace_bytes < 2 * region || reinterpret_cast<uintptr_t>(workspace) % 16 != 0) {
             return fail(HSTU_ERR_WORKSPACE, "the paged forward needs a 16-byte aligned workspace of at least %llu bytes",
@@ -527,7 +558,7 @@ HSTU_API int hstu_paged_fwd(const hstu_paged_fwd_params* p, void* workspace, uin
         g.v = static_cast<char*>(workspace) + region;
     }
     const uint64_t used = p->fwd.total_k > 0 ? 2 * region : 0;
-    return hstu_jagged_fwd(&g, static_cast<char*>(workspace) + used, workspace_bytes > used ? workspace_bytes - used : 0, stream);
+    return launch_forward(&g, nullptr, static_cast<char*>(workspace) + used, workspace_bytes > used ? workspace_bytes - used : 0, stream);
 }
 
 HSTU_API int hstu_jagged_bwd_workspace_size(const hstu_jagged_bwd_params* params, uint64_t* workspace_bytes)
@@ -662,7 +693,13 @@ HSTU_API const char* hstu_jagged_fwd_kernel_name(const hstu_jagged_fwd_params* p
     return may_take_split_variant(v, params, nullptr) ? v->name_split : v->name;  // (given the workspace asked for)
 }
 
-HSTU_API int hstu_jagged_fwd(const hstu_jagged_fwd_params* p, void* workspace, uint64_t workspace_bytes, void* stream)
+}  // extern "C"
+
+namespace {
+
+// the forward launch; `paged` (optional) makes it the paged variant, which the caller has checked to exist
+int launch_forward(const hstu_jagged_fwd_params* p, const hstu_paged_fwd_params* paged, void* workspace,
+                   uint64_t workspace_bytes, void* stream)
 {
     const int rc = validate(p);
     if (rc != HSTU_OK) {
@@ -719,6 +756,14 @@ HSTU_API int hstu_jagged_fwd(const hstu_jagged_fwd_params* p, void* workspace, u
     a.q_descale = p->q_descale;
     a.k_descale = p->k_descale;
     a.v_descale = p->v_descale;
+    if (paged != nullptr) {
+        a.kv_cache = paged->kv_cache;
+        a.page_offsets = paged->page_offsets;
+        a.page_ids = paged->page_ids;
+        a.num_pages = paged->num_pages;
+        a.n_page_ids = paged->n_page_ids;
+        a.page_shift = paged->page_size == 32 ? 5 : paged->page_size == 64 ? 6 : paged->page_size == 128 ? 7 : 8;
+    }
 
 #ifdef HSTU_TIMELINE
     // development builds only: the first MiB of the workspace receives the timeline
@@ -752,6 +797,9 @@ HSTU_API int hstu_jagged_fwd(const hstu_jagged_fwd_params* p, void* workspace, u
             a.ws_parts = static_cast<uint32_t>(parts < 0x7fffffffull ? parts : 0x7fffffffull);
             n_blocks = resident;  // the list may have more entries than items: all resident workgroups take part
         }
+        if (paged != nullptr) {
+            kernel = var->kernel_paged;  // (splits when it was given room above, otherwise not)
+        }
         a.counter_slot = static_cast<int>(g_next_counter_slot.fetch_add(1) % hstu::kCounterSlots);
     }
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(n_blocks)), dim3(static_cast<unsigned>(var->threads)), 0,
@@ -761,6 +809,15 @@ HSTU_API int hstu_jagged_fwd(const hstu_jagged_fwd_params* p, void* workspace, u
         return fail(HSTU_ERR_RUNTIME, "launch of %s failed: %s", var->name, hipGetErrorString(err));
     }
     return HSTU_OK;
+}
+
+}  // namespace
+
+extern "C" {
+
+HSTU_API int hstu_jagged_fwd(const hstu_jagged_fwd_params* p, void* workspace, uint64_t workspace_bytes, void* stream)
+{
+    return launch_forward(p, nullptr, workspace, workspace_bytes, stream);
 }
 
 }  // extern "C"
