@@ -955,9 +955,13 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         // that holds row n_cached takes its rows from both sources (two requests under complementary lane masks).
         // The physical page of sub-tile x is kept in pid_ring[x mod 4]: it is looked up (a scalar load) one time
         // step before the request for K(x) needs it and stays until the request for V(x), two steps later, is out.
+        // (All of this runs on the scalar unit, which the wavefronts of a CU share: the per-step part is kept to a
+        // handful of 32-bit instructions; 64-bit products are formed once per item.)
         int n_new = 0, n_cached = 0;
-        int64_t page_first = 0, page_last = 0;
+        int page_first = 0, page_hi = 0;  // indices into page_ids: first page of the sequence, last valid index
         int pid_ring[4] = {0, 0, 0, 0};
+        const uint8_t* cache_head = nullptr;       // row 0 of page 0, this K/V head
+        uint32_t page_bytes = 0;                   // one page of K (or V) rows
         if constexpr (PAGED) {
             if (a.num_tgt) {
                 n_new = static_cast<int>(load_index_uniform(a.num_tgt, b, a.idx64));
@@ -965,17 +969,23 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             n_new = n_new < 0 ? 0 : (n_new > sk ? sk : n_new);
             n_new = n_new > sq ? sq : n_new;
             n_cached = sk - n_new;
-            page_first = load_index_uniform(a.page_offsets, b, a.idx64);
-            page_last = load_index_uniform(a.page_offsets, b + 1, a.idx64);
+            const int64_t pf = load_index_uniform(a.page_offsets, b, a.idx64);
+            const int64_t pl = load_index_uniform(a.page_offsets, b + 1, a.idx64);
+            const int64_t top = a.n_page_ids - 1;
+            const int64_t hi = (pl - 1 < top) ? pl - 1 : top;
+            page_hi = static_cast<int>(hi < 0 ? 0 : hi);
+            page_first = static_cast<int>(pf < 0 ? 0 : (pf > page_hi ? page_hi : pf));
+            cache_head = static_cast<const uint8_t*>(a.kv_cache) + static_cast<int64_t>(hk) * a.d_qk * ES;
+            page_bytes = k_stride << a.page_shift;
         }
+        const int sub_shift = a.page_shift - 5;  // sub-tiles per page, as a shift
+        const int last_pid = static_cast<int>(a.num_pages - 1);
         auto page_of = [&](int x) -> int {
-            int64_t idx = page_first + ((static_cast<int64_t>(x) * 32) >> a.page_shift);
-            idx = idx < page_last ? idx : page_last - 1;
-            idx = idx < a.n_page_ids ? idx : a.n_page_ids - 1;
-            idx = idx < 0 ? 0 : idx;
-            int64_t pid = load_index_uniform(a.page_ids, idx, a.idx64);
-            pid = pid < a.num_pages ? pid : a.num_pages - 1;
-            return static_cast<int>(pid < 0 ? 0 : pid);
+            int idx = page_first + (x >> sub_shift);
+            idx = idx < page_hi ? idx : page_hi;
+            int pid = static_cast<int>(load_index_uniform(a.page_ids, idx, a.idx64));
+            pid = pid < last_pid ? pid : last_pid;
+            return pid < 0 ? 0 : pid;
         };
 
         // ---- buffer descriptors sized to this sequence / head ----
@@ -1043,11 +1053,10 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             const bool live = x < x_end;
             const int bnd = live ? n_cached - x * 32 : 0;
             const int rows_c = bnd < 0 ? 0 : (bnd > 32 ? 32 : bnd);
-            const int page_size = 1 << a.page_shift;
-            const int64_t row0 = (static_cast<int64_t>(pid) * 2 + kv) * page_size + ((x * 32) & (page_size - 1));
+            const uint32_t in_page = static_cast<uint32_t>(x & ((1 << sub_shift) - 1)) * 32u * k_stride;
+            const uint64_t page_off = static_cast<uint64_t>(static_cast<uint32_t>(2 * pid + kv)) * page_bytes + in_page;
             const __amdgpu_buffer_rsrc_t page_rsrc =
-                make_rsrc(static_cast<const uint8_t*>(a.kv_cache) + (row0 * a.n_heads_k + hk) * static_cast<int64_t>(a.d_qk) * ES,
-                          rows_c > 0 ? static_cast<uint32_t>(rows_c - 1) * k_stride + a.d_qk * ES : 0u);
+                make_rsrc(cache_head + page_off, rows_c > 0 ? static_cast<uint32_t>(rows_c - 1) * k_stride + a.d_qk * ES : 0u);
             // offset of sub-tile row 0 among the new rows (negative, as a wrapped unsigned, while bnd > 0: the
             // lanes that use it have rows >= bnd, which brings the sum back into range)
             const uint32_t new_base = live ? static_cast<uint32_t>(x * 32 - n_cached) * k_stride : kPastEnd;
