@@ -295,3 +295,105 @@ def test_dense_op_is_registered_with_meta_inference():
     assert out.shape == (3, 40, 2, 32) and out.dtype == torch.bfloat16
     with pytest.raises(RuntimeError, match="4D in dense layout"):
         op(q[0], q[0], v[0], None, None, 0, 40, 0.0)
+
+
+def _copy_fwd(dst, src):
+    ctypes.memmove(ctypes.byref(dst), ctypes.byref(src), ctypes.sizeof(_native.FwdParams))
+
+
+def test_backward_c_abi_validation_codes():
+    lib = _native.load()
+    ws = ctypes.c_uint64(7)
+    fake = 0x1000
+
+    def make(**over):
+        b = _native.new_bwd_params()
+        f = _valid_params()
+        for k, v in over.pop("fwd", {}).items():
+            setattr(f, k, v)
+        _copy_fwd(b.fwd, f)
+        b.grad = b.grad_q = b.grad_k = b.grad_v = fake
+        for k, v in over.items():
+            setattr(b, k, v)
+        return b
+
+    def rc(b):
+        return lib.hstu_jagged_bwd_workspace_size(ctypes.byref(b), ctypes.byref(ws))
+
+    assert rc(make()) == 0 and ws.value == 0
+    assert lib.hstu_jagged_bwd_workspace_size(None, ctypes.byref(ws)) == 161001
+    assert lib.hstu_jagged_bwd_workspace_size(ctypes.byref(make()), None) == 161001
+    assert rc(make(fwd=dict(out=None))) == 0  # the forward's output is not an input of the backward
+    for over, code, text in [
+        (dict(struct_size=8), 161002, "struct_size"),
+        (dict(grad=None), 161001, "grad"),
+        (dict(grad_k=None), 161001, "grad_k"),
+        (dict(grad_attn_bias=fake), 161002, "without attn_bias"),
+        (dict(fwd=dict(mask_type=1)), 161002, "triu"),
+        (dict(fwd=dict(num_heads_k=3)), 161002, "divisible"),
+        (dict(fwd=dict(dtype=_native.DT_FP32, out_dtype=_native.DT_FP32)), 161003, "bf16 and fp16"),
+        (dict(fwd=dict(head_dim_qk=256, head_dim_v=256)), 161003, "up to 128"),
+        (dict(fwd=dict(head_dim_qk=12, head_dim_v=16)), 161003, "multiple of 8"),
+    ]:
+        got = rc(make(**over))
+        assert got == code, (over, got, _native.last_error())
+        assert re.search(text, _native.last_error()), (over, _native.last_error())
+    # launching with an invalid description is refused before any device call
+    assert lib.hstu_jagged_bwd(ctypes.byref(make(fwd=dict(mask_type=1))), None, 0, None) == 161002
+
+
+def test_paged_c_abi_validation_codes():
+    lib = _native.load()
+    ws = ctypes.c_uint64(7)
+    fake = 0x1000
+
+    def make(**over):
+        pp = _native.PagedParams()
+        pp.struct_size = ctypes.sizeof(_native.PagedParams)
+        f = _valid_params()
+        for k, v in over.pop("fwd", {}).items():
+            setattr(f, k, v)
+        _copy_fwd(pp.fwd, f)
+        pp.kv_cache = pp.page_offsets = pp.page_ids = fake
+        pp.num_pages, pp.page_size, pp.n_page_ids = 4, 64, 4
+        for k, v in over.items():
+            setattr(pp, k, v)
+        return pp
+
+    def rc(pp):
+        return lib.hstu_paged_fwd_workspace_size(ctypes.byref(pp), ctypes.byref(ws))
+
+    assert rc(make()) == 0  # (no device here: the optional split workspace is reported as 0)
+    # fp32 has no paged kernel: the rows are gathered into the workspace first, K and V of total_k rows each
+    assert rc(make(fwd=dict(dtype=_native.DT_FP32, out_dtype=_native.DT_FP32))) == 0
+    assert ws.value == 2 * 10 * 4 * 128 * 4
+    for over, code, text in [
+        (dict(struct_size=8), 161002, "struct_size"),
+        (dict(kv_cache=None), 161001, "kv_cache"),
+        (dict(page_ids=None), 161001, "page_ids"),
+        (dict(page_size=48), 161002, "32, 64, 128 or 256"),
+        (dict(num_pages=0), 161002, "must not be empty"),
+        (dict(fwd=dict(head_dim_v=64)), 161002, "one head dim"),
+        (dict(fwd=dict(dtype=_native.DT_FP8_E4M3, out_dtype=_native.DT_FP16)), 161003, "fp8"),
+        (dict(fwd=dict(max_seq_len_q=0)), 161002, "20480"),
+    ]:
+        got = rc(make(**over))
+        assert got == code, (over, got, _native.last_error())
+        assert re.search(text, _native.last_error()), (over, _native.last_error())
+    assert lib.hstu_paged_fwd(ctypes.byref(make(page_size=48)), None, 0, None) == 161002
+    # the gather path refuses to run without its workspace
+    pp = make(fwd=dict(dtype=_native.DT_FP32, out_dtype=_native.DT_FP32))
+    assert lib.hstu_paged_fwd(ctypes.byref(pp), None, 0, None) == 161004 and "workspace" in _native.last_error()
+
+
+def test_paged_and_dense_backward_ops_are_registered():
+    assert [a.name for a in torch.ops.ops_rec.hstu_paged.default._schema.arguments][:4] == ["q", "k", "v", "kv_cache"]
+    assert len(torch.ops.ops_rec.hstu_paged.default._schema.arguments) == 20
+    q = torch.empty(10, 4, 32, device="meta", dtype=torch.float16)
+    idx = torch.empty(3, device="meta", dtype=torch.int32)
+    cache = torch.empty(2, 2, 32, 4, 32, device="meta", dtype=torch.float16)
+    out = torch.ops.ops_rec.hstu_paged(q, q, q, cache, None, None, 0, 6, 6, 0.0, idx, idx, idx, idx, idx, idx[:2], idx[:2], 1)
+    assert out.shape == q.shape and out.dtype == torch.float16
+    g = torch.empty(2, 5, 4, 32, device="meta", dtype=torch.bfloat16)
+    dq, dk, dv, db = torch.ops.ops_rec.hstu_dense_backward(g, g, g, g, None, None, 0, 5, 0.0)
+    assert dq.shape == g.shape and tuple(db.shape) == (2, 4, 256, 256)
