@@ -445,11 +445,27 @@ __global__ __launch_bounds__(256, 2) void hstu_bwd_dq_kernel(const BwdArgs a)
                 if constexpr (HAS_MASK) {
                     ds *= e2 ? hi_to_float<Tag>(mw[i]) : lo_to_float<Tag>(mw[i]);
                 }
-                const int key = c0 + 8 * (e / 4) + 4 * lh + (e % 4);
-                const bool vis = (key < lim) && !(key >= hole_lo && key < hole_hi);
-                ds2[e2] = vis ? ds : 0.f;
+                ds2[e2] = ds;
             }
             pk[i] = pack2<Tag>(ds2[0], ds2[1]);
+        }
+        // visibility, applied to the packed values and only when the sub-tile is not fully visible to this
+        // wavefront's rows (as in the forward): key c0 + 8 (e / 4) + 4 lh + e % 4 of element e is hidden at or past
+        // lim and inside the hole
+        const bool full = (c0 + 32 <= wb.lim_min) && !(wb.any_hole && c0 + 32 > sq_info.hist_k && c0 < wb.hole_hi_max);
+        if (!full) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                uint32_t keep = 0;
+#pragma unroll
+                for (int e2 = 0; e2 < 2; ++e2) {
+                    const int e = 2 * i + e2;
+                    const int key = c0 + 8 * (e / 4) + 4 * lh + (e % 4);
+                    const bool vis = (key < lim) && !(key >= hole_lo && key < hole_hi);
+                    keep |= vis ? (0xffffu << (16 * e2)) : 0u;
+                }
+                pk[i] &= keep;
+            }
         }
         if constexpr (WANT_DRAB) {
 #pragma unroll
