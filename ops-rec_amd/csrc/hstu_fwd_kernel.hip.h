@@ -499,18 +499,9 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
     const int n_levels = a.n_qtiles;
     const int n_heads = a.n_heads_q;
 
-    // ---- rows past the last offset belong to no sequence: zero-fill them (all workgroups share the job) ----
-    {
-        const int64_t last = load_index_uniform(a.offs_q, a.n_batch, a.idx64);
-        const int64_t first_tail = last < 0 ? 0 : (last < a.total_q ? last : a.total_q);
-        const int64_t row_elems = static_cast<int64_t>(n_heads) * a.d_v;
-        const int64_t n_tail = (a.total_q - first_tail) * row_elems;
-        uint16_t* tail = out16 + first_tail * row_elems;
-        for (int64_t e = static_cast<int64_t>(blockIdx.x) * kThreads + tid; e < n_tail;
-             e += static_cast<int64_t>(gridDim.x) * kThreads) {
-            tail[e] = 0;
-        }
-    }
+    // rows past the last offset belong to no sequence and are zero-filled when the workgroup leaves (all workgroups
+    // share the job); the offset is requested here, so that nothing waits for it
+    const int64_t last_offset = load_index_uniform(a.offs_q, a.n_batch, a.idx64);
 
     // ---- work list: bucket the sequences by their number of query tiles ----
     for (int i = tid; i <= n_levels; i += kThreads) {
@@ -1683,6 +1674,18 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
 #endif
 
         // (the barriers of the sweep separate this item's reads of s_item from the next fetch)
+    }
+
+    // ---- rows past the last offset: zero-fill ----
+    {
+        const int64_t first_tail = last_offset < 0 ? 0 : (last_offset < a.total_q ? last_offset : a.total_q);
+        const int64_t row_elems = static_cast<int64_t>(n_heads) * a.d_v;
+        const int64_t n_tail = (a.total_q - first_tail) * row_elems;
+        uint16_t* tail = out16 + first_tail * row_elems;
+        for (int64_t e = static_cast<int64_t>(blockIdx.x) * kThreads + tid; e < n_tail;
+             e += static_cast<int64_t>(gridDim.x) * kThreads) {
+            tail[e] = 0;
+        }
     }
 
     // ---- leave: the last workgroup out puts the counters of this slot back to zero ----
