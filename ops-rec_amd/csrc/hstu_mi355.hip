@@ -327,7 +327,8 @@ bool may_take_split_variant(const Variant* var, const hstu_jagged_fwd_params* p,
     }
     const int64_t n_qtiles = (p->max_seq_len_q + hstu::kBlockM - 1) / hstu::kBlockM;
     const int64_t n_blocks = n_qtiles * (p->n_offsets - 1) * p->num_heads_q;
-    return n_blocks < 2 * resident;
+    // (an item of at most 8 sub-tiles is never split: the kernel's parts are at least that long)
+    return n_blocks < 2 * resident && p->max_seq_len_k > 8 * 32;
 }
 uint64_t split_workspace_bytes(const Variant* var, const hstu_jagged_fwd_params* p)
 {
