@@ -143,7 +143,7 @@ HSTU_API int hstu_jagged_fwd(const hstu_jagged_fwd_params* params, void* workspa
  *   C usage        ascendc/attention/hstu_v1/hstu_backward_v1/examples/aclnn/test_aclnn_hstu_backward_v1_jagged.cpp:174-186
  *
  * `fwd` describes q, k, v, mask, attn_bias, the offsets and the scalars exactly as for the forward (fwd.out is
- * not used and may be NULL).  Built for bf16 / fp16 with head dims up to 128 (q/k head dim a multiple of 8);
+ * not used and may be NULL).  Built for bf16 / fp16 with head dims up to 256 (q/k head dim a multiple of 8);
  * other valid descriptions return HSTU_ERR_UNSUPPORTED.
  * grad_q / grad_k / grad_v: every row is written (rows past the last offset are zero-filled), so the caller
  * need not clear them.  grad_attn_bias (optional; requires attn_bias): only the elements inside a

@@ -1,0 +1,120 @@
+// Argument blocks of the kernels and the few constants the host side shares with them (no device code here).
+#pragma once
+#include <stdint.h>
+
+namespace hstu {
+
+constexpr int kBlockM = 128;  // query rows per workgroup
+constexpr int kWaveM = 32;    // query rows per wavefront
+constexpr int kCounterSlots = 64;  // sets of device-side work counters (see the forward kernel)
+constexpr int kDkvThreads = 256;   // threads of a workgroup of the key-tile backward kernel
+constexpr int kGatherThreads = 128;
+
+struct FwdArgs {
+    const void* q;
+    const void* k;
+    const void* v;
+    const void* rab;
+    const void* mask;
+    void* out;
+    const void* offs_q;
+    const void* offs_k;
+    const void* num_ctx;
+    const void* num_tgt;
+    int64_t total_q;
+    int64_t total_k;
+    int n_batch;   // n_offsets - 1
+    int n_heads_q;
+    int n_heads_k;
+    int head_ratio;  // n_heads_q / n_heads_k
+    int d_qk;        // real head dims (<= the padded template dim)
+    int d_v;
+    int max_q;
+    int max_k;
+    int mask_type;
+    int target_group;
+    int idx64;       // offsets / context / target are int64
+    int n_qtiles;    // ceil(max_q / kBlockM)
+    int bh;          // n_batch * n_heads_q
+    int bias_vec_ok; // rab / mask rows may be read 4 elements (8 bytes) at a time
+    float c_exp;     // -alpha * log2(e)
+    float c_out;     // alpha * silu_scale
+    float alpha;     // fp8 inputs only: the kernel folds the per-head scales in itself
+    float silu_scale;
+    const float* q_descale;  // fp8 inputs only; per head, nullptr = 1
+    const float* k_descale;
+    const float* v_descale;
+    int counter_slot;  // which pair of device-side work counters this launch uses
+    float* ws;           // split variant: room for ws_parts partial outputs of kBlockM x D floats each (may be null)
+    uint32_t ws_parts;
+    // paged variant: the first (key count - num_target) key rows of a sequence live in pages of kv_cache
+    // [num_pages, 2 (K, V), page_size, n_heads_k, d]; k / v then hold the rows of ALL query tokens, of which the last
+    // num_target of each sequence are its remaining keys
+    const void* kv_cache;
+    const void* page_offsets;  // [n_batch + 1]
+    const void* page_ids;      // [n_page_ids]
+    int64_t num_pages;
+    int64_t n_page_ids;
+    int page_shift;  // log2(page_size); page_size is 32, 64, 128 or 256
+#ifdef HSTU_TIMELINE
+    unsigned long long* timeline;
+#endif
+};
+
+struct BwdArgs {
+    const void* q;
+    const void* k;
+    const void* v;
+    const void* grad;  // dO
+    const void* rab;
+    const void* mask;
+    void* dq;
+    void* dk;
+    void* dv;
+    void* drab;  // may be null
+    const void* offs_q;
+    const void* offs_k;
+    const void* num_ctx;
+    const void* num_tgt;
+    int64_t total_q;
+    int64_t total_k;
+    int n_batch;
+    int n_heads_q;
+    int n_heads_k;
+    int head_ratio;
+    int d_qk;
+    int d_v;
+    int max_q;
+    int max_k;
+    int mask_type;
+    int target_group;
+    int idx64;
+    int n_qtiles;     // ceil(max_q / 128)
+    int n_ktiles;     // ceil(max_k / 128)
+    int bias_vec_ok;  // rab / mask / d rab rows may be accessed 4 elements (8 bytes) at a time (1), 16 bytes (2)
+    float alpha;
+    float scale;  // silu_scale, resolved
+};
+
+struct PagedGatherArgs {
+    const void* k;         // [total_q, heads_k, dim]: rows of all tokens; only the target rows are used
+    const void* v;
+    const void* kv_cache;  // [num_pages, 2, page_size, heads_k, dim]
+    void* k_out;           // [total_k, heads_k, dim]
+    void* v_out;
+    const void* offs_q;    // [n_batch + 1]
+    const void* offs_k;    // [n_batch + 1]
+    const void* page_offsets;  // [n_batch + 1]
+    const void* page_ids;      // [page_offsets[n_batch]]
+    const void* num_tgt;       // [n_batch]
+    int64_t total_q;
+    int64_t total_k;
+    int64_t num_pages;
+    int64_t n_page_ids;
+    int n_batch;
+    int page_size;
+    int row_bytes;  // heads_k * dim * element size, a multiple of 16
+    int idx64;
+};
+
+}  // namespace hstu

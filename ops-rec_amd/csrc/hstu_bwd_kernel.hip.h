@@ -33,40 +33,6 @@
 
 namespace hstu {
 
-struct BwdArgs {
-    const void* q;
-    const void* k;
-    const void* v;
-    const void* grad;  // dO
-    const void* rab;
-    const void* mask;
-    void* dq;
-    void* dk;
-    void* dv;
-    void* drab;  // may be null
-    const void* offs_q;
-    const void* offs_k;
-    const void* num_ctx;
-    const void* num_tgt;
-    int64_t total_q;
-    int64_t total_k;
-    int n_batch;
-    int n_heads_q;
-    int n_heads_k;
-    int head_ratio;
-    int d_qk;
-    int d_v;
-    int max_q;
-    int max_k;
-    int mask_type;
-    int target_group;
-    int idx64;
-    int n_qtiles;     // ceil(max_q / 128)
-    int n_ktiles;     // ceil(max_k / 128)
-    int bias_vec_ok;  // rab / mask / d rab rows may be accessed 4 elements (8 bytes) at a time (1), 16 bytes (2)
-    float alpha;
-    float scale;  // silu_scale, resolved
-};
 
 struct SeqInfo {
     int64_t q0;
@@ -174,8 +140,8 @@ __device__ __forceinline__ void score_grad(float s, float dp, float alpha, float
 template <int D>
 __device__ __forceinline__ int both_ways_swizzle(int row, int chunk)
 {
-    static_assert(D == 64 || D == 128, "layouts exist for 64 and 128 elements per row");
-    if constexpr (D == 128) {
+    static_assert(D == 64 || D == 128 || D == 256, "layouts exist for 64, 128 and 256 elements per row");
+    if constexpr (D >= 128) {  // (a row of 256 elements is two bank sweeps: only the low four chunk bits matter)
         return chunk ^ (((row & 3) << 2) | ((row >> 2) & 3));
     } else {
         const int p = row >> 1;
@@ -198,7 +164,7 @@ struct SubTile {
 // dQ (and d rab)
 // ---------------------------------------------------------------------------------------------------------
 template <typename Tag, int D, bool HAS_RAB, bool HAS_MASK, bool WANT_DRAB>
-__global__ __launch_bounds__(256, 2) void hstu_bwd_dq_kernel(const BwdArgs a)
+__global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_bwd_dq_kernel(const BwdArgs a)
 {
     typedef SubTile<D> T;
     constexpr int LPW = T::LPW, NLW = T::NLW, KSTEPS = T::KSTEPS, MTILES = T::MTILES, NCH = 2 * T::MTILES;
@@ -535,10 +501,9 @@ __global__ __launch_bounds__(256, 2) void hstu_bwd_dq_kernel(const BwdArgs a)
 // ---------------------------------------------------------------------------------------------------------
 // dK, dV
 // ---------------------------------------------------------------------------------------------------------
-constexpr int kDkvThreads = 256;
 
 template <typename Tag, int D, bool HAS_RAB, bool HAS_MASK>
-__global__ __launch_bounds__(kDkvThreads, 2) void hstu_bwd_dkv_kernel(const BwdArgs a)
+__global__ __launch_bounds__(kDkvThreads, (D <= 128 ? 2 : 1)) void hstu_bwd_dkv_kernel(const BwdArgs a)
 {
     typedef SubTile<D> T;
     constexpr int LPW = T::LPW, NLW = T::NLW, KSTEPS = T::KSTEPS, MTILES = T::MTILES, NCH = 2 * T::MTILES;

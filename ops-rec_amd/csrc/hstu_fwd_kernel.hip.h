@@ -41,6 +41,8 @@
 
 #include <type_traits>
 
+#include "hstu_args.h"
+
 namespace hstu {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
@@ -65,8 +67,6 @@ struct elem_traits<f8_tag> {
     static constexpr bool kF8 = true;
 };
 
-constexpr int kBlockM = 128;  // query rows per workgroup
-constexpr int kWaveM = 32;    // query rows per wavefront
 constexpr uint32_t kBufferFlags = 0x00020000u;  // raw buffer, 32-bit data format (gfx9 family)
 constexpr uint32_t kOutOfRange = 0x80000000u;   // byte offset no descriptor here can contain
 
@@ -89,56 +89,6 @@ constexpr uint32_t kOutOfRange = 0x80000000u;   // byte offset no descriptor her
     } while (0)
 #endif
 
-struct FwdArgs {
-    const void* q;
-    const void* k;
-    const void* v;
-    const void* rab;
-    const void* mask;
-    void* out;
-    const void* offs_q;
-    const void* offs_k;
-    const void* num_ctx;
-    const void* num_tgt;
-    int64_t total_q;
-    int64_t total_k;
-    int n_batch;   // n_offsets - 1
-    int n_heads_q;
-    int n_heads_k;
-    int head_ratio;  // n_heads_q / n_heads_k
-    int d_qk;        // real head dims (<= the padded template dim)
-    int d_v;
-    int max_q;
-    int max_k;
-    int mask_type;
-    int target_group;
-    int idx64;       // offsets / context / target are int64
-    int n_qtiles;    // ceil(max_q / kBlockM)
-    int bh;          // n_batch * n_heads_q
-    int bias_vec_ok; // rab / mask rows may be read 4 elements (8 bytes) at a time
-    float c_exp;     // -alpha * log2(e)
-    float c_out;     // alpha * silu_scale
-    float alpha;     // fp8 inputs only: the kernel folds the per-head scales in itself
-    float silu_scale;
-    const float* q_descale;  // fp8 inputs only; per head, nullptr = 1
-    const float* k_descale;
-    const float* v_descale;
-    int counter_slot;  // which pair of device-side work counters this launch uses
-    float* ws;           // split variant: room for ws_parts partial outputs of kBlockM x D floats each (may be null)
-    uint32_t ws_parts;
-    // paged variant: the first (key count - num_target) key rows of a sequence live in pages of kv_cache
-    // [num_pages, 2 (K, V), page_size, n_heads_k, d]; k / v then hold the rows of ALL query tokens, of which the last
-    // num_target of each sequence are its remaining keys
-    const void* kv_cache;
-    const void* page_offsets;  // [n_batch + 1]
-    const void* page_ids;      // [n_page_ids]
-    int64_t num_pages;
-    int64_t n_page_ids;
-    int page_shift;  // log2(page_size); page_size is 32, 64, 128 or 256
-#ifdef HSTU_TIMELINE
-    unsigned long long* timeline;
-#endif
-};
 
 __device__ __forceinline__ int64_t load_index(const void* p, int64_t i, int idx64)
 {
@@ -366,7 +316,6 @@ __device__ __forceinline__ void load_to_lds_b128(__amdgpu_buffer_rsrc_t rsrc, ui
 // robin), so launches that overlap on one GPU do not share a set unless more than kCounterSlots of
 // them are in flight.  Zero at module load; the last workgroup of a launch to leave puts its set
 // back to zero.
-constexpr int kCounterSlots = 64;
 constexpr int kQueues = 8;          // one work queue per XCD (MI355X: 8 XCDs; workgroup w runs on XCD w mod 8)
 constexpr int kCounterStride = 32;  // counters of different queues sit in different 128-byte lines
 static __device__ unsigned int g_work_counter[kCounterSlots][kQueues * kCounterStride];

@@ -15,12 +15,12 @@
 #include <cstdio>
 #include <cstring>
 
-#include "hstu_fwd_f32_kernel.hip.h"
-#include "hstu_bwd_kernel.hip.h"
-#include "hstu_fwd_kernel.hip.h"
-#include "hstu_paged_gather.hip.h"
+#include "hstu_variants.h"
 
 namespace {
+
+using hstu::BwdVariant;
+using hstu::Variant;
 
 thread_local char g_err[512] = "";
 
@@ -33,20 +33,6 @@ int fail(int code, const char* fmt, ...)
     return code;
 }
 
-// kernel variants with the per-XCD work queues, and with split items, exist for the head-dim slots 64 and 128
-// (nullptr elsewhere)
-struct Variant {
-    const char* name;
-    const char* name_queues;
-    const char* name_split;
-    void (*kernel)(const hstu::FwdArgs);
-    void (*kernel_queues)(const hstu::FwdArgs);  // the same with per-XCD work queues, for long lists; may be nullptr
-    void (*kernel_split)(const hstu::FwdArgs);   // the same with long items split over workgroups, for short lists
-    void (*kernel_paged)(const hstu::FwdArgs);   // split variant that reads K / V through a page table; may be nullptr
-    int d_pad;
-    int threads;
-    int persistent_wgs_per_cu;  // > 0: persistent kernel, this many workgroups per CU; 0: one workgroup per tile
-};
 
 // compute units of each device, looked up once
 int compute_units(int* out)
@@ -74,76 +60,6 @@ int compute_units(int* out)
 
 std::atomic<unsigned> g_next_counter_slot{0};
 
-template <typename Tag, typename OutTag, int D, bool RAB, bool MASK>
-constexpr auto queues_kernel() -> void (*)(const hstu::FwdArgs)
-{
-    if constexpr (D == 64 || D == 128) {
-        return hstu::hstu_fwd_kernel<Tag, OutTag, D, RAB, MASK, true>;
-    } else {
-        return nullptr;
-    }
-}
-
-template <typename Tag, typename OutTag, int D, bool RAB, bool MASK>
-constexpr auto split_kernel() -> void (*)(const hstu::FwdArgs)
-{
-    if constexpr (D == 64 || D == 128) {
-        return hstu::hstu_fwd_kernel<Tag, OutTag, D, RAB, MASK, false, true>;
-    } else {
-        return nullptr;
-    }
-}
-
-template <typename Tag, typename OutTag, int D, bool RAB, bool MASK>
-constexpr auto paged_kernel() -> void (*)(const hstu::FwdArgs)
-{
-    if constexpr (D == 64 || D == 128) {
-        return hstu::hstu_fwd_kernel<Tag, OutTag, D, RAB, MASK, false, true, true>;
-    } else {
-        return nullptr;
-    }
-}
-
-#define HSTU_VARIANT(tag, tagname, D, RAB, MASK, WGS)                                               \
-    {"hstu_fwd_" tagname "_d" #D "_rab" #RAB "_mask" #MASK,                                        \
-     "hstu_fwd_" tagname "_d" #D "_rab" #RAB "_mask" #MASK "_queues",                               \
-     "hstu_fwd_" tagname "_d" #D "_rab" #RAB "_mask" #MASK "_split",                                \
-     hstu::hstu_fwd_kernel<hstu::tag, hstu::tag, D, RAB, MASK>,                                     \
-     queues_kernel<hstu::tag, hstu::tag, D, RAB, MASK>(),                                           \
-     split_kernel<hstu::tag, hstu::tag, D, RAB, MASK>(), paged_kernel<hstu::tag, hstu::tag, D, RAB, MASK>(), D, 256, WGS}
-#define HSTU_DIMS(tag, tagname, RAB, MASK)                                                           \
-    {HSTU_VARIANT(tag, tagname, 32, RAB, MASK, 2), HSTU_VARIANT(tag, tagname, 64, RAB, MASK, 2), \
-     HSTU_VARIANT(tag, tagname, 128, RAB, MASK, 2), HSTU_VARIANT(tag, tagname, 256, RAB, MASK, 1)}
-
-// [dtype: bf16, f16][rab: 0, 1][custom mask: 0, 1][dim slot: 32, 64, 128, 256]
-const Variant kVariants[2][2][2][4] = {
-    {{HSTU_DIMS(bf16_tag, "bf16", false, false), HSTU_DIMS(bf16_tag, "bf16", false, true)},
-     {HSTU_DIMS(bf16_tag, "bf16", true, false), HSTU_DIMS(bf16_tag, "bf16", true, true)}},
-    {{HSTU_DIMS(f16_tag, "f16", false, false), HSTU_DIMS(f16_tag, "f16", false, true)},
-     {HSTU_DIMS(f16_tag, "f16", true, false), HSTU_DIMS(f16_tag, "f16", true, true)}},
-};
-
-#define HSTU_F32_VARIANT(D, RAB, MASK) \
-    {"hstu_fwd_f32_d" #D "_rab" #RAB "_mask" #MASK, nullptr, nullptr, hstu::hstu_fwd_f32_kernel<D, RAB, MASK>, nullptr, nullptr, nullptr, D, 256, 0}
-#define HSTU_F32_DIMS(RAB, MASK) \
-    {HSTU_F32_VARIANT(32, RAB, MASK), HSTU_F32_VARIANT(64, RAB, MASK), HSTU_F32_VARIANT(128, RAB, MASK), \
-     HSTU_F32_VARIANT(256, RAB, MASK)}
-// fp32 inputs: [rab][custom mask][dim slot]
-// fp8-e4m3 inputs: [output: fp16, bf16][dim slot: 64, 128, 256] (no rab, no custom mask)
-#define HSTU_F8_VARIANT(otag, oname, D, WGS)                                                         \
-    {"hstu_fwd_f8e4m3_" oname "_d" #D, "hstu_fwd_f8e4m3_" oname "_d" #D "_queues",                              \
-     "hstu_fwd_f8e4m3_" oname "_d" #D "_split",                                                                  \
-     hstu::hstu_fwd_kernel<hstu::f8_tag, hstu::otag, D, false, false>,                                         \
-     queues_kernel<hstu::f8_tag, hstu::otag, D, false, false>(),                                               \
-     split_kernel<hstu::f8_tag, hstu::otag, D, false, false>(), nullptr, D, 256, WGS}
-const Variant kVariantsF8[2][3] = {
-    {HSTU_F8_VARIANT(f16_tag, "f16", 64, 2), HSTU_F8_VARIANT(f16_tag, "f16", 128, 2), HSTU_F8_VARIANT(f16_tag, "f16", 256, 1)},
-    {HSTU_F8_VARIANT(bf16_tag, "bf16", 64, 2), HSTU_F8_VARIANT(bf16_tag, "bf16", 128, 2),
-     HSTU_F8_VARIANT(bf16_tag, "bf16", 256, 1)},
-};
-
-const Variant kVariantsF32[2][2][4] = {{HSTU_F32_DIMS(false, false), HSTU_F32_DIMS(false, true)},
-                                       {HSTU_F32_DIMS(true, false), HSTU_F32_DIMS(true, true)}};
 
 int validate(const hstu_jagged_fwd_params* p, bool need_out = true)
 {
@@ -272,13 +188,13 @@ const Variant* select(const hstu_jagged_fwd_params* p)
         }
     }
     if (p->dtype == HSTU_DT_FP8_E4M3) {
-        return &kVariantsF8[p->out_dtype == HSTU_DT_FP16 ? 0 : 1][slot <= 1 ? 0 : slot - 1];
+        return &hstu::fwd_variants_f8()[p->out_dtype == HSTU_DT_FP16 ? 0 : 1][slot <= 1 ? 0 : slot - 1];
     }
     if (p->dtype == HSTU_DT_FP32) {
-        return &kVariantsF32[p->attn_bias != nullptr ? 1 : 0][p->mask_type == HSTU_MASK_CUSTOM ? 1 : 0][slot];
+        return &hstu::fwd_variants_f32()[p->attn_bias != nullptr ? 1 : 0][p->mask_type == HSTU_MASK_CUSTOM ? 1 : 0][slot];
     }
-    return &kVariants[p->dtype == HSTU_DT_BF16 ? 0 : 1][p->attn_bias != nullptr ? 1 : 0]
-                     [p->mask_type == HSTU_MASK_CUSTOM ? 1 : 0][slot];
+    const auto* table = p->dtype == HSTU_DT_BF16 ? hstu::fwd_variants_bf16() : hstu::fwd_variants_f16();
+    return &table[p->attn_bias != nullptr ? 1 : 0][p->mask_type == HSTU_MASK_CUSTOM ? 1 : 0][slot];
 }
 
 // whether the launch described by p takes the variant with per-XCD work queues: only when the list may hold
@@ -341,34 +257,6 @@ uint64_t split_workspace_bytes(const Variant* var, const hstu_jagged_fwd_params*
 }
 
 // ---- backward -------------------------------------------------------------------------------------------
-struct BwdVariant {
-    const char* name;
-    void (*dkv)(const hstu::BwdArgs);
-    void (*dq)(const hstu::BwdArgs);       // without d rab
-    void (*dq_drab)(const hstu::BwdArgs);  // with d rab (nullptr when the variant has no rab)
-};
-template <typename Tag, int D, bool RAB, bool MASK>
-constexpr auto dq_drab_kernel() -> void (*)(const hstu::BwdArgs)
-{
-    if constexpr (RAB) {
-        return hstu::hstu_bwd_dq_kernel<Tag, D, RAB, MASK, true>;
-    } else {
-        return nullptr;
-    }
-}
-#define HSTU_BWD_VARIANT(tag, tagname, D, RAB, MASK)                                             \
-    {"hstu_bwd_" tagname "_d" #D "_rab" #RAB "_mask" #MASK,                                      \
-     hstu::hstu_bwd_dkv_kernel<hstu::tag, D, RAB, MASK>,                                         \
-     hstu::hstu_bwd_dq_kernel<hstu::tag, D, RAB, MASK, false>, dq_drab_kernel<hstu::tag, D, RAB, MASK>()}
-#define HSTU_BWD_DIMS(tag, tagname, RAB, MASK) \
-    {HSTU_BWD_VARIANT(tag, tagname, 64, RAB, MASK), HSTU_BWD_VARIANT(tag, tagname, 128, RAB, MASK)}
-// [dtype: bf16, f16][rab][custom mask][dim slot: 64, 128]
-const BwdVariant kBwdVariants[2][2][2][2] = {
-    {{HSTU_BWD_DIMS(bf16_tag, "bf16", false, false), HSTU_BWD_DIMS(bf16_tag, "bf16", false, true)},
-     {HSTU_BWD_DIMS(bf16_tag, "bf16", true, false), HSTU_BWD_DIMS(bf16_tag, "bf16", true, true)}},
-    {{HSTU_BWD_DIMS(f16_tag, "f16", false, false), HSTU_BWD_DIMS(f16_tag, "f16", false, true)},
-     {HSTU_BWD_DIMS(f16_tag, "f16", true, false), HSTU_BWD_DIMS(f16_tag, "f16", true, true)}},
-};
 
 int validate_bwd(const hstu_jagged_bwd_params* p)
 {
@@ -403,8 +291,8 @@ const BwdVariant* select_bwd(const hstu_jagged_bwd_params* p)
         return nullptr;
     }
     const int64_t dmax = f->head_dim_qk > f->head_dim_v ? f->head_dim_qk : f->head_dim_v;
-    if (dmax > 128 || f->head_dim_qk % 8 != 0) {
-        fail(HSTU_ERR_UNSUPPORTED, "the backward is built for head dims up to 128, q/k head dim a multiple of 8 (got %lld / %lld)",
+    if (dmax > 256 || f->head_dim_qk % 8 != 0) {
+        fail(HSTU_ERR_UNSUPPORTED, "the backward is built for head dims up to 256, q/k head dim a multiple of 8 (got %lld / %lld)",
              (long long)f->head_dim_qk, (long long)f->head_dim_v);
         return nullptr;
     }
@@ -416,8 +304,8 @@ const BwdVariant* select_bwd(const hstu_jagged_bwd_params* p)
         fail(HSTU_ERR_UNSUPPORTED, "max_seq_len x heads x head dim spans 1 GiB or more per sequence");
         return nullptr;
     }
-    return &kBwdVariants[f->dtype == HSTU_DT_BF16 ? 0 : 1][f->attn_bias != nullptr ? 1 : 0]
-                        [f->mask_type == HSTU_MASK_CUSTOM ? 1 : 0][dmax <= 64 ? 0 : 1];
+    const auto* table = f->dtype == HSTU_DT_BF16 ? hstu::bwd_variants_bf16() : hstu::bwd_variants_f16();
+    return &table[f->attn_bias != nullptr ? 1 : 0][f->mask_type == HSTU_MASK_CUSTOM ? 1 : 0][dmax <= 64 ? 0 : (dmax <= 128 ? 1 : 2)];
 }
 
 // ---- paged K/V --------------------------------------------------------------------------------------------
@@ -549,8 +437,7 @@ HSTU_API int hstu_paged_fwd(const hstu_paged_fwd_params* p, void* workspace, uin
         a.page_size = static_cast<int>(p->page_size);
         a.row_bytes = static_cast<int>(p->fwd.num_heads_k * p->fwd.head_dim_qk * (p->fwd.dtype == HSTU_DT_FP32 ? 4 : 2));
         a.idx64 = (p->fwd.index_dtype == HSTU_IDX_I64) ? 1 : 0;
-        hipLaunchKernelGGL(hstu::hstu_paged_gather_kernel, dim3(static_cast<unsigned>(p->fwd.total_k)),
-                           dim3(hstu::kGatherThreads), 0, static_cast<hipStream_t>(stream), a);
+        hstu::launch_paged_gather(a, static_cast<unsigned>(p->fwd.total_k), static_cast<hipStream_t>(stream));
         const hipError_t err = hipGetLastError();
         if (err != hipSuccess) {
             return fail(HSTU_ERR_RUNTIME, "launch of the paged gather failed: %s", hipGetErrorString(err));

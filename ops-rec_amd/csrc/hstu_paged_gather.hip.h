@@ -16,28 +16,7 @@
 
 namespace hstu {
 
-struct PagedGatherArgs {
-    const void* k;         // [total_q, heads_k, dim]: rows of all tokens; only the target rows are used
-    const void* v;
-    const void* kv_cache;  // [num_pages, 2, page_size, heads_k, dim]
-    void* k_out;           // [total_k, heads_k, dim]
-    void* v_out;
-    const void* offs_q;    // [n_batch + 1]
-    const void* offs_k;    // [n_batch + 1]
-    const void* page_offsets;  // [n_batch + 1]
-    const void* page_ids;      // [page_offsets[n_batch]]
-    const void* num_tgt;       // [n_batch]
-    int64_t total_q;
-    int64_t total_k;
-    int64_t num_pages;
-    int64_t n_page_ids;
-    int n_batch;
-    int page_size;
-    int row_bytes;  // heads_k * dim * element size, a multiple of 16
-    int idx64;
-};
 
-constexpr int kGatherThreads = 128;
 
 __global__ __launch_bounds__(kGatherThreads) void hstu_paged_gather_kernel(const PagedGatherArgs a)
 {

@@ -1,0 +1,54 @@
+// Builders of the variant tables; included by the translation units that instantiate forward kernels.
+#pragma once
+#include "hstu_fwd_kernel.hip.h"
+#include "hstu_variants.h"
+
+namespace hstu {
+
+template <typename Tag, typename OutTag, int D, bool RAB, bool MASK>
+constexpr auto queues_kernel() -> void (*)(const FwdArgs)
+{
+    if constexpr (D == 64 || D == 128) {
+        return hstu_fwd_kernel<Tag, OutTag, D, RAB, MASK, true>;
+    } else {
+        return nullptr;
+    }
+}
+
+template <typename Tag, typename OutTag, int D, bool RAB, bool MASK>
+constexpr auto split_kernel() -> void (*)(const FwdArgs)
+{
+    if constexpr (D == 64 || D == 128) {
+        return hstu_fwd_kernel<Tag, OutTag, D, RAB, MASK, false, true>;
+    } else {
+        return nullptr;
+    }
+}
+
+template <typename Tag, typename OutTag, int D, bool RAB, bool MASK>
+constexpr auto paged_kernel() -> void (*)(const FwdArgs)
+{
+    if constexpr (D == 64 || D == 128) {
+        return hstu_fwd_kernel<Tag, OutTag, D, RAB, MASK, false, true, true>;
+    } else {
+        return nullptr;
+    }
+}
+
+}  // namespace hstu
+
+#define HSTU_VARIANT(tag, tagname, D, RAB, MASK, WGS)                                               \
+    {"hstu_fwd_" tagname "_d" #D "_rab" #RAB "_mask" #MASK,                                        \
+     "hstu_fwd_" tagname "_d" #D "_rab" #RAB "_mask" #MASK "_queues",                               \
+     "hstu_fwd_" tagname "_d" #D "_rab" #RAB "_mask" #MASK "_split",                                \
+     hstu::hstu_fwd_kernel<hstu::tag, hstu::tag, D, RAB, MASK>,                                     \
+     hstu::queues_kernel<hstu::tag, hstu::tag, D, RAB, MASK>(),                                     \
+     hstu::split_kernel<hstu::tag, hstu::tag, D, RAB, MASK>(),                                      \
+     hstu::paged_kernel<hstu::tag, hstu::tag, D, RAB, MASK>(), D, 256, WGS}
+#define HSTU_DIMS(tag, tagname, RAB, MASK)                                                           \
+    {HSTU_VARIANT(tag, tagname, 32, RAB, MASK, 2), HSTU_VARIANT(tag, tagname, 64, RAB, MASK, 2), \
+     HSTU_VARIANT(tag, tagname, 128, RAB, MASK, 2), HSTU_VARIANT(tag, tagname, 256, RAB, MASK, 1)}
+// one 16-bit input type: [rab][custom mask][dim slot]
+#define HSTU_FWD16_TABLE(tag, tagname)                                         \
+    {{HSTU_DIMS(tag, tagname, false, false), HSTU_DIMS(tag, tagname, false, true)}, \
+     {HSTU_DIMS(tag, tagname, true, false), HSTU_DIMS(tag, tagname, true, true)}}

@@ -1,0 +1,45 @@
+// Tables of kernel variants.  The kernels are instantiated in several translation units (one per input type and
+// direction, so that they compile side by side); each unit hands out its table through one of the functions below.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "hstu_args.h"
+
+namespace hstu {
+
+// kernel variants with the per-XCD work queues, with split items and with paged keys exist for the head-dim slots
+// 64 and 128 (nullptr elsewhere)
+struct Variant {
+    const char* name;
+    const char* name_queues;
+    const char* name_split;
+    void (*kernel)(const FwdArgs);
+    void (*kernel_queues)(const FwdArgs);  // the same with per-XCD work queues, for long lists; may be nullptr
+    void (*kernel_split)(const FwdArgs);   // the same with long items split over workgroups, for short lists
+    void (*kernel_paged)(const FwdArgs);   // split variant that reads K / V through a page table; may be nullptr
+    int d_pad;
+    int threads;
+    int persistent_wgs_per_cu;  // > 0: persistent kernel, this many workgroups per CU; 0: one workgroup per tile
+};
+
+struct BwdVariant {
+    const char* name;
+    void (*dkv)(const BwdArgs);
+    void (*dq)(const BwdArgs);       // without d rab
+    void (*dq_drab)(const BwdArgs);  // with d rab (nullptr when the variant has no rab)
+};
+
+// forward, 16-bit inputs: [rab: 0, 1][custom mask: 0, 1][dim slot: 32, 64, 128, 256]
+const Variant (*fwd_variants_bf16())[2][4];
+const Variant (*fwd_variants_f16())[2][4];
+// forward, fp8-e4m3 inputs: [output: fp16, bf16][dim slot: 64, 128, 256] (no rab, no custom mask)
+const Variant (*fwd_variants_f8())[3];
+// forward, fp32 inputs: [rab][custom mask][dim slot: 32, 64, 128, 256]
+const Variant (*fwd_variants_f32())[2][4];
+// backward: [rab][custom mask][dim slot: 64, 128, 256]
+const BwdVariant (*bwd_variants_bf16())[2][3];
+const BwdVariant (*bwd_variants_f16())[2][3];
+// the copy kernel in front of the forward for paged keys that no paged kernel variant covers
+void launch_paged_gather(const PagedGatherArgs& a, unsigned grid, hipStream_t stream);
+
+}  // namespace hstu

@@ -5,19 +5,29 @@ from __future__ import annotations
 import os
 import shutil
 import subprocess
+import tempfile
+from concurrent.futures import ThreadPoolExecutor
 
 _PKG = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(os.path.dirname(_PKG), "csrc")
 LIB_DIR = os.path.join(_PKG, "_lib")
 LIB_PATH = os.path.join(LIB_DIR, "libhstu_mi355.so")
 
-SOURCES = ["hstu_mi355.hip"]
+# the host side, and the kernels by input type and direction: one translation unit each, compiled side by side
+SOURCES = [
+    "hstu_mi355.hip",
+    "hstu_kernels_fwd_bf16.hip",
+    "hstu_kernels_fwd_f16.hip",
+    "hstu_kernels_fwd_f8.hip",
+    "hstu_kernels_fwd_f32.hip",
+    "hstu_kernels_bwd_bf16.hip",
+    "hstu_kernels_bwd_f16.hip",
+]
 HIPCC_FLAGS = [
     "--offload-arch=gfx950",
     "-O3",
     "-std=c++17",
     "-fPIC",
-    "-shared",
     "-fvisibility=hidden",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
 ]  # fmt: skip
@@ -30,15 +40,29 @@ def hipcc_path() -> str:
     raise RuntimeError("hipcc not found; the HIP library cannot be built")
 
 
-def build(verbose: bool = False) -> str:
-    """Compile ``csrc/*.hip`` into ``ops_rec/_lib/libhstu_mi355.so`` (always recompiles)."""
-    os.makedirs(LIB_DIR, exist_ok=True)
-    tmp = LIB_PATH + ".tmp"
-    cmd = [hipcc_path(), *HIPCC_FLAGS, "-o", tmp, *[os.path.join(CSRC, s) for s in SOURCES]]
+def _run(cmd: list[str], verbose: bool) -> None:
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if res.returncode != 0:
-        raise RuntimeError(f"hipcc failed ({res.returncode}):\n{res.stdout}")
+        raise RuntimeError(f"hipcc failed ({res.returncode}): {' '.join(cmd)}\n{res.stdout}")
+
+
+def build(verbose: bool = False, jobs: int | None = None) -> str:
+    """Compile ``csrc/*.hip`` into ``ops_rec/_lib/libhstu_mi355.so`` (always recompiles every source)."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    hipcc = hipcc_path()
+    jobs = jobs or max(1, min(len(SOURCES), os.cpu_count() or 1, int(os.environ.get("MAX_JOBS", "16"))))
+    with tempfile.TemporaryDirectory(prefix="hstu_build_") as obj_dir:
+        objects = [os.path.join(obj_dir, os.path.splitext(s)[0] + ".o") for s in SOURCES]
+        with ThreadPoolExecutor(max_workers=jobs) as pool:
+            jobs_done = [
+                pool.submit(_run, [hipcc, *HIPCC_FLAGS, "-c", os.path.join(CSRC, s), "-o", o], verbose)
+                for s, o in zip(SOURCES, objects)
+            ]
+            for j in jobs_done:
+                j.result()
+        tmp = LIB_PATH + ".tmp"
+        _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objects], verbose)
     os.replace(tmp, LIB_PATH)
     return LIB_PATH

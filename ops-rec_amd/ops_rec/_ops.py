@@ -318,7 +318,7 @@ def hstu_jagged_delta_meta(q, k, v, mask=None, attn_bias=None, mask_type=0, max_
 
 
 # ----------------------------------------------------------------------------------------------
-# backward op: HIP kernels through the C ABI for bf16 / fp16 with head dims up to 128 (_backward_hip); a
+# backward op: HIP kernels through the C ABI for bf16 / fp16 with head dims up to 256 (_backward_hip); a
 # device-side composite (torch ops on the GPU, per sequence, fp32) for the rest (fp32 inputs, larger head
 # dims), which is also what HSTU_MI355_COMPOSITE_BACKWARD=1 selects for comparisons.
 #   X = alpha (S + rab),  sig = sigmoid(X),  P = X sig scale M
@@ -343,9 +343,9 @@ def _device_builtin_mask(s_q, s_k, ctx, tgt, group, device):
 
 
 def hip_backward_available(q, k, v) -> bool:
-    """Whether the HIP backward kernels cover these tensors (bf16 / fp16, head dims up to 128, q/k head dim a
+    """Whether the HIP backward kernels cover these tensors (bf16 / fp16, head dims up to 256, q/k head dim a
     multiple of 8); everything else takes the composite below."""
-    return (q.dtype in (torch.bfloat16, torch.float16) and max(q.shape[2], v.shape[2]) <= 128 and q.shape[2] % 8 == 0
+    return (q.dtype in (torch.bfloat16, torch.float16) and max(q.shape[2], v.shape[2]) <= 256 and q.shape[2] % 8 == 0
             and v.shape[2] % 16 == 0)  # fmt: skip
 
 

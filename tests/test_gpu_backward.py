@@ -81,7 +81,7 @@ def make(**kw):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
-@pytest.mark.parametrize("dim,dim_v", [(64, 64), (128, 128), (96, 64), (32, 16), (8, 128)])
+@pytest.mark.parametrize("dim,dim_v", [(64, 64), (128, 128), (96, 64), (32, 16), (8, 128), (256, 256), (136, 192)])
 def test_plain_causal(dim, dim_v, dtype, monkeypatch):
     check(make(batch=3, heads=2, dim=dim, dim_v=dim_v, lo=1, hi=300, seed=dim + dim_v, dtype=dtype), monkeypatch)
 

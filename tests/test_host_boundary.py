@@ -332,7 +332,7 @@ def test_backward_c_abi_validation_codes():
         (dict(fwd=dict(mask_type=1)), 161002, "triu"),
         (dict(fwd=dict(num_heads_k=3)), 161002, "divisible"),
         (dict(fwd=dict(dtype=_native.DT_FP32, out_dtype=_native.DT_FP32)), 161003, "bf16 and fp16"),
-        (dict(fwd=dict(head_dim_qk=256, head_dim_v=256)), 161003, "up to 128"),
+        (dict(fwd=dict(head_dim_qk=512, head_dim_v=512)), 161003, "up to 256"),
         (dict(fwd=dict(head_dim_qk=12, head_dim_v=16)), 161003, "multiple of 8"),
     ]:
         got = rc(make(**over))
