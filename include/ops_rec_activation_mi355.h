@@ -1,0 +1,51 @@
+/*
+ * C ABI of the MI355X (gfx950) build of the operators around HSTU attention in an HSTU layer.  Same library, status
+ * codes, dtype codes and error text (hstu_last_error) as hstu_mi355.h.
+ *
+ * ln_mul: out = LayerNorm(x) * u over the rows of a [rows, cols] matrix, with
+ *   LayerNorm(x) = (x - mean) * rstd * gamma + beta,  rstd = 1 / sqrt(var + epsilon),  var = mean((x - mean)^2).
+ *
+ * Replaces the two-phase pair aclnnLnMulGetWorkspaceSize / aclnnLnMul
+ * (ascendc/activation/ln_mul/docs/aclnn_ln_mul.md:26-41), which the reference's torch adapter calls through
+ * EXEC_NPU_CMD (ascendc/activation/ln_mul/torch_extension/ln_mul_plugin.cpp:49).  The aclTensor handles become plain
+ * device pointers plus the two extents; the op needs no workspace, so one call does both phases.
+ *
+ * Beyond the reference (fp32 only, ascendc/activation/ln_mul/op_host/ln_mul.cpp:111-135): x / u / out may be bf16
+ * or fp16 (the types the attention kernels write), with gamma / beta in fp32 or in that type; arithmetic is fp32.
+ */
+#ifndef OPS_REC_ACTIVATION_MI355_H
+#define OPS_REC_ACTIVATION_MI355_H
+
+#include "hstu_mi355.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct ln_mul_params {
+    uint32_t struct_size; /* sizeof(ln_mul_params), checked */
+    uint32_t reserved0;
+    const void* x;     /* [rows, cols], contiguous */
+    const void* u;     /* [rows, cols], contiguous */
+    const void* gamma; /* [cols] */
+    const void* beta;  /* [cols] */
+    void* out;         /* [rows, cols]; every element is written */
+    int64_t rows;
+    int64_t cols;
+    int32_t dtype;        /* of x, u, out: HSTU_DT_FP32 (the reference's), HSTU_DT_BF16, HSTU_DT_FP16 */
+    int32_t affine_dtype; /* of gamma, beta: HSTU_DT_FP32 or equal to dtype */
+    float epsilon;        /* the reference fixes 1e-5 (ascendc/activation/ln_mul/op_host/ln_mul.cpp:75) */
+    uint32_t reserved1;
+} ln_mul_params;
+
+/* Launches the kernel on `stream` (a hipStream_t; NULL = the default stream) and returns without waiting.
+ * HSTU_OK, or HSTU_ERR_NULLPTR / HSTU_ERR_INVALID (nothing launched) / HSTU_ERR_RUNTIME. */
+HSTU_API int ln_mul_fwd(const ln_mul_params* params, void* stream);
+
+/* name of the kernel variant ln_mul_fwd would launch (for profiles and logs), or NULL after an error */
+HSTU_API const char* ln_mul_fwd_kernel_name(const ln_mul_params* params);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -117,4 +117,19 @@ struct PagedGatherArgs {
     int idx64;
 };
 
+// LayerNorm(x) * u over rows (ln_mul_kernel.hip.h)
+constexpr int kLnMulThreads = 256;
+
+struct LnMulArgs {
+    const void* x;      // [rows, cols]
+    const void* u;      // [rows, cols]
+    const void* gamma;  // [cols], fp32 or the element type of x
+    const void* beta;   // [cols], like gamma
+    void* out;          // [rows, cols]
+    int64_t rows;
+    int64_t cols;
+    float epsilon;
+    int affine_f32;  // 1: gamma / beta are fp32; 0: they have the element type of x
+};
+
 }  // namespace hstu

@@ -15,16 +15,14 @@
 #include <cstdio>
 #include <cstring>
 
+#include "hstu_error.h"
 #include "hstu_variants.h"
 
 namespace {
-
-using hstu::BwdVariant;
-using hstu::Variant;
-
 thread_local char g_err[512] = "";
+}
 
-int fail(int code, const char* fmt, ...)
+int hstu::set_error(int code, const char* fmt, ...)
 {
     va_list ap;
     va_start(ap, fmt);
@@ -32,6 +30,13 @@ int fail(int code, const char* fmt, ...)
     va_end(ap);
     return code;
 }
+
+namespace {
+
+using hstu::BwdVariant;
+using hstu::Variant;
+
+#define fail(...) hstu::set_error(__VA_ARGS__)
 
 
 // compute units of each device, looked up once

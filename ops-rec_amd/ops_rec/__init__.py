@@ -13,7 +13,8 @@ from __future__ import annotations
 
 import logging
 
-from . import _ops  # noqa: F401  (defines the operators)
+from . import _ops  # noqa: F401  (defines the attention operators)
+from . import _activation  # noqa: F401  (defines ln_mul)
 from . import ascendc  # noqa: F401
 from . import autograd  # noqa: F401  (registers the autograd formulas)
 from ._ops import hstu_jagged_fp8  # noqa: F401  (extension: fp8 inputs with per-head scales)

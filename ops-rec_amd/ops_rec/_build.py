@@ -16,6 +16,7 @@ LIB_PATH = os.path.join(LIB_DIR, "libhstu_mi355.so")
 # the host side, and the kernels by input type and direction: one translation unit each, compiled side by side
 SOURCES = [
     "hstu_mi355.hip",
+    "ln_mul_mi355.hip",
     "hstu_kernels_fwd_bf16.hip",
     "hstu_kernels_fwd_f16.hip",
     "hstu_kernels_fwd_f8.hip",

@@ -26,6 +26,8 @@ EXPORTED_SYMBOLS = (
     "hstu_jagged_bwd",
     "hstu_paged_fwd_workspace_size",
     "hstu_paged_fwd",
+    "ln_mul_fwd",
+    "ln_mul_fwd_kernel_name",
 )
 
 
@@ -101,6 +103,26 @@ class PagedParams(ctypes.Structure):
     ]
 
 
+class LnMulParams(ctypes.Structure):
+    """Mirror of ``ln_mul_params`` (include/ops_rec_activation_mi355.h)."""
+
+    _fields_ = [
+        ("struct_size", ctypes.c_uint32),
+        ("reserved0", ctypes.c_uint32),
+        ("x", ctypes.c_void_p),
+        ("u", ctypes.c_void_p),
+        ("gamma", ctypes.c_void_p),
+        ("beta", ctypes.c_void_p),
+        ("out", ctypes.c_void_p),
+        ("rows", ctypes.c_int64),
+        ("cols", ctypes.c_int64),
+        ("dtype", ctypes.c_int32),
+        ("affine_dtype", ctypes.c_int32),
+        ("epsilon", ctypes.c_float),
+        ("reserved1", ctypes.c_uint32),
+    ]
+
+
 _lib: Optional[ctypes.CDLL] = None
 
 
@@ -138,6 +160,10 @@ def load() -> ctypes.CDLL:
     lib.hstu_paged_fwd_workspace_size.argtypes = [ctypes.POINTER(PagedParams), ctypes.POINTER(ctypes.c_uint64)]
     lib.hstu_paged_fwd.restype = ctypes.c_int
     lib.hstu_paged_fwd.argtypes = [ctypes.POINTER(PagedParams), ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]
+    lib.ln_mul_fwd.restype = ctypes.c_int
+    lib.ln_mul_fwd.argtypes = [ctypes.POINTER(LnMulParams), ctypes.c_void_p]
+    lib.ln_mul_fwd_kernel_name.restype = ctypes.c_char_p
+    lib.ln_mul_fwd_kernel_name.argtypes = [ctypes.POINTER(LnMulParams)]
     _lib = lib
     return lib
 
@@ -149,6 +175,12 @@ def last_error() -> str:
 def new_params() -> FwdParams:
     p = FwdParams()
     p.struct_size = ctypes.sizeof(FwdParams)
+    return p
+
+
+def new_ln_mul_params() -> LnMulParams:
+    p = LnMulParams()
+    p.struct_size = ctypes.sizeof(LnMulParams)
     return p
 
 

@@ -8,7 +8,7 @@ hstu_jagged`` work, and an unknown name raises ``AttributeError`` listing what e
 import torch
 
 _NS = torch.ops.ops_rec
-_OPS = ("hstu_jagged", "hstu_jagged_backward")
+_OPS = ("hstu_jagged", "hstu_jagged_backward", "hstu_dense", "hstu_dense_backward", "hstu_paged")
 
 __all__ = [name for name in _OPS if hasattr(_NS, name)]
 for _name in __all__:
