@@ -51,6 +51,78 @@ def algorithmic_bytes(w, out_element_size: int) -> int:
     return n
 
 
+# HBM bytes per ln_mul launch by rows (cols 512, bf16), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a plain
+# copy of known size (profiles/ln_mul_bf16_c512_trace_and_counters.md)
+LN_MUL_MEASURED_TRAFFIC_BYTES = {20292: 62_457_000, 324672: 997_512_000}
+
+
+def bench_ln_mul(attn_out, stream, args):
+    """ln_mul through ``ln_mul_fwd`` of the C ABI, events on the launch stream.  Algorithmic bytes per launch:
+    x and u read once, out written once = 3 * rows * cols * element size (gamma / beta stay in cache)."""
+    import ctypes
+
+    import numpy as np
+    import torch
+
+    from ops_rec import _native
+    from oracle import ln_mul_oracle
+
+    lib = _native.load()
+    dev = attn_out.device
+    tokens, cols = attn_out.shape[0], attn_out.shape[1] * attn_out.shape[2]
+    cases = []
+    for rows in (tokens, 16 * tokens):
+        x = attn_out.reshape(tokens, cols).repeat(rows // tokens, 1).contiguous()
+        u = torch.randn(rows, cols, device=dev).to(x.dtype)
+        gamma, beta = torch.randn(cols, device=dev), torch.randn(cols, device=dev)
+        out = torch.empty_like(x)
+        p = _native.new_ln_mul_params()
+        p.x, p.u, p.gamma, p.beta, p.out = (t.data_ptr() for t in (x, u, gamma, beta, out))
+        p.rows, p.cols = rows, cols
+        p.dtype = _native.DT_BF16 if x.dtype == torch.bfloat16 else _native.DT_FP16
+        p.affine_dtype = _native.DT_FP32
+        p.epsilon = ln_mul_oracle.EPSILON
+        raw = ctypes.c_void_p(stream.cuda_stream)
+        n = max(20, args.steps)
+        for _ in range(5):
+            assert lib.ln_mul_fwd(ctypes.byref(p), raw) == 0, _native.last_error()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(n):
+            lib.ln_mul_fwd(ctypes.byref(p), raw)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) / n * 1e3
+        nbytes = 3 * rows * cols * x.element_size()
+        case = {
+            "rows": rows,
+            "cols": cols,
+            "kernel": lib.ln_mul_fwd_kernel_name(ctypes.byref(p)).decode(),
+            "avg_launch_us": round(us, 3),
+            "algorithmic_bytes": nbytes,
+            "roofline": {"bound": "hbm", "achieved": round(nbytes / us / 1e3, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                         "frac": round(nbytes / us / 1e3 / PEAK_HBM_GBS, 4),
+                         "traffic": LN_MUL_MEASURED_TRAFFIC_BYTES.get(rows) if cols == 512 else None},
+        }  # fmt: skip
+        if rows == tokens and not args.no_cpu:
+            # CPU: the numpy oracle (float64) on a sample of rows, single-threaded numpy
+            sample = min(rows, 4096)
+            f = lambda t: t[:sample].float().cpu().numpy()  # noqa: E731
+            xs, us_, gs, bs = f(x), f(u), gamma.cpu().numpy(), beta.cpu().numpy()
+            t0 = time.perf_counter()
+            want = ln_mul_oracle.ln_mul(xs, us_, gs, bs)
+            cpu_s = time.perf_counter() - t0
+            np.testing.assert_allclose(out[:sample].double().cpu().numpy(), want, rtol=2.0**-8, atol=2e-3)
+            case["cpu_baseline"] = {"value": round(3 * sample * cols * x.element_size() / cpu_s / 1e9, 3),
+                                    "unit": "GB/s", "cores": 1, "kind": "port",
+                                    "sample": f"first {sample} rows, numpy float64 oracle"}  # fmt: skip
+        cases.append(case)
+        del x, u, out
+    return {"note": "ln_mul_fwd of the C ABI back-to-back on one stream; x = the attention output as [tokens, heads * dim]",
+            "cases": cases}  # fmt: skip
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -58,6 +130,10 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="C2", choices=["C2", "C3", "C4", "C5"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--ln-mul", action="store_true",
+                    help="also time ln_mul (LayerNorm(x) * u, the operator that consumes the attention output) on the "
+                    "output of this workload viewed as [tokens, heads * dim] and on a matrix 16 times as tall, and add "
+                    "an 'ln_mul' object with its HBM roofline to the line")  # fmt: skip
     ap.add_argument("--backward", action="store_true",
                     help="also time hstu_jagged_backward (the two HIP backward kernels) on the same workload and add a "
                     "'backward' object to the line (bf16 workloads only)")  # fmt: skip
@@ -229,6 +305,10 @@ def main() -> int:
             "zero-fill of the attn_bias gradient when there is one); the kernels recompute S and dP (eight products "
             "issued for the five of the formula)",
         }
+
+    # ---- ln_mul (optional): the operator that takes the attention output next in an HSTU layer ----
+    if args.ln_mul:
+        result["ln_mul"] = bench_ln_mul(prepared.out, stream, args)
 
     # ---- CPU baseline: dense-padded fp32 golden path on this host's cores ----
     if not args.no_cpu and w_cpu is not None:

@@ -23,12 +23,17 @@ struct LnVariant {
 #define LN_VEC(tag, tagname, G, NV) \
     {"ln_mul_" tagname "_g" #G "_v" #NV, hstu::ln_mul_kernel<hstu::tag, G, NV, true>, G, (G) * (NV)}
 #define LN_ANY(tag, tagname, G) {"ln_mul_" tagname "_g" #G "_any", hstu::ln_mul_kernel<hstu::tag, G, 1, false>, G, 0}
-// by growing row length; the two element-wise forms (short rows, long rows) come last
-#define LN_TABLE(tag, tagname)                                                                                    \
-    {LN_VEC(tag, tagname, 8, 1),  LN_VEC(tag, tagname, 16, 1), LN_VEC(tag, tagname, 32, 1), LN_VEC(tag, tagname, 64, 1), \
-     LN_VEC(tag, tagname, 64, 2), LN_VEC(tag, tagname, 64, 4), LN_VEC(tag, tagname, 64, 8), LN_VEC(tag, tagname, 256, 4), \
-     LN_VEC(tag, tagname, 256, 8), LN_VEC(tag, tagname, 256, 16), LN_ANY(tag, tagname, 64), LN_ANY(tag, tagname, 256)}
-constexpr int kVecVariants = 10;
+// By growing capacity (lanes x chunks per lane); a row takes the first variant that holds it.  Measured on MI355X: a
+// tight fit with few chunks per lane streams fastest (lanes past the end of a row still issue their loads), and rows
+// of up to 64 chunks do better with several rows per wavefront than with one; the two element-wise forms (short
+// rows, long rows) come last.
+#define LN_TABLE(tag, tagname)                                                                                        \
+    {LN_VEC(tag, tagname, 8, 1),   LN_VEC(tag, tagname, 16, 1),  LN_VEC(tag, tagname, 8, 3),   LN_VEC(tag, tagname, 16, 2),  \
+     LN_VEC(tag, tagname, 16, 3),  LN_VEC(tag, tagname, 16, 4),  LN_VEC(tag, tagname, 32, 3),  LN_VEC(tag, tagname, 64, 2),  \
+     LN_VEC(tag, tagname, 64, 3),  LN_VEC(tag, tagname, 64, 4),  LN_VEC(tag, tagname, 64, 6),  LN_VEC(tag, tagname, 64, 8),  \
+     LN_VEC(tag, tagname, 256, 3), LN_VEC(tag, tagname, 256, 4), LN_VEC(tag, tagname, 256, 6), LN_VEC(tag, tagname, 256, 8), \
+     LN_VEC(tag, tagname, 256, 12), LN_VEC(tag, tagname, 256, 16), LN_ANY(tag, tagname, 64),   LN_ANY(tag, tagname, 256)}
+constexpr int kVecVariants = 18;
 const LnVariant kVariants[3][kVecVariants + 2] = {LN_TABLE(ln_bf16_tag, "bf16"), LN_TABLE(ln_f16_tag, "f16"),
                                                   LN_TABLE(ln_f32_tag, "f32")};
 

@@ -54,7 +54,8 @@ def test_reference_shape_matrix_fp32(r):
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("affine_f32", [False, True])
-@pytest.mark.parametrize("r", [8, 16, 64, 104, 512, 1000, 1024, 2048, 4096, 8192, 16384, 32768])
+@pytest.mark.parametrize("r", [8, 16, 64, 104, 192, 384, 512, 768, 1000, 1024, 1536, 2048, 3072, 4096, 6144, 8192, 12288,
+                               16384, 24576, 32768])
 def test_sixteen_bit_rows(dtype, affine_f32, r):
     for a in (1, 3, 130):
         check(*inputs(a, r, dtype, seed=a + r, affine_dtype=torch.float32 if affine_f32 else None))
@@ -68,8 +69,8 @@ def test_rows_that_are_not_whole_chunks(dtype, r):
         check(*inputs(a, r, dtype, seed=7 * a + r, affine_dtype=torch.float32))
 
 
-@pytest.mark.parametrize("r", [4096, 8192, 16384, 16388, 50000])
-def test_long_rows_fp32(r):
+@pytest.mark.parametrize("r", [96, 384, 768, 1536, 3072, 4096, 6144, 8192, 12288, 16384, 16388, 50000])
+def test_more_row_lengths_fp32(r):
     check(*inputs(9, r, torch.float32, seed=r))
 
 
@@ -169,7 +170,7 @@ def test_raw_c_abi_call_on_a_side_stream():
     s = torch.cuda.Stream(device=DEV)
     s.wait_stream(torch.cuda.current_stream())
     lib = _native.load()
-    assert lib.ln_mul_fwd_kernel_name(ctypes.byref(p)).decode() == "ln_mul_f32_g64_v4"
+    assert lib.ln_mul_fwd_kernel_name(ctypes.byref(p)).decode() == "ln_mul_f32_g64_v3"
     assert lib.ln_mul_fwd(ctypes.byref(p), ctypes.c_void_p(s.cuda_stream)) == 0
     s.synchronize()
     np.testing.assert_allclose(out.double().cpu().numpy(), oracle(x.cpu(), u.cpu(), gamma.cpu(), beta.cpu()),

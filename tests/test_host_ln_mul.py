@@ -85,14 +85,17 @@ def test_kernel_variant_selection():
         return lib.ln_mul_fwd_kernel_name(ctypes.byref(p)).decode()
 
     bf16 = dict(dtype=_native.DT_BF16)
-    # a row goes to as many lanes as it has 16-byte chunks, then to more chunks per lane, then to a whole workgroup
+    # a row goes to the variant with the smallest capacity (lanes x 16-byte chunks per lane) that holds it
     assert name(cols=4) == "ln_mul_f32_g8_v1"
     assert name(cols=32) == "ln_mul_f32_g8_v1"
     assert name(cols=64) == "ln_mul_f32_g16_v1"
-    assert name(cols=256) == "ln_mul_f32_g64_v1"
+    assert name(cols=96) == "ln_mul_f32_g8_v3"
+    assert name(cols=256) == "ln_mul_f32_g16_v4"
     assert name(cols=512) == "ln_mul_f32_g64_v2"
-    assert name(cols=512, **bf16) == "ln_mul_bf16_g64_v1"
-    assert name(cols=512, dtype=_native.DT_FP16, affine_dtype=_native.DT_FP16) == "ln_mul_f16_g64_v1"
+    assert name(cols=768) == "ln_mul_f32_g64_v3"
+    assert name(cols=512, **bf16) == "ln_mul_bf16_g16_v4"
+    assert name(cols=512, dtype=_native.DT_FP16, affine_dtype=_native.DT_FP16) == "ln_mul_f16_g16_v4"
+    assert name(cols=12288) == "ln_mul_f32_g256_v12"
     assert name(cols=2048) == "ln_mul_f32_g64_v8"
     assert name(cols=4096) == "ln_mul_f32_g256_v4"
     assert name(cols=16384) == "ln_mul_f32_g256_v16"
