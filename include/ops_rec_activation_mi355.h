@@ -2,6 +2,8 @@
  * C ABI of the MI355X (gfx950) build of the operators around HSTU attention in an HSTU layer.  Same library, status
  * codes, dtype codes and error text (hstu_last_error) as hstu_mi355.h.
  *
+ * Two operators: ln_mul (consumes the attention output) and in_linear_silu (produces U, V, Q, K in front of it).
+ *
  * ln_mul: out = LayerNorm(x) * u over the rows of a [rows, cols] matrix, with
  *   LayerNorm(x) = (x - mean) * rstd * gamma + beta,  rstd = 1 / sqrt(var + epsilon),  var = mean((x - mean)^2).
  *
@@ -44,6 +46,43 @@ HSTU_API int ln_mul_fwd(const ln_mul_params* params, void* stream);
 
 /* name of the kernel variant ln_mul_fwd would launch (for profiles and logs), or NULL after an error */
 HSTU_API const char* ln_mul_fwd_kernel_name(const ln_mul_params* params);
+
+/*
+ * in_linear_silu forward: mixed = x @ weight^T + bias; linear_output = mixed; (user, value, query, key) =
+ * split(silu(mixed), split, last dim).  linear_output is mixed rounded to the type of x, and SiLU is taken of that
+ * rounded value, as the reference's kernel does.
+ *
+ * Replaces the two-phase pair aclnnInLinearSiluGetWorkspaceSize / aclnnInLinearSilu
+ * (ascendc/activation/in_linear_silu/in_linear_silu_forward/docs/aclnn_in_linear_silu.md), which the reference's torch
+ * adapter calls through EXEC_NPU_CMD (ascendc/activation/in_linear_silu/torch_extension/in_linear_silu_plugin.cpp:85-86).
+ * Limits as in that adapter (in_linear_silu_plugin.cpp:36-66): k in [16, 8192] and n in [64, 32768], multiples of 16;
+ * every split in [16, 8192], a multiple of 16, the four adding up to n; n a multiple of 4 k.
+ */
+typedef struct in_linear_silu_params {
+    uint32_t struct_size; /* sizeof(in_linear_silu_params), checked */
+    uint32_t reserved0;
+    const void* x;       /* [m, k], bf16 or fp16, contiguous, 16-byte aligned */
+    const void* weight;  /* [n, k], type of x */
+    const float* bias;   /* [n] fp32, or NULL for no bias */
+    void* user;          /* [m, split[0]], type of x */
+    void* value;         /* [m, split[1]] */
+    void* query;         /* [m, split[2]] */
+    void* key;           /* [m, split[3]] */
+    void* linear_output; /* [m, n] */
+    int64_t m;
+    int64_t n;
+    int64_t k;
+    int64_t split[4];
+    int32_t dtype; /* HSTU_DT_BF16 or HSTU_DT_FP16 */
+    uint32_t reserved1;
+} in_linear_silu_params;
+
+/* Launches the kernel on `stream` and returns without waiting.  HSTU_OK, or HSTU_ERR_NULLPTR / HSTU_ERR_INVALID
+ * (nothing launched) / HSTU_ERR_RUNTIME. */
+HSTU_API int in_linear_silu_fwd(const in_linear_silu_params* params, void* stream);
+
+/* name of the kernel variant in_linear_silu_fwd would launch, or NULL after an error */
+HSTU_API const char* in_linear_silu_fwd_kernel_name(const in_linear_silu_params* params);
 
 #ifdef __cplusplus
 }

@@ -132,4 +132,20 @@ struct LnMulArgs {
     int affine_f32;  // 1: gamma / beta are fp32; 0: they have the element type of x
 };
 
+// in_linear_silu forward (in_linear_silu_kernel.hip.h)
+struct InLinearSiluArgs {
+    const void* x;       // [m, k], 16-bit
+    const void* weight;  // [n, k], 16-bit
+    const float* bias;   // [n] or nullptr
+    void* user;          // [m, split_end[0]]
+    void* value;         // [m, split_end[1] - split_end[0]]
+    void* query;         // [m, split_end[2] - split_end[1]]
+    void* key;           // [m, n - split_end[2]]
+    void* linear_output; // [m, n]
+    int64_t m;
+    int n;
+    int k;
+    int split_end[3];  // first column after the user, value and query parts
+};
+
 }  // namespace hstu

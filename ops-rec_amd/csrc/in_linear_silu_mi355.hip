@@ -1,0 +1,133 @@
+// C ABI of in_linear_silu forward: argument checks, choice of the kernel variant, launch.  Host-side counterpart of
+// the reference's adapter checks (ascendc/activation/in_linear_silu/torch_extension/in_linear_silu_plugin.cpp:36-66)
+// and of its host tiling (ascendc/activation/in_linear_silu/in_linear_silu_forward/op_host/in_linear_silu.cpp).
+#include "../../include/ops_rec_activation_mi355.h"
+
+#include <hip/hip_runtime.h>
+
+#include "hstu_error.h"
+#include "in_linear_silu_kernel.hip.h"
+
+namespace {
+
+using hstu::InLinearSiluArgs;
+
+struct IlsVariant {
+    const char* name;
+    void (*kernel)(const InLinearSiluArgs);
+};
+
+// [type: bf16, fp16][k <= 64: a ring of 2 stages, four workgroups per CU; longer k: 4 stages]
+const IlsVariant kVariants[2][2] = {
+    {{"in_linear_silu_bf16_stages2", hstu::in_linear_silu_kernel<hstu::bf16_tag, 2>},
+     {"in_linear_silu_bf16_stages4", hstu::in_linear_silu_kernel<hstu::bf16_tag, 4>}},
+    {{"in_linear_silu_f16_stages2", hstu::in_linear_silu_kernel<hstu::f16_tag, 2>},
+     {"in_linear_silu_f16_stages4", hstu::in_linear_silu_kernel<hstu::f16_tag, 4>}},
+};
+
+constexpr int64_t kMinDim = 16;
+constexpr int64_t kMaxDim = 512 * 16;
+
+bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
+
+int validate(const in_linear_silu_params* p)
+{
+    if (p == nullptr) {
+        return hstu::set_error(HSTU_ERR_NULLPTR, "params is NULL");
+    }
+    if (p->struct_size != sizeof(in_linear_silu_params)) {
+        return hstu::set_error(HSTU_ERR_INVALID, "struct_size %u does not match this library (%zu)", p->struct_size,
+                               sizeof(in_linear_silu_params));
+    }
+    if (p->x == nullptr || p->weight == nullptr || p->user == nullptr || p->value == nullptr || p->query == nullptr ||
+        p->key == nullptr || p->linear_output == nullptr) {
+        return hstu::set_error(HSTU_ERR_NULLPTR, "x, weight and the five outputs must all be given");
+    }
+    if (p->dtype != HSTU_DT_BF16 && p->dtype != HSTU_DT_FP16) {
+        return hstu::set_error(HSTU_ERR_INVALID, "dtype %d is not bf16 or fp16", p->dtype);
+    }
+    if (p->m < 1) {
+        return hstu::set_error(HSTU_ERR_INVALID, "x tensor must be non-empty");
+    }
+    int64_t total = 0;
+    for (int i = 0; i < 4; ++i) {
+        if (p->split[i] < kMinDim || p->split[i] > kMaxDim || p->split[i] % kMinDim != 0) {
+            return hstu::set_error(HSTU_ERR_INVALID, "uvqk dim must in range[16, 8192] and multiples of 16.");
+        }
+        total += p->split[i];
+    }
+    if (p->k < kMinDim || p->k > kMaxDim || p->k % kMinDim != 0) {
+        return hstu::set_error(HSTU_ERR_INVALID, "x dim[1] must in range[16, 8192] and multiples of 16.");
+    }
+    if (p->n < 4 * kMinDim || p->n > 4 * kMaxDim || p->n % kMinDim != 0) {
+        return hstu::set_error(HSTU_ERR_INVALID, "weight dim[0] must in range[64, 32768] and multiples of 16.");
+    }
+    if (total != p->n) {
+        return hstu::set_error(HSTU_ERR_INVALID, "weight_dim[0] must equal to sum(splitList).");
+    }
+    if (p->n % (4 * p->k) != 0) {
+        return hstu::set_error(HSTU_ERR_INVALID, "weight dim[0] must be a multiple of 4 x dim[1]");
+    }
+    const void* ptrs[] = {p->x, p->weight, p->bias, p->user, p->value, p->query, p->key, p->linear_output};
+    for (const void* ptr : ptrs) {
+        if (!aligned16(ptr)) {
+            return hstu::set_error(HSTU_ERR_INVALID, "every tensor must start at a multiple of 16 bytes");
+        }
+    }
+    const int64_t tiles =
+        ((p->m + hstu::kIlsTileM - 1) / hstu::kIlsTileM) * ((p->n + hstu::kIlsTileN - 1) / hstu::kIlsTileN);
+    if (tiles > 0x7fffffff) {
+        return hstu::set_error(HSTU_ERR_INVALID, "too many rows: %lld tiles of %d x %d", static_cast<long long>(tiles),
+                               hstu::kIlsTileM, hstu::kIlsTileN);
+    }
+    return HSTU_OK;
+}
+
+const IlsVariant* select(const in_linear_silu_params* p)
+{
+    return &kVariants[p->dtype == HSTU_DT_BF16 ? 0 : 1][p->k <= 64 ? 0 : 1];
+}
+
+}  // namespace
+
+extern "C" {
+
+HSTU_API const char* in_linear_silu_fwd_kernel_name(const in_linear_silu_params* params)
+{
+    return validate(params) == HSTU_OK ? select(params)->name : nullptr;
+}
+
+HSTU_API int in_linear_silu_fwd(const in_linear_silu_params* p, void* stream)
+{
+    const int rc = validate(p);
+    if (rc != HSTU_OK) {
+        return rc;
+    }
+    const IlsVariant* v = select(p);
+    InLinearSiluArgs a;
+    a.x = p->x;
+    a.weight = p->weight;
+    a.bias = p->bias;
+    a.user = p->user;
+    a.value = p->value;
+    a.query = p->query;
+    a.key = p->key;
+    a.linear_output = p->linear_output;
+    a.m = p->m;
+    a.n = static_cast<int>(p->n);
+    a.k = static_cast<int>(p->k);
+    a.split_end[0] = static_cast<int>(p->split[0]);
+    a.split_end[1] = a.split_end[0] + static_cast<int>(p->split[1]);
+    a.split_end[2] = a.split_end[1] + static_cast<int>(p->split[2]);
+    const int64_t tiles =
+        ((p->m + hstu::kIlsTileM - 1) / hstu::kIlsTileM) * ((p->n + hstu::kIlsTileN - 1) / hstu::kIlsTileN);
+    hipLaunchKernelGGL(v->kernel, dim3(static_cast<unsigned>(tiles)), dim3(hstu::kIlsThreads), 0,
+                       static_cast<hipStream_t>(stream), a);
+    const hipError_t err = hipGetLastError();
+    if (err != hipSuccess) {
+        return hstu::set_error(HSTU_ERR_RUNTIME, "launch of %s failed: %s", v->name, hipGetErrorString(err));
+    }
+    return HSTU_OK;
+}
+
+}  // extern "C"

@@ -5,11 +5,18 @@ reference's adapter (ascendc/activation/ln_mul/torch_extension/ln_mul_plugin.cpp
 fixed by its host tiling (ascendc/activation/ln_mul/op_host/ln_mul.cpp:75).  The reference takes fp32 only; here
 x / u may also be bf16 / fp16 (what the attention kernels write) with gamma / beta in fp32 or in that type.  Like
 the reference's registration, the operator carries no autograd formula.
+
+``distance_in_linear_silu(x, weight, bias, attr_dict)`` (``in_linear_silu`` in the reference's documentation):
+``mixed = x @ weight^T + bias``, ``linear_output = mixed``, ``(user, value, query, key) = split(silu(mixed))``; schema
+and checks of ascendc/activation/in_linear_silu/torch_extension/in_linear_silu_plugin.cpp:36-110.  Its backward
+operator ``in_linear_silu_backward`` (schema of in_linear_silu_backward_plugin.cpp:155-160) is a composite of device
+operations here; the autograd formula that joins the two is the reference's (torch_extension/_autograd.py:33-86).
 """
 
 from __future__ import annotations
 
 import ctypes
+from typing import List, Optional
 
 import torch
 
@@ -75,3 +82,149 @@ def ln_mul_meta(x, u, gamma, beta):
 
 _lib_cuda.impl("ln_mul", ln_mul)
 _lib_meta.impl("ln_mul", ln_mul_meta)
+
+
+# ---------------------------------------------------------------- in_linear_silu ----
+
+_MIN_DIM, _MAX_DIM = 16, 512 * 16
+
+_lib_def.define("distance_in_linear_silu(Tensor x, Tensor weight, Tensor bias, int[] attr_dict) -> "
+                "(Tensor, Tensor, Tensor, Tensor, Tensor)")  # fmt: skip
+_lib_def.define("in_linear_silu_backward(Tensor x, Tensor weight, Tensor? bias, Tensor user_grad, Tensor value_grad, "
+                "Tensor query_grad, Tensor key_grad, Tensor linear_output, int[] attr_dict) -> "
+                "(Tensor, Tensor, Tensor, Tensor)")  # fmt: skip
+
+
+def _in_linear_silu_shapes(x, weight, bias, split: List[int]) -> None:
+    # IsValidShape (in_linear_silu_plugin.cpp:36-66)
+    _non_empty(x, "x")
+    _non_empty(weight, "weight")
+    _check(x.dim() == 2, "x must be 2D")
+    _check(weight.dim() == 2, "weight must be 2D")
+    _check(len(split) == 4, "splitList must have 4 elements.")
+    for s in split:
+        _check(_MIN_DIM <= s <= _MAX_DIM and s % _MIN_DIM == 0, "uvqk dim must in range[16, 8192] and multiples of 16.")
+    k, n = x.size(1), weight.size(0)
+    _check(_MIN_DIM <= k <= _MAX_DIM and k % _MIN_DIM == 0, "x dim[1] must in range[16, 8192] and multiples of 16.")
+    _check(4 * _MIN_DIM <= n <= 4 * _MAX_DIM and n % _MIN_DIM == 0,
+           "weight dim[0] must in range[64, 32768] and multiples of 16.")  # fmt: skip
+    _check(sum(split) == n, "weight_dim[0] must equal to sum(splitList).")
+    _check(weight.size(1) == k, "weight dim[1] must equal to x dim[1].")
+    _check(n % (4 * k) == 0, "weight dim[0] must be a multiple of 4 x dim[1]")
+    if bias is not None:
+        _non_empty(bias, "bias")
+        _check(bias.dim() == 1, "bias must be 1D")
+        _check(bias.size(0) == n, "bias dim[0] must equal to weight dim[0].")
+
+
+def distance_in_linear_silu(x, weight, bias, attr_dict):
+    split = [int(s) for s in attr_dict]
+    _in_linear_silu_shapes(x, weight, bias, split)
+    _check(x.dtype in (torch.bfloat16, torch.float16), f"x must be float16 or bfloat16, got {x.dtype}")
+    _check(weight.dtype == x.dtype, "weight must have the dtype of x")
+    _check(x.is_cuda and weight.device == x.device, "x and weight must be on the same GPU")
+    m, k, n = x.size(0), x.size(1), weight.size(0)
+    x_c, w_c = x.contiguous(), weight.contiguous()
+    b_c = None
+    if bias is not None:
+        _check(bias.device == x.device, "bias must be on the GPU of x")
+        _check(bias.dtype == torch.float32, "bias must be float32")
+        b_c = bias.contiguous()
+    outs = [torch.empty((m, s), dtype=x.dtype, device=x.device) for s in split]
+    linear_output = torch.empty((m, n), dtype=x.dtype, device=x.device)
+    p = _native.new_in_linear_silu_params()
+    p.x, p.weight, p.bias = x_c.data_ptr(), w_c.data_ptr(), (b_c.data_ptr() if b_c is not None else None)
+    p.user, p.value, p.query, p.key = (t.data_ptr() for t in outs)
+    p.linear_output = linear_output.data_ptr()
+    p.m, p.n, p.k = m, n, k
+    for i, s in enumerate(split):
+        p.split[i] = s
+    p.dtype = _DTYPE_CODE[x.dtype]
+    lib = _native.load()
+    with torch.cuda.device(x.device):
+        rc = lib.in_linear_silu_fwd(ctypes.byref(p), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    if rc != 0:
+        raise RuntimeError(f"in_linear_silu failed ({rc}): {_native.last_error()}")
+    return outs[0], outs[1], outs[2], outs[3], linear_output
+
+
+def distance_in_linear_silu_meta(x, weight, bias, attr_dict):
+    # in_linear_silu_plugin.cpp:90-103
+    m, n = x.size(0), weight.size(0)
+    outs = [x.new_empty((m, s)) for s in attr_dict]
+    return outs[0], outs[1], outs[2], outs[3], x.new_empty((m, n))
+
+
+def in_linear_silu_backward(x, weight, bias: Optional[torch.Tensor], user_grad, value_grad, query_grad, key_grad,
+                            linear_output, attr_dict):  # fmt: skip
+    """Gradients of x, weight and bias (in_linear_silu_backward_plugin.cpp:40-153): with z = linear_output,
+    d mixed = cat(grads) * sigmoid(z) * (1 + z * (1 - sigmoid(z))); d x = d mixed @ weight; d weight = d mixed^T @ x;
+    d bias = column sums of d mixed.  A composite of device operations (fp32 element-wise part, library products)."""
+    split = [int(s) for s in attr_dict]
+    _in_linear_silu_shapes(x, weight, bias, split)
+    grads = (user_grad, value_grad, query_grad, key_grad)
+    for g, name in zip(grads, ("user_grad", "value_grad", "query_grad", "key_grad")):
+        _non_empty(g, name)
+        _check(g.dim() == 2, f"{name} must be 2D")
+    _non_empty(linear_output, "linear_output")
+    _check(linear_output.dim() == 2, "linear_output must be 2D")
+    _check(all(g.size(1) == s for g, s in zip(grads, split)),
+           "user_grad, value_grad, query_grad, key_grad dim[1] must be equal to split_list.")  # fmt: skip
+    _check(all(g.size(0) == x.size(0) for g in grads) and linear_output.size(0) == x.size(0),
+           "user_grad, value_grad, query_grad, key_grad linear_output dim[0] must equal to x dim[0].")  # fmt: skip
+    _check(linear_output.size(1) == weight.size(0), "linear_output dim[1] must equal to weight dim[0].")
+    z = linear_output.float()
+    sig = torch.sigmoid(z)
+    d_mixed = torch.cat([g.float() for g in grads], dim=1) * (sig * (1.0 + z * (1.0 - sig)))
+    d_low = d_mixed.to(x.dtype)
+    x_grad = d_low @ weight
+    weight_grad = d_low.t() @ x
+    bias_grad = d_mixed.sum(dim=0).to(bias.dtype) if bias is not None else None
+    return x_grad, weight_grad, bias_grad, None
+
+
+def in_linear_silu_backward_meta(x, weight, bias, user_grad, value_grad, query_grad, key_grad, linear_output, attr_dict):
+    return torch.empty_like(x), torch.empty_like(weight), (torch.empty_like(bias) if bias is not None else None), None
+
+
+_lib_cuda.impl("distance_in_linear_silu", distance_in_linear_silu)
+_lib_meta.impl("distance_in_linear_silu", distance_in_linear_silu_meta)
+_lib_cuda.impl("in_linear_silu_backward", in_linear_silu_backward)
+_lib_meta.impl("in_linear_silu_backward", in_linear_silu_backward_meta)
+
+
+def _ils_setup_context(ctx, inputs, output):
+    # torch_extension/_autograd.py:33-52
+    x, weight, bias, attr_dict = inputs
+    ctx.has_bias = bias is not None
+    if ctx.has_bias:
+        ctx.save_for_backward(x, weight, bias, output[-1])
+    else:
+        ctx.save_for_backward(x, weight, output[-1])
+    ctx.attr_dict = list(attr_dict)
+
+
+def _ils_backward(ctx, user_grad, value_grad, query_grad, key_grad, linear_output_grad):
+    # torch_extension/_autograd.py:55-86: the gradient of linear_output is ignored, as there
+    if ctx.has_bias:
+        x, weight, bias, linear_output = ctx.saved_tensors
+    else:
+        (x, weight, linear_output), bias = ctx.saved_tensors, None
+    x_grad, weight_grad, bias_grad, _ = torch.ops.ops_rec.in_linear_silu_backward(
+        x, weight, bias, user_grad, value_grad, query_grad, key_grad, linear_output, ctx.attr_dict)  # fmt: skip
+    return x_grad, weight_grad, bias_grad, None
+
+
+_ils_autograd_registered = False
+
+
+def register_in_linear_silu_autograd() -> None:
+    """Idempotent, like the reference's ``register_autograd`` (torch_extension/_autograd.py:89-101)."""
+    global _ils_autograd_registered
+    if _ils_autograd_registered:
+        return
+    torch.library.register_autograd("ops_rec::distance_in_linear_silu", _ils_backward, setup_context=_ils_setup_context)
+    _ils_autograd_registered = True
+
+
+register_in_linear_silu_autograd()

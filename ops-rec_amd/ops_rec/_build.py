@@ -17,6 +17,7 @@ LIB_PATH = os.path.join(LIB_DIR, "libhstu_mi355.so")
 SOURCES = [
     "hstu_mi355.hip",
     "ln_mul_mi355.hip",
+    "in_linear_silu_mi355.hip",
     "hstu_kernels_fwd_bf16.hip",
     "hstu_kernels_fwd_f16.hip",
     "hstu_kernels_fwd_f8.hip",

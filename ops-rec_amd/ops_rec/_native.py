@@ -28,6 +28,8 @@ EXPORTED_SYMBOLS = (
     "hstu_paged_fwd",
     "ln_mul_fwd",
     "ln_mul_fwd_kernel_name",
+    "in_linear_silu_fwd",
+    "in_linear_silu_fwd_kernel_name",
 )
 
 
@@ -123,6 +125,29 @@ class LnMulParams(ctypes.Structure):
     ]
 
 
+class InLinearSiluParams(ctypes.Structure):
+    """Mirror of ``in_linear_silu_params`` (include/ops_rec_activation_mi355.h)."""
+
+    _fields_ = [
+        ("struct_size", ctypes.c_uint32),
+        ("reserved0", ctypes.c_uint32),
+        ("x", ctypes.c_void_p),
+        ("weight", ctypes.c_void_p),
+        ("bias", ctypes.c_void_p),
+        ("user", ctypes.c_void_p),
+        ("value", ctypes.c_void_p),
+        ("query", ctypes.c_void_p),
+        ("key", ctypes.c_void_p),
+        ("linear_output", ctypes.c_void_p),
+        ("m", ctypes.c_int64),
+        ("n", ctypes.c_int64),
+        ("k", ctypes.c_int64),
+        ("split", ctypes.c_int64 * 4),
+        ("dtype", ctypes.c_int32),
+        ("reserved1", ctypes.c_uint32),
+    ]
+
+
 _lib: Optional[ctypes.CDLL] = None
 
 
@@ -164,6 +189,10 @@ def load() -> ctypes.CDLL:
     lib.ln_mul_fwd.argtypes = [ctypes.POINTER(LnMulParams), ctypes.c_void_p]
     lib.ln_mul_fwd_kernel_name.restype = ctypes.c_char_p
     lib.ln_mul_fwd_kernel_name.argtypes = [ctypes.POINTER(LnMulParams)]
+    lib.in_linear_silu_fwd.restype = ctypes.c_int
+    lib.in_linear_silu_fwd.argtypes = [ctypes.POINTER(InLinearSiluParams), ctypes.c_void_p]
+    lib.in_linear_silu_fwd_kernel_name.restype = ctypes.c_char_p
+    lib.in_linear_silu_fwd_kernel_name.argtypes = [ctypes.POINTER(InLinearSiluParams)]
     _lib = lib
     return lib
 
@@ -175,6 +204,12 @@ def last_error() -> str:
 def new_params() -> FwdParams:
     p = FwdParams()
     p.struct_size = ctypes.sizeof(FwdParams)
+    return p
+
+
+def new_in_linear_silu_params() -> InLinearSiluParams:
+    p = InLinearSiluParams()
+    p.struct_size = ctypes.sizeof(InLinearSiluParams)
     return p
 
 

@@ -8,11 +8,16 @@ unknown name raises ``AttributeError`` listing what exists.
 import torch
 
 _NS = torch.ops.ops_rec
-_OPS = ("ln_mul",)
+_OPS = ("ln_mul", "distance_in_linear_silu", "in_linear_silu_backward")
 
 __all__ = [name for name in _OPS if hasattr(_NS, name)]
 for _name in __all__:
     globals()[_name] = getattr(_NS, _name)
+# the name the reference's documentation uses for the differentiable forward (docs/zh/ops_rec_api.md:42); the
+# autograd formula is attached to distance_in_linear_silu itself
+if hasattr(_NS, "distance_in_linear_silu"):
+    in_linear_silu = _NS.distance_in_linear_silu
+    __all__.append("in_linear_silu")
 
 
 def __getattr__(name: str):
