@@ -53,6 +53,10 @@ def algorithmic_bytes(w, out_element_size: int) -> int:
 
 # HBM bytes per ln_mul launch by rows (cols 512, bf16), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a plain
 # copy of known size (profiles/ln_mul_bf16_c512_trace_and_counters.md)
+# (m, n, k) -> bytes, same method (profiles/in_linear_silu_bf16_trace_and_counters.md)
+IN_LINEAR_SILU_MEASURED_TRAFFIC_BYTES = {(16384, 9216, 64): 623_700_000, (20292, 2048, 512): 341_800_000}
+
+
 LN_MUL_MEASURED_TRAFFIC_BYTES = {20292: 62_457_000, 324672: 997_512_000}
 
 
@@ -123,6 +127,75 @@ def bench_ln_mul(attn_out, stream, args):
             "cases": cases}  # fmt: skip
 
 
+def bench_in_linear_silu(tokens, stream, args):
+    """in_linear_silu through ``in_linear_silu_fwd`` of the C ABI, events on the launch stream.  Algorithmic bytes per
+    launch: x, weight and bias read once, linear_output and the four splits written once =
+    2 (m k + n k) + 4 n + 4 m n; flops 2 m n k."""
+    import ctypes
+
+    import torch
+
+    from ops_rec import _native
+    from oracle import in_linear_silu_oracle
+
+    lib = _native.load()
+    dev = torch.device("cuda", 0)
+    cases = []
+    # (m, n, k): a shape of the reference's own test (test_in_linear_silu.py:127-130), store-bound; and the layer of
+    # this workload: its tokens, embedding 512 -> U, V, Q, K of 512 each (heads x dim of the attention workload)
+    for m, n, k, what in ((16384, 9216, 64, "reference test shape"), (tokens, 2048, 512, "layer of this workload")):
+        x = torch.randn(m, k, device=dev).to(torch.bfloat16)
+        wt = (torch.randn(n, k, device=dev) / k**0.5).to(torch.bfloat16)
+        bias = torch.randn(n, device=dev)
+        split = [n // 4] * 4
+        outs = [torch.empty(m, s, dtype=torch.bfloat16, device=dev) for s in split + [n]]
+        p = _native.new_in_linear_silu_params()
+        p.x, p.weight, p.bias = x.data_ptr(), wt.data_ptr(), bias.data_ptr()
+        p.user, p.value, p.query, p.key, p.linear_output = (t.data_ptr() for t in outs)
+        p.m, p.n, p.k = m, n, k
+        for i, s_ in enumerate(split):
+            p.split[i] = s_
+        p.dtype = _native.DT_BF16
+        raw = ctypes.c_void_p(stream.cuda_stream)
+        n_it = max(20, args.steps // 2)
+        for _ in range(5):
+            assert lib.in_linear_silu_fwd(ctypes.byref(p), raw) == 0, _native.last_error()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record(stream)
+        for _ in range(n_it):
+            lib.in_linear_silu_fwd(ctypes.byref(p), raw)
+        e1.record(stream)
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) / n_it * 1e3
+        nbytes = 2 * (m * k + n * k) + 4 * n + 4 * m * n
+        flops = 2 * m * n * k
+        hbm_bound = nbytes / PEAK_HBM_GBS / 1e3 > flops / PEAK_BF16_TFLOPS / 1e6  # the longer of the two floors, in us
+        roof = ({"bound": "hbm", "achieved": round(nbytes / us / 1e3, 1), "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                 "frac": round(nbytes / us / 1e3 / PEAK_HBM_GBS, 4)} if hbm_bound else
+                {"bound": "mfma", "achieved": round(flops / us / 1e6, 1), "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                 "frac": round(flops / us / 1e6 / PEAK_BF16_TFLOPS, 4)})  # fmt: skip
+        roof["traffic"] = IN_LINEAR_SILU_MEASURED_TRAFFIC_BYTES.get((m, n, k))
+        case = {"m": m, "n": n, "k": k, "shape": what,
+                "kernel": lib.in_linear_silu_fwd_kernel_name(ctypes.byref(p)).decode(), "avg_launch_us": round(us, 3),
+                "algorithmic_bytes": nbytes, "flops": flops, "GBs": round(nbytes / us / 1e3, 1),
+                "tflops": round(flops / us / 1e6, 1), "roofline": roof}  # fmt: skip
+        if not args.no_cpu:
+            sample = 256
+            xs, ws, bs = x[:sample].cpu(), wt.cpu(), bias.cpu()
+            t0 = time.perf_counter()
+            want = in_linear_silu_oracle.in_linear_silu(xs, ws, bs, split, round_to=torch.bfloat16)
+            cpu_s = time.perf_counter() - t0
+            torch.testing.assert_close(outs[4][:sample].double().cpu(), want[4], rtol=2.0**-7, atol=1e-2)
+            torch.testing.assert_close(outs[2][:sample].double().cpu(), want[2], rtol=2.0**-6, atol=1e-2)
+            case["cpu_baseline"] = {"value": round(2 * sample * n * k / cpu_s / 1e12, 5), "unit": "TFLOP/s",
+                                    "cores": torch.get_num_threads(), "kind": "port",
+                                    "sample": f"first {sample} rows, float64 torch oracle"}  # fmt: skip
+        cases.append(case)
+        del x, wt, outs
+    return {"note": "in_linear_silu_fwd of the C ABI back-to-back on one stream, bf16", "cases": cases}
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -134,6 +207,10 @@ def main() -> int:
                     help="also time ln_mul (LayerNorm(x) * u, the operator that consumes the attention output) on the "
                     "output of this workload viewed as [tokens, heads * dim] and on a matrix 16 times as tall, and add "
                     "an 'ln_mul' object with its HBM roofline to the line")  # fmt: skip
+    ap.add_argument("--in-linear-silu", action="store_true",
+                    help="also time in_linear_silu (the linear + SiLU + split that produces U, V, Q, K in front of "
+                    "attention) on one of the reference's test shapes and on the layer shape of this workload, and "
+                    "add an 'in_linear_silu' object with its rooflines to the line")  # fmt: skip
     ap.add_argument("--backward", action="store_true",
                     help="also time hstu_jagged_backward (the two HIP backward kernels) on the same workload and add a "
                     "'backward' object to the line (bf16 workloads only)")  # fmt: skip
@@ -309,6 +386,9 @@ def main() -> int:
     # ---- ln_mul (optional): the operator that takes the attention output next in an HSTU layer ----
     if args.ln_mul:
         result["ln_mul"] = bench_ln_mul(prepared.out, stream, args)
+
+    if args.in_linear_silu:
+        result["in_linear_silu"] = bench_in_linear_silu(sum(w.lengths), stream, args)
 
     # ---- CPU baseline: dense-padded fp32 golden path on this host's cores ----
     if not args.no_cpu and w_cpu is not None:

@@ -146,6 +146,7 @@ struct InLinearSiluArgs {
     int n;
     int k;
     int split_end[3];  // first column after the user, value and query parts
+    int xcd_groups;    // 1: tiles dealt so that all n tiles of an m tile run on one XCD (grid padded to 8 m tiles)
 };
 
 }  // namespace hstu

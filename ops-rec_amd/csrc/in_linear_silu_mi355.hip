@@ -30,6 +30,20 @@ constexpr int64_t kMaxDim = 512 * 16;
 
 bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
 
+// a weight matrix beyond what the eight L2s hold between them several times over: x tiles are kept to one XCD each
+bool xcd_groups(const in_linear_silu_params* p) { return p->n * p->k * 2 > (int64_t{64} << 20); }
+
+// workgroups of a launch: m tiles (rounded up to whole groups of one per XCD in the grouped order) times n tiles
+int64_t grid_size(const in_linear_silu_params* p)
+{
+    int64_t tiles_m = (p->m + hstu::kIlsTileM - 1) / hstu::kIlsTileM;
+    const int64_t tiles_n = (p->n + hstu::kIlsTileN - 1) / hstu::kIlsTileN;
+    if (xcd_groups(p)) {
+        tiles_m = (tiles_m + hstu::kIlsXcds - 1) / hstu::kIlsXcds * hstu::kIlsXcds;
+    }
+    return tiles_m * tiles_n;
+}
+
 int validate(const in_linear_silu_params* p)
 {
     if (p == nullptr) {
@@ -74,8 +88,7 @@ int validate(const in_linear_silu_params* p)
             return hstu::set_error(HSTU_ERR_INVALID, "every tensor must start at a multiple of 16 bytes");
         }
     }
-    const int64_t tiles =
-        ((p->m + hstu::kIlsTileM - 1) / hstu::kIlsTileM) * ((p->n + hstu::kIlsTileN - 1) / hstu::kIlsTileN);
+    const int64_t tiles = grid_size(p);
     if (tiles > 0x7fffffff) {
         return hstu::set_error(HSTU_ERR_INVALID, "too many rows: %lld tiles of %d x %d", static_cast<long long>(tiles),
                                hstu::kIlsTileM, hstu::kIlsTileN);
@@ -119,8 +132,8 @@ HSTU_API int in_linear_silu_fwd(const in_linear_silu_params* p, void* stream)
     a.split_end[0] = static_cast<int>(p->split[0]);
     a.split_end[1] = a.split_end[0] + static_cast<int>(p->split[1]);
     a.split_end[2] = a.split_end[1] + static_cast<int>(p->split[2]);
-    const int64_t tiles =
-        ((p->m + hstu::kIlsTileM - 1) / hstu::kIlsTileM) * ((p->n + hstu::kIlsTileN - 1) / hstu::kIlsTileN);
+    a.xcd_groups = xcd_groups(p) ? 1 : 0;
+    const int64_t tiles = grid_size(p);
     hipLaunchKernelGGL(v->kernel, dim3(static_cast<unsigned>(tiles)), dim3(hstu::kIlsThreads), 0,
                        static_cast<hipStream_t>(stream), a);
     const hipError_t err = hipGetLastError();

@@ -166,7 +166,7 @@ def test_mask_requiring_grad_is_rejected():
 def test_library_exports_every_declared_symbol():
     header = open(os.path.join(_ROOT, "include", "hstu_mi355.h")).read()
     header += open(os.path.join(_ROOT, "include", "ops_rec_activation_mi355.h")).read()
-    declared = set(re.findall(r"HSTU_API\s+[\w\s\*]+?\b((?:hstu|ln_mul)_\w+)\s*\(", header))
+    declared = set(re.findall(r"HSTU_API\s+[\w\s\*]+?\b((?:hstu|ln_mul|in_linear_silu)_\w+)\s*\(", header))
     assert declared == set(_native.EXPORTED_SYMBOLS)
     lib = _native.load()
     for sym in declared:
