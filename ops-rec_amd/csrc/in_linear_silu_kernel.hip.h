@@ -17,7 +17,7 @@
 // of 32 through a ring of STAGES tiles in LDS filled by direct-to-LDS loads (16 KB per stage: 256 rows of 64 bytes,
 // chunk index XOR-ed with (row / 4) % 4 so that the 16-byte operand reads of 16 consecutive rows fall into 16
 // different bank groups).  STAGES = 2 (36 KB with the epilogue's staging: four workgroups per CU overlap their load /
-// product / store phases) for the short-k shapes, STAGES = 4 (prefetch distance 3) for long k.
+// product / store phases) 3 (48 KB, three workgroups per CU, prefetch distance 2) or 4 (64 KB, two); the host picks by k.
 #pragma once
 #include "hstu_fwd_kernel.hip.h"
 
@@ -67,7 +67,7 @@ __device__ __forceinline__ float ils_silu(float v)
 }
 
 template <typename Tag, int STAGES>
-__global__ __launch_bounds__(kIlsThreads, (STAGES == 2 ? 4 : 2)) void in_linear_silu_kernel(const InLinearSiluArgs a)
+__global__ __launch_bounds__(kIlsThreads, (STAGES == 2 ? 4 : (STAGES == 3 ? 3 : 2))) void in_linear_silu_kernel(const InLinearSiluArgs a)
 {
     constexpr int kStageElems = (kIlsTileM + kIlsTileN) * kIlsStepK;  // 16-bit elements per stage
     // the epilogue stages both results of 32 x rows by 64 columns per wavefront in the same memory

@@ -17,11 +17,16 @@ struct IlsVariant {
     void (*kernel)(const InLinearSiluArgs);
 };
 
-// [type: bf16, fp16][k <= 64: a ring of 2 stages, four workgroups per CU; longer k: 4 stages]
-const IlsVariant kVariants[2][2] = {
+// [type: bf16, fp16][ring of 2 stages, four workgroups per CU; ring of 3 stages, three workgroups per CU].  Measured
+// on MI355X over k = 64 .. 2048 with rings of 2, 3 and 4 stages: workgroups per CU count for more than prefetch depth
+// (4 stages, two workgroups per CU, was slowest everywhere); 3 stages win by 3-7 % for k = 128 .. 512, 2 stages by
+// 2-4 % at k <= 64 and at k = 768 .. 2048; at k = 8192 (weights of 512 MB, grouped tile order) 4 stages win by 10 %.
+const IlsVariant kVariants[2][3] = {
     {{"in_linear_silu_bf16_stages2", hstu::in_linear_silu_kernel<hstu::bf16_tag, 2>},
+     {"in_linear_silu_bf16_stages3", hstu::in_linear_silu_kernel<hstu::bf16_tag, 3>},
      {"in_linear_silu_bf16_stages4", hstu::in_linear_silu_kernel<hstu::bf16_tag, 4>}},
     {{"in_linear_silu_f16_stages2", hstu::in_linear_silu_kernel<hstu::f16_tag, 2>},
+     {"in_linear_silu_f16_stages3", hstu::in_linear_silu_kernel<hstu::f16_tag, 3>},
      {"in_linear_silu_f16_stages4", hstu::in_linear_silu_kernel<hstu::f16_tag, 4>}},
 };
 
@@ -98,7 +103,8 @@ int validate(const in_linear_silu_params* p)
 
 const IlsVariant* select(const in_linear_silu_params* p)
 {
-    return &kVariants[p->dtype == HSTU_DT_BF16 ? 0 : 1][p->k <= 64 ? 0 : 1];
+    const int ring = p->k > 4096 ? 2 : ((p->k <= 64 || p->k > 512) ? 0 : 1);
+    return &kVariants[p->dtype == HSTU_DT_BF16 ? 0 : 1][ring];
 }
 
 }  // namespace

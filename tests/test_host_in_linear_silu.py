@@ -109,10 +109,13 @@ def test_kernel_variant_selection():
             p.split[i] = n // 4
         return lib.in_linear_silu_fwd_kernel_name(ctypes.byref(p)).decode()
 
-    # short k (the store-bound shapes): a ring of two k steps and four workgroups per CU; longer k: four stages
+    # a ring of two k steps and four workgroups per CU for short and for long k, three stages in between, four for the longest (measured)
     assert name(16, 64) == "in_linear_silu_bf16_stages2"
     assert name(64, 9216) == "in_linear_silu_bf16_stages2"
-    assert name(128, 1024) == "in_linear_silu_bf16_stages4"
+    assert name(128, 1024) == "in_linear_silu_bf16_stages3"
+    assert name(512, 2048) == "in_linear_silu_bf16_stages3"
+    assert name(768, 3072) == "in_linear_silu_bf16_stages2"
+    assert name(4096, 16384) == "in_linear_silu_bf16_stages2"
     assert name(8192, 32768, _native.DT_FP16) == "in_linear_silu_f16_stages4"
 
 
