@@ -84,6 +84,40 @@ HSTU_API int in_linear_silu_fwd(const in_linear_silu_params* params, void* strea
 /* name of the kernel variant in_linear_silu_fwd would launch, or NULL after an error */
 HSTU_API const char* in_linear_silu_fwd_kernel_name(const in_linear_silu_params* params);
 
+/*
+ * The element-wise stage of in_linear_silu's backward (the reference does the whole backward in one call,
+ * aclnnInLinearSiluBackward, ascendc/activation/in_linear_silu/in_linear_silu_backward/docs/aclnn_in_linear_silu_backward.md;
+ * its adapter: torch_extension/in_linear_silu_backward_plugin.cpp:112-153):
+ *   d_mixed = cat(user_grad, value_grad, query_grad, key_grad) * silu'(linear_output),  bias_grad = column sums.
+ * The two products that follow (d x = d_mixed @ weight, d weight = d_mixed^T @ x) are plain matrix products and are left
+ * to the caller's BLAS.
+ */
+typedef struct in_linear_silu_bwd_params {
+    uint32_t struct_size; /* sizeof(in_linear_silu_bwd_params), checked */
+    uint32_t reserved0;
+    const void* linear_output; /* [m, n], bf16 or fp16: the forward's fifth output */
+    const void* user_grad;     /* [m, split[0]], same type */
+    const void* value_grad;    /* [m, split[1]] */
+    const void* query_grad;    /* [m, split[2]] */
+    const void* key_grad;      /* [m, split[3]] */
+    void* d_mixed;             /* [m, n], same type; every element is written */
+    float* bias_grad;          /* [n] fp32, or NULL when there is no bias */
+    int64_t m;
+    int64_t n;
+    int64_t split[4];
+    int32_t dtype; /* HSTU_DT_BF16 or HSTU_DT_FP16 */
+    uint32_t reserved1;
+} in_linear_silu_bwd_params;
+
+/* bytes of device scratch in_linear_silu_bwd_dmixed needs (partial column sums: ceil(m / 64) * n floats; 0 when
+ * bias_grad is NULL) */
+HSTU_API int in_linear_silu_bwd_dmixed_workspace_size(const in_linear_silu_bwd_params* params, uint64_t* workspace_bytes);
+
+/* Launches on `stream` and returns without waiting.  HSTU_OK, or HSTU_ERR_NULLPTR / HSTU_ERR_INVALID /
+ * HSTU_ERR_WORKSPACE (nothing launched) / HSTU_ERR_RUNTIME. */
+HSTU_API int in_linear_silu_bwd_dmixed(const in_linear_silu_bwd_params* params, void* workspace, uint64_t workspace_bytes,
+                                       void* stream);
+
 #ifdef __cplusplus
 }
 #endif

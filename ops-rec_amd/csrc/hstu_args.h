@@ -149,4 +149,18 @@ struct InLinearSiluArgs {
     int xcd_groups;    // 1: tiles dealt so that all n tiles of an m tile run on one XCD (grid padded to 8 m tiles)
 };
 
+// element-wise stage of in_linear_silu's backward (in_linear_silu_bwd_kernel.hip.h)
+struct InLinearSiluBwdArgs {
+    const void* linear_output;  // [m, n], 16-bit
+    const void* user_grad;      // [m, split_end[0]]
+    const void* value_grad;     // [m, split_end[1] - split_end[0]]
+    const void* query_grad;     // [m, split_end[2] - split_end[1]]
+    const void* key_grad;       // [m, n - split_end[2]]
+    void* d_mixed;              // [m, n], 16-bit
+    float* partial_sums;        // [ceil(m / 64), n] column sums per workgroup row, or nullptr when no bias gradient is wanted
+    int64_t m;
+    int n;
+    int split_end[3];
+};
+
 }  // namespace hstu

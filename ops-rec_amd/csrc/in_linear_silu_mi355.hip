@@ -6,6 +6,7 @@
 #include <hip/hip_runtime.h>
 
 #include "hstu_error.h"
+#include "in_linear_silu_bwd_kernel.hip.h"
 #include "in_linear_silu_kernel.hip.h"
 
 namespace {
@@ -107,9 +108,122 @@ const IlsVariant* select(const in_linear_silu_params* p)
     return &kVariants[p->dtype == HSTU_DT_BF16 ? 0 : 1][ring];
 }
 
+int validate_bwd(const in_linear_silu_bwd_params* p)
+{
+    if (p == nullptr) {
+        return hstu::set_error(HSTU_ERR_NULLPTR, "params is NULL");
+    }
+    if (p->struct_size != sizeof(in_linear_silu_bwd_params)) {
+        return hstu::set_error(HSTU_ERR_INVALID, "struct_size %u does not match this library (%zu)", p->struct_size,
+                               sizeof(in_linear_silu_bwd_params));
+    }
+    if (p->linear_output == nullptr || p->user_grad == nullptr || p->value_grad == nullptr || p->query_grad == nullptr ||
+        p->key_grad == nullptr || p->d_mixed == nullptr) {
+        return hstu::set_error(HSTU_ERR_NULLPTR, "linear_output, the four gradients and d_mixed must all be given");
+    }
+    if (p->dtype != HSTU_DT_BF16 && p->dtype != HSTU_DT_FP16) {
+        return hstu::set_error(HSTU_ERR_INVALID, "dtype %d is not bf16 or fp16", p->dtype);
+    }
+    if (p->m < 1) {
+        return hstu::set_error(HSTU_ERR_INVALID, "linear_output tensor must be non-empty");
+    }
+    int64_t total = 0;
+    for (int i = 0; i < 4; ++i) {
+        if (p->split[i] < kMinDim || p->split[i] > kMaxDim || p->split[i] % kMinDim != 0) {
+            return hstu::set_error(HSTU_ERR_INVALID, "uvqk dim must in range[16, 8192] and multiples of 16.");
+        }
+        total += p->split[i];
+    }
+    if (p->n < 4 * kMinDim || p->n > 4 * kMaxDim || p->n % kMinDim != 0) {
+        return hstu::set_error(HSTU_ERR_INVALID, "weight dim[0] must in range[64, 32768] and multiples of 16.");
+    }
+    if (total != p->n) {
+        return hstu::set_error(HSTU_ERR_INVALID, "linear_output dim[1] must equal to sum(split_list).");
+    }
+    const void* ptrs[] = {p->linear_output, p->user_grad, p->value_grad, p->query_grad, p->key_grad, p->d_mixed};
+    for (const void* ptr : ptrs) {
+        if (!aligned16(ptr)) {
+            return hstu::set_error(HSTU_ERR_INVALID, "every tensor must start at a multiple of 16 bytes");
+        }
+    }
+    if ((p->m + hstu::kIlsBwdRows - 1) / hstu::kIlsBwdRows > 0x7fffffff / 2) {
+        return hstu::set_error(HSTU_ERR_INVALID, "too many rows");
+    }
+    return HSTU_OK;
+}
+
+int64_t bwd_row_blocks(const in_linear_silu_bwd_params* p) { return (p->m + hstu::kIlsBwdRows - 1) / hstu::kIlsBwdRows; }
+
+uint64_t bwd_workspace_bytes(const in_linear_silu_bwd_params* p)
+{
+    return p->bias_grad == nullptr ? 0 : static_cast<uint64_t>(bwd_row_blocks(p)) * static_cast<uint64_t>(p->n) * sizeof(float);
+}
+
 }  // namespace
 
 extern "C" {
+
+HSTU_API int in_linear_silu_bwd_dmixed_workspace_size(const in_linear_silu_bwd_params* p, uint64_t* workspace_bytes)
+{
+    if (workspace_bytes == nullptr) {
+        return hstu::set_error(HSTU_ERR_NULLPTR, "workspace_bytes is NULL");
+    }
+    *workspace_bytes = 0;
+    const int rc = validate_bwd(p);
+    if (rc != HSTU_OK) {
+        return rc;
+    }
+    *workspace_bytes = bwd_workspace_bytes(p);
+    return HSTU_OK;
+}
+
+HSTU_API int in_linear_silu_bwd_dmixed(const in_linear_silu_bwd_params* p, void* workspace, uint64_t workspace_bytes,
+                                       void* stream)
+{
+    const int rc = validate_bwd(p);
+    if (rc != HSTU_OK) {
+        return rc;
+    }
+    const uint64_t need = bwd_workspace_bytes(p);
+    if (need > 0 && (workspace == nullptr || workspace_bytes < need || !aligned16(workspace))) {
+        return hstu::set_error(HSTU_ERR_WORKSPACE, "workspace of %llu bytes (16-byte aligned) needed for the bias gradient, got %llu",
+                               static_cast<unsigned long long>(need), static_cast<unsigned long long>(workspace_bytes));
+    }
+    hstu::InLinearSiluBwdArgs a;
+    a.linear_output = p->linear_output;
+    a.user_grad = p->user_grad;
+    a.value_grad = p->value_grad;
+    a.query_grad = p->query_grad;
+    a.key_grad = p->key_grad;
+    a.d_mixed = p->d_mixed;
+    a.partial_sums = need > 0 ? static_cast<float*>(workspace) : nullptr;
+    a.m = p->m;
+    a.n = static_cast<int>(p->n);
+    a.split_end[0] = static_cast<int>(p->split[0]);
+    a.split_end[1] = a.split_end[0] + static_cast<int>(p->split[1]);
+    a.split_end[2] = a.split_end[1] + static_cast<int>(p->split[2]);
+    const unsigned col_blocks = static_cast<unsigned>((p->n + hstu::kIlsBwdCols - 1) / hstu::kIlsBwdCols);
+    const unsigned row_blocks = static_cast<unsigned>(bwd_row_blocks(p));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (p->dtype == HSTU_DT_BF16) {
+        hipLaunchKernelGGL(hstu::in_linear_silu_dmixed_kernel<hstu::bf16_tag>, dim3(col_blocks, row_blocks),
+                           dim3(hstu::kIlsBwdThreads), 0, s, a);
+    } else {
+        hipLaunchKernelGGL(hstu::in_linear_silu_dmixed_kernel<hstu::f16_tag>, dim3(col_blocks, row_blocks),
+                           dim3(hstu::kIlsBwdThreads), 0, s, a);
+    }
+    if (need > 0) {
+        hipLaunchKernelGGL(hstu::in_linear_silu_bias_grad_kernel,
+                           dim3(static_cast<unsigned>((p->n + hstu::kIlsBiasCols - 1) / hstu::kIlsBiasCols)),
+                           dim3(hstu::kIlsBiasCols * hstu::kIlsBiasLanes), 0, s, a.partial_sums, p->bias_grad,
+                           static_cast<int>(row_blocks), a.n);
+    }
+    const hipError_t err = hipGetLastError();
+    if (err != hipSuccess) {
+        return hstu::set_error(HSTU_ERR_RUNTIME, "launch of in_linear_silu_dmixed failed: %s", hipGetErrorString(err));
+    }
+    return HSTU_OK;
+}
 
 HSTU_API const char* in_linear_silu_fwd_kernel_name(const in_linear_silu_params* params)
 {

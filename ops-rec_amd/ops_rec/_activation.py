@@ -9,8 +9,8 @@ the reference's registration, the operator carries no autograd formula.
 ``distance_in_linear_silu(x, weight, bias, attr_dict)`` (``in_linear_silu`` in the reference's documentation):
 ``mixed = x @ weight^T + bias``, ``linear_output = mixed``, ``(user, value, query, key) = split(silu(mixed))``; schema
 and checks of ascendc/activation/in_linear_silu/torch_extension/in_linear_silu_plugin.cpp:36-110.  Its backward
-operator ``in_linear_silu_backward`` (schema of in_linear_silu_backward_plugin.cpp:155-160) is a composite of device
-operations here; the autograd formula that joins the two is the reference's (torch_extension/_autograd.py:33-86).
+operator ``in_linear_silu_backward`` (schema of in_linear_silu_backward_plugin.cpp:155-160) runs its element-wise stage
+and the bias gradient as one HIP kernel and the two products as library matrix products; the autograd formula that joins the two is the reference's (torch_extension/_autograd.py:33-86).
 """
 
 from __future__ import annotations
@@ -155,11 +155,43 @@ def distance_in_linear_silu_meta(x, weight, bias, attr_dict):
     return outs[0], outs[1], outs[2], outs[3], x.new_empty((m, n))
 
 
+def silu_backward_stage(linear_output, grads, split, want_bias_grad=True):
+    """``d_mixed`` [m, n] in the type of ``linear_output`` and the fp32 column sums (or None), through
+    ``in_linear_silu_bwd_dmixed`` of the C ABI."""
+    lin = linear_output.contiguous()
+    gs = [g.contiguous() for g in grads]
+    m, n = lin.shape
+    d_mixed = torch.empty_like(lin)
+    sums = torch.empty(n, dtype=torch.float32, device=lin.device) if want_bias_grad else None
+    p = _native.new_in_linear_silu_bwd_params()
+    p.linear_output = lin.data_ptr()
+    p.user_grad, p.value_grad, p.query_grad, p.key_grad = (g.data_ptr() for g in gs)
+    p.d_mixed = d_mixed.data_ptr()
+    p.bias_grad = sums.data_ptr() if sums is not None else None
+    p.m, p.n = m, n
+    for i, s_ in enumerate(split):
+        p.split[i] = int(s_)
+    p.dtype = _DTYPE_CODE[lin.dtype]
+    lib = _native.load()
+    need = ctypes.c_uint64(0)
+    rc = lib.in_linear_silu_bwd_dmixed_workspace_size(ctypes.byref(p), ctypes.byref(need))
+    if rc != 0:
+        raise RuntimeError(f"in_linear_silu_backward failed ({rc}): {_native.last_error()}")
+    ws = torch.empty(need.value, dtype=torch.uint8, device=lin.device) if need.value else None
+    with torch.cuda.device(lin.device):
+        rc = lib.in_linear_silu_bwd_dmixed(ctypes.byref(p), ctypes.c_void_p(ws.data_ptr() if ws is not None else None),
+                                           need.value, ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))  # fmt: skip
+    if rc != 0:
+        raise RuntimeError(f"in_linear_silu_backward failed ({rc}): {_native.last_error()}")
+    return d_mixed, sums
+
+
 def in_linear_silu_backward(x, weight, bias: Optional[torch.Tensor], user_grad, value_grad, query_grad, key_grad,
                             linear_output, attr_dict):  # fmt: skip
     """Gradients of x, weight and bias (in_linear_silu_backward_plugin.cpp:40-153): with z = linear_output,
     d mixed = cat(grads) * sigmoid(z) * (1 + z * (1 - sigmoid(z))); d x = d mixed @ weight; d weight = d mixed^T @ x;
-    d bias = column sums of d mixed.  A composite of device operations (fp32 element-wise part, library products)."""
+    d bias = column sums of d mixed.  The element-wise stage and the column sums are one HIP kernel
+    (``in_linear_silu_bwd_dmixed`` of the C ABI); the two products are library matrix products."""
     split = [int(s) for s in attr_dict]
     _in_linear_silu_shapes(x, weight, bias, split)
     grads = (user_grad, value_grad, query_grad, key_grad)
@@ -173,13 +205,15 @@ def in_linear_silu_backward(x, weight, bias: Optional[torch.Tensor], user_grad, 
     _check(all(g.size(0) == x.size(0) for g in grads) and linear_output.size(0) == x.size(0),
            "user_grad, value_grad, query_grad, key_grad linear_output dim[0] must equal to x dim[0].")  # fmt: skip
     _check(linear_output.size(1) == weight.size(0), "linear_output dim[1] must equal to weight dim[0].")
-    z = linear_output.float()
-    sig = torch.sigmoid(z)
-    d_mixed = torch.cat([g.float() for g in grads], dim=1) * (sig * (1.0 + z * (1.0 - sig)))
-    d_low = d_mixed.to(x.dtype)
-    x_grad = d_low @ weight
-    weight_grad = d_low.t() @ x
-    bias_grad = d_mixed.sum(dim=0).to(bias.dtype) if bias is not None else None
+    _check(x.dtype in (torch.bfloat16, torch.float16), f"x must be float16 or bfloat16, got {x.dtype}")
+    _check(all(t.dtype == x.dtype for t in (weight, linear_output, *grads)),
+           "weight, linear_output and the gradients must have the dtype of x")  # fmt: skip
+    _check(all(t.is_cuda and t.device == x.device for t in (weight, linear_output, *grads)),
+           "all tensors must be on the GPU of x")  # fmt: skip
+    d_mixed, bias_sums = silu_backward_stage(linear_output, grads, split, want_bias_grad=bias is not None)
+    x_grad = d_mixed @ weight
+    weight_grad = d_mixed.t() @ x
+    bias_grad = bias_sums.to(bias.dtype) if bias is not None else None
     return x_grad, weight_grad, bias_grad, None
 
 

@@ -30,6 +30,8 @@ EXPORTED_SYMBOLS = (
     "ln_mul_fwd_kernel_name",
     "in_linear_silu_fwd",
     "in_linear_silu_fwd_kernel_name",
+    "in_linear_silu_bwd_dmixed_workspace_size",
+    "in_linear_silu_bwd_dmixed",
 )
 
 
@@ -148,6 +150,27 @@ class InLinearSiluParams(ctypes.Structure):
     ]
 
 
+class InLinearSiluBwdParams(ctypes.Structure):
+    """Mirror of ``in_linear_silu_bwd_params`` (include/ops_rec_activation_mi355.h)."""
+
+    _fields_ = [
+        ("struct_size", ctypes.c_uint32),
+        ("reserved0", ctypes.c_uint32),
+        ("linear_output", ctypes.c_void_p),
+        ("user_grad", ctypes.c_void_p),
+        ("value_grad", ctypes.c_void_p),
+        ("query_grad", ctypes.c_void_p),
+        ("key_grad", ctypes.c_void_p),
+        ("d_mixed", ctypes.c_void_p),
+        ("bias_grad", ctypes.c_void_p),
+        ("m", ctypes.c_int64),
+        ("n", ctypes.c_int64),
+        ("split", ctypes.c_int64 * 4),
+        ("dtype", ctypes.c_int32),
+        ("reserved1", ctypes.c_uint32),
+    ]
+
+
 _lib: Optional[ctypes.CDLL] = None
 
 
@@ -193,6 +216,12 @@ def load() -> ctypes.CDLL:
     lib.in_linear_silu_fwd.argtypes = [ctypes.POINTER(InLinearSiluParams), ctypes.c_void_p]
     lib.in_linear_silu_fwd_kernel_name.restype = ctypes.c_char_p
     lib.in_linear_silu_fwd_kernel_name.argtypes = [ctypes.POINTER(InLinearSiluParams)]
+    lib.in_linear_silu_bwd_dmixed_workspace_size.restype = ctypes.c_int
+    lib.in_linear_silu_bwd_dmixed_workspace_size.argtypes = [ctypes.POINTER(InLinearSiluBwdParams),
+                                                             ctypes.POINTER(ctypes.c_uint64)]  # fmt: skip
+    lib.in_linear_silu_bwd_dmixed.restype = ctypes.c_int
+    lib.in_linear_silu_bwd_dmixed.argtypes = [ctypes.POINTER(InLinearSiluBwdParams), ctypes.c_void_p, ctypes.c_uint64,
+                                              ctypes.c_void_p]  # fmt: skip
     _lib = lib
     return lib
 
@@ -210,6 +239,12 @@ def new_params() -> FwdParams:
 def new_in_linear_silu_params() -> InLinearSiluParams:
     p = InLinearSiluParams()
     p.struct_size = ctypes.sizeof(InLinearSiluParams)
+    return p
+
+
+def new_in_linear_silu_bwd_params() -> InLinearSiluBwdParams:
+    p = InLinearSiluBwdParams()
+    p.struct_size = ctypes.sizeof(InLinearSiluBwdParams)
     return p
 
 

@@ -54,9 +54,14 @@ def in_linear_silu(x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.T
     return parts + (mixed,)
 
 
-def in_linear_silu_backward(x, weight, grads: Sequence[torch.Tensor], linear_output):
-    """(d x, d weight, d bias) in float64."""
+def silu_backward_stage(grads: Sequence[torch.Tensor], linear_output):
+    """d mixed = cat(grads) * silu'(linear_output) in float64."""
     z = linear_output.double()
     sig = 1.0 / (1.0 + torch.exp(-z))
-    d_mixed = torch.cat([g.double() for g in grads], dim=1) * sig * (1.0 + z * (1.0 - sig))
+    return torch.cat([g.double() for g in grads], dim=1) * sig * (1.0 + z * (1.0 - sig))
+
+
+def in_linear_silu_backward(x, weight, grads: Sequence[torch.Tensor], linear_output):
+    """(d x, d weight, d bias) in float64."""
+    d_mixed = silu_backward_stage(grads, linear_output)
     return d_mixed @ weight.double(), d_mixed.t() @ x.double(), d_mixed.sum(dim=0)

@@ -223,3 +223,31 @@ def test_autograd_through_the_operator(dtype):
         scale = want.abs().max().item()
         torch.testing.assert_close(got.double().cpu(), want, rtol=tol, atol=tol * scale)
     assert xd.grad.dtype == dtype and wd.grad.dtype == dtype and bd.grad.dtype == torch.float32
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m,split", [(1, [16, 16, 16, 16]), (63, [16, 48, 32, 32]), (200, [512, 496, 528, 512]),
+                                     (1000, [2304] * 4), (4097, [256, 128, 64, 64])])  # fmt: skip
+def test_backward_silu_stage_through_the_c_abi(dtype, m, split):
+    # in_linear_silu_bwd_dmixed: d_mixed = cat(grads) * silu'(linear_output) and its column sums, against the oracle;
+    # d_mixed within one rounding step of the type, the sums within the fp32 summation error of m terms
+    from ops_rec import _activation
+
+    n = sum(split)
+    g = torch.Generator().manual_seed(m + n)
+    lin = (torch.randn(m, n, generator=g) * 2).to(dtype)
+    grads = [torch.randn(m, s, generator=g).to(dtype) for s in split]
+    lin_d, grads_d = lin.to(DEV), [t.to(DEV) for t in grads]
+    d_mixed, sums = _activation.silu_backward_stage(lin_d, grads_d, split)
+    want = O.silu_backward_stage(grads, lin)
+    got = d_mixed.double().cpu()
+    step = ULP[dtype] * torch.clamp(want.abs(), min=2.0**-14)
+    assert ((got - want).abs() <= 0.51 * step + 1e-7).all()
+    want_sums = want.sum(dim=0)
+    mass = want.abs().sum(dim=0)
+    assert ((sums.double().cpu() - want_sums).abs() <= mass * 2.0**-20 + 1e-6).all()
+    # the same bits on a second launch (no atomics), and no bias gradient when none is wanted
+    d2, s2 = _activation.silu_backward_stage(lin_d, grads_d, split)
+    assert torch.equal(d2, d_mixed) and torch.equal(s2, sums)
+    d3, s3 = _activation.silu_backward_stage(lin_d, grads_d, split, want_bias_grad=False)
+    assert s3 is None and torch.equal(d3, d_mixed)

@@ -123,3 +123,46 @@ def test_no_cpu_implementation():
     x = torch.zeros(4, 16, dtype=torch.float16)
     with pytest.raises((NotImplementedError, RuntimeError)):
         torch.ops.ops_rec.distance_in_linear_silu(x, torch.zeros(64, 16, dtype=torch.float16), torch.zeros(64), [16] * 4)
+
+
+def test_backward_stage_c_abi_validation_codes():
+    lib = _native.load()
+    ws = ctypes.c_uint64(99)
+
+    def valid():
+        p = _native.new_in_linear_silu_bwd_params()
+        p.linear_output, p.user_grad, p.value_grad, p.query_grad, p.key_grad = 0x1000, 0x2000, 0x3000, 0x4000, 0x5000
+        p.d_mixed, p.bias_grad = 0x6000, 0x7000
+        p.m, p.n = 130, 256
+        for i in range(4):
+            p.split[i] = 64
+        p.dtype = _native.DT_FP16
+        return p
+
+    p = valid()
+    assert lib.in_linear_silu_bwd_dmixed_workspace_size(ctypes.byref(p), ctypes.byref(ws)) == 0
+    assert ws.value == 3 * 256 * 4  # ceil(130 / 64) partial rows of n floats
+    p.bias_grad = None
+    assert lib.in_linear_silu_bwd_dmixed_workspace_size(ctypes.byref(p), ctypes.byref(ws)) == 0 and ws.value == 0
+    assert lib.in_linear_silu_bwd_dmixed_workspace_size(ctypes.byref(p), None) == 161001
+    assert lib.in_linear_silu_bwd_dmixed(None, None, 0, None) == 161001
+    # a missing or short workspace is refused before any device call
+    p = valid()
+    assert lib.in_linear_silu_bwd_dmixed(ctypes.byref(p), None, 0, None) == 161004
+    assert lib.in_linear_silu_bwd_dmixed(ctypes.byref(p), ctypes.c_void_p(0x9000), 100, None) == 161004
+    for name, value, code, text in [
+        ("struct_size", 4, 161002, "struct_size"),
+        ("linear_output", None, 161001, "must all be given"),
+        ("key_grad", None, 161001, "must all be given"),
+        ("d_mixed", None, 161001, "must all be given"),
+        ("dtype", _native.DT_FP32, 161002, "bf16 or fp16"),
+        ("m", 0, 161002, "non-empty"),
+        ("n", 272, 161002, "sum\\(split_list\\)"),
+        ("n", 48, 161002, "weight dim\\[0\\]"),
+        ("user_grad", 0x2004, 161002, "multiple of 16 bytes"),
+    ]:
+        p = valid()
+        setattr(p, name, value)
+        got = lib.in_linear_silu_bwd_dmixed_workspace_size(ctypes.byref(p), ctypes.byref(ws))
+        assert got == code, (name, got, _native.last_error())
+        assert re.search(text, _native.last_error()), _native.last_error()
