@@ -27,8 +27,12 @@ __global__ __launch_bounds__(kIlsBwdThreads) void in_linear_silu_dmixed_kernel(c
 {
     __shared__ float s_sums[4][kIlsBwdCols];
     const int col_lane = threadIdx.x & 63, row_lane = threadIdx.x >> 6;
-    const int col = blockIdx.x * kIlsBwdCols + col_lane * 8;
-    const int64_t row0 = static_cast<int64_t>(blockIdx.y) * kIlsBwdRows;
+    // one grid dimension, column blocks fastest: the workgroups in flight write whole rows between them
+    const int col_blocks = (a.n + kIlsBwdCols - 1) / kIlsBwdCols;
+    const int row_block = blockIdx.x / col_blocks;
+    const int col_block = blockIdx.x - row_block * col_blocks;
+    const int col = col_block * kIlsBwdCols + col_lane * 8;
+    const int64_t row0 = static_cast<int64_t>(row_block) * kIlsBwdRows;
     const bool in_cols = col < a.n;
     const uint16_t* grad = nullptr;
     int grad_cols = 0, grad_col = 0;
@@ -90,9 +94,9 @@ __global__ __launch_bounds__(kIlsBwdThreads) void in_linear_silu_dmixed_kernel(c
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         const int c = threadIdx.x + j * kIlsBwdThreads;
-        const int gc = blockIdx.x * kIlsBwdCols + c;
+        const int gc = col_block * kIlsBwdCols + c;
         if (gc < a.n) {
-            a.partial_sums[static_cast<int64_t>(blockIdx.y) * a.n + gc] =
+            a.partial_sums[static_cast<int64_t>(row_block) * a.n + gc] =
                 (s_sums[0][c] + s_sums[1][c]) + (s_sums[2][c] + s_sums[3][c]);
         }
     }

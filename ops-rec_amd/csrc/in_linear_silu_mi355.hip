@@ -146,7 +146,7 @@ int validate_bwd(const in_linear_silu_bwd_params* p)
             return hstu::set_error(HSTU_ERR_INVALID, "every tensor must start at a multiple of 16 bytes");
         }
     }
-    if ((p->m + hstu::kIlsBwdRows - 1) / hstu::kIlsBwdRows > 0x7fffffff / 2) {
+    if ((p->m + hstu::kIlsBwdRows - 1) / hstu::kIlsBwdRows * ((p->n + hstu::kIlsBwdCols - 1) / hstu::kIlsBwdCols) > 0x7fffffff) {
         return hstu::set_error(HSTU_ERR_INVALID, "too many rows");
     }
     return HSTU_OK;
@@ -206,10 +206,10 @@ HSTU_API int in_linear_silu_bwd_dmixed(const in_linear_silu_bwd_params* p, void*
     const unsigned row_blocks = static_cast<unsigned>(bwd_row_blocks(p));
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (p->dtype == HSTU_DT_BF16) {
-        hipLaunchKernelGGL(hstu::in_linear_silu_dmixed_kernel<hstu::bf16_tag>, dim3(col_blocks, row_blocks),
+        hipLaunchKernelGGL(hstu::in_linear_silu_dmixed_kernel<hstu::bf16_tag>, dim3(row_blocks * col_blocks),
                            dim3(hstu::kIlsBwdThreads), 0, s, a);
     } else {
-        hipLaunchKernelGGL(hstu::in_linear_silu_dmixed_kernel<hstu::f16_tag>, dim3(col_blocks, row_blocks),
+        hipLaunchKernelGGL(hstu::in_linear_silu_dmixed_kernel<hstu::f16_tag>, dim3(row_blocks * col_blocks),
                            dim3(hstu::kIlsBwdThreads), 0, s, a);
     }
     if (need > 0) {
