@@ -25,7 +25,6 @@ namespace hstu {
 
 constexpr int kIlsThreads = 256;
 constexpr int kIlsTileM = 128;  // x rows per workgroup
-constexpr int kIlsTileN = 128;  // weight rows (output columns) per workgroup
 constexpr int kIlsStepK = 32;
 constexpr int kIlsXcds = 8;  // MI355X: 8 XCDs, workgroups dealt round-robin
 
@@ -66,9 +65,17 @@ __device__ __forceinline__ float ils_silu(float v)
     return v * __builtin_amdgcn_rcpf(1.0f + t);
 }
 
-template <typename Tag, int STAGES>
-__global__ __launch_bounds__(kIlsThreads, (STAGES == 2 ? 4 : (STAGES == 3 ? 3 : 2))) void in_linear_silu_kernel(const InLinearSiluArgs a)
+// workgroups per CU a variant is compiled for (registers and LDS)
+constexpr int ils_workgroups_per_cu(int stages, int wnb) { return wnb == 4 ? 2 : (stages == 2 ? 4 : (stages == 3 ? 3 : 2)); }
+
+// WNB = 32-row weight blocks per wavefront: 2 (tile 128 x 128, 64 accumulator registers) or 4 (tile 128 x 256,
+// 128 accumulator registers: twice the MFMAs per k step and per byte staged, for the shapes bound by the products)
+template <typename Tag, int STAGES, int WNB = 2>
+__global__ __launch_bounds__(kIlsThreads, ils_workgroups_per_cu(STAGES, WNB)) void in_linear_silu_kernel(const InLinearSiluArgs a)
 {
+    constexpr int kIlsTileN = 64 * WNB;  // weight rows (output columns) per workgroup: 2 wavefronts x WNB blocks of 32
+    constexpr int kReqs = (kIlsTileM + kIlsTileN) / 16 / 4;  // direct-to-LDS instructions per wavefront and stage
+    constexpr int kReqsW = kIlsTileN / 16 / 4;               // of which for weight rows (the first ones)
     constexpr int kStageElems = (kIlsTileM + kIlsTileN) * kIlsStepK;  // 16-bit elements per stage
     // the epilogue stages both results of 32 x rows by 64 columns per wavefront in the same memory
     constexpr int kEpiRowElems = 64 + 8;
@@ -108,18 +115,18 @@ __global__ __launch_bounds__(kIlsThreads, (STAGES == 2 ? 4 : (STAGES == 3 ? 3 : 
     const __amdgpu_buffer_rsrc_t x_rsrc =
         make_rsrc(static_cast<const uint8_t*>(a.x) + m0 * row_bytes, rows_x * row_bytes);
 
-    // ---- requests: a stage is 256 LDS rows of 64 bytes (weight rows 0..127, x rows 128..255); one direct-to-LDS
-    // instruction of a wavefront fills 16 rows (lane -> row lane / 4, physical chunk lane % 4); the 16 instructions of
+    // ---- requests: a stage is LDS rows of 64 bytes (the tile's weight rows, then its 128 x rows); one direct-to-LDS
+    // instruction of a wavefront fills 16 rows (lane -> row lane / 4, physical chunk lane % 4); the instructions of
     // a stage are dealt round-robin to the 4 wavefronts
-    uint32_t req_off[4];   // byte offset of the lane's source row (+ logical chunk) for k = 0
-    int req_chunk[4];      // logical 16-byte chunk (0..3) the lane fetches
+    uint32_t req_off[kReqs];   // byte offset of the lane's source row (+ logical chunk) for k = 0
+    int req_chunk[kReqs];      // logical 16-byte chunk (0..3) the lane fetches
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int q = wave + 4 * i;               // instruction 0..15 of the stage
-        const int lds_row = 16 * q + (lane >> 2);  // 0..255
+    for (int i = 0; i < kReqs; ++i) {
+        const int q = wave + 4 * i;               // instruction of the stage
+        const int lds_row = 16 * q + (lane >> 2);
         const int chunk = (lane & 3) ^ ((lds_row >> 2) & 3);
-        // instructions 0..7 (i < 2) fill the weight rows, 8..15 the x rows
-        const int src_row = i < 2 ? (lds_row & ~31) + ils_column_of_mfma_row(lds_row & 31) : lds_row - kIlsTileN;
+        // the first kReqsW instructions of a wavefront fill weight rows, the others x rows
+        const int src_row = i < kReqsW ? (lds_row & ~31) + ils_column_of_mfma_row(lds_row & 31) : lds_row - kIlsTileN;
         req_chunk[i] = chunk;
         req_off[i] = static_cast<uint32_t>(src_row) * row_bytes + chunk * 16u;
     }
@@ -127,29 +134,32 @@ __global__ __launch_bounds__(kIlsThreads, (STAGES == 2 ? 4 : (STAGES == 3 ? 3 : 
         const int k0 = step * kIlsStepK;
         uint16_t* base = s_tiles + stage * kStageElems;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
+        for (int i = 0; i < kReqs; ++i) {
             const int q = wave + 4 * i;
             // chunks past the end of a row must read as zeros: they would otherwise be the next row's first values
             const bool in_row = k0 + 8 * req_chunk[i] < a.k;
             const uint32_t off = in_row ? req_off[i] + static_cast<uint32_t>(k0) * 2u : kOutOfRange;
-            load_to_lds_b128(i < 2 ? w_rsrc : x_rsrc, base + q * 16 * kIlsStepK, off);
+            load_to_lds_b128(i < kReqsW ? w_rsrc : x_rsrc, base + q * 16 * kIlsStepK, off);
         }
     };
 
-    // ---- operand reads: wavefront (wm, wn) owns x rows 64 wm .. +64 and weight rows 64 wn .. +64 of the tile
+    // ---- operand reads: wavefront (wm, wn) owns x rows 64 wm .. +64 and weight rows 32 WNB wn .. +32 WNB of the tile
     const int wm = wave >> 1, wn = wave & 1;
-    int a_off[2], b_off[2];  // element offsets within a stage of the lane's row for the two 32-row blocks, k chunk 0
+    int a_off[WNB], b_off[2];  // element offsets within a stage of the lane's row of each 32-row block, k chunk 0
     const int r = lane & 31, half = lane >> 5;
 #pragma unroll
+    for (int blk = 0; blk < WNB; ++blk) {
+        a_off[blk] = (32 * WNB * wn + 32 * blk + r) * kIlsStepK;
+    }
+#pragma unroll
     for (int blk = 0; blk < 2; ++blk) {
-        a_off[blk] = (64 * wn + 32 * blk + r) * kIlsStepK;
         b_off[blk] = (kIlsTileN + 64 * wm + 32 * blk + r) * kIlsStepK;
     }
-    const int swz = (r >> 2) & 3;  // the same for all four rows above: they differ by multiples of 32
+    const int swz = (r >> 2) & 3;  // the same for all the rows above: they differ by multiples of 32
 
-    f32x16_t acc[2][2];  // [weight block][x block]
+    f32x16_t acc[WNB][2];  // [weight block][x block]
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
+    for (int i = 0; i < WNB; ++i) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
 #pragma unroll
@@ -165,10 +175,11 @@ __global__ __launch_bounds__(kIlsThreads, (STAGES == 2 ? 4 : (STAGES == 3 ? 3 : 
         request(s, s);
     }
     constexpr int kWait0 = 0 | (7 << 4) | (15 << 8);
-    constexpr int kWait4 = 4 | (7 << 4) | (15 << 8);
-    constexpr int kWait8 = 8 | (7 << 4) | (15 << 8);
+    constexpr int kWait4 = kReqs | (7 << 4) | (15 << 8);
+    constexpr int kWait8 = 2 * kReqs | (7 << 4) | (15 << 8);
+    static_assert(2 * kReqs <= 15, "the count must fit the low bits of the wait instruction");
     for (int t = 0; t < n_steps; ++t) {
-        // requests issued after step t's own: steps t+1 .. t+STAGES-2 (4 instructions each)
+        // requests issued after step t's own: steps t+1 .. t+STAGES-2 (kReqs instructions each)
         const int later = min(STAGES - 2, n_steps - 1 - t);
         __builtin_amdgcn_sched_barrier(0);
         if (later >= 2) {
@@ -188,14 +199,17 @@ __global__ __launch_bounds__(kIlsThreads, (STAGES == 2 ? 4 : (STAGES == 3 ? 3 : 
 #pragma unroll
         for (int kk = 0; kk < 2; ++kk) {
             const int chunk = ((2 * kk + half) ^ swz) * 8;
-            u32x4_t wa[2], xb[2];
+            u32x4_t wa[WNB], xb[2];
+#pragma unroll
+            for (int blk = 0; blk < WNB; ++blk) {
+                wa[blk] = *reinterpret_cast<const u32x4_t*>(st + a_off[blk] + chunk);
+            }
 #pragma unroll
             for (int blk = 0; blk < 2; ++blk) {
-                wa[blk] = *reinterpret_cast<const u32x4_t*>(st + a_off[blk] + chunk);
                 xb[blk] = *reinterpret_cast<const u32x4_t*>(st + b_off[blk] + chunk);
             }
 #pragma unroll
-            for (int i = 0; i < 2; ++i) {
+            for (int i = 0; i < WNB; ++i) {
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
                     acc[i][j] = mfma32<Tag>(wa[i], xb[j], acc[i][j]);
@@ -214,75 +228,80 @@ __global__ __launch_bounds__(kIlsThreads, (STAGES == 2 ? 4 : (STAGES == 3 ? 3 : 
     __builtin_amdgcn_s_barrier();  // every wavefront is done reading the last stage
     uint16_t* staged = s_tiles + wave * kEpiWaveElems;
     const int out_row = lane >> 3, out_chunk = lane & 7;
-    const int out_col = n0 + 64 * wn + 8 * out_chunk;  // first of the lane's 8 columns when it writes back
-    // the split these 8 columns belong to (split sizes are multiples of 16, the 8 columns are aligned to 8)
-    uint16_t* split_base;
-    int split_cols, split_col;
-    if (out_col < split1) {
-        split_base = static_cast<uint16_t*>(a.user), split_cols = split1, split_col = out_col;
-    } else if (out_col < split2) {
-        split_base = static_cast<uint16_t*>(a.value), split_cols = split2 - split1, split_col = out_col - split1;
-    } else if (out_col < split3) {
-        split_base = static_cast<uint16_t*>(a.query), split_cols = split3 - split2, split_col = out_col - split2;
-    } else {
-        split_base = static_cast<uint16_t*>(a.key), split_cols = a.n - split3, split_col = out_col - split3;
-    }
-    float bias[2][2][8];
+    // the wavefront's columns go out 64 at a time (two weight blocks): WNB / 2 rounds
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-#pragma unroll
-        for (int run = 0; run < 2; ++run) {
-            const int col = n0 + 64 * wn + 32 * i + 16 * run + 8 * half;
-            const bool have = a.bias != nullptr && col < a.n;
-            const float4 b0 = have ? *reinterpret_cast<const float4*>(a.bias + col) : make_float4(0.f, 0.f, 0.f, 0.f);
-            const float4 b1 = have ? *reinterpret_cast<const float4*>(a.bias + col + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
-            bias[i][run][0] = b0.x, bias[i][run][1] = b0.y, bias[i][run][2] = b0.z, bias[i][run][3] = b0.w;
-            bias[i][run][4] = b1.x, bias[i][run][5] = b1.y, bias[i][run][6] = b1.z, bias[i][run][7] = b1.w;
+    for (int ch = 0; ch < WNB / 2; ++ch) {
+        const int col0 = n0 + 32 * WNB * wn + 64 * ch;  // first column of this round
+        const int out_col = col0 + 8 * out_chunk;      // first of the lane's 8 columns when it writes back
+        // the split these 8 columns belong to (split sizes are multiples of 16, the 8 columns are aligned to 8)
+        uint16_t* split_base;
+        int split_cols, split_col;
+        if (out_col < split1) {
+            split_base = static_cast<uint16_t*>(a.user), split_cols = split1, split_col = out_col;
+        } else if (out_col < split2) {
+            split_base = static_cast<uint16_t*>(a.value), split_cols = split2 - split1, split_col = out_col - split1;
+        } else if (out_col < split3) {
+            split_base = static_cast<uint16_t*>(a.query), split_cols = split3 - split2, split_col = out_col - split2;
+        } else {
+            split_base = static_cast<uint16_t*>(a.key), split_cols = a.n - split3, split_col = out_col - split3;
         }
-    }
-#pragma unroll
-    for (int j = 0; j < 2; ++j) {
+        float bias[2][2][8];
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
 #pragma unroll
             for (int run = 0; run < 2; ++run) {
-                // accumulator element 8 * run + e is MFMA row 8g + 4h + (e % 4) with g = 2 * run + e / 4: column
-                // 32 i + 16 run + 8 h + e of the wavefront's 64.  linear_output = the sum rounded once; SiLU is taken
-                // of the rounded value, as in the reference.
-                u32x4_t lin, out;
+                const int col = col0 + 32 * i + 16 * run + 8 * half;
+                const bool have = a.bias != nullptr && col < a.n;
+                const float4 b0 = have ? *reinterpret_cast<const float4*>(a.bias + col) : make_float4(0.f, 0.f, 0.f, 0.f);
+                const float4 b1 = have ? *reinterpret_cast<const float4*>(a.bias + col + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+                bias[i][run][0] = b0.x, bias[i][run][1] = b0.y, bias[i][run][2] = b0.z, bias[i][run][3] = b0.w;
+                bias[i][run][4] = b1.x, bias[i][run][5] = b1.y, bias[i][run][6] = b1.z, bias[i][run][7] = b1.w;
+            }
+        }
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    lin[e] = pack2<Tag>(acc[i][j][8 * run + 2 * e] + bias[i][run][2 * e],
-                                        acc[i][j][8 * run + 2 * e + 1] + bias[i][run][2 * e + 1]);
-                    float lo, hi;
-                    ils_unpack2<Tag>(lin[e], lo, hi);
-                    out[e] = pack2<Tag>(ils_silu(lo), ils_silu(hi));
+        for (int j = 0; j < 2; ++j) {
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+#pragma unroll
+                for (int run = 0; run < 2; ++run) {
+                    // accumulator element 8 * run + e is MFMA row 8g + 4h + (e % 4) with g = 2 * run + e / 4: column
+                    // 32 i + 16 run + 8 h + e of the round's 64.  linear_output = the sum rounded once; SiLU is taken
+                    // of the rounded value, as in the reference.
+                    u32x4_t lin, out;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        lin[e] = pack2<Tag>(acc[2 * ch + i][j][8 * run + 2 * e] + bias[i][run][2 * e],
+                                            acc[2 * ch + i][j][8 * run + 2 * e + 1] + bias[i][run][2 * e + 1]);
+                        float lo, hi;
+                        ils_unpack2<Tag>(lin[e], lo, hi);
+                        out[e] = pack2<Tag>(ils_silu(lo), ils_silu(hi));
+                    }
+                    uint16_t* at = staged + r * kEpiRowElems + 32 * i + 16 * run + 8 * half;
+                    *reinterpret_cast<u32x4_t*>(at) = lin;
+                    *reinterpret_cast<u32x4_t*>(at + 32 * kEpiRowElems) = out;
                 }
-                uint16_t* at = staged + r * kEpiRowElems + 32 * i + 16 * run + 8 * half;
-                *reinterpret_cast<u32x4_t*>(at) = lin;
-                *reinterpret_cast<u32x4_t*>(at + 32 * kEpiRowElems) = out;
             }
-        }
-        // the wavefront's own lanes wrote what its lanes now read: LDS keeps a wavefront's accesses in order; the fence
-        // keeps the compiler from moving the reads up
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            // the wavefront's own lanes wrote what its lanes now read: LDS keeps a wavefront's accesses in order; the
+            // fence keeps the compiler from moving the reads up
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int row_in_block = 8 * q + out_row;
-            const int64_t row = m0 + 64 * wm + 32 * j + row_in_block;
-            const uint16_t* from = staged + row_in_block * kEpiRowElems + 8 * out_chunk;
-            const u32x4_t lin = *reinterpret_cast<const u32x4_t*>(from);
-            const u32x4_t out = *reinterpret_cast<const u32x4_t*>(from + 32 * kEpiRowElems);
-            if (row < a.m && out_col < a.n) {
-                *reinterpret_cast<u32x4_t*>(static_cast<uint16_t*>(a.linear_output) + row * a.n + out_col) = lin;
-                *reinterpret_cast<u32x4_t*>(split_base + row * split_cols + split_col) = out;
+            for (int q = 0; q < 4; ++q) {
+                const int row_in_block = 8 * q + out_row;
+                const int64_t row = m0 + 64 * wm + 32 * j + row_in_block;
+                const uint16_t* from = staged + row_in_block * kEpiRowElems + 8 * out_chunk;
+                const u32x4_t lin = *reinterpret_cast<const u32x4_t*>(from);
+                const u32x4_t out = *reinterpret_cast<const u32x4_t*>(from + 32 * kEpiRowElems);
+                if (row < a.m && out_col < a.n) {
+                    *reinterpret_cast<u32x4_t*>(static_cast<uint16_t*>(a.linear_output) + row * a.n + out_col) = lin;
+                    *reinterpret_cast<u32x4_t*>(split_base + row * split_cols + split_col) = out;
+                }
             }
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
 }
 

@@ -16,20 +16,34 @@ using hstu::InLinearSiluArgs;
 struct IlsVariant {
     const char* name;
     void (*kernel)(const InLinearSiluArgs);
+    int tile_n;  // output columns per workgroup
 };
 
-// [type: bf16, fp16][ring of 2 stages, four workgroups per CU; ring of 3 stages, three workgroups per CU].  Measured
-// on MI355X over k = 64 .. 2048 with rings of 2, 3 and 4 stages: workgroups per CU count for more than prefetch depth
-// (4 stages, two workgroups per CU, was slowest everywhere); 3 stages win by 3-7 % for k = 128 .. 512, 2 stages by
-// 2-4 % at k <= 64 and at k = 768 .. 2048; at k = 8192 (weights of 512 MB, grouped tile order) 4 stages win by 10 %.
-const IlsVariant kVariants[2][3] = {
-    {{"in_linear_silu_bf16_stages2", hstu::in_linear_silu_kernel<hstu::bf16_tag, 2>},
-     {"in_linear_silu_bf16_stages3", hstu::in_linear_silu_kernel<hstu::bf16_tag, 3>},
-     {"in_linear_silu_bf16_stages4", hstu::in_linear_silu_kernel<hstu::bf16_tag, 4>}},
-    {{"in_linear_silu_f16_stages2", hstu::in_linear_silu_kernel<hstu::f16_tag, 2>},
-     {"in_linear_silu_f16_stages3", hstu::in_linear_silu_kernel<hstu::f16_tag, 3>},
-     {"in_linear_silu_f16_stages4", hstu::in_linear_silu_kernel<hstu::f16_tag, 4>}},
+// [type: bf16, fp16][ring of 2 stages; 3 stages; 4 stages; 2 stages with 128 x 256 tiles].  Measured on MI355X over
+// k = 64 .. 8192: for 128 x 128 tiles, workgroups per CU count for more than prefetch depth (4 stages, two workgroups
+// per CU, slowest everywhere up to k = 2048); 3 stages win by 3-7 % for k = 128 .. 512, 2 stages by 2-4 % at k <= 64
+// and k = 768.  From k = 1024 on the products dominate and the 128 x 256 tile (twice the MFMAs per k step and per byte
+// staged, two workgroups per CU) wins: 633 -> 549 us at k = 2048, 607 -> 484 us at m = n = 8192, k = 4096
+// (1.14 PFLOP/s).
+#define ILS_VARIANT(tag, tagname, S, W) \
+    {"in_linear_silu_" tagname "_stages" #S "_tile" #W, hstu::in_linear_silu_kernel<hstu::tag, S, (W) / 64>, W}
+const IlsVariant kVariants[2][4] = {
+    {ILS_VARIANT(bf16_tag, "bf16", 2, 128), ILS_VARIANT(bf16_tag, "bf16", 3, 128), ILS_VARIANT(bf16_tag, "bf16", 4, 128),
+     ILS_VARIANT(bf16_tag, "bf16", 2, 256)},
+    {ILS_VARIANT(f16_tag, "f16", 2, 128), ILS_VARIANT(f16_tag, "f16", 3, 128), ILS_VARIANT(f16_tag, "f16", 4, 128),
+     ILS_VARIANT(f16_tag, "f16", 2, 256)},
 };
+
+const IlsVariant* select(const in_linear_silu_params* p)
+{
+    int ring;
+    if (p->k >= 1024) {
+        ring = 3;
+    } else {
+        ring = (p->k <= 64 || p->k > 512) ? 0 : 1;
+    }
+    return &kVariants[p->dtype == HSTU_DT_BF16 ? 0 : 1][ring];
+}
 
 constexpr int64_t kMinDim = 16;
 constexpr int64_t kMaxDim = 512 * 16;
@@ -42,8 +56,9 @@ bool xcd_groups(const in_linear_silu_params* p) { return p->n * p->k * 2 > (int6
 // workgroups of a launch: m tiles (rounded up to whole groups of one per XCD in the grouped order) times n tiles
 int64_t grid_size(const in_linear_silu_params* p)
 {
+    const int tile_n = select(p)->tile_n;
     int64_t tiles_m = (p->m + hstu::kIlsTileM - 1) / hstu::kIlsTileM;
-    const int64_t tiles_n = (p->n + hstu::kIlsTileN - 1) / hstu::kIlsTileN;
+    const int64_t tiles_n = (p->n + tile_n - 1) / tile_n;
     if (xcd_groups(p)) {
         tiles_m = (tiles_m + hstu::kIlsXcds - 1) / hstu::kIlsXcds * hstu::kIlsXcds;
     }
@@ -96,16 +111,10 @@ int validate(const in_linear_silu_params* p)
     }
     const int64_t tiles = grid_size(p);
     if (tiles > 0x7fffffff) {
-        return hstu::set_error(HSTU_ERR_INVALID, "too many rows: %lld tiles of %d x %d", static_cast<long long>(tiles),
-                               hstu::kIlsTileM, hstu::kIlsTileN);
+        return hstu::set_error(HSTU_ERR_INVALID, "too many rows: %lld tiles of %d rows", static_cast<long long>(tiles),
+                               hstu::kIlsTileM);
     }
     return HSTU_OK;
-}
-
-const IlsVariant* select(const in_linear_silu_params* p)
-{
-    const int ring = p->k > 4096 ? 2 : ((p->k <= 64 || p->k > 512) ? 0 : 1);
-    return &kVariants[p->dtype == HSTU_DT_BF16 ? 0 : 1][ring];
 }
 
 int validate_bwd(const in_linear_silu_bwd_params* p)

@@ -102,6 +102,8 @@ def test_reference_common_input(dtype):
     (40, 8192, 2048, [2048] * 4),
     (33, 32768, 8192, [8192] * 4),           # the largest legal k and n
     (200, 1024, 240 + 16, [256] * 4),
+    (333, 4096, 1024, [1024, 1008, 1040, 1024]),  # 128 x 256 tiles: partial tiles in m, split edges inside a tile
+    (130, 4096 + 64, 1040, [1040, 1040, 1040, 1040]),  # ... and a last n tile of 64 columns, k = 32.5 steps
 ])  # fmt: skip
 def test_edges_and_long_k(m, n, k, split):
     g = torch.Generator().manual_seed(m + n + k)
@@ -141,7 +143,7 @@ def test_no_bias_through_the_c_abi_on_a_side_stream():
     s_ = torch.cuda.Stream(device=DEV)
     s_.wait_stream(torch.cuda.current_stream())
     lib = _native.load()
-    assert lib.in_linear_silu_fwd_kernel_name(ctypes.byref(p)).decode() == "in_linear_silu_f16_stages2"
+    assert lib.in_linear_silu_fwd_kernel_name(ctypes.byref(p)).decode() == "in_linear_silu_f16_stages2_tile128"
     assert lib.in_linear_silu_fwd(ctypes.byref(p), ctypes.c_void_p(s_.cuda_stream)) == 0
     s_.synchronize()
     want = O.in_linear_silu(x, w, None, split, round_to=torch.float16)

@@ -60,9 +60,9 @@ def test_c_abi_validation_codes():
     lib = _native.load()
     assert lib.in_linear_silu_fwd(None, None) == 161001
     p = _valid()
-    assert lib.in_linear_silu_fwd_kernel_name(ctypes.byref(p)).decode() == "in_linear_silu_bf16_stages2"
+    assert lib.in_linear_silu_fwd_kernel_name(ctypes.byref(p)).decode() == "in_linear_silu_bf16_stages2_tile128"
     p.bias = None  # no bias is allowed
-    assert lib.in_linear_silu_fwd_kernel_name(ctypes.byref(p)).decode() == "in_linear_silu_bf16_stages2"
+    assert lib.in_linear_silu_fwd_kernel_name(ctypes.byref(p)).decode() == "in_linear_silu_bf16_stages2_tile128"
 
     def split(*v):
         def apply(p):
@@ -109,14 +109,14 @@ def test_kernel_variant_selection():
             p.split[i] = n // 4
         return lib.in_linear_silu_fwd_kernel_name(ctypes.byref(p)).decode()
 
-    # a ring of two k steps and four workgroups per CU for short and for long k, three stages in between, four for the longest (measured)
-    assert name(16, 64) == "in_linear_silu_bf16_stages2"
-    assert name(64, 9216) == "in_linear_silu_bf16_stages2"
-    assert name(128, 1024) == "in_linear_silu_bf16_stages3"
-    assert name(512, 2048) == "in_linear_silu_bf16_stages3"
-    assert name(768, 3072) == "in_linear_silu_bf16_stages2"
-    assert name(4096, 16384) == "in_linear_silu_bf16_stages2"
-    assert name(8192, 32768, _native.DT_FP16) == "in_linear_silu_f16_stages4"
+    # a ring of two k steps and four workgroups per CU for short k, three stages in the middle, 128 x 256 tiles from k = 1024 on (measured)
+    assert name(16, 64) == "in_linear_silu_bf16_stages2_tile128"
+    assert name(64, 9216) == "in_linear_silu_bf16_stages2_tile128"
+    assert name(128, 1024) == "in_linear_silu_bf16_stages3_tile128"
+    assert name(512, 2048) == "in_linear_silu_bf16_stages3_tile128"
+    assert name(768, 3072) == "in_linear_silu_bf16_stages2_tile128"
+    assert name(1024, 4096) == "in_linear_silu_bf16_stages2_tile256"
+    assert name(8192, 32768, _native.DT_FP16) == "in_linear_silu_f16_stages2_tile256"
 
 
 def test_no_cpu_implementation():
