@@ -1,5 +1,6 @@
-// forward kernels for fp32 inputs, and the paged gather kernel
+// forward kernels for fp32 inputs, the kernel for the shapes no tuned kernel takes, and the paged gather kernel
 #include "hstu_fwd_f32_kernel.hip.h"
+#include "hstu_fwd_generic_kernel.hip.h"
 #include "hstu_paged_gather.hip.h"
 #include "hstu_variants.h"
 
@@ -16,6 +17,14 @@ const Variant kTable[2][2][4] = {{HSTU_F32_DIMS(false, false), HSTU_F32_DIMS(fal
                                  {HSTU_F32_DIMS(true, false), HSTU_F32_DIMS(true, true)}};
 }
 const Variant (*fwd_variants_f32())[2][4] { return kTable; }
+
+namespace {
+#define HSTU_GENERIC_VARIANT(T, name) \
+    {"hstu_fwd_generic_" name, nullptr, nullptr, hstu_fwd_generic_kernel<T>, nullptr, nullptr, nullptr, kGenericMaxDim, 256, 0}
+const Variant kGeneric[3] = {HSTU_GENERIC_VARIANT(__bf16, "bf16"), HSTU_GENERIC_VARIANT(_Float16, "f16"),
+                             HSTU_GENERIC_VARIANT(float, "f32")};
+}  // namespace
+const Variant* fwd_variants_generic() { return kGeneric; }
 
 void launch_paged_gather(const PagedGatherArgs& a, unsigned grid, hipStream_t stream)
 {

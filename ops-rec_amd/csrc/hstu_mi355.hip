@@ -160,38 +160,25 @@ const Variant* select(const hstu_jagged_fwd_params* p)
         fail(HSTU_ERR_UNSUPPORTED, "out_dtype must equal dtype for bf16 / fp16 / fp32 inputs");
         return nullptr;
     }
-    if (p->head_dim_qk % 8 != 0) {
-        fail(HSTU_ERR_UNSUPPORTED, "q/k head dim %lld is not a multiple of 8", (long long)p->head_dim_qk);
-        return nullptr;
-    }
     const int64_t dmax = p->head_dim_qk > p->head_dim_v ? p->head_dim_qk : p->head_dim_v;
-    int slot;
-    if (dmax <= 32) {
-        slot = 0;
-    } else if (dmax <= 64) {
-        slot = 1;
-    } else if (dmax <= 128) {
-        slot = 2;
-    } else if (dmax <= 256) {
-        slot = 3;
-    } else {
-        fail(HSTU_ERR_UNSUPPORTED, "head dims above 256 are not built in this library version (got %lld)",
-             (long long)dmax);
-        return nullptr;
-    }
-    {
-        // one sequence of one head group is addressed through a 32-bit buffer descriptor, with room above it
-        // for the offsets that mark a request as out of range
-        const int64_t esize = p->dtype == HSTU_DT_FP32 ? 4 : 2;
-        const int64_t span_q = p->max_seq_len_q * p->num_heads_q * dmax * esize;
-        const int64_t span_k = p->max_seq_len_k * p->num_heads_k * dmax * esize;
-        const int64_t span_b = p->max_seq_len_q * p->max_seq_len_k * esize;
-        if (span_q >= (1LL << 30) || span_k >= (1LL << 30) ||
-            ((p->attn_bias != nullptr || p->mask_type == HSTU_MASK_CUSTOM) && span_b >= (1LL << 31))) {
-            fail(HSTU_ERR_UNSUPPORTED, "max_seq_len x heads x head dim spans 1 GiB or more per sequence");
+    // The tuned kernels take head dims up to 256 with a q/k head dim that is a multiple of 8 (16-byte chunks), and
+    // address one sequence of one head group through a 32-bit buffer descriptor, with room above it for the offsets
+    // that mark a request as out of range.  Whatever else the reference accepts (head dims up to 512, any q/k head
+    // dim) goes to the kernel written for coverage.
+    const int64_t esize = p->dtype == HSTU_DT_FP32 ? 4 : 2;
+    const int64_t span_q = p->max_seq_len_q * p->num_heads_q * dmax * esize;
+    const int64_t span_k = p->max_seq_len_k * p->num_heads_k * dmax * esize;
+    const int64_t span_b = p->max_seq_len_q * p->max_seq_len_k * esize;
+    const bool wide_span = span_q >= (1LL << 30) || span_k >= (1LL << 30) ||
+                           ((p->attn_bias != nullptr || p->mask_type == HSTU_MASK_CUSTOM) && span_b >= (1LL << 31));
+    if (p->head_dim_qk % 8 != 0 || dmax > 256 || wide_span) {
+        if (p->dtype == HSTU_DT_FP8_E4M3) {
+            fail(HSTU_ERR_UNSUPPORTED, "fp8 inputs are built for head dims up to 256 (got %lld)", (long long)dmax);
             return nullptr;
         }
+        return &hstu::fwd_variants_generic()[p->dtype == HSTU_DT_BF16 ? 0 : (p->dtype == HSTU_DT_FP16 ? 1 : 2)];
     }
+    const int slot = dmax <= 32 ? 0 : (dmax <= 64 ? 1 : (dmax <= 128 ? 2 : 3));
     if (p->dtype == HSTU_DT_FP8_E4M3) {
         return &hstu::fwd_variants_f8()[p->out_dtype == HSTU_DT_FP16 ? 0 : 1][slot <= 1 ? 0 : slot - 1];
     }

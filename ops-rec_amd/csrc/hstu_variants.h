@@ -36,6 +36,8 @@ const Variant (*fwd_variants_f16())[2][4];
 const Variant (*fwd_variants_f8())[3];
 // forward, fp32 inputs: [rab][custom mask][dim slot: 32, 64, 128, 256]
 const Variant (*fwd_variants_f32())[2][4];
+// forward, any head dims up to 512 (written for coverage, not speed): [bf16, fp16, fp32]
+const Variant* fwd_variants_generic();
 // backward: [rab][custom mask][dim slot: 64, 128, 256]
 const BwdVariant (*bwd_variants_bf16())[2][3];
 const BwdVariant (*bwd_variants_f16())[2][3];

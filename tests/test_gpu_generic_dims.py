@@ -1,0 +1,80 @@
+"""Head dims the tuned kernels do not take -- above 256 (the reference goes to 512,
+hstu_forward_v1/op_host/tiling_policy.cpp:68-93) or a q/k head dim that is not a multiple of 8 -- run through the
+kernel written for coverage.  Same oracle, same tolerances as the parity tests (bf16 / fp16: atol = rtol = 1e-2 of
+the largest reference value; fp32: 1e-4)."""
+
+import dataclasses
+
+import pytest
+import torch
+
+import ops_rec
+from ops_rec import _ops
+from oracle import hstu_oracle as O
+from helpers import small_case
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def check(w, expect_generic=True):
+    d = w.to(DEV)
+    k_offs = d.seq_offset if d.seq_offset_k is None else d.seq_offset_k
+    max_k = d.max_seq_len if d.max_seq_len_k is None else d.max_seq_len_k
+    prepared = _ops.prepare_forward(d.q, d.k, d.v, d.mask, d.attn_bias, d.mask_type, d.max_seq_len, max_k, d.silu_scale,
+                                    d.seq_offset, k_offs, d.num_context, d.num_target, d.target_group_size, d.alpha)  # fmt: skip
+    assert prepared.kernel_name().startswith("hstu_fwd_generic_") == expect_generic, prepared.kernel_name()
+    out = ops_rec.ascendc.attention.hstu_jagged(*d.op_args())
+    ref = O.hstu_jagged_forward(w.q, w.k, w.v, out_dtype=torch.float32, **w.oracle_kwargs())
+    assert out.dtype == w.q.dtype and out.shape == ref.shape
+    tol = 1e-4 if w.q.dtype == torch.float32 else 1e-2
+    scale = max(1.0, float(ref.abs().max()))
+    torch.testing.assert_close(out.float().cpu(), ref, rtol=tol, atol=tol * scale)
+    return out
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("dim,dim_v", [(1, 16), (4, 16), (12, 48), (20, 32), (100, 112), (130, 64), (260, 272), (384, 384),
+                                       (512, 512), (64, 512), (512, 16)])  # fmt: skip
+def test_head_dims_beyond_the_tuned_kernels(dtype, dim, dim_v):
+    check(small_case(seed=dim + dim_v, batch=3, heads=2, dim=dim, dim_v=dim_v, lo=1, hi=150, dtype=dtype, std=0.5))
+
+
+@pytest.mark.parametrize("kw", [
+    dict(rab=True), dict(custom_mask=True), dict(rab=True, custom_mask=True), dict(ctx=5, max_target=7, group=2),
+    dict(ctx=3, max_target=4, group=1, rab=True), dict(heads=4, heads_k=2), dict(heads=8, heads_k=1, rab=True),
+    dict(delta=True), dict(delta=True, rab=True, index_dtype=torch.int64), dict(alpha=0.3, rab=True),
+])  # fmt: skip
+def test_all_the_semantics_at_an_odd_head_dim(kw):
+    base = dict(seed=len(kw) + 11, batch=4, heads=2, dim=36, dim_v=48, lo=20, hi=160, dtype=torch.bfloat16, std=0.5)
+    base.update(kw)
+    check(small_case(**base))
+
+
+def test_no_mask_and_long_rows_at_head_dim_512():
+    w = small_case(seed=5, batch=2, heads=2, dim=512, dim_v=512, lo=200, hi=300, dtype=torch.float16, std=0.3)
+    check(dataclasses.replace(w, mask_type=2))
+
+
+def test_rows_past_the_last_offset_are_zero_and_empty_sequences_cost_nothing():
+    w = small_case(seed=6, batch=4, heads=2, dim=20, dim_v=32, lo=1, hi=40, dtype=torch.bfloat16, std=0.5)
+    # two more rows than the offsets cover, and a repeated trailing offset (an empty last sequence)
+    pad = lambda t: torch.cat([t, torch.ones(2, *t.shape[1:], dtype=t.dtype)])  # noqa: E731
+    offs = torch.cat([w.seq_offset, w.seq_offset[-1:]])
+    w2 = dataclasses.replace(w, q=pad(w.q), k=pad(w.k), v=pad(w.v), seq_offset=offs, lengths=w.lengths + [0])
+    out = check(w2)
+    assert torch.count_nonzero(out[-2:]) == 0
+
+
+def test_backward_falls_to_the_composite_for_these_dims():
+    w = small_case(seed=7, batch=2, heads=2, dim=12, dim_v=16, lo=10, hi=50, dtype=torch.bfloat16, std=0.5).to(DEV)
+    q, k, v = (t.clone().requires_grad_() for t in (w.q, w.k, w.v))
+    args = list(w.op_args())
+    args[0], args[1], args[2] = q, k, v
+    out = ops_rec.ascendc.attention.hstu_jagged(*args)
+    out.float().sum().backward()
+    c = w.to("cpu")
+    qc, kc, vc = (t.float().clone().requires_grad_() for t in (c.q, c.k, c.v))
+    O.hstu_jagged_forward(qc, kc, vc, out_dtype=torch.float32, **c.oracle_kwargs()).sum().backward()
+    for g, r in ((q.grad, qc.grad), (k.grad, kc.grad), (v.grad, vc.grad)):
+        torch.testing.assert_close(g.float().cpu(), r, rtol=2e-2, atol=2e-2 * float(r.abs().max()))

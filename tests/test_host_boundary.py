@@ -228,12 +228,9 @@ def test_c_abi_validation_codes():
         ("head_dim_qk", 513, 161002, "512"),
         ("index_dtype", 5, 161002, "index_dtype"),
         ("dtype", 9, 161002, "unknown dtype"),
-        ("head_dim_qk", 12, 161003, "multiple of 8"),
     ]:
         p = _valid_params()
         setattr(p, field, value)
-        if field == "head_dim_qk" and value == 12:
-            p.head_dim_v = 16
         got = rc(p)
         assert got == code, (field, value, got, _native.last_error())
         assert re.search(text, _native.last_error()), (field, _native.last_error())
@@ -260,6 +257,12 @@ def test_kernel_variant_selection():
     assert "rabtrue" in name(attn_bias=0x2000)
     assert "masktrue" in name(mask=0x2000, mask_type=3)
     assert "f16" in name(dtype=_native.DT_FP16, out_dtype=_native.DT_FP16)
+    # what the reference accepts beyond the tuned kernels (head dims up to 512, any q/k head dim) goes to the kernel
+    # written for coverage
+    assert name(head_dim_qk=12, head_dim_v=16) == "hstu_fwd_generic_bf16"
+    assert name(head_dim_qk=1, head_dim_v=512, dtype=_native.DT_FP16, out_dtype=_native.DT_FP16) == "hstu_fwd_generic_f16"
+    assert name(head_dim_qk=512, head_dim_v=512, dtype=_native.DT_FP32, out_dtype=_native.DT_FP32) == "hstu_fwd_generic_f32"
+    assert name(head_dim_qk=264, head_dim_v=64, attn_bias=0x2000) == "hstu_fwd_generic_bf16"
 
 
 def test_fp8_variant_selection_and_limits():
@@ -283,6 +286,7 @@ def test_fp8_variant_selection_and_limits():
         (dict(attn_bias=0x2000), "not built for fp8"),
         (dict(mask=0x2000, mask_type=3), "not built for fp8"),
         (dict(head_dim_qk=24, head_dim_v=16), "multiple of 16"),
+        (dict(head_dim_qk=512, head_dim_v=512), "head dims up to 256"),
     ]:
         assert name(**kw) is None
         assert re.search(text, _native.last_error()), (kw, _native.last_error())
