@@ -2,6 +2,7 @@
 """Benchmark of the HSTU jagged attention forward on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2|C3|C4|C5] [--no-cpu]
+                    [--forward-only | --backward --ln-mul --in-linear-silu]
 
 A "step" is one forward over one synthetic jagged batch whose inputs already sit in HBM.
 The default workload is the configuration the headline metric is quoted on (C2: bf16, batch 32,
@@ -19,6 +20,11 @@ timed with events on that same stream; the cost of one call through the Python e
                     same launch against the HBM bound on compulsory bytes.
 ``cpu_baseline`` -- the oracle's dense-padded fp32 restatement of the reference's PyTorch golden path,
                     timed on this host's cores on the same batch (a reported baseline, not a target).
+
+After the timed forward steps the same line also carries, each with its own roofline and measured outside the timed
+region of the headline: ``backward`` (hstu_jagged_backward on the same workload), ``ln_mul`` (the operator that
+consumes the attention output) and ``in_linear_silu`` (the operator that produces U, V, Q, K).  Naming any of
+--backward / --ln-mul / --in-linear-silu runs only those; --forward-only runs none.
 """
 
 from __future__ import annotations
@@ -127,7 +133,7 @@ def bench_ln_mul(attn_out, stream, args):
             "cases": cases}  # fmt: skip
 
 
-def bench_in_linear_silu(tokens, stream, args):
+def bench_in_linear_silu(tokens, width, stream, args):
     """in_linear_silu through ``in_linear_silu_fwd`` of the C ABI, events on the launch stream.  Algorithmic bytes per
     launch: x, weight and bias read once, linear_output and the four splits written once =
     2 (m k + n k) + 4 n + 4 m n; flops 2 m n k."""
@@ -142,8 +148,8 @@ def bench_in_linear_silu(tokens, stream, args):
     dev = torch.device("cuda", 0)
     cases = []
     # (m, n, k): a shape of the reference's own test (test_in_linear_silu.py:127-130), store-bound; and the layer of
-    # this workload: its tokens, embedding 512 -> U, V, Q, K of 512 each (heads x dim of the attention workload)
-    for m, n, k, what in ((16384, 9216, 64, "reference test shape"), (tokens, 2048, 512, "layer of this workload")):
+    # this workload: its tokens, embedding `width` = heads x dim of the attention workload -> U, V, Q, K of `width` each
+    for m, n, k, what in ((16384, 9216, 64, "reference test shape"), (tokens, 4 * width, width, "layer of this workload")):
         x = torch.randn(m, k, device=dev).to(torch.bfloat16)
         wt = (torch.randn(n, k, device=dev) / k**0.5).to(torch.bfloat16)
         bias = torch.randn(n, device=dev)
@@ -214,6 +220,9 @@ def main() -> int:
     ap.add_argument("--backward", action="store_true",
                     help="also time hstu_jagged_backward (the two HIP backward kernels) on the same workload and add a "
                     "'backward' object to the line (bf16 workloads only)")  # fmt: skip
+    ap.add_argument("--forward-only", action="store_true",
+                    help="time the attention forward only; by default (none of --backward / --ln-mul / --in-linear-silu "
+                    "given) the line also carries the 'backward', 'ln_mul' and 'in_linear_silu' objects")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="after the timed steps also run 5 plain device-to-device copies of this many MiB, so that a "
                     "counter run (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) can be scaled by a kernel of known traffic")  # fmt: skip
@@ -353,8 +362,19 @@ def main() -> int:
         },
     }
 
-    # ---- backward (optional): d q, d k, d v (and d attn_bias) through the operator ----
-    if args.backward and not fp8:
+    # The operators either side of the forward: the ones asked for, or all of them when none is named.  The headline
+    # numbers above are complete at this point; a leg that fails reports its error instead of its figures.
+    asked = args.backward or args.ln_mul or args.in_linear_silu
+    legs = {name: (getattr(args, name) if asked else not args.forward_only) for name in ("backward", "ln_mul", "in_linear_silu")}
+
+    def guarded(name, fn):
+        try:
+            result[name] = fn()
+        except Exception as exc:  # noqa: BLE001
+            result[name] = {"error": f"{type(exc).__name__}: {exc}"[:300]}
+
+    # ---- backward: d q, d k, d v (and d attn_bias) through the operator ----
+    def bench_backward():
         grad = torch.randn(prepared.out.shape, device=dev).to(prepared.out.dtype)
         zeros = None if w.num_context is None and w.num_target is None else torch.zeros(len(w.lengths), dtype=w.seq_offset.dtype, device=dev)
         bwd_args = (grad, w.q, w.k, w.v, w.mask, w.attn_bias, w.mask_type, w.max_seq_len, w.silu_scale, w.seq_offset,
@@ -372,7 +392,7 @@ def main() -> int:
         torch.cuda.synchronize()
         bwd_ms = e0.elapsed_time(e1) / n_bwd
         bwd_flops = flops * 5 // 2  # five products (S, dP, dV, dK, dQ) against the forward's two
-        result["backward"] = {
+        return {
             "ms_per_step": round(bwd_ms, 6),
             "steps": n_bwd,
             "flops_per_step": bwd_flops,
@@ -383,12 +403,14 @@ def main() -> int:
             "issued for the five of the formula)",
         }
 
-    # ---- ln_mul (optional): the operator that takes the attention output next in an HSTU layer ----
-    if args.ln_mul:
-        result["ln_mul"] = bench_ln_mul(prepared.out, stream, args)
-
-    if args.in_linear_silu:
-        result["in_linear_silu"] = bench_in_linear_silu(sum(w.lengths), stream, args)
+    if legs["backward"] and not fp8:
+        guarded("backward", bench_backward)
+    # ---- ln_mul: the operator that takes the attention output next in an HSTU layer ----
+    if legs["ln_mul"] and not fp8:
+        guarded("ln_mul", lambda: bench_ln_mul(prepared.out, stream, args))
+    # ---- in_linear_silu: the operator that produces U, V, Q, K in front of attention ----
+    if legs["in_linear_silu"] and not fp8:
+        guarded("in_linear_silu", lambda: bench_in_linear_silu(sum(w.lengths), n_q * d_v, stream, args))
 
     # ---- CPU baseline: dense-padded fp32 golden path on this host's cores ----
     if not args.no_cpu and w_cpu is not None:
