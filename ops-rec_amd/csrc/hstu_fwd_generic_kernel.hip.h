@@ -10,10 +10,10 @@
 // hstu_fwd_f32_kernel so that the host launches both the same way.
 //
 // A workgroup walks its 128 rows 16 at a time.  For 16 rows and 16 keys, thread (r, c) of the 256 computes the
-// score of row r and key c from fp32 copies of the Q and K rows in LDS (row stride padded by one float: the 16 key
-// rows a wavefront reads at the same head-dim position fall into different banks), applies bias, SiLU, scale and
-// visibility, and leaves P in LDS; thread (r, c) then owns the output columns c, c + 16, ... of row r and adds
-// P[r, :] . V[:, column].  Scores are not rounded to the input type before the second product.
+// score of row r and key c from fp32 copies of the Q and K rows in LDS (zero-padded to a multiple of 4 floats and
+// read 16 bytes at a time; row stride padded by 4 floats so that the 16 key rows read together fall into different
+// banks), applies bias, SiLU, scale and visibility, and leaves P in LDS; thread (r, c) then owns the output columns
+// 4c .. 4c + 3, 4c + 64 .. of row r and adds P[r, :] . V[:, columns].  Scores are not rounded to the input type before the second product.
 #pragma once
 #include "hstu_fwd_kernel.hip.h"
 
@@ -33,10 +33,10 @@ __global__ __launch_bounds__(256) void hstu_fwd_generic_kernel(const FwdArgs a)
     constexpr int kThreads = 256;
     constexpr int RB = 16;  // query rows per pass
     constexpr int KB = 16;  // keys per tile
-    constexpr int kStride = kGenericMaxDim + 1;
-    __shared__ float s_q[RB * kStride];
-    __shared__ float s_k[KB * kStride];
-    __shared__ float s_v[KB * kGenericMaxDim];
+    constexpr int kStride = kGenericMaxDim + 4;  // floats per staged Q / K row: 16-byte reads, rows 4 banks apart
+    __shared__ __attribute__((aligned(16))) float s_q[RB * kStride];
+    __shared__ __attribute__((aligned(16))) float s_k[KB * kStride];
+    __shared__ __attribute__((aligned(16))) float s_v[KB * kGenericMaxDim];
     __shared__ float s_p[RB][KB + 1];
 
     const int tid = threadIdx.x;
@@ -93,7 +93,9 @@ __global__ __launch_bounds__(256) void hstu_fwd_generic_kernel(const FwdArgs a)
     const int64_t v_row_elems = static_cast<int64_t>(a.n_heads_k) * a.d_v;
     const int64_t bias_plane = (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k);
     const int r = tid >> 4, c = tid & 15;
-    constexpr int kMaxCols = kGenericMaxDim / 16;
+    constexpr int kMaxCols = kGenericMaxDim / 64;  // groups of 4 consecutive output columns per thread
+    const int d_qk4 = (a.d_qk + 3) & ~3;                 // Q / K rows are staged zero-padded to a multiple of 4
+    typedef __attribute__((ext_vector_type(4))) float f32x4_t;
 
     for (int pass = 0; pass < kBlockM / RB; ++pass) {
         const int rb = r0 + pass * RB;
@@ -130,23 +132,23 @@ __global__ __launch_bounds__(256) void hstu_fwd_generic_kernel(const FwdArgs a)
             kmax = kmax < 0 ? 0 : (kmax > sk ? sk : kmax);
         }
         __syncthreads();  // the previous pass is done with s_q
-        for (int e = tid; e < RB * a.d_qk; e += kThreads) {
-            const int rr = e / a.d_qk, dd = e - rr * a.d_qk;
+        for (int e = tid; e < RB * d_qk4; e += kThreads) {
+            const int rr = e / d_qk4, dd = e - rr * d_qk4;
             const int qrow = rb + rr;
-            s_q[rr * kStride + dd] = qrow < sq ? generic_load<T>(a.q, (q0 + qrow) * q_row_elems + static_cast<int64_t>(h) * a.d_qk + dd) : 0.0f;
+            s_q[rr * kStride + dd] = (qrow < sq && dd < a.d_qk) ? generic_load<T>(a.q, (q0 + qrow) * q_row_elems + static_cast<int64_t>(h) * a.d_qk + dd) : 0.0f;
         }
-        float acc[kMaxCols];
+        f32x4_t acc[kMaxCols];
 #pragma unroll
         for (int jj = 0; jj < kMaxCols; ++jj) {
-            acc[jj] = 0.0f;
+            acc[jj] = f32x4_t{0.0f, 0.0f, 0.0f, 0.0f};
         }
         for (int kt = 0; kt * KB < kmax; ++kt) {
             const int key0 = kt * KB;
             __syncthreads();  // the previous tile's products are done (and s_q is written)
-            for (int e = tid; e < KB * a.d_qk; e += kThreads) {
-                const int kr = e / a.d_qk, dd = e - kr * a.d_qk;
+            for (int e = tid; e < KB * d_qk4; e += kThreads) {
+                const int kr = e / d_qk4, dd = e - kr * d_qk4;
                 const int key = key0 + kr;
-                s_k[kr * kStride + dd] = key < sk ? generic_load<T>(a.k, (k0 + key) * k_row_elems + static_cast<int64_t>(hk) * a.d_qk + dd) : 0.0f;
+                s_k[kr * kStride + dd] = (key < sk && dd < a.d_qk) ? generic_load<T>(a.k, (k0 + key) * k_row_elems + static_cast<int64_t>(hk) * a.d_qk + dd) : 0.0f;
             }
             for (int e = tid; e < KB * a.d_v; e += kThreads) {
                 const int kr = e / a.d_v, dd = e - kr * a.d_v;
@@ -157,12 +159,13 @@ __global__ __launch_bounds__(256) void hstu_fwd_generic_kernel(const FwdArgs a)
             const int key = key0 + c;
             float p = 0.0f;
             if (row_in && key < lim && !(key >= hole_lo && key < hole_hi)) {
-                float s = 0.0f;
-                const float* qr = s_q + r * kStride;
-                const float* kr = s_k + c * kStride;
-                for (int dd = 0; dd < a.d_qk; ++dd) {
-                    s += qr[dd] * kr[dd];
+                const f32x4_t* qr = reinterpret_cast<const f32x4_t*>(s_q + r * kStride);
+                const f32x4_t* kr = reinterpret_cast<const f32x4_t*>(s_k + c * kStride);
+                f32x4_t s4 = {0.0f, 0.0f, 0.0f, 0.0f};
+                for (int dd = 0; dd < d_qk4 / 4; ++dd) {
+                    s4 += qr[dd] * kr[dd];
                 }
+                float s = (s4[0] + s4[1]) + (s4[2] + s4[3]);
                 const int64_t at = bias_plane + static_cast<int64_t>(row) * a.max_k + key;
                 if (a.rab != nullptr) {
                     s += generic_load<T>(a.rab, at);
@@ -175,14 +178,19 @@ __global__ __launch_bounds__(256) void hstu_fwd_generic_kernel(const FwdArgs a)
             }
             s_p[r][c] = p;
             __syncthreads();
+            float pr[KB];
+#pragma unroll
+            for (int cc = 0; cc < KB; ++cc) {
+                pr[cc] = s_p[r][cc];
+            }
 #pragma unroll
             for (int jj = 0; jj < kMaxCols; ++jj) {
-                const int col = c + 16 * jj;
+                const int col = 4 * c + 64 * jj;  // d_v is a multiple of 16: a group of 4 columns is inside or outside
                 if (col < a.d_v) {
-                    float t = acc[jj];
+                    f32x4_t t = acc[jj];
 #pragma unroll
                     for (int cc = 0; cc < KB; ++cc) {
-                        t += s_p[r][cc] * s_v[cc * kGenericMaxDim + col];
+                        t += pr[cc] * *reinterpret_cast<const f32x4_t*>(s_v + cc * kGenericMaxDim + col);
                     }
                     acc[jj] = t;
                 }
@@ -191,9 +199,12 @@ __global__ __launch_bounds__(256) void hstu_fwd_generic_kernel(const FwdArgs a)
         if (row_in) {
 #pragma unroll
             for (int jj = 0; jj < kMaxCols; ++jj) {
-                const int col = c + 16 * jj;
+                const int col = 4 * c + 64 * jj;
                 if (col < a.d_v) {
-                    out[(q0 + row) * o_row_elems + static_cast<int64_t>(h) * a.d_v + col] = static_cast<T>(acc[jj]);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        out[(q0 + row) * o_row_elems + static_cast<int64_t>(h) * a.d_v + col + e] = static_cast<T>(acc[jj][e]);
+                    }
                 }
             }
         }
