@@ -10,7 +10,7 @@
     python hstu_layer_example.py [--batch 32] [--heads 4] [--dim 128] [--embed 512] [--lo 256] [--hi 1024] [--steps 50]
 
 Checks the chain against the same chain in fp32 torch operations on the device, then times it; prints one JSON line
-with the time of each operator and of the block.
+with the time of each operator, of the block through the Python entry points, and of the block replayed from a HIP graph.
 """
 
 import argparse
@@ -62,6 +62,20 @@ def timed(fn, steps):
     return e0.elapsed_time(e1) / steps * 1e3
 
 
+def graph_replay_us(fn, steps):
+    """The same calls captured once in a HIP graph and replayed: what a serving loop pays per block."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        fn()
+    return timed(graph.replay, steps)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--batch", type=int, default=32)
@@ -103,6 +117,7 @@ def main():
                                                         None, 0, args.dim**-0.5), args.steps),  # fmt: skip
         "ln_mul_us": timed(lambda: act.ln_mul(o.view(t, hd), u, gamma, beta), args.steps),
         "block_us": timed(lambda: block(*common), args.steps),
+        "block_graph_replay_us": graph_replay_us(lambda: block(*common), args.steps),
         "fp32_torch_chain_us": timed(lambda: block_fp32(*common), 2),
     }
     print(json.dumps({"tokens": t, "batch": args.batch, "heads": args.heads, "dim": args.dim, "embed": args.embed,
