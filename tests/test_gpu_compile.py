@@ -1,0 +1,96 @@
+"""The operators under torch.compile (the reference's "graph" tests: torch.compile(op, dynamic=True, fullgraph=True),
+e.g. ascendc/activation/ln_mul/test/pytest/test_ln_mul.py:69-85): tracing needs the schemas, the Meta
+implementations and the autograd formulas to agree with what the kernels return.  The "aot_eager" backend is used:
+it runs dynamo, fake-tensor propagation and AOT autograd exactly as inductor would, and then calls the operators
+themselves (they are opaque to a code generator anyway).  torch.library.opcheck repeats the same checks per operator."""
+
+import pytest
+import torch
+
+import ops_rec
+from helpers import small_case
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def compiled(fn):
+    return torch.compile(fn, backend="aot_eager", fullgraph=True, dynamic=True)
+
+
+def test_ln_mul_compiled_matches_eager():
+    op = ops_rec.ascendc.activation.ln_mul
+    fn = compiled(op)
+    for a, r, dtype in [(8, 64, torch.float32), (33, 512, torch.bfloat16), (5, 100, torch.float32)]:
+        x, u = torch.randn(a, r, device=DEV).to(dtype), torch.randn(a, r, device=DEV).to(dtype)
+        g, b = torch.randn(r, device=DEV), torch.randn(r, device=DEV)
+        assert torch.equal(fn(x=x, u=u, gamma=g, beta=b), op(x, u, g, b))
+
+
+def test_in_linear_silu_compiled_forward_and_backward():
+    op = ops_rec.ascendc.activation.distance_in_linear_silu
+    fn = compiled(op)
+    for m in (100, 257):
+        x = torch.randn(m, 64, device=DEV).to(torch.bfloat16)
+        w = (torch.randn(512, 64, device=DEV) / 8).to(torch.bfloat16)
+        b = torch.randn(512, device=DEV)
+        split = [96, 96, 160, 160]
+        got, want = fn(x=x, weight=w, bias=b, attr_dict=split), op(x, w, b, split)
+        assert all(torch.equal(g, t) for g, t in zip(got, want))
+
+    def loss(x, w, b):
+        u, v, q, k, _ = op(x, w, b, [128] * 4)
+        return (u.float() * 0.5).sum() + (v.float() * q.float()).sum() - k.float().sum()
+
+    args = [t.requires_grad_() for t in (torch.randn(130, 64, device=DEV).to(torch.bfloat16),
+                                        (torch.randn(512, 64, device=DEV) / 8).to(torch.bfloat16),
+                                        torch.randn(512, device=DEV))]  # fmt: skip
+    loss(*args).backward()
+    eager = [t.grad.clone() for t in args]
+    for t in args:
+        t.grad = None
+    compiled(loss)(*args).backward()
+    for t, e in zip(args, eager):
+        assert torch.equal(t.grad, e)
+
+
+@pytest.mark.parametrize("kw", [dict(), dict(rab=True, ctx=3, max_target=5, group=1), dict(delta=True)])
+def test_hstu_jagged_compiled_forward_and_backward(kw):
+    w = small_case(seed=3, batch=3, heads=2, dim=64, lo=10, hi=200, dtype=torch.bfloat16, std=0.5, **kw).to(DEV)
+    op = ops_rec.ascendc.attention.hstu_jagged
+    args = list(w.op_args())
+    want = op(*args)
+    got = compiled(lambda *a: op(*a))(*args)
+    assert torch.equal(got, want)
+
+    def loss(q, k, v):
+        a = list(args)
+        a[0], a[1], a[2] = q, k, v
+        return op(*a).float().square().sum()
+
+    qkv = [t.clone().requires_grad_() for t in (w.q, w.k, w.v)]
+    loss(*qkv).backward()
+    eager = [t.grad.clone() for t in qkv]
+    for t in qkv:
+        t.grad = None
+    compiled(loss)(*qkv).backward()
+    for t, e in zip(qkv, eager):
+        assert torch.equal(t.grad, e)
+
+
+def test_opcheck_of_every_operator():
+    checks = ("test_schema", "test_faketensor", "test_aot_dispatch_dynamic")
+    x, u = torch.randn(16, 64, device=DEV), torch.randn(16, 64, device=DEV)
+    torch.library.opcheck(torch.ops.ops_rec.ln_mul.default, (x, u, torch.randn(64, device=DEV), torch.randn(64, device=DEV)),
+                          test_utils=checks)  # fmt: skip
+    xb = torch.randn(40, 32, device=DEV).to(torch.float16).requires_grad_()
+    wb = (torch.randn(128, 32, device=DEV) / 6).to(torch.float16).requires_grad_()
+    bb = torch.randn(128, device=DEV).requires_grad_()
+    torch.library.opcheck(torch.ops.ops_rec.distance_in_linear_silu.default, (xb, wb, bb, [32, 32, 32, 32]),
+                          test_utils=checks + ("test_autograd_registration",))  # fmt: skip
+    w = small_case(seed=5, batch=2, heads=2, dim=32, lo=5, hi=60, dtype=torch.float16, std=0.5).to(DEV)
+    args = list(w.op_args())
+    args[0], args[1], args[2] = (t.clone().requires_grad_() for t in (w.q, w.k, w.v))
+    torch.library.opcheck(torch.ops.ops_rec.hstu_jagged.equal, tuple(args), test_utils=checks + ("test_autograd_registration",))
+    q4 = torch.randn(2, 40, 2, 32, device=DEV).to(torch.bfloat16)
+    torch.library.opcheck(torch.ops.ops_rec.hstu_dense.default, (q4, q4, q4, None, None, 0, 40, 0.0), test_utils=checks)
