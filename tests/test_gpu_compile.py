@@ -94,3 +94,33 @@ def test_opcheck_of_every_operator():
     torch.library.opcheck(torch.ops.ops_rec.hstu_jagged.equal, tuple(args), test_utils=checks + ("test_autograd_registration",))
     q4 = torch.randn(2, 40, 2, 32, device=DEV).to(torch.bfloat16)
     torch.library.opcheck(torch.ops.ops_rec.hstu_dense.default, (q4, q4, q4, None, None, 0, 40, 0.0), test_utils=checks)
+
+
+def test_opcheck_of_the_backward_and_paged_operators():
+    from helpers import paged_case
+
+    checks = ("test_schema", "test_faketensor", "test_aot_dispatch_dynamic")
+    w = small_case(seed=8, batch=2, heads=2, dim=64, lo=5, hi=90, dtype=torch.bfloat16, std=0.5).to(DEV)
+    out = ops_rec.ascendc.attention.hstu_jagged(*w.op_args())
+    grad = torch.randn_like(out)
+    torch.library.opcheck(torch.ops.ops_rec.hstu_jagged_backward.equal,
+                          (grad, w.q, w.k, w.v, None, None, 0, w.max_seq_len, w.silu_scale, w.seq_offset, None, None, 0, w.alpha),
+                          test_utils=checks)  # fmt: skip
+    q4 = torch.randn(2, 48, 2, 64, device=DEV).to(torch.bfloat16)
+    torch.library.opcheck(torch.ops.ops_rec.hstu_dense_backward.default,
+                          (torch.randn_like(q4), q4, q4, q4, None, None, 0, 48, 0.0), test_utils=checks)  # fmt: skip
+    c = {n: (t.to(DEV) if torch.is_tensor(t) else t)
+         for n, t in paged_case(hist=[32, 48], prev=[0, 70], targets=[4, 6], page_size=32, heads=2, dim=32,
+                                dtype=torch.float16, seed=1).items()}  # fmt: skip
+    torch.library.opcheck(
+        torch.ops.ops_rec.hstu_paged.default,
+        (c["q"], c["k"], c["v"], c["kv_cache"], None, None, 0, c["max_seq_len"], c["max_seq_len_k"], 0.0, c["seq_offset"],
+         c["seq_offset_k"], c["seq_offset_t"], c["page_offsets"], c["page_ids"], c["last_page_len"], c["num_target"], 1, 1.0),
+        test_utils=checks)  # fmt: skip
+    x = torch.randn(40, 32, device=DEV).to(torch.float16)
+    wt = (torch.randn(128, 32, device=DEV) / 6).to(torch.float16)
+    b = torch.randn(128, device=DEV)
+    outs = torch.ops.ops_rec.distance_in_linear_silu(x, wt, b, [32] * 4)
+    grads = [torch.randn_like(t) for t in outs[:4]]
+    torch.library.opcheck(torch.ops.ops_rec.in_linear_silu_backward.default, (x, wt, b, *grads, outs[4], [32] * 4),
+                          test_utils=checks)  # fmt: skip

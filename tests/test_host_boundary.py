@@ -402,3 +402,32 @@ def test_paged_and_dense_backward_ops_are_registered():
     g = torch.empty(2, 5, 4, 32, device="meta", dtype=torch.bfloat16)
     dq, dk, dv, db = torch.ops.ops_rec.hstu_dense_backward(g, g, g, g, None, None, 0, 5, 0.0)
     assert dq.shape == g.shape and tuple(db.shape) == (2, 4, 256, 256)
+
+
+def test_public_headers_are_plain_c(tmp_path):
+    # the boundary is a C ABI: both headers must compile as C99 and as C++11 on their own, and the struct sizes the
+    # Python mirrors assume must be the ones the C compiler sees
+    import shutil
+    import subprocess
+
+    gcc = shutil.which("gcc")
+    if gcc is None:
+        pytest.skip("no gcc on this host")
+    src = tmp_path / "abi.c"
+    src.write_text(
+        '#include "hstu_mi355.h"\n#include "ops_rec_activation_mi355.h"\n#include <stdio.h>\n'
+        "int main(void) { printf(\"%zu %zu %zu %zu %zu %zu %zu\\n\", sizeof(hstu_jagged_fwd_params), "
+        "sizeof(hstu_jagged_bwd_params), sizeof(hstu_paged_fwd_params), sizeof(ln_mul_params), "
+        "sizeof(in_linear_silu_params), sizeof(in_linear_silu_bwd_params), sizeof(void*)); return 0; }\n"
+    )
+    inc = os.path.join(_ROOT, "include")
+    exe = tmp_path / "abi"
+    subprocess.run([gcc, "-std=c99", "-Wall", "-Wextra", "-pedantic", "-Werror", "-I", inc, str(src), "-o", str(exe)], check=True)
+    sizes = [int(v) for v in subprocess.run([str(exe)], capture_output=True, text=True, check=True).stdout.split()]
+    mirrors = [_native.FwdParams, _native.BwdParams, _native.PagedParams, _native.LnMulParams, _native.InLinearSiluParams,
+               _native.InLinearSiluBwdParams, ctypes.c_void_p]  # fmt: skip
+    assert sizes == [ctypes.sizeof(m) for m in mirrors]
+    gxx = shutil.which("g++")
+    if gxx is not None:
+        subprocess.run([gxx, "-std=c++11", "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", "-x", "c++", "-I", inc,
+                        str(src)], check=True)  # fmt: skip
