@@ -533,10 +533,13 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         // to its own buffer in the workspace and counts itself in; the part that finds all others counted in adds
         // the m buffers in part order (so the sum does not depend on who came last) and stores the rows.
         // A level is split only while arrival counters and workspace buffers last, and nothing is split when the
-        // list has an item for every workgroup anyway: measured on MI355X, a part costs about 2 us on top of its
-        // sweep (its own start-up, the hand-over of its accumulators), which a list of 1.4 items per workgroup
-        // (batch 32 x 4 heads, lengths 256..1024) no longer earns back, while a list that leaves workgroups idle
-        // (one 20480-row sequence, or 4 sequences x 2 heads up to 3000 rows) finishes in 0.5 - 0.65 of the time.
+        // list has an item for every workgroup anyway: measured on MI355X, an entry of the list costs 4 - 6 us on
+        // top of its sweep (its own start-up, the hand-over of its accumulators), which a list of 1.4 items per
+        // workgroup (batch 32 x 4 heads, lengths 256..1024) no longer earns back, while a list that leaves workgroups
+        // idle (one 20480-row sequence, or 4 sequences x 2 heads up to 3000 rows) finishes in 0.5 - 0.65 of the time.
+        // For the same reason the target is raised until the list with its parts still has at most one entry per
+        // workgroup: a second round of entries costs more than shorter parts gain (12 x 4 items of 1024 rows:
+        // 42.5 us with the mean as the target, 35.2 us with this rule, 33.5 us unsplit).
         uint32_t split_target = 0;
         uint32_t split_items = 0, split_bufs = 0;
         auto nominal_steps = [&](int qt) -> uint32_t {
@@ -558,6 +561,12 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             split_target = split_target < 8u ? 8u : split_target;
             if (a.ws == nullptr || items >= gridDim.x) {
                 split_target = 0x7fffffffu;  // nothing is split
+            } else {
+                // one round: the entries that splitting adds (at most nominal / target per item) go to the
+                // workgroups that would have had no item
+                const uint32_t spare = gridDim.x - items;
+                const uint32_t fit = (steps - 3u * items + spare - 1u) / spare;
+                split_target = split_target < fit ? fit : split_target;
             }
         }
         uint32_t acc = 0;

@@ -235,8 +235,9 @@ bool may_take_split_variant(const Variant* var, const hstu_jagged_fwd_params* p,
     }
     const int64_t n_qtiles = (p->max_seq_len_q + hstu::kBlockM - 1) / hstu::kBlockM;
     const int64_t n_blocks = n_qtiles * (p->n_offsets - 1) * p->num_heads_q;
-    // (an item of at most 8 sub-tiles is never split: the kernel's parts are at least that long)
-    return n_blocks < 2 * resident && p->max_seq_len_k > 8 * 32;
+    // (items of at most 16 sub-tiles: parts of 8, the kernel's shortest, do not earn back what a part costs --
+    // 8 x 4 sequences of 512 rows: 23.0 us split, 20.7 us not)
+    return n_blocks < 2 * resident && p->max_seq_len_k > 16 * 32;
 }
 uint64_t split_workspace_bytes(const Variant* var, const hstu_jagged_fwd_params* p)
 {
