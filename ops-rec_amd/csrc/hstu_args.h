@@ -37,6 +37,7 @@ struct FwdArgs {
     int n_qtiles;    // ceil(max_q / kBlockM)
     int bh;          // n_batch * n_heads_q
     int bias_vec_ok; // rab / mask rows may be read 4 elements (8 bytes) at a time
+    int out_vec_ok;  // d_v is a multiple of 8 and `out` is 16-byte aligned: output rows may be written 16 bytes at a time
     float c_exp;     // -alpha * log2(e)
     float c_out;     // alpha * silu_scale
     float alpha;     // fp8 inputs only: the kernel folds the per-head scales in itself

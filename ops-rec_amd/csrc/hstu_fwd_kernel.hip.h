@@ -1608,7 +1608,55 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         }
 
         // ---- store O: lane holds query row (wr0 + ln), dims 32*mt + 8*g + 4*lh + 0..3 ----
-        if (store_rows) {
+        // Written as they lie in the registers, the rows would go out in 8-byte pieces, 16 store instructions
+        // touching every 128-byte line of the tile; measured, these partial-line writes cost a 42 us launch 6 us.
+        // So the wavefront passes its 32 rows through LDS (its own K slot of the ring, idle between two sweeps;
+        // 16-byte chunks XOR-ed with the row so that neither side has bank conflicts to speak of) and writes them
+        // 16 bytes per lane, whole lines per instruction.
+        constexpr bool kStagedStore = !F8;  // (fp8 sub-tiles are half the size of the 16-bit output rows)
+        const bool staged = kStagedStore && a.out_vec_ok != 0;
+        if (staged) {
+            // every wavefront's tile requests have landed (the last ones, past the end, move nothing, but they
+            // name the slots) before anybody writes a slot
+            __builtin_amdgcn_s_waitcnt(0);
+            __syncthreads();
+        }
+        if (store_rows && staged) {
+            if constexpr (kStagedStore) {
+                uint16_t* const stage = wave == 0 ? s_k0 : (wave == 1 ? s_k1 : (wave == 2 ? s_k2 : s_k3));
+                constexpr int OCPR = D / 8;  // 16-byte chunks per staged row
+                // the LDS offsets below depend on the lane only; opaque copies of the lane's coordinates keep the
+                // compiler from working them out once, ahead of the item loop, and carrying two dozen registers
+                // through the sweep, where there is none to spare
+                int ln_e = ln, lh_e = lh, lane_e = lane;
+                asm volatile("" : "+v"(ln_e), "+v"(lh_e), "+v"(lane_e));
+#pragma unroll
+                for (int mt = 0; mt < MTILES; ++mt) {
+#pragma unroll
+                    for (int g = 0; g < 4; ++g) {
+                        u32x2_t w;
+                        w[0] = pack2<OutTag>(o_acc[mt][4 * g + 0] * c_out, o_acc[mt][4 * g + 1] * c_out);
+                        w[1] = pack2<OutTag>(o_acc[mt][4 * g + 2] * c_out, o_acc[mt][4 * g + 3] * c_out);
+                        const int chunk = (4 * mt + g) ^ (ln_e & (OCPR - 1));
+                        *reinterpret_cast<u32x2_t*>(stage + ln_e * D + chunk * 8 + 4 * lh_e) = w;
+                    }
+                }
+                // (one wavefront: its LDS accesses execute in order; the fences keep the compiler from moving the reads up)
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                constexpr int RPI = 64 / OCPR;  // rows per store instruction
+                const int rr = lane_e / OCPR;
+                const int cc = lane_e % OCPR;
+#pragma unroll
+                for (int i = 0; i < 32 / RPI; ++i) {
+                    const int r = i * RPI + rr;
+                    const u32x4_t piece = *reinterpret_cast<const u32x4_t*>(stage + r * D + (cc ^ (r & (OCPR - 1))) * 8);
+                    const uint32_t off = (cc * 8 < a.d_v) ? static_cast<uint32_t>(wr0 + r) * o_stride + cc * 16u : kOutOfRange;
+                    __builtin_amdgcn_raw_buffer_store_b128(piece, o_rsrc, static_cast<int>(off), 0, 0);
+                }
+            }
+        } else if (store_rows) {
             const uint32_t row_off = static_cast<uint32_t>(wr0 + ln) * o_stride;
 #pragma unroll
             for (int mt = 0; mt < MTILES; ++mt) {

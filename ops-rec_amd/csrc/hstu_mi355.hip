@@ -625,6 +625,7 @@ int launch_forward(const hstu_jagged_fwd_params* p, const hstu_paged_fwd_params*
     const bool bias_aligned = (reinterpret_cast<uintptr_t>(p->attn_bias) % vec_bytes == 0) &&
                               (reinterpret_cast<uintptr_t>(p->mask) % vec_bytes == 0) && (p->max_seq_len_k % 4 == 0);
     a.bias_vec_ok = bias_aligned ? 1 : 0;
+    a.out_vec_ok = (p->head_dim_v % 8 == 0 && reinterpret_cast<uintptr_t>(p->out) % 16 == 0) ? 1 : 0;
     if (bias_aligned && p->dtype != HSTU_DT_FP32 && reinterpret_cast<uintptr_t>(p->attn_bias) % 16 == 0 &&
         reinterpret_cast<uintptr_t>(p->mask) % 16 == 0 && p->max_seq_len_k % 8 == 0) {
         a.bias_vec_ok = 2;  // 16-byte row alignment: the 16-bit kernels read rab / mask rows 32 bytes per lane
