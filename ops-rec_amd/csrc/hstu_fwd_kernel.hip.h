@@ -730,6 +730,15 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         }
     };
 
+#ifdef HSTU_TIMELINE
+    if (a.timeline && lane == 0) {
+        // where this wavefront runs: HW_ID (CU, shader array, shader engine) and the XCD
+        a.timeline[(static_cast<int64_t>(blockIdx.x) * 4 + wave) * 64 + 62] =
+            static_cast<unsigned long long>(__builtin_amdgcn_s_getreg(0xF804)) |
+            (static_cast<unsigned long long>(__builtin_amdgcn_s_getreg(0xF814)) << 32);
+        a.timeline[(static_cast<int64_t>(blockIdx.x) * 4 + wave) * 64 + 61] = HSTU_CLOCK();
+    }
+#endif
     // =============================== item loop ===============================
     // The first item of a workgroup is fixed (workgroup w: item w / nq of queue w mod nq, nq = number of queues);
     // later ones are pulled from the queue's counter.  With the pull, the position of the next non-empty queue is
@@ -1646,6 +1655,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                 __builtin_amdgcn_wave_barrier();
                 __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
                 constexpr int RPI = 64 / OCPR;  // rows per store instruction
+                constexpr int kNonTemporal = 2;  // cache policy bit nt: the rows are not read again by this kernel (measured: 1 - 4 % of a launch)
                 const int rr = lane_e / OCPR;
                 const int cc = lane_e % OCPR;
 #pragma unroll
@@ -1653,7 +1663,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                     const int r = i * RPI + rr;
                     const u32x4_t piece = *reinterpret_cast<const u32x4_t*>(stage + r * D + (cc ^ (r & (OCPR - 1))) * 8);
                     const uint32_t off = (cc * 8 < a.d_v) ? static_cast<uint32_t>(wr0 + r) * o_stride + cc * 16u : kOutOfRange;
-                    __builtin_amdgcn_raw_buffer_store_b128(piece, o_rsrc, static_cast<int>(off), 0, 0);
+                    __builtin_amdgcn_raw_buffer_store_b128(piece, o_rsrc, static_cast<int>(off), 0, kNonTemporal);
                 }
             }
         } else if (store_rows) {
