@@ -562,11 +562,23 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             if (a.ws == nullptr || items >= gridDim.x) {
                 split_target = 0x7fffffffu;  // nothing is split
             } else {
-                // one round: the entries that splitting adds (at most nominal / target per item) go to the
+                // one round: if the list cut at the mean has more entries than there are workgroups, the target
+                // is raised so that the entries splitting adds (at most nominal / target per item) go to the
                 // workgroups that would have had no item
-                const uint32_t spare = gridDim.x - items;
-                const uint32_t fit = (steps - 3u * items + spare - 1u) / spare;
-                split_target = split_target < fit ? fit : split_target;
+                // (counted in floating point: one thread does this for up to 160 levels, and the count only picks
+                // the rule, so a part more or less at an exact multiple does not matter)
+                uint32_t entries = 0;
+                const float inv_target = 1.0f / static_cast<float>(split_target);
+                for (int l = 0; l < n_levels; ++l) {
+                    const uint32_t cnt = s_rank_start[n_levels - 1 - l] * static_cast<uint32_t>(n_heads);
+                    const uint32_t m = static_cast<uint32_t>(static_cast<float>(nominal_steps(n_levels - 1 - l)) * inv_target + 0.999f);
+                    entries += cnt * (m > static_cast<uint32_t>(kMaxParts) ? static_cast<uint32_t>(kMaxParts) : (m < 1u ? 1u : m));
+                }
+                if (entries > gridDim.x) {
+                    const uint32_t spare = gridDim.x - items;
+                    const uint32_t fit = (steps - 3u * items + spare - 1u) / spare;
+                    split_target = split_target < fit ? fit : split_target;
+                }
             }
         }
         uint32_t acc = 0;
