@@ -93,6 +93,7 @@ struct BwdArgs {
     int n_qtiles;     // ceil(max_q / 128)
     int n_ktiles;     // ceil(max_k / 128)
     int bias_vec_ok;  // rab / mask / d rab rows may be accessed 4 elements (8 bytes) at a time (1), 16 bytes (2)
+    int grad_vec_ok;  // dq / dk / dv are 16-byte aligned and both head dims multiples of 8: rows may be written 16 bytes at a time
     float alpha;
     float scale;  // silu_scale, resolved
 };

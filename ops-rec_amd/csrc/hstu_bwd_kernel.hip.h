@@ -160,6 +160,48 @@ struct SubTile {
     static constexpr int MTILES = D / 32;
 };
 
+// The 32 rows x D columns a wavefront holds in MFMA accumulator layout (lane (ln, lh): row ln, columns
+// 32 mt + 8 g + 4 lh .. + 3), rounded to the 16-bit type, passed through the wavefront's own 32 x D elements of LDS
+// (16-byte chunks XOR-ed with the row) and written 16 bytes per lane: every store instruction writes whole 128-byte
+// lines, where storing the accumulators as they lie writes every line in eight pieces.  `first_row_off` = byte
+// offset of the tile's row 0 under `rsrc`, whose bound drops rows past the end of the sequence.
+template <typename Tag, int D>
+__device__ __forceinline__ void store_tile_rows(uint16_t* stage, const f32x16_t (&acc)[D / 32], const __amdgpu_buffer_rsrc_t rsrc,
+                                                uint32_t first_row_off, uint32_t stride, int dim_limit, int lane)
+{
+    constexpr int CPR = D / 8;  // 16-byte chunks per row
+    // opaque copy of the lane id: the LDS offsets depend on the lane only, and worked out ahead of the sweep they
+    // would take two dozen registers through it
+    int lane_e = lane;
+    asm volatile("" : "+v"(lane_e));
+    const int ln = lane_e & 31, lh = lane_e >> 5;
+#pragma unroll
+    for (int mt = 0; mt < D / 32; ++mt) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            u32x2_t w;
+            w[0] = pack2<Tag>(acc[mt][4 * g + 0], acc[mt][4 * g + 1]);
+            w[1] = pack2<Tag>(acc[mt][4 * g + 2], acc[mt][4 * g + 3]);
+            const int chunk = (4 * mt + g) ^ (ln & (CPR - 1));
+            *reinterpret_cast<u32x2_t*>(stage + ln * D + chunk * 8 + 4 * lh) = w;
+        }
+    }
+    // (one wavefront: its LDS accesses execute in order; the fences keep the compiler from moving the reads up)
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    constexpr int RPI = 64 / CPR;  // rows per store instruction
+    constexpr int kNonTemporal = 2;  // cache policy bit nt: the rows are not read again by this kernel
+    const int rr = lane_e / CPR, cc = lane_e % CPR;
+#pragma unroll
+    for (int i = 0; i < 32 / RPI; ++i) {
+        const int r = i * RPI + rr;
+        const u32x4_t piece = *reinterpret_cast<const u32x4_t*>(stage + r * D + (cc ^ (r & (CPR - 1))) * 8);
+        const uint32_t off = (cc * 8 < dim_limit) ? first_row_off + static_cast<uint32_t>(r) * stride + cc * 16u : kOutOfRange;
+        __builtin_amdgcn_raw_buffer_store_b128(piece, rsrc, static_cast<int>(off), 0, kNonTemporal);
+    }
+}
+
 // ---------------------------------------------------------------------------------------------------------
 // dQ (and d rab)
 // ---------------------------------------------------------------------------------------------------------
@@ -481,7 +523,13 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_bwd_dq_kernel(co
     }
 
     // store dQ: lane holds query row (wr0 + ln), dims 32*mt + 8*g + 4*lh + 0..3
-    {
+    if (a.grad_vec_ok != 0) {
+        // (every wavefront is done with the ring before anybody writes its rows into a stage)
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        uint16_t* const stage = wave == 0 ? s_k0 : (wave == 1 ? s_k1 : (wave == 2 ? s_k2 : s_v0));
+        store_tile_rows<Tag, D>(stage, dq_acc, dq_rsrc, static_cast<uint32_t>(wr0) * q_stride, q_stride, a.d_qk, lane);
+    } else {
         const uint32_t row_off = static_cast<uint32_t>(wr0 + ln) * q_stride;
 #pragma unroll
         for (int mt = 0; mt < MTILES; ++mt) {
@@ -877,7 +925,12 @@ __global__ __launch_bounds__(kDkvThreads, (D <= 128 ? 2 : 1)) void hstu_bwd_dkv_
     }
 
     // store dK or dV: lane holds key (cw0 + ln), dims 32*mt + 8*g + 4*lh + 0..3
-    {
+    if (a.grad_vec_ok != 0) {
+        __builtin_amdgcn_s_waitcnt(0);
+        __syncthreads();
+        uint16_t* const stage = wave == 0 ? s_st0 : (wave == 1 ? s_st1 : (wave == 2 ? s_st2 : s_st3));
+        store_tile_rows<Tag, D>(stage, acc, out_rsrc, static_cast<uint32_t>(cw0) * out_stride, out_stride, out_dim, lane);
+    } else {
         const uint32_t row_off = static_cast<uint32_t>(key) * out_stride;
 #pragma unroll
         for (int mt = 0; mt < MTILES; ++mt) {

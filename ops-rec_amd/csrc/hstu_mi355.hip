@@ -483,6 +483,10 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
     a.dk = p->grad_k;
     a.dv = p->grad_v;
     a.drab = p->grad_attn_bias;
+    a.grad_vec_ok = (f->head_dim_qk % 8 == 0 && f->head_dim_v % 8 == 0 && reinterpret_cast<uintptr_t>(p->grad_q) % 16 == 0 &&
+                     reinterpret_cast<uintptr_t>(p->grad_k) % 16 == 0 && reinterpret_cast<uintptr_t>(p->grad_v) % 16 == 0)
+                        ? 1
+                        : 0;
     a.offs_q = f->seq_offset_q;
     a.offs_k = f->seq_offset_k;
     a.num_ctx = f->num_context;

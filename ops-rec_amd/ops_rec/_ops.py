@@ -349,6 +349,11 @@ def hip_backward_available(q, k, v) -> bool:
             and v.shape[2] % 16 == 0)  # fmt: skip
 
 
+def _new_grad(like: torch.Tensor) -> torch.Tensor:
+    """Storage for one of dq / dk / dv (a function of its own so that a test can hand out other storage)."""
+    return torch.empty_like(like)
+
+
 def _backward_hip(grad, q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max_seq_len_k, silu_scale, seq_offset,
                   seq_offset_k, num_context, num_target, group, alpha):  # fmt: skip
     """The backward through the C ABI (``hstu_jagged_bwd``): two kernels on the current stream."""
@@ -372,7 +377,7 @@ def _backward_hip(grad, q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max_
         mask_c = mask.contiguous()
     # every row of dq / dk / dv is written by the kernels (rows past the last offset are zero-filled there); the
     # bias gradient is written only where a query tile sweeps
-    dq, dk, dv = torch.empty_like(q_c), torch.empty_like(k_c), torch.empty_like(v_c)
+    dq, dk, dv = _new_grad(q_c), _new_grad(k_c), _new_grad(v_c)
     dbias = torch.zeros_like(bias) if bias is not None else None
     if q_c.numel() == 0 and k_c.numel() == 0:
         return dq, dk, dv, dbias

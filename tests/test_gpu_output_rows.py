@@ -44,3 +44,32 @@ def test_misaligned_output_pointer_gives_the_same_bits(dtype, dim, heads):
     got = raw[guard : guard + n_bytes].view(dtype).view(want.shape)
     assert torch.equal(got, want)
     assert bool((raw[:guard] == 0x5A).all()) and bool((raw[guard + n_bytes :] == 0x5A).all())
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dim, heads, heads_k", [(64, 2, 2), (128, 4, 2), (256, 1, 1)])
+def test_misaligned_gradient_pointers_give_the_same_bits(monkeypatch, dtype, dim, heads, heads_k):
+    """dq / dk / dv rows are written 16 bytes per lane into 16-byte aligned tensors and in 8-byte pieces otherwise."""
+    w = workloads.make("grads", dtype=dtype, device=DEV, seed=22, batch=4, heads=heads, heads_k=heads_k, dim=dim, lo=1, hi=300)
+    g = torch.Generator(device=DEV).manual_seed(5)
+    grad = (torch.randn(w.q.shape[0], heads, dim, generator=g, device=DEV) * 0.1).to(dtype)
+    args = (grad, w.q, w.k, w.v, None, None, 0, w.max_seq_len, w.max_seq_len, w.silu_scale, w.seq_offset, w.seq_offset,
+            None, None, 1, w.alpha)  # fmt: skip
+    want = _ops._backward_hip(*args)[:3]
+    torch.cuda.synchronize()
+    assert all(t.data_ptr() % 16 == 0 for t in want)
+
+    def off_by_eight_bytes(like):
+        buf = torch.full((like.numel() + 16,), 7.0, dtype=like.dtype, device=like.device)
+        view = buf[4 : 4 + like.numel()].view(like.shape)
+        assert view.data_ptr() % 16 == 8
+        view._keep = buf  # noqa: SLF001  (the guard elements are checked below)
+        return view
+
+    monkeypatch.setattr(_ops, "_new_grad", off_by_eight_bytes)
+    got = _ops._backward_hip(*args)[:3]
+    torch.cuda.synchronize()
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+        buf = a._keep
+        assert bool((buf[:4] == 7.0).all()) and bool((buf[4 + a.numel() :] == 7.0).all())
