@@ -340,6 +340,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_bwd_dq_kernel(co
     const uint32_t bias_row_off =
         (wr0 + ln < sq) ? static_cast<uint32_t>(wr0 + ln) * static_cast<uint32_t>(a.max_k) * 2u : kOutOfRange;
     const bool vec = a.bias_vec_ok != 0;
+    const bool vec16 = a.bias_vec_ok == 2;  // rab / mask / d rab rows are 16-byte aligned
 
     // words 2g, 2g+1 = the row's values at keys c0 + 8g + 4 lh + 0..3 (accumulator order)
     auto load_words = [&](__amdgpu_buffer_rsrc_t rsrc, int c0, uint32_t (&w)[8]) {
@@ -476,20 +477,36 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_bwd_dq_kernel(co
             }
         }
         if constexpr (WANT_DRAB) {
+            if (vec16) {
+                // 16-byte aligned rows: the two lanes of a row trade halves (v_permlane32_swap), so that each holds 8
+                // consecutive keys and a store instruction writes whole 32-byte sectors of 32 rows instead of 16-byte
+                // pieces.  Lane (row, 0) ends up with keys 16 h2 + 0..7, lane (row, 1) with keys 16 h2 + 8..15.
+                typedef __attribute__((ext_vector_type(2))) unsigned u2_t;
 #pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const int key = c0 + 8 * g + 4 * lh;
-                const uint32_t off = bias_row_off + static_cast<uint32_t>(key) * 2u;
-                if (vec) {
-                    const u32x2_t w2 = {pk[2 * g], pk[2 * g + 1]};
-                    __builtin_amdgcn_raw_buffer_store_b64(w2, drab_rsrc, static_cast<int>(key < sk ? off : kOutOfRange), 0, 0);
-                } else {
+                for (int h2 = 0; h2 < 2; ++h2) {
+                    const u2_t r0 = __builtin_amdgcn_permlane32_swap(pk[4 * h2 + 0], pk[4 * h2 + 2], false, false);
+                    const u2_t r1 = __builtin_amdgcn_permlane32_swap(pk[4 * h2 + 1], pk[4 * h2 + 3], false, false);
+                    const u32x4_t w4 = {r0[0], r1[0], r0[1], r1[1]};
+                    const int key = c0 + 16 * h2 + 8 * lh;
+                    const uint32_t off = bias_row_off + static_cast<uint32_t>(key) * 2u;
+                    __builtin_amdgcn_raw_buffer_store_b128(w4, drab_rsrc, static_cast<int>(key < sk ? off : kOutOfRange), 0, 0);
+                }
+            } else {
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const uint32_t word = pk[2 * g + i / 2];
-                        const uint16_t val = static_cast<uint16_t>((i & 1) ? (word >> 16) : (word & 0xffffu));
-                        __builtin_amdgcn_raw_buffer_store_b16(val, drab_rsrc,
-                                                              static_cast<int>(key + i < sk ? off + 2u * i : kOutOfRange), 0, 0);
+                for (int g = 0; g < 4; ++g) {
+                    const int key = c0 + 8 * g + 4 * lh;
+                    const uint32_t off = bias_row_off + static_cast<uint32_t>(key) * 2u;
+                    if (vec) {
+                        const u32x2_t w2 = {pk[2 * g], pk[2 * g + 1]};
+                        __builtin_amdgcn_raw_buffer_store_b64(w2, drab_rsrc, static_cast<int>(key < sk ? off : kOutOfRange), 0, 0);
+                    } else {
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const uint32_t word = pk[2 * g + i / 2];
+                            const uint16_t val = static_cast<uint16_t>((i & 1) ? (word >> 16) : (word & 0xffffu));
+                            __builtin_amdgcn_raw_buffer_store_b16(val, drab_rsrc,
+                                                                  static_cast<int>(key + i < sk ? off + 2u * i : kOutOfRange), 0, 0);
+                        }
                     }
                 }
             }

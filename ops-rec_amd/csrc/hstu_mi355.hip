@@ -511,7 +511,7 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
                         ? 1
                         : 0;
     if (a.bias_vec_ok != 0 && reinterpret_cast<uintptr_t>(f->attn_bias) % 16 == 0 && reinterpret_cast<uintptr_t>(f->mask) % 16 == 0 &&
-        f->max_seq_len_k % 8 == 0) {
+        reinterpret_cast<uintptr_t>(p->grad_attn_bias) % 16 == 0 && f->max_seq_len_k % 8 == 0) {
         a.bias_vec_ok = 2;  // 16-byte aligned rows: the key-tile kernel reads rab / mask rows 16 bytes per lane
     }
     a.alpha = static_cast<float>(f->alpha);
