@@ -1633,9 +1633,9 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         // touching every 128-byte line of the tile; measured, these partial-line writes cost a 42 us launch 6 us.
         // So the wavefront passes its 32 rows through LDS (its own K slot of the ring, idle between two sweeps;
         // 16-byte chunks XOR-ed with the row so that neither side has bank conflicts to speak of) and writes them
-        // 16 bytes per lane, whole lines per instruction.
-        constexpr bool kStagedStore = !F8;  // (fp8 sub-tiles are half the size of the 16-bit output rows)
-        const bool staged = kStagedStore && a.out_vec_ok != 0;
+        // 16 bytes per lane, whole lines per instruction.  (fp8 sub-tiles are half the size of the 16-bit output
+        // rows: rows 0..15 go through the wavefront's K slot, rows 16..31 through its V slot.)
+        const bool staged = a.out_vec_ok != 0;
         if (staged) {
             // every wavefront's tile requests have landed (the last ones, past the end, move nothing, but they
             // name the slots) before anybody writes a slot
@@ -1643,8 +1643,9 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             __syncthreads();
         }
         if (store_rows && staged) {
-            if constexpr (kStagedStore) {
-                uint16_t* const stage = wave == 0 ? s_k0 : (wave == 1 ? s_k1 : (wave == 2 ? s_k2 : s_k3));
+            {
+                uint16_t* const stage_lo = wave == 0 ? s_k0 : (wave == 1 ? s_k1 : (wave == 2 ? s_k2 : s_k3));
+                uint16_t* const stage_hi = F8 ? (wave == 0 ? s_v0 : (wave == 1 ? s_v1 : (wave == 2 ? s_v2 : s_v3))) : stage_lo + 16 * D;
                 constexpr int OCPR = D / 8;  // 16-byte chunks per staged row
                 // the LDS offsets below depend on the lane only; opaque copies of the lane's coordinates keep the
                 // compiler from working them out once, ahead of the item loop, and carrying two dozen registers
@@ -1659,7 +1660,8 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                         w[0] = pack2<OutTag>(o_acc[mt][4 * g + 0] * c_out, o_acc[mt][4 * g + 1] * c_out);
                         w[1] = pack2<OutTag>(o_acc[mt][4 * g + 2] * c_out, o_acc[mt][4 * g + 3] * c_out);
                         const int chunk = (4 * mt + g) ^ (ln_e & (OCPR - 1));
-                        *reinterpret_cast<u32x2_t*>(stage + ln_e * D + chunk * 8 + 4 * lh_e) = w;
+                        uint16_t* const row_at = (ln_e < 16 ? stage_lo : stage_hi) + (ln_e & 15) * D;
+                        *reinterpret_cast<u32x2_t*>(row_at + chunk * 8 + 4 * lh_e) = w;
                     }
                 }
                 // (one wavefront: its LDS accesses execute in order; the fences keep the compiler from moving the reads up)
@@ -1672,8 +1674,9 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                 const int cc = lane_e % OCPR;
 #pragma unroll
                 for (int i = 0; i < 32 / RPI; ++i) {
-                    const int r = i * RPI + rr;
-                    const u32x4_t piece = *reinterpret_cast<const u32x4_t*>(stage + r * D + (cc ^ (r & (OCPR - 1))) * 8);
+                    const int r = i * RPI + rr;  // (the rows of one instruction lie in one half: RPI divides 16)
+                    const uint16_t* const row_at = (i * RPI < 16 ? stage_lo : stage_hi) + (((i * RPI) & 15) + rr) * D;
+                    const u32x4_t piece = *reinterpret_cast<const u32x4_t*>(row_at + (cc ^ (r & (OCPR - 1))) * 8);
                     const uint32_t off = (cc * 8 < a.d_v) ? static_cast<uint32_t>(wr0 + r) * o_stride + cc * 16u : kOutOfRange;
                     __builtin_amdgcn_raw_buffer_store_b128(piece, o_rsrc, static_cast<int>(off), 0, kNonTemporal);
                 }
