@@ -398,8 +398,8 @@ def main() -> int:
             "flops_per_step": bwd_flops,
             "tflops": round(bwd_flops / (bwd_ms * 1e-3) / 1e12, 3),
             "pct_of_bf16_mfma_peak": round(100.0 * bwd_flops / (bwd_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 2),
-            "note": "through torch.ops.ops_rec.hstu_jagged_backward: hstu_bwd_dkv_kernel + hstu_bwd_dq_kernel per step (plus a "
-            "zero-fill of the attn_bias gradient when there is one); the kernels recompute S and dP (eight products "
+            "note": "through torch.ops.ops_rec.hstu_jagged_backward: hstu_bwd_dkv_kernel + hstu_bwd_dq_kernel per step (the "
+            "first also clears the attn_bias gradient when there is one); the kernels recompute S and dP (eight products "
             "issued for the five of the formula)",
         }
 

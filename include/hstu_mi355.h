@@ -148,8 +148,9 @@ HSTU_API int hstu_jagged_fwd(const hstu_jagged_fwd_params* params, void* workspa
  * not used and may be NULL).  Built for bf16 / fp16 with head dims up to 256 (q/k head dim a multiple of 8);
  * other valid descriptions return HSTU_ERR_UNSUPPORTED.
  * grad_q / grad_k / grad_v: every row is written (rows past the last offset are zero-filled), so the caller
- * need not clear them.  grad_attn_bias (optional; requires attn_bias): only the elements inside a
- * sequence's [S_q, S_k] corner that a query tile sweeps are written -- the caller clears the tensor beforehand. */
+ * need not clear them.  grad_attn_bias (optional; requires attn_bias): written in full as well -- zeros outside
+ * the part of a sequence's [S_q, S_k] corner that its query tiles sweep -- so the caller need not clear it either
+ * (the kernel that produces grad_k / grad_v clears it beside its work). */
 typedef struct hstu_jagged_bwd_params {
     uint32_t struct_size; /* sizeof(hstu_jagged_bwd_params) */
     uint32_t reserved0;

@@ -73,6 +73,7 @@ struct BwdArgs {
     void* dk;
     void* dv;
     void* drab;  // may be null
+    int64_t drab_clear_bytes;  // > 0: the key-tile kernel clears this many bytes at drab beside its work
     const void* offs_q;
     const void* offs_k;
     const void* num_ctx;

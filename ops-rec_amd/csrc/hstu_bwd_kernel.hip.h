@@ -30,6 +30,7 @@
 // freedom from atomics and from a dQ workspace (8 with the S computed by both wavefronts of a key set).
 #pragma once
 #include "hstu_fwd_kernel.hip.h"
+#include "hstu_clear.hip.h"
 
 namespace hstu {
 
@@ -602,6 +603,11 @@ __global__ __launch_bounds__(kDkvThreads, (D <= 128 ? 2 : 1)) void hstu_bwd_dkv_
     const int hk = rem - b * a.n_heads_k;
     zero_tail_rows(a.dk, a.offs_k, a.n_batch, a.idx64, a.total_k, static_cast<int64_t>(a.n_heads_k) * a.d_qk, kDkvThreads);
     zero_tail_rows(a.dv, a.offs_k, a.n_batch, a.idx64, a.total_k, static_cast<int64_t>(a.n_heads_k) * a.d_v, kDkvThreads);
+    if (a.drab_clear_bytes > 0) {
+        // the attn_bias gradient is cleared here, by all workgroups alike (also those of absent tiles, which leave
+        // below), and written by the query-tile kernel that runs after this one
+        clear_share(a.drab, a.drab_clear_bytes, blockIdx.x, gridDim.x, tid, kDkvThreads);
+    }
     const SeqInfo si = load_seq(a, b);
     const int sq = si.sq, sk = si.sk;
     const int c0 = kt_idx * kBlockM;

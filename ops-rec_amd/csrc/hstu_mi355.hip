@@ -15,6 +15,7 @@
 #include <cstdio>
 #include <cstring>
 
+#include "hstu_clear.hip.h"
 #include "hstu_error.h"
 #include "hstu_variants.h"
 
@@ -251,6 +252,18 @@ uint64_t split_workspace_bytes(const Variant* var, const hstu_jagged_fwd_params*
 
 // ---- backward -------------------------------------------------------------------------------------------
 
+// clears the attn_bias gradient when the key-tile kernel, which does it beside its work, is not launched
+__global__ __launch_bounds__(256) void hstu_clear_kernel(void* p, int64_t n_bytes)
+{
+    hstu::clear_share(p, n_bytes, blockIdx.x, gridDim.x, static_cast<int>(threadIdx.x), 256);
+}
+void launch_clear(void* p, int64_t n_bytes, void* stream)
+{
+    const int64_t want = (n_bytes + 256 * 16 * 8 - 1) / (256 * 16 * 8);  // eight pieces per thread
+    const unsigned grid = static_cast<unsigned>(want < 1 ? 1 : (want > 4096 ? 4096 : want));
+    hipLaunchKernelGGL(hstu_clear_kernel, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream), p, n_bytes);
+}
+
 int validate_bwd(const hstu_jagged_bwd_params* p)
 {
     if (p == nullptr) {
@@ -468,7 +481,15 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
         return HSTU_ERR_UNSUPPORTED;
     }
     const hstu_jagged_fwd_params* f = &p->fwd;
+    // the attn_bias gradient is written in full: cleared by the key-tile kernel beside its work (or by a fill of
+    // its own when that kernel has nothing to run on), then written by the query-tile kernel where its tiles sweep
+    const int64_t drab_bytes = (p->grad_attn_bias != nullptr)
+                                   ? (f->n_offsets - 1) * f->num_heads_q * f->max_seq_len_q * f->max_seq_len_k * 2
+                                   : 0;
     if (f->total_q == 0 && f->total_k == 0) {
+        if (drab_bytes > 0) {
+            launch_clear(p->grad_attn_bias, drab_bytes, stream);
+        }
         return HSTU_OK;
     }
     hstu::BwdArgs a;
@@ -523,8 +544,11 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
         return fail(HSTU_ERR_INVALID, "grid out of range");
     }
     if (f->total_k > 0 && grid_kv > 0) {
+        a.drab_clear_bytes = drab_bytes;
         hipLaunchKernelGGL(var->dkv, dim3(static_cast<unsigned>(grid_kv)), dim3(hstu::kDkvThreads), 0,
                            static_cast<hipStream_t>(stream), a);
+    } else if (drab_bytes > 0) {
+        launch_clear(p->grad_attn_bias, drab_bytes, stream);
     }
     if (f->total_q > 0 && grid_q > 0) {
         hipLaunchKernelGGL(p->grad_attn_bias != nullptr ? var->dq_drab : var->dq, dim3(static_cast<unsigned>(grid_q)), dim3(256),

@@ -375,12 +375,12 @@ def _backward_hip(grad, q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max_
         _check(mask is not None and mask.dtype == q.dtype and tuple(mask.shape) == bias_shape,
                f"mask must be {bias_shape} of q's dtype")  # fmt: skip
         mask_c = mask.contiguous()
-    # every row of dq / dk / dv is written by the kernels (rows past the last offset are zero-filled there); the
-    # bias gradient is written only where a query tile sweeps
+    # every row of dq / dk / dv and every element of the bias gradient is written by the call (rows past the last
+    # offset and the bias gradient outside what the query tiles sweep are zero-filled there)
     dq, dk, dv = _new_grad(q_c), _new_grad(k_c), _new_grad(v_c)
-    dbias = torch.zeros_like(bias) if bias is not None else None
     if q_c.numel() == 0 and k_c.numel() == 0:
-        return dq, dk, dv, dbias
+        return dq, dk, dv, (torch.zeros_like(bias) if bias is not None else None)
+    dbias = _new_grad(bias) if bias is not None else None
     p = _native.new_bwd_params()
     f = p.fwd
     f.dtype = f.out_dtype = _DTYPE_CODE[q_c.dtype]

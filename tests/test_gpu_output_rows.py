@@ -73,3 +73,35 @@ def test_misaligned_gradient_pointers_give_the_same_bits(monkeypatch, dtype, dim
         assert torch.equal(a, b)
         buf = a._keep
         assert bool((buf[:4] == 7.0).all()) and bool((buf[4 + a.numel() :] == 7.0).all())
+
+
+@pytest.mark.parametrize("max_len", [203, 208])
+@pytest.mark.parametrize("shift", [0, 1, 4, 7])
+def test_bias_gradient_is_written_in_full(monkeypatch, shift, max_len):
+    """The call clears the attn_bias gradient itself (the key-tile kernel does it beside its work): a tensor full of
+    other values, at any 2-byte alignment, comes back equal to the gradient written into a cleared one, and the
+    memory around it is left alone."""
+    w = workloads.make("dbias", dtype=torch.bfloat16, device=DEV, seed=23, batch=3, heads=2, dim=64, lo=10, hi=200,
+                       max_seq_len=max_len, rab_std=0.3)  # fmt: skip
+    g = torch.Generator(device=DEV).manual_seed(6)
+    grad = (torch.randn(w.q.shape[0], 2, 64, generator=g, device=DEV) * 0.1).to(torch.bfloat16)
+    args = (grad, w.q, w.k, w.v, None, w.attn_bias, 0, w.max_seq_len, w.max_seq_len, w.silu_scale, w.seq_offset,
+            w.seq_offset, None, None, 1, w.alpha)  # fmt: skip
+    monkeypatch.setattr(_ops, "_new_grad", torch.zeros_like)
+    want = _ops._backward_hip(*args)
+    torch.cuda.synchronize()
+    assert float(want[3].float().abs().max()) > 0
+
+    def poisoned(like):
+        buf = torch.full((like.numel() + 32,), 7.0, dtype=like.dtype, device=like.device)
+        view = buf[8 + shift : 8 + shift + like.numel()].view(like.shape)
+        view._keep = buf  # noqa: SLF001
+        return view
+
+    monkeypatch.setattr(_ops, "_new_grad", poisoned)
+    got = _ops._backward_hip(*args)
+    torch.cuda.synchronize()
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+        buf = a._keep
+        assert bool((buf[: 8 + shift] == 7.0).all()) and bool((buf[8 + shift + a.numel() :] == 7.0).all())
