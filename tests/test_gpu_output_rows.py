@@ -105,3 +105,27 @@ def test_bias_gradient_is_written_in_full(monkeypatch, shift, max_len):
         assert torch.equal(a, b)
         buf = a._keep
         assert bool((buf[: 8 + shift] == 7.0).all()) and bool((buf[8 + shift + a.numel() :] == 7.0).all())
+
+
+@pytest.mark.parametrize("out_dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("dim", [64, 128, 256])
+def test_fp8_misaligned_output_pointer_gives_the_same_bits(out_dtype, dim):
+    """fp8 inputs: a sub-tile slot holds 16 of a wavefront's 32 output rows, so the rows pass through two slots."""
+    w = workloads.make("rows8", dtype=torch.bfloat16, device=DEV, seed=24, batch=4, heads=2, dim=dim, lo=1, hi=300)
+    (q8, qs), (k8, ks), (v8, vs) = (workloads.quantize_fp8(t) for t in (w.q, w.k, w.v))
+    p = _ops.prepare_forward(q8, k8, v8, None, None, 0, w.max_seq_len, w.max_seq_len, w.silu_scale, w.seq_offset,
+                             w.seq_offset, None, None, 1, w.alpha, out_dtype=out_dtype, q_descale=qs, k_descale=ks,
+                             v_descale=vs)  # fmt: skip
+    want = p.launch().clone()
+    torch.cuda.synchronize()
+    assert want.dtype == out_dtype and float(want.float().abs().max()) > 0
+    n_bytes = want.numel() * want.element_size()
+    guard = 256
+    for shift in (8, 0):
+        raw = torch.full((n_bytes + 2 * guard,), 0x5A, dtype=torch.uint8, device=DEV)
+        p.params.out = raw.data_ptr() + guard + shift
+        p.launch()
+        torch.cuda.synchronize()
+        got = raw[guard + shift : guard + shift + n_bytes].view(out_dtype).view(want.shape)
+        assert torch.equal(got, want)
+        assert bool((raw[: guard + shift] == 0x5A).all()) and bool((raw[guard + shift + n_bytes :] == 0x5A).all())
