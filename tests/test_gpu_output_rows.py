@@ -129,3 +129,23 @@ def test_fp8_misaligned_output_pointer_gives_the_same_bits(out_dtype, dim):
         got = raw[guard + shift : guard + shift + n_bytes].view(out_dtype).view(want.shape)
         assert torch.equal(got, want)
         assert bool((raw[: guard + shift] == 0x5A).all()) and bool((raw[guard + shift + n_bytes :] == 0x5A).all())
+
+
+def test_no_keys_at_all_still_clears_every_gradient(monkeypatch):
+    """Every sequence without keys: the key-tile kernel has nothing to run on, so the bias gradient is cleared by a
+    fill of its own; dq is all zeros."""
+    dt, heads, dim, max_q, max_k = torch.bfloat16, 2, 64, 40, 16
+    g = torch.Generator(device=DEV).manual_seed(7)
+    q = torch.randn(45, heads, dim, generator=g, device=DEV).to(dt)
+    k = torch.empty(0, heads, dim, device=DEV, dtype=dt)
+    v = torch.empty(0, heads, dim, device=DEV, dtype=dt)
+    offs_q = torch.tensor([0, 5, 45], dtype=torch.int32, device=DEV)
+    offs_k = torch.zeros(3, dtype=torch.int32, device=DEV)
+    bias = torch.randn(2, heads, max_q, max_k, generator=g, device=DEV).to(dt)
+    grad = torch.randn(45, heads, dim, generator=g, device=DEV).to(dt)
+    monkeypatch.setattr(_ops, "_new_grad", lambda like: torch.full_like(like, 7.0))
+    dq, dk, dv, dbias = _ops._backward_hip(grad, q, k, v, None, bias, 0, max_q, max_k, 1.0, offs_q, offs_k, None, None,
+                                           1, 0.125)  # fmt: skip
+    torch.cuda.synchronize()
+    assert dk.numel() == 0 and dv.numel() == 0
+    assert float(dq.float().abs().max()) == 0.0 and float(dbias.float().abs().max()) == 0.0
