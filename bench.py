@@ -45,7 +45,7 @@ PEAK_HBM_GBS = 8000.0  # MI355X HBM3E bandwidth (published)
 
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), scaled by the same
 # counters' reading of a plain copy kernel of known size; see profiles/.  None = not measured yet.
-MEASURED_TRAFFIC_BYTES = {"C2": 113_600_000, "C4": 1_575_000_000, "C5": 847_000_000}  # profiles/*counters*.md
+MEASURED_TRAFFIC_BYTES = {"C2": 113_600_000, "C4": 1_575_000_000, "C5": 811_000_000}  # profiles/*counters*.md
 
 
 def algorithmic_bytes(w, out_element_size: int) -> int:
