@@ -78,7 +78,10 @@ typedef struct hstu_jagged_fwd_params {
     const void* v;            /* [total_k, num_heads_k, head_dim_v] */
     const void* mask;         /* NULL or [batch, num_heads_q, max_seq_len_q, max_seq_len_k]; read iff mask_type == 3 */
     const void* attn_bias;    /* NULL or [batch, num_heads_q, max_seq_len_q, max_seq_len_k] */
-    const void* seq_offset_q; /* [n_offsets], non-decreasing, first element 0 */
+    const void* seq_offset_q; /* [n_offsets], non-decreasing, first element 0, no span longer than max_seq_len_q
+                                 (rows before the first offset, and rows of a sequence past max_seq_len_q, belong to
+                                 no work item: the kernels neither read nor write them, so `out` keeps whatever the
+                                 caller's buffer held there; the reference's adapter hands out zeros) */
     const void* seq_offset_k; /* [n_offsets]; may equal seq_offset_q */
     const void* num_context;  /* NULL (= zeros) or [n_offsets - 1] */
     const void* num_target;   /* NULL (= zeros) or [n_offsets - 1] */
@@ -178,14 +181,16 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* params, void* workspa
  * num_target[b] new target tokens, which are the LAST num_target[b] rows of its segment [seq_offset_q[b],
  * seq_offset_q[b+1]) of the k / v inputs (the other rows of k / v are not read).  fwd.seq_offset_k gives the
  * resulting key ranges (cached + targets per sequence) and fwd.total_k an upper bound on their end
- * (page_ids count x page_size + total_q is always enough); fwd.k / fwd.v are the inputs with total_q rows;
+ * (page_ids count x page_size + total_q is always enough); fwd.k / fwd.v MUST hold total_q rows each (the new rows
+ * are addressed by query row index, bounded by total_q only; the torch adapter checks the row counts);
  * fwd.num_context is ignored (zeros, as in the reference adapter); everything else as in the forward.
  * Implementation: for bf16 / fp16 with head dims up to 128 the forward kernel reads the pages itself (a page
  * look-up per 32-key sub-tile, page_size being a multiple of 32), and the workspace is only the optional room for
  * splitting long key ranges over workgroups, as in hstu_jagged_fwd.  Otherwise (fp32, larger head dims) the library
  * first gathers the rows into the workspace (one copy kernel: 2 x total_k rows, required) and runs the jagged
- * forward on them.  last_page_len and seq_offset_t are taken for signature parity; the number of cached rows of a
- * sequence is its key count minus its targets. */
+ * forward on them.  last_page_len and seq_offset_t are taken for signature parity and never read: the number of
+ * cached rows of a sequence is its key count minus its targets, so page metadata that disagrees with
+ * fwd.seq_offset_k / fwd.num_target is the caller's to keep consistent. */
 typedef struct hstu_paged_fwd_params {
     uint32_t struct_size; /* sizeof(hstu_paged_fwd_params) */
     uint32_t reserved0;

@@ -85,6 +85,16 @@ def _mask_check(mask_type: int, mask_defined: bool) -> None:
     _check(not (mask_type == 3 and not mask_defined), "use custome mask must have valide mask tensor")
 
 
+def _check_devices(device: torch.device, named) -> None:
+    """Every tensor argument must live on the GPU the call runs on.  The kernels read the offsets, counts and page
+    tables through raw device addresses: a host tensor among them (``seq_offset=torch.tensor([...])`` without
+    ``device=``) would hand the kernel a host pointer, which is a GPU memory fault, not a Python error.
+    (That q itself is a GPU tensor is checked where a launch is about to happen.)"""
+    for name, t in named:
+        if t is not None:
+            _check(t.device == device, f"{name} must be on the device of q ({device}), but it is on {t.device}")
+
+
 def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
     if t is None or t.numel() == 0:
         return None
@@ -113,6 +123,7 @@ class PreparedForward:
     def launch(self, stream: Optional[int] = None) -> torch.Tensor:
         if self.out.numel() == 0:
             return self.out
+        _check(self.device.type == "cuda", f"q must be a GPU tensor, but it is on {self.device}")
         lib = _native.load()
         if stream is None:
             stream = torch.cuda.current_stream(self.device).cuda_stream
@@ -165,6 +176,9 @@ def prepare_forward(
     _check(k.dim() == 3 and v.dim() == 3, "The k and v should be 3D in jagged layout")
     _check(q.dtype == k.dtype == v.dtype, "q, k, v must share one dtype")
     _check(q.dtype in _DTYPE_CODE, f"unsupported dtype {q.dtype}")
+    _check_devices(q.device, (("k", k), ("v", v), ("mask", mask), ("attn_bias", attn_bias), ("seq_offset", seq_offset),
+                              ("seq_offset_k", seq_offset_k), ("num_context", num_context), ("num_target", num_target),
+                              ("q_descale", q_descale), ("k_descale", k_descale), ("v_descale", v_descale)))  # fmt: skip
 
     idx_dtype = seq_offset.dtype
     offs_q = seq_offset.contiguous()
@@ -357,6 +371,10 @@ def _new_grad(like: torch.Tensor) -> torch.Tensor:
 def _backward_hip(grad, q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max_seq_len_k, silu_scale, seq_offset,
                   seq_offset_k, num_context, num_target, group, alpha):  # fmt: skip
     """The backward through the C ABI (``hstu_jagged_bwd``): two kernels on the current stream."""
+    _check(q.device.type == "cuda", f"q must be a GPU tensor, but it is on {q.device}")
+    _check_devices(q.device, (("grad", grad), ("k", k), ("v", v), ("mask", mask), ("attn_bias", attn_bias),
+                              ("seq_offset", seq_offset), ("seq_offset_k", seq_offset_k), ("num_context", num_context),
+                              ("num_target", num_target)))  # fmt: skip
     idx_dtype = seq_offset.dtype
     offs_q = seq_offset.contiguous()
     offs_k = offs_q if seq_offset_k is seq_offset else seq_offset_k.to(idx_dtype).contiguous()
@@ -427,6 +445,7 @@ def _backward_impl(grad, q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max
         _mask_check(int(mask_type), mask is not None)
         return _backward_hip(grad, q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max_seq_len_k, silu_scale,
                              seq_offset, seq_offset_k, num_context, num_target, group, a)  # fmt: skip
+    _check_devices(q.device, (("grad", grad), ("k", k), ("v", v), ("mask", mask), ("attn_bias", attn_bias)))
     scale = (1.0 / float(max_seq_len_q)) if float(silu_scale) == 0.0 else float(silu_scale)
     offs_q = seq_offset.tolist()
     offs_k = seq_offset_k.tolist()
@@ -551,6 +570,13 @@ def hstu_paged(q, k, v, kv_cache=None, mask=None, attn_bias=None, mask_type=0, m
         _check(t.dim() == 1 and t.size(0) >= 2, f"{name} params error should have at least two element.")
     _check(num_target is None or int(target_group_size) > 0,
            "targetGroupSize must be greater than 0 when numTarget is defined")  # fmt: skip
+    _check(k.dim() == 3 and v.dim() == 3, "The k and v should be 3D in jagged layout")
+    # the new key / value rows of a sequence are read at the row indices of its query segment
+    _check(k.size(0) == q.size(0) and v.size(0) == q.size(0),
+           f"k and v must hold one row per row of q ({q.size(0)}), but have {k.size(0)} and {v.size(0)}")  # fmt: skip
+    _check(q.device.type == "cuda", f"q must be a GPU tensor, but it is on {q.device}")
+    _check_devices(q.device, (("kv_cache", kv_cache), ("seq_offset_t", seq_offset_t), ("page_offsets", page_offsets),
+                              ("page_ids", page_ids), ("last_page_len", last_page_len)))  # fmt: skip
     _check(kv_cache.dim() == 5 and kv_cache.size(1) == 2, "kv_cache must be [num_pages, 2, page_size, heads, dim]")
     _check(kv_cache.dtype == q.dtype, "kv_cache must have the dtype of q")
     _check(kv_cache.size(3) == k.size(1) and kv_cache.size(4) == k.size(2) and v.size(2) == k.size(2),

@@ -1,35 +1,28 @@
-"""Autograd plug-ins: every module here that exposes ``register_autograd()`` is imported and
-registered when the package is imported; a failure in one module is logged and does not stop
-the others (ops_rec/autograd/__init__.py:26-48 in the reference)."""
+"""Attaches the autograd formula of the HSTU attention operators when the package is imported.
 
-import importlib
+This package carries exactly one plug-in, ``hstu_v1_autograd``; it is imported by name and its
+``register_autograd()`` is called once.  The reference walks its ``autograd`` directory and registers
+whatever module it finds there (ops_rec/autograd/__init__.py:26-48); the observable contract kept here is
+the same: importing ``ops_rec`` must not fail because a formula could not be attached (the forward
+operators stay usable, a message goes to the log), and ``__all__`` names the plug-ins that are active.
+"""
+
 import logging
-import pkgutil
 
-logger = logging.getLogger(__name__)
+_log = logging.getLogger(__name__)
 
 __all__: list = []
 
 
-def _register_modules() -> None:
-    for _, mod_name, is_pkg in pkgutil.iter_modules(__path__):
-        if is_pkg:
-            continue
-        try:
-            mod = importlib.import_module(f"{__name__}.{mod_name}")
-        except Exception as exc:  # noqa: BLE001
-            logger.warning("ops_rec.autograd: failed to import '%s': %s", mod_name, exc)
-            continue
-        fn = getattr(mod, "register_autograd", None)
-        if fn is None:
-            logger.warning("ops_rec.autograd: module '%s' has no register_autograd(), skipping", mod_name)
-            continue
-        try:
-            fn()
-        except Exception as exc:  # noqa: BLE001
-            logger.warning("ops_rec.autograd: register_autograd() in '%s' failed: %s", mod_name, exc)
-            continue
-        __all__.append(mod_name)
+def _attach(name: str) -> None:
+    """Import plug-in ``name`` of this package and run its ``register_autograd()``; log instead of raising."""
+    try:
+        module = __import__(f"{__name__}.{name}", fromlist=[name])
+        module.register_autograd()
+    except Exception as err:  # noqa: BLE001  (an import of ops_rec must survive a broken plug-in)
+        _log.warning("autograd formula '%s' is not active (%s: %s)", name, type(err).__name__, err)
+        return
+    __all__.append(name)
 
 
-_register_modules()
+_attach("hstu_v1_autograd")

@@ -120,6 +120,49 @@ def test_adapter_rejects_bad_arguments(over, msg):
         _ops.prepare_forward(**_cpu_args(**over))
 
 
+def test_tensors_on_another_device_are_rejected_before_any_pointer_is_taken():
+    # a host seq_offset next to device q / k / v is a common slip; its data_ptr() must never reach a kernel
+    dev = torch.device("cuda:0")  # (constructing the device object needs no GPU)
+    host = torch.tensor([0, 4, 10], dtype=torch.int32)
+    with pytest.raises(RuntimeError, match=r"seq_offset must be on the device of q \(cuda:0\), but it is on cpu"):
+        _ops._check_devices(dev, (("k", None), ("seq_offset", host)))
+    _ops._check_devices(torch.device("cpu"), (("seq_offset", host), ("mask", None)))  # same device: accepted
+    # through the adapter: q, k, v on the "meta" device stand in for device tensors, the offsets are host tensors
+    qm = torch.zeros(10, 4, 32, dtype=torch.bfloat16, device="meta")
+    for name in ("seq_offset", "num_target", "attn_bias"):
+        over = dict(q=qm, k=qm, v=qm)
+        if name == "num_target":
+            over.update(seq_offset=host.to("meta"), seq_offset_k=host.to("meta"), num_target=torch.zeros(2, dtype=torch.int32))
+        elif name == "attn_bias":
+            over.update(seq_offset=host.to("meta"), seq_offset_k=host.to("meta"), attn_bias=torch.zeros(2, 4, 6, 6, dtype=torch.bfloat16))
+        with pytest.raises(RuntimeError, match=f"{name} must be on the device of q"):
+            _ops.prepare_forward(**_cpu_args(**over))
+    # the backward and the paged adapter refuse host q outright, before they look at anything else
+    q = torch.zeros(10, 4, 32, dtype=torch.bfloat16)
+    with pytest.raises(RuntimeError, match="q must be a GPU tensor"):
+        _ops._backward_hip(q, q, q, q, None, None, 0, 6, 6, 0.0, host, host, None, None, 0, 1.0)
+    with pytest.raises(RuntimeError, match="q must be a GPU tensor"):
+        _ops.prepare_forward(**_cpu_args()).launch()
+
+
+def test_paged_adapter_checks_the_row_counts_of_k_and_v():
+    # the new key / value rows are addressed by query row index: k and v must have q's row count
+    # (checked before anything touches the device; the tensors here are on the "meta" device)
+    m = dict(device="meta")
+    q = torch.zeros(10, 4, 32, dtype=torch.bfloat16, **m)
+    short = torch.zeros(6, 4, 32, dtype=torch.bfloat16, **m)
+    offs = torch.zeros(3, dtype=torch.int32, **m)
+    cache = torch.zeros(4, 2, 32, 4, 32, dtype=torch.bfloat16, **m)
+    ids = torch.zeros(4, dtype=torch.int32, **m)
+    kw = dict(kv_cache=cache, max_seq_len=6, max_seq_len_k=70, seq_offset=offs, seq_offset_k=offs, seq_offset_t=offs,
+              page_offsets=offs, page_ids=ids, last_page_len=torch.zeros(2, dtype=torch.int32, **m),
+              num_target=torch.zeros(2, dtype=torch.int32, **m), target_group_size=1)  # fmt: skip
+    with pytest.raises(RuntimeError, match=r"one row per row of q \(10\), but have 6 and 6"):
+        _ops.hstu_paged(q, short, short, **kw)
+    with pytest.raises(RuntimeError, match="q must be a GPU tensor"):
+        _ops.hstu_paged(q, q, q, **kw)
+
+
 def test_empty_input_returns_empty_output_without_touching_the_library():
     q = torch.zeros(0, 4, 32, dtype=torch.bfloat16)
     p = _ops.prepare_forward(**_cpu_args(q=q, k=q, v=q, seq_offset=torch.tensor([0, 0], dtype=torch.int32),
