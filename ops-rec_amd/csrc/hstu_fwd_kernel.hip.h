@@ -327,6 +327,7 @@ constexpr int kMaxSplitItems = 2048;
 constexpr int kMaxParts = 8;
 static __device__ unsigned int g_split_arrived[kCounterSlots][kMaxSplitItems];
 
+constexpr int kInteriorMinSteps = 20;  // sweeps shorter than this take the general time step throughout
 constexpr int kMaxBatchSlots = 2048;  // sequences per call (the reference's limit)
 constexpr int kMaxLevels = 160;       // ceil(20480 / 128) query-tile levels
 
@@ -339,6 +340,18 @@ __device__ __forceinline__ int64_t load_index_uniform(const void* p, int64_t i, 
         return ((cptr64_t)(reinterpret_cast<uintptr_t>(p)))[i];
     }
     return static_cast<int64_t>(((cptr32_t)(reinterpret_cast<uintptr_t>(p)))[i]);
+}
+
+// floor(x / d) for 0 <= x < 2^23 and d >= 1, without the long integer-division sequence: the product with the
+// hardware reciprocal (accurate to one unit in the last place) is off by less than one, so the truncated
+// quotient is off by at most one either way.
+__device__ __forceinline__ int div_small(int x, int d)
+{
+    int q = static_cast<int>(static_cast<float>(x) * __builtin_amdgcn_rcpf(static_cast<float>(d)));
+    const int r = x - q * d;
+    q += (r >= d) ? 1 : 0;
+    q -= (r < 0) ? 1 : 0;
+    return q;
 }
 
 struct U32Pair {
@@ -469,21 +482,40 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         atomicAdd(&s_bucket[nt], 1u);
     }
     __syncthreads();
-    if (tid == 0) {
-        // bucket start in "most tiles first" order = number of sequences with more tiles
-        uint32_t run = 0;
-        for (int nt = n_levels; nt >= 0; --nt) {
-            const uint32_t c = s_bucket[nt];
-            s_bucket[nt] = run;
-            run += c;
+    // Bucket starts in "most tiles first" order: s_rank_start[nt] = number of sequences with more than nt tiles.
+    // Thread nt sums the counts above its own level by itself: its reads are independent, so they stream through
+    // the LDS back to back, where a prefix walk by one thread waits a full LDS round trip per level (with at most
+    // 161 levels the extra additions cost nothing).  In the same pass it gets the first item of list level l = nt
+    // of the plain list (one queue, by tile, nothing split): level l' holds the items of query tile
+    // n_levels - 1 - l', i.e. n_heads per sequence with more tiles than that, so the levels before l hold
+    // n_heads * sum over nt' of count[nt'] * max(0, nt' - (n_levels - l)) items.
+    static_assert(kMaxLevels + 2 <= kThreads, "one thread per level");
+    {
+        uint32_t above = 0;
+        uint32_t items_before = 0;
+        if (tid <= n_levels) {
+            const int floor_tiles = n_levels - tid;
+            for (int nt = n_levels; nt >= 1; --nt) {
+                const uint32_t c = s_bucket[nt];
+                above += nt > tid ? c : 0u;
+                items_before += nt > floor_tiles ? c * static_cast<uint32_t>(nt - floor_tiles) : 0u;
+            }
         }
-        for (int nt = 0; nt <= n_levels; ++nt) {
-            s_rank_start[nt] = s_bucket[nt];
+        __syncthreads();  // the counts have been read by everybody
+        if (tid <= n_levels) {
+            s_rank_start[tid] = above;
+            s_bucket[tid] = above;  // from here on: scatter cursors
+            if constexpr (!QUEUES && !SPLIT) {
+                s_queue_start[0][tid] = items_before * static_cast<uint32_t>(n_heads);
+            }
+        }
+        if constexpr (!QUEUES && !SPLIT) {
+            if (tid == 0) {
+                s_item[4] = 0u;  // by tile
+            }
         }
     }
-    if constexpr (QUEUES) {
-        __syncthreads();  // (without queues, thread 0 alone goes on to build the one table)
-    }
+    __syncthreads();
     // Work queues.  A "pair" is one (sequence, K/V head): its K / V rows are read by every query tile of every
     // query head that shares the K/V head.  Pairs are numbered p = sorted position * n_heads_k + kv head; pair p
     // belongs to queue p mod 8, and a queue is served first by the workgroups of one XCD, so that the rows of a
@@ -503,7 +535,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
     // at most 0.7 of the largest.
     // "By tile" runs as ONE queue shared by all workgroups (the order that matters there is global), "by pair" as
     // one queue per XCD.
-    if (tid < (QUEUES ? kQueues : 1)) {
+    if ((QUEUES || SPLIT) && tid < (QUEUES ? kQueues : 1)) {
         bool by_pair = false;
         if constexpr (QUEUES) {
             // total tiles = sum over nt of nt * (sequences with nt tiles); sequences with nt tiles =
@@ -618,26 +650,31 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
     // Stable scatter (sequences of one bucket stay in index order) by wavefront 0 alone: every workgroup
     // must arrive at the very same list, which an order-of-arrival scatter over four wavefronts would
     // not give.  64 sequences per trip; lanes holding the same tile count are ranked with a ballot.
+    // (the cursors of all 64 sequences of a trip are read in one go before the loop over the distinct tile counts
+    // among them, which then runs on ballots alone: no LDS round trip per distinct count)
     if (wave == 0) {
         for (int base = 0; base < a.n_batch; base += 64) {
             const int b = base + lane;
             const bool valid = b < a.n_batch;
             const int key = valid ? static_cast<int>(s_ntiles[valid ? b : 0]) : -1;
+            const uint32_t start = s_bucket[valid ? key : 0];
+            uint32_t before = 0;
             uint64_t todo = __builtin_amdgcn_ballot_w64(valid);
             while (todo != 0) {
                 const int leader = __builtin_ctzll(todo);
                 const int k0 = __builtin_amdgcn_readlane(key, leader);
                 const bool mine = valid && key == k0;
                 const uint64_t same = __builtin_amdgcn_ballot_w64(mine);
-                const uint32_t start = s_bucket[k0];
                 if (mine) {
-                    const uint32_t before = __builtin_popcountll(same & ((1ull << lane) - 1ull));
-                    s_order[start + before] = static_cast<uint16_t>(b);
+                    before = __builtin_popcountll(same & ((1ull << lane) - 1ull));
                 }
                 if (lane == leader) {
                     s_bucket[k0] = start + static_cast<uint32_t>(__builtin_popcountll(same));
                 }
                 todo &= ~same;
+            }
+            if (valid) {
+                s_order[start + before] = static_cast<uint16_t>(b);
             }
         }
     }
@@ -758,10 +795,13 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
     // around the ring), otherwise it leaves.  Every queue keeps the workgroups of its own XCD until it is empty,
     // so moving on only ever adds help.  One lane does this bookkeeping and the decoding of the item and hands
     // the result to the workgroup through LDS.
-    int fq_queue = 0;           // lane 0 only: the queue this workgroup pulls from
-    uint32_t fq_idx = 0;        //              the item index it holds in that queue
-    bool fq_first = true;       //              nothing pulled yet
-    auto fetch_item = [&]() {   // executed by thread 0
+    // (run by wavefront 0 as a whole, with uniform control flow: the levels of the list are searched by its lanes
+    // side by side, one ballot per 64 levels, where a walk by one thread waits an LDS round trip per level; the
+    // counters are touched by lane 0 alone)
+    int fq_queue = 0;           // the queue this workgroup pulls from
+    uint32_t fq_idx = 0;        // the item index it holds in that queue
+    bool fq_first = true;       // nothing pulled yet
+    auto fetch_item = [&]() {   // executed by wavefront 0
         const bool by_pair = QUEUES && s_item[4] != 0;
         const int nq = by_pair ? kQueues : 1;
         const int nq_shift = by_pair ? 3 : 0;
@@ -780,6 +820,23 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             }
             return qu;
         };
+        // pulls the next index of queue qu and, when `peek` names another queue, reads where that one stands
+        auto pull = [&](int qu, int peek, uint32_t& peeked) -> uint32_t {
+            uint32_t got = 0, seen = 0;
+            if (lane == 0) {
+                got = atomicAdd(&counters[qu * kCounterStride], 1u);
+                if (peek != qu) {
+                    seen = __hip_atomic_load(&counters[peek * kCounterStride], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+            peeked = static_cast<uint32_t>(uniform(static_cast<int>(seen)));
+            return static_cast<uint32_t>(uniform(static_cast<int>(got)));
+        };
+        auto no_item = [&]() {
+            if (lane == 0) {
+                s_item[0] = 0;
+            }
+        };
         uint32_t other_next = 0;  // where the next non-empty queue stands, as far as known
         bool other_known = false;
         if (fq_first) {
@@ -788,10 +845,10 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             fq_idx = blockIdx.x >> nq_shift;
         } else {
             const int other = next_queue(fq_queue);
-            const uint32_t got = atomicAdd(&counters[fq_queue * kCounterStride], 1u);
+            uint32_t seen = 0;
+            const uint32_t got = pull(fq_queue, other, seen);
             if (other != fq_queue) {
-                other_next = fixed_items(other) + __hip_atomic_load(&counters[other * kCounterStride], __ATOMIC_RELAXED,
-                                                                    __HIP_MEMORY_SCOPE_AGENT);
+                other_next = fixed_items(other) + seen;
                 other_known = true;
             }
             fq_idx = fixed_items(fq_queue) + got;
@@ -800,40 +857,45 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             // this queue is drained (or empty from the start): help the next one if it has work left
             const int other = next_queue(fq_queue);
             if (other == fq_queue) {
-                s_item[0] = 0;
+                no_item();
                 return;
             }
             if (!other_known) {
                 other_next = fixed_items(other);  // optimistic: nothing pulled there yet
             }
             if (other_next >= s_queue_start[other][n_levels]) {
-                s_item[0] = 0;
+                no_item();
                 return;
             }
             fq_queue = other;
             const int after = next_queue(other);
-            const uint32_t got = atomicAdd(&counters[other * kCounterStride], 1u);
+            uint32_t seen = 0;
+            const uint32_t got = pull(other, after, seen);
             other_known = after != other;
             if (other_known) {
-                other_next = fixed_items(after) + __hip_atomic_load(&counters[after * kCounterStride], __ATOMIC_RELAXED,
-                                                                    __HIP_MEMORY_SCOPE_AGENT);
+                other_next = fixed_items(after) + seen;
             }
             fq_idx = fixed_items(other) + got;
         }
+        // level of the item: the number of levels that end at or before it
         int lvl = 0;
-        while (fq_idx >= s_queue_start[fq_queue][lvl + 1]) {
-            ++lvl;
+        for (int base = 0; base < n_levels; base += 64) {
+            const int l = base + lane;
+            const bool ends_before = l < n_levels && s_queue_start[fq_queue][(l < n_levels ? l : 0) + 1] <= fq_idx;
+            lvl += __builtin_popcountll(__builtin_amdgcn_ballot_w64(ends_before));
         }
+        lvl = lvl < n_levels - 1 ? lvl : n_levels - 1;
         const int j_item = static_cast<int>(fq_idx - s_queue_start[fq_queue][lvl]);
         int qt, p_item, r_item;
+        uint32_t part_word = 0, split_counter = 0, split_buffer = 0;
         if (by_pair) {
             // item j of bucket lvl (pairs with nt tiles) = pair j / (nt * ratio) of this queue there, query tile
             // nt - 1 - (j % (nt * ratio)) / ratio, query head (kv head) * ratio + j % ratio
             const int nt_item = n_levels - lvl;
             const int per_pair = nt_item * ratio;
-            const int m_item = j_item / per_pair;
+            const int m_item = div_small(j_item, per_pair);
             const int rem_item = j_item - m_item * per_pair;
-            const int t_item = rem_item / ratio;
+            const int t_item = div_small(rem_item, ratio);
             qt = nt_item - 1 - t_item;
             r_item = rem_item - t_item * ratio;
             const int p_first = static_cast<int>(s_rank_start[nt_item]) * n_heads_k;
@@ -845,25 +907,33 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             if constexpr (SPLIT) {
                 // entry j of a split level = part j % m of item j / m
                 const int m = s_parts[lvl];
-                j_whole = j_item / m;
-                s_item[7] = static_cast<uint32_t>(j_item - j_whole * m) | (static_cast<uint32_t>(m) << 8);
-                s_item[8] = s_split_first[lvl] + static_cast<uint32_t>(j_whole);
-                s_item[9] = s_ws_first[lvl] + static_cast<uint32_t>(j_whole * m);
+                j_whole = div_small(j_item, m);
+                part_word = static_cast<uint32_t>(j_item - j_whole * m) | (static_cast<uint32_t>(m) << 8);
+                split_counter = s_split_first[lvl] + static_cast<uint32_t>(j_whole);
+                split_buffer = s_ws_first[lvl] + static_cast<uint32_t>(j_whole * m);
             }
-            p_item = j_whole / ratio;
+            p_item = div_small(j_whole, ratio);
             r_item = j_whole - p_item * ratio;
         }
-        const int rank = p_item / n_heads_k;
+        const int rank = div_small(p_item, n_heads_k);
         const int hk_item = p_item - rank * n_heads_k;
-        s_item[0] = 1;
-        s_item[1] = static_cast<uint32_t>(qt);
-        s_item[2] = static_cast<uint32_t>(s_order[rank]);
-        s_item[3] = static_cast<uint32_t>(hk_item * ratio + r_item);
-        s_item[5] = (static_cast<uint32_t>(fq_queue) << 28) | fq_idx;  // (for the development item log)
-        s_item[6] = static_cast<uint32_t>(hk_item);
+        const uint32_t seq_item = s_order[rank];
+        if (lane == 0) {
+            s_item[0] = 1;
+            s_item[1] = static_cast<uint32_t>(qt);
+            s_item[2] = seq_item;
+            s_item[3] = static_cast<uint32_t>(hk_item * ratio + r_item);
+            s_item[5] = (static_cast<uint32_t>(fq_queue) << 28) | fq_idx;  // (for the development item log)
+            s_item[6] = static_cast<uint32_t>(hk_item);
+            if constexpr (SPLIT) {
+                s_item[7] = part_word;
+                s_item[8] = split_counter;
+                s_item[9] = split_buffer;
+            }
+        }
     };
     for (;;) {
-        if (tid == 0) {
+        if (wave == 0) {
             fetch_item();
         }
         __syncthreads();
@@ -1275,9 +1345,14 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
 
         }
 
-        // one time step, for this wavefront; S = t mod 4
-        auto time_step = [&](auto sc, const int t) {
+        // one time step, for this wavefront; S = t mod 4.  INTERIOR (compile time) promises that sub-tiles t - 1, t
+        // and t + 1 all exist for this wavefront, that sub-tile t is fully visible and (with rab) that sub-tile t + 2
+        // exists: the step is then straight-line code -- no flags, no branches, a dozen scalar instructions.
+        // (Measured on MI355X: 3 - 6 % on sweeps of 32 steps and more; the general step spends about fifty scalar
+        // instructions and ten branches on its flags.)
+        auto time_step = [&](auto sc, auto interior, const int t) {
             constexpr int S = decltype(sc)::value;
+            constexpr bool INTERIOR = decltype(interior)::value;
             constexpr int PAR = S & 1;  // parity of t
             const f32x16_t& s_cur = PAR ? s_blk1 : s_blk0;  // S^T(t), transformed in this step
             f32x16_t& s_nxt = PAR ? s_blk0 : s_blk1;        // S^T(t+1), accumulated in this step
@@ -1291,20 +1366,20 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             const uint16_t* const vt = v_slot(std::integral_constant<int, (S + 3) & 3>{});  // V(t-1)
             const int c0 = t * 32;
 
-            const bool do_qk = t + 1 < nx_w;
-            const bool do_silu = t >= x_begin && t < nx_w;
-            const bool do_pv = t >= x_begin + 1 && t <= nx_w;
-            const bool full = (c0 + 32 <= lim_min) && !(any_hole && c0 + 32 > hist_k && c0 < hole_hi_max);
+            const bool do_qk = INTERIOR || t + 1 < nx_w;
+            const bool do_silu = INTERIOR || (t >= x_begin && t < nx_w);
+            const bool do_pv = INTERIOR || (t >= x_begin + 1 && t <= nx_w);
+            const bool full = INTERIOR || ((c0 + 32 <= lim_min) && !(any_hole && c0 + 32 > hist_k && c0 < hole_hi_max));
 
             // (1) bias / mask requests for later steps; they go out before the tile requests of this step so
             //     that waiting for them never waits for a younger tile
             if constexpr (HAS_RAB) {
-                if (t + 2 < nx_w) {
+                if (INTERIOR || t + 2 < nx_w) {
                     load_rab(c0 + 64, rab_far);
                 }
             }
             if constexpr (HAS_MASK) {
-                if (t + 1 < nx_w) {
+                if (do_qk) {
                     load_bias(mask_rsrc, c0 + 32, mw_nxt);
                 }
             }
@@ -1330,8 +1405,10 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                     return *reinterpret_cast<const u32x4_t*>(kt + k_lane_off[r]);
                 }
             };
+            // chunk c of the PV block = key half c % 2 of output tile c / 2: two consecutive MFMAs accumulate into the
+            // same registers
             auto read_v = [&](int c) -> u32x4_t {
-                const int j2 = c / MTILES, mt = c % MTILES;
+                const int j2 = c % 2, mt = c / 2;
                 if constexpr (F8) {
                     const u32x2_t t8 = lds_read_tr8_b64(reinterpret_cast<const uint8_t*>(vt) + v_lane_off[mt] + 16 * j2 * D);
                     const u32x4_t r = {t8[0], t8[1], 0u, 0u};
@@ -1405,7 +1482,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                 __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
                 for (int c = 0; c < NCH; ++c) {
-                    const int j2 = c / MTILES, mt = c % MTILES;
+                    const int j2 = c % 2, mt = c / 2;
                     if constexpr (F8) {
                         const u32x2_t va = {vop[c][0], vop[c][1]};
                         const u32x2_t pb = {pk_prev[2 * j2 + 0], pk_prev[2 * j2 + 1]};
@@ -1530,21 +1607,52 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         }
 #endif
         if (x_end > x_begin) {
+            // interior steps of this wavefront: [x_begin + 1, t_interior).  Sub-tile t + 1 (t + 2 with rab) must exist,
+            // and sub-tile t must be fully visible: it ends at or before the smallest row limit and, when target
+            // rows carve holes, before the first target key.  The wavefronts of a workgroup run different numbers
+            // of interior steps; every step of either kind ends in the same one barrier, so the counts match.
+            int t_interior = nx_w - (HAS_RAB ? 2 : 1);
+            {
+                int full_tiles = lim_min >> 5;
+                if (any_hole) {
+                    const int before_targets = hist_k > 0 ? hist_k >> 5 : 0;
+                    full_tiles = full_tiles < before_targets ? full_tiles : before_targets;
+                }
+                t_interior = t_interior < full_tiles ? t_interior : full_tiles;
+            }
+            // (short sweeps stay on the general step: measured on MI355X, sweeps under about twenty steps gain nothing
+            // from the second copy of the step and lose a little to fetching its instructions)
+            if (x_end - x_begin < kInteriorMinSteps) {
+                t_interior = -1;
+            }
+            typedef std::false_type general_t;
+            typedef std::true_type interior_t;
             int t = x_begin - 1;
             while (true) {
-                time_step(ic3_t{}, t);
+                time_step(ic3_t{}, general_t{}, t);
                 if (++t > x_end) {
                     break;
                 }
-                time_step(ic0_t{}, t);
+                time_step(ic0_t{}, general_t{}, t);
                 if (++t > x_end) {
                     break;
                 }
-                time_step(ic1_t{}, t);
+                // (t mod 4 == 1 and t >= x_begin + 1 here; at head dim 256 a step is 32 MFMAs long and the general
+                // step's overhead is small beside it, so that variant is not given the second copy)
+                if constexpr (D <= 128) {
+                    while (t + 4 <= t_interior) {
+                        time_step(ic1_t{}, interior_t{}, t);
+                        time_step(ic2_t{}, interior_t{}, t + 1);
+                        time_step(ic3_t{}, interior_t{}, t + 2);
+                        time_step(ic0_t{}, interior_t{}, t + 3);
+                        t += 4;
+                    }
+                }
+                time_step(ic1_t{}, general_t{}, t);
                 if (++t > x_end) {
                     break;
                 }
-                time_step(ic2_t{}, t);
+                time_step(ic2_t{}, general_t{}, t);
                 if (++t > x_end) {
                     break;
                 }
