@@ -447,6 +447,9 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
     __shared__ uint32_t s_queue_start[QUEUES ? kQueues : 1][kMaxLevels + 2];  // per queue: first item of each level / bucket
     __shared__ uint32_t s_item[12];  // [0..3]: the item handed to the workgroup (valid, query tile, sequence, head); [4]: queue order
                                      // [7]: part | parts << 8, [8]: arrival counter, [9]: first partial buffer, [10]: arrivals before
+    // plain list: the next item of the workgroup, decoded one item ahead ([parity][valid, query tile, sequence, head,
+    // K/V head, q0 lo/hi, q1 lo/hi, k0 lo/hi, k1 lo/hi, context count, target count])
+    __shared__ uint32_t s_next[(!QUEUES && !SPLIT) ? 2 : 1][16];
     __shared__ uint8_t s_parts[SPLIT ? kMaxLevels + 2 : 1];         // parts per item of each level
     __shared__ uint32_t s_split_first[SPLIT ? kMaxLevels + 2 : 1];  // first arrival counter of each split level
     __shared__ uint32_t s_ws_first[SPLIT ? kMaxLevels + 2 : 1];     // first partial buffer of each split level
@@ -932,18 +935,120 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             }
         }
     };
-    for (;;) {
+    // Plain list (one queue, by tile, nothing split): no counter at all.  The items of workgroup w are fixed by the
+    // list alone: in round r it takes item r * grid + w (r even) or r * grid + grid - 1 - w (r odd), so that the
+    // workgroups whose item of one round was heaviest get the lightest of the next -- what pulling from a counter
+    // gives such a short list as well (measured equal on MI355X), without the counter's round trip, without device
+    // state shared between launches, and with the next item known in advance: wavefront 0 decodes it, offsets
+    // included, while the tile requests of the current item are under way, and leaves it in LDS for the others.
+    constexpr bool kStaticList = !QUEUES && !SPLIT;
+    auto decode_ahead = [&](int round) {  // executed by wavefront 0; fills s_next[round & 1]
+        uint32_t(&rec)[16] = s_next[kStaticList ? (round & 1) : 0];
+        const uint32_t g = gridDim.x;
+        const uint32_t idx = static_cast<uint32_t>(round) * g + ((round & 1) ? g - 1u - blockIdx.x : blockIdx.x);
+        if (idx >= s_queue_start[0][n_levels]) {
+            if (lane == 0) {
+                rec[0] = 0;
+            }
+            return;
+        }
+        int lvl = 0;
+        for (int base = 0; base < n_levels; base += 64) {
+            const int l = base + lane;
+            const bool ends_before = l < n_levels && s_queue_start[0][(l < n_levels ? l : 0) + 1] <= idx;
+            lvl += __builtin_popcountll(__builtin_amdgcn_ballot_w64(ends_before));
+        }
+        lvl = lvl < n_levels - 1 ? lvl : n_levels - 1;
+        const int j_item = static_cast<int>(idx - s_queue_start[0][lvl]);
+        const int p_item = div_small(j_item, a.head_ratio);
+        const int r_item = j_item - p_item * a.head_ratio;
+        const int rank = div_small(p_item, a.n_heads_k);
+        const int hk_item = p_item - rank * a.n_heads_k;
+        const int seq = uniform(static_cast<int>(s_order[rank]));
+        const int64_t q0 = load_index_uniform(a.offs_q, seq, a.idx64);
+        const int64_t q1 = load_index_uniform(a.offs_q, seq + 1, a.idx64);
+        const int64_t k0 = load_index_uniform(a.offs_k, seq, a.idx64);
+        const int64_t k1 = load_index_uniform(a.offs_k, seq + 1, a.idx64);
+        int ctx = 0, tgt = 0;
+        if (a.mask_type == 0) {
+            if (a.num_ctx) {
+                ctx = static_cast<int>(load_index_uniform(a.num_ctx, seq, a.idx64));
+            }
+            if (a.num_tgt) {
+                tgt = static_cast<int>(load_index_uniform(a.num_tgt, seq, a.idx64));
+            }
+        }
+        if (lane == 0) {
+            rec[1] = static_cast<uint32_t>(n_levels - 1 - lvl);
+            rec[2] = static_cast<uint32_t>(seq);
+            rec[3] = static_cast<uint32_t>(hk_item * a.head_ratio + r_item);
+            rec[4] = static_cast<uint32_t>(hk_item);
+            rec[5] = static_cast<uint32_t>(q0);
+            rec[6] = static_cast<uint32_t>(static_cast<uint64_t>(q0) >> 32);
+            rec[7] = static_cast<uint32_t>(q1);
+            rec[8] = static_cast<uint32_t>(static_cast<uint64_t>(q1) >> 32);
+            rec[9] = static_cast<uint32_t>(k0);
+            rec[10] = static_cast<uint32_t>(static_cast<uint64_t>(k0) >> 32);
+            rec[11] = static_cast<uint32_t>(k1);
+            rec[12] = static_cast<uint32_t>(static_cast<uint64_t>(k1) >> 32);
+            rec[13] = static_cast<uint32_t>(ctx);
+            rec[14] = static_cast<uint32_t>(tgt);
+            rec[0] = 1;
+        }
+    };
+    int round = 0;
+    if constexpr (kStaticList) {
         if (wave == 0) {
-            fetch_item();
+            decode_ahead(0);
         }
         __syncthreads();
-        if (s_item[0] == 0) {
-            break;
+    }
+    for (;;) {
+        int qt, b, h, hk;
+        int64_t q0, q1, k0, k1;
+        int n_ctx = 0;
+        int n_tgt = 0;
+        if constexpr (kStaticList) {
+            const uint32_t(&rec)[16] = s_next[kStaticList ? (round & 1) : 0];
+            if (rec[0] == 0) {
+                break;
+            }
+            auto word = [&](int i) -> uint32_t { return static_cast<uint32_t>(uniform(static_cast<int>(rec[i]))); };
+            qt = static_cast<int>(word(1));
+            b = static_cast<int>(word(2));
+            h = static_cast<int>(word(3));
+            hk = static_cast<int>(word(4));
+            q0 = static_cast<int64_t>(word(5) | (static_cast<uint64_t>(word(6)) << 32));
+            q1 = static_cast<int64_t>(word(7) | (static_cast<uint64_t>(word(8)) << 32));
+            k0 = static_cast<int64_t>(word(9) | (static_cast<uint64_t>(word(10)) << 32));
+            k1 = static_cast<int64_t>(word(11) | (static_cast<uint64_t>(word(12)) << 32));
+            n_ctx = static_cast<int>(word(13));
+            n_tgt = static_cast<int>(word(14));
+        } else {
+            if (wave == 0) {
+                fetch_item();
+            }
+            __syncthreads();
+            if (s_item[0] == 0) {
+                break;
+            }
+            qt = uniform(static_cast<int>(s_item[1]));
+            b = uniform(static_cast<int>(s_item[2]));
+            h = uniform(static_cast<int>(s_item[3]));
+            hk = uniform(static_cast<int>(s_item[6]));
+            q0 = load_index_uniform(a.offs_q, b, a.idx64);
+            q1 = load_index_uniform(a.offs_q, b + 1, a.idx64);
+            k0 = load_index_uniform(a.offs_k, b, a.idx64);
+            k1 = load_index_uniform(a.offs_k, b + 1, a.idx64);
+            if (a.mask_type == 0) {
+                if (a.num_ctx) {
+                    n_ctx = static_cast<int>(load_index_uniform(a.num_ctx, b, a.idx64));
+                }
+                if (a.num_tgt) {
+                    n_tgt = static_cast<int>(load_index_uniform(a.num_tgt, b, a.idx64));
+                }
+            }
         }
-        const int qt = uniform(static_cast<int>(s_item[1]));
-        const int b = uniform(static_cast<int>(s_item[2]));
-        const int h = uniform(static_cast<int>(s_item[3]));
-        const int hk = uniform(static_cast<int>(s_item[6]));
 #ifdef HSTU_TIMELINE
         int log_slot = 0;
         if (a.timeline && lane == 0) {
@@ -956,10 +1061,6 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         }
 #endif
 
-        int64_t q0 = load_index_uniform(a.offs_q, b, a.idx64);
-        int64_t q1 = load_index_uniform(a.offs_q, b + 1, a.idx64);
-        int64_t k0 = load_index_uniform(a.offs_k, b, a.idx64);
-        int64_t k1 = load_index_uniform(a.offs_k, b + 1, a.idx64);
         // defensive clamps: malformed offsets must not turn into out-of-bounds addresses
         q1 = q1 < a.total_q ? q1 : a.total_q;
         k1 = k1 < a.total_k ? k1 : a.total_k;
@@ -974,15 +1075,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         const int wr0 = r0 + wave * kWaveM;
         const bool wave_active = wr0 < sq;  // inactive wavefronts still take part in loads and barriers
 
-        int n_ctx = 0;
-        int n_tgt = 0;
         if (a.mask_type == 0) {
-            if (a.num_ctx) {
-                n_ctx = static_cast<int>(load_index_uniform(a.num_ctx, b, a.idx64));
-            }
-            if (a.num_tgt) {
-                n_tgt = static_cast<int>(load_index_uniform(a.num_tgt, b, a.idx64));
-            }
             n_ctx = n_ctx < 0 ? 0 : n_ctx;
             n_tgt = n_tgt < 0 ? 0 : (n_tgt > sk ? sk : n_tgt);
         }
@@ -1164,6 +1257,13 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                 const int d0 = F8 ? 32 * js + 16 * lh : 16 * js + 8 * lh;
                 const uint32_t off = (d0 < a.d_qk) ? row_off + d0 * ES : kOutOfRange;
                 qf[js] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, static_cast<int>(off), 0, 0);
+            }
+        }
+
+        // the next item of this workgroup, while the requests of this one are under way
+        if constexpr (kStaticList) {
+            if (wave == 0) {
+                decode_ahead(round + 1);
             }
         }
 
@@ -1813,6 +1913,10 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
 #endif
 
         // (the barriers of the sweep separate this item's reads of s_item from the next fetch)
+        if constexpr (kStaticList) {
+            ++round;
+            __syncthreads();  // every wavefront has read its staged rows back before the next requests write the slots
+        }
     }
 
     // ---- rows past the last offset: zero-fill ----
@@ -1828,7 +1932,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
     }
 
     // ---- leave: the last workgroup out puts the counters of this slot back to zero ----
-    if (tid == 0) {
+    if (!kStaticList && tid == 0) {  // (the plain list has no counters)
         const unsigned int left = atomicAdd(&g_done_counter[a.counter_slot], 1u);
         if (left == gridDim.x - 1) {
             for (int qu = 0; qu < kQueues; ++qu) {
