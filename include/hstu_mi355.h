@@ -17,7 +17,7 @@
  * every buffer including the workspace, optional inputs are NULL, the launch is enqueued on the
  * caller's stream and returns before completion.  Differences: tensors are described by one
  * plain struct of device pointers and sizes instead of opaque handles, and there is no executor
- * object (the library keeps no per-call state).
+ * object (the library keeps no per-call state, on the host or on the device).
  *
  * The library never allocates or frees device memory and never synchronises the device.
  */
@@ -123,13 +123,18 @@ typedef struct hstu_jagged_fwd_params {
 
 /* replaces aclnnHstuJaggedForwardGetWorkspaceSize: validates the description and reports the scratch
  * size (may be 0).  No device work.
- * Scratch is asked for by calls whose work list may be shorter than the machine (few, long sequences): the
- * kernel then cuts the key range of long items into parts that run on different workgroups and adds their
- * fp32 partial outputs, in a fixed order, through the workspace (contents undefined before and after; 16-byte
- * aligned).  A caller that passes less than asked for, or nothing, gets the same results computed without
- * that split.  Because a split changes the order of the fp32 sums, the last bit of an output element may then
- * depend on what else is in the batch; HSTU_MI355_SPLIT=0 in the environment turns the split off (the size
- * reported is then 0). */
+ * Scratch is asked for by two kinds of calls.  A work list that may be several times longer than the machine
+ * (long, jagged batches) runs on per-XCD work queues and needs 16 KiB for their counters.  A work list that may be
+ * shorter than the machine (few, long sequences) cuts the key range of long items into parts that run on different
+ * workgroups and adds their fp32 partial outputs, in a fixed order: 16 KiB of counters plus room for one partial
+ * output per resident workgroup.  Lists in between run on a fixed schedule and need nothing.  The workspace is 16-byte
+ * aligned; its contents are undefined before and after the call (the library clears the counters on the launch
+ * stream ahead of its kernel) and it belongs to the call until the launch has completed: launches that overlap
+ * on a GPU -- several streams, captured graphs replayed side by side -- are independent of each other as long as
+ * each has a workspace (and an output) of its own.  The library keeps no device state between calls.
+ * A caller that passes less than asked for, or nothing, gets the same results from the fixed schedule.  Because a
+ * split changes the order of the fp32 sums, the last bit of an output element may then depend on what else is in
+ * the batch; HSTU_MI355_SPLIT=0 in the environment turns the split off. */
 HSTU_API int hstu_jagged_fwd_workspace_size(const hstu_jagged_fwd_params* params, uint64_t* workspace_bytes);
 
 /* replaces aclnnHstuJaggedForward: enqueues the forward on `stream` (a hipStream_t passed as void*;
@@ -185,8 +190,9 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* params, void* workspa
  * are addressed by query row index, bounded by total_q only; the torch adapter checks the row counts);
  * fwd.num_context is ignored (zeros, as in the reference adapter); everything else as in the forward.
  * Implementation: for bf16 / fp16 with head dims up to 128 the forward kernel reads the pages itself (a page
- * look-up per 32-key sub-tile, page_size being a multiple of 32), and the workspace is only the optional room for
- * splitting long key ranges over workgroups, as in hstu_jagged_fwd.  Otherwise (fp32, larger head dims) the library
+ * look-up per 32-key sub-tile, page_size being a multiple of 32); the workspace then holds 16 KiB of work counters
+ * (required: HSTU_ERR_WORKSPACE without them) and the optional room for splitting long key ranges over workgroups,
+ * as in hstu_jagged_fwd.  Otherwise (fp32, larger head dims) the library
  * first gathers the rows into the workspace (one copy kernel: 2 x total_k rows, required) and runs the jagged
  * forward on them.  last_page_len and seq_offset_t are taken for signature parity and never read: the number of
  * cached rows of a sequence is its key count minus its targets, so page metadata that disagrees with

@@ -6,7 +6,7 @@ namespace hstu {
 
 constexpr int kBlockM = 128;  // query rows per workgroup
 constexpr int kWaveM = 32;    // query rows per wavefront
-constexpr int kCounterSlots = 64;  // sets of device-side work counters (see the forward kernel)
+constexpr int kCounterBlockBytes = 16384;  // head of the workspace: device-side work counters (see the forward kernel)
 constexpr int kDkvThreads = 256;   // threads of a workgroup of the key-tile backward kernel
 constexpr int kGatherThreads = 128;
 
@@ -45,7 +45,7 @@ struct FwdArgs {
     const float* q_descale;  // fp8 inputs only; per head, nullptr = 1
     const float* k_descale;
     const float* v_descale;
-    int counter_slot;  // which pair of device-side work counters this launch uses
+    unsigned int* counters;  // kCounterBlockBytes at the head of the workspace, cleared ahead of the launch; null for the plain list
     float* ws;           // split variant: room for ws_parts partial outputs of kBlockM x D floats each (may be null)
     uint32_t ws_parts;
     // paged variant: the first (key count - num_target) key rows of a sequence live in pages of kv_cache

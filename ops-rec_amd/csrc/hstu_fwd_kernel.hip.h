@@ -312,20 +312,17 @@ __device__ __forceinline__ void load_to_lds_b128(__amdgpu_buffer_rsrc_t rsrc, ui
 }
 
 // ---- device-side work counters ---------------------------------------------------------------
-// One set of (work x kQueues, done) counters per slot; a launch is given a slot by the host (round
-// robin), so launches that overlap on one GPU do not share a set unless more than kCounterSlots of
-// them are in flight.  Zero at module load; the last workgroup of a launch to leave puts its set
-// back to zero.
+// The variants that pull items from counters (per-XCD queues, split items, paged keys) keep them in a block at the
+// head of the caller's workspace (FwdArgs::counters, kCounterBlockBytes): one work counter per queue, each in a
+// 128-byte line of its own, then one arrival counter per split item.  The host clears the block on the launch
+// stream ahead of every launch, so the library holds no device state of its own: launches that overlap on one
+// GPU, on streams or as replays of captured graphs, are independent as long as their workspaces are.
 constexpr int kQueues = 8;          // one work queue per XCD (MI355X: 8 XCDs; workgroup w runs on XCD w mod 8)
 constexpr int kCounterStride = 32;  // counters of different queues sit in different 128-byte lines
-static __device__ unsigned int g_work_counter[kCounterSlots][kQueues * kCounterStride];
-static __device__ unsigned int g_done_counter[kCounterSlots];
-
-// Split items (see "Splitting long items" in the kernel): one arrival counter per split item, same life cycle
-// as the work counters (zero at load; the workgroup that completes an item puts its counter back to zero).
 constexpr int kMaxSplitItems = 2048;
 constexpr int kMaxParts = 8;
-static __device__ unsigned int g_split_arrived[kCounterSlots][kMaxSplitItems];
+constexpr int kSplitCounterBase = kQueues * kCounterStride;  // first arrival counter, in 32-bit words
+static_assert((kSplitCounterBase + kMaxSplitItems) * 4 <= kCounterBlockBytes, "the counter block holds all counters");
 
 constexpr int kInteriorMinSteps = 20;  // sweeps shorter than this take the general time step throughout
 constexpr int kMaxBatchSlots = 2048;  // sequences per call (the reference's limit)
@@ -810,7 +807,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         const int nq_shift = by_pair ? 3 : 0;
         const int ratio = a.head_ratio;
         const int n_heads_k = a.n_heads_k;
-        unsigned int* const counters = &g_work_counter[a.counter_slot][0];
+        unsigned int* const counters = a.counters;
         auto fixed_items = [&](int qu) -> uint32_t {  // workgroups qu, qu + nq, ... took the first items of queue qu
             return gridDim.x > static_cast<uint32_t>(qu) ? (gridDim.x - qu + nq - 1) >> nq_shift : 0u;
         };
@@ -1795,16 +1792,13 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                 }
                 __builtin_amdgcn_s_waitcnt(0);
                 __syncthreads();  // every wavefront's stores have completed
-                unsigned int* const arrived = &g_split_arrived[a.counter_slot][s_item[8]];
+                unsigned int* const arrived = a.counters + kSplitCounterBase + s_item[8];
                 if (tid == 0) {
                     s_item[10] = __hip_atomic_fetch_add(arrived, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                 }
                 __syncthreads();
                 store_rows = s_item[10] == static_cast<uint32_t>(n_parts - 1);
                 if (store_rows) {
-                    if (tid == 0) {
-                        __hip_atomic_store(arrived, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    }
                     // the m partial outputs, added in part order whoever arrived last; the loads of one part
                     // are all in flight together
                     f32x4_t tot[kQuads];
@@ -1931,17 +1925,6 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         }
     }
 
-    // ---- leave: the last workgroup out puts the counters of this slot back to zero ----
-    if (!kStaticList && tid == 0) {  // (the plain list has no counters)
-        const unsigned int left = atomicAdd(&g_done_counter[a.counter_slot], 1u);
-        if (left == gridDim.x - 1) {
-            for (int qu = 0; qu < kQueues; ++qu) {
-                g_work_counter[a.counter_slot][qu * kCounterStride] = 0;
-            }
-            __threadfence();
-            g_done_counter[a.counter_slot] = 0;
-        }
-    }
     HSTU_STAMP(63);
 }
 

@@ -64,8 +64,6 @@ int compute_units(int* out)
     return HSTU_OK;
 }
 
-std::atomic<unsigned> g_next_counter_slot{0};
-
 
 int validate(const hstu_jagged_fwd_params* p, bool need_out = true)
 {
@@ -211,9 +209,12 @@ bool takes_queue_variant(const Variant* var, const hstu_jagged_fwd_params* p, in
 }
 
 // Split items: a list that cannot have two items per resident workgroup takes the variant that may cut long items
-// into parts (it does so when there are fewer items than workgroups), if the caller brings a workspace.  The workspace holds the fp32 partial outputs, kBlockM x d_pad
-// floats each; room for two per resident workgroup is asked for (the kernel splits only as far as the room goes).
+// into parts (it does so when there are fewer items than workgroups), if the caller brings a workspace.  Behind the
+// counter block the workspace holds the fp32 partial outputs, kBlockM x d_pad floats each; room for one per resident
+// workgroup is asked for: the kernel never lists more entries than there are workgroups when it splits, and splits
+// only as far as the room goes.
 constexpr uint64_t kMaxWorkspaceBytes = 128ull << 20;
+constexpr uint64_t kCounterBytes = hstu::kCounterBlockBytes;  // head of the workspace of the variants that pull from counters
 uint64_t split_part_bytes(const Variant* var) { return static_cast<uint64_t>(hstu::kBlockM) * var->d_pad * sizeof(float); }
 bool may_take_split_variant(const Variant* var, const hstu_jagged_fwd_params* p, int64_t* resident_out)
 {
@@ -246,8 +247,24 @@ uint64_t split_workspace_bytes(const Variant* var, const hstu_jagged_fwd_params*
     if (!may_take_split_variant(var, p, &resident)) {
         return 0;
     }
-    const uint64_t bytes = 2ull * static_cast<uint64_t>(resident) * split_part_bytes(var);
+    const uint64_t bytes = kCounterBytes + static_cast<uint64_t>(resident) * split_part_bytes(var);
     return bytes < kMaxWorkspaceBytes ? bytes : kMaxWorkspaceBytes;
+}
+
+// what a forward launch described by p asks of its caller: the counter block when the list may be long enough for
+// the variant with per-XCD queues, the counter block and room for partial outputs when it may be short enough to
+// split items, nothing for the lists in between (fixed schedule, no device counters)
+uint64_t forward_workspace_bytes(const Variant* var, const hstu_jagged_fwd_params* p)
+{
+    if (takes_queue_variant(var, p, nullptr)) {
+        return kCounterBytes;
+    }
+    return split_workspace_bytes(var, p);
+}
+
+bool usable_workspace(const void* workspace, uint64_t bytes, uint64_t need)
+{
+    return workspace != nullptr && bytes >= need && reinterpret_cast<uintptr_t>(workspace) % 16 == 0;
 }
 
 // ---- backward -------------------------------------------------------------------------------------------
@@ -383,8 +400,10 @@ HSTU_API int hstu_paged_fwd_workspace_size(const hstu_paged_fwd_params* params, 
         return HSTU_ERR_UNSUPPORTED;
     }
     if (var->kernel_paged != nullptr) {
-        // the kernel reads the pages itself; scratch only for splitting long items (optional, may be 0)
-        *workspace_bytes = split_workspace_bytes(var, &g);
+        // the kernel reads the pages itself; the counter block (required: the variant pulls its items from a
+        // counter) and, for short lists, room for the partial outputs of split items (optional)
+        const uint64_t split = split_workspace_bytes(var, &g);
+        *workspace_bytes = split > kCounterBytes ? split : kCounterBytes;
         return HSTU_OK;
     }
     uint64_t inner = 0;
@@ -412,6 +431,10 @@ HSTU_API int hstu_paged_fwd(const hstu_paged_fwd_params* p, void* workspace, uin
         return HSTU_ERR_UNSUPPORTED;
     }
     if (var->kernel_paged != nullptr) {
+        if (!usable_workspace(workspace, workspace_bytes, kCounterBytes)) {
+            return fail(HSTU_ERR_WORKSPACE, "the paged forward needs a 16-byte aligned workspace of at least %llu bytes",
+                        (unsigned long long)kCounterBytes);
+        }
         return launch_forward(&g, p, workspace, workspace_bytes, stream);
     }
     // no paged kernel for this combination (fp32, head dims above 128): gather the rows, then the plain forward
@@ -579,10 +602,11 @@ HSTU_API int hstu_jagged_fwd_workspace_size(const hstu_jagged_fwd_params* params
     if (v == nullptr) {
         return HSTU_ERR_UNSUPPORTED;
     }
-    // The tile schedule is derived inside the kernel from seq_offset.  Scratch is asked for only by short lists
-    // (room for the partial outputs of split items, see split_workspace_bytes); a caller that brings less, or
-    // none, is served without splitting.  Without a usable device the answer is 0.
-    *workspace_bytes = split_workspace_bytes(v, params);
+    // The tile schedule is derived inside the kernel from seq_offset.  Scratch is asked for by long lists (work
+    // counters of the per-XCD queues) and by short ones (counters and room for the partial outputs of split items,
+    // see split_workspace_bytes); a caller that brings less, or none, is served by the fixed schedule of the plain
+    // list.  Without a usable device the answer is 0.
+    *workspace_bytes = forward_workspace_bytes(v, params);
     return HSTU_OK;
 }
 
@@ -595,11 +619,11 @@ HSTU_API const char* hstu_jagged_fwd_kernel_name(const hstu_jagged_fwd_params* p
     if (v == nullptr) {
         return nullptr;
     }
-    // (without a usable device the plain name is reported)
+    // (given the workspace asked for; without a usable device the plain name is reported)
     if (takes_queue_variant(v, params, nullptr)) {
         return v->name_queues;
     }
-    return may_take_split_variant(v, params, nullptr) ? v->name_split : v->name;  // (given the workspace asked for)
+    return may_take_split_variant(v, params, nullptr) ? v->name_split : v->name;
 }
 
 }  // extern "C"
@@ -694,23 +718,30 @@ int launch_forward(const hstu_jagged_fwd_params* p, const hstu_paged_fwd_params*
             return rc_cu;
         }
         int64_t resident = static_cast<int64_t>(cus) * var->persistent_wgs_per_cu;
-        if (takes_queue_variant(var, p, &resident)) {
+        // the variants that pull items from counters need the counter block at the head of the workspace; without
+        // it every list runs on the plain variant's fixed schedule
+        const bool have_counters = usable_workspace(workspace, workspace_bytes, kCounterBytes);
+        if (have_counters && takes_queue_variant(var, p, &resident)) {
             kernel = var->kernel_queues;
+            a.counters = static_cast<unsigned int*>(workspace);
         }
         n_blocks = n_blocks < resident ? n_blocks : resident;
         const uint64_t part_bytes = split_part_bytes(var);
-        if (workspace != nullptr && workspace_bytes >= 2 * part_bytes && reinterpret_cast<uintptr_t>(workspace) % 16 == 0 &&
-            may_take_split_variant(var, p, nullptr)) {
+        if (usable_workspace(workspace, workspace_bytes, kCounterBytes + 2 * part_bytes) && may_take_split_variant(var, p, nullptr)) {
             kernel = var->kernel_split;
-            a.ws = static_cast<float*>(workspace);
-            const uint64_t parts = workspace_bytes / part_bytes;
+            a.counters = static_cast<unsigned int*>(workspace);
+            a.ws = reinterpret_cast<float*>(static_cast<char*>(workspace) + kCounterBytes);
+            const uint64_t parts = (workspace_bytes - kCounterBytes) / part_bytes;
             a.ws_parts = static_cast<uint32_t>(parts < 0x7fffffffull ? parts : 0x7fffffffull);
             n_blocks = resident;  // the list may have more entries than items: all resident workgroups take part
         }
         if (paged != nullptr) {
-            kernel = var->kernel_paged;  // (splits when it was given room above, otherwise not)
+            kernel = var->kernel_paged;  // (splits when it was given room above, otherwise not; the caller checked the block)
+            a.counters = static_cast<unsigned int*>(workspace);
         }
-        a.counter_slot = static_cast<int>(g_next_counter_slot.fetch_add(1) % hstu::kCounterSlots);
+        if (a.counters != nullptr) {
+            launch_clear(a.counters, static_cast<int64_t>(kCounterBytes), stream);
+        }
     }
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(n_blocks)), dim3(static_cast<unsigned>(var->threads)), 0,
                        static_cast<hipStream_t>(stream), a);

@@ -2,8 +2,8 @@
 forward that takes the split variant with its device-side counters) is replayed several times, with eager work and
 synchronisations of the program's own between the replays, and every replay is compared with the eager result bit for
 bit.  Nothing in these entry points allocates device memory behind torch's back or clears memory with a memset node:
-outputs and workspaces come from torch's allocator (its graph-private pool during capture), counters are put back by
-the kernels themselves."""
+outputs and workspaces come from torch's allocator (its graph-private pool during capture), and the counter block at
+the head of a workspace is cleared by a small kernel on the launch stream ahead of the forward."""
 
 import pytest
 import torch
@@ -70,8 +70,8 @@ def test_layer_chain_replays():
 
 
 def test_split_variant_replays():
-    # one long sequence: the forward cuts its items into parts, with arrival counters in device memory that the last
-    # part of an item puts back to zero -- which a replay must find as the capture left them
+    # one long sequence: the forward cuts its items into parts, with arrival counters at the head of its workspace
+    # that a fill kernel ahead of it clears -- at every replay as at the capture
     def make(seed):
         w = workloads.make("long", dtype=torch.bfloat16, device=DEV, seed=seed, batch=1, heads=2, dim=128, lo=3000, hi=3000)
         return w
