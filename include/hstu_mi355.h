@@ -141,6 +141,18 @@ HSTU_API int hstu_jagged_fwd_workspace_size(const hstu_jagged_fwd_params* params
  * NULL = the default stream) and returns without waiting for it. */
 HSTU_API int hstu_jagged_fwd(const hstu_jagged_fwd_params* params, void* workspace, uint64_t workspace_bytes, void* stream);
 
+/* hstu_jagged_fwd for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid it).  No counterpart in the reference.  Same results as hstu_jagged_fwd called with
+ * the workspace hstu_jagged_fwd_workspace_size reports, but the workspace is a device array of the library itself
+ * (32 MiB + 16 KiB per GPU, held from the first use of the library on that GPU until the process ends): the call
+ * takes inputs and outputs only and calls no hipMalloc, hipFree or other allocating routine.  A description whose
+ * workspace request exceeds that array (hstu_jagged_fwd_noalloc_max_workspace) is refused with HSTU_ERR_WORKSPACE
+ * and nothing is launched.  All calls on one GPU share the one array: two calls that overlap there (different
+ * streams, replays of two graphs side by side) race on it and are the caller's to serialise; calls that follow each
+ * other on a stream are safe, whatever their sizes (the counters are cleared ahead of every launch). */
+HSTU_API int hstu_jagged_fwd_noalloc(const hstu_jagged_fwd_params* params, void* stream);
+HSTU_API uint64_t hstu_jagged_fwd_noalloc_max_workspace(void);
+
 /* ---- backward ------------------------------------------------------------------------------------------
  * Replaces the two-phase pair the reference's adapter binds for the backward of this path:
  *

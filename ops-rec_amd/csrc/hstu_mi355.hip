@@ -9,11 +9,11 @@
 #include <hip/hip_runtime.h>
 #include <stdlib.h>
 
-#include <atomic>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 
 #include "hstu_clear.hip.h"
 #include "hstu_error.h"
@@ -22,6 +22,13 @@
 namespace {
 thread_local char g_err[512] = "";
 }
+
+// Scratch of the entry point that allocates nothing (hstu_jagged_fwd_noalloc): the workspace a caller of
+// hstu_jagged_fwd would bring -- the counter block and one fp32 partial output per resident workgroup of the split
+// variant (256 compute units: 512 x 64 KiB at head dim 128, 256 x 128 KiB at 256) -- as a device array of the
+// library.  Every GPU the library runs on holds its own copy, at its own address, until the process ends.
+constexpr uint64_t kScratchBytes = (32ull << 20) + hstu::kCounterBlockBytes;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 
 int hstu::set_error(int code, const char* fmt, ...)
 {
@@ -754,11 +761,72 @@ int launch_forward(const hstu_jagged_fwd_params* p, const hstu_paged_fwd_params*
 
 }  // namespace
 
+namespace {
+
+// device address of `scratch` on the current GPU, looked up once per device (with that device current); the array's
+// name is a host-side stand-in and never goes to a kernel itself
+int scratch_address(void** out)
+{
+    static void* address[64] = {nullptr};
+    static std::mutex guard;
+    int dev = 0;
+    hipError_t err = hipGetDevice(&dev);
+    if (err != hipSuccess) {
+        return fail(HSTU_ERR_RUNTIME, "hipGetDevice failed: %s", hipGetErrorString(err));
+    }
+    if (dev < 0 || dev >= 64) {
+        return fail(HSTU_ERR_RUNTIME, "device index %d is beyond the %d this library keeps scratch addresses for", dev, 64);
+    }
+    std::lock_guard<std::mutex> lock(guard);
+    if (address[dev] == nullptr) {
+        void* ptr = nullptr;
+        err = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (err != hipSuccess || ptr == nullptr) {
+            return fail(HSTU_ERR_RUNTIME, "cannot find the scratch array on device %d: %s", dev, hipGetErrorString(err));
+        }
+        address[dev] = ptr;
+    }
+    *out = address[dev];
+    return HSTU_OK;
+}
+
+}  // namespace
+
 extern "C" {
 
 HSTU_API int hstu_jagged_fwd(const hstu_jagged_fwd_params* p, void* workspace, uint64_t workspace_bytes, void* stream)
 {
     return launch_forward(p, nullptr, workspace, workspace_bytes, stream);
+}
+
+HSTU_API uint64_t hstu_jagged_fwd_noalloc_max_workspace(void) { return kScratchBytes; }
+
+HSTU_API int hstu_jagged_fwd_noalloc(const hstu_jagged_fwd_params* p, void* stream)
+{
+    const int rc = validate(p);
+    if (rc != HSTU_OK) {
+        return rc;
+    }
+    const Variant* var = select(p);
+    if (var == nullptr) {
+        return HSTU_ERR_UNSUPPORTED;
+    }
+    const uint64_t need = forward_workspace_bytes(var, p);
+    if (need > kScratchBytes) {
+        return fail(HSTU_ERR_WORKSPACE,
+                    "this call asks for %llu bytes of workspace, the built-in scratch of hstu_jagged_fwd_noalloc holds %llu: "
+                    "use hstu_jagged_fwd with a workspace of the caller's",
+                    (unsigned long long)need, (unsigned long long)kScratchBytes);
+    }
+    if (p->total_q == 0) {
+        return HSTU_OK;
+    }
+    void* ptr = nullptr;
+    const int rc_scratch = scratch_address(&ptr);
+    if (rc_scratch != HSTU_OK) {
+        return rc_scratch;
+    }
+    return launch_forward(p, nullptr, ptr, kScratchBytes, stream);
 }
 
 }  // extern "C"

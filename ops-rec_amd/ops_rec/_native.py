@@ -19,6 +19,8 @@ IDX_I32, IDX_I64 = 0, 1
 EXPORTED_SYMBOLS = (
     "hstu_jagged_fwd_workspace_size",
     "hstu_jagged_fwd",
+    "hstu_jagged_fwd_noalloc",
+    "hstu_jagged_fwd_noalloc_max_workspace",
     "hstu_last_error",
     "hstu_version",
     "hstu_jagged_fwd_kernel_name",
@@ -194,6 +196,10 @@ def load() -> ctypes.CDLL:
     lib.hstu_jagged_fwd_workspace_size.argtypes = [ctypes.POINTER(FwdParams), ctypes.POINTER(ctypes.c_uint64)]
     lib.hstu_jagged_fwd.restype = ctypes.c_int
     lib.hstu_jagged_fwd.argtypes = [ctypes.POINTER(FwdParams), ctypes.c_void_p, ctypes.c_uint64, ctypes.c_void_p]
+    lib.hstu_jagged_fwd_noalloc.restype = ctypes.c_int
+    lib.hstu_jagged_fwd_noalloc.argtypes = [ctypes.POINTER(FwdParams), ctypes.c_void_p]
+    lib.hstu_jagged_fwd_noalloc_max_workspace.restype = ctypes.c_uint64
+    lib.hstu_jagged_fwd_noalloc_max_workspace.argtypes = []
     lib.hstu_last_error.restype = ctypes.c_char_p
     lib.hstu_last_error.argtypes = []
     lib.hstu_version.restype = ctypes.c_int
