@@ -105,15 +105,18 @@ typedef struct hstu_jagged_fwd_params {
     double silu_scale; /* already resolved by the caller (0.0 is treated as 1 / max_seq_len_q here too) */
     double alpha;
     int32_t deterministic; /* accepted for signature parity; results are bitwise reproducible either way */
-    int32_t reserved0;
+    int32_t fp8_scaled_p;  /* fp8 inputs only.  1: P = e4m3(silu(X) * silu_scale * M), the reference's rounding point
+                              (op_kernel/atlas950/hstu_dense_forward_kernel_patten_bsnd.h:448-459; with the default
+                              silu_scale = 1 / max_seq_len most of P then falls below e4m3's range);
+                              0: P = e4m3(silu(X) * M), silu_scale applied to the fp32 output */
 
     /* fp8 inputs (dtype HSTU_DT_FP8_E4M3, OCP e4m3fn; the reference takes them on its 950 target,
      * op_host/atlas950/op_def_arch.h:23-24): S is kept in fp32, P is clamped to +-448 and re-quantised to
      * e4m3 (round to nearest even), P.V accumulates in fp32, the output is fp16 (the reference's choice,
-     * torch_extension/hstu_jagged_plugin.cpp:53-54) or bf16.  P is quantised BEFORE silu_scale is applied
-     * (the reference quantises silu(X) * silu_scale, which for the default 1 / max_seq_len falls below
-     * e4m3's normal range); with silu_scale = 1 the two coincide.  No attn_bias / custom mask; head_dim_qk
-     * must be a multiple of 16.
+     * torch_extension/hstu_jagged_plugin.cpp:53-54) or bf16.  attn_bias and a custom mask, when given, are e4m3
+     * tensors as well (they follow q's type, op_host/hstu_jagged_forward.cpp:65-66) and are used in fp32; such calls
+     * run on the fixed schedule (no per-XCD queues, no split items).  head_dim_qk must be a multiple of 16.  Where
+     * silu_scale is applied relative to the rounding of P is chosen by fp8_scaled_p above.
      * Extension with no counterpart in the reference (its fp8 path is unscaled): per-head dequantisation
      * scales, x = x8 * descale[head]; device pointers, NULL = 1.0.  Ignored unless dtype is fp8. */
     const float* q_descale; /* [num_heads_q] */

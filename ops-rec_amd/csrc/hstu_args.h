@@ -42,6 +42,7 @@ struct FwdArgs {
     float c_out;     // alpha * silu_scale
     float alpha;     // fp8 inputs only: the kernel folds the per-head scales in itself
     float silu_scale;
+    int fp8_scaled_p;        // fp8 inputs only: 1 = P is multiplied by silu_scale before it is quantised (reference), 0 = after
     const float* q_descale;  // fp8 inputs only; per head, nullptr = 1
     const float* k_descale;
     const float* v_descale;

@@ -408,7 +408,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
     constexpr int kThreads = 256;
     constexpr bool F8 = elem_traits<Tag>::kF8;
     constexpr uint32_t ES = elem_traits<Tag>::kBytes;  // bytes per input element
-    static_assert(!F8 || (!HAS_RAB && !HAS_MASK), "no rab / custom mask with fp8 inputs");
+    static_assert(!F8 || !(HAS_RAB || HAS_MASK) || !(QUEUES || SPLIT), "fp8 with rab / custom mask: plain list only");
     static_assert(!F8 || D >= 64, "fp8 rows are at least 64 bytes");
     static_assert(!(QUEUES && SPLIT), "one list policy per variant");
     static_assert(!PAGED || (SPLIT && !F8), "the paged variant builds on the split variant, 16-bit inputs");
@@ -736,6 +736,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
     float c_exp = a.c_exp;
     float c_out = a.c_out;
     float c_x = 1.0f;  // fp8 only: raw score -> alpha * (dequantised score)
+    float c_p = 1.0f;  // fp8 only: what P is multiplied by before it is quantised (1, or silu_scale)
     // rab is added to S^T by the matrix pipe: S^T += E_j . R_j (j = 0, 1), where R_j holds, per lane (query row,
     // half lh), the 8 consecutive rab values of keys 16 lh + 8 j .. + 7 exactly as they lie in memory (B operand)
     // and E_j is the constant 0/1 matrix that routes k-slot (lh, e) to key row 16 lh + 8 j + e (A operand).
@@ -1143,7 +1144,10 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             const float vs = a.v_descale ? ((cfloat_t)(reinterpret_cast<uintptr_t>(a.v_descale)))[hk] : 1.0f;
             c_x = a.alpha * qs * ks;
             c_exp = -1.4426950408889634f * c_x;
-            c_out = a.silu_scale * vs;
+            // where silu_scale is applied: to the fp32 output (P quantised at its own scale), or, the reference's
+            // rounding point, to P before it is quantised (fp8_scaled_p)
+            c_out = (a.fp8_scaled_p ? 1.0f : a.silu_scale) * vs;
+            c_p = a.fp8_scaled_p ? a.silu_scale : 1.0f;
         }
 
         // ---- keys needed by this item ----
@@ -1299,14 +1303,53 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         const int hole_hi_lane = hole_hi - 4 * lh;
 
         // ---- rab / custom mask: per (sequence, head) descriptor, rows indexed by the local (i, j) ----
-        const uint32_t bias_bytes = static_cast<uint32_t>(a.max_q) * static_cast<uint32_t>(a.max_k) * 2u;
+        const uint32_t bias_bytes = static_cast<uint32_t>(a.max_q) * static_cast<uint32_t>(a.max_k) * ES;
         const int64_t bias_plane =
             (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k);
         const __amdgpu_buffer_rsrc_t rab_rsrc =
-            make_rsrc(HAS_RAB ? static_cast<const uint16_t*>(a.rab) + bias_plane : nullptr, HAS_RAB ? bias_bytes : 0u);
+            make_rsrc(HAS_RAB ? static_cast<const uint8_t*>(a.rab) + bias_plane * ES : nullptr, HAS_RAB ? bias_bytes : 0u);
         const __amdgpu_buffer_rsrc_t mask_rsrc = make_rsrc(
-            HAS_MASK ? static_cast<const uint16_t*>(a.mask) + bias_plane : nullptr, HAS_MASK ? bias_bytes : 0u);
-        const uint32_t bias_row_off = static_cast<uint32_t>(wr0 + ln) * static_cast<uint32_t>(a.max_k) * 2u;
+            HAS_MASK ? static_cast<const uint8_t*>(a.mask) + bias_plane * ES : nullptr, HAS_MASK ? bias_bytes : 0u);
+        const uint32_t bias_row_off = static_cast<uint32_t>(wr0 + ln) * static_cast<uint32_t>(a.max_k) * ES;
+
+        // fp8 inputs: rab and the custom mask are e4m3 tensors like q.  The 16 values of a 32-key sub-tile a lane
+        // needs -- keys c0 + 8 g + 4 lh + 0..3 for g = 0..3, the order of its score registers -- are four words of
+        // four bytes (one 32-bit load each when rows are 4-byte aligned, byte loads otherwise); they are turned into
+        // floats on the vector ALU where they are used (the reference adds the bias and multiplies the mask in fp32 as
+        // well, op_kernel/atlas950/hstu_dense_forward_kernel_patten_bsnd.h:412-470).
+        auto load_bias_f8 = [&](__amdgpu_buffer_rsrc_t rsrc, int c0, uint32_t (&w)[8]) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const uint32_t off = bias_row_off + static_cast<uint32_t>(c0 + 8 * g + 4 * lh);
+                if (bias_mode != 0) {
+                    w[g] = __builtin_amdgcn_raw_buffer_load_b32(rsrc, static_cast<int>(off), 0, 0);
+                } else {
+                    uint32_t eoff = off;
+                    asm volatile("" : "+v"(eoff));
+                    uint32_t word = 0;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const uint32_t byte = __builtin_amdgcn_raw_buffer_load_b8(rsrc, static_cast<int>(eoff + e), 0, 0);
+                        word |= (byte & 0xffu) << (8 * e);
+                    }
+                    w[g] = word;
+                }
+            }
+        };
+        // element e (0..15, score register order) of such a block of words, as a float
+        auto f8_element = [&](const uint32_t (&w)[8], int e) -> float {
+            const uint32_t word = w[e / 4];
+            switch (e % 4) {
+            case 0:
+                return __builtin_amdgcn_cvt_f32_fp8(static_cast<int>(word), 0);
+            case 1:
+                return __builtin_amdgcn_cvt_f32_fp8(static_cast<int>(word), 1);
+            case 2:
+                return __builtin_amdgcn_cvt_f32_fp8(static_cast<int>(word), 2);
+            default:
+                return __builtin_amdgcn_cvt_f32_fp8(static_cast<int>(word), 3);
+            }
+        };
 
         // Requests the rab values of keys c0 + 16 lh .. + 15 of this lane's row, 8 packed words in memory order
         // (what the routing MFMAs above take as their B operands).
@@ -1435,11 +1478,10 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             mw0[i] = 0;
             mw1[i] = 0;
         }
-        if constexpr (HAS_RAB) {
+        if constexpr (HAS_RAB && !F8) {
             if (nx_w > x_begin) {
                 load_rab(x_begin * 32, rabw0);
             }
-
         }
 
         // one time step, for this wavefront; S = t mod 4.  INTERIOR (compile time) promises that sub-tiles t - 1, t
@@ -1470,14 +1512,23 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
 
             // (1) bias / mask requests for later steps; they go out before the tile requests of this step so
             //     that waiting for them never waits for a younger tile
-            if constexpr (HAS_RAB) {
+            if constexpr (HAS_RAB && !F8) {
                 if (INTERIOR || t + 2 < nx_w) {
                     load_rab(c0 + 64, rab_far);
                 }
             }
+            if constexpr (HAS_RAB && F8) {
+                if (do_qk) {
+                    load_bias_f8(rab_rsrc, c0 + 32, rab_nxt);  // used one step on, by the SiLU of sub-tile t + 1
+                }
+            }
             if constexpr (HAS_MASK) {
                 if (do_qk) {
-                    load_bias(mask_rsrc, c0 + 32, mw_nxt);
+                    if constexpr (F8) {
+                        load_bias_f8(mask_rsrc, c0 + 32, mw_nxt);
+                    } else {
+                        load_bias(mask_rsrc, c0 + 32, mw_nxt);
+                    }
                 }
             }
             // (2) tile requests of this time step
@@ -1521,6 +1572,30 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             // unmasked P^T pair i (score elements 2i, 2i+1)
             auto silu_pair = [&](int i) {
                 float tt[2], p[2];
+                if constexpr (F8 && HAS_RAB) {
+                    // the score at its real scale with the bias: x = alpha (qs ks S + rab); (rab_far is the block of the
+                    // parity of t: it was filled one step ago)
+                    float x[2];
+#pragma unroll
+                    for (int e = 0; e < 2; ++e) {
+                        x[e] = __builtin_fmaf(s_cur[2 * i + e], c_x, a.alpha * f8_element(rab_far, 2 * i + e));
+                        tt[e] = __builtin_amdgcn_exp2f(x[e] * -1.4426950408889634f);
+                    }
+#pragma unroll
+                    for (int e = 0; e < 2; ++e) {
+                        p[e] = x[e] * __builtin_amdgcn_rcpf(1.0f + tt[e]) * c_p;
+                    }
+                    if constexpr (HAS_MASK) {
+                        p[0] *= f8_element(mw_cur, 2 * i);
+                        p[1] *= f8_element(mw_cur, 2 * i + 1);
+                    }
+                    if (i & 1) {
+                        pk_cur[i / 2] = pack2_f8<true>(p[0], p[1], pk_cur[i / 2]);
+                    } else {
+                        pk_cur[i / 2] = pack2_f8<false>(p[0], p[1], pk_cur[i / 2]);
+                    }
+                    return;
+                }
 #pragma unroll
                 for (int e = 0; e < 2; ++e) {
                     tt[e] = s_cur[2 * i + e] * c_exp;
@@ -1542,15 +1617,22 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                     p[e] = s_cur[2 * i + e] * tt[e];
                 }
                 if constexpr (HAS_MASK) {
-                    p[0] *= lo_to_float<Tag>(mw_cur[i]);
-                    p[1] *= hi_to_float<Tag>(mw_cur[i]);
+                    if constexpr (F8) {
+                        p[0] *= f8_element(mw_cur, 2 * i);
+                        p[1] *= f8_element(mw_cur, 2 * i + 1);
+                    } else {
+                        p[0] *= lo_to_float<Tag>(mw_cur[i]);
+                        p[1] *= hi_to_float<Tag>(mw_cur[i]);
+                    }
                 }
                 if constexpr (F8) {
-                    // bring P^T to its real scale before it is quantised; pair i = bytes 2 (i % 2), +1 of word i / 2
+                    // bring P^T to its real scale (times silu_scale at the reference's rounding point) before it is
+                    // quantised; pair i = bytes 2 (i % 2), +1 of word i / 2
+                    const float c_q = c_x * c_p;
                     if (i & 1) {
-                        pk_cur[i / 2] = pack2_f8<true>(p[0] * c_x, p[1] * c_x, pk_cur[i / 2]);
+                        pk_cur[i / 2] = pack2_f8<true>(p[0] * c_q, p[1] * c_q, pk_cur[i / 2]);
                     } else {
-                        pk_cur[i / 2] = pack2_f8<false>(p[0] * c_x, p[1] * c_x, pk_cur[i / 2]);
+                        pk_cur[i / 2] = pack2_f8<false>(p[0] * c_q, p[1] * c_q, pk_cur[i / 2]);
                     }
                 } else {
                     pk_cur[i] = pack2<Tag>(p[0], p[1]);
@@ -1565,7 +1647,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             };
             constexpr int LOOKAHEAD = NCH >= 4 ? 2 : 1;
 
-            if constexpr (HAS_MASK) {
+            if constexpr (HAS_MASK && !F8) {
                 if (do_silu) {
                     order_bias(mw_cur);
                 }
@@ -1657,7 +1739,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                     silu_chunk(4, c);
                     __builtin_amdgcn_sched_barrier(0);
                 }
-                if constexpr (HAS_RAB) {
+                if constexpr (HAS_RAB && !F8) {
                     // S^T(t+1) += rab^T, last so that the rab request has had the whole block to land
                     const u32x4_t r0 = {rab_nxt[0], rab_nxt[1], rab_nxt[2], rab_nxt[3]};
                     const u32x4_t r1 = {rab_nxt[4], rab_nxt[5], rab_nxt[6], rab_nxt[7]};

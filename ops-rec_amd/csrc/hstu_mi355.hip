@@ -154,10 +154,6 @@ const Variant* select(const hstu_jagged_fwd_params* p)
             fail(HSTU_ERR_UNSUPPORTED, "fp8 inputs produce fp16 (the reference's choice) or bf16 output");
             return nullptr;
         }
-        if (p->attn_bias != nullptr || p->mask_type == HSTU_MASK_CUSTOM) {
-            fail(HSTU_ERR_UNSUPPORTED, "attn_bias and custom masks are not built for fp8 inputs");
-            return nullptr;
-        }
         if (p->head_dim_qk % 16 != 0) {
             fail(HSTU_ERR_UNSUPPORTED, "fp8 q/k head dim %lld is not a multiple of 16", (long long)p->head_dim_qk);
             return nullptr;
@@ -171,7 +167,7 @@ const Variant* select(const hstu_jagged_fwd_params* p)
     // address one sequence of one head group through a 32-bit buffer descriptor, with room above it for the offsets
     // that mark a request as out of range.  Whatever else the reference accepts (head dims up to 512, any q/k head
     // dim) goes to the kernel written for coverage.
-    const int64_t esize = p->dtype == HSTU_DT_FP32 ? 4 : 2;
+    const int64_t esize = p->dtype == HSTU_DT_FP32 ? 4 : (p->dtype == HSTU_DT_FP8_E4M3 ? 1 : 2);
     const int64_t span_q = p->max_seq_len_q * p->num_heads_q * dmax * esize;
     const int64_t span_k = p->max_seq_len_k * p->num_heads_k * dmax * esize;
     const int64_t span_b = p->max_seq_len_q * p->max_seq_len_k * esize;
@@ -186,7 +182,8 @@ const Variant* select(const hstu_jagged_fwd_params* p)
     }
     const int slot = dmax <= 32 ? 0 : (dmax <= 64 ? 1 : (dmax <= 128 ? 2 : 3));
     if (p->dtype == HSTU_DT_FP8_E4M3) {
-        return &hstu::fwd_variants_f8()[p->out_dtype == HSTU_DT_FP16 ? 0 : 1][slot <= 1 ? 0 : slot - 1];
+        return &hstu::fwd_variants_f8()[p->out_dtype == HSTU_DT_FP16 ? 0 : 1][p->attn_bias != nullptr ? 1 : 0]
+                                        [p->mask_type == HSTU_MASK_CUSTOM ? 1 : 0][slot <= 1 ? 0 : slot - 1];
     }
     if (p->dtype == HSTU_DT_FP32) {
         return &hstu::fwd_variants_f32()[p->attn_bias != nullptr ? 1 : 0][p->mask_type == HSTU_MASK_CUSTOM ? 1 : 0][slot];
@@ -680,12 +677,12 @@ int launch_forward(const hstu_jagged_fwd_params* p, const hstu_paged_fwd_params*
     a.idx64 = (p->index_dtype == HSTU_IDX_I64) ? 1 : 0;
     a.n_qtiles = (a.max_q + hstu::kBlockM - 1) / hstu::kBlockM;
     a.bh = a.n_batch * a.n_heads_q;
-    const uintptr_t vec_bytes = (p->dtype == HSTU_DT_FP32) ? 16 : 8;  // four elements
+    const uintptr_t vec_bytes = (p->dtype == HSTU_DT_FP32) ? 16 : (p->dtype == HSTU_DT_FP8_E4M3 ? 4 : 8);  // four elements
     const bool bias_aligned = (reinterpret_cast<uintptr_t>(p->attn_bias) % vec_bytes == 0) &&
                               (reinterpret_cast<uintptr_t>(p->mask) % vec_bytes == 0) && (p->max_seq_len_k % 4 == 0);
     a.bias_vec_ok = bias_aligned ? 1 : 0;
     a.out_vec_ok = (p->head_dim_v % 8 == 0 && reinterpret_cast<uintptr_t>(p->out) % 16 == 0) ? 1 : 0;
-    if (bias_aligned && p->dtype != HSTU_DT_FP32 && reinterpret_cast<uintptr_t>(p->attn_bias) % 16 == 0 &&
+    if (bias_aligned && (p->dtype == HSTU_DT_BF16 || p->dtype == HSTU_DT_FP16) && reinterpret_cast<uintptr_t>(p->attn_bias) % 16 == 0 &&
         reinterpret_cast<uintptr_t>(p->mask) % 16 == 0 && p->max_seq_len_k % 8 == 0) {
         a.bias_vec_ok = 2;  // 16-byte row alignment: the 16-bit kernels read rab / mask rows 32 bytes per lane
     }
@@ -694,6 +691,7 @@ int launch_forward(const hstu_jagged_fwd_params* p, const hstu_paged_fwd_params*
     a.c_out = static_cast<float>(p->alpha * scale);
     a.alpha = static_cast<float>(p->alpha);
     a.silu_scale = static_cast<float>(scale);
+    a.fp8_scaled_p = p->fp8_scaled_p != 0 ? 1 : 0;
     a.q_descale = p->q_descale;
     a.k_descale = p->k_descale;
     a.v_descale = p->v_descale;

@@ -32,8 +32,8 @@ struct BwdVariant {
 // forward, 16-bit inputs: [rab: 0, 1][custom mask: 0, 1][dim slot: 32, 64, 128, 256]
 const Variant (*fwd_variants_bf16())[2][4];
 const Variant (*fwd_variants_f16())[2][4];
-// forward, fp8-e4m3 inputs: [output: fp16, bf16][dim slot: 64, 128, 256] (no rab, no custom mask)
-const Variant (*fwd_variants_f8())[3];
+// forward, fp8-e4m3 inputs: [output: fp16, bf16][rab][custom mask][dim slot: 64, 128, 256]
+const Variant (*fwd_variants_f8())[2][2][3];
 // forward, fp32 inputs: [rab][custom mask][dim slot: 32, 64, 128, 256]
 const Variant (*fwd_variants_f32())[2][4];
 // forward, any head dims up to 512 (written for coverage, not speed): [bf16, fp16, fp32]

@@ -69,7 +69,7 @@ class FwdParams(ctypes.Structure):
         ("silu_scale", ctypes.c_double),
         ("alpha", ctypes.c_double),
         ("deterministic", ctypes.c_int32),
-        ("reserved0", ctypes.c_int32),
+        ("fp8_scaled_p", ctypes.c_int32),
         ("q_descale", ctypes.c_void_p),
         ("k_descale", ctypes.c_void_p),
         ("v_descale", ctypes.c_void_p),

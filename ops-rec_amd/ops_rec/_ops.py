@@ -160,12 +160,17 @@ def prepare_forward(
     q_descale: Optional[torch.Tensor] = None,
     k_descale: Optional[torch.Tensor] = None,
     v_descale: Optional[torch.Tensor] = None,
+    fp8_scaled_p: bool = True,
 ) -> PreparedForward:
     """Argument normalisation and checks of the reference adapter
     (torch_extension/hstu_jagged_plugin.cpp:22-67), ending in a filled parameter block.
 
     The keyword-only arguments belong to the fp8 extension (``hstu_jagged_fp8``): output type
-    (fp16 as in the reference, or bf16) and per-head fp32 dequantisation scales."""
+    (fp16 as in the reference, or bf16), per-head fp32 dequantisation scales, and the rounding point of P:
+    ``fp8_scaled_p=True`` is the reference's, ``P = e4m3(silu(X) * silu_scale * M)``
+    (hstu_forward_v1/test/pytest/test_hstu_jagged.py:183-195), and what a call through the reference's own
+    entry point with e4m3 tensors gets; ``False`` quantises ``silu(X) * M`` and applies ``silu_scale`` to the
+    fp32 output."""
     _check(q.dim() == 3, "The q should be 3D in jagged layout")
     _check(seq_offset is not None and seq_offset_k is not None, "seq_offset is required")
     _check(seq_offset.dim() == 1 and seq_offset.size(0) >= 2,
@@ -256,6 +261,7 @@ def prepare_forward(
     p.silu_scale = real_scale
     p.alpha = real_alpha
     p.deterministic = 1 if deterministic else 0
+    p.fp8_scaled_p = 1 if (is_fp8 and fp8_scaled_p) else 0
     p.q_descale, p.k_descale, p.v_descale = (_ptr(t) for t in scales)
 
     ws_bytes = ctypes.c_uint64(0)
@@ -277,21 +283,23 @@ def _forward_impl(q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max_seq_le
         return prepared.launch()
 
 
-def hstu_jagged_fp8(q, k, v, q_descale=None, k_descale=None, v_descale=None, *, mask_type=0, max_seq_len=0,
-                    max_seq_len_k=None, silu_scale=0.0, seq_offset=None, seq_offset_k=None, num_context=None,
-                    num_target=None, target_group_size=0, alpha=1.0, out_dtype=torch.bfloat16):  # fmt: skip
+def hstu_jagged_fp8(q, k, v, q_descale=None, k_descale=None, v_descale=None, *, mask=None, attn_bias=None, mask_type=0,
+                    max_seq_len=0, max_seq_len_k=None, silu_scale=0.0, seq_offset=None, seq_offset_k=None,
+                    num_context=None, num_target=None, target_group_size=0, alpha=1.0, out_dtype=torch.bfloat16):  # fmt: skip
     """Forward on fp8-e4m3 (``torch.float8_e4m3fn``) Q / K / V with per-head fp32 dequantisation scales.
 
-    An extension: the reference's fp8 path (``hstu_jagged`` called with e4m3 tensors, which this
-    package serves too) has no scales and a half output.  Here ``x = x8 * descale[head]`` for each of
-    q, k, v (``None`` = 1), P is re-quantised to e4m3 before ``silu_scale`` is applied, and the
-    output is ``out_dtype`` (bf16 or fp16).  No attn_bias, no custom mask."""
+    An extension: the reference's fp8 path (``hstu_jagged`` called with e4m3 tensors, which this package serves
+    too, rounding point and all) has no scales and a half output.  Here ``x = x8 * descale[head]`` for each of
+    q, k, v (``None`` = 1), P is re-quantised to e4m3 BEFORE ``silu_scale`` is applied (the reference's order puts
+    ``silu(X) / max_seq_len`` below e4m3's range), and the output is ``out_dtype`` (bf16 or fp16).  ``attn_bias``
+    and a custom ``mask`` are e4m3 tensors like q."""
     _check(q.dtype == torch.float8_e4m3fn, "hstu_jagged_fp8 takes float8_e4m3fn tensors")
     offs_k = seq_offset if seq_offset_k is None else seq_offset_k
     max_k = max_seq_len if max_seq_len_k is None else max_seq_len_k
-    prepared = prepare_forward(q, k, v, None, None, mask_type, max_seq_len, max_k, silu_scale, seq_offset, offs_k,
+    prepared = prepare_forward(q, k, v, mask, attn_bias, mask_type, max_seq_len, max_k, silu_scale, seq_offset, offs_k,
                                num_context, num_target, target_group_size, alpha, False, out_dtype=out_dtype,
-                               q_descale=q_descale, k_descale=k_descale, v_descale=v_descale)  # fmt: skip
+                               q_descale=q_descale, k_descale=k_descale, v_descale=v_descale,
+                               fp8_scaled_p=False)  # fmt: skip
     with torch.cuda.device(prepared.device):
         return prepared.launch()
 

@@ -306,10 +306,15 @@ def hstu_jagged_forward_fp8(
     v_descale: Optional[torch.Tensor],
     *,
     quantize_p: bool = True,
+    scaled_p: bool = False,
     out_dtype: torch.dtype = torch.float16,
     **kwargs,
 ) -> torch.Tensor:
-    """fp8 forward as this build defines it, on CPU in fp32.
+    """fp8 forward, on CPU in fp32.  ``scaled_p=True`` is the reference's definition,
+    ``P = e4m3(silu(X) * silu_scale * M)`` (hstu_forward_v1/test/pytest/test_hstu_jagged.py:183-195: the golden
+    multiplies by silu_scale and the mask, then casts to float8_e4m3fn and back); ``scaled_p=False`` is this
+    build's own variant described below.  attn_bias and a custom mask, when given, are e4m3 tensors used as fp32
+    values (they follow q's type in the reference, op_host/hstu_jagged_forward.cpp:65-66).
 
     The reference's fp8 path takes raw e4m3 Q / K / V, keeps S in fp32, re-quantises P to e4m3
     (round to nearest) and accumulates P.V in fp32 into a half output
@@ -334,16 +339,17 @@ def hstu_jagged_forward_fp8(
     kf = k8.float() * ks[None, :, None]
     scale = resolve_silu_scale(kwargs.get("silu_scale", 0.0), kwargs["max_seq_len"])
     kw = dict(kwargs)
-    kw["silu_scale"] = 1.0  # P is formed (and rounded) unscaled
-    if kw.get("attn_bias") is not None or kw.get("mask_type", 0) == MASK_CUSTOM:
-        raise ValueError("the fp8 path takes no attn_bias / custom mask")
+    kw["silu_scale"] = scale if scaled_p else 1.0  # own variant: P is formed (and rounded) unscaled
+    for name in ("attn_bias", "mask"):
+        if kw.get(name) is not None:
+            kw[name] = kw[name].float()
     # V enters unscaled so that P (e4m3) x V (e4m3) is what is accumulated; its scale goes on the output
     out = hstu_jagged_forward(
         qf, kf, v8.float(), compute_dtype=torch.float32,
         emulate_lowp=None, out_dtype=torch.float32, _p_hook=(quantize_e4m3 if quantize_p else None), **kw,
     )  # fmt: skip
     ratio = n_q // n_k
-    out = out * (scale * vs.repeat_interleave(ratio))[None, :, None]
+    out = out * ((1.0 if scaled_p else scale) * vs.repeat_interleave(ratio))[None, :, None]
     return out.to(out_dtype)
 
 

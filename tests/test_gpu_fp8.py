@@ -65,7 +65,7 @@ def test_fp8_forward_matrix(batch, heads, heads_k, d, dv, lo, hi, ctx, tgt, grou
 
 def test_reference_entry_point_with_e4m3_tensors_gives_half_output():
     # the reference's fp8 call: raw e4m3 tensors through hstu_jagged, no scales, fp16 out
-    # (torch_extension/hstu_jagged_plugin.cpp:53-54); silu_scale 1 makes the two rounding points coincide
+    # (torch_extension/hstu_jagged_plugin.cpp:53-54); with silu_scale 1 the rounding point makes no difference
     w, x8, _ = make_case(3, 2, 2, 128, 128, 10, 200, seed=11, scales=False, std=1.0)
     out = ops_rec.ascendc.attention.hstu_jagged(*(dev(t) for t in x8), None, None, 0, w.max_seq_len, 1.0,
                                                 dev(w.seq_offset), None, None, 0, 128**-0.5)  # fmt: skip
@@ -105,9 +105,61 @@ def test_fp8_rejections():
         ops_rec.hstu_jagged_fp8(*a, dev(sc[0])[:1], None, None, max_seq_len=w.max_seq_len, seq_offset=dev(w.seq_offset))
     with pytest.raises(RuntimeError, match="fp16 or bf16"):
         ops_rec.hstu_jagged_fp8(*a, max_seq_len=w.max_seq_len, seq_offset=dev(w.seq_offset), out_dtype=torch.float32)
-    bias = torch.zeros(2, 2, w.max_seq_len, w.max_seq_len, dtype=torch.float8_e4m3fn, device=DEV)
-    with pytest.raises(RuntimeError, match="not built for fp8"):
+    bias = torch.zeros(2, 2, w.max_seq_len, w.max_seq_len, dtype=torch.float16, device=DEV)
+    with pytest.raises(RuntimeError, match="attn_bias must have the dtype of q"):
         ops_rec.ascendc.attention.hstu_jagged(*a, None, bias, 0, w.max_seq_len, 1.0, dev(w.seq_offset))
+
+
+def e4m3(t):
+    return t.to(torch.float8_e4m3fn)
+
+
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("enable_bias,mask_type", [(True, 0), (True, 2), (False, 3), (True, 3)])
+@pytest.mark.parametrize("batch,heads,heads_k,d,dv,max_len", [
+    (3, 4, 4, 128, 128, 300), (3, 4, 2, 64, 64, 257), (2, 2, 1, 256, 256, 200), (4, 2, 2, 128, 64, 131),
+])  # fmt: skip
+def test_fp8_with_attn_bias_and_custom_mask(batch, heads, heads_k, d, dv, max_len, enable_bias, mask_type, out_dtype):
+    # attn_bias and the custom mask follow q's type in the reference (e4m3 on its fp8 target,
+    # op_host/hstu_jagged_forward.cpp:65-66; bias and MaskType.CUSTOM are part of its fp8 test matrix, disabled there);
+    # max_len 257 and 131 give rows that are not 4-byte aligned (the byte-load path)
+    w, x8, sc = make_case(batch, heads, heads_k, d, dv, max_len // 3, max_len, seed=batch * 31 + max_len)
+    g = torch.Generator().manual_seed(max_len)
+    shape = (batch, heads, w.max_seq_len, w.max_seq_len)
+    bias = e4m3(torch.randn(shape, generator=g) * 0.5) if enable_bias else None
+    mask = e4m3((torch.rand(shape, generator=g) < 0.7).float()) if mask_type == 3 else None
+    kw = dict(mask=mask, attn_bias=bias, mask_type=mask_type, max_seq_len=w.max_seq_len, silu_scale=0.0,
+              seq_offset=w.seq_offset, alpha=d**-0.5)  # fmt: skip
+    kwd = dict(kw, mask=dev(mask), attn_bias=dev(bias), seq_offset=dev(w.seq_offset))
+    out = ops_rec.hstu_jagged_fp8(*(dev(t) for t in x8), *(dev(t) for t in sc), out_dtype=out_dtype, **kwd)
+    assert out.dtype == out_dtype
+    check(out, x8, sc, kw)
+
+
+@pytest.mark.parametrize("silu_scale", [0.0, 0.25])
+def test_reference_entry_point_keeps_the_reference_rounding_point(silu_scale):
+    # through hstu_jagged with raw e4m3 tensors P is quantised AFTER silu_scale and the mask, as the reference's golden
+    # does (test_hstu_jagged.py:183-195); with the default silu_scale = 1 / max_seq_len most of P falls below e4m3's
+    # smallest subnormal and rounds to zero there as well
+    w, x8, _ = make_case(3, 2, 2, 128, 128, 40, 200, seed=23, scales=False, std=1.0)
+    bias = e4m3(torch.randn(3, 2, w.max_seq_len, w.max_seq_len, generator=torch.Generator().manual_seed(2)) * 0.5)
+    out = ops_rec.ascendc.attention.hstu_jagged(*(dev(t) for t in x8), None, dev(bias), 0, w.max_seq_len, silu_scale,
+                                                dev(w.seq_offset), None, None, 0, 128**-0.5)  # fmt: skip
+    assert out.dtype == torch.float16
+    kw = dict(attn_bias=bias, mask_type=0, max_seq_len=w.max_seq_len, silu_scale=silu_scale, seq_offset=w.seq_offset,
+              alpha=128**-0.5)  # fmt: skip
+    want = O.hstu_jagged_forward_fp8(*x8, None, None, None, scaled_p=True, out_dtype=torch.float32, **kw)
+    other = O.hstu_jagged_forward_fp8(*x8, None, None, None, scaled_p=False, out_dtype=torch.float32, **kw)
+    got = out.float().cpu()
+    peak = want.abs().max().item()
+    assert peak > 0
+    # elements of P on a rounding boundary may fall the other way in the kernel (hardware exp2 / rcp): by fraction of
+    # outliers plus a bound on the largest, as in the test above
+    assert O.mismatch_fraction(got, want, 2e-3 * peak + 1e-3) < 5e-3, (peak, (got - want).abs().max().item())
+    assert (got - want).abs().max() <= 0.06 * peak + 1e-3
+    if silu_scale == 0.0:
+        # ... and it is not this build's own variant, which keeps the information the reference's order rounds away
+        assert (other - want).abs().max() > 10 * (got - want).abs().max()
 
 
 @pytest.fixture(scope="module")

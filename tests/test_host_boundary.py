@@ -324,10 +324,11 @@ def test_fp8_variant_selection_and_limits():
     assert name(out_dtype=_native.DT_BF16) == "hstu_fwd_f8e4m3_bf16_d128"
     assert name(head_dim_qk=32, head_dim_v=48).endswith("_d64")  # fp8 rows are padded to at least 64 bytes
     assert name(head_dim_qk=256, head_dim_v=256).endswith("_d256")
+    # attn_bias / custom mask in e4m3, as the reference's OpDef allows (op_host/hstu_jagged_forward.cpp:65-66)
+    assert name(attn_bias=0x2000) == "hstu_fwd_f8e4m3_f16_d128_rabtrue_maskfalse"
+    assert name(mask=0x2000, mask_type=3, out_dtype=_native.DT_BF16) == "hstu_fwd_f8e4m3_bf16_d128_rabfalse_masktrue"
     for kw, text in [
         (dict(out_dtype=_native.DT_FP32), "fp16 .* or bf16"),
-        (dict(attn_bias=0x2000), "not built for fp8"),
-        (dict(mask=0x2000, mask_type=3), "not built for fp8"),
         (dict(head_dim_qk=24, head_dim_v=16), "multiple of 16"),
         (dict(head_dim_qk=512, head_dim_v=512), "head dims up to 256"),
     ]:

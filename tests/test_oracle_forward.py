@@ -265,7 +265,31 @@ def test_fp8_reduces_to_the_reference_definition_without_scales_and_silu_scale_o
     assert torch.equal(got, want)
 
 
-def test_fp8_rejects_bias_and_custom_mask():
-    (q8, k8, v8), (qs, ks, vs), kw = _fp8_case()
-    with pytest.raises(ValueError):
-        O.hstu_jagged_forward_fp8(q8, k8, v8, qs, ks, vs, **dict(kw, mask_type=3, mask=torch.ones(4, 4, 40, 40)))
+def test_fp8_reference_rounding_point_is_the_reference_golden_on_one_sequence():
+    # scaled_p=True against the lines of the reference's own fp8 golden, written out with library calls for one
+    # sequence (hstu_forward_v1/test/pytest/test_hstu_jagged.py:160-198): qk + bias, * alpha, silu, * silu_scale,
+    # * mask, cast to float8_e4m3fn and back, matmul with V; GQA by repeating the K/V heads
+    import torch.nn.functional as F
+
+    g = torch.Generator().manual_seed(9)
+    s_len, heads, heads_k, d = 37, 4, 2, 32
+    q8, k8, v8 = (torch.randn(s_len, n, d, generator=g).to(torch.float8_e4m3fn) for n in (heads, heads_k, heads_k))
+    bias = (torch.randn(1, heads, s_len, s_len, generator=g) * 0.5).to(torch.float8_e4m3fn)
+    mask = (torch.rand(1, heads, s_len, s_len, generator=g) < 0.6).float().to(torch.float8_e4m3fn)
+    offs = torch.tensor([0, s_len], dtype=torch.int32)
+    for silu_scale in (1.0, 0.25, 1.0 / s_len):
+        qk = torch.einsum("nhd,mhd->hnm", q8.float(), k8.float().repeat_interleave(heads // heads_k, dim=1))
+        p = F.silu((qk + bias[0].float()) * 0.3) * silu_scale * mask[0].float()
+        p = p.to(torch.float8_e4m3fn).float()
+        want = torch.einsum("hnm,mhd->nhd", p, v8.float().repeat_interleave(heads // heads_k, dim=1))
+        got = O.hstu_jagged_forward_fp8(q8, k8, v8, None, None, None, scaled_p=True, out_dtype=torch.float32, mask=mask,
+                                        attn_bias=bias, mask_type=3, max_seq_len=s_len, silu_scale=silu_scale,
+                                        seq_offset=offs, alpha=0.3)  # fmt: skip
+        torch.testing.assert_close(got, want, atol=1e-5, rtol=1e-5)
+        own = O.hstu_jagged_forward_fp8(q8, k8, v8, None, None, None, scaled_p=False, out_dtype=torch.float32, mask=mask,
+                                        attn_bias=bias, mask_type=3, max_seq_len=s_len, silu_scale=silu_scale,
+                                        seq_offset=offs, alpha=0.3)  # fmt: skip
+        if silu_scale == 1.0:
+            torch.testing.assert_close(own, want, atol=1e-5, rtol=1e-5)  # the two rounding points coincide
+        else:
+            assert not torch.allclose(own, want, atol=1e-4, rtol=1e-3)
