@@ -160,7 +160,7 @@ def prepare_forward(
     q_descale: Optional[torch.Tensor] = None,
     k_descale: Optional[torch.Tensor] = None,
     v_descale: Optional[torch.Tensor] = None,
-    fp8_scaled_p: bool = True,
+    fp8_scaled_p: bool = False,
 ) -> PreparedForward:
     """Argument normalisation and checks of the reference adapter
     (torch_extension/hstu_jagged_plugin.cpp:22-67), ending in a filled parameter block.
@@ -219,8 +219,9 @@ def prepare_forward(
         mask_c = mask.contiguous()
 
     is_fp8 = q_c.dtype == torch.float8_e4m3fn
-    _check(is_fp8 or (out_dtype is None and q_descale is None and k_descale is None and v_descale is None),
-           "out_dtype and descales are only taken with fp8 inputs")  # fmt: skip
+    _check(is_fp8 or (out_dtype is None and q_descale is None and k_descale is None and v_descale is None
+                      and not fp8_scaled_p),
+           "out_dtype, descales and fp8_scaled_p are only taken with fp8 inputs")  # fmt: skip
     if out_dtype is None:
         out_dtype = _out_dtype(q_c)
     _check(not is_fp8 or out_dtype in (torch.float16, torch.bfloat16), "fp8 inputs produce fp16 or bf16 output")
@@ -276,9 +277,10 @@ def prepare_forward(
 
 def _forward_impl(q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max_seq_len_k, silu_scale, seq_offset,
                   seq_offset_k, num_context, num_target, target_group_size, alpha, deterministic=False):  # fmt: skip
+    # (e4m3 tensors through the reference's entry point: the reference's rounding point of P)
     prepared = prepare_forward(q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max_seq_len_k, silu_scale,
                                seq_offset, seq_offset_k, num_context, num_target, target_group_size, alpha,
-                               deterministic)  # fmt: skip
+                               deterministic, fp8_scaled_p=q.dtype == torch.float8_e4m3fn)  # fmt: skip
     with torch.cuda.device(prepared.device):
         return prepared.launch()
 
@@ -298,8 +300,7 @@ def hstu_jagged_fp8(q, k, v, q_descale=None, k_descale=None, v_descale=None, *, 
     max_k = max_seq_len if max_seq_len_k is None else max_seq_len_k
     prepared = prepare_forward(q, k, v, mask, attn_bias, mask_type, max_seq_len, max_k, silu_scale, seq_offset, offs_k,
                                num_context, num_target, target_group_size, alpha, False, out_dtype=out_dtype,
-                               q_descale=q_descale, k_descale=k_descale, v_descale=v_descale,
-                               fp8_scaled_p=False)  # fmt: skip
+                               q_descale=q_descale, k_descale=k_descale, v_descale=v_descale)  # fmt: skip
     with torch.cuda.device(prepared.device):
         return prepared.launch()
 

@@ -35,7 +35,12 @@ def test_one_json_line_with_the_contract_fields():
     assert r["dtype"] == "bf16" and r["data"] == "synthetic" and "workload" in r["config"] and "model" not in r["config"]
     roof = r["roofline"]
     assert roof["bound"] == "mfma" and roof["peak"] == 2500.0 and abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-3
-    assert 0.02 < roof["frac"] < 1.0 and roof["traffic"] > 0
+    assert 0.02 < roof["frac"] < 1.0
+    # measured HBM traffic comes from a committed profile of this very kernel source, or is null with the reason
+    assert (roof["traffic"] or 0) > 0 or "stale" in roof["traffic_source"] or "not measured" in roof["traffic_source"]
+    # C2's working set fits the memory-side cache: the line also carries the time with cold caches, which cannot be
+    # meaningfully faster than the replay of one set
+    assert r["ms_per_step_cold"] > 0.9 * r["ms_per_step_events"] and r["value_cold"] > 0 and "sets" in r["cold_note"]
     cpu = r["cpu_baseline"]
     assert cpu["kind"] == "port" and cpu["cores"] >= 1 and cpu["value"] > 0 and cpu["sample"]
     # the value and the time per step are two views of the same measurement
