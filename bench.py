@@ -50,9 +50,10 @@ INFINITY_CACHE_BYTES = 256 << 20  # MI355X memory-side cache; a working set belo
 # the forward kernel's source at the time).  A figure whose hash no longer matches the source in the tree is stale
 # and is reported as null.
 MEASURED_TRAFFIC = {
-    "C2": (113_600_000, "profiles/hstu_fwd_bf16_d128_C2_counters.md", ""),
-    "C4": (1_575_000_000, "profiles/hstu_fwd_bf16_d128_rab_C4_trace_and_counters.md", ""),
-    "C5": (811_000_000, "profiles/hstu_fwd_f8e4m3_d128_C5_trace_and_counters.md", ""),
+    "C2": (110_800_000, "profiles/hstu_fwd_bf16_d128_C2_trace_and_counters.md", "cc1c4397874942bc"),
+    "C3": (300_400_000, "profiles/hstu_fwd_bf16_d128_rab_C3_trace_and_counters.md", "cc1c4397874942bc"),
+    "C4": (1_626_200_000, "profiles/hstu_fwd_bf16_d128_rab_C4_trace_and_counters.md", "cc1c4397874942bc"),
+    "C5": (837_400_000, "profiles/hstu_fwd_f8e4m3_d128_C5_trace_and_counters.md", "cc1c4397874942bc"),
 }
 KERNEL_SOURCE = os.path.join(_ROOT, "ops-rec_amd", "csrc", "hstu_fwd_kernel.hip.h")
 
@@ -250,6 +251,11 @@ def main() -> int:
     ap.add_argument("--forward-only", action="store_true",
                     help="time the attention forward only; by default (none of --backward / --ln-mul / --in-linear-silu "
                     "given) the line also carries the 'backward', 'ln_mul' and 'in_linear_silu' objects")
+    ap.add_argument("--no-cold", action="store_true",
+                    help="skip the cold-cache loop (profiler runs: every traced launch is then one of the timed loop's)")
+    ap.add_argument("--drop-rab", action="store_true",
+                    help="run the workload without its attn_bias (C3, C4): the difference of a counter run with and "
+                    "one without is the HBM traffic that the bias stream alone causes")
     ap.add_argument("--calibration-copy-mib", type=int, default=0,
                     help="after the timed steps also run 5 plain device-to-device copies of this many MiB, so that a "
                     "counter run (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE) can be scaled by a kernel of known traffic")  # fmt: skip
@@ -277,6 +283,8 @@ def main() -> int:
     heavy = args.workload != "C2"
     w_cpu = None if heavy else workloads.config(args.workload)
     w = workloads.config(args.workload, device=dev) if heavy else w_cpu.to(dev)
+    if args.drop_rab:
+        w.attn_bias = None
     n_q, d_qk, d_v = w.q.shape[1], w.q.shape[2], w.v.shape[2]
     ctx = None if w.num_context is None else w.num_context.cpu()
     tgt = None if w.num_target is None else w.num_target.cpu()
@@ -323,7 +331,7 @@ def main() -> int:
     # inputs (own outputs, own workspaces), together more than twice the cache, take turns, so that every launch
     # finds its rows in HBM only.
     cold_ms, cold_sets = None, 0
-    if alg_bytes <= INFINITY_CACHE_BYTES:
+    if alg_bytes <= INFINITY_CACHE_BYTES and not args.no_cold:
         cold_sets = max(4, -(-(5 * INFINITY_CACHE_BYTES // 2) // alg_bytes))
         clones = []
         for _ in range(cold_sets):
@@ -403,6 +411,7 @@ def main() -> int:
         "cold_note": (f"{cold_sets} independent input / output sets of {alg_bytes / 1e6:.0f} MB take turns "
                       f"({cold_sets * alg_bytes / 1e6:.0f} MB against a 256 MiB memory-side cache); 'value' and "
                       "'ms_per_step' replay one set" if cold_ms is not None else
+                      "skipped (--no-cold)" if args.no_cold else
                       "one set already exceeds the 256 MiB memory-side cache: the timed loop is cold as it is"),
         "ms_per_step_events": round(ev_ms, 6),
         "ms_per_step_wall": round(wall_ms, 6),
@@ -414,8 +423,8 @@ def main() -> int:
             "peak": peak,
             "unit": "TFLOP/s",
             "frac": round(kernel_tflops / peak, 4),
-            "traffic": measured_traffic(args.workload)[0],
-            "traffic_source": measured_traffic(args.workload)[1],
+            "traffic": None if args.drop_rab else measured_traffic(args.workload)[0],
+            "traffic_source": "not measured" if args.drop_rab else measured_traffic(args.workload)[1],
             "avg_launch_us": round(ev_ms * 1e3, 3),
             "hbm_achieved_GBs": round(alg_bytes / (ev_ms * 1e-3) / 1e9, 1),
             "hbm_peak_GBs": PEAK_HBM_GBS,

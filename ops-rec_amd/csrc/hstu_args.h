@@ -58,9 +58,6 @@ struct FwdArgs {
     int64_t num_pages;
     int64_t n_page_ids;
     int page_shift;  // log2(page_size); page_size is 32, 64, 128 or 256
-#ifdef HSTU_TIMELINE
-    unsigned long long* timeline;
-#endif
 };
 
 struct BwdArgs {

@@ -70,25 +70,6 @@ struct elem_traits<f8_tag> {
 constexpr uint32_t kBufferFlags = 0x00020000u;  // raw buffer, 32-bit data format (gfx9 family)
 constexpr uint32_t kOutOfRange = 0x80000000u;   // byte offset no descriptor here can contain
 
-// Optional per-wavefront timeline for kernel development (compile with -DHSTU_TIMELINE and pass a
-// buffer of 64 x uint64 per wavefront in FwdArgs::timeline); compiled out of the shipped library.
-#ifdef HSTU_TIMELINE
-#ifdef HSTU_TIMELINE_REALTIME
-#define HSTU_CLOCK() __builtin_amdgcn_s_memrealtime() /* 100 MHz, same base on every XCD */
-#else
-#define HSTU_CLOCK() __builtin_amdgcn_s_memtime() /* core clock, per-XCD base */
-#endif
-#define HSTU_STAMP(slot)                                                                              \
-    do {                                                                                              \
-        if (a.timeline && lane == 0 && (slot) < 64)                                                   \
-            a.timeline[(static_cast<int64_t>(blockIdx.x) * 4 + wave) * 64 + (slot)] = HSTU_CLOCK();   \
-    } while (0)
-#else
-#define HSTU_STAMP(slot) \
-    do {                 \
-    } while (0)
-#endif
-
 
 __device__ __forceinline__ int64_t load_index(const void* p, int64_t i, int idx64)
 {
@@ -780,15 +761,6 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         }
     };
 
-#ifdef HSTU_TIMELINE
-    if (a.timeline && lane == 0) {
-        // where this wavefront runs: HW_ID (CU, shader array, shader engine) and the XCD
-        a.timeline[(static_cast<int64_t>(blockIdx.x) * 4 + wave) * 64 + 62] =
-            static_cast<unsigned long long>(__builtin_amdgcn_s_getreg(0xF804)) |
-            (static_cast<unsigned long long>(__builtin_amdgcn_s_getreg(0xF814)) << 32);
-        a.timeline[(static_cast<int64_t>(blockIdx.x) * 4 + wave) * 64 + 61] = HSTU_CLOCK();
-    }
-#endif
     // =============================== item loop ===============================
     // The first item of a workgroup is fixed (workgroup w: item w / nq of queue w mod nq, nq = number of queues);
     // later ones are pulled from the queue's counter.  With the pull, the position of the next non-empty queue is
@@ -1047,17 +1019,6 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                 }
             }
         }
-#ifdef HSTU_TIMELINE
-        int log_slot = 0;
-        if (a.timeline && lane == 0) {
-            unsigned long long* row = a.timeline + (static_cast<int64_t>(blockIdx.x) * 4 + wave) * 64;
-            log_slot = static_cast<int>(row[0]);
-            if (log_slot < 12) {
-                row[1 + 5 * log_slot + 0] = s_item[5] | (static_cast<unsigned long long>(SPLIT ? s_item[7] : 0u) << 32);
-                row[1 + 5 * log_slot + 1] = HSTU_CLOCK();
-            }
-        }
-#endif
 
         // defensive clamps: malformed offsets must not turn into out-of-bounds addresses
         q1 = q1 < a.total_q ? q1 : a.total_q;
@@ -1780,11 +1741,6 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         // ---- key sweep ----
         __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
-#ifdef HSTU_TIMELINE
-        if (a.timeline && lane == 0 && log_slot < 12) {
-            a.timeline[(static_cast<int64_t>(blockIdx.x) * 4 + wave) * 64 + 1 + 5 * log_slot + 2] = HSTU_CLOCK();
-        }
-#endif
         if (x_end > x_begin) {
             // interior steps of this wavefront: [x_begin + 1, t_interior).  Sub-tile t + 1 (t + 2 with rab) must exist,
             // and sub-tile t must be fully visible: it ends at or before the smallest row limit and, when target
@@ -1838,11 +1794,6 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             }
         }
 
-#ifdef HSTU_TIMELINE
-        if (a.timeline && lane == 0 && log_slot < 12) {
-            a.timeline[(static_cast<int64_t>(blockIdx.x) * 4 + wave) * 64 + 1 + 5 * log_slot + 3] = HSTU_CLOCK();
-        }
-#endif
         // ---- split item: hand in this part; the part that completes the item adds all of them up ----
         bool store_rows = true;
         if constexpr (SPLIT) {
@@ -1980,13 +1931,6 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                 }
             }
         }
-#ifdef HSTU_TIMELINE
-        if (a.timeline && lane == 0 && log_slot < 12) {
-            unsigned long long* row = a.timeline + (static_cast<int64_t>(blockIdx.x) * 4 + wave) * 64;
-            row[1 + 5 * log_slot + 4] = HSTU_CLOCK();
-            row[0] = log_slot + 1;
-        }
-#endif
 
         // (the barriers of the sweep separate this item's reads of s_item from the next fetch)
         if constexpr (kStaticList) {
@@ -2007,7 +1951,6 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         }
     }
 
-    HSTU_STAMP(63);
 }
 
 }  // namespace hstu

@@ -704,12 +704,6 @@ int launch_forward(const hstu_jagged_fwd_params* p, const hstu_paged_fwd_params*
         a.page_shift = paged->page_size == 32 ? 5 : paged->page_size == 64 ? 6 : paged->page_size == 128 ? 7 : 8;
     }
 
-#ifdef HSTU_TIMELINE
-    // development builds only: the first MiB of the workspace receives the timeline
-    a.timeline = static_cast<unsigned long long*>(workspace);
-    workspace = static_cast<char*>(workspace) + (1 << 20);
-    workspace_bytes = workspace_bytes > (1u << 20) ? workspace_bytes - (1 << 20) : 0;
-#endif
     int64_t n_blocks = static_cast<int64_t>(a.n_qtiles) * a.bh;  // one per (query tile, sequence, head) slot
     if (n_blocks <= 0 || n_blocks > 0x7fffffffLL) {
         return fail(HSTU_ERR_INVALID, "grid of %lld workgroups is out of range", (long long)n_blocks);
