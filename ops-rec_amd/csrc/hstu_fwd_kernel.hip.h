@@ -182,10 +182,18 @@ __device__ __forceinline__ uint32_t pack2<f16_tag>(float lo, float hi)
     return __builtin_bit_cast(uint32_t, r);
 }
 
-// fp8: 8 e4m3 values per operand and lane (same row / column / k mapping as the 16-bit 32x32x16 form)
-__device__ __forceinline__ f32x16_t mfma32_f8(u32x2_t a, u32x2_t b, f32x16_t c)
+// fp8: D[32][32] += A[32][64] . B[64][32] on e4m3 operands, v_mfma_f32_32x32x64_f8f6f4 (both formats fp8, no block scales):
+// twice the rate per product term of the 32x32x16 form.  Lane (i, half) holds the 32 consecutive k values
+// 32 * half .. + 31 of row i of A (column i of B), lowest k in the lowest byte of the first register (checked on
+// the device against a host product); the accumulator layout is that of every 32x32 MFMA.
+typedef __attribute__((ext_vector_type(8))) int i32x8_t;
+__device__ __forceinline__ f32x16_t mfma32x64_f8(u32x4_t a_lo, u32x4_t a_hi, u32x4_t b_lo, u32x4_t b_hi, f32x16_t c)
 {
-    return __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(__builtin_bit_cast(long, a), __builtin_bit_cast(long, b), c, 0, 0, 0);
+    const i32x8_t a = {static_cast<int>(a_lo[0]), static_cast<int>(a_lo[1]), static_cast<int>(a_lo[2]), static_cast<int>(a_lo[3]),
+                       static_cast<int>(a_hi[0]), static_cast<int>(a_hi[1]), static_cast<int>(a_hi[2]), static_cast<int>(a_hi[3])};
+    const i32x8_t b = {static_cast<int>(b_lo[0]), static_cast<int>(b_lo[1]), static_cast<int>(b_lo[2]), static_cast<int>(b_lo[3]),
+                       static_cast<int>(b_hi[0]), static_cast<int>(b_hi[1]), static_cast<int>(b_hi[2]), static_cast<int>(b_hi[3])};
+    return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
 }
 // two floats -> two e4m3 bytes in the low (hi = false) or high half of `old`; round to nearest even.
 // The conversion turns magnitudes above 464 into NaN, so the values are clamped to the format's range first.
@@ -366,10 +374,13 @@ struct U32Quad {
 //
 // fp8 inputs (Tag = f8_tag; OutTag picks the 16-bit output type): same structure with one-byte elements.  The
 // score is brought to its real scale (alpha x per-head dequantisation scales) before SiLU, P^T is clamped to
-// +-448 and re-quantised to e4m3 (round to nearest even) BEFORE silu_scale is applied, silu_scale and the V
-// scale are applied to the fp32 output.  K is read 16 bytes per lane for two MFMA steps at a time (k index
-// (half, byte) of step 2p / 2p+1 = dim 16 (2p + half) + byte / + 8 + byte), V^T by one 8-bit transposed read
-// per MFMA.  rab and custom masks are not available for fp8 inputs.
+// +-448 and re-quantised to e4m3 (round to nearest even) before or after silu_scale is applied (fp8_scaled_p), the
+// V scale (and silu_scale in the first case) goes on the fp32 output.  Both products run on the 64-deep MFMA
+// (v_mfma_f32_32x32x64_f8f6f4, twice the rate of the 16-deep fp8 form): an operand is 32 bytes per lane.  For QK
+// these are two 16-byte reads of a K row (and the matching two pieces of the Q fragment: k index (half, byte) =
+// dim 16 (2p + half) + byte of piece p); PV contracts over the 64 keys of a pair of sub-tiles, its V^T operand
+// being four 8-bit transposed reads (16 keys x 32 dims each) in the order in which P^T holds the keys.  rab and the
+// custom mask are e4m3 tensors like q (plain list only).
 //
 // QUEUES: build the per-XCD queue machinery (see "Work queues" below).  It pays on long, jagged batches with many
 // items per workgroup; its code is on the path of every item, so launches that cannot profit (the host decides by
@@ -405,6 +416,13 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
     static_assert(2 * MTILES == NCH, "QK and PV products must have the same number of MFMAs");
     constexpr int VM_OUTSTANDING = 2 * 2 * LPW;  // tile requests of two time steps
     constexpr int kWaitTiles = (VM_OUTSTANDING & 15) | (7 << 4) | (15 << 8) | ((VM_OUTSTANDING >> 4) << 14);
+    // fp8: both products on the 64-deep MFMA.  QK takes D / 64 of them per sub-tile; PV contracts over the 64 keys of
+    // a PAIR of sub-tiles (2u, 2u + 1), half of its D / 32 output tiles in time step 2u + 2 and half in 2u + 3, so a
+    // step carries D / 64 MFMAs of either product.  V sub-tiles are requested two at a time in the even steps.
+    constexpr bool K64 = F8;
+    constexpr int NCH2 = D / 64;
+    constexpr int kWaitEven64 = ((4 * LPW) & 15) | (7 << 4) | (15 << 8);  // after an even step: V, V, K of it and K of the step before
+    constexpr int kWaitOdd64 = ((2 * LPW) & 15) | (7 << 4) | (15 << 8);   // after an odd step: its K and the K of the step before
     constexpr uint32_t kPastEnd = 0x40000000u;   // added to a source offset: leaves every descriptor
 
     // eight separate arrays (not one block) so that the compiler can tell the slot being filled by the
@@ -1206,7 +1224,9 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             }
         }
         request_k(ic0_t{}, x_begin);
-        request_v(ic0_t{}, x_begin);
+        if constexpr (!K64) {
+            request_v(ic0_t{}, x_begin);  // (64-deep PV: V(x_begin) and V(x_begin + 1) go out in time step x_begin)
+        }
         request_k(ic1_t{}, x_begin + 1);
         request_k(ic2_t{}, x_begin + 2);
         // Q fragment: lane (ln, lh) holds Q[row][16*js + 8*lh .. +7] for js = 0..KSTEPS-1
@@ -1423,6 +1443,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         // register blocks of the rolling pipeline: sub-tile x uses block x & 1
         f32x16_t s_blk0, s_blk1;     // S^T
         uint32_t p_blk0[8], p_blk1[8];  // P^T, packed pairs
+        uint32_t p_blk2[8], p_blk3[8];  // 64-deep PV only: sub-tile x uses P^T block x & 3 (a pair is consumed two and three steps on)
         uint32_t rabw0[8], rabw1[8];  // rab words of sub-tile x in block x & 1
         uint32_t mw0[8], mw1[8];      // custom mask words of sub-tile x in block x & 1
 #pragma unroll
@@ -1434,6 +1455,8 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
         for (int i = 0; i < 8; ++i) {
             p_blk0[i] = 0;
             p_blk1[i] = 0;
+            p_blk2[i] = 0;
+            p_blk3[i] = 0;
             rabw0[i] = 0;
             rabw1[i] = 0;
             mw0[i] = 0;
@@ -1456,8 +1479,25 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             constexpr int PAR = S & 1;  // parity of t
             const f32x16_t& s_cur = PAR ? s_blk1 : s_blk0;  // S^T(t), transformed in this step
             f32x16_t& s_nxt = PAR ? s_blk0 : s_blk1;        // S^T(t+1), accumulated in this step
-            uint32_t(&pk_cur)[8] = PAR ? p_blk1 : p_blk0;         // P^T(t), written
-            const uint32_t(&pk_prev)[8] = PAR ? p_blk0 : p_blk1;  // P^T(t-1), consumed
+            // P^T block of sub-tile x: x & 1, or x & 3 with the 64-deep PV
+            auto p_block = [&](auto ic) -> uint32_t(&)[8] {
+                constexpr int I = decltype(ic)::value & 3;
+                if constexpr (I == 0) {
+                    return p_blk0;
+                } else if constexpr (I == 1) {
+                    return p_blk1;
+                } else if constexpr (I == 2) {
+                    return p_blk2;
+                } else {
+                    return p_blk3;
+                }
+            };
+            uint32_t(&pk_cur)[8] = p_block(std::integral_constant<int, K64 ? S : PAR>{});        // P^T(t), written
+            const uint32_t(&pk_prev)[8] = p_block(std::integral_constant<int, PAR ? 0 : 1>{});   // P^T(t-1), consumed (32-deep PV)
+            // 64-deep PV: the pair of sub-tiles consumed in this step, t - 2 and t - 1 (t even) or t - 3 and t - 2 (t odd)
+            constexpr int LO = PAR ? (S + 1) & 3 : (S + 2) & 3;
+            constexpr int HI = (LO + 1) & 3;
+            const int t0 = PAR ? t - 3 : t - 2;
             uint32_t(&mw_cur)[8] = PAR ? mw1 : mw0;               // custom mask words of sub-tile t
             uint32_t(&mw_nxt)[8] = PAR ? mw0 : mw1;
             uint32_t(&rab_far)[8] = PAR ? rabw1 : rabw0;          // receives rab(t+2)
@@ -1468,7 +1508,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
 
             const bool do_qk = INTERIOR || t + 1 < nx_w;
             const bool do_silu = INTERIOR || (t >= x_begin && t < nx_w);
-            const bool do_pv = INTERIOR || (t >= x_begin + 1 && t <= nx_w);
+            const bool do_pv = INTERIOR || (K64 ? (t0 >= x_begin && t0 < nx_w) : (t >= x_begin + 1 && t <= nx_w));
             const bool full = INTERIOR || ((c0 + 32 <= lim_min) && !(any_hole && c0 + 32 > hist_k && c0 < hole_hi_max));
 
             // (1) bias / mask requests for later steps; they go out before the tile requests of this step so
@@ -1493,8 +1533,18 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                 }
             }
             // (2) tile requests of this time step
-            request_k(sc, t + 4);
-            request_v(std::integral_constant<int, (S + 2) & 3>{}, t + 2);
+            if constexpr (K64) {
+                // V(t) and V(t + 1), both in the even steps (their slots held V(t - 4) and V(t - 3), read for the last
+                // time in step t - 1), ahead of K so that the wait after an odd step may leave two K requests open
+                if constexpr (!PAR) {
+                    request_v(std::integral_constant<int, S>{}, t);
+                    request_v(std::integral_constant<int, (S + 1) & 3>{}, t + 1);
+                }
+                request_k(sc, t + 4);
+            } else {
+                request_k(sc, t + 4);
+                request_v(std::integral_constant<int, (S + 2) & 3>{}, t + 2);
+            }
             if constexpr (PAGED) {
                 pid_ring[(S + 1) & 3] = page_of(t + 5);  // for the request of K(t + 5) in the next time step
             }
@@ -1518,17 +1568,11 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             // same registers
             auto read_v = [&](int c) -> u32x4_t {
                 const int j2 = c % 2, mt = c / 2;
-                if constexpr (F8) {
-                    const u32x2_t t8 = lds_read_tr8_b64(reinterpret_cast<const uint8_t*>(vt) + v_lane_off[mt] + 16 * j2 * D);
-                    const u32x4_t r = {t8[0], t8[1], 0u, 0u};
-                    return r;
-                } else {
-                    const uint16_t* p = vt + v_lane_off[mt] + 16 * j2 * D;
-                    const u32x2_t lo = lds_read_tr16_b64(p);
-                    const u32x2_t hi = lds_read_tr16_b64(p + 8 * D);
-                    const u32x4_t r = {lo[0], lo[1], hi[0], hi[1]};
-                    return r;
-                }
+                const uint16_t* p = vt + v_lane_off[mt] + 16 * j2 * D;
+                const u32x2_t lo = lds_read_tr16_b64(p);
+                const u32x2_t hi = lds_read_tr16_b64(p + 8 * D);
+                const u32x4_t r = {lo[0], lo[1], hi[0], hi[1]};
+                return r;
             };
             // unmasked P^T pair i (score elements 2i, 2i+1)
             auto silu_pair = [&](int i) {
@@ -1613,7 +1657,89 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                     order_bias(mw_cur);
                 }
             }
-            if (do_pv) {
+            if constexpr (K64) {
+                // ---- both products on the 64-deep MFMA ----
+                if (do_pv) {
+                    const uint8_t* const v_lo = reinterpret_cast<const uint8_t*>(v_slot(std::integral_constant<int, LO>{}));
+                    const uint8_t* const v_hi = reinterpret_cast<const uint8_t*>(v_slot(std::integral_constant<int, HI>{}));
+                    const uint32_t(&p_lo)[8] = p_block(std::integral_constant<int, LO>{});
+                    const uint32_t(&p_hi)[8] = p_block(std::integral_constant<int, HI>{});
+                    constexpr int MT0 = PAR ? MTILES / 2 : 0;  // this step's half of the output tiles
+                    // sub-tile t0 + 1 may lie past the end of the sweep: its P^T block is zero, and its slot then holds
+                    // whatever an earlier sweep left there, so its half of the operand is zero as well
+                    const bool hi_ok = INTERIOR || (t0 + 1 < x_end);
+                    // V^T operand of output tile mt: keys of the two 16-key groups of either sub-tile, in P^T's order
+                    auto read_v64 = [&](int mt, u32x4_t& lo, u32x4_t& hi) {
+                        const u32x2_t a0 = lds_read_tr8_b64(v_lo + v_lane_off[mt]);
+                        const u32x2_t a1 = lds_read_tr8_b64(v_lo + v_lane_off[mt] + 16 * D);
+                        const u32x2_t b0 = lds_read_tr8_b64(v_hi + v_lane_off[mt]);
+                        const u32x2_t b1 = lds_read_tr8_b64(v_hi + v_lane_off[mt] + 16 * D);
+                        lo = u32x4_t{a0[0], a0[1], a1[0], a1[1]};
+                        hi = u32x4_t{b0[0], b0[1], b1[0], b1[1]};
+                    };
+                    u32x4_t va_lo[NCH2], va_hi[NCH2];
+                    read_v64(MT0, va_lo[0], va_hi[0]);
+                    __builtin_amdgcn_sched_barrier(0);
+                    const u32x4_t pb_lo = {p_lo[0], p_lo[1], p_lo[2], p_lo[3]};
+                    const u32x4_t pb_hi = {p_hi[0], p_hi[1], p_hi[2], p_hi[3]};
+#pragma unroll
+                    for (int c = 0; c < NCH2; ++c) {
+                        u32x4_t hi = va_hi[c];
+                        if constexpr (!INTERIOR) {
+                            if (!hi_ok) {
+                                hi = u32x4_t{0u, 0u, 0u, 0u};
+                            }
+                        }
+                        o_acc[MT0 + c] = mfma32x64_f8(va_lo[c], hi, pb_lo, pb_hi, o_acc[MT0 + c]);
+                        if (c + 1 < NCH2) {
+                            read_v64(MT0 + c + 1, va_lo[c + 1], va_hi[c + 1]);
+                        }
+#pragma unroll
+                        for (int i = c * 4 / NCH2; i < (c + 1) * 4 / NCH2; ++i) {
+                            silu_pair(i);
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                } else if (do_silu) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        silu_pair(i);
+                    }
+                }
+                if (do_qk) {
+                    u32x4_t kop[KREADS];
+                    kop[0] = read_k(0);
+                    kop[1] = read_k(1);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int c = 0; c < NCH2; ++c) {
+                        if (c == 0) {
+                            f32x16_t zero;
+#pragma unroll
+                            for (int i = 0; i < 16; ++i) {
+                                zero[i] = 0.f;
+                            }
+                            s_nxt = mfma32x64_f8(kop[0], kop[1], qf[0], qf[1], zero);
+                        } else {
+                            s_nxt = mfma32x64_f8(kop[2 * c], kop[2 * c + 1], qf[2 * c], qf[2 * c + 1], s_nxt);
+                        }
+                        if (c + 1 < NCH2) {
+                            kop[2 * c + 2] = read_k(2 * c + 2);
+                            kop[2 * c + 3] = read_k(2 * c + 3);
+                        }
+#pragma unroll
+                        for (int i = c * 4 / NCH2; i < (c + 1) * 4 / NCH2; ++i) {
+                            silu_pair(4 + i);
+                        }
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                } else if (do_silu) {
+#pragma unroll
+                    for (int i = 4; i < 8; ++i) {
+                        silu_pair(i);
+                    }
+                }
+            } else if (do_pv) {
                 u32x4_t vop[NCH];
 #pragma unroll
                 for (int c = 0; c < LOOKAHEAD; ++c) {
@@ -1623,14 +1749,8 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
 #pragma unroll
                 for (int c = 0; c < NCH; ++c) {
                     const int j2 = c % 2, mt = c / 2;
-                    if constexpr (F8) {
-                        const u32x2_t va = {vop[c][0], vop[c][1]};
-                        const u32x2_t pb = {pk_prev[2 * j2 + 0], pk_prev[2 * j2 + 1]};
-                        o_acc[mt] = mfma32_f8(va, pb, o_acc[mt]);
-                    } else {
-                        const u32x4_t pb = {pk_prev[4 * j2 + 0], pk_prev[4 * j2 + 1], pk_prev[4 * j2 + 2], pk_prev[4 * j2 + 3]};
-                        o_acc[mt] = mfma32<Tag>(vop[c], pb, o_acc[mt]);
-                    }
+                    const u32x4_t pb = {pk_prev[4 * j2 + 0], pk_prev[4 * j2 + 1], pk_prev[4 * j2 + 2], pk_prev[4 * j2 + 3]};
+                    o_acc[mt] = mfma32<Tag>(vop[c], pb, o_acc[mt]);
                     if (c + LOOKAHEAD < NCH) {
                         vop[c + LOOKAHEAD] = read_v(c + LOOKAHEAD);
                     }
@@ -1643,38 +1763,8 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                     silu_pair(i);
                 }
             }
-            if constexpr (F8) {
-                if (do_qk) {
-                    u32x4_t kop[KREADS];
-                    kop[0] = read_k(0);
-                    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-                    for (int c = 0; c < NCH; ++c) {
-                        const int r = c / 2;
-                        const u32x2_t ka = (c & 1) ? u32x2_t{kop[r][2], kop[r][3]} : u32x2_t{kop[r][0], kop[r][1]};
-                        const u32x2_t qb = (c & 1) ? u32x2_t{qf[r][2], qf[r][3]} : u32x2_t{qf[r][0], qf[r][1]};
-                        if (c == 0) {
-                            f32x16_t zero;
-#pragma unroll
-                            for (int i = 0; i < 16; ++i) {
-                                zero[i] = 0.f;
-                            }
-                            s_nxt = mfma32_f8(ka, qb, zero);
-                        } else {
-                            s_nxt = mfma32_f8(ka, qb, s_nxt);
-                        }
-                        if (!(c & 1) && r + 1 < KREADS) {
-                            kop[r + 1] = read_k(r + 1);
-                        }
-                        silu_chunk(4, c);
-                        __builtin_amdgcn_sched_barrier(0);
-                    }
-                } else if (do_silu) {
-#pragma unroll
-                    for (int i = 4; i < 8; ++i) {
-                        silu_pair(i);
-                    }
-                }
+            if constexpr (K64) {
+                // (done above)
             } else if (do_qk) {
                 u32x4_t kop[NCH];
 #pragma unroll
@@ -1731,9 +1821,19 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                 }
             }
 
+            if constexpr (K64 && !INTERIOR) {
+                // a step past the end of this wavefront's sweep: its P^T block may be the upper half of the last pair
+                if (!do_silu) {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        pk_cur[i] = 0u;
+                    }
+                }
+            }
+
             // (4) the requests made two time steps ago have landed (mine), then everybody's
             __builtin_amdgcn_sched_barrier(0);
-            __builtin_amdgcn_s_waitcnt(kWaitTiles);
+            __builtin_amdgcn_s_waitcnt(K64 ? (PAR ? kWaitOdd64 : kWaitEven64) : kWaitTiles);
             __builtin_amdgcn_s_barrier();
             __builtin_amdgcn_sched_barrier(0);
         };
@@ -1762,20 +1862,23 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             }
             typedef std::false_type general_t;
             typedef std::true_type interior_t;
+            // (64-deep PV: the pair that holds the last sub-tile is consumed two and three steps after its first half)
+            const int x_last = K64 ? x_end + 1 + (x_end & 1) : x_end;
             int t = x_begin - 1;
             while (true) {
                 time_step(ic3_t{}, general_t{}, t);
-                if (++t > x_end) {
+                if (++t > x_last) {
                     break;
                 }
                 time_step(ic0_t{}, general_t{}, t);
-                if (++t > x_end) {
+                if (++t > x_last) {
                     break;
                 }
                 // (t mod 4 == 1 and t >= x_begin + 1 here; at head dim 256 a step is 32 MFMAs long and the general
                 // step's overhead is small beside it, so that variant is not given the second copy)
                 if constexpr (D <= 128) {
-                    while (t + 4 <= t_interior) {
+                    // (64-deep PV: the pair consumed in step t begins at t - 3, which must lie in this sweep)
+                    while (t + 4 <= t_interior && (!K64 || t > x_begin + 1)) {
                         time_step(ic1_t{}, interior_t{}, t);
                         time_step(ic2_t{}, interior_t{}, t + 1);
                         time_step(ic3_t{}, interior_t{}, t + 2);
@@ -1784,11 +1887,11 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                     }
                 }
                 time_step(ic1_t{}, general_t{}, t);
-                if (++t > x_end) {
+                if (++t > x_last) {
                     break;
                 }
                 time_step(ic2_t{}, general_t{}, t);
-                if (++t > x_end) {
+                if (++t > x_last) {
                     break;
                 }
             }
