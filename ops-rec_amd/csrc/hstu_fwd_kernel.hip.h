@@ -196,13 +196,20 @@ __device__ __forceinline__ f32x16_t mfma32x64_f8(u32x4_t a_lo, u32x4_t a_hi, u32
     return __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(a, b, c, 0, 0, 0, 0, 0, 0);
 }
 // two floats -> two e4m3 bytes in the low (hi = false) or high half of `old`; round to nearest even.
-// The conversion turns magnitudes above 464 into NaN, so the values are clamped to the format's range first.
+// By default the conversion turns magnitudes above 464 into NaN; the fp8 kernels run with the overflow-clamp bit of
+// the wavefront's MODE register set (fp8_saturating_conversions()), under which they become +-448 instead (checked
+// on the device: 1000 -> 0x7e, -1e30 -> 0xfe), so no clamp is spent per element.
 template <bool HI>
 __device__ __forceinline__ uint32_t pack2_f8(float a, float b, uint32_t old)
 {
-    a = __builtin_amdgcn_fmed3f(a, -448.0f, 448.0f);
-    b = __builtin_amdgcn_fmed3f(b, -448.0f, 448.0f);
     return static_cast<uint32_t>(__builtin_amdgcn_cvt_pk_fp8_f32(a, b, static_cast<int>(old), HI));
+}
+
+// MODE.FP16_OVFL (bit 23 of hardware register 1): conversions to fp8 (and to fp16) saturate at the largest finite
+// value instead of overflowing.  Per wavefront, set once at kernel entry; the state ends with the wavefront.
+__device__ __forceinline__ void fp8_saturating_conversions()
+{
+    __builtin_amdgcn_s_setreg(1 | (23 << 6) | (0 << 11), 1);
 }
 
 template <typename Tag>
@@ -399,6 +406,9 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
 {
     constexpr int kThreads = 256;
     constexpr bool F8 = elem_traits<Tag>::kF8;
+    if constexpr (F8) {
+        fp8_saturating_conversions();  // P^T beyond +-448 becomes +-448, not NaN (an fp16 output saturates likewise)
+    }
     constexpr uint32_t ES = elem_traits<Tag>::kBytes;  // bytes per input element
     static_assert(!F8 || !(HAS_RAB || HAS_MASK) || !(QUEUES || SPLIT), "fp8 with rab / custom mask: plain list only");
     static_assert(!F8 || D >= 64, "fp8 rows are at least 64 bytes");
@@ -736,6 +746,8 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
     float c_out = a.c_out;
     float c_x = 1.0f;  // fp8 only: raw score -> alpha * (dequantised score)
     float c_p = 1.0f;  // fp8 only: what P is multiplied by before it is quantised (1, or silu_scale)
+    float c_pi = 1.0f;  // fp8 only: 1 / c_p, and 1 / (c_x c_p): the factors of (1 + t) in the sigmoid's reciprocal
+    float c_qi = 1.0f;
     // rab is added to S^T by the matrix pipe: S^T += E_j . R_j (j = 0, 1), where R_j holds, per lane (query row,
     // half lh), the 8 consecutive rab values of keys 16 lh + 8 j .. + 7 exactly as they lie in memory (B operand)
     // and E_j is the constant 0/1 matrix that routes k-slot (lh, e) to key row 16 lh + 8 j + e (A operand).
@@ -1127,6 +1139,8 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
             // rounding point, to P before it is quantised (fp8_scaled_p)
             c_out = (a.fp8_scaled_p ? 1.0f : a.silu_scale) * vs;
             c_p = a.fp8_scaled_p ? a.silu_scale : 1.0f;
+            c_pi = 1.0f / c_p;
+            c_qi = 1.0f / (c_x * c_p);
         }
 
         // ---- keys needed by this item ----
@@ -1588,7 +1602,8 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                     }
 #pragma unroll
                     for (int e = 0; e < 2; ++e) {
-                        p[e] = x[e] * __builtin_amdgcn_rcpf(1.0f + tt[e]) * c_p;
+                        // x sigmoid(x) c_p = x / ((1 + t) / c_p)
+                        p[e] = x[e] * __builtin_amdgcn_rcpf(__builtin_fmaf(tt[e], c_pi, c_pi));
                     }
                     if constexpr (HAS_MASK) {
                         p[0] *= f8_element(mw_cur, 2 * i);
@@ -1611,7 +1626,13 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                 }
 #pragma unroll
                 for (int e = 0; e < 2; ++e) {
-                    tt[e] = 1.0f + tt[e];
+                    if constexpr (F8) {
+                        // the scale that brings P^T to where it is quantised rides on the reciprocal:
+                        // s sigma c_q = s / ((1 + t) / c_q)
+                        tt[e] = __builtin_fmaf(tt[e], c_qi, c_qi);
+                    } else {
+                        tt[e] = 1.0f + tt[e];
+                    }
                 }
 #pragma unroll
                 for (int e = 0; e < 2; ++e) {
@@ -1631,13 +1652,12 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const
                     }
                 }
                 if constexpr (F8) {
-                    // bring P^T to its real scale (times silu_scale at the reference's rounding point) before it is
-                    // quantised; pair i = bytes 2 (i % 2), +1 of word i / 2
-                    const float c_q = c_x * c_p;
+                    // (P^T is at its real scale, times silu_scale at the reference's rounding point: see c_qi);
+                    // pair i = bytes 2 (i % 2), +1 of word i / 2
                     if (i & 1) {
-                        pk_cur[i / 2] = pack2_f8<true>(p[0] * c_q, p[1] * c_q, pk_cur[i / 2]);
+                        pk_cur[i / 2] = pack2_f8<true>(p[0], p[1], pk_cur[i / 2]);
                     } else {
-                        pk_cur[i / 2] = pack2_f8<false>(p[0] * c_q, p[1] * c_q, pk_cur[i / 2]);
+                        pk_cur[i / 2] = pack2_f8<false>(p[0], p[1], pk_cur[i / 2]);
                     }
                 } else {
                     pk_cur[i] = pack2<Tag>(p[0], p[1]);

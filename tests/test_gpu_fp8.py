@@ -82,6 +82,29 @@ def test_reference_entry_point_with_e4m3_tensors_gives_half_output():
     assert (got - want).abs().max() <= 0.05 * peak
 
 
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("d", [64, 128])
+def test_p_beyond_the_e4m3_range_saturates(d, out_dtype):
+    # scores in the thousands: silu(x) ~ x lies far beyond +-448, the largest e4m3 value; the rounded P must be
+    # +-448 there (as the oracle's quantiser clamps), never NaN.  Half of the keys give large negative scores (P ~ 0).
+    g = torch.Generator().manual_seed(d)
+    lengths = [70, 33]
+    total = sum(lengths)
+    sign = torch.where(torch.arange(total) % 2 == 0, 1.0, -1.0).view(total, 1, 1)
+    q8 = O.quantize_e4m3(torch.full((total, 2, d), 16.0))
+    k8 = O.quantize_e4m3(torch.full((total, 2, d), 16.0) * sign)
+    v8 = O.quantize_e4m3(torch.randn(total, 2, d, generator=g) * 0.25)
+    offs = torch.tensor([0, 70, 103], dtype=torch.int32)
+    kw = dict(mask_type=0, max_seq_len=70, silu_scale=1.0, seq_offset=offs, alpha=1.0)
+    out = ops_rec.hstu_jagged_fp8(dev(q8), dev(k8), dev(v8), None, None, None, out_dtype=out_dtype,
+                                  **dict(kw, seq_offset=dev(offs)))  # fmt: skip
+    got = out.float().cpu()
+    assert torch.isfinite(got).all()
+    want = O.hstu_jagged_forward_fp8(q8, k8, v8, None, None, None, quantize_p=True, out_dtype=torch.float32, **kw)
+    assert want.abs().max() > 448  # sums of saturated terms
+    torch.testing.assert_close(got, want, atol=1e-2 * want.abs().max().item(), rtol=1e-2)
+
+
 def test_fp8_int64_offsets_and_delta_lengths():
     # K / V longer than Q (delta form through seq_offset_k), int64 offsets
     g = torch.Generator().manual_seed(4)
