@@ -118,16 +118,42 @@ __device__ __forceinline__ void row_bounds(const SeqInfo& s, int mask_type, int 
     }
 }
 
-// P (without mask) and dS (without mask) of one score element
-__device__ __forceinline__ void score_grad(float s, float dp, float alpha, float c_exp, float scale, float ascale,
-                                           float& p, float& ds)
+// The score algebra of the backward, per element, with X = alpha s, sig = sigmoid(X), t = exp(-X):
+//   P  = X sig scale                       = s * [alpha scale sig]
+//   dS = alpha scale dP sig (1 + X (1 - sig)) = dP * [alpha scale sig] * (1 + s * [alpha (1 - sig)])
+// The constants ride on the reciprocal: alpha scale sig = rcp((1 + t) / (alpha scale)) = rcp(fma(t, ci, ci)), and
+// alpha (1 - sig) = alpha - [alpha scale sig] / scale.  That is 3 vector instructions and the two transcendental
+// ones for P, 6 and two for dS (9 and 8 written out term by term) -- the vector unit is what the steps of these
+// kernels wait for as much as the matrix pipe.  alpha = 0 gives P = dS = 0 (ci = inf, rcp(inf) = 0), as it must.
+struct ScoreConsts {
+    float c_exp;      // -alpha log2(e)
+    float ci;         // 1 / (alpha scale)
+    float inv_scale;  // 1 / scale
+    float alpha;
+};
+__device__ __forceinline__ ScoreConsts score_consts(float alpha, float scale)
 {
-    const float x = s * alpha;
-    const float e = __builtin_amdgcn_exp2f(s * c_exp);
-    const float sig = __builtin_amdgcn_rcpf(1.0f + e);
-    const float xs = x * sig;
-    p = xs * scale;
-    ds = ascale * dp * (sig + xs * (1.0f - sig));
+    ScoreConsts c;
+    c.c_exp = -alpha * 1.4426950408889634f;
+    c.ci = 1.0f / (alpha * scale);
+    c.inv_scale = 1.0f / scale;
+    c.alpha = alpha;
+    return c;
+}
+// alpha scale sigmoid(alpha s)
+__device__ __forceinline__ float scaled_sigmoid(float s, const ScoreConsts& c)
+{
+    const float t = __builtin_amdgcn_exp2f(s * c.c_exp);
+    return __builtin_amdgcn_rcpf(__builtin_fmaf(t, c.ci, c.ci));
+}
+// P (without mask)
+__device__ __forceinline__ float score_p(float s, const ScoreConsts& c) { return s * scaled_sigmoid(s, c); }
+// dS (without mask)
+__device__ __forceinline__ float score_ds(float s, float dp, const ScoreConsts& c)
+{
+    const float sg = scaled_sigmoid(s, c);
+    const float u = __builtin_fmaf(-sg, c.inv_scale, c.alpha);  // alpha (1 - sig)
+    return dp * (sg * __builtin_fmaf(s, u, 1.0f));
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -376,8 +402,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_bwd_dq_kernel(co
             dq_acc[mt][i] = 0.f;
         }
     }
-    const float c_exp = -a.alpha * 1.4426950408889634f;
-    const float ascale = a.alpha * a.scale;
+    const ScoreConsts sconst = score_consts(a.alpha, a.scale);
 
     static_assert(NLW == 4, "every wavefront takes part in the loads");
     auto request = [&](uint16_t* kd, uint16_t* vd, int x) {
@@ -450,8 +475,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_bwd_dq_kernel(co
                 if constexpr (HAS_RAB) {
                     sv += e2 ? hi_to_float<Tag>(rw[i]) : lo_to_float<Tag>(rw[i]);
                 }
-                float p, ds;
-                score_grad(sv, dp[e], a.alpha, c_exp, a.scale, ascale, p, ds);
+                float ds = score_ds(sv, dp[e], sconst);
                 if constexpr (HAS_MASK) {
                     ds *= e2 ? hi_to_float<Tag>(mw[i]) : lo_to_float<Tag>(mw[i]);
                 }
@@ -694,8 +718,7 @@ __global__ __launch_bounds__(kDkvThreads, (D <= 128 ? 2 : 1)) void hstu_bwd_dkv_
             acc[mt][i] = 0.f;
         }
     }
-    const float c_exp = -a.alpha * 1.4426950408889634f;
-    const float ascale = a.alpha * a.scale;
+    const ScoreConsts sconst = score_consts(a.alpha, a.scale);
     const uint32_t bias_bytes = static_cast<uint32_t>(a.max_q) * static_cast<uint32_t>(a.max_k) * 2u;
     const bool targets = a.mask_type == 0 && si.n_tgt > 0 && a.target_group > 0;
     // rab / custom mask tiles are wanted with lane = key and registers = query rows, but lie in memory with the
@@ -886,15 +909,12 @@ __global__ __launch_bounds__(kDkvThreads, (D <= 128 ? 2 : 1)) void hstu_bwd_dkv_
             if (dk_role) {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
-                    float p, ds;
-                    score_grad(xs[e], dp[e], a.alpha, c_exp, a.scale, ascale, p, ds);
-                    o[e] = ds * ms[e];
+                    o[e] = score_ds(xs[e], dp[e], sconst) * ms[e];
                 }
             } else {
 #pragma unroll
                 for (int e = 0; e < 16; ++e) {
-                    const float sig = __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(xs[e] * c_exp));
-                    o[e] = xs[e] * sig * ascale * ms[e];  // P = X sig scale, X = alpha (S + rab)
+                    o[e] = score_p(xs[e], sconst) * ms[e];  // P = X sig scale, X = alpha (S + rab)
                 }
             }
             if (!full) {
