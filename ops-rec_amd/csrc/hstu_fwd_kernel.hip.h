@@ -402,7 +402,7 @@ struct U32Quad {
 // of the SPLIT variant, because its callers (inference: few query rows against a long cache) have short lists.
 template <typename Tag, typename OutTag, int D, bool HAS_RAB, bool HAS_MASK, bool QUEUES = false, bool SPLIT = false,
           bool PAGED = false>
-__global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_fwd_kernel(const FwdArgs a)
+__global__ __launch_bounds__(256, fwd_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hstu_fwd_kernel(const FwdArgs a)
 {
     constexpr int kThreads = 256;
     constexpr bool F8 = elem_traits<Tag>::kF8;

@@ -37,17 +37,17 @@ constexpr auto paged_kernel() -> void (*)(const FwdArgs)
 
 }  // namespace hstu
 
-#define HSTU_VARIANT(tag, tagname, D, RAB, MASK, WGS)                                               \
+#define HSTU_VARIANT(tag, tagname, D, RAB, MASK)                                              \
     {"hstu_fwd_" tagname "_d" #D "_rab" #RAB "_mask" #MASK,                                        \
      "hstu_fwd_" tagname "_d" #D "_rab" #RAB "_mask" #MASK "_queues",                               \
      "hstu_fwd_" tagname "_d" #D "_rab" #RAB "_mask" #MASK "_split",                                \
      hstu::hstu_fwd_kernel<hstu::tag, hstu::tag, D, RAB, MASK>,                                     \
      hstu::queues_kernel<hstu::tag, hstu::tag, D, RAB, MASK>(),                                     \
      hstu::split_kernel<hstu::tag, hstu::tag, D, RAB, MASK>(),                                      \
-     hstu::paged_kernel<hstu::tag, hstu::tag, D, RAB, MASK>(), D, 256, WGS}
+     hstu::paged_kernel<hstu::tag, hstu::tag, D, RAB, MASK>(), D, 256, hstu::fwd_wgs_per_cu(D, RAB, MASK)}
 #define HSTU_DIMS(tag, tagname, RAB, MASK)                                                           \
-    {HSTU_VARIANT(tag, tagname, 32, RAB, MASK, 2), HSTU_VARIANT(tag, tagname, 64, RAB, MASK, 2), \
-     HSTU_VARIANT(tag, tagname, 128, RAB, MASK, 2), HSTU_VARIANT(tag, tagname, 256, RAB, MASK, 1)}
+    {HSTU_VARIANT(tag, tagname, 32, RAB, MASK), HSTU_VARIANT(tag, tagname, 64, RAB, MASK), \
+     HSTU_VARIANT(tag, tagname, 128, RAB, MASK), HSTU_VARIANT(tag, tagname, 256, RAB, MASK)}
 // one 16-bit input type: [rab][custom mask][dim slot]
 #define HSTU_FWD16_TABLE(tag, tagname)                                         \
     {{HSTU_DIMS(tag, tagname, false, false), HSTU_DIMS(tag, tagname, false, true)}, \
