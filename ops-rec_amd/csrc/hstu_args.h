@@ -6,9 +6,12 @@ namespace hstu {
 
 constexpr int kBlockM = 128;  // query rows per workgroup
 constexpr int kWaveM = 32;    // query rows per wavefront
-// resident workgroups per CU of the forward kernel (registers and LDS): three for head dims up to 64 without bias or
-// custom mask (168 registers, 45 KB of LDS), two up to 128, one above
-constexpr int fwd_wgs_per_cu(int d, bool rab, bool mask) { return (d <= 64 && !rab && !mask) ? 3 : (d <= 128 ? 2 : 1); }
+// resident workgroups per CU of the forward kernel (registers and LDS): without bias or custom mask four for the
+// head-dim slot 32 (127 registers, 25 KB of LDS) and three for 64 (168 registers, 45 KB); two up to 128, one above
+constexpr int fwd_wgs_per_cu(int d, bool rab, bool mask)
+{
+    return (!rab && !mask && d <= 64) ? (d <= 32 ? 4 : 3) : (d <= 128 ? 2 : 1);
+}
 constexpr int kCounterBlockBytes = 16384;  // head of the workspace: device-side work counters (see the forward kernel)
 constexpr int kDkvThreads = 256;   // threads of a workgroup of the key-tile backward kernel
 constexpr int kGatherThreads = 128;
