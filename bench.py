@@ -50,10 +50,10 @@ INFINITY_CACHE_BYTES = 256 << 20  # MI355X memory-side cache; a working set belo
 # the forward kernel's source at the time).  A figure whose hash no longer matches the source in the tree is stale
 # and is reported as null.
 MEASURED_TRAFFIC = {
-    "C2": (110_800_000, "profiles/hstu_fwd_bf16_d128_C2_trace_and_counters.md", "cc1c4397874942bc"),
-    "C3": (300_400_000, "profiles/hstu_fwd_bf16_d128_rab_C3_trace_and_counters.md", "cc1c4397874942bc"),
-    "C4": (1_626_200_000, "profiles/hstu_fwd_bf16_d128_rab_C4_trace_and_counters.md", "cc1c4397874942bc"),
-    "C5": (837_400_000, "profiles/hstu_fwd_f8e4m3_d128_C5_trace_and_counters.md", "cc1c4397874942bc"),
+    "C2": (110_900_000, "profiles/hstu_fwd_bf16_d128_C2_trace_and_counters.md", "3c4ead5508d44b99"),
+    "C3": (300_000_000, "profiles/hstu_fwd_bf16_d128_rab_C3_trace_and_counters.md", "3c4ead5508d44b99"),
+    "C4": (1_622_400_000, "profiles/hstu_fwd_bf16_d128_rab_C4_trace_and_counters.md", "3c4ead5508d44b99"),
+    "C5": (841_400_000, "profiles/hstu_fwd_f8e4m3_d128_C5_trace_and_counters.md", "3c4ead5508d44b99"),
 }
 KERNEL_SOURCE = os.path.join(_ROOT, "ops-rec_amd", "csrc", "hstu_fwd_kernel.hip.h")
 
