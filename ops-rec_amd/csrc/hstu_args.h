@@ -6,6 +6,12 @@ namespace hstu {
 
 constexpr int kBlockM = 128;  // query rows per workgroup
 constexpr int kWaveM = 32;    // query rows per wavefront
+// workgroups per CU the backward kernels are compiled for (not persistent: the hardware places as many as fit).  At
+// the head-dim slot 64 a third one fits where the kernel needs no more than 168 registers: the key-tile kernel
+// without bias or custom mask (173 as compiled for two), the query-tile kernel unless it takes both (158 - 167; 180
+// with both); 25 - 33 KB of LDS each.  Measured (bf16, B32 H8 d64 L1024): backward 304 -> 267 us.
+constexpr int bwd_dkv_wgs_per_cu(int d, bool rab, bool mask) { return (!rab && !mask && d <= 64) ? 3 : (d <= 128 ? 2 : 1); }
+constexpr int bwd_dq_wgs_per_cu(int d, bool rab, bool mask) { return (!(rab && mask) && d <= 64) ? 3 : (d <= 128 ? 2 : 1); }
 // resident workgroups per CU of the forward kernel (registers and LDS): without bias or custom mask four for the
 // head-dim slot 32 (127 registers, 25 KB of LDS) and three for 64 (168 registers, 45 KB); two up to 128, one above
 constexpr int fwd_wgs_per_cu(int d, bool rab, bool mask)

@@ -233,7 +233,7 @@ __device__ __forceinline__ void store_tile_rows(uint16_t* stage, const f32x16_t 
 // dQ (and d rab)
 // ---------------------------------------------------------------------------------------------------------
 template <typename Tag, int D, bool HAS_RAB, bool HAS_MASK, bool WANT_DRAB>
-__global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_bwd_dq_kernel(const BwdArgs a)
+__global__ __launch_bounds__(256, bwd_dq_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hstu_bwd_dq_kernel(const BwdArgs a)
 {
     typedef SubTile<D> T;
     constexpr int LPW = T::LPW, NLW = T::NLW, KSTEPS = T::KSTEPS, MTILES = T::MTILES, NCH = 2 * T::MTILES;
@@ -593,7 +593,7 @@ __global__ __launch_bounds__(256, (D <= 128 ? 2 : 1)) void hstu_bwd_dq_kernel(co
 // ---------------------------------------------------------------------------------------------------------
 
 template <typename Tag, int D, bool HAS_RAB, bool HAS_MASK>
-__global__ __launch_bounds__(kDkvThreads, (D <= 128 ? 2 : 1)) void hstu_bwd_dkv_kernel(const BwdArgs a)
+__global__ __launch_bounds__(kDkvThreads, bwd_dkv_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hstu_bwd_dkv_kernel(const BwdArgs a)
 {
     typedef SubTile<D> T;
     constexpr int LPW = T::LPW, NLW = T::NLW, KSTEPS = T::KSTEPS, MTILES = T::MTILES, NCH = 2 * T::MTILES;
