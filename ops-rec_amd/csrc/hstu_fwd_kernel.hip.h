@@ -1,11 +1,13 @@
 // HSTU jagged attention forward for gfx950 (MI355X): device code.
 //
 // Work item = one 128-row query tile of one (sequence, head): four wavefronts of 32 query rows each.
-// The kernel is persistent: a fixed number of workgroups (two per CU) is launched, each builds the
-// work list in its own LDS from seq_offset (sequences bucketed by their number of query tiles,
-// heaviest tiles first, tiles past the end of a sequence never listed) and then pulls item after
-// item from a device-side counter, so that the jagged, causal mix of long and short items is
-// balanced dynamically and the launch / set-up cost of a workgroup is paid once, not per tile.
+// The kernel is persistent: a fixed number of workgroups (fwd_wgs_per_cu: two per CU at head dim 128)
+// is launched, each builds the work list in its own LDS from seq_offset (sequences bucketed by
+// their number of query tiles, heaviest tiles first, tiles past the end of a sequence never
+// listed) and then takes item after item: by a fixed schedule over the list (plain variant: no
+// device counters at all) or from counters in the caller's workspace (per-XCD queues, split items,
+// paged keys), so that the jagged, causal mix of long and short items is balanced and the launch /
+// set-up cost of a workgroup is paid once, not per tile.
 //
 // Per wavefront: its Q rows stay in registers for the whole key sweep of an item; K and V are
 // streamed global -> LDS, 32 keys at a time, by buffer loads that write LDS directly (no register
@@ -23,7 +25,10 @@
 // = 4 consecutive keys) is exactly the B-operand layout the second product needs, so P never
 // leaves registers.  There is no row reduction (no softmax), every output row is produced by
 // one wavefront and stored once: no atomics on data, bitwise deterministic whatever workgroup
-// happens to pull an item.
+// happens to run an item (split items add their parts in part order).
+//
+// fp8-e4m3 inputs run the same structure on v_mfma_f32_32x32x64_f8f6f4, with PV contracting over pairs
+// of sub-tiles (see "fp8 inputs" at the kernel).
 //
 // Out-of-range rows (past the end of a sequence) are never branched on: all global accesses go
 // through buffer descriptors sized to the sequence, whose out-of-range reads return zero and
