@@ -1,8 +1,11 @@
 """The operators under torch.compile (the reference's "graph" tests: torch.compile(op, dynamic=True, fullgraph=True),
-e.g. ascendc/activation/ln_mul/test/pytest/test_ln_mul.py:69-85): tracing needs the schemas, the Meta
-implementations and the autograd formulas to agree with what the kernels return.  The "aot_eager" backend is used:
-it runs dynamo, fake-tensor propagation and AOT autograd exactly as inductor would, and then calls the operators
-themselves (they are opaque to a code generator anyway).  torch.library.opcheck repeats the same checks per operator."""
+e.g. ascendc/activation/ln_mul/test/pytest/test_ln_mul.py:69-85, hstu_forward_v1/test/pytest/test_hstu_jagged.py:1202-1338):
+tracing needs the schemas, the Meta implementations and the autograd formulas to agree with what the kernels return.
+Two backends: the default one, as the reference's tests use it (inductor: it generates the code around the
+operators, which stay opaque calls), and "aot_eager", which runs dynamo, fake-tensor propagation and AOT autograd
+the same way and then calls everything as it is.  The operators' own outputs must be bit-identical to eager under
+both; gradients that pass through arithmetic inductor generates itself (the float losses below) are compared
+bit for bit under aot_eager and to rounding under inductor.  torch.library.opcheck repeats the checks per operator."""
 
 import pytest
 import torch
@@ -14,22 +17,45 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
-def compiled(fn):
-    return torch.compile(fn, backend="aot_eager", fullgraph=True, dynamic=True)
+BACKENDS = ["aot_eager", "inductor"]
 
 
-def test_ln_mul_compiled_matches_eager():
+def compiled(fn, backend):
+    graph = torch.compile(fn, backend=backend, fullgraph=True, dynamic=True)
+    if backend != "inductor":
+        return graph
+
+    def call(*args, **kwargs):
+        # a code generator that cannot build its own kernels on this machine (no compiler, no cache directory) says
+        # nothing about the operators: that is a skip; anything dynamo or the operators raise is a failure
+        try:
+            return graph(*args, **kwargs)
+        except torch._dynamo.exc.BackendCompilerFailed as err:
+            pytest.skip(f"inductor could not generate code here: {str(err)[:200]}")
+
+    return call
+
+
+def same_grad(got, want, backend):
+    if backend == "aot_eager":
+        return torch.equal(got, want)
+    return torch.allclose(got.float(), want.float(), rtol=2e-2, atol=2e-2 * float(want.float().abs().max()))
+
+
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_ln_mul_compiled_matches_eager(backend):
     op = ops_rec.ascendc.activation.ln_mul
-    fn = compiled(op)
+    fn = compiled(op, backend)
     for a, r, dtype in [(8, 64, torch.float32), (33, 512, torch.bfloat16), (5, 100, torch.float32)]:
         x, u = torch.randn(a, r, device=DEV).to(dtype), torch.randn(a, r, device=DEV).to(dtype)
         g, b = torch.randn(r, device=DEV), torch.randn(r, device=DEV)
         assert torch.equal(fn(x=x, u=u, gamma=g, beta=b), op(x, u, g, b))
 
 
-def test_in_linear_silu_compiled_forward_and_backward():
+@pytest.mark.parametrize("backend", BACKENDS)
+def test_in_linear_silu_compiled_forward_and_backward(backend):
     op = ops_rec.ascendc.activation.distance_in_linear_silu
-    fn = compiled(op)
+    fn = compiled(op, backend)
     for m in (100, 257):
         x = torch.randn(m, 64, device=DEV).to(torch.bfloat16)
         w = (torch.randn(512, 64, device=DEV) / 8).to(torch.bfloat16)
@@ -49,18 +75,19 @@ def test_in_linear_silu_compiled_forward_and_backward():
     eager = [t.grad.clone() for t in args]
     for t in args:
         t.grad = None
-    compiled(loss)(*args).backward()
+    compiled(loss, backend)(*args).backward()
     for t, e in zip(args, eager):
-        assert torch.equal(t.grad, e)
+        assert same_grad(t.grad, e, backend)
 
 
+@pytest.mark.parametrize("backend", BACKENDS)
 @pytest.mark.parametrize("kw", [dict(), dict(rab=True, ctx=3, max_target=5, group=1), dict(delta=True)])
-def test_hstu_jagged_compiled_forward_and_backward(kw):
+def test_hstu_jagged_compiled_forward_and_backward(kw, backend):
     w = small_case(seed=3, batch=3, heads=2, dim=64, lo=10, hi=200, dtype=torch.bfloat16, std=0.5, **kw).to(DEV)
     op = ops_rec.ascendc.attention.hstu_jagged
     args = list(w.op_args())
     want = op(*args)
-    got = compiled(lambda *a: op(*a))(*args)
+    got = compiled(lambda *a: op(*a), backend)(*args)
     assert torch.equal(got, want)
 
     def loss(q, k, v):
@@ -73,9 +100,9 @@ def test_hstu_jagged_compiled_forward_and_backward(kw):
     eager = [t.grad.clone() for t in qkv]
     for t in qkv:
         t.grad = None
-    compiled(loss)(*qkv).backward()
+    compiled(loss, backend)(*qkv).backward()
     for t, e in zip(qkv, eager):
-        assert torch.equal(t.grad, e)
+        assert same_grad(t.grad, e, backend)
 
 
 def test_opcheck_of_every_operator():
