@@ -1551,21 +1551,29 @@ __global__ __launch_bounds__(256, fwd_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hst
                     }
                 }
             }
-            // (2) tile requests of this time step
-            if constexpr (K64) {
-                // V(t) and V(t + 1), both in the even steps (their slots held V(t - 4) and V(t - 3), read for the last
-                // time in step t - 1), ahead of K so that the wait after an odd step may leave two K requests open
-                if constexpr (!PAR) {
-                    request_v(std::integral_constant<int, S>{}, t);
-                    request_v(std::integral_constant<int, (S + 1) & 3>{}, t + 1);
+            // (2) tile requests of this time step.  With a 16-bit bias they go out at the end of the step, just ahead of
+            //     the wait, instead of here behind the bias requests (measured: C3 64.3 -> 62.3 us, C4 407 -> 403 us,
+            //     4096-key uniform sequences with bias 447 -> 437 us; without a bias the place makes no difference)
+            constexpr bool kRequestsAtEnd = HAS_RAB && !F8;
+            auto tile_requests = [&]() {
+                if constexpr (K64) {
+                    // V(t) and V(t + 1), both in the even steps (their slots held V(t - 4) and V(t - 3), read for the last
+                    // time in step t - 1), ahead of K so that the wait after an odd step may leave two K requests open
+                    if constexpr (!PAR) {
+                        request_v(std::integral_constant<int, S>{}, t);
+                        request_v(std::integral_constant<int, (S + 1) & 3>{}, t + 1);
+                    }
+                    request_k(sc, t + 4);
+                } else {
+                    request_k(sc, t + 4);
+                    request_v(std::integral_constant<int, (S + 2) & 3>{}, t + 2);
                 }
-                request_k(sc, t + 4);
-            } else {
-                request_k(sc, t + 4);
-                request_v(std::integral_constant<int, (S + 2) & 3>{}, t + 2);
-            }
-            if constexpr (PAGED) {
-                pid_ring[(S + 1) & 3] = page_of(t + 5);  // for the request of K(t + 5) in the next time step
+                if constexpr (PAGED) {
+                    pid_ring[(S + 1) & 3] = page_of(t + 5);  // for the request of K(t + 5) in the next time step
+                }
+            };
+            if constexpr (!kRequestsAtEnd) {
+                tile_requests();
             }
 
             // (3) arithmetic.  Two straight-line blocks, each entered on one wavefront-uniform flag:
@@ -1854,6 +1862,11 @@ __global__ __launch_bounds__(256, fwd_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hst
                         pk_cur[i] = 0u;
                     }
                 }
+            }
+
+            if constexpr (kRequestsAtEnd) {
+                __builtin_amdgcn_sched_barrier(0);
+                tile_requests();
             }
 
             // (4) the requests made two time steps ago have landed (mine), then everybody's
