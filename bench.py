@@ -50,10 +50,10 @@ INFINITY_CACHE_BYTES = 256 << 20  # MI355X memory-side cache; a working set belo
 # the forward kernel's source at the time).  A figure whose hash no longer matches the source in the tree is stale
 # and is reported as null.
 MEASURED_TRAFFIC = {
-    "C2": (110_900_000, "profiles/hstu_fwd_bf16_d128_C2_trace_and_counters.md", "83a97fc254517b61"),
-    "C3": (300_000_000, "profiles/hstu_fwd_bf16_d128_rab_C3_trace_and_counters.md", "83a97fc254517b61"),
-    "C4": (1_622_400_000, "profiles/hstu_fwd_bf16_d128_rab_C4_trace_and_counters.md", "83a97fc254517b61"),
-    "C5": (841_400_000, "profiles/hstu_fwd_f8e4m3_d128_C5_trace_and_counters.md", "83a97fc254517b61"),
+    "C2": (111_200_000, "profiles/hstu_fwd_bf16_d128_C2_trace_and_counters.md", "c3d9640e53904869"),
+    "C3": (298_900_000, "profiles/hstu_fwd_bf16_d128_rab_C3_trace_and_counters.md", "c3d9640e53904869"),
+    "C4": (1_608_700_000, "profiles/hstu_fwd_bf16_d128_rab_C4_trace_and_counters.md", "c3d9640e53904869"),
+    "C5": (842_000_000, "profiles/hstu_fwd_f8e4m3_d128_C5_trace_and_counters.md", "c3d9640e53904869"),
 }
 KERNEL_SOURCE = os.path.join(_ROOT, "ops-rec_amd", "csrc", "hstu_fwd_kernel.hip.h")
 
