@@ -1,4 +1,6 @@
-// forward kernels for fp32 inputs, the kernel for the shapes no tuned kernel takes, and the paged gather kernel
+// forward kernels for fp32 inputs, the forward and backward kernels for the shapes no tuned kernel takes, and the
+// paged gather kernel
+#include "hstu_bwd_generic_kernel.hip.h"
 #include "hstu_fwd_f32_kernel.hip.h"
 #include "hstu_fwd_generic_kernel.hip.h"
 #include "hstu_paged_gather.hip.h"
@@ -25,6 +27,14 @@ const Variant kGeneric[3] = {HSTU_GENERIC_VARIANT(__bf16, "bf16"), HSTU_GENERIC_
                              HSTU_GENERIC_VARIANT(float, "f32")};
 }  // namespace
 const Variant* fwd_variants_generic() { return kGeneric; }
+
+namespace {
+#define HSTU_GENERIC_BWD_VARIANT(T, name) \
+    {"hstu_bwd_generic_" name, hstu_bwd_generic_dkv_kernel<T>, hstu_bwd_generic_dq_kernel<T>, hstu_bwd_generic_dq_kernel<T>}
+const BwdVariant kGenericBwd[3] = {HSTU_GENERIC_BWD_VARIANT(__bf16, "bf16"), HSTU_GENERIC_BWD_VARIANT(_Float16, "f16"),
+                                   HSTU_GENERIC_BWD_VARIANT(float, "f32")};
+}  // namespace
+const BwdVariant* bwd_variants_generic() { return kGenericBwd; }
 
 void launch_paged_gather(const PagedGatherArgs& a, unsigned grid, hipStream_t stream)
 {

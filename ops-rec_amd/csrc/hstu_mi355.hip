@@ -310,26 +310,38 @@ int validate_bwd(const hstu_jagged_bwd_params* p)
     return HSTU_OK;
 }
 
+bool is_generic_bwd(const BwdVariant* v)
+{
+    const BwdVariant* g = hstu::bwd_variants_generic();
+    return v >= g && v < g + 3;
+}
+
+// The tuned kernels take bf16 / fp16 with head dims up to 256, a q/k head dim that is a multiple of 8 and sequences
+// whose rows span less than 1 GiB (32-bit offsets); everything else the reference's backward accepts (fp32, head
+// dims up to 512, any q/k head dim) runs on the generic kernels, which HSTU_MI355_GENERIC_BACKWARD=1 in the
+// environment also selects for inputs the tuned kernels would take (for comparisons).
 const BwdVariant* select_bwd(const hstu_jagged_bwd_params* p)
 {
     const hstu_jagged_fwd_params* f = &p->fwd;
-    if (f->dtype != HSTU_DT_BF16 && f->dtype != HSTU_DT_FP16) {
-        fail(HSTU_ERR_UNSUPPORTED, "the backward is built for bf16 and fp16");
+    if (f->dtype != HSTU_DT_BF16 && f->dtype != HSTU_DT_FP16 && f->dtype != HSTU_DT_FP32) {
+        fail(HSTU_ERR_UNSUPPORTED, "the backward is built for bf16, fp16 and fp32");
         return nullptr;
     }
+    const BwdVariant* generic = &hstu::bwd_variants_generic()[f->dtype == HSTU_DT_BF16 ? 0 : (f->dtype == HSTU_DT_FP16 ? 1 : 2)];
     const int64_t dmax = f->head_dim_qk > f->head_dim_v ? f->head_dim_qk : f->head_dim_v;
-    if (dmax > 256 || f->head_dim_qk % 8 != 0) {
-        fail(HSTU_ERR_UNSUPPORTED, "the backward is built for head dims up to 256, q/k head dim a multiple of 8 (got %lld / %lld)",
-             (long long)f->head_dim_qk, (long long)f->head_dim_v);
-        return nullptr;
+    if (f->dtype == HSTU_DT_FP32 || dmax > 256 || f->head_dim_qk % 8 != 0) {
+        return generic;
     }
     const int64_t span_q = f->max_seq_len_q * f->num_heads_q * dmax * 2;
     const int64_t span_k = f->max_seq_len_k * f->num_heads_k * dmax * 2;
     const int64_t span_b = f->max_seq_len_q * f->max_seq_len_k * 2;
     if (span_q >= (1LL << 30) || span_k >= (1LL << 30) ||
         ((f->attn_bias != nullptr || f->mask_type == HSTU_MASK_CUSTOM) && span_b >= (1LL << 31))) {
-        fail(HSTU_ERR_UNSUPPORTED, "max_seq_len x heads x head dim spans 1 GiB or more per sequence");
-        return nullptr;
+        return generic;
+    }
+    const char* const env = getenv("HSTU_MI355_GENERIC_BACKWARD");
+    if (env != nullptr && env[0] == '1') {
+        return generic;
     }
     const auto* table = f->dtype == HSTU_DT_BF16 ? hstu::bwd_variants_bf16() : hstu::bwd_variants_f16();
     return &table[f->attn_bias != nullptr ? 1 : 0][f->mask_type == HSTU_MASK_CUSTOM ? 1 : 0][dmax <= 64 ? 0 : (dmax <= 128 ? 1 : 2)];
@@ -510,8 +522,9 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
     const hstu_jagged_fwd_params* f = &p->fwd;
     // the attn_bias gradient is written in full: cleared by the key-tile kernel beside its work (or by a fill of
     // its own when that kernel has nothing to run on), then written by the query-tile kernel where its tiles sweep
+    const int64_t es = f->dtype == HSTU_DT_FP32 ? 4 : 2;
     const int64_t drab_bytes = (p->grad_attn_bias != nullptr)
-                                   ? (f->n_offsets - 1) * f->num_heads_q * f->max_seq_len_q * f->max_seq_len_k * 2
+                                   ? (f->n_offsets - 1) * f->num_heads_q * f->max_seq_len_q * f->max_seq_len_k * es
                                    : 0;
     if (f->total_q == 0 && f->total_k == 0) {
         if (drab_bytes > 0) {
@@ -565,19 +578,33 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
     a.alpha = static_cast<float>(f->alpha);
     a.scale = static_cast<float>((f->silu_scale == 0.0) ? 1.0 / static_cast<double>(f->max_seq_len_q) : f->silu_scale);
 
-    const int64_t grid_kv = 2 * static_cast<int64_t>(a.n_ktiles) * a.n_batch * a.n_heads_k;  // a dV and a dK workgroup per tile
+    const bool generic = is_generic_bwd(var);
+    // the tuned key-tile kernel runs a dV and a dK workgroup per tile, the generic one a workgroup per tile
+    const int64_t grid_kv = (generic ? 1 : 2) * static_cast<int64_t>(a.n_ktiles) * a.n_batch * a.n_heads_k;
     const int64_t grid_q = static_cast<int64_t>(a.n_qtiles) * a.n_batch * a.n_heads_q;
     if (grid_kv > 0x7fffffffLL || grid_q > 0x7fffffffLL) {
         return fail(HSTU_ERR_INVALID, "grid out of range");
     }
-    if (f->total_k > 0 && grid_kv > 0) {
+    if (generic) {
+        // the generic kernels write what they compute and nothing else: every output starts from zero
+        launch_clear(p->grad_q, f->total_q * f->num_heads_q * f->head_dim_qk * es, stream);
+        launch_clear(p->grad_k, f->total_k * f->num_heads_k * f->head_dim_qk * es, stream);
+        launch_clear(p->grad_v, f->total_k * f->num_heads_k * f->head_dim_v * es, stream);
+        if (drab_bytes > 0) {
+            launch_clear(p->grad_attn_bias, drab_bytes, stream);
+        }
+        if (f->total_k > 0 && f->total_q > 0 && grid_kv > 0 && grid_q > 0) {
+            hipLaunchKernelGGL(var->dkv, dim3(static_cast<unsigned>(grid_kv)), dim3(256), 0, static_cast<hipStream_t>(stream), a);
+            hipLaunchKernelGGL(var->dq, dim3(static_cast<unsigned>(grid_q)), dim3(256), 0, static_cast<hipStream_t>(stream), a);
+        }
+    } else if (f->total_k > 0 && grid_kv > 0) {
         a.drab_clear_bytes = drab_bytes;
         hipLaunchKernelGGL(var->dkv, dim3(static_cast<unsigned>(grid_kv)), dim3(hstu::kDkvThreads), 0,
                            static_cast<hipStream_t>(stream), a);
     } else if (drab_bytes > 0) {
         launch_clear(p->grad_attn_bias, drab_bytes, stream);
     }
-    if (f->total_q > 0 && grid_q > 0) {
+    if (!generic && f->total_q > 0 && grid_q > 0) {
         hipLaunchKernelGGL(p->grad_attn_bias != nullptr ? var->dq_drab : var->dq, dim3(static_cast<unsigned>(grid_q)), dim3(256),
                            0, static_cast<hipStream_t>(stream), a);
     }

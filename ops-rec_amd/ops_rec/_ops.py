@@ -341,35 +341,13 @@ def hstu_jagged_delta_meta(q, k, v, mask=None, attn_bias=None, mask_type=0, max_
 
 
 # ----------------------------------------------------------------------------------------------
-# backward op: HIP kernels through the C ABI for bf16 / fp16 with head dims up to 256 (_backward_hip); a
-# device-side composite (torch ops on the GPU, per sequence, fp32) for the rest (fp32 inputs, larger head
-# dims), which is also what HSTU_MI355_COMPOSITE_BACKWARD=1 selects for comparisons.
+# backward op: HIP kernels through the C ABI (_backward_hip) -- the tuned MFMA kernels for bf16 / fp16 with head
+# dims up to 256, the library's generic fp32-arithmetic kernels for the rest (fp32 inputs, larger or odd head dims),
+# which HSTU_MI355_GENERIC_BACKWARD=1 in the environment also selects for comparisons.
 #   X = alpha (S + rab),  sig = sigmoid(X),  P = X sig scale M
 #   dV = P^T dO,  dX = (dO V^T) scale M sig (1 + X (1 - sig)),  dS = dRab = alpha dX,  dQ = dS K,  dK = dS^T Q
 # (ascendc/attention/hstu_v1/hstu_backward_v1/op_kernel/vector_score.h:159-205)
 # ----------------------------------------------------------------------------------------------
-
-
-def _device_builtin_mask(s_q, s_k, ctx, tgt, group, device):
-    rows = torch.arange(s_q, device=device)[:, None]
-    cols = torch.arange(s_k, device=device)[None, :]
-    m = cols <= rows + (s_k - s_q)
-    if ctx > 0:
-        m = m | ((rows < ctx) & (cols < s_k - tgt))
-    if tgt > 0 and group > 0:
-        ti = rows - (s_q - tgt)
-        tj = cols - (s_k - tgt)
-        inside = (ti >= 0) & (tj >= 0)
-        blk = (tj <= ti) & (torch.div(ti, group, rounding_mode="floor") == torch.div(tj, group, rounding_mode="floor"))
-        m = torch.where(inside, blk, m)
-    return m
-
-
-def hip_backward_available(q, k, v) -> bool:
-    """Whether the HIP backward kernels cover these tensors (bf16 / fp16, head dims up to 256, q/k head dim a
-    multiple of 8); everything else takes the composite below."""
-    return (q.dtype in (torch.bfloat16, torch.float16) and max(q.shape[2], v.shape[2]) <= 256 and q.shape[2] % 8 == 0
-            and v.shape[2] % 16 == 0)  # fmt: skip
 
 
 def _new_grad(like: torch.Tensor) -> torch.Tensor:
@@ -450,57 +428,10 @@ def _backward_impl(grad, q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max
         _check(num_target is not None, "numTarget is required when numContext or targetGroupSize is not None")
     group = 0 if target_group_size is None else int(target_group_size)
     a = 1.0 if alpha is None else float(alpha)
-    if hip_backward_available(q, k, v) and os.environ.get("HSTU_MI355_COMPOSITE_BACKWARD", "0") != "1":
-        _mask_check(int(mask_type), mask is not None)
-        return _backward_hip(grad, q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max_seq_len_k, silu_scale,
-                             seq_offset, seq_offset_k, num_context, num_target, group, a)  # fmt: skip
-    _check_devices(q.device, (("grad", grad), ("k", k), ("v", v), ("mask", mask), ("attn_bias", attn_bias)))
-    scale = (1.0 / float(max_seq_len_q)) if float(silu_scale) == 0.0 else float(silu_scale)
-    offs_q = seq_offset.tolist()
-    offs_k = seq_offset_k.tolist()
-    ctx = num_context.tolist() if num_context is not None else None
-    tgt = num_target.tolist() if num_target is not None else None
-    n_q, n_k = q.shape[1], k.shape[1]
-    ratio = n_q // n_k
-    f32 = torch.float32
-    dq = torch.zeros(q.shape, dtype=f32, device=q.device)
-    dk = torch.zeros(k.shape, dtype=f32, device=q.device)
-    dv = torch.zeros(v.shape, dtype=f32, device=q.device)
-    dbias = torch.zeros(attn_bias.shape, dtype=f32, device=q.device) if attn_bias is not None else None
-    last = offs_q[-1]
-    batch = offs_q.index(last)
-    for b in range(batch):
-        q0, q1, k0, k1 = offs_q[b], offs_q[b + 1], offs_k[b], offs_k[b + 1]
-        s_q, s_k = q1 - q0, k1 - k0
-        if s_q <= 0 or s_k <= 0:
-            continue
-        qb = q[q0:q1].to(f32).transpose(0, 1)  # [n_q, s_q, d]
-        kb = k[k0:k1].to(f32).transpose(0, 1).repeat_interleave(ratio, dim=0)
-        vb = v[k0:k1].to(f32).transpose(0, 1).repeat_interleave(ratio, dim=0)
-        go = grad[q0:q1].to(f32).transpose(0, 1)  # [n_q, s_q, d_v]
-        s = qb @ kb.transpose(1, 2)
-        if attn_bias is not None:
-            s = s + attn_bias[b, :, :s_q, :s_k].to(f32)
-        x = s * a
-        sig = torch.sigmoid(x)
-        if mask_type == 3:
-            m = mask[b, :, :s_q, :s_k].to(f32)
-        elif mask_type == 0:
-            m = _device_builtin_mask(s_q, s_k, ctx[b] if ctx else 0, tgt[b] if tgt else 0, group, q.device).to(f32)[None]
-        else:
-            m = torch.ones((), dtype=f32, device=q.device)
-        p = x * sig * scale * m
-        dvb = p.transpose(1, 2) @ go  # [n_q, s_k, d_v]
-        dx = (go @ vb.transpose(1, 2)) * scale * m * (sig * (1.0 + x * (1.0 - sig)))
-        ds = dx * a
-        dq[q0:q1] = (ds @ kb).transpose(0, 1)
-        dkb = ds.transpose(1, 2) @ qb  # [n_q, s_k, d]
-        dk[k0:k1] = dkb.reshape(n_k, ratio, s_k, -1).sum(1).transpose(0, 1)
-        dv[k0:k1] = dvb.reshape(n_k, ratio, s_k, -1).sum(1).transpose(0, 1)
-        if dbias is not None:
-            dbias[b, :, :s_q, :s_k] = ds
-    out_bias = dbias.to(attn_bias.dtype) if dbias is not None else None
-    return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype), out_bias
+    _check(q.dtype in (torch.bfloat16, torch.float16, torch.float32), f"q must be bfloat16, float16 or float32, got {q.dtype}")
+    _mask_check(int(mask_type), mask is not None)
+    return _backward_hip(grad, q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max_seq_len_k, silu_scale,
+                         seq_offset, seq_offset_k, num_context, num_target, group, a)  # fmt: skip
 
 
 def hstu_jagged_backward_equal(grad, q, k, v, mask=None, attn_bias=None, mask_type=0, max_seq_len=0, silu_scale=0.0,

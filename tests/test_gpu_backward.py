@@ -5,9 +5,9 @@ Tolerance: the kernels round P and dS to the input type before the products that
 backward does, hstu_backward_v1/op_kernel/vector_score.h:159-205), so a gradient element carries the rounding of a
 sum of up to S products: each gradient tensor must agree with the fp32 oracle within atol = 1e-2 x max|reference|
 and rtol = 1e-2 (bf16) / atol = 2e-3 x max|reference|, rtol = 2e-3 (fp16) -- the forward's 1e-2 bar relative to the
-tensor's scale -- and must not be further from it than 2 x the device-side fp32 composite's own rounding to the
-output type plus that bound.  The same cases run through the composite (HSTU_MI355_COMPOSITE_BACKWARD=1) pin that the
-two device paths agree.
+tensor's scale -- and must not be further from it than 2 x the rounding to the output type of the library's generic
+backward kernels (fp32 arithmetic, P and dS unrounded) plus that bound.  The same cases run through those kernels
+(HSTU_MI355_GENERIC_BACKWARD=1) pin that the two device paths agree.
 """
 
 import dataclasses
@@ -53,10 +53,10 @@ def device_grads(w, grad_out):
 def check(w, monkeypatch, seed=5):
     g = torch.Generator(device=DEV).manual_seed(seed)
     grad_out = torch.randn(w.q.shape[0], w.q.shape[1], w.v.shape[2], generator=g, device=DEV).to(w.q.dtype)
-    monkeypatch.setenv("HSTU_MI355_COMPOSITE_BACKWARD", "0")
+    monkeypatch.setenv("HSTU_MI355_GENERIC_BACKWARD", "0")
     got = device_grads(w, grad_out)
     assert torch.equal(device_grads(w, grad_out)[0], got[0])  # reproducible
-    monkeypatch.setenv("HSTU_MI355_COMPOSITE_BACKWARD", "1")
+    monkeypatch.setenv("HSTU_MI355_GENERIC_BACKWARD", "1")
     comp = device_grads(w, grad_out)
     ref = oracle_grads(w, grad_out)
     tol = 1e-2 if w.q.dtype == torch.bfloat16 else 2e-3
@@ -69,7 +69,7 @@ def check(w, monkeypatch, seed=5):
         assert torch.isfinite(a).all(), name
         scale = r.abs().max().item()
         torch.testing.assert_close(a, r, atol=tol * scale, rtol=tol, msg=lambda m, n=name: f"{n} vs oracle: {m}")
-        torch.testing.assert_close(a, c, atol=tol * scale, rtol=tol, msg=lambda m, n=name: f"{n} vs composite: {m}")
+        torch.testing.assert_close(a, c, atol=tol * scale, rtol=tol, msg=lambda m, n=name: f"{n} vs generic kernels: {m}")
         assert (a - r).abs().max() <= 2 * (c - r).abs().max() + tol * scale, name
 
 
@@ -129,7 +129,7 @@ def test_long_sequences_and_rows_past_the_last_offset(monkeypatch):
     w = dataclasses.replace(w, q=pad(w.q), k=pad(w.k), v=pad(w.v))
     check(w, monkeypatch)
     grad_out = torch.ones(w.q.shape[0], 2, 128, dtype=torch.bfloat16, device=DEV)
-    monkeypatch.setenv("HSTU_MI355_COMPOSITE_BACKWARD", "0")
+    monkeypatch.setenv("HSTU_MI355_GENERIC_BACKWARD", "0")
     dq, dk, dv, _ = device_grads(w, grad_out)
     assert not dq[-40:].any() and not dk[-40:].any() and not dv[-40:].any()
 
@@ -140,7 +140,7 @@ def test_empty_sequences_and_trailing_repeated_offset(monkeypatch):
 
 
 def test_loss_backward_uses_the_kernels(monkeypatch):
-    monkeypatch.setenv("HSTU_MI355_COMPOSITE_BACKWARD", "0")
+    monkeypatch.setenv("HSTU_MI355_GENERIC_BACKWARD", "0")
     w = make(batch=2, heads=2, dim=64, lo=100, hi=200, seed=11, rab_std=0.3)
     q, k, v, bias = (t.clone().requires_grad_(True) for t in (w.q, w.k, w.v, w.attn_bias))
     args = list(w.op_args())
@@ -158,7 +158,7 @@ def test_loss_backward_uses_the_kernels(monkeypatch):
 def test_dense_layout_backward(dtype, dim, use_bias, monkeypatch):
     # hstu_dense / hstu_dense_backward: [B, S, N, D], alpha 1, every sequence of full length
     # (torch_extension/hstu_dense_plugin.cpp:41-151); loss.backward() through the registered autograd as well
-    monkeypatch.setenv("HSTU_MI355_COMPOSITE_BACKWARD", "0")
+    monkeypatch.setenv("HSTU_MI355_GENERIC_BACKWARD", "0")
     batch, seq, heads = 3, 200, 2
     g = torch.Generator().manual_seed(dim)
     mk = lambda *shape, std=0.5: (torch.randn(*shape, generator=g) * std).to(dtype)  # noqa: E731

@@ -66,7 +66,64 @@ def test_rows_past_the_last_offset_are_zero_and_empty_sequences_cost_nothing():
     assert torch.count_nonzero(out[-2:]) == 0
 
 
-def test_backward_falls_to_the_composite_for_these_dims():
+def check_backward(w, seed=3):
+    """dq, dk, dv (and the attn_bias gradient) of the generic backward kernels, through loss.backward(), against
+    autograd on the fp32 oracle: fp32 inputs within 2e-4 of the largest reference value, 16-bit inputs within 1e-2
+    (their gradients are rounded to the input type)."""
+    d = w.to(DEV)
+    q, k, v = (t.clone().requires_grad_() for t in (d.q, d.k, d.v))
+    bias = d.attn_bias.clone().requires_grad_() if d.attn_bias is not None else None
+    args = list(d.op_args())
+    args[0], args[1], args[2], args[4] = q, k, v, bias
+    out = ops_rec.ascendc.attention.hstu_jagged(*args)
+    g = torch.Generator().manual_seed(seed)
+    grad_out = torch.randn(out.shape, generator=g).to(out.dtype)
+    out.backward(grad_out.to(DEV))
+    qc, kc, vc = (t.float().clone().requires_grad_() for t in (w.q, w.k, w.v))
+    kw = w.oracle_kwargs()
+    bc = None
+    if w.attn_bias is not None:
+        bc = w.attn_bias.float().clone().requires_grad_()
+        kw["attn_bias"] = bc
+    O.hstu_jagged_forward(qc, kc, vc, out_dtype=torch.float32, **kw).backward(grad_out.float())
+    tol = 2e-4 if w.q.dtype == torch.float32 else 1e-2
+    pairs = [("dq", q.grad, qc.grad), ("dk", k.grad, kc.grad), ("dv", v.grad, vc.grad)]
+    if bias is not None:
+        pairs.append(("dbias", bias.grad, bc.grad))
+    for name, got, ref in pairs:
+        assert got.dtype == w.q.dtype and got.shape == ref.shape, name
+        assert torch.isfinite(got).all(), name
+        torch.testing.assert_close(got.float().cpu(), ref, rtol=tol, atol=tol * max(1e-3, float(ref.abs().max())),
+                                   msg=lambda m, n=name: f"{n}: {m}")  # fmt: skip
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("dim,dim_v", [(1, 16), (12, 48), (20, 32), (130, 64), (260, 272), (512, 512), (64, 512), (512, 16)])
+def test_backward_at_head_dims_beyond_the_tuned_kernels(dtype, dim, dim_v):
+    check_backward(small_case(seed=dim + dim_v, batch=3, heads=2, dim=dim, dim_v=dim_v, lo=1, hi=90, dtype=dtype, std=0.5))
+
+
+@pytest.mark.parametrize("kw", [
+    dict(), dict(rab=True), dict(custom_mask=True), dict(rab=True, custom_mask=True), dict(ctx=5, max_target=7, group=2),
+    dict(ctx=3, max_target=4, group=1, rab=True), dict(heads=4, heads_k=2), dict(heads=8, heads_k=1, rab=True),
+    dict(delta=True), dict(delta=True, rab=True, index_dtype=torch.int64), dict(alpha=0.3, rab=True),
+    dict(dim=64, dim_v=64), dict(dim=128, dim_v=128, rab=True, hi=300),
+])  # fmt: skip
+def test_backward_of_fp32_inputs_with_all_the_semantics(kw):
+    # fp32 inputs at head dims the tuned forward takes too: the backward runs on the generic kernels all the same
+    base = dict(seed=len(kw) + 23, batch=4, heads=2, dim=32, dim_v=48, lo=20, hi=160, dtype=torch.float32, std=0.5)
+    base.update(kw)
+    check_backward(small_case(**base))
+
+
+def test_backward_without_mask_and_with_rows_past_the_last_offset():
+    w = small_case(seed=9, batch=3, heads=2, dim=24, dim_v=32, lo=1, hi=70, dtype=torch.float32, std=0.5)
+    pad = lambda t: torch.cat([t, torch.ones(3, *t.shape[1:], dtype=t.dtype)])  # noqa: E731
+    w = dataclasses.replace(w, q=pad(w.q), k=pad(w.k), v=pad(w.v), mask_type=2)
+    check_backward(w)
+
+
+def test_backward_runs_on_the_generic_kernels_for_these_dims():
     w = small_case(seed=7, batch=2, heads=2, dim=12, dim_v=16, lo=10, hi=50, dtype=torch.bfloat16, std=0.5).to(DEV)
     q, k, v = (t.clone().requires_grad_() for t in (w.q, w.k, w.v))
     args = list(w.op_args())
