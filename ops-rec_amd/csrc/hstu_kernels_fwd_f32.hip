@@ -1,8 +1,9 @@
-// forward kernels for fp32 inputs, the forward and backward kernels for the shapes no tuned kernel takes, and the
-// paged gather kernel
+// forward kernels for fp32 inputs, for 16-bit inputs with head dims in (256, 512], the forward and backward kernels
+// for the shapes no other kernel takes, and the paged gather kernel
 #include "hstu_bwd_generic_kernel.hip.h"
 #include "hstu_fwd_f32_kernel.hip.h"
 #include "hstu_fwd_generic_kernel.hip.h"
+#include "hstu_fwd_wide_kernel.hip.h"
 #include "hstu_paged_gather.hip.h"
 #include "hstu_variants.h"
 
@@ -27,6 +28,17 @@ const Variant kGeneric[3] = {HSTU_GENERIC_VARIANT(__bf16, "bf16"), HSTU_GENERIC_
                              HSTU_GENERIC_VARIANT(float, "f32")};
 }  // namespace
 const Variant* fwd_variants_generic() { return kGeneric; }
+
+namespace {
+#define HSTU_WIDE_VARIANT(tag, name, RAB, MASK)                                                                          \
+    {"hstu_fwd_wide_" name "_rab" #RAB "_mask" #MASK, nullptr, nullptr, hstu_fwd_wide_kernel<tag, RAB, MASK>, nullptr, nullptr, \
+     nullptr, kWideDim, 256, 0}
+#define HSTU_WIDE_TYPE(tag, name)                                                                       \
+    {{HSTU_WIDE_VARIANT(tag, name, 0, 0), HSTU_WIDE_VARIANT(tag, name, 0, 1)}, \
+     {HSTU_WIDE_VARIANT(tag, name, 1, 0), HSTU_WIDE_VARIANT(tag, name, 1, 1)}}
+const Variant kWide[2][2][2] = {HSTU_WIDE_TYPE(bf16_tag, "bf16"), HSTU_WIDE_TYPE(f16_tag, "f16")};
+}  // namespace
+const Variant (*fwd_variants_wide())[2][2] { return kWide; }
 
 namespace {
 #define HSTU_GENERIC_BWD_VARIANT(T, name) \

@@ -173,6 +173,16 @@ const Variant* select(const hstu_jagged_fwd_params* p)
     const int64_t span_b = p->max_seq_len_q * p->max_seq_len_k * esize;
     const bool wide_span = span_q >= (1LL << 30) || span_k >= (1LL << 30) ||
                            ((p->attn_bias != nullptr || p->mask_type == HSTU_MASK_CUSTOM) && span_b >= (1LL << 31));
+    if ((p->dtype == HSTU_DT_BF16 || p->dtype == HSTU_DT_FP16) && dmax > 256 && p->head_dim_qk % 8 == 0) {
+        // head dims in (256, 512]: the matrix-pipe kernel without the tuned kernel's pipeline (one sequence of one head
+        // group behind a 32-bit descriptor at the padded head dim 512)
+        const int64_t wide_q = p->max_seq_len_q * p->num_heads_q * 512 * 2;
+        const int64_t wide_k = p->max_seq_len_k * p->num_heads_k * 512 * 2;
+        if (wide_q < (1LL << 30) && wide_k < (1LL << 30) && !wide_span) {
+            return &hstu::fwd_variants_wide()[p->dtype == HSTU_DT_BF16 ? 0 : 1][p->attn_bias != nullptr ? 1 : 0]
+                                             [p->mask_type == HSTU_MASK_CUSTOM ? 1 : 0];
+        }
+    }
     if (p->head_dim_qk % 8 != 0 || dmax > 256 || wide_span) {
         if (p->dtype == HSTU_DT_FP8_E4M3) {
             fail(HSTU_ERR_UNSUPPORTED, "fp8 inputs are built for head dims up to 256 (got %lld)", (long long)dmax);

@@ -36,6 +36,8 @@ const Variant (*fwd_variants_f16())[2][4];
 const Variant (*fwd_variants_f8())[2][2][3];
 // forward, fp32 inputs: [rab][custom mask][dim slot: 32, 64, 128, 256]
 const Variant (*fwd_variants_f32())[2][4];
+// forward, 16-bit inputs with head dims in (256, 512], q/k head dim a multiple of 8: [bf16, fp16][rab][custom mask]
+const Variant (*fwd_variants_wide())[2][2];
 // forward, any head dims up to 512 (written for coverage, not speed): [bf16, fp16, fp32]
 const Variant* fwd_variants_generic();
 // backward: [rab][custom mask][dim slot: 64, 128, 256]

@@ -1,6 +1,7 @@
 """Head dims the tuned kernels do not take -- above 256 (the reference goes to 512,
 hstu_forward_v1/op_host/tiling_policy.cpp:68-93) or a q/k head dim that is not a multiple of 8 -- run through the
-kernel written for coverage.  Same oracle, same tolerances as the parity tests (bf16 / fp16: atol = rtol = 1e-2 of
+matrix-pipe kernel for head dims up to 512 (16-bit inputs, q/k head dim a multiple of 8) or the kernel written for
+coverage.  Same oracle, same tolerances as the parity tests (bf16 / fp16: atol = rtol = 1e-2 of
 the largest reference value; fp32: 1e-4)."""
 
 import dataclasses
@@ -17,13 +18,24 @@ pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
 
 
+def expected_kernel(w):
+    """16-bit inputs with a head dim above 256 and a q/k head dim that is a multiple of 8 take the matrix-pipe kernel
+    for head dims up to 512; everything else here takes the kernel written for coverage."""
+    d_qk, d_v = w.q.shape[2], w.v.shape[2]
+    wide = w.q.dtype != torch.float32 and max(d_qk, d_v) > 256 and d_qk % 8 == 0
+    return "hstu_fwd_wide_" if wide else "hstu_fwd_generic_"
+
+
 def check(w, expect_generic=True):
     d = w.to(DEV)
     k_offs = d.seq_offset if d.seq_offset_k is None else d.seq_offset_k
     max_k = d.max_seq_len if d.max_seq_len_k is None else d.max_seq_len_k
     prepared = _ops.prepare_forward(d.q, d.k, d.v, d.mask, d.attn_bias, d.mask_type, d.max_seq_len, max_k, d.silu_scale,
                                     d.seq_offset, k_offs, d.num_context, d.num_target, d.target_group_size, d.alpha)  # fmt: skip
-    assert prepared.kernel_name().startswith("hstu_fwd_generic_") == expect_generic, prepared.kernel_name()
+    if expect_generic:
+        assert prepared.kernel_name().startswith(expected_kernel(w)), prepared.kernel_name()
+    else:
+        assert not prepared.kernel_name().startswith(("hstu_fwd_generic_", "hstu_fwd_wide_")), prepared.kernel_name()
     out = ops_rec.ascendc.attention.hstu_jagged(*d.op_args())
     ref = O.hstu_jagged_forward(w.q, w.k, w.v, out_dtype=torch.float32, **w.oracle_kwargs())
     assert out.dtype == w.q.dtype and out.shape == ref.shape
@@ -49,6 +61,22 @@ def test_all_the_semantics_at_an_odd_head_dim(kw):
     base = dict(seed=len(kw) + 11, batch=4, heads=2, dim=36, dim_v=48, lo=20, hi=160, dtype=torch.bfloat16, std=0.5)
     base.update(kw)
     check(small_case(**base))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("kw", [
+    dict(), dict(rab=True), dict(custom_mask=True), dict(rab=True, custom_mask=True), dict(ctx=5, max_target=7, group=2),
+    dict(ctx=3, max_target=40, group=3, rab=True), dict(heads=4, heads_k=2), dict(heads=8, heads_k=1, rab=True),
+    dict(delta=True), dict(delta=True, rab=True, index_dtype=torch.int64), dict(alpha=0.3, rab=True),
+    dict(dim=264, dim_v=512), dict(dim=512, dim_v=272, rab=True), dict(lo=257, hi=257, rab=True, custom_mask=True),
+])  # fmt: skip
+def test_all_the_semantics_at_head_dims_above_256(kw, dtype):
+    # several 32-key sub-tiles and query tiles per sequence, bias rows of every alignment (lengths are random)
+    base = dict(seed=len(kw) + 31, batch=3, heads=2, dim=320, dim_v=384, lo=90, hi=330, dtype=dtype, std=0.4)
+    base.update(kw)
+    w = small_case(**base)
+    assert expected_kernel(w) == "hstu_fwd_wide_"
+    check(w)
 
 
 def test_no_mask_and_long_rows_at_head_dim_512():
