@@ -305,7 +305,11 @@ def test_kernel_variant_selection():
     assert name(head_dim_qk=12, head_dim_v=16) == "hstu_fwd_generic_bf16"
     assert name(head_dim_qk=1, head_dim_v=512, dtype=_native.DT_FP16, out_dtype=_native.DT_FP16) == "hstu_fwd_generic_f16"
     assert name(head_dim_qk=512, head_dim_v=512, dtype=_native.DT_FP32, out_dtype=_native.DT_FP32) == "hstu_fwd_generic_f32"
-    assert name(head_dim_qk=264, head_dim_v=64, attn_bias=0x2000) == "hstu_fwd_generic_bf16"
+    # 16-bit inputs with a head dim above 256 and a q/k head dim that is a multiple of 8: the matrix-pipe kernel for 512
+    assert name(head_dim_qk=264, head_dim_v=64, attn_bias=0x2000) == "hstu_fwd_wide_bf16_rab1_mask0"
+    assert name(head_dim_qk=64, head_dim_v=512, dtype=_native.DT_FP16, out_dtype=_native.DT_FP16, mask=0x2000,
+                mask_type=3) == "hstu_fwd_wide_f16_rab0_mask1"  # fmt: skip
+    assert name(head_dim_qk=260, head_dim_v=272) == "hstu_fwd_generic_bf16"
 
 
 def test_fp8_variant_selection_and_limits():
