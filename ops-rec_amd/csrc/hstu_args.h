@@ -13,10 +13,11 @@ constexpr int kWaveM = 32;    // query rows per wavefront
 constexpr int bwd_dkv_wgs_per_cu(int d, bool rab, bool mask) { return (!rab && !mask && d <= 64) ? 3 : (d <= 128 ? 2 : 1); }
 constexpr int bwd_dq_wgs_per_cu(int d, bool rab, bool mask) { return (!(rab && mask) && d <= 64) ? 3 : (d <= 128 ? 2 : 1); }
 // resident workgroups per CU of the forward kernel (registers and LDS): without bias or custom mask four for the
-// head-dim slot 32 (127 registers, 25 KB of LDS) and three for 64 (168 registers, 45 KB); two up to 128, one above
+// head-dim slot 32 (127 registers, 25 KB of LDS) and three for 64 (168 registers, 45 KB); three for the slot 32 with
+// either a bias or a custom mask (158 / 151 registers); two up to 128, one above
 constexpr int fwd_wgs_per_cu(int d, bool rab, bool mask)
 {
-    return (!rab && !mask && d <= 64) ? (d <= 32 ? 4 : 3) : (d <= 128 ? 2 : 1);
+    return (!rab && !mask && d <= 64) ? (d <= 32 ? 4 : 3) : (d <= 32 && !(rab && mask)) ? 3 : (d <= 128 ? 2 : 1);
 }
 constexpr int kCounterBlockBytes = 16384;  // head of the workspace: device-side work counters (see the forward kernel)
 constexpr int kDkvThreads = 256;   // threads of a workgroup of the key-tile backward kernel
