@@ -202,6 +202,19 @@ const Variant* select(const hstu_jagged_fwd_params* p)
     return &table[p->attn_bias != nullptr ? 1 : 0][p->mask_type == HSTU_MASK_CUSTOM ? 1 : 0][slot];
 }
 
+// persistent workgroups per CU of a launch: what the variant is compiled for, except that the slot-32 variants with a
+// bias or a custom mask, compiled for three, are launched two per CU when rows are longer than 2048 keys -- there the
+// bias stream is the bound and a third reader per CU costs 3 % (B32 H8 L4096 1351 -> 1391 us), where it is worth
+// 9 % at L1024 (98.5 -> 89.2 us) and 1 % at L2048
+int wgs_per_cu(const Variant* var, const hstu_jagged_fwd_params* p)
+{
+    const bool biased = p->attn_bias != nullptr || p->mask_type == HSTU_MASK_CUSTOM;
+    if (biased && var->d_pad <= 32 && var->persistent_wgs_per_cu == 3 && p->max_seq_len_k > 2048) {
+        return 2;
+    }
+    return var->persistent_wgs_per_cu;
+}
+
 // whether the launch described by p takes the variant with per-XCD work queues: only when the list may hold
 // several items per resident workgroup.  *resident_out (optional) receives the resident grid.
 bool takes_queue_variant(const Variant* var, const hstu_jagged_fwd_params* p, int64_t* resident_out)
@@ -213,7 +226,7 @@ bool takes_queue_variant(const Variant* var, const hstu_jagged_fwd_params* p, in
     if (compute_units(&cus) != HSTU_OK) {
         return false;
     }
-    const int64_t resident = static_cast<int64_t>(cus) * var->persistent_wgs_per_cu;
+    const int64_t resident = static_cast<int64_t>(cus) * wgs_per_cu(var, p);
     if (resident_out != nullptr) {
         *resident_out = resident;
     }
@@ -245,7 +258,7 @@ bool may_take_split_variant(const Variant* var, const hstu_jagged_fwd_params* p,
     if (compute_units(&cus) != HSTU_OK) {
         return false;
     }
-    const int64_t resident = static_cast<int64_t>(cus) * var->persistent_wgs_per_cu;
+    const int64_t resident = static_cast<int64_t>(cus) * wgs_per_cu(var, p);
     if (resident_out != nullptr) {
         *resident_out = resident;
     }
@@ -753,7 +766,7 @@ int launch_forward(const hstu_jagged_fwd_params* p, const hstu_paged_fwd_params*
         if (rc_cu != HSTU_OK) {
             return rc_cu;
         }
-        int64_t resident = static_cast<int64_t>(cus) * var->persistent_wgs_per_cu;
+        int64_t resident = static_cast<int64_t>(cus) * wgs_per_cu(var, p);
         // the variants that pull items from counters need the counter block at the head of the workspace; without
         // it every list runs on the plain variant's fixed schedule
         const bool have_counters = usable_workspace(workspace, workspace_bytes, kCounterBytes);
