@@ -169,8 +169,9 @@ HSTU_API uint64_t hstu_jagged_fwd_noalloc_max_workspace(void);
  *
  * `fwd` describes q, k, v, mask, attn_bias, the offsets and the scalars exactly as for the forward (fwd.out is
  * not used and may be NULL).  bf16 / fp16 with head dims up to 256 and a q/k head dim that is a multiple of 8 run
- * on the tuned kernels; fp32 and every other head dim the forward takes run on generic fp32-arithmetic kernels
- * (correct, slow).  fp8 inputs return HSTU_ERR_UNSUPPORTED.
+ * on the tuned kernels; fp32 with head dims up to 128 and a q/k head dim that is a multiple of 8 runs on kernels
+ * built on the fp32 matrix instruction; every other input the forward takes runs on generic fp32-arithmetic
+ * kernels (correct, slow).  fp8 inputs return HSTU_ERR_UNSUPPORTED.
  * grad_q / grad_k / grad_v: every row is written (rows past the last offset are zero-filled), so the caller
  * need not clear them.  grad_attn_bias (optional; requires attn_bias): written in full as well -- zeros outside
  * the part of a sequence's [S_q, S_k] corner that its query tiles sweep -- so the caller need not clear it either

@@ -28,21 +28,25 @@
 
 namespace hstu {
 
-constexpr int kGenericBwdRows = 16;                    // rows (query rows or keys) of a pass, and of a tile
-constexpr int kGenericBwdStride = kGenericMaxDim + 4;  // floats per staged row: 16-byte reads, rows 4 banks apart
-constexpr int kGenericBwdCols = kGenericMaxDim / 16;   // columns c + 16 j a thread owns
+constexpr int kGenericBwdRows = 16;  // rows (query rows or keys) of a pass, and of a tile
 
-// `rows` rows of `dim` elements, starting at row `row0` of a [*, row_elems] matrix at column `col0`, as floats into
-// `dst` (row stride kGenericBwdStride), zero beyond `n_rows` and up to `dim_padded`
+// The kernels are instantiated for head dims up to MAXD = 128, 256 and 512: the four staged blocks take
+// 4 x 16 x (MAXD + 4) floats of LDS (34 / 67 / 132 KB), so the smaller the bound the more workgroups share a CU and
+// hide each other's load latency (a workgroup waits for its loads at every block: nothing is double-buffered here).
+
+// 16 rows of `dim` elements, starting at row `row0` of a [*, row_elems] matrix at column `col0`, as floats into `dst`
+// (row stride `stride`), zero beyond `n_rows` and up to `dim_padded`; thread t takes row t / 16, columns t % 16 + 16 i
 template <typename T>
-__device__ __forceinline__ void generic_stage_rows(float* dst, const void* src, int64_t first_row, int64_t row_elems,
-                                                   int64_t col0, int row0, int n_rows, int dim, int dim_padded, int tid)
+__device__ __forceinline__ void generic_stage_rows(float* dst, int stride, const void* src, int64_t first_row,
+                                                   int64_t row_elems, int64_t col0, int row0, int n_rows, int dim,
+                                                   int dim_padded, int tid)
 {
-    for (int e = tid; e < kGenericBwdRows * dim_padded; e += 256) {
-        const int rr = e / dim_padded, dd = e - rr * dim_padded;
-        const int row = row0 + rr;
-        dst[rr * kGenericBwdStride + dd] =
-            (row < n_rows && dd < dim) ? generic_load<T>(src, (first_row + row) * row_elems + col0 + dd) : 0.0f;
+    const int rr = tid >> 4;
+    const int row = row0 + rr;
+    const bool in = row < n_rows;
+    const int64_t at = (first_row + row) * row_elems + col0;
+    for (int dd = tid & 15; dd < dim_padded; dd += 16) {
+        dst[rr * stride + dd] = (in && dd < dim) ? generic_load<T>(src, at + dd) : 0.0f;
     }
 }
 
@@ -58,10 +62,10 @@ __device__ __forceinline__ float generic_dot(const float* x, const float* y, int
     return (s4[0] + s4[1]) + (s4[2] + s4[3]);
 }
 
-template <typename T>
+template <typename T, int MAXD>
 __global__ __launch_bounds__(256) void hstu_bwd_generic_dq_kernel(const BwdArgs a)
 {
-    constexpr int RB = kGenericBwdRows, KB = kGenericBwdRows, kStride = kGenericBwdStride;
+    constexpr int RB = kGenericBwdRows, KB = kGenericBwdRows, kStride = MAXD + 4, kCols = MAXD / 16;
     __shared__ __attribute__((aligned(16))) float s_q[RB * kStride];
     __shared__ __attribute__((aligned(16))) float s_g[RB * kStride];
     __shared__ __attribute__((aligned(16))) float s_k[KB * kStride];
@@ -112,18 +116,18 @@ __global__ __launch_bounds__(256) void hstu_bwd_generic_dq_kernel(const BwdArgs 
             kmax = kmax < 0 ? 0 : (kmax > sk ? sk : kmax);
         }
         __syncthreads();  // the previous pass is done with s_q / s_g
-        generic_stage_rows<T>(s_q, a.q, si.q0, q_row_elems, static_cast<int64_t>(h) * a.d_qk, rb, sq, a.d_qk, d_qk4, tid);
-        generic_stage_rows<T>(s_g, a.grad, si.q0, g_row_elems, static_cast<int64_t>(h) * a.d_v, rb, sq, a.d_v, a.d_v, tid);
-        float dq[kGenericBwdCols];
+        generic_stage_rows<T>(s_q, kStride, a.q, si.q0, q_row_elems, static_cast<int64_t>(h) * a.d_qk, rb, sq, a.d_qk, d_qk4, tid);
+        generic_stage_rows<T>(s_g, kStride, a.grad, si.q0, g_row_elems, static_cast<int64_t>(h) * a.d_v, rb, sq, a.d_v, a.d_v, tid);
+        float dq[kCols];
 #pragma unroll
-        for (int j = 0; j < kGenericBwdCols; ++j) {
+        for (int j = 0; j < kCols; ++j) {
             dq[j] = 0.0f;
         }
         for (int kt = 0; kt * KB < kmax; ++kt) {
             const int key0 = kt * KB;
             __syncthreads();  // the previous tile's products are done (and s_q / s_g are written)
-            generic_stage_rows<T>(s_k, a.k, si.k0, k_row_elems, static_cast<int64_t>(hk) * a.d_qk, key0, sk, a.d_qk, d_qk4, tid);
-            generic_stage_rows<T>(s_v, a.v, si.k0, v_row_elems, static_cast<int64_t>(hk) * a.d_v, key0, sk, a.d_v, a.d_v, tid);
+            generic_stage_rows<T>(s_k, kStride, a.k, si.k0, k_row_elems, static_cast<int64_t>(hk) * a.d_qk, key0, sk, a.d_qk, d_qk4, tid);
+            generic_stage_rows<T>(s_v, kStride, a.v, si.k0, v_row_elems, static_cast<int64_t>(hk) * a.d_v, key0, sk, a.d_v, a.d_v, tid);
             __syncthreads();
             const int key = key0 + c;
             float ds = 0.0f;
@@ -152,7 +156,7 @@ __global__ __launch_bounds__(256) void hstu_bwd_generic_dq_kernel(const BwdArgs 
                 dr[cc] = s_ds[r][cc];
             }
 #pragma unroll
-            for (int j = 0; j < kGenericBwdCols; ++j) {
+            for (int j = 0; j < kCols; ++j) {
                 const int col = c + 16 * j;
                 if (col < a.d_qk) {
                     float t = dq[j];
@@ -166,7 +170,7 @@ __global__ __launch_bounds__(256) void hstu_bwd_generic_dq_kernel(const BwdArgs 
         }
         if (row_in) {
 #pragma unroll
-            for (int j = 0; j < kGenericBwdCols; ++j) {
+            for (int j = 0; j < kCols; ++j) {
                 const int col = c + 16 * j;
                 if (col < a.d_qk) {
                     dq_out[(si.q0 + row) * q_row_elems + static_cast<int64_t>(h) * a.d_qk + col] = static_cast<T>(dq[j]);
@@ -176,10 +180,10 @@ __global__ __launch_bounds__(256) void hstu_bwd_generic_dq_kernel(const BwdArgs 
     }
 }
 
-template <typename T>
+template <typename T, int MAXD>
 __global__ __launch_bounds__(256) void hstu_bwd_generic_dkv_kernel(const BwdArgs a)
 {
-    constexpr int RB = kGenericBwdRows, KB = kGenericBwdRows, kStride = kGenericBwdStride;
+    constexpr int RB = kGenericBwdRows, KB = kGenericBwdRows, kStride = MAXD + 4, kCols = MAXD / 16;
     __shared__ __attribute__((aligned(16))) float s_q[RB * kStride];
     __shared__ __attribute__((aligned(16))) float s_g[RB * kStride];
     __shared__ __attribute__((aligned(16))) float s_k[KB * kStride];
@@ -216,11 +220,11 @@ __global__ __launch_bounds__(256) void hstu_bwd_generic_dkv_kernel(const BwdArgs
         const int key = kb + kr;
         const bool key_in = key < sk;
         __syncthreads();  // the previous pass is done with s_k / s_v
-        generic_stage_rows<T>(s_k, a.k, si.k0, k_row_elems, static_cast<int64_t>(hk) * a.d_qk, kb, sk, a.d_qk, d_qk4, tid);
-        generic_stage_rows<T>(s_v, a.v, si.k0, v_row_elems, static_cast<int64_t>(hk) * a.d_v, kb, sk, a.d_v, a.d_v, tid);
-        float dk[kGenericBwdCols], dv[kGenericBwdCols];
+        generic_stage_rows<T>(s_k, kStride, a.k, si.k0, k_row_elems, static_cast<int64_t>(hk) * a.d_qk, kb, sk, a.d_qk, d_qk4, tid);
+        generic_stage_rows<T>(s_v, kStride, a.v, si.k0, v_row_elems, static_cast<int64_t>(hk) * a.d_v, kb, sk, a.d_v, a.d_v, tid);
+        float dk[kCols], dv[kCols];
 #pragma unroll
-        for (int j = 0; j < kGenericBwdCols; ++j) {
+        for (int j = 0; j < kCols; ++j) {
             dk[j] = 0.0f;
             dv[j] = 0.0f;
         }
@@ -235,8 +239,8 @@ __global__ __launch_bounds__(256) void hstu_bwd_generic_dkv_kernel(const BwdArgs
             const int64_t bias_plane = (static_cast<int64_t>(b) * a.n_heads_q + hq) * a.max_q * static_cast<int64_t>(a.max_k);
             for (int rb = row_first; rb < sq; rb += RB) {
                 __syncthreads();  // the previous tile's products are done (and s_k / s_v are written)
-                generic_stage_rows<T>(s_q, a.q, si.q0, q_row_elems, static_cast<int64_t>(hq) * a.d_qk, rb, sq, a.d_qk, d_qk4, tid);
-                generic_stage_rows<T>(s_g, a.grad, si.q0, g_row_elems, static_cast<int64_t>(hq) * a.d_v, rb, sq, a.d_v, a.d_v, tid);
+                generic_stage_rows<T>(s_q, kStride, a.q, si.q0, q_row_elems, static_cast<int64_t>(hq) * a.d_qk, rb, sq, a.d_qk, d_qk4, tid);
+                generic_stage_rows<T>(s_g, kStride, a.grad, si.q0, g_row_elems, static_cast<int64_t>(hq) * a.d_v, rb, sq, a.d_v, a.d_v, tid);
                 __syncthreads();
                 const int row = rb + c;
                 float p = 0.0f, ds = 0.0f;
@@ -267,7 +271,7 @@ __global__ __launch_bounds__(256) void hstu_bwd_generic_dkv_kernel(const BwdArgs
                     dr[cc] = s_ds[kr][cc];
                 }
 #pragma unroll
-                for (int j = 0; j < kGenericBwdCols; ++j) {
+                for (int j = 0; j < kCols; ++j) {
                     const int col = c + 16 * j;
                     if (col < a.d_v) {
                         float t = dv[j];
@@ -290,7 +294,7 @@ __global__ __launch_bounds__(256) void hstu_bwd_generic_dkv_kernel(const BwdArgs
         }
         if (key_in) {
 #pragma unroll
-            for (int j = 0; j < kGenericBwdCols; ++j) {
+            for (int j = 0; j < kCols; ++j) {
                 const int col = c + 16 * j;
                 if (col < a.d_qk) {
                     dk_out[(si.k0 + key) * k_row_elems + static_cast<int64_t>(hk) * a.d_qk + col] = static_cast<T>(dk[j]);

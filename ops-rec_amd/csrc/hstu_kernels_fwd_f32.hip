@@ -1,5 +1,6 @@
 // forward kernels for fp32 inputs, for 16-bit inputs with head dims in (256, 512], the forward and backward kernels
 // for the shapes no other kernel takes, and the paged gather kernel
+#include "hstu_bwd_f32_kernel.hip.h"
 #include "hstu_bwd_generic_kernel.hip.h"
 #include "hstu_fwd_f32_kernel.hip.h"
 #include "hstu_fwd_generic_kernel.hip.h"
@@ -41,12 +42,26 @@ const Variant kWide[2][2][2] = {HSTU_WIDE_TYPE(bf16_tag, "bf16"), HSTU_WIDE_TYPE
 const Variant (*fwd_variants_wide())[2][2] { return kWide; }
 
 namespace {
-#define HSTU_GENERIC_BWD_VARIANT(T, name) \
-    {"hstu_bwd_generic_" name, hstu_bwd_generic_dkv_kernel<T>, hstu_bwd_generic_dq_kernel<T>, hstu_bwd_generic_dq_kernel<T>}
-const BwdVariant kGenericBwd[3] = {HSTU_GENERIC_BWD_VARIANT(__bf16, "bf16"), HSTU_GENERIC_BWD_VARIANT(_Float16, "f16"),
-                                   HSTU_GENERIC_BWD_VARIANT(float, "f32")};
+#define HSTU_GENERIC_BWD_VARIANT(T, name, M)                                                                          \
+    {"hstu_bwd_generic_" name "_d" #M, hstu_bwd_generic_dkv_kernel<T, M>, hstu_bwd_generic_dq_kernel<T, M>, \
+     hstu_bwd_generic_dq_kernel<T, M>}
+#define HSTU_GENERIC_BWD_TYPE(T, name) \
+    {HSTU_GENERIC_BWD_VARIANT(T, name, 128), HSTU_GENERIC_BWD_VARIANT(T, name, 256), HSTU_GENERIC_BWD_VARIANT(T, name, 512)}
+const BwdVariant kGenericBwd[3][3] = {HSTU_GENERIC_BWD_TYPE(__bf16, "bf16"), HSTU_GENERIC_BWD_TYPE(_Float16, "f16"),
+                                      HSTU_GENERIC_BWD_TYPE(float, "f32")};
 }  // namespace
-const BwdVariant* bwd_variants_generic() { return kGenericBwd; }
+const BwdVariant (*bwd_variants_generic())[3] { return kGenericBwd; }
+
+namespace {
+#define HSTU_F32_BWD_VARIANT(D, RAB, MASK)                                                                    \
+    {"hstu_bwd_f32_d" #D "_rab" #RAB "_mask" #MASK, hstu_bwd_f32_dkv_kernel<D, RAB, MASK>, hstu_bwd_f32_dq_kernel<D, RAB, MASK>, \
+     hstu_bwd_f32_dq_kernel<D, RAB, MASK>}
+#define HSTU_F32_BWD_DIMS(RAB, MASK) \
+    {HSTU_F32_BWD_VARIANT(32, RAB, MASK), HSTU_F32_BWD_VARIANT(64, RAB, MASK), HSTU_F32_BWD_VARIANT(128, RAB, MASK)}
+const BwdVariant kF32Bwd[2][2][3] = {{HSTU_F32_BWD_DIMS(0, 0), HSTU_F32_BWD_DIMS(0, 1)},
+                                     {HSTU_F32_BWD_DIMS(1, 0), HSTU_F32_BWD_DIMS(1, 1)}};
+}  // namespace
+const BwdVariant (*bwd_variants_f32())[2][3] { return kF32Bwd; }
 
 void launch_paged_gather(const PagedGatherArgs& a, unsigned grid, hipStream_t stream)
 {

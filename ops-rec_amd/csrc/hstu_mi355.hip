@@ -333,10 +333,12 @@ int validate_bwd(const hstu_jagged_bwd_params* p)
     return HSTU_OK;
 }
 
+// the generic and the fp32 variants: one workgroup per key tile, outputs cleared by fills ahead of the two kernels
 bool is_generic_bwd(const BwdVariant* v)
 {
-    const BwdVariant* g = hstu::bwd_variants_generic();
-    return v >= g && v < g + 3;
+    const BwdVariant* g = &hstu::bwd_variants_generic()[0][0];
+    const BwdVariant* f = &hstu::bwd_variants_f32()[0][0][0];
+    return (v >= g && v < g + 9) || (v >= f && v < f + 12);
 }
 
 // The tuned kernels take bf16 / fp16 with head dims up to 256, a q/k head dim that is a multiple of 8 and sequences
@@ -350,8 +352,22 @@ const BwdVariant* select_bwd(const hstu_jagged_bwd_params* p)
         fail(HSTU_ERR_UNSUPPORTED, "the backward is built for bf16, fp16 and fp32");
         return nullptr;
     }
-    const BwdVariant* generic = &hstu::bwd_variants_generic()[f->dtype == HSTU_DT_BF16 ? 0 : (f->dtype == HSTU_DT_FP16 ? 1 : 2)];
     const int64_t dmax = f->head_dim_qk > f->head_dim_v ? f->head_dim_qk : f->head_dim_v;
+    const BwdVariant* generic = &hstu::bwd_variants_generic()[f->dtype == HSTU_DT_BF16 ? 0 : (f->dtype == HSTU_DT_FP16 ? 1 : 2)]
+                                                             [dmax <= 128 ? 0 : (dmax <= 256 ? 1 : 2)];
+    const char* const env = getenv("HSTU_MI355_GENERIC_BACKWARD");
+    const bool force_generic = env != nullptr && env[0] == '1';
+    if (f->dtype == HSTU_DT_FP32 && dmax <= 128 && f->head_dim_qk % 8 == 0 && !force_generic) {
+        // fp32 MFMA kernels: one sequence of one head group behind a 32-bit descriptor
+        const int64_t sq4 = f->max_seq_len_q * f->num_heads_q * dmax * 4;
+        const int64_t sk4 = f->max_seq_len_k * f->num_heads_k * dmax * 4;
+        const int64_t sb4 = f->max_seq_len_q * f->max_seq_len_k * 4;
+        if (sq4 < (1LL << 30) && sk4 < (1LL << 30) &&
+            !((f->attn_bias != nullptr || f->mask_type == HSTU_MASK_CUSTOM) && sb4 >= (1LL << 31))) {
+            return &hstu::bwd_variants_f32()[f->attn_bias != nullptr ? 1 : 0][f->mask_type == HSTU_MASK_CUSTOM ? 1 : 0]
+                                            [dmax <= 32 ? 0 : (dmax <= 64 ? 1 : 2)];
+        }
+    }
     if (f->dtype == HSTU_DT_FP32 || dmax > 256 || f->head_dim_qk % 8 != 0) {
         return generic;
     }
@@ -362,8 +378,7 @@ const BwdVariant* select_bwd(const hstu_jagged_bwd_params* p)
         ((f->attn_bias != nullptr || f->mask_type == HSTU_MASK_CUSTOM) && span_b >= (1LL << 31))) {
         return generic;
     }
-    const char* const env = getenv("HSTU_MI355_GENERIC_BACKWARD");
-    if (env != nullptr && env[0] == '1') {
+    if (force_generic) {
         return generic;
     }
     const auto* table = f->dtype == HSTU_DT_BF16 ? hstu::bwd_variants_bf16() : hstu::bwd_variants_f16();
@@ -597,6 +612,12 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
     if (a.bias_vec_ok != 0 && reinterpret_cast<uintptr_t>(f->attn_bias) % 16 == 0 && reinterpret_cast<uintptr_t>(f->mask) % 16 == 0 &&
         reinterpret_cast<uintptr_t>(p->grad_attn_bias) % 16 == 0 && f->max_seq_len_k % 8 == 0) {
         a.bias_vec_ok = 2;  // 16-byte aligned rows: the key-tile kernel reads rab / mask rows 16 bytes per lane
+    }
+    if (f->dtype == HSTU_DT_FP32) {  // four fp32 elements = 16 bytes
+        a.bias_vec_ok = (reinterpret_cast<uintptr_t>(f->attn_bias) % 16 == 0 && reinterpret_cast<uintptr_t>(f->mask) % 16 == 0 &&
+                         reinterpret_cast<uintptr_t>(p->grad_attn_bias) % 16 == 0 && f->max_seq_len_k % 4 == 0)
+                            ? 1
+                            : 0;
     }
     a.alpha = static_cast<float>(f->alpha);
     a.scale = static_cast<float>((f->silu_scale == 0.0) ? 1.0 / static_cast<double>(f->max_seq_len_q) : f->silu_scale);

@@ -43,9 +43,12 @@ const Variant* fwd_variants_generic();
 // backward: [rab][custom mask][dim slot: 64, 128, 256]
 const BwdVariant (*bwd_variants_bf16())[2][3];
 const BwdVariant (*bwd_variants_f16())[2][3];
+// backward, fp32 inputs with head dims up to 128 (fp32 MFMA, one workgroup per key tile, the same kernel with and
+// without d rab; launched like the generic ones, behind fills of the outputs): [rab][custom mask][dim slot: 32, 64, 128]
+const BwdVariant (*bwd_variants_f32())[2][3];
 // backward, fp32 inputs and any head dims up to 512 (written for coverage, not speed; one workgroup per key tile,
-// the same kernel with and without d rab): [bf16, fp16, fp32]
-const BwdVariant* bwd_variants_generic();
+// the same kernel with and without d rab): [bf16, fp16, fp32][head dims up to 128, 256, 512]
+const BwdVariant (*bwd_variants_generic())[3];
 // the copy kernel in front of the forward for paged keys that no paged kernel variant covers
 void launch_paged_gather(const PagedGatherArgs& a, unsigned grid, hipStream_t stream);
 

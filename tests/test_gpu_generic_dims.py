@@ -137,9 +137,23 @@ def test_backward_at_head_dims_beyond_the_tuned_kernels(dtype, dim, dim_v):
     dict(delta=True), dict(delta=True, rab=True, index_dtype=torch.int64), dict(alpha=0.3, rab=True),
     dict(dim=64, dim_v=64), dict(dim=128, dim_v=128, rab=True, hi=300),
 ])  # fmt: skip
-def test_backward_of_fp32_inputs_with_all_the_semantics(kw):
-    # fp32 inputs at head dims the tuned forward takes too: the backward runs on the generic kernels all the same
+@pytest.mark.parametrize("generic", ["0", "1"])
+def test_backward_of_fp32_inputs_with_all_the_semantics(kw, generic, monkeypatch):
+    # fp32 inputs with head dims up to 128 and a q/k head dim that is a multiple of 8 run on the fp32 matrix-instruction
+    # backward kernels; HSTU_MI355_GENERIC_BACKWARD=1 sends the same cases through the generic kernels
+    monkeypatch.setenv("HSTU_MI355_GENERIC_BACKWARD", generic)
     base = dict(seed=len(kw) + 23, batch=4, heads=2, dim=32, dim_v=48, lo=20, hi=160, dtype=torch.float32, std=0.5)
+    base.update(kw)
+    check_backward(small_case(**base))
+
+
+@pytest.mark.parametrize("kw", [
+    dict(dim=32, dim_v=32, lo=1, hi=700), dict(dim=64, dim_v=48, lo=100, hi=520, rab=True, custom_mask=True),
+    dict(dim=128, dim_v=128, lo=0, hi=400, ctx=9, max_target=50, group=4), dict(dim=16, dim_v=16, lo=0, hi=260, delta=True, rab=True),
+    dict(dim=8, dim_v=128, lo=127, hi=129, heads=6, heads_k=2, rab=True), dict(dim=104, dim_v=80, lo=255, hi=257, custom_mask=True),
+], ids=lambda kw: "-".join(f"{k}{v}" for k, v in kw.items()))  # fmt: skip
+def test_backward_of_fp32_inputs_over_several_query_and_key_tiles(kw):
+    base = dict(seed=len(kw) + 41, batch=3, heads=2, dtype=torch.float32, std=0.5)
     base.update(kw)
     check_backward(small_case(**base))
 
