@@ -251,7 +251,7 @@ def main() -> int:
                     "attention) on one of the reference's test shapes and on the layer shape of this workload, and "
                     "add an 'in_linear_silu' object with its rooflines to the line")  # fmt: skip
     ap.add_argument("--backward", action="store_true",
-                    help="also time hstu_jagged_backward (the two HIP backward kernels) on the same workload and add a "
+                    help="also time hstu_jagged_backward (the HIP backward kernels) on the same workload and add a "
                     "'backward' object to the line (bf16 workloads only)")  # fmt: skip
     ap.add_argument("--forward-only", action="store_true",
                     help="time the attention forward only; by default (none of --backward / --ln-mul / --in-linear-silu "
@@ -474,9 +474,10 @@ def main() -> int:
             "flops_per_step": bwd_flops,
             "tflops": round(bwd_flops / (bwd_ms * 1e-3) / 1e12, 3),
             "pct_of_bf16_mfma_peak": round(100.0 * bwd_flops / (bwd_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 2),
-            "note": "through torch.ops.ops_rec.hstu_jagged_backward: hstu_bwd_dkv_kernel + hstu_bwd_dq_kernel per step (the "
-            "first also clears the attn_bias gradient when there is one); the kernels recompute S and dP (eight products "
-            "issued for the five of the formula)",
+            "note": "through torch.ops.ops_rec.hstu_jagged_backward: dV workgroups of hstu_bwd_dkv_kernel (which also clear "
+            "the attn_bias gradient when there is one), hstu_bwd_dq_kernel, which leaves dS in that gradient or in a workspace, "
+            "and dK workgroups that read it back (six products issued for the five of the formula); two launches and "
+            "eight products at head dims up to 64 without an attn_bias gradient and for planes above 1 GiB",
         }
 
     if legs["backward"] and not fp8:

@@ -11,6 +11,9 @@ constexpr int kWaveM = 32;    // query rows per wavefront
 // without bias or custom mask (173 as compiled for two), the query-tile kernel unless it takes both (158 - 167; 180
 // with both); 25 - 33 KB of LDS each.  Measured (bf16, B32 H8 d64 L1024): backward 304 -> 267 us.
 constexpr int bwd_dkv_wgs_per_cu(int d, bool rab, bool mask) { return (!rab && !mask && d <= 64) ? 3 : (d <= 128 ? 2 : 1); }
+// the dK workgroups that read dS back from memory keep neither V nor dO nor the score blocks: 90 / 148 / 137 registers
+// and 16 / 32 / 64 KB of LDS at the head-dim slots 64 / 128 / 256
+constexpr int bwd_dk_from_ds_wgs_per_cu(int d) { return d <= 64 ? 4 : (d <= 128 ? 3 : 2); }
 constexpr int bwd_dq_wgs_per_cu(int d, bool rab, bool mask) { return (!(rab && mask) && d <= 64) ? 3 : (d <= 128 ? 2 : 1); }
 // resident workgroups per CU of the forward kernel (registers and LDS): without bias or custom mask four for the
 // head-dim slot 32 (127 registers, 25 KB of LDS) and three for 64 (168 registers, 45 KB); three for the slot 32 with

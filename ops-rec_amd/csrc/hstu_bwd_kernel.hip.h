@@ -592,19 +592,23 @@ __global__ __launch_bounds__(256, bwd_dq_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void 
 // dK, dV
 // ---------------------------------------------------------------------------------------------------------
 
-template <typename Tag, int D, bool HAS_RAB, bool HAS_MASK>
-__global__ __launch_bounds__(kDkvThreads, bwd_dkv_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hstu_bwd_dkv_kernel(const BwdArgs a)
+// MODE 0: a dV and a dK workgroup per key tile (even / odd workgroups).  MODE 1 and 2 serve the three-launch order
+// dV / dQ / dK: all workgroups of a launch have one role, and the dK ones (MODE 2; rab and mask play no part in it)
+// take dS from the attn_bias gradient that the query-tile kernel wrote between the two launches.
+template <typename Tag, int D, bool HAS_RAB, bool HAS_MASK, int MODE = 0>
+__global__ __launch_bounds__(kDkvThreads, MODE == 2 ? bwd_dk_from_ds_wgs_per_cu(D) : bwd_dkv_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hstu_bwd_dkv_kernel(const BwdArgs a)
 {
     typedef SubTile<D> T;
     constexpr int LPW = T::LPW, NLW = T::NLW, KSTEPS = T::KSTEPS, MTILES = T::MTILES, NCH = 2 * T::MTILES;
+    constexpr int kHalves = MODE == 2 ? 1 : 2;  // (the dK workgroups that read dS need no dO)
     // four stages, each the Q sub-tile followed by the dO sub-tile (separate arrays per stage, see the dQ kernel;
     // Q and dO of a stage share an array so that a wavefront can address "the tile of my role" by an offset)
-    __shared__ __attribute__((aligned(1024))) uint16_t s_st0[2 * T::ELEMS];
-    __shared__ __attribute__((aligned(1024))) uint16_t s_st1[2 * T::ELEMS];
-    __shared__ __attribute__((aligned(1024))) uint16_t s_st2[2 * T::ELEMS];
-    __shared__ __attribute__((aligned(1024))) uint16_t s_st3[2 * T::ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_st0[kHalves * T::ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_st1[kHalves * T::ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_st2[kHalves * T::ELEMS];
+    __shared__ __attribute__((aligned(1024))) uint16_t s_st3[kHalves * T::ELEMS];
     // a sub-tile is requested three steps ahead: the requests of two later steps may be outstanding at a step's start
-    constexpr int kReqs = 2 * 2 * LPW;
+    constexpr int kReqs = 2 * kHalves * LPW;
     constexpr int kWaitStage = (kReqs & 15) | (7 << 4) | (15 << 8) | ((kReqs >> 4) << 14);
     constexpr uint32_t kPastEnd = 0x40000000u;
     static_assert(NLW == 4, "every wavefront takes part in the loads");
@@ -614,13 +618,14 @@ __global__ __launch_bounds__(kDkvThreads, bwd_dkv_wgs_per_cu(D, HAS_RAB, HAS_MAS
     const int wave = uniform(tid >> 6);
     // even workgroups produce dV, odd ones dK of the same key tile (neighbours in the grid, so that they tend to
     // run side by side and find each other's Q / dO rows in the L2)
-    const bool dk_role = (blockIdx.x & 1) != 0;
+    constexpr bool from_plane = MODE == 2;
+    const bool dk_role = MODE == 0 ? (blockIdx.x & 1) != 0 : MODE == 2;
     const int ln = lane & 31;
     const int lh = lane >> 5;
 
     // key tile 0 is seen by the most query rows: heaviest first
     const int per_level = a.n_batch * a.n_heads_k;
-    const int tile_slot = static_cast<int>(blockIdx.x >> 1);
+    const int tile_slot = static_cast<int>(MODE == 0 ? blockIdx.x >> 1 : blockIdx.x);
     const int kt_idx = tile_slot / per_level;
     const int rem = tile_slot - kt_idx * per_level;
     const int b = rem / a.n_heads_k;
@@ -629,7 +634,9 @@ __global__ __launch_bounds__(kDkvThreads, bwd_dkv_wgs_per_cu(D, HAS_RAB, HAS_MAS
     zero_tail_rows(a.dv, a.offs_k, a.n_batch, a.idx64, a.total_k, static_cast<int64_t>(a.n_heads_k) * a.d_v, kDkvThreads);
     if (a.drab_clear_bytes > 0) {
         // the attn_bias gradient is cleared here, by all workgroups alike (also those of absent tiles, which leave
-        // below), and written by the query-tile kernel that runs after this one
+        // below), and written by the query-tile kernel that runs after this one.  (Dealing the share out over the
+        // steps of the sweep instead, a few stores per thread and step, was measured slower: stores and tile
+        // requests retire through one in-order counter.)
         clear_share(a.drab, a.drab_clear_bytes, blockIdx.x, gridDim.x, tid, kDkvThreads);
     }
     const SeqInfo si = load_seq(a, b);
@@ -696,7 +703,7 @@ __global__ __launch_bounds__(kDkvThreads, bwd_dkv_wgs_per_cu(D, HAS_RAB, HAS_MAS
         for (int js = 0; js < KSTEPS; ++js) {
             const int d0 = 16 * js + 8 * lh;
             kf[js] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, static_cast<int>(d0 < a.d_qk ? k_off + d0 * 2u : kOutOfRange), 0, 0);
-            vf[js] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, static_cast<int>(dk_role && d0 < a.d_v ? v_off + d0 * 2u : kOutOfRange), 0, 0);
+            vf[js] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, static_cast<int>(dk_role && !from_plane && d0 < a.d_v ? v_off + d0 * 2u : kOutOfRange), 0, 0);
         }
     }
 
@@ -728,7 +735,7 @@ __global__ __launch_bounds__(kDkvThreads, bwd_dkv_wgs_per_cu(D, HAS_RAB, HAS_MAS
     // the transposition (exactly: every product is a value times 1 or 0), and rab lands in the S accumulators.
     const bool vec16 = a.bias_vec_ok == 2;
     u32x4_t route[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
-    if constexpr (HAS_RAB || HAS_MASK) {
+    if constexpr (HAS_RAB || HAS_MASK || from_plane) {
         const uint32_t one = std::is_same<Tag, bf16_tag>::value ? 0x3f80u : 0x3c00u;  // 1.0 in the input type
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
@@ -756,7 +763,9 @@ __global__ __launch_bounds__(kDkvThreads, bwd_dkv_wgs_per_cu(D, HAS_RAB, HAS_MAS
 #pragma unroll
         for (int i = 0; i < LPW; ++i) {
             load_to_lds_b128(q_rsrc, stage + (wave * LPW + i) * 512, q_src[i] + qb);
-            load_to_lds_b128(g_rsrc, stage + T::ELEMS + (wave * LPW + i) * 512, g_src[i] + gb);
+            if constexpr (!from_plane) {
+                load_to_lds_b128(g_rsrc, stage + T::ELEMS + (wave * LPW + i) * 512, g_src[i] + gb);
+            }
         }
         ++req_it;
         if (++req_x >= n_qsub) {
@@ -809,7 +818,25 @@ __global__ __launch_bounds__(kDkvThreads, bwd_dkv_wgs_per_cu(D, HAS_RAB, HAS_MAS
         // cw0 + 16 j + 8 lh .. + 7 (whole chunks are in or out of the row: max_seq_len_k is a multiple of 8 here).
         u32x4_t ra[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
         u32x4_t ma[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
-        if constexpr (HAS_RAB || HAS_MASK) {
+        if constexpr (from_plane) {
+            // dS rows of this step, as the query-tile kernel stored them (rounded to the input type, masked): read
+            // like rab rows and transposed by the same routing products.  Only what that kernel wrote is read -- whole
+            // 16-byte pieces that start ahead of the sequence's last key, in the 32 x 32 blocks that it swept, which
+            // are the blocks `active` here -- so the plane need not be cleared when it is a workspace.
+            if (active) {
+                const __amdgpu_buffer_rsrc_t ds_rsrc = make_rsrc(
+                    static_cast<const uint16_t*>(a.drab) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k),
+                    bias_bytes);
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int key0 = cw0 + 16 * j + 8 * lh;
+                    const uint32_t off = (rq0 + ln < sq && key0 < sk)
+                                             ? (static_cast<uint32_t>(rq0 + ln) * static_cast<uint32_t>(a.max_k) + static_cast<uint32_t>(key0)) * 2u
+                                             : kOutOfRange;
+                    ra[j] = __builtin_amdgcn_raw_buffer_load_b128(ds_rsrc, static_cast<int>(off), 0, 0);
+                }
+            }
+        } else if constexpr (HAS_RAB || HAS_MASK) {
             if (vec16 && active) {
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
@@ -829,7 +856,28 @@ __global__ __launch_bounds__(kDkvThreads, bwd_dkv_wgs_per_cu(D, HAS_RAB, HAS_MAS
         __builtin_amdgcn_sched_barrier(0);
         request(stage_o);
         __builtin_amdgcn_sched_barrier(0);
-        if (active) {
+        if constexpr (from_plane) {
+          if (active) {
+            f32x16_t s;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                s[i] = 0.f;
+            }
+            s = mfma32<Tag>(ra[0], route[0], s);
+            s = mfma32<Tag>(ra[1], route[1], s);
+            uint32_t pk[8];
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                pk[i] = pack2<Tag>(s[2 * i], s[2 * i + 1]);  // (exact: the values are of the input type)
+            }
+#pragma unroll
+            for (int c = 0; c < NCH; ++c) {
+                const int j2 = c / MTILES, mt = c % MTILES;
+                const u32x4_t pb = {pk[4 * j2 + 0], pk[4 * j2 + 1], pk[4 * j2 + 2], pk[4 * j2 + 3]};
+                acc[mt] = mfma32<Tag>(read_t(stage, c), pb, acc[mt]);
+            }
+          }
+        } else if (active) {
             f32x16_t s, dp;
 #pragma unroll
             for (int i = 0; i < 16; ++i) {

@@ -4,18 +4,10 @@
 
 namespace hstu {
 namespace {
-template <typename Tag, int D, bool RAB, bool MASK>
-constexpr auto dq_drab_kernel() -> void (*)(const BwdArgs)
-{
-    if constexpr (RAB) {
-        return hstu_bwd_dq_kernel<Tag, D, RAB, MASK, true>;
-    } else {
-        return nullptr;
-    }
-}
 #define HSTU_BWD_VARIANT(D, RAB, MASK)                                                        \
     {"hstu_bwd_f16_d" #D "_rab" #RAB "_mask" #MASK, hstu_bwd_dkv_kernel<f16_tag, D, RAB, MASK>, \
-     hstu_bwd_dq_kernel<f16_tag, D, RAB, MASK, false>, dq_drab_kernel<f16_tag, D, RAB, MASK>()}
+     hstu_bwd_dq_kernel<f16_tag, D, RAB, MASK, false>, hstu_bwd_dq_kernel<f16_tag, D, RAB, MASK, true>, \
+     hstu_bwd_dkv_kernel<f16_tag, D, RAB, MASK, 1>, hstu_bwd_dkv_kernel<f16_tag, D, false, false, 2>}
 #define HSTU_BWD_DIMS(RAB, MASK) {HSTU_BWD_VARIANT(64, RAB, MASK), HSTU_BWD_VARIANT(128, RAB, MASK), HSTU_BWD_VARIANT(256, RAB, MASK)}
 const BwdVariant kTable[2][2][3] = {{HSTU_BWD_DIMS(false, false), HSTU_BWD_DIMS(false, true)},
                                     {HSTU_BWD_DIMS(true, false), HSTU_BWD_DIMS(true, true)}};

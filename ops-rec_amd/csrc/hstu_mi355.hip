@@ -532,6 +532,69 @@ HSTU_API int hstu_paged_fwd(const hstu_paged_fwd_params* p, void* workspace, uin
     return launch_forward(&g, nullptr, static_cast<char*>(workspace) + used, workspace_bytes > used ? workspace_bytes - used : 0, stream);
 }
 
+// The tuned kernels recompute S, dP and dS in the dK workgroups (two launches: dV and dK workgroups side by side, then
+// the query-tile kernel) unless the query-tile kernel's dS is kept: then the order is dV workgroups, query-tile
+// kernel, dK workgroups that read dS back (six matrix products instead of eight).  dS is the attn_bias gradient when
+// that is asked for; otherwise it goes into a workspace of the same shape, [batch, heads, max_seq_len_q,
+// max_seq_len_k] in the input type, as far as hstu_jagged_bwd_workspace_size asks for one.  Rows of 16 bytes are
+// needed either way (max_seq_len_k a multiple of 8, 16-byte aligned planes).
+//
+// Three launches in a row have three tails and hide the clearing of the attn_bias gradient behind less arithmetic,
+// so the order is chosen by what was measured (bf16, two launches -> three):
+//   through the workspace (4 bytes of traffic per pair against 8 x head dim flops saved): head dims above 64 and
+//     max_seq_len_k up to 2048 -- C2 162 -> 144 us, B16 H4 d256 L1024 317 -> 227 us, B64 H4 d128 L256..1024
+//     272 -> 242 us, B16 H4 d128 L512..2048 240 -> 230 us; not at head dims up to 64 (B32 H8 d64 L1024 278 -> 300 us)
+//     nor for longer rows (B4 H8 d128 L1024..4096 410 -> 528 us, B2 H4 d128 L8192 747 -> 947 us); planes up to 1 GiB
+//     (HSTU_MI355_BWD_WORKSPACE_MB in the environment moves that limit);
+//   through the attn_bias gradient: head dims above 128 (B16 H4 d256 L100..1504 501 -> 404 us), max_seq_len_k up to
+//     1024 (B64 H4 d128 L256..1024 431 -> 382 us, B128 H4 d64 L64..512 177 -> 146 us) and batches without padding,
+//     total_q = batch x max_seq_len_q (B32 H8 d128 L2048 2599 -> 2311 us, B32 H8 d32 L4096 8013 -> 6810 us); not for
+//     long jagged batches (B32 H4 d64 L100..1504 310 -> 341 us, B8 H8 d128 L1024..4096 1492 -> 1657 us; C3 396 -> 401 us).
+// HSTU_MI355_BWD_HANDOFF in the environment overrides the choice: 0 = two launches, 1 = three wherever possible.
+static int handoff_policy()  // 0: never, 1: wherever possible, 2: by the rule above
+{
+    const char* const env = getenv("HSTU_MI355_BWD_HANDOFF");
+    return env == nullptr ? 2 : (env[0] == '0' ? 0 : 1);
+}
+
+static int64_t ds_plane_bytes(const hstu_jagged_fwd_params* f)
+{
+    return (f->n_offsets - 1) * f->num_heads_q * f->max_seq_len_q * f->max_seq_len_k * 2;
+}
+
+// dS handed over through the attn_bias gradient
+static bool hands_over_through_gradient(const hstu_jagged_bwd_params* p, const BwdVariant* var)
+{
+    const hstu_jagged_fwd_params* f = &p->fwd;
+    const int policy = handoff_policy();
+    if (var->dk_from_ds == nullptr || p->grad_attn_bias == nullptr || policy == 0) {
+        return false;
+    }
+    const int64_t dmax = f->head_dim_qk > f->head_dim_v ? f->head_dim_qk : f->head_dim_v;
+    return policy == 1 || dmax > 128 || f->max_seq_len_k <= 1024 || f->total_q == (f->n_offsets - 1) * f->max_seq_len_q;
+}
+
+// bytes of the workspace through which dS is handed over when there is no attn_bias gradient (0: two launches)
+static uint64_t ds_workspace_bytes(const hstu_jagged_bwd_params* p, const BwdVariant* var)
+{
+    const hstu_jagged_fwd_params* f = &p->fwd;
+    const int policy = handoff_policy();
+    if (var->dk_from_ds == nullptr || p->grad_attn_bias != nullptr || f->max_seq_len_k % 8 != 0 || policy == 0 ||
+        f->total_q == 0 || f->total_k == 0) {
+        return 0;
+    }
+    const int64_t dmax = f->head_dim_qk > f->head_dim_v ? f->head_dim_qk : f->head_dim_v;
+    if (policy != 1 && (dmax <= 64 || f->max_seq_len_k > 2048)) {
+        return 0;
+    }
+    int64_t cap_mb = 1024;
+    if (const char* const env = getenv("HSTU_MI355_BWD_WORKSPACE_MB")) {
+        cap_mb = atoll(env);
+    }
+    const int64_t bytes = ds_plane_bytes(f);
+    return bytes <= cap_mb * (1LL << 20) ? static_cast<uint64_t>(bytes) : 0;
+}
+
 HSTU_API int hstu_jagged_bwd_workspace_size(const hstu_jagged_bwd_params* params, uint64_t* workspace_bytes)
 {
     if (workspace_bytes == nullptr) {
@@ -542,13 +605,16 @@ HSTU_API int hstu_jagged_bwd_workspace_size(const hstu_jagged_bwd_params* params
     if (rc != HSTU_OK) {
         return rc;
     }
-    return select_bwd(params) == nullptr ? HSTU_ERR_UNSUPPORTED : HSTU_OK;
+    const BwdVariant* var = select_bwd(params);
+    if (var == nullptr) {
+        return HSTU_ERR_UNSUPPORTED;
+    }
+    *workspace_bytes = ds_workspace_bytes(params, var);
+    return HSTU_OK;
 }
 
 HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, uint64_t workspace_bytes, void* stream)
 {
-    (void)workspace;
-    (void)workspace_bytes;
     const int rc = validate_bwd(p);
     if (rc != HSTU_OK) {
         return rc;
@@ -641,6 +707,28 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
             hipLaunchKernelGGL(var->dkv, dim3(static_cast<unsigned>(grid_kv)), dim3(256), 0, static_cast<hipStream_t>(stream), a);
             hipLaunchKernelGGL(var->dq, dim3(static_cast<unsigned>(grid_q)), dim3(256), 0, static_cast<hipStream_t>(stream), a);
         }
+    } else if (f->total_k > 0 && grid_kv > 0 && f->total_q > 0 && grid_q > 0 && a.bias_vec_ok == 2 &&
+               (hands_over_through_gradient(p, var) ||
+                (ds_workspace_bytes(p, var) > 0 && usable_workspace(workspace, workspace_bytes, ds_workspace_bytes(p, var)) &&
+                 reinterpret_cast<uintptr_t>(workspace) % 16 == 0))) {
+        // dV workgroups (which clear the attn_bias gradient beside their work), the query-tile kernel (which writes
+        // dS into it, or into the workspace, where nothing needs clearing: the dK workgroups read what was written),
+        // dK workgroups (which read dS back instead of computing S, dP and dS a second time)
+        if (p->grad_attn_bias == nullptr) {
+            a.drab = workspace;
+        }
+        a.drab_clear_bytes = drab_bytes;
+        hipLaunchKernelGGL(var->dv_only, dim3(static_cast<unsigned>(grid_kv / 2)), dim3(hstu::kDkvThreads), 0,
+                           static_cast<hipStream_t>(stream), a);
+        a.drab_clear_bytes = 0;
+        hipLaunchKernelGGL(var->dq_drab, dim3(static_cast<unsigned>(grid_q)), dim3(256), 0, static_cast<hipStream_t>(stream), a);
+        hipLaunchKernelGGL(var->dk_from_ds, dim3(static_cast<unsigned>(grid_kv / 2)), dim3(hstu::kDkvThreads), 0,
+                           static_cast<hipStream_t>(stream), a);
+        const hipError_t err3 = hipGetLastError();
+        if (err3 != hipSuccess) {
+            return fail(HSTU_ERR_RUNTIME, "launch of %s failed: %s", var->name, hipGetErrorString(err3));
+        }
+        return HSTU_OK;
     } else if (f->total_k > 0 && grid_kv > 0) {
         a.drab_clear_bytes = drab_bytes;
         hipLaunchKernelGGL(var->dkv, dim3(static_cast<unsigned>(grid_kv)), dim3(hstu::kDkvThreads), 0,

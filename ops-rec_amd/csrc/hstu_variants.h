@@ -26,7 +26,10 @@ struct BwdVariant {
     const char* name;
     void (*dkv)(const BwdArgs);
     void (*dq)(const BwdArgs);       // without d rab
-    void (*dq_drab)(const BwdArgs);  // with d rab (nullptr when the variant has no rab)
+    void (*dq_drab)(const BwdArgs);  // storing dS (the attn_bias gradient) as well; nullptr in the generic and fp32 tables
+    // the three-launch order dV / dQ storing dS / dK from that dS (nullptr in the generic and fp32 tables)
+    void (*dv_only)(const BwdArgs);
+    void (*dk_from_ds)(const BwdArgs);
 };
 
 // forward, 16-bit inputs: [rab: 0, 1][custom mask: 0, 1][dim slot: 32, 64, 128, 256]

@@ -410,6 +410,8 @@ def _backward_hip(grad, q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max_
     if rc != _native.HSTU_OK:
         raise RuntimeError(f"hstu_jagged_bwd_workspace_size failed ({rc}): {_native.last_error()}")
     ws = torch.empty(ws_bytes.value, dtype=torch.uint8, device=q_c.device) if ws_bytes.value else None
+    if ws is not None and os.environ.get("HSTU_MI355_POISON_WORKSPACE") == "1":
+        ws.fill_(0xFF)  # (for tests: NaN in every element, so that a read of something never written shows)
     stream = torch.cuda.current_stream(q_c.device).cuda_stream
     rc = lib.hstu_jagged_bwd(ctypes.byref(p), _ptr(ws), ws_bytes.value, ctypes.c_void_p(stream))
     if rc != _native.HSTU_OK:

@@ -54,6 +54,9 @@ def check(w, monkeypatch, seed=5):
     g = torch.Generator(device=DEV).manual_seed(seed)
     grad_out = torch.randn(w.q.shape[0], w.q.shape[1], w.v.shape[2], generator=g, device=DEV).to(w.q.dtype)
     monkeypatch.setenv("HSTU_MI355_GENERIC_BACKWARD", "0")
+    # the workspace in which the query-tile kernel leaves dS for the dK workgroups is not cleared: filled with NaN
+    # here, so that a read of an element that was never written would show in dk
+    monkeypatch.setenv("HSTU_MI355_POISON_WORKSPACE", "1")
     got = device_grads(w, grad_out)
     assert torch.equal(device_grads(w, grad_out)[0], got[0])  # reproducible
     monkeypatch.setenv("HSTU_MI355_GENERIC_BACKWARD", "1")
@@ -100,6 +103,74 @@ def test_custom_mask_and_rab_alignment(max_len, monkeypatch):
     g = torch.Generator(device=DEV).manual_seed(1)
     mask = (torch.rand(2, 2, max_len, max_len, generator=g, device=DEV) < 0.6).to(torch.float16)
     check(dataclasses.replace(w, mask=mask, mask_type=3), monkeypatch)
+
+
+@pytest.mark.parametrize("kw", [
+    dict(dim=64, lo=260, hi=424, max_seq_len=424), dict(dim=128, lo=1, hi=520, max_seq_len=520, heads=4, heads_k=2),
+    dict(dim=256, lo=100, hi=264, max_seq_len=264), dict(dim=64, lo=200, hi=400, max_seq_len=400, num_context=6, max_target=30, target_group_size=3),
+    dict(dim=128, dim_v=64, lo=0, hi=296, max_seq_len=296, dtype=torch.float16), dict(dim=32, lo=300, hi=1200, max_seq_len=1200),
+], ids=lambda kw: "-".join(f"{k}{v}" for k, v in kw.items() if k != "dtype"))  # fmt: skip
+@pytest.mark.parametrize("custom_mask", [False, True], ids=["causal", "custom"])
+def test_attn_bias_gradient_handed_to_the_dk_workgroups(kw, custom_mask, monkeypatch):
+    """With the attn_bias gradient asked for and 16-byte aligned bias rows the library runs dV workgroups, the
+    query-tile kernel and then dK workgroups that read dS back from the attn_bias gradient;
+    HSTU_MI355_BWD_HANDOFF=0 keeps the order in which the dK workgroups recompute it.  dq, dv and the bias gradient
+    come from the same arithmetic in both orders (bit-identical), dk from dS rounded at the same point."""
+    kw = dict(kw)
+    w = make(batch=3, heads=kw.pop("heads", 2), seed=len(kw) + 50, rab_std=0.5, **kw)
+    assert w.max_seq_len % 8 == 0
+    if custom_mask:
+        g = torch.Generator(device=DEV).manual_seed(2)
+        shape = (3, w.q.shape[1], w.max_seq_len, w.max_seq_len)
+        mask = (torch.rand(shape, generator=g, device=DEV) < 0.7).to(w.q.dtype)
+        w = dataclasses.replace(w, mask=mask, mask_type=3, num_context=None, num_target=None, target_group_size=0)
+    check(w, monkeypatch)
+    g = torch.Generator(device=DEV).manual_seed(6)
+    grad_out = torch.randn(w.q.shape[0], w.q.shape[1], w.v.shape[2], generator=g, device=DEV).to(w.q.dtype)
+    monkeypatch.setenv("HSTU_MI355_GENERIC_BACKWARD", "0")
+    monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "0")
+    two = device_grads(w, grad_out)
+    monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "1")
+    three = device_grads(w, grad_out)
+    for name, i in (("dq", 0), ("dv", 2), ("dbias", 3)):
+        assert torch.equal(two[i], three[i]), name
+    scale = two[1].float().abs().max().item()
+    tol = 1e-2 if w.q.dtype == torch.bfloat16 else 2e-3
+    torch.testing.assert_close(three[1].float(), two[1].float(), atol=tol * scale, rtol=tol)
+
+
+@pytest.mark.parametrize("kw", [
+    dict(dim=128, lo=1, hi=520, max_seq_len=520, heads=4, heads_k=2), dict(dim=256, lo=100, hi=264, max_seq_len=264),
+    dict(dim=128, lo=200, hi=400, max_seq_len=400, num_context=6, max_target=30, target_group_size=3),
+    dict(dim=128, lo=0, hi=296, max_seq_len=296, num_context=40, max_target=9, target_group_size=1, dtype=torch.float16),
+    dict(dim=72, dim_v=128, lo=300, hi=1200, max_seq_len=1200), dict(dim=128, lo=33, hi=33, max_seq_len=40),
+], ids=lambda kw: "-".join(f"{k}{v}" for k, v in kw.items() if k != "dtype"))  # fmt: skip
+@pytest.mark.parametrize("mask", ["causal", "custom", "none"])
+def test_ds_handed_to_the_dk_workgroups_through_a_workspace(kw, mask, monkeypatch):
+    """Without an attn_bias gradient, head dims above 64 and max_seq_len_k a multiple of 8, the query-tile kernel
+    leaves dS in a workspace for the dK workgroups (hstu_jagged_bwd_workspace_size asks for it).  Checked against
+    the oracle and the generic kernels with the workspace full of NaN, and against the two-launch order."""
+    kw = dict(kw)
+    w = make(batch=3, heads=kw.pop("heads", 2), seed=len(kw) + 60, **kw)
+    if mask == "custom":
+        g = torch.Generator(device=DEV).manual_seed(2)
+        shape = (3, w.q.shape[1], w.max_seq_len, w.max_seq_len)
+        m = (torch.rand(shape, generator=g, device=DEV) < 0.7).to(w.q.dtype)
+        w = dataclasses.replace(w, mask=m, mask_type=3, num_context=None, num_target=None, target_group_size=0)
+    elif mask == "none":
+        w = dataclasses.replace(w, mask_type=2, num_context=None, num_target=None, target_group_size=0)
+    check(w, monkeypatch)
+    g = torch.Generator(device=DEV).manual_seed(6)
+    grad_out = torch.randn(w.q.shape[0], w.q.shape[1], w.v.shape[2], generator=g, device=DEV).to(w.q.dtype)
+    monkeypatch.setenv("HSTU_MI355_GENERIC_BACKWARD", "0")
+    monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "0")
+    two = device_grads(w, grad_out)
+    monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "1")
+    three = device_grads(w, grad_out)
+    assert torch.equal(two[0], three[0]) and torch.equal(two[2], three[2])  # dq and dv: the same arithmetic
+    scale = two[1].float().abs().max().item()
+    tol = 1e-2 if w.q.dtype == torch.bfloat16 else 2e-3
+    torch.testing.assert_close(three[1].float(), two[1].float(), atol=tol * scale, rtol=tol)
 
 
 def test_no_mask(monkeypatch):
