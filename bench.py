@@ -477,7 +477,7 @@ def main() -> int:
             "note": "through torch.ops.ops_rec.hstu_jagged_backward: dV workgroups of hstu_bwd_dkv_kernel (which also clear "
             "the attn_bias gradient when there is one), hstu_bwd_dq_kernel, which leaves dS in that gradient or in a workspace, "
             "and dK workgroups that read it back (six products issued for the five of the formula); two launches and "
-            "eight products at head dims up to 64 without an attn_bias gradient and for planes above 1 GiB",
+            "eight products at head dims up to 64 without an attn_bias gradient and for planes above 4 GiB",
         }
 
     if legs["backward"] and not fp8:

@@ -180,7 +180,7 @@ HSTU_API uint64_t hstu_jagged_fwd_noalloc_max_workspace(void);
  * then grad_k from that dS -- when dS has somewhere to stay: in grad_attn_bias (which is dS) when that is asked
  * for, otherwise in a workspace of [batch, num_heads_q, max_seq_len_q, max_seq_len_k] elements of the input
  * type, which hstu_jagged_bwd_workspace_size asks for when it pays (head dims above 64, max_seq_len_k a multiple
- * of 8, at most 1 GiB or HSTU_MI355_BWD_WORKSPACE_MB in the environment).  Without the workspace, or with less
+ * of 8, at most 4 GiB or HSTU_MI355_BWD_WORKSPACE_MB in the environment).  Without the workspace, or with less
  * than was asked for, the call still works: two launches in which the grad_k workgroups recompute dS.  The
  * workspace needs no clearing and holds nothing afterwards. */
 typedef struct hstu_jagged_bwd_params {

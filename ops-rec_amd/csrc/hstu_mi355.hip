@@ -544,8 +544,9 @@ HSTU_API int hstu_paged_fwd(const hstu_paged_fwd_params* p, void* workspace, uin
 //   through the workspace (4 bytes of traffic per pair against 8 x head dim flops saved): head dims above 64 and
 //     max_seq_len_k up to 2048 -- C2 162 -> 144 us, B16 H4 d256 L1024 317 -> 227 us, B64 H4 d128 L256..1024
 //     272 -> 242 us, B16 H4 d128 L512..2048 240 -> 230 us; not at head dims up to 64 (B32 H8 d64 L1024 278 -> 300 us)
-//     nor for longer rows (B4 H8 d128 L1024..4096 410 -> 528 us, B2 H4 d128 L8192 747 -> 947 us); planes up to 1 GiB
-//     (HSTU_MI355_BWD_WORKSPACE_MB in the environment moves that limit);
+//     nor for longer rows (B4 H8 d128 L1024..4096 410 -> 528 us, B2 H4 d128 L8192 747 -> 947 us); planes up to 4 GiB
+//     (B32 H8 d256 L2048 4310 -> 3009 us, d128 1566 -> 1512 us; HSTU_MI355_BWD_WORKSPACE_MB in the environment moves
+//     that limit);
 //   through the attn_bias gradient: head dims above 128 (B16 H4 d256 L100..1504 501 -> 404 us), max_seq_len_k up to
 //     1024 (B64 H4 d128 L256..1024 431 -> 382 us, B128 H4 d64 L64..512 177 -> 146 us) and batches without padding,
 //     total_q = batch x max_seq_len_q (B32 H8 d128 L2048 2599 -> 2311 us, B32 H8 d32 L4096 8013 -> 6810 us); not for
@@ -587,7 +588,7 @@ static uint64_t ds_workspace_bytes(const hstu_jagged_bwd_params* p, const BwdVar
     if (policy != 1 && (dmax <= 64 || f->max_seq_len_k > 2048)) {
         return 0;
     }
-    int64_t cap_mb = 1024;
+    int64_t cap_mb = 4096;
     if (const char* const env = getenv("HSTU_MI355_BWD_WORKSPACE_MB")) {
         cap_mb = atoll(env);
     }
