@@ -357,7 +357,8 @@ def _new_grad(like: torch.Tensor) -> torch.Tensor:
 
 def _backward_hip(grad, q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max_seq_len_k, silu_scale, seq_offset,
                   seq_offset_k, num_context, num_target, group, alpha):  # fmt: skip
-    """The backward through the C ABI (``hstu_jagged_bwd``): two kernels on the current stream."""
+    """The backward through the C ABI (``hstu_jagged_bwd``): two or three kernels on the current stream, the latter
+    with the workspace the library asks for (dS handed from the query-tile kernel to the dK workgroups)."""
     _check(q.device.type == "cuda", f"q must be a GPU tensor, but it is on {q.device}")
     _check_devices(q.device, (("grad", grad), ("k", k), ("v", v), ("mask", mask), ("attn_bias", attn_bias),
                               ("seq_offset", seq_offset), ("seq_offset_k", seq_offset_k), ("num_context", num_context),
@@ -410,10 +411,13 @@ def _backward_hip(grad, q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max_
     if rc != _native.HSTU_OK:
         raise RuntimeError(f"hstu_jagged_bwd_workspace_size failed ({rc}): {_native.last_error()}")
     ws = torch.empty(ws_bytes.value, dtype=torch.uint8, device=q_c.device) if ws_bytes.value else None
-    if ws is not None and os.environ.get("HSTU_MI355_POISON_WORKSPACE") == "1":
-        ws.fill_(0xFF)  # (for tests: NaN in every element, so that a read of something never written shows)
+    poison = os.environ.get("HSTU_MI355_POISON_WORKSPACE")  # (for tests)
+    if ws is not None and poison == "1":
+        ws.fill_(0xFF)  # NaN in every element, so that a read of something never written shows
+    if poison == "withhold":
+        ws = None  # the call must work without the workspace it asked for
     stream = torch.cuda.current_stream(q_c.device).cuda_stream
-    rc = lib.hstu_jagged_bwd(ctypes.byref(p), _ptr(ws), ws_bytes.value, ctypes.c_void_p(stream))
+    rc = lib.hstu_jagged_bwd(ctypes.byref(p), _ptr(ws), ws_bytes.value if ws is not None else 0, ctypes.c_void_p(stream))
     if rc != _native.HSTU_OK:
         raise RuntimeError(f"hstu_jagged_bwd failed ({rc}): {_native.last_error()}")
     return dq, dk, dv, dbias

@@ -168,6 +168,10 @@ def test_ds_handed_to_the_dk_workgroups_through_a_workspace(kw, mask, monkeypatc
     monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "1")
     three = device_grads(w, grad_out)
     assert torch.equal(two[0], three[0]) and torch.equal(two[2], three[2])  # dq and dv: the same arithmetic
+    # a caller that does not bring the workspace the library asked for gets the two-launch order
+    monkeypatch.setenv("HSTU_MI355_POISON_WORKSPACE", "withhold")
+    without = device_grads(w, grad_out)
+    assert all(torch.equal(x, y) for x, y in zip(two[:3], without[:3]))
     scale = two[1].float().abs().max().item()
     tol = 1e-2 if w.q.dtype == torch.bfloat16 else 2e-3
     torch.testing.assert_close(three[1].float(), two[1].float(), atol=tol * scale, rtol=tol)
