@@ -608,7 +608,11 @@ __global__ __launch_bounds__(kDkvThreads, MODE == 2 ? bwd_dk_from_ds_wgs_per_cu(
     __shared__ __attribute__((aligned(1024))) uint16_t s_st2[kHalves * T::ELEMS];
     __shared__ __attribute__((aligned(1024))) uint16_t s_st3[kHalves * T::ELEMS];
     // a sub-tile is requested three steps ahead: the requests of two later steps may be outstanding at a step's start
-    constexpr int kReqs = 2 * kHalves * LPW;
+    // (plus, in MODE 2, the two loads of the next step's dS rows, issued between the two requests.  Reading rab / mask
+    // rows a step ahead in the same way was tried for the other modes: nothing for the dV-only launch, 277 -> 314 us
+    // at C3 for the two-role one, which has no registers to spare at the head-dim slot 128.)
+    constexpr int kAhead = MODE == 2 ? 2 : 0;
+    constexpr int kReqs = 2 * kHalves * LPW + kAhead;
     constexpr int kWaitStage = (kReqs & 15) | (7 << 4) | (15 << 8) | ((kReqs >> 4) << 14);
     constexpr uint32_t kPastEnd = 0x40000000u;
     static_assert(NLW == 4, "every wavefront takes part in the loads");
@@ -630,8 +634,12 @@ __global__ __launch_bounds__(kDkvThreads, MODE == 2 ? bwd_dk_from_ds_wgs_per_cu(
     const int rem = tile_slot - kt_idx * per_level;
     const int b = rem / a.n_heads_k;
     const int hk = rem - b * a.n_heads_k;
-    zero_tail_rows(a.dk, a.offs_k, a.n_batch, a.idx64, a.total_k, static_cast<int64_t>(a.n_heads_k) * a.d_qk, kDkvThreads);
-    zero_tail_rows(a.dv, a.offs_k, a.n_batch, a.idx64, a.total_k, static_cast<int64_t>(a.n_heads_k) * a.d_v, kDkvThreads);
+    if constexpr (MODE != 1) {
+        zero_tail_rows(a.dk, a.offs_k, a.n_batch, a.idx64, a.total_k, static_cast<int64_t>(a.n_heads_k) * a.d_qk, kDkvThreads);
+    }
+    if constexpr (MODE != 2) {
+        zero_tail_rows(a.dv, a.offs_k, a.n_batch, a.idx64, a.total_k, static_cast<int64_t>(a.n_heads_k) * a.d_v, kDkvThreads);
+    }
     if (a.drab_clear_bytes > 0) {
         // the attn_bias gradient is cleared here, by all workgroups alike (also those of absent tiles, which leave
         // below), and written by the query-tile kernel that runs after this one.  (Dealing the share out over the
@@ -786,6 +794,43 @@ __global__ __launch_bounds__(kDkvThreads, MODE == 2 ? bwd_dk_from_ds_wgs_per_cu(
         return r;
     };
 
+    // whole block hidden from the keys of this wavefront?  (rows rq0 .. rq0 + 31, keys cw0 .. cw0 + 31)
+    auto block_active = [&](int rq0) -> bool {
+        bool active = cw0 < sk;
+        if (a.mask_type == 0) {
+            int lim_max = rq0 + 32 + si.delta;  // lim of the last row
+            if (rq0 < si.n_ctx) {
+                lim_max = lim_max > si.hist_k ? lim_max : si.hist_k;
+            }
+            active = active && cw0 < lim_max;
+        }
+        return active;
+    };
+    // MODE 2: the dS rows of a step, as the query-tile kernel stored them (rounded to the input type, masked), are
+    // read like rab rows -- lane (ln, lh) reads row rq0 + ln, keys cw0 + 16 j + 8 lh .. + 7 -- one step ahead of
+    // their use, and transposed by the same routing products.  Only what that kernel wrote is read -- whole 16-byte
+    // pieces that start ahead of the sequence's last key, in the 32 x 32 blocks that it swept, which are the active
+    // blocks here -- so the plane need not be cleared when it is a workspace.  The two loads go out every step
+    // (out of range when there is nothing to read: no data moves), so that the number of requests in flight at the
+    // start of a step is the same whatever the blocks are.
+    u32x4_t ds_next[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
+    int ds_steps = 0;  // steps whose dS rows have been asked for
+    auto load_ds = [&](int h, int rq0) {
+        const bool wanted = ds_steps < n_iter && block_active(rq0);
+        ++ds_steps;
+        const __amdgpu_buffer_rsrc_t ds_rsrc = make_rsrc(
+            static_cast<const uint16_t*>(a.drab) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k),
+            bias_bytes);
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int key0 = cw0 + 16 * j + 8 * lh;
+            const uint32_t off = (wanted && rq0 + ln < sq && key0 < sk)
+                                     ? (static_cast<uint32_t>(rq0 + ln) * static_cast<uint32_t>(a.max_k) + static_cast<uint32_t>(key0)) * 2u
+                                     : kOutOfRange;
+            ds_next[j] = __builtin_amdgcn_raw_buffer_load_b128(ds_rsrc, static_cast<int>(off), 0, 0);
+        }
+    };
+
     auto step = [&](const uint16_t* stage, uint16_t* stage_o) {
         // this step's sub-tile has landed for everybody; the stage of the previous step is free (see the dQ kernel)
         __builtin_amdgcn_sched_barrier(0);
@@ -798,45 +843,24 @@ __global__ __launch_bounds__(kDkvThreads, MODE == 2 ? bwd_dk_from_ds_wgs_per_cu(
             cur_x = x_first;
             ++cur_h;
         }
-        // whole block hidden from the keys of this wavefront?  (rows rq0 .. rq0 + 31, keys cw0 .. cw0 + 31)
-        bool active = cw0 < sk;
-        if (a.mask_type == 0) {
-            int lim_max = rq0 + 32 + si.delta;  // lim of the last row
-            if (rq0 < si.n_ctx) {
-                lim_max = lim_max > si.hist_k ? lim_max : si.hist_k;
-            }
-            active = active && cw0 < lim_max;
-        }
+        const bool active = block_active(rq0);
         const __amdgpu_buffer_rsrc_t rab_rsrc = make_rsrc(
             HAS_RAB ? static_cast<const uint16_t*>(a.rab) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k) : nullptr,
             HAS_RAB ? bias_bytes : 0u);
         const __amdgpu_buffer_rsrc_t mask_rsrc = make_rsrc(
             HAS_MASK ? static_cast<const uint16_t*>(a.mask) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k) : nullptr,
             HAS_MASK ? bias_bytes : 0u);
-        // rab / mask rows of this step (16-byte path) go out before the tile requests: loads return in order, so
-        // waiting for them then only waits for requests of earlier steps.  Lane (ln, lh) reads row rq0 + ln, keys
-        // cw0 + 16 j + 8 lh .. + 7 (whole chunks are in or out of the row: max_seq_len_k is a multiple of 8 here).
+        // rab / mask rows of this step (16-byte path): lane (ln, lh) has row rq0 + ln, keys cw0 + 16 j + 8 lh .. + 7
+        // (whole chunks are in or out of the row: max_seq_len_k is a multiple of 8 here)
         u32x4_t ra[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
         u32x4_t ma[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
         if constexpr (from_plane) {
-            // dS rows of this step, as the query-tile kernel stored them (rounded to the input type, masked): read
-            // like rab rows and transposed by the same routing products.  Only what that kernel wrote is read -- whole
-            // 16-byte pieces that start ahead of the sequence's last key, in the 32 x 32 blocks that it swept, which
-            // are the blocks `active` here -- so the plane need not be cleared when it is a workspace.
-            if (active) {
-                const __amdgpu_buffer_rsrc_t ds_rsrc = make_rsrc(
-                    static_cast<const uint16_t*>(a.drab) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k),
-                    bias_bytes);
-#pragma unroll
-                for (int j = 0; j < 2; ++j) {
-                    const int key0 = cw0 + 16 * j + 8 * lh;
-                    const uint32_t off = (rq0 + ln < sq && key0 < sk)
-                                             ? (static_cast<uint32_t>(rq0 + ln) * static_cast<uint32_t>(a.max_k) + static_cast<uint32_t>(key0)) * 2u
-                                             : kOutOfRange;
-                    ra[j] = __builtin_amdgcn_raw_buffer_load_b128(ds_rsrc, static_cast<int>(off), 0, 0);
-                }
-            }
+            ra[0] = ds_next[0];  // asked for a step ago
+            ra[1] = ds_next[1];
+            load_ds(cur_h, cur_x * 32);  // (cur_h, cur_x: already those of the next step)
         } else if constexpr (HAS_RAB || HAS_MASK) {
+            // (ahead of the tile requests: loads return in order, so waiting for them then only waits for requests
+            // of earlier steps)
             if (vec16 && active) {
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
@@ -993,6 +1017,9 @@ __global__ __launch_bounds__(kDkvThreads, MODE == 2 ? bwd_dk_from_ds_wgs_per_cu(
     if (n_iter > 0) {
         request(s_st0);
         request(s_st1);
+        if constexpr (from_plane) {
+            load_ds(cur_h, cur_x * 32);  // (where the steps issue theirs: ahead of the request of two stages on)
+        }
         request(s_st2);
         int it = 0;
         while (true) {  // (step it reads stage it mod 4 and has stage (it + 3) mod 4 filled)
