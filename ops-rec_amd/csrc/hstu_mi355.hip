@@ -551,11 +551,23 @@ HSTU_API int hstu_paged_fwd(const hstu_paged_fwd_params* p, void* workspace, uin
 //     1024 (B64 H4 d128 L256..1024 431 -> 382 us, B128 H4 d64 L64..512 177 -> 146 us) and batches without padding,
 //     total_q = batch x max_seq_len_q (B32 H8 d128 L2048 2599 -> 2311 us, B32 H8 d32 L4096 8013 -> 6810 us); not for
 //     long jagged batches (B32 H4 d64 L100..1504 310 -> 341 us, B8 H8 d128 L1024..4096 1492 -> 1657 us; C3 396 -> 401 us).
+// Either way only from 512 workgroups per launch on (enough_tiles_for_three_launches).  Running the dV workgroups on a
+// second stream beside the query-tile kernel, which the workspace makes independent of them, was tried as well: no
+// gain (C2 143 -> 149 us; the launches do not interleave enough to fill each other's tails).
 // HSTU_MI355_BWD_HANDOFF in the environment overrides the choice: 0 = two launches, 1 = three wherever possible.
 static int handoff_policy()  // 0: never, 1: wherever possible, 2: by the rule above
 {
     const char* const env = getenv("HSTU_MI355_BWD_HANDOFF");
     return env == nullptr ? 2 : (env[0] == '0' ? 0 : 1);
+}
+
+// key tiles x sequences x K/V heads: the workgroups of a launch of either role.  Below about two per CU three launches
+// in a row cost more than the products they save (bf16 d128, two launches -> three: B4 H4 L300..700 66 -> 75 us,
+// B8 H4 L512..1024 92 -> 102 us; from there on B16 H4 L512..1024 118 -> 108 us, B32 H4 L128..512 79 -> 72 us).
+static bool enough_tiles_for_three_launches(const hstu_jagged_fwd_params* f)
+{
+    const int64_t n_ktiles = (f->max_seq_len_k + hstu::kBlockM - 1) / hstu::kBlockM;
+    return n_ktiles * (f->n_offsets - 1) * f->num_heads_k >= 512;
 }
 
 static int64_t ds_plane_bytes(const hstu_jagged_fwd_params* f)
@@ -572,7 +584,8 @@ static bool hands_over_through_gradient(const hstu_jagged_bwd_params* p, const B
         return false;
     }
     const int64_t dmax = f->head_dim_qk > f->head_dim_v ? f->head_dim_qk : f->head_dim_v;
-    return policy == 1 || dmax > 128 || f->max_seq_len_k <= 1024 || f->total_q == (f->n_offsets - 1) * f->max_seq_len_q;
+    return policy == 1 || (enough_tiles_for_three_launches(f) &&
+                           (dmax > 128 || f->max_seq_len_k <= 1024 || f->total_q == (f->n_offsets - 1) * f->max_seq_len_q));
 }
 
 // bytes of the workspace through which dS is handed over when there is no attn_bias gradient (0: two launches)
@@ -585,7 +598,7 @@ static uint64_t ds_workspace_bytes(const hstu_jagged_bwd_params* p, const BwdVar
         return 0;
     }
     const int64_t dmax = f->head_dim_qk > f->head_dim_v ? f->head_dim_qk : f->head_dim_v;
-    if (policy != 1 && (dmax <= 64 || f->max_seq_len_k > 2048)) {
+    if (policy != 1 && (dmax <= 64 || f->max_seq_len_k > 2048 || !enough_tiles_for_three_launches(f))) {
         return 0;
     }
     int64_t cap_mb = 4096;
