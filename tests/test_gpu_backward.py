@@ -199,6 +199,31 @@ def test_more_keys_than_queries(monkeypatch):
     check(w, monkeypatch)
 
 
+@pytest.mark.parametrize("rab", [False, True], ids=["workspace", "bias_gradient"])
+def test_ds_hand_over_with_more_keys_than_queries(rab, monkeypatch):
+    # the three-launch order on key ranges longer than the query ranges (delta), grouped heads, 16-byte aligned rows
+    lq, lk = [70, 200, 1, 0, 129], [376, 333, 129, 40, 129]
+    g = torch.Generator(device=DEV).manual_seed(18)
+    mk = lambda n, h, d: (torch.randn(n, h, d, generator=g, device=DEV) * 0.5).to(torch.bfloat16)  # noqa: E731
+    offs = lambda ls: torch.tensor([0] + list(torch.tensor(ls).cumsum(0)), dtype=torch.int64, device=DEV)  # noqa: E731
+    bias = (torch.randn(5, 4, 200, 376, generator=g, device=DEV) * 0.5).to(torch.bfloat16) if rab else None
+    w = workloads.Workload(name="delta", q=mk(sum(lq), 4, 128), k=mk(sum(lk), 2, 128), v=mk(sum(lk), 2, 128),
+                           seq_offset=offs(lq), max_seq_len=200, silu_scale=1.0, alpha=0.09, seq_offset_k=offs(lk),
+                           max_seq_len_k=376, attn_bias=bias, lengths=lq)  # fmt: skip
+    monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "1")
+    check(w, monkeypatch)
+    g2 = torch.Generator(device=DEV).manual_seed(6)
+    grad_out = torch.randn(w.q.shape[0], 4, 128, generator=g2, device=DEV).to(torch.bfloat16)
+    monkeypatch.setenv("HSTU_MI355_GENERIC_BACKWARD", "0")
+    monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "0")
+    two = device_grads(w, grad_out)
+    monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "1")
+    three = device_grads(w, grad_out)
+    assert torch.equal(two[0], three[0]) and torch.equal(two[2], three[2])
+    if rab:
+        assert torch.equal(two[3], three[3])
+
+
 def test_long_sequences_and_rows_past_the_last_offset(monkeypatch):
     w = make(batch=2, heads=2, dim=128, lo=1500, hi=2500, seed=7, std=0.3)
     # 40 rows that belong to no sequence: their gradients must come back as zeros
