@@ -224,6 +224,50 @@ def test_ds_hand_over_with_more_keys_than_queries(rab, monkeypatch):
         assert torch.equal(two[3], three[3])
 
 
+def test_random_shapes_in_both_launch_orders(monkeypatch):
+    """60 seeded random cases (head dims, grouped heads, lengths from empty to 1030, context / targets, every mask
+    type, with and without attn_bias, both index types): the three-launch order, its workspace full of NaN, against
+    the two-launch order -- dq, dv and the bias gradient bit for bit, dk to rounding."""
+    import random
+
+    rnd = random.Random(5)
+    monkeypatch.setenv("HSTU_MI355_GENERIC_BACKWARD", "0")
+    monkeypatch.setenv("HSTU_MI355_POISON_WORKSPACE", "1")
+    for case in range(60):
+        d = rnd.choice([32, 64, 64, 128, 128, 128, 256, 80, 96, 48, 208])
+        heads_k = rnd.choice([1, 2, 3])
+        heads = heads_k * rnd.choice([1, 1, 2, 4])
+        hi = rnd.choice([8, 31, 32, 33, 64, 100, 127, 128, 129, 200, 256, 300, 511, 520, 777, 1030])
+        max_len = (hi + rnd.choice([0, 0, 5, 40]) + 7) // 8 * 8
+        kw = dict(batch=rnd.choice([1, 2, 3, 5, 9]), heads=heads, heads_k=heads_k, dim=d,
+                  dim_v=rnd.choice([d, d, max(16, (d // 2 + 15) // 16 * 16)]), lo=rnd.choice([0, 1, hi // 2, hi]), hi=hi,
+                  max_seq_len=max_len, dtype=rnd.choice([torch.bfloat16, torch.float16]), silu_scale=rnd.choice([0.0, 1.0]),
+                  seed=case, rab_std=rnd.choice([None, 0.5]), index_dtype=rnd.choice([torch.int32, torch.int64]))  # fmt: skip
+        if rnd.random() < 0.4:
+            kw.update(num_context=rnd.choice([0, 3, 40]), max_target=rnd.choice([0, 5, 60]), target_group_size=rnd.choice([0, 1, 3]))
+        mask_type = rnd.choice([0, 0, 0, 2, 3])
+        w = make(**kw)
+        if mask_type == 3:
+            g = torch.Generator(device=DEV).manual_seed(case)
+            m = (torch.rand(len(w.lengths), heads, max_len, max_len, generator=g, device=DEV) < 0.7).to(w.q.dtype)
+            w = dataclasses.replace(w, mask=m, mask_type=3, num_context=None, num_target=None, target_group_size=0)
+        elif mask_type == 2:
+            w = dataclasses.replace(w, mask_type=2, num_context=None, num_target=None, target_group_size=0)
+        g = torch.Generator(device=DEV).manual_seed(1000 + case)
+        grad_out = torch.randn(w.q.shape[0], heads, w.v.shape[2], generator=g, device=DEV).to(w.q.dtype)
+        monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "0")
+        two = device_grads(w, grad_out)
+        monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "1")
+        three = device_grads(w, grad_out)
+        label = f"case {case}: {kw}, mask_type {mask_type}"
+        assert all(torch.isfinite(t).all() for t in three if t is not None), label
+        assert torch.equal(two[0], three[0]) and torch.equal(two[2], three[2]), label
+        assert two[3] is None or torch.equal(two[3], three[3]), label
+        scale = max(two[1].float().abs().max().item(), 1e-6)
+        tol = 1e-2 if w.q.dtype == torch.bfloat16 else 2e-3
+        assert (two[1].float() - three[1].float()).abs().max().item() <= tol * scale, label
+
+
 def test_long_sequences_and_rows_past_the_last_offset(monkeypatch):
     w = make(batch=2, heads=2, dim=128, lo=1500, hi=2500, seed=7, std=0.3)
     # 40 rows that belong to no sequence: their gradients must come back as zeros
