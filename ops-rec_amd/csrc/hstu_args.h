@@ -87,6 +87,7 @@ struct BwdArgs {
     void* dk;
     void* dv;
     void* drab;  // may be null
+    void* p_plane;  // where the query-tile kernel leaves P for dV workgroups that read it back (same shape as drab), or null
     int64_t drab_clear_bytes;  // > 0: the key-tile kernel clears this many bytes at drab beside its work
     const void* offs_q;
     const void* offs_k;

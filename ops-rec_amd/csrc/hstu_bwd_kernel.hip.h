@@ -232,9 +232,13 @@ __device__ __forceinline__ void store_tile_rows(uint16_t* stage, const f32x16_t 
 // ---------------------------------------------------------------------------------------------------------
 // dQ (and d rab)
 // ---------------------------------------------------------------------------------------------------------
-template <typename Tag, int D, bool HAS_RAB, bool HAS_MASK, bool WANT_DRAB>
+// STORE: 0 = dQ only; 1 = dS stored as well (it is the attn_bias gradient; or into a workspace, for dK workgroups that
+// read it back); 2 = dS and P stored (P for dV workgroups that read it back: no product is then computed twice)
+template <typename Tag, int D, bool HAS_RAB, bool HAS_MASK, int STORE>
 __global__ __launch_bounds__(256, bwd_dq_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hstu_bwd_dq_kernel(const BwdArgs a)
 {
+    constexpr bool WANT_DRAB = STORE >= 1;
+    constexpr bool WANT_P = STORE == 2;
     typedef SubTile<D> T;
     constexpr int LPW = T::LPW, NLW = T::NLW, KSTEPS = T::KSTEPS, MTILES = T::MTILES, NCH = 2 * T::MTILES;
     // three stages of {K, V} sub-tiles; separate arrays so that the compiler can tell the stage being filled by
@@ -363,6 +367,15 @@ __global__ __launch_bounds__(256, bwd_dq_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void 
         make_rsrc(HAS_MASK ? static_cast<const uint16_t*>(a.mask) + bias_plane : nullptr, HAS_MASK ? bias_bytes : 0u);
     const __amdgpu_buffer_rsrc_t drab_rsrc =
         make_rsrc(WANT_DRAB ? static_cast<uint16_t*>(a.drab) + bias_plane : nullptr, WANT_DRAB ? bias_bytes : 0u);
+    // dS and P together (STORE 2) go to a plane of their own layout: per query row, the 32 dS values of a 32-key block
+    // followed by its 32 P values -- one whole 128-byte line per row and step, where two planes of the bias layout would
+    // each get half a line
+    const uint32_t pair_pitch = 64u * static_cast<uint32_t>((a.max_k + 31) / 32);  // elements per row
+    const __amdgpu_buffer_rsrc_t p_rsrc =
+        make_rsrc(WANT_P ? static_cast<uint16_t*>(a.p_plane) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(pair_pitch)
+                         : nullptr,
+                  WANT_P ? static_cast<uint32_t>(a.max_q) * pair_pitch * 2u : 0u);
+    const uint32_t pair_row_off = (wr0 + ln < sq) ? static_cast<uint32_t>(wr0 + ln) * pair_pitch * 2u : kOutOfRange;
     // rows past the sequence lie inside the plane but must stay untouched / unread: their offset leaves it
     const uint32_t bias_row_off =
         (wr0 + ln < sq) ? static_cast<uint32_t>(wr0 + ln) * static_cast<uint32_t>(a.max_k) * 2u : kOutOfRange;
@@ -465,9 +478,10 @@ __global__ __launch_bounds__(256, bwd_dq_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void 
             dp = mfma32<Tag>(read_n(vn, js), gf[js], dp);
         }
         uint32_t pk[8];
+        uint32_t pp[8];  // P, when it is stored
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
-            float ds2[2];
+            float ds2[2], p2[2];
 #pragma unroll
             for (int e2 = 0; e2 < 2; ++e2) {
                 const int e = 2 * i + e2;
@@ -476,12 +490,19 @@ __global__ __launch_bounds__(256, bwd_dq_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void 
                     sv += e2 ? hi_to_float<Tag>(rw[i]) : lo_to_float<Tag>(rw[i]);
                 }
                 float ds = score_ds(sv, dp[e], sconst);
+                float pv = WANT_P ? score_p(sv, sconst) : 0.f;
                 if constexpr (HAS_MASK) {
-                    ds *= e2 ? hi_to_float<Tag>(mw[i]) : lo_to_float<Tag>(mw[i]);
+                    const float mv = e2 ? hi_to_float<Tag>(mw[i]) : lo_to_float<Tag>(mw[i]);
+                    ds *= mv;
+                    pv *= mv;
                 }
                 ds2[e2] = ds;
+                p2[e2] = pv;
             }
             pk[i] = pack2<Tag>(ds2[0], ds2[1]);
+            if constexpr (WANT_P) {
+                pp[i] = pack2<Tag>(p2[0], p2[1]);
+            }
         }
         // visibility, applied to the packed values and only when the sub-tile is not fully visible to this
         // wavefront's rows (as in the forward): key c0 + 8 (e / 4) + 4 lh + e % 4 of element e is hidden at or past
@@ -499,9 +520,29 @@ __global__ __launch_bounds__(256, bwd_dq_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void 
                     keep |= vis ? (0xffffu << (16 * e2)) : 0u;
                 }
                 pk[i] &= keep;
+                if constexpr (WANT_P) {
+                    pp[i] &= keep;
+                }
             }
         }
-        if constexpr (WANT_DRAB) {
+        if constexpr (WANT_P) {
+            // the two lanes of a row trade halves (see below), then four 16-byte pieces per lane pair: dS, dS, P, P
+            typedef __attribute__((ext_vector_type(2))) unsigned u2_t;
+#pragma unroll
+            for (int h2 = 0; h2 < 2; ++h2) {
+                const int key = c0 + 16 * h2 + 8 * lh;
+                const uint32_t off = pair_row_off + static_cast<uint32_t>(2 * c0 + 16 * h2 + 8 * lh) * 2u;
+                const u2_t d0 = __builtin_amdgcn_permlane32_swap(pk[4 * h2 + 0], pk[4 * h2 + 2], false, false);
+                const u2_t d1 = __builtin_amdgcn_permlane32_swap(pk[4 * h2 + 1], pk[4 * h2 + 3], false, false);
+                const u32x4_t wd = {d0[0], d1[0], d0[1], d1[1]};
+                __builtin_amdgcn_raw_buffer_store_b128(wd, p_rsrc, static_cast<int>(key < sk ? off : kOutOfRange), 0, 0);
+                const u2_t r0 = __builtin_amdgcn_permlane32_swap(pp[4 * h2 + 0], pp[4 * h2 + 2], false, false);
+                const u2_t r1 = __builtin_amdgcn_permlane32_swap(pp[4 * h2 + 1], pp[4 * h2 + 3], false, false);
+                const u32x4_t wp = {r0[0], r1[0], r0[1], r1[1]};
+                __builtin_amdgcn_raw_buffer_store_b128(wp, p_rsrc, static_cast<int>(key < sk ? off + 64u : kOutOfRange), 0, 0);
+            }
+        }
+        if constexpr (WANT_DRAB && !WANT_P) {
             if (vec16) {
                 // 16-byte aligned rows: the two lanes of a row trade halves (v_permlane32_swap), so that each holds 8
                 // consecutive keys and a store instruction writes whole 32-byte sectors of 32 rows instead of 16-byte
@@ -595,12 +636,15 @@ __global__ __launch_bounds__(256, bwd_dq_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void 
 // MODE 0: a dV and a dK workgroup per key tile (even / odd workgroups).  MODE 1 and 2 serve the three-launch order
 // dV / dQ / dK: all workgroups of a launch have one role, and the dK ones (MODE 2; rab and mask play no part in it)
 // take dS from the attn_bias gradient that the query-tile kernel wrote between the two launches.
+// MODE 4: launched after a query-tile kernel that stored dS and P: a workgroup that takes dV from P (even) and one
+// that takes dK from dS (odd) per key tile, both of MODE 2's build (one product each; the dV ones stream dO
+// where the dK ones stream Q).
 template <typename Tag, int D, bool HAS_RAB, bool HAS_MASK, int MODE = 0>
-__global__ __launch_bounds__(kDkvThreads, MODE == 2 ? bwd_dk_from_ds_wgs_per_cu(D) : bwd_dkv_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hstu_bwd_dkv_kernel(const BwdArgs a)
+__global__ __launch_bounds__(kDkvThreads, (MODE == 2 || MODE == 4) ? bwd_dk_from_ds_wgs_per_cu(D) : bwd_dkv_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hstu_bwd_dkv_kernel(const BwdArgs a)
 {
     typedef SubTile<D> T;
     constexpr int LPW = T::LPW, NLW = T::NLW, KSTEPS = T::KSTEPS, MTILES = T::MTILES, NCH = 2 * T::MTILES;
-    constexpr int kHalves = MODE == 2 ? 1 : 2;  // (the dK workgroups that read dS need no dO)
+    constexpr int kHalves = (MODE == 2 || MODE == 4) ? 1 : 2;  // (a workgroup that reads dS or P streams Q or dO only)
     // four stages, each the Q sub-tile followed by the dO sub-tile (separate arrays per stage, see the dQ kernel;
     // Q and dO of a stage share an array so that a wavefront can address "the tile of my role" by an offset)
     __shared__ __attribute__((aligned(1024))) uint16_t s_st0[kHalves * T::ELEMS];
@@ -611,7 +655,7 @@ __global__ __launch_bounds__(kDkvThreads, MODE == 2 ? bwd_dk_from_ds_wgs_per_cu(
     // (plus, in MODE 2, the two loads of the next step's dS rows, issued between the two requests.  Reading rab / mask
     // rows a step ahead in the same way was tried for the other modes: nothing for the dV-only launch, 277 -> 314 us
     // at C3 for the two-role one, which has no registers to spare at the head-dim slot 128.)
-    constexpr int kAhead = MODE == 2 ? 2 : 0;
+    constexpr int kAhead = (MODE == 2 || MODE == 4) ? 2 : 0;
     constexpr int kReqs = 2 * kHalves * LPW + kAhead;
     constexpr int kWaitStage = (kReqs & 15) | (7 << 4) | (15 << 8) | ((kReqs >> 4) << 14);
     constexpr uint32_t kPastEnd = 0x40000000u;
@@ -622,14 +666,14 @@ __global__ __launch_bounds__(kDkvThreads, MODE == 2 ? bwd_dk_from_ds_wgs_per_cu(
     const int wave = uniform(tid >> 6);
     // even workgroups produce dV, odd ones dK of the same key tile (neighbours in the grid, so that they tend to
     // run side by side and find each other's Q / dO rows in the L2)
-    constexpr bool from_plane = MODE == 2;
-    const bool dk_role = MODE == 0 ? (blockIdx.x & 1) != 0 : MODE == 2;
+    constexpr bool from_plane = MODE == 2 || MODE == 4;
+    const bool dk_role = (MODE == 0 || MODE == 4) ? (blockIdx.x & 1) != 0 : MODE == 2;
     const int ln = lane & 31;
     const int lh = lane >> 5;
 
     // key tile 0 is seen by the most query rows: heaviest first
     const int per_level = a.n_batch * a.n_heads_k;
-    const int tile_slot = static_cast<int>(MODE == 0 ? blockIdx.x >> 1 : blockIdx.x);
+    const int tile_slot = static_cast<int>((MODE == 0 || MODE == 4) ? blockIdx.x >> 1 : blockIdx.x);
     const int kt_idx = tile_slot / per_level;
     const int rem = tile_slot - kt_idx * per_level;
     const int b = rem / a.n_heads_k;
@@ -693,7 +737,7 @@ __global__ __launch_bounds__(kDkvThreads, MODE == 2 ? bwd_dk_from_ds_wgs_per_cu(
     {
         const int vr0 = 4 * lh + ((lane & 15) >> 2);
         // the transposed operand of this role: Q^T (first half of a stage) for dK, dO^T (second half) for dV
-        const int role_half = dk_role ? 0 : T::ELEMS;
+        const int role_half = (dk_role || from_plane) ? 0 : T::ELEMS;  // (a stage of one half holds the role's tile)
 #pragma unroll
         for (int mt = 0; mt < MTILES; ++mt) {
             const int col = 32 * mt + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
@@ -770,8 +814,14 @@ __global__ __launch_bounds__(kDkvThreads, MODE == 2 ? bwd_dk_from_ds_wgs_per_cu(
         const uint32_t gb = past ? kPastEnd : static_cast<uint32_t>(req_x * 32) * g_stride;
 #pragma unroll
         for (int i = 0; i < LPW; ++i) {
-            load_to_lds_b128(q_rsrc, stage + (wave * LPW + i) * 512, q_src[i] + qb);
-            if constexpr (!from_plane) {
+            if constexpr (from_plane) {
+                if (dk_role) {
+                    load_to_lds_b128(q_rsrc, stage + (wave * LPW + i) * 512, q_src[i] + qb);
+                } else {
+                    load_to_lds_b128(g_rsrc, stage + (wave * LPW + i) * 512, g_src[i] + gb);
+                }
+            } else {
+                load_to_lds_b128(q_rsrc, stage + (wave * LPW + i) * 512, q_src[i] + qb);
                 load_to_lds_b128(g_rsrc, stage + T::ELEMS + (wave * LPW + i) * 512, g_src[i] + gb);
             }
         }
@@ -806,7 +856,7 @@ __global__ __launch_bounds__(kDkvThreads, MODE == 2 ? bwd_dk_from_ds_wgs_per_cu(
         }
         return active;
     };
-    // MODE 2: the dS rows of a step, as the query-tile kernel stored them (rounded to the input type, masked), are
+    // MODE 2 and 4: the dS (or P) rows of a step, as the query-tile kernel stored them (rounded to the input type, masked), are
     // read like rab rows -- lane (ln, lh) reads row rq0 + ln, keys cw0 + 16 j + 8 lh .. + 7 -- one step ahead of
     // their use, and transposed by the same routing products.  Only what that kernel wrote is read -- whole 16-byte
     // pieces that start ahead of the sequence's last key, in the 32 x 32 blocks that it swept, which are the active
@@ -818,14 +868,18 @@ __global__ __launch_bounds__(kDkvThreads, MODE == 2 ? bwd_dk_from_ds_wgs_per_cu(
     auto load_ds = [&](int h, int rq0) {
         const bool wanted = ds_steps < n_iter && block_active(rq0);
         ++ds_steps;
+        // (MODE 4: dS and P share a plane of their own layout, see the query-tile kernel: per row and 32-key block, 32
+        // dS values followed by 32 P values)
+        const uint32_t pitch = MODE == 4 ? 64u * static_cast<uint32_t>((a.max_k + 31) / 32) : static_cast<uint32_t>(a.max_k);
         const __amdgpu_buffer_rsrc_t ds_rsrc = make_rsrc(
-            static_cast<const uint16_t*>(a.drab) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k),
-            bias_bytes);
+            static_cast<const uint16_t*>(MODE == 4 ? a.p_plane : a.drab) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(pitch),
+            static_cast<uint32_t>(a.max_q) * pitch * 2u);
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int key0 = cw0 + 16 * j + 8 * lh;
+            const uint32_t col = MODE == 4 ? static_cast<uint32_t>(2 * cw0 + 16 * j + 8 * lh + (dk_role ? 0 : 32)) : static_cast<uint32_t>(key0);
             const uint32_t off = (wanted && rq0 + ln < sq && key0 < sk)
-                                     ? (static_cast<uint32_t>(rq0 + ln) * static_cast<uint32_t>(a.max_k) + static_cast<uint32_t>(key0)) * 2u
+                                     ? (static_cast<uint32_t>(rq0 + ln) * pitch + col) * 2u
                                      : kOutOfRange;
             ds_next[j] = __builtin_amdgcn_raw_buffer_load_b128(ds_rsrc, static_cast<int>(off), 0, 0);
         }

@@ -532,81 +532,93 @@ HSTU_API int hstu_paged_fwd(const hstu_paged_fwd_params* p, void* workspace, uin
     return launch_forward(&g, nullptr, static_cast<char*>(workspace) + used, workspace_bytes > used ? workspace_bytes - used : 0, stream);
 }
 
-// The tuned kernels recompute S, dP and dS in the dK workgroups (two launches: dV and dK workgroups side by side, then
-// the query-tile kernel) unless the query-tile kernel's dS is kept: then the order is dV workgroups, query-tile
-// kernel, dK workgroups that read dS back (six matrix products instead of eight).  dS is the attn_bias gradient when
-// that is asked for; otherwise it goes into a workspace of the same shape, [batch, heads, max_seq_len_q,
-// max_seq_len_k] in the input type, as far as hstu_jagged_bwd_workspace_size asks for one.  Rows of 16 bytes are
-// needed either way (max_seq_len_k a multiple of 8, 16-byte aligned planes).
+// The tuned backward kernels, in the three orders the entry point knows:
+//   two launches     dV and dK workgroups side by side (the dK ones recompute S, dP and dS), then the query-tile
+//                    kernel: eight matrix products, no workspace;
+//   three launches   dV workgroups, the query-tile kernel storing dS, dK workgroups that read dS back: six products.
+//                    dS is the attn_bias gradient when that is asked for (the dV workgroups clear it beside their
+//                    work), otherwise it goes into a workspace of that shape, [batch, heads, max_seq_len_q,
+//                    max_seq_len_k] in the input type;
+//   planes           the query-tile kernel storing dS and P, then a dV workgroup that reads P and a dK workgroup that
+//                    reads dS per key tile: the five products of the formula, nothing computed twice; two such planes
+//                    of workspace; only without an attn_bias gradient (which would have to be cleared first).
+// Rows of 16 bytes are needed for the planes (max_seq_len_k a multiple of 8, 16-byte aligned pointers).  Nothing in a
+// workspace is cleared: the workgroups that read a plane read exactly the pieces the query-tile kernel wrote.
 //
-// Three launches in a row have three tails and hide the clearing of the attn_bias gradient behind less arithmetic,
-// so the order is chosen by what was measured (bf16, two launches -> three):
-//   through the workspace (4 bytes of traffic per pair against 8 x head dim flops saved): head dims above 64 and
-//     max_seq_len_k up to 2048 -- C2 162 -> 144 us, B16 H4 d256 L1024 317 -> 227 us, B64 H4 d128 L256..1024
-//     272 -> 242 us, B16 H4 d128 L512..2048 240 -> 230 us; not at head dims up to 64 (B32 H8 d64 L1024 278 -> 300 us)
-//     nor for longer rows (B4 H8 d128 L1024..4096 410 -> 528 us, B2 H4 d128 L8192 747 -> 947 us); planes up to 4 GiB
-//     (B32 H8 d256 L2048 4310 -> 3009 us, d128 1566 -> 1512 us; HSTU_MI355_BWD_WORKSPACE_MB in the environment moves
-//     that limit);
-//   through the attn_bias gradient: head dims above 128 (B16 H4 d256 L100..1504 501 -> 404 us), max_seq_len_k up to
-//     1024 (B64 H4 d128 L256..1024 431 -> 382 us, B128 H4 d64 L64..512 177 -> 146 us) and batches without padding,
-//     total_q = batch x max_seq_len_q (B32 H8 d128 L2048 2599 -> 2311 us, B32 H8 d32 L4096 8013 -> 6810 us); not for
-//     long jagged batches (B32 H4 d64 L100..1504 310 -> 341 us, B8 H8 d128 L1024..4096 1492 -> 1657 us; C3 396 -> 401 us).
-// Either way only from 512 workgroups per launch on (enough_tiles_for_three_launches).  Running the dV workgroups on a
-// second stream beside the query-tile kernel, which the workspace makes independent of them, was tried as well: no
-// gain (C2 143 -> 149 us; the launches do not interleave enough to fill each other's tails).
-// HSTU_MI355_BWD_HANDOFF in the environment overrides the choice: 0 = two launches, 1 = three wherever possible.
-static int handoff_policy()  // 0: never, 1: wherever possible, 2: by the rule above
+// Which order is taken follows what was measured (bf16, events through the operator, two launches -> three -> planes):
+//   C2 (B32 H4 d128 L278..1004)  162 -> 142 -> 125 us      B128 H4 d128 L64..512    175 -> 144 -> 133 us
+//   B8 H4 d128 L512..1024         88 -> 100 ->  70 us      B4 H4 d128 L300..700      65 ->  74 ->  54 us
+//   B16 H4 d256 L100..1504       402 -> 290 -> 212 us      B32 H8 d256 L1024       1285 -> 900 -> 800 us
+//   B64 H4 d128 L256..1024       269 -> 240 -> 245 us      B16 H4 d128 L512..2048   240 -> 219 -> 246 us
+//   B32 H8 d128 L1024            438 -> 418 -> 487 us      B32 H8 d64 L1024         277 -> 300 -> 408 us
+//   B4 H8 d128 L1024..4096       409 -> 509 -> 530 us      B2 H4 d128 L8192         738 -> 921 -> 1061 us
+// A plane costs 4 bytes of traffic per (query, key) pair, written and read back, against two products of
+// 4 x head dim flops per pair each: it pays from the head-dim slot 128 on, and at 128 the second plane only while both
+// stay in the memory-side cache (256 MB) between the launches; few long sequences lose either way (each launch is
+// as long as its heaviest workgroup).  The rule:
+//   without an attn_bias gradient, head dims above 64, max_seq_len_k up to 2048, workspace within the limit (4 GiB,
+//   or HSTU_MI355_BWD_WORKSPACE_MB in the environment):  planes for head dims above 128, and for those up to 128 when
+//   total_q x max_seq_len_k x heads x 2 bytes -- an upper bound of what the two planes hold under a causal mask,
+//   doubled for the other mask types -- is at most 200 MB; else three launches from 512 workgroups per launch on
+//   (key tiles x sequences x K/V heads: B8 H4 d128 L512..1024 and smaller lose with three); else two;
+//   with an attn_bias gradient: three launches from 512 workgroups per launch on when the head dims are above 128
+//   (B16 H4 d256 L100..1504 501 -> 404 us), max_seq_len_k is at most 1024 (B64 H4 d128 L256..1024 431 -> 382 us,
+//   B128 H4 d64 L64..512 177 -> 146 us) or the batch has no padding, total_q = batch x max_seq_len_q (B32 H8 d128
+//   L2048 2599 -> 2311 us, B32 H8 d32 L4096 8013 -> 6810 us); not for long jagged batches, where the clearing of the
+//   gradient no longer hides behind the dV workgroups alone (B32 H4 d64 L100..1504 310 -> 341 us, B8 H8 d128
+//   L1024..4096 1492 -> 1657 us; C3 396 -> 401 us).
+// Also tried, not kept: the dV workgroups on a second stream beside the query-tile kernel (C2 143 -> 149 us), and the
+// query-tile kernel first with dV and dK-from-dS workgroups in one launch behind it (C2 160 us).
+// HSTU_MI355_BWD_HANDOFF in the environment overrides the rule: 0 = two launches, 1 = three wherever possible,
+// 2 = planes wherever possible.
+enum BwdOrder { kTwoLaunches, kThreeLaunches, kPlanes };
+struct BwdPlan {
+    BwdOrder order;
+    uint64_t workspace_bytes;  // what the order needs (0: none)
+};
+
+static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
 {
+    const hstu_jagged_fwd_params* f = &p->fwd;
+    const BwdPlan two = {kTwoLaunches, 0};
     const char* const env = getenv("HSTU_MI355_BWD_HANDOFF");
-    return env == nullptr ? 2 : (env[0] == '0' ? 0 : 1);
-}
-
-// key tiles x sequences x K/V heads: the workgroups of a launch of either role.  Below about two per CU three launches
-// in a row cost more than the products they save (bf16 d128, two launches -> three: B4 H4 L300..700 66 -> 75 us,
-// B8 H4 L512..1024 92 -> 102 us; from there on B16 H4 L512..1024 118 -> 108 us, B32 H4 L128..512 79 -> 72 us).
-static bool enough_tiles_for_three_launches(const hstu_jagged_fwd_params* f)
-{
+    const int forced = env == nullptr ? -1 : (env[0] == '0' ? 0 : (env[0] == '2' ? 2 : 1));
+    if (var->dk_from_ds == nullptr || forced == 0 || f->total_q == 0 || f->total_k == 0 || f->max_seq_len_k % 8 != 0) {
+        return two;
+    }
+    const int64_t batch = f->n_offsets - 1;
+    const int64_t dmax = f->head_dim_qk > f->head_dim_v ? f->head_dim_qk : f->head_dim_v;
     const int64_t n_ktiles = (f->max_seq_len_k + hstu::kBlockM - 1) / hstu::kBlockM;
-    return n_ktiles * (f->n_offsets - 1) * f->num_heads_k >= 512;
-}
-
-static int64_t ds_plane_bytes(const hstu_jagged_fwd_params* f)
-{
-    return (f->n_offsets - 1) * f->num_heads_q * f->max_seq_len_q * f->max_seq_len_k * 2;
-}
-
-// dS handed over through the attn_bias gradient
-static bool hands_over_through_gradient(const hstu_jagged_bwd_params* p, const BwdVariant* var)
-{
-    const hstu_jagged_fwd_params* f = &p->fwd;
-    const int policy = handoff_policy();
-    if (var->dk_from_ds == nullptr || p->grad_attn_bias == nullptr || policy == 0) {
-        return false;
-    }
-    const int64_t dmax = f->head_dim_qk > f->head_dim_v ? f->head_dim_qk : f->head_dim_v;
-    return policy == 1 || (enough_tiles_for_three_launches(f) &&
-                           (dmax > 128 || f->max_seq_len_k <= 1024 || f->total_q == (f->n_offsets - 1) * f->max_seq_len_q));
-}
-
-// bytes of the workspace through which dS is handed over when there is no attn_bias gradient (0: two launches)
-static uint64_t ds_workspace_bytes(const hstu_jagged_bwd_params* p, const BwdVariant* var)
-{
-    const hstu_jagged_fwd_params* f = &p->fwd;
-    const int policy = handoff_policy();
-    if (var->dk_from_ds == nullptr || p->grad_attn_bias != nullptr || f->max_seq_len_k % 8 != 0 || policy == 0 ||
-        f->total_q == 0 || f->total_k == 0) {
-        return 0;
-    }
-    const int64_t dmax = f->head_dim_qk > f->head_dim_v ? f->head_dim_qk : f->head_dim_v;
-    if (policy != 1 && (dmax <= 64 || f->max_seq_len_k > 2048 || !enough_tiles_for_three_launches(f))) {
-        return 0;
+    const bool many_tiles = n_ktiles * batch * f->num_heads_k >= 512;
+    if (p->grad_attn_bias != nullptr) {
+        const bool by_rule = many_tiles && (dmax > 128 || f->max_seq_len_k <= 1024 || f->total_q == batch * f->max_seq_len_q);
+        return (forced >= 1 || (forced < 0 && by_rule)) ? BwdPlan{kThreeLaunches, 0} : two;
     }
     int64_t cap_mb = 4096;
-    if (const char* const env = getenv("HSTU_MI355_BWD_WORKSPACE_MB")) {
-        cap_mb = atoll(env);
+    if (const char* const cap_env = getenv("HSTU_MI355_BWD_WORKSPACE_MB")) {
+        cap_mb = atoll(cap_env);
     }
-    const int64_t bytes = ds_plane_bytes(f);
-    return bytes <= cap_mb * (1LL << 20) ? static_cast<uint64_t>(bytes) : 0;
+    const int64_t plane = batch * f->num_heads_q * f->max_seq_len_q * f->max_seq_len_k * 2;
+    const bool three_fits = plane <= cap_mb * (1LL << 20);
+    // (dS and P share rows of whole 32-key blocks, 64 elements each)
+    const int64_t pair_plane = batch * f->num_heads_q * f->max_seq_len_q * (64 * ((f->max_seq_len_k + 31) / 32)) * 2;
+    const bool planes_fit = pair_plane <= cap_mb * (1LL << 20);
+    const BwdPlan three = {kThreeLaunches, static_cast<uint64_t>(plane)};
+    const BwdPlan planes = {kPlanes, static_cast<uint64_t>(pair_plane)};
+    if (forced == 2) {
+        return planes_fit ? planes : (three_fits ? three : two);
+    }
+    if (forced == 1) {
+        return three_fits ? three : two;
+    }
+    if (dmax <= 64 || f->max_seq_len_k > 2048) {
+        return two;
+    }
+    const int64_t held = f->total_q * f->max_seq_len_k * f->num_heads_q * 2 * (f->mask_type == HSTU_MASK_TRIL ? 1 : 2);
+    if (planes_fit && (dmax > 128 || held <= 200LL * 1000 * 1000)) {
+        return planes;
+    }
+    return (three_fits && many_tiles) ? three : two;
 }
 
 HSTU_API int hstu_jagged_bwd_workspace_size(const hstu_jagged_bwd_params* params, uint64_t* workspace_bytes)
@@ -623,7 +635,7 @@ HSTU_API int hstu_jagged_bwd_workspace_size(const hstu_jagged_bwd_params* params
     if (var == nullptr) {
         return HSTU_ERR_UNSUPPORTED;
     }
-    *workspace_bytes = ds_workspace_bytes(params, var);
+    *workspace_bytes = plan_bwd(params, var).workspace_bytes;
     return HSTU_OK;
 }
 
@@ -703,6 +715,7 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
     a.scale = static_cast<float>((f->silu_scale == 0.0) ? 1.0 / static_cast<double>(f->max_seq_len_q) : f->silu_scale);
 
     const bool generic = is_generic_bwd(var);
+    const BwdPlan plan = plan_bwd(p, var);
     // the tuned key-tile kernel runs a dV and a dK workgroup per tile, the generic one a workgroup per tile
     const int64_t grid_kv = (generic ? 1 : 2) * static_cast<int64_t>(a.n_ktiles) * a.n_batch * a.n_heads_k;
     const int64_t grid_q = static_cast<int64_t>(a.n_qtiles) * a.n_batch * a.n_heads_q;
@@ -721,16 +734,26 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
             hipLaunchKernelGGL(var->dkv, dim3(static_cast<unsigned>(grid_kv)), dim3(256), 0, static_cast<hipStream_t>(stream), a);
             hipLaunchKernelGGL(var->dq, dim3(static_cast<unsigned>(grid_q)), dim3(256), 0, static_cast<hipStream_t>(stream), a);
         }
-    } else if (f->total_k > 0 && grid_kv > 0 && f->total_q > 0 && grid_q > 0 && a.bias_vec_ok == 2 &&
-               (hands_over_through_gradient(p, var) ||
-                (ds_workspace_bytes(p, var) > 0 && usable_workspace(workspace, workspace_bytes, ds_workspace_bytes(p, var)) &&
-                 reinterpret_cast<uintptr_t>(workspace) % 16 == 0))) {
-        // dV workgroups (which clear the attn_bias gradient beside their work), the query-tile kernel (which writes
-        // dS into it, or into the workspace, where nothing needs clearing: the dK workgroups read what was written),
-        // dK workgroups (which read dS back instead of computing S, dP and dS a second time)
+    } else if (f->total_k > 0 && grid_kv > 0 && f->total_q > 0 && grid_q > 0 && a.bias_vec_ok == 2 && plan.order != kTwoLaunches &&
+               (plan.workspace_bytes == 0 || (usable_workspace(workspace, workspace_bytes, plan.workspace_bytes) &&
+                                              reinterpret_cast<uintptr_t>(workspace) % 16 == 0))) {
         if (p->grad_attn_bias == nullptr) {
             a.drab = workspace;
         }
+        if (plan.order == kPlanes) {
+            // the query-tile kernel with dS and P, then a dV-from-P and a dK-from-dS workgroup per key tile
+            a.p_plane = workspace;
+            hipLaunchKernelGGL(var->dq_ds_p, dim3(static_cast<unsigned>(grid_q)), dim3(256), 0, static_cast<hipStream_t>(stream), a);
+            hipLaunchKernelGGL(var->dv_dk_from_planes, dim3(static_cast<unsigned>(grid_kv)), dim3(hstu::kDkvThreads), 0,
+                               static_cast<hipStream_t>(stream), a);
+            const hipError_t err2 = hipGetLastError();
+            if (err2 != hipSuccess) {
+                return fail(HSTU_ERR_RUNTIME, "launch of %s failed: %s", var->name, hipGetErrorString(err2));
+            }
+            return HSTU_OK;
+        }
+        // dV workgroups (which clear the attn_bias gradient beside their work), the query-tile kernel (which writes
+        // dS into it, or into the workspace), dK workgroups (which read dS back)
         a.drab_clear_bytes = drab_bytes;
         hipLaunchKernelGGL(var->dv_only, dim3(static_cast<unsigned>(grid_kv / 2)), dim3(hstu::kDkvThreads), 0,
                            static_cast<hipStream_t>(stream), a);

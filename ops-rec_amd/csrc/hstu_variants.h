@@ -30,6 +30,9 @@ struct BwdVariant {
     // the three-launch order dV / dQ storing dS / dK from that dS (nullptr in the generic and fp32 tables)
     void (*dv_only)(const BwdArgs);
     void (*dk_from_ds)(const BwdArgs);
+    // the order dQ storing dS and P / dV workgroups that read P beside dK workgroups that read dS
+    void (*dq_ds_p)(const BwdArgs);
+    void (*dv_dk_from_planes)(const BwdArgs);
 };
 
 // forward, 16-bit inputs: [rab: 0, 1][custom mask: 0, 1][dim slot: 32, 64, 128, 256]

@@ -148,9 +148,10 @@ def test_attn_bias_gradient_handed_to_the_dk_workgroups(kw, custom_mask, monkeyp
 ], ids=lambda kw: "-".join(f"{k}{v}" for k, v in kw.items() if k != "dtype"))  # fmt: skip
 @pytest.mark.parametrize("mask", ["causal", "custom", "none"])
 def test_ds_handed_to_the_dk_workgroups_through_a_workspace(kw, mask, monkeypatch):
-    """Without an attn_bias gradient, head dims above 64 and max_seq_len_k a multiple of 8, the query-tile kernel
-    leaves dS in a workspace for the dK workgroups (hstu_jagged_bwd_workspace_size asks for it).  Checked against
-    the oracle and the generic kernels with the workspace full of NaN, and against the two-launch order."""
+    """Without an attn_bias gradient and with max_seq_len_k a multiple of 8, the query-tile kernel can leave dS -- or
+    dS and P -- in a workspace for dK (and dV) workgroups that read them back (hstu_jagged_bwd_workspace_size asks for
+    it where that pays; HSTU_MI355_BWD_HANDOFF=1 / 2 force the two orders).  Checked against the oracle and the
+    generic kernels with the workspace full of NaN, and against the two-launch order."""
     kw = dict(kw)
     w = make(batch=3, heads=kw.pop("heads", 2), seed=len(kw) + 60, **kw)
     if mask == "custom":
@@ -160,23 +161,28 @@ def test_ds_handed_to_the_dk_workgroups_through_a_workspace(kw, mask, monkeypatc
         w = dataclasses.replace(w, mask=m, mask_type=3, num_context=None, num_target=None, target_group_size=0)
     elif mask == "none":
         w = dataclasses.replace(w, mask_type=2, num_context=None, num_target=None, target_group_size=0)
-    monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "1")  # (batches this small take two launches by the library's own rule)
-    check(w, monkeypatch)
+    tol = 1e-2 if w.q.dtype == torch.bfloat16 else 2e-3
     g = torch.Generator(device=DEV).manual_seed(6)
     grad_out = torch.randn(w.q.shape[0], w.q.shape[1], w.v.shape[2], generator=g, device=DEV).to(w.q.dtype)
-    monkeypatch.setenv("HSTU_MI355_GENERIC_BACKWARD", "0")
-    monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "0")
-    two = device_grads(w, grad_out)
-    monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "1")
-    three = device_grads(w, grad_out)
-    assert torch.equal(two[0], three[0]) and torch.equal(two[2], three[2])  # dq and dv: the same arithmetic
-    # a caller that does not bring the workspace the library asked for gets the two-launch order
-    monkeypatch.setenv("HSTU_MI355_POISON_WORKSPACE", "withhold")
-    without = device_grads(w, grad_out)
-    assert all(torch.equal(x, y) for x, y in zip(two[:3], without[:3]))
-    scale = two[1].float().abs().max().item()
-    tol = 1e-2 if w.q.dtype == torch.bfloat16 else 2e-3
-    torch.testing.assert_close(three[1].float(), two[1].float(), atol=tol * scale, rtol=tol)
+    for order in ("1", "2"):  # three launches (dS handed over) and the planes order (dS and P handed over)
+        monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", order)
+        monkeypatch.setenv("HSTU_MI355_POISON_WORKSPACE", "1")
+        check(w, monkeypatch)  # against the oracle and the generic kernels
+        monkeypatch.setenv("HSTU_MI355_GENERIC_BACKWARD", "0")
+        monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "0")
+        two = device_grads(w, grad_out)
+        monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", order)
+        other = device_grads(w, grad_out)
+        assert torch.equal(two[0], other[0])  # dq: the same kernel arithmetic in every order
+        if order == "1":
+            assert torch.equal(two[2], other[2])  # dv as well
+        for i in (1, 2):  # dk from the stored dS, dv from the stored P: rounded at the same points
+            scale = two[i].float().abs().max().item()
+            torch.testing.assert_close(other[i].float(), two[i].float(), atol=tol * scale, rtol=tol)
+        # a caller that does not bring the workspace the library asked for gets the two-launch order
+        monkeypatch.setenv("HSTU_MI355_POISON_WORKSPACE", "withhold")
+        without = device_grads(w, grad_out)
+        assert all(torch.equal(x, y) for x, y in zip(two[:3], without[:3]))
 
 
 def test_no_mask(monkeypatch):
@@ -226,8 +232,9 @@ def test_ds_hand_over_with_more_keys_than_queries(rab, monkeypatch):
 
 def test_random_shapes_in_both_launch_orders(monkeypatch):
     """60 seeded random cases (head dims, grouped heads, lengths from empty to 1030, context / targets, every mask
-    type, with and without attn_bias, both index types): the three-launch order, its workspace full of NaN, against
-    the two-launch order -- dq, dv and the bias gradient bit for bit, dk to rounding."""
+    type, with and without attn_bias, both index types): the three-launch and the planes order, their workspace
+    full of NaN, against the two-launch order -- dq and the bias gradient bit for bit, dv as well with three launches,
+    what is computed from a stored dS or P to rounding."""
     import random
 
     rnd = random.Random(5)
@@ -257,15 +264,19 @@ def test_random_shapes_in_both_launch_orders(monkeypatch):
         grad_out = torch.randn(w.q.shape[0], heads, w.v.shape[2], generator=g, device=DEV).to(w.q.dtype)
         monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "0")
         two = device_grads(w, grad_out)
-        monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "1")
-        three = device_grads(w, grad_out)
         label = f"case {case}: {kw}, mask_type {mask_type}"
-        assert all(torch.isfinite(t).all() for t in three if t is not None), label
-        assert torch.equal(two[0], three[0]) and torch.equal(two[2], three[2]), label
-        assert two[3] is None or torch.equal(two[3], three[3]), label
-        scale = max(two[1].float().abs().max().item(), 1e-6)
         tol = 1e-2 if w.q.dtype == torch.bfloat16 else 2e-3
-        assert (two[1].float() - three[1].float()).abs().max().item() <= tol * scale, label
+        for order in ("1", "2"):  # (2: dS and P through the workspace; with an attn_bias gradient it is order 1 again)
+            monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", order)
+            other = device_grads(w, grad_out)
+            assert all(torch.isfinite(t).all() for t in other if t is not None), label
+            assert torch.equal(two[0], other[0]), label
+            assert two[3] is None or torch.equal(two[3], other[3]), label
+            if order == "1":
+                assert torch.equal(two[2], other[2]), label
+            for i in (1, 2):
+                scale = max(two[i].float().abs().max().item(), 1e-6)
+                assert (two[i].float() - other[i].float()).abs().max().item() <= tol * scale, label
 
 
 def test_long_sequences_and_rows_past_the_last_offset(monkeypatch):

@@ -5,8 +5,9 @@ The oracle (autograd on the fp32 golden path) cannot finish these sizes in secon
     launch wrote for them, against autograd on the oracle for those sequences alone (sequences are independent);
   * size-independent properties: the gradients are linear in grad_out (doubling it doubles every gradient exactly: a
     power of two commutes with every rounding on the way), bitwise reproducible, finite with the dS workspace
-    filled with NaN beforehand, and the two launch orders of the library (dK workgroups that recompute dS / that read
-    the query-tile kernel's dS back) agree: bit for bit in dq, dv and the attn_bias gradient, to rounding in dk.
+    filled with NaN beforehand, and the launch orders of the library (dK workgroups that recompute dS / that read the
+    query-tile kernel's dS back / dV workgroups that read its P back as well) agree: bit for bit in dq and the
+    attn_bias gradient, to rounding in what is computed from a stored dS or P.
 Tolerances as in tests/test_gpu_backward.py: 1e-2 of the largest reference value (bf16).
 """
 
@@ -44,11 +45,11 @@ def config(request):
     torch.cuda.empty_cache()
 
 
-@pytest.mark.parametrize("order", ["library's choice", "two launches", "three launches"])
+@pytest.mark.parametrize("order", ["library's choice", "two launches", "three launches", "planes"])
 def test_subbatch_matches_autograd_on_the_oracle(config, order, monkeypatch):
     name, w, grad_out = config
     if order != "library's choice":
-        monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "0" if order == "two launches" else "1")
+        monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", {"two launches": "0", "three launches": "1", "planes": "2"}[order])
     monkeypatch.setenv("HSTU_MI355_POISON_WORKSPACE", "1")
     dq, dk, dv, dbias = backward(w, grad_out)
     for t in (dq, dk, dv) + ((dbias,) if dbias is not None else ()):
@@ -83,15 +84,19 @@ def test_linear_in_grad_out_and_reproducible(config):
         assert torch.equal(a * 2, c)
 
 
-def test_the_two_launch_orders_agree(config, monkeypatch):
+def test_the_launch_orders_agree(config, monkeypatch):
     name, w, grad_out = config
     monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "0")
     two = backward(w, grad_out)
-    monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "1")
     monkeypatch.setenv("HSTU_MI355_POISON_WORKSPACE", "1")
-    three = backward(w, grad_out)
-    assert torch.equal(two[0], three[0]) and torch.equal(two[2], three[2])
-    if two[3] is not None:
-        assert torch.equal(two[3], three[3])
-    scale = two[1].float().abs().max().item()
-    torch.testing.assert_close(three[1].float(), two[1].float(), atol=1e-2 * scale, rtol=1e-2)
+    for order in ("1", "2"):
+        monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", order)
+        other = backward(w, grad_out)
+        assert torch.equal(two[0], other[0])
+        if order == "1":
+            assert torch.equal(two[2], other[2])
+        if two[3] is not None:
+            assert torch.equal(two[3], other[3])
+        for i in (1, 2):
+            scale = two[i].float().abs().max().item()
+            torch.testing.assert_close(other[i].float(), two[i].float(), atol=1e-2 * scale, rtol=1e-2)
