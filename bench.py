@@ -474,10 +474,10 @@ def main() -> int:
             "flops_per_step": bwd_flops,
             "tflops": round(bwd_flops / (bwd_ms * 1e-3) / 1e12, 3),
             "pct_of_bf16_mfma_peak": round(100.0 * bwd_flops / (bwd_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 2),
-            "note": "through torch.ops.ops_rec.hstu_jagged_backward: dV workgroups of hstu_bwd_dkv_kernel (which also clear "
-            "the attn_bias gradient when there is one), hstu_bwd_dq_kernel, which leaves dS in that gradient or in a workspace, "
-            "and dK workgroups that read it back (six products issued for the five of the formula); two launches and "
-            "eight products at head dims up to 64 without an attn_bias gradient and for planes above 4 GiB",
+            "note": "through torch.ops.ops_rec.hstu_jagged_backward, in the order the library picks for the shape: on this "
+            "workload hstu_bwd_dq_kernel storing dS and P, then hstu_bwd_dkv_kernel with a dV and a dK workgroup per key "
+            "tile that read them back (the five products of the formula issued once each); with an attn_bias gradient, "
+            "head dims up to 64 or long rows two or three launches that recompute S (and dP)",
         }
 
     if legs["backward"] and not fp8:

@@ -176,13 +176,14 @@ HSTU_API uint64_t hstu_jagged_fwd_noalloc_max_workspace(void);
  * need not clear them.  grad_attn_bias (optional; requires attn_bias): written in full as well -- zeros outside
  * the part of a sequence's [S_q, S_k] corner that its query tiles sweep -- so the caller need not clear it either
  * (the kernel that produces grad_v clears it beside its work).
- * Workspace (optional): the tuned kernels run as three launches -- grad_v, then grad_q, which leaves dS behind,
- * then grad_k from that dS -- when dS has somewhere to stay: in grad_attn_bias (which is dS) when that is asked
- * for, otherwise in a workspace of [batch, num_heads_q, max_seq_len_q, max_seq_len_k] elements of the input
- * type, which hstu_jagged_bwd_workspace_size asks for when it pays (head dims above 64, max_seq_len_k a multiple
- * of 8, at most 4 GiB or HSTU_MI355_BWD_WORKSPACE_MB in the environment).  Without the workspace, or with less
- * than was asked for, the call still works: two launches in which the grad_k workgroups recompute dS.  The
- * workspace needs no clearing and holds nothing afterwards. */
+ * Workspace (optional): the tuned kernels recompute nothing, or less, when the query-tile kernel's dS (and P) have
+ * somewhere to stay until the kernels that produce grad_k (and grad_v) read them back: dS in grad_attn_bias (which
+ * is dS) when that is asked for, otherwise in a workspace of [batch, num_heads_q, max_seq_len_q, max_seq_len_k]
+ * elements of the input type -- twice that (rounded up to whole 32-key blocks) for dS and P together --, which
+ * hstu_jagged_bwd_workspace_size asks for where it was measured to pay (head dims above 64, max_seq_len_k a
+ * multiple of 8 and at most 2048, at most 4 GiB or HSTU_MI355_BWD_WORKSPACE_MB in the environment).  Without the
+ * workspace, or with less than was asked for, the call still works: the kernels that produce grad_k then recompute
+ * dS.  The workspace needs no clearing and holds nothing afterwards. */
 typedef struct hstu_jagged_bwd_params {
     uint32_t struct_size; /* sizeof(hstu_jagged_bwd_params) */
     uint32_t reserved0;

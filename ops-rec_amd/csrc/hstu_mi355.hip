@@ -540,18 +540,20 @@ HSTU_API int hstu_paged_fwd(const hstu_paged_fwd_params* p, void* workspace, uin
 //                    work), otherwise it goes into a workspace of that shape, [batch, heads, max_seq_len_q,
 //                    max_seq_len_k] in the input type;
 //   planes           the query-tile kernel storing dS and P, then a dV workgroup that reads P and a dK workgroup that
-//                    reads dS per key tile: the five products of the formula, nothing computed twice; two such planes
-//                    of workspace; only without an attn_bias gradient (which would have to be cleared first).
+//                    reads dS per key tile: the five products of the formula, nothing computed twice; a workspace of
+//                    twice that size (per query row and 32-key block the 32 dS values, then the 32 P values: a whole
+//                    128-byte line per row and step); only without an attn_bias gradient (which would have to be
+//                    cleared first).
 // Rows of 16 bytes are needed for the planes (max_seq_len_k a multiple of 8, 16-byte aligned pointers).  Nothing in a
 // workspace is cleared: the workgroups that read a plane read exactly the pieces the query-tile kernel wrote.
 //
 // Which order is taken follows what was measured (bf16, events through the operator, two launches -> three -> planes):
-//   C2 (B32 H4 d128 L278..1004)  162 -> 142 -> 125 us      B128 H4 d128 L64..512    175 -> 144 -> 133 us
-//   B8 H4 d128 L512..1024         88 -> 100 ->  70 us      B4 H4 d128 L300..700      65 ->  74 ->  54 us
-//   B16 H4 d256 L100..1504       402 -> 290 -> 212 us      B32 H8 d256 L1024       1285 -> 900 -> 800 us
-//   B64 H4 d128 L256..1024       269 -> 240 -> 245 us      B16 H4 d128 L512..2048   240 -> 219 -> 246 us
-//   B32 H8 d128 L1024            438 -> 418 -> 487 us      B32 H8 d64 L1024         277 -> 300 -> 408 us
-//   B4 H8 d128 L1024..4096       409 -> 509 -> 530 us      B2 H4 d128 L8192         738 -> 921 -> 1061 us
+//   C2 (B32 H4 d128 L278..1004)  163 -> 143 -> 119 us      B128 H4 d128 L64..512    175 -> 147 -> 131 us
+//   B8 H4 d128 L512..1024         88 -> 100 ->  69 us      B4 H4 d128 L300..700      64 ->  75 ->  52 us
+//   B16 H4 d256 L100..1504       401 -> 291 -> 216 us      B32 H8 d256 L1024       1275 -> 889 -> 827 us
+//   B64 H4 d128 L256..1024       266 -> 239 -> 254 us      B16 H4 d128 L512..2048   237 -> 220 -> 257 us
+//   B32 H8 d128 L1024            442 -> 422 -> 492 us      B32 H8 d64 L1024         261 -> 295 -> 403 us
+//   B4 H8 d128 L1024..4096       406 -> 508 -> 520 us      B2 H4 d128 L8192         732 -> 924 -> 1255 us
 // A plane costs 4 bytes of traffic per (query, key) pair, written and read back, against two products of
 // 4 x head dim flops per pair each: it pays from the head-dim slot 128 on, and at 128 the second plane only while both
 // stay in the memory-side cache (256 MB) between the launches; few long sequences lose either way (each launch is
