@@ -560,8 +560,9 @@ HSTU_API int hstu_paged_fwd(const hstu_paged_fwd_params* p, void* workspace, uin
 // as long as its heaviest workgroup).  The rule:
 //   without an attn_bias gradient, head dims above 64, max_seq_len_k up to 2048, workspace within the limit (4 GiB,
 //   or HSTU_MI355_BWD_WORKSPACE_MB in the environment):  planes for head dims above 128, and for those up to 128 when
-//   total_q x max_seq_len_k x heads x 2 bytes -- an upper bound of what the two planes hold under a causal mask,
-//   doubled for the other mask types -- is at most 200 MB; else three launches from 512 workgroups per launch on
+//   the plane holds at most about 120 MB (estimated from total_q, the batch and max_seq_len: C2 103 MB, B128 H4
+//   L64..512 85 MB; B32 H8 L512 unpadded 134 MB: 132 us with three launches, 141 us with planes); else three launches
+//   from 512 workgroups per launch on
 //   (key tiles x sequences x K/V heads: B8 H4 d128 L512..1024 and smaller lose with three); else two;
 //   with an attn_bias gradient: three launches from 512 workgroups per launch on when the head dims are above 128
 //   (B16 H4 d256 L100..1504 501 -> 404 us), max_seq_len_k is at most 1024 (B64 H4 d128 L256..1024 431 -> 382 us,
@@ -616,8 +617,12 @@ static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
     if (dmax <= 64 || f->max_seq_len_k > 2048) {
         return two;
     }
-    const int64_t held = f->total_q * f->max_seq_len_k * f->num_heads_q * 2 * (f->mask_type == HSTU_MASK_TRIL ? 1 : 2);
-    if (planes_fit && (dmax > 128 || held <= 200LL * 1000 * 1000)) {
+    // what the plane holds under a causal mask, sum of L^2 / 2 pairs x 4 bytes per head, estimated from what the host
+    // knows as (mean L) x max_seq_len_k x batch with the mean taken twice for padded batches; doubled for other masks
+    const double fill = static_cast<double>(f->total_q) / static_cast<double>(batch * f->max_seq_len_q);
+    const double held = static_cast<double>(f->total_q) * fill * static_cast<double>(f->max_seq_len_k) * f->num_heads_q * 2.0 *
+                        (f->mask_type == HSTU_MASK_TRIL ? 1.0 : 2.0);
+    if (planes_fit && (dmax > 128 || held <= 120e6)) {
         return planes;
     }
     return (three_fits && many_tiles) ? three : two;
