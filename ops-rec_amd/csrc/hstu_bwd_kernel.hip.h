@@ -664,16 +664,19 @@ __global__ __launch_bounds__(kDkvThreads, (MODE == 2 || MODE == 4) ? bwd_dk_from
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = uniform(tid >> 6);
-    // even workgroups produce dV, odd ones dK of the same key tile (neighbours in the grid, so that they tend to
-    // run side by side and find each other's Q / dO rows in the L2)
+    // In the launches with both roles the dV and the dK workgroup of a key tile are 8 apart in the grid: workgroups go
+    // to the 8 XCDs in turn, so the two land on one XCD and find each other's Q / dO rows (MODE 0), or the other half of
+    // every line of the dS / P plane (MODE 4), in its L2.  (The host rounds the grid up to whole groups of 16; the
+    // slots past the last tile leave below like those of absent tiles.)
     constexpr bool from_plane = MODE == 2 || MODE == 4;
-    const bool dk_role = (MODE == 0 || MODE == 4) ? (blockIdx.x & 1) != 0 : MODE == 2;
+    constexpr bool paired = MODE == 0 || MODE == 4;
+    const bool dk_role = paired ? ((blockIdx.x >> 3) & 1) != 0 : MODE == 2;
     const int ln = lane & 31;
     const int lh = lane >> 5;
 
     // key tile 0 is seen by the most query rows: heaviest first
     const int per_level = a.n_batch * a.n_heads_k;
-    const int tile_slot = static_cast<int>((MODE == 0 || MODE == 4) ? blockIdx.x >> 1 : blockIdx.x);
+    const int tile_slot = static_cast<int>(paired ? (blockIdx.x >> 4) * 8 + (blockIdx.x & 7) : blockIdx.x);
     const int kt_idx = tile_slot / per_level;
     const int rem = tile_slot - kt_idx * per_level;
     const int b = rem / a.n_heads_k;

@@ -548,12 +548,12 @@ HSTU_API int hstu_paged_fwd(const hstu_paged_fwd_params* p, void* workspace, uin
 // workspace is cleared: the workgroups that read a plane read exactly the pieces the query-tile kernel wrote.
 //
 // Which order is taken follows what was measured (bf16, events through the operator, two launches -> three -> planes):
-//   C2 (B32 H4 d128 L278..1004)  163 -> 143 -> 119 us      B128 H4 d128 L64..512    175 -> 147 -> 131 us
-//   B8 H4 d128 L512..1024         88 -> 100 ->  69 us      B4 H4 d128 L300..700      64 ->  75 ->  52 us
-//   B16 H4 d256 L100..1504       401 -> 291 -> 216 us      B32 H8 d256 L1024       1275 -> 889 -> 827 us
-//   B64 H4 d128 L256..1024       266 -> 239 -> 254 us      B16 H4 d128 L512..2048   237 -> 220 -> 257 us
-//   B32 H8 d128 L1024            442 -> 422 -> 492 us      B32 H8 d64 L1024         261 -> 295 -> 403 us
-//   B4 H8 d128 L1024..4096       406 -> 508 -> 520 us      B2 H4 d128 L8192         732 -> 924 -> 1255 us
+//   C2 (B32 H4 d128 L278..1004)  161 -> 142 -> 109 us      B128 H4 d128 L64..512    166 -> 146 -> 123 us
+//   B8 H4 d128 L512..1024         85 ->  99 ->  65 us      B4 H4 d128 L300..700      64 ->  74 ->  49 us
+//   B16 H4 d256 L100..1504       396 -> 290 -> 213 us      B32 H8 d256 L1024       1258 -> 897 -> 792 us
+//   B64 H4 d128 L256..1024       254 -> 238 -> 235 us      B16 H4 d128 L512..2048   234 -> 219 -> 244 us
+//   B32 H8 d128 L1024            441 -> 430 -> 447 us      B32 H8 d64 L1024         257 -> 298 -> 359 us
+//   B4 H8 d128 L1024..4096       400 -> 503 -> 479 us      B2 H4 d128 L8192         743 -> 928 -> 1201 us
 // A plane costs 4 bytes of traffic per (query, key) pair, written and read back, against two products of
 // 4 x head dim flops per pair each: it pays from the head-dim slot 128 on, and at 128 the second plane only while both
 // stay in the memory-side cache (256 MB) between the launches; few long sequences lose either way (each launch is
@@ -724,7 +724,9 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
     const bool generic = is_generic_bwd(var);
     const BwdPlan plan = plan_bwd(p, var);
     // the tuned key-tile kernel runs a dV and a dK workgroup per tile, the generic one a workgroup per tile
-    const int64_t grid_kv = (generic ? 1 : 2) * static_cast<int64_t>(a.n_ktiles) * a.n_batch * a.n_heads_k;
+    const int64_t n_kv_slots = static_cast<int64_t>(a.n_ktiles) * a.n_batch * a.n_heads_k;
+    // (with both roles in a launch: groups of 8 dV workgroups followed by their 8 dK workgroups, whole groups)
+    const int64_t grid_kv = generic ? n_kv_slots : 16 * ((n_kv_slots + 7) / 8);
     const int64_t grid_q = static_cast<int64_t>(a.n_qtiles) * a.n_batch * a.n_heads_q;
     if (grid_kv > 0x7fffffffLL || grid_q > 0x7fffffffLL) {
         return fail(HSTU_ERR_INVALID, "grid out of range");
@@ -762,11 +764,11 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
         // dV workgroups (which clear the attn_bias gradient beside their work), the query-tile kernel (which writes
         // dS into it, or into the workspace), dK workgroups (which read dS back)
         a.drab_clear_bytes = drab_bytes;
-        hipLaunchKernelGGL(var->dv_only, dim3(static_cast<unsigned>(grid_kv / 2)), dim3(hstu::kDkvThreads), 0,
+        hipLaunchKernelGGL(var->dv_only, dim3(static_cast<unsigned>(n_kv_slots)), dim3(hstu::kDkvThreads), 0,
                            static_cast<hipStream_t>(stream), a);
         a.drab_clear_bytes = 0;
         hipLaunchKernelGGL(var->dq_drab, dim3(static_cast<unsigned>(grid_q)), dim3(256), 0, static_cast<hipStream_t>(stream), a);
-        hipLaunchKernelGGL(var->dk_from_ds, dim3(static_cast<unsigned>(grid_kv / 2)), dim3(hstu::kDkvThreads), 0,
+        hipLaunchKernelGGL(var->dk_from_ds, dim3(static_cast<unsigned>(n_kv_slots)), dim3(hstu::kDkvThreads), 0,
                            static_cast<hipStream_t>(stream), a);
         const hipError_t err3 = hipGetLastError();
         if (err3 != hipSuccess) {
