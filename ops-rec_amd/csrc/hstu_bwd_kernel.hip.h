@@ -263,6 +263,13 @@ __global__ __launch_bounds__(256, bwd_dq_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void 
     const int lh = lane >> 5;
 
     // heaviest (last) query tiles first
+    if constexpr (STORE == 2) {
+        if (a.drab_clear_bytes > 0) {
+            // (the order in which the dK workgroups of the next launch write the attn_bias gradient: cleared here,
+            // beside this kernel's work, by all workgroups alike)
+            clear_share(a.drab, a.drab_clear_bytes, blockIdx.x, gridDim.x, threadIdx.x, 256);
+        }
+    }
     const int per_level = a.n_batch * a.n_heads_q;
     const int lvl = static_cast<int>(blockIdx.x) / per_level;
     const int rem = static_cast<int>(blockIdx.x) - lvl * per_level;
@@ -636,15 +643,16 @@ __global__ __launch_bounds__(256, bwd_dq_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void 
 // MODE 0: a dV and a dK workgroup per key tile (even / odd workgroups).  MODE 1 and 2 serve the three-launch order
 // dV / dQ / dK: all workgroups of a launch have one role, and the dK ones (MODE 2; rab and mask play no part in it)
 // take dS from the attn_bias gradient that the query-tile kernel wrote between the two launches.
-// MODE 4: launched after a query-tile kernel that stored dS and P: a workgroup that takes dV from P (even) and one
-// that takes dK from dS (odd) per key tile, both of MODE 2's build (one product each; the dV ones stream dO
-// where the dK ones stream Q).
+// MODE 4: launched after a query-tile kernel that stored dS and P: a workgroup that takes dV from P and one that
+// takes dK from dS per key tile, both of MODE 2's build (one product each; the dV ones stream dO where the dK ones
+// stream Q).  MODE 5: the same, and the dK workgroups write the dS pieces they read into the attn_bias gradient, which
+// the query-tile kernel cleared beside its work: the order for a call that wants that gradient.
 template <typename Tag, int D, bool HAS_RAB, bool HAS_MASK, int MODE = 0>
-__global__ __launch_bounds__(kDkvThreads, (MODE == 2 || MODE == 4) ? bwd_dk_from_ds_wgs_per_cu(D) : bwd_dkv_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hstu_bwd_dkv_kernel(const BwdArgs a)
+__global__ __launch_bounds__(kDkvThreads, (MODE == 2 || MODE >= 4) ? bwd_dk_from_ds_wgs_per_cu(D) : bwd_dkv_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hstu_bwd_dkv_kernel(const BwdArgs a)
 {
     typedef SubTile<D> T;
     constexpr int LPW = T::LPW, NLW = T::NLW, KSTEPS = T::KSTEPS, MTILES = T::MTILES, NCH = 2 * T::MTILES;
-    constexpr int kHalves = (MODE == 2 || MODE == 4) ? 1 : 2;  // (a workgroup that reads dS or P streams Q or dO only)
+    constexpr int kHalves = (MODE == 2 || MODE >= 4) ? 1 : 2;  // (a workgroup that reads dS or P streams Q or dO only)
     // four stages, each the Q sub-tile followed by the dO sub-tile (separate arrays per stage, see the dQ kernel;
     // Q and dO of a stage share an array so that a wavefront can address "the tile of my role" by an offset)
     __shared__ __attribute__((aligned(1024))) uint16_t s_st0[kHalves * T::ELEMS];
@@ -655,7 +663,7 @@ __global__ __launch_bounds__(kDkvThreads, (MODE == 2 || MODE == 4) ? bwd_dk_from
     // (plus, in MODE 2, the two loads of the next step's dS rows, issued between the two requests.  Reading rab / mask
     // rows a step ahead in the same way was tried for the other modes: nothing for the dV-only launch, 277 -> 314 us
     // at C3 for the two-role one, which has no registers to spare at the head-dim slot 128.)
-    constexpr int kAhead = (MODE == 2 || MODE == 4) ? 2 : 0;
+    constexpr int kAhead = (MODE == 2 || MODE >= 4) ? 2 : 0;  // (MODE 5's stores only make the wait stricter: the count must hold from the first step on)
     constexpr int kReqs = 2 * kHalves * LPW + kAhead;
     constexpr int kWaitStage = (kReqs & 15) | (7 << 4) | (15 << 8) | ((kReqs >> 4) << 14);
     constexpr uint32_t kPastEnd = 0x40000000u;
@@ -668,8 +676,8 @@ __global__ __launch_bounds__(kDkvThreads, (MODE == 2 || MODE == 4) ? bwd_dk_from
     // to the 8 XCDs in turn, so the two land on one XCD and find each other's Q / dO rows (MODE 0), or the other half of
     // every line of the dS / P plane (MODE 4), in its L2.  (The host rounds the grid up to whole groups of 16; the
     // slots past the last tile leave below like those of absent tiles.)
-    constexpr bool from_plane = MODE == 2 || MODE == 4;
-    constexpr bool paired = MODE == 0 || MODE == 4;
+    constexpr bool from_plane = MODE == 2 || MODE >= 4;
+    constexpr bool paired = MODE == 0 || MODE >= 4;
     const bool dk_role = paired ? ((blockIdx.x >> 3) & 1) != 0 : MODE == 2;
     const int ln = lane & 31;
     const int lh = lane >> 5;
@@ -873,14 +881,14 @@ __global__ __launch_bounds__(kDkvThreads, (MODE == 2 || MODE == 4) ? bwd_dk_from
         ++ds_steps;
         // (MODE 4: dS and P share a plane of their own layout, see the query-tile kernel: per row and 32-key block, 32
         // dS values followed by 32 P values)
-        const uint32_t pitch = MODE == 4 ? 64u * static_cast<uint32_t>((a.max_k + 31) / 32) : static_cast<uint32_t>(a.max_k);
+        const uint32_t pitch = MODE >= 4 ? 64u * static_cast<uint32_t>((a.max_k + 31) / 32) : static_cast<uint32_t>(a.max_k);
         const __amdgpu_buffer_rsrc_t ds_rsrc = make_rsrc(
-            static_cast<const uint16_t*>(MODE == 4 ? a.p_plane : a.drab) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(pitch),
+            static_cast<const uint16_t*>(MODE >= 4 ? a.p_plane : a.drab) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(pitch),
             static_cast<uint32_t>(a.max_q) * pitch * 2u);
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int key0 = cw0 + 16 * j + 8 * lh;
-            const uint32_t col = MODE == 4 ? static_cast<uint32_t>(2 * cw0 + 16 * j + 8 * lh + (dk_role ? 0 : 32)) : static_cast<uint32_t>(key0);
+            const uint32_t col = MODE >= 4 ? static_cast<uint32_t>(2 * cw0 + 16 * j + 8 * lh + (dk_role ? 0 : 32)) : static_cast<uint32_t>(key0);
             const uint32_t off = (wanted && rq0 + ln < sq && key0 < sk)
                                      ? (static_cast<uint32_t>(rq0 + ln) * pitch + col) * 2u
                                      : kOutOfRange;
@@ -936,6 +944,29 @@ __global__ __launch_bounds__(kDkvThreads, (MODE == 2 || MODE == 4) ? bwd_dk_from
         }
         __builtin_amdgcn_sched_barrier(0);
         request(stage_o);
+        if constexpr (MODE == 5) {
+            // d rab = dS: the 16-byte pieces just read (row rq0 + ln, keys cw0 + 16 j + 8 lh .. + 7) go to the attn_bias
+            // gradient as they are; both stores every step (out of range when there is nothing to write), behind the
+            // step's loads, so that no load waits for them
+            if (dk_role) {
+                const __amdgpu_buffer_rsrc_t drab_rsrc = make_rsrc(
+                    static_cast<uint16_t*>(a.drab) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k),
+                    bias_bytes);
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int key0 = cw0 + 16 * j + 8 * lh;
+                    const uint32_t off = (active && rq0 + ln < sq && key0 < sk)
+                                             ? (static_cast<uint32_t>(rq0 + ln) * static_cast<uint32_t>(a.max_k) + static_cast<uint32_t>(key0)) * 2u
+                                             : kOutOfRange;
+                    __builtin_amdgcn_raw_buffer_store_b128(ra[j], drab_rsrc, static_cast<int>(off), 0, 0);
+                }
+            } else {
+                // (the dV workgroups keep the same count of requests in flight)
+                const __amdgpu_buffer_rsrc_t none = make_rsrc(static_cast<uint16_t*>(nullptr), 0u);
+                __builtin_amdgcn_raw_buffer_store_b128(ra[0], none, static_cast<int>(kOutOfRange), 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b128(ra[1], none, static_cast<int>(kOutOfRange), 0, 0);
+            }
+        }
         __builtin_amdgcn_sched_barrier(0);
         if constexpr (from_plane) {
           if (active) {

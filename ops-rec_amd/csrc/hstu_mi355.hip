@@ -542,8 +542,8 @@ HSTU_API int hstu_paged_fwd(const hstu_paged_fwd_params* p, void* workspace, uin
 //   planes           the query-tile kernel storing dS and P, then a dV workgroup that reads P and a dK workgroup that
 //                    reads dS per key tile: the five products of the formula, nothing computed twice; a workspace of
 //                    twice that size (per query row and 32-key block the 32 dS values, then the 32 P values: a whole
-//                    128-byte line per row and step); only without an attn_bias gradient (which would have to be
-//                    cleared first).
+//                    128-byte line per row and step).  With an attn_bias gradient the query-tile kernel clears it
+//                    beside its work and the dK workgroups write the dS pieces they read into it.
 // Rows of 16 bytes are needed for the planes (max_seq_len_k a multiple of 8, 16-byte aligned pointers).  Nothing in a
 // workspace is cleared: the workgroups that read a plane read exactly the pieces the query-tile kernel wrote.
 //
@@ -558,18 +558,23 @@ HSTU_API int hstu_paged_fwd(const hstu_paged_fwd_params* p, void* workspace, uin
 // 4 x head dim flops per pair each: it pays from the head-dim slot 128 on, and at 128 the second plane only while both
 // stay in the memory-side cache (256 MB) between the launches; few long sequences lose either way (each launch is
 // as long as its heaviest workgroup).  The rule:
-//   without an attn_bias gradient, head dims above 64, max_seq_len_k up to 2048, workspace within the limit (4 GiB,
-//   or HSTU_MI355_BWD_WORKSPACE_MB in the environment):  planes for head dims above 128, and for those up to 128 when
-//   the plane holds at most about 120 MB (estimated from total_q, the batch and max_seq_len: C2 103 MB, B128 H4
-//   L64..512 85 MB; B32 H8 L512 unpadded 134 MB: 132 us with three launches, 141 us with planes); else three launches
-//   from 512 workgroups per launch on
-//   (key tiles x sequences x K/V heads: B8 H4 d128 L512..1024 and smaller lose with three); else two;
-//   with an attn_bias gradient: three launches from 512 workgroups per launch on when the head dims are above 128
-//   (B16 H4 d256 L100..1504 501 -> 404 us), max_seq_len_k is at most 1024 (B64 H4 d128 L256..1024 431 -> 382 us,
-//   B128 H4 d64 L64..512 177 -> 146 us) or the batch has no padding, total_q = batch x max_seq_len_q (B32 H8 d128
-//   L2048 2599 -> 2311 us, B32 H8 d32 L4096 8013 -> 6810 us); not for long jagged batches, where the clearing of the
-//   gradient no longer hides behind the dV workgroups alone (B32 H4 d64 L100..1504 310 -> 341 us, B8 H8 d128
-//   L1024..4096 1492 -> 1657 us; C3 396 -> 401 us).
+//   head dims above 128 (workspace within the limit: 4 GiB, or HSTU_MI355_BWD_WORKSPACE_MB in the environment): planes,
+//   with or without an attn_bias gradient -- with one the query-tile kernel clears it beside its work and the dK
+//   workgroups write the dS pieces they read into it (B32 H8 d256 L1024 with d rab 1632 -> 1196 -> 1046 us, B8 H4 d256
+//   L512..1024 203 -> 213 -> 139 us, B32 H4 d192 L256..1024 502 -> 402 -> 296 us); long rows included (no d rab: B4 H4
+//   d256 L1024..4096 885 -> 613 -> 465 us, B8 H4 d256 L4096 1845 -> 1257 -> 1135 us) up to max_seq_len_k 4096, three
+//   launches beyond (B2 H4 d256 L8192 1794 -> 1343 -> 1444 us);
+//   head dims 65 .. 128 without an attn_bias gradient, max_seq_len_k up to 2048:  planes when the plane holds at most
+//   about 120 MB (estimated from total_q, the batch and max_seq_len: C2 103 MB, B128 H4 L64..512 85 MB; B32 H8 L512
+//   unpadded 134 MB: 132 us with three launches, 141 us with planes); else three launches from 512 workgroups per
+//   launch on (key tiles x sequences x K/V heads: B8 H4 d128 L512..1024 and smaller lose with three); else two;
+//   head dims up to 128 with an attn_bias gradient: three launches from 512 workgroups per launch on when
+//   max_seq_len_k is at most 1024 (B64 H4 d128 L256..1024 431 -> 382 us, B128 H4 d64 L64..512 177 -> 146 us) or the
+//   batch has no padding, total_q = batch x max_seq_len_q (B32 H8 d128 L2048 2599 -> 2311 us, B32 H8 d32 L4096
+//   8013 -> 6810 us); not for long jagged batches, where the clearing of the gradient no longer hides behind the dV
+//   workgroups alone (B32 H4 d64 L100..1504 310 -> 341 us, B8 H8 d128 L1024..4096 1492 -> 1657 us; C3 396 -> 401 us,
+//   planes 408 us);
+//   everything else (head dims up to 64 without an attn_bias gradient, long rows at head dims up to 128): two launches.
 // Also tried, not kept: the dV workgroups on a second stream beside the query-tile kernel (C2 143 -> 149 us), and the
 // query-tile kernel first with dV and dK-from-dS workgroups in one launch behind it (C2 160 us).
 // HSTU_MI355_BWD_HANDOFF in the environment overrides the rule: 0 = two launches, 1 = three wherever possible,
@@ -593,13 +598,17 @@ static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
     const int64_t dmax = f->head_dim_qk > f->head_dim_v ? f->head_dim_qk : f->head_dim_v;
     const int64_t n_ktiles = (f->max_seq_len_k + hstu::kBlockM - 1) / hstu::kBlockM;
     const bool many_tiles = n_ktiles * batch * f->num_heads_k >= 512;
-    if (p->grad_attn_bias != nullptr) {
-        const bool by_rule = many_tiles && (dmax > 128 || f->max_seq_len_k <= 1024 || f->total_q == batch * f->max_seq_len_q);
-        return (forced >= 1 || (forced < 0 && by_rule)) ? BwdPlan{kThreeLaunches, 0} : two;
-    }
     int64_t cap_mb = 4096;
     if (const char* const cap_env = getenv("HSTU_MI355_BWD_WORKSPACE_MB")) {
         cap_mb = atoll(cap_env);
+    }
+    if (p->grad_attn_bias != nullptr) {
+        const int64_t pair_bytes = batch * f->num_heads_q * f->max_seq_len_q * (64 * ((f->max_seq_len_k + 31) / 32)) * 2;
+        if ((forced == 2 || (forced < 0 && dmax > 128)) && var->dv_dk_from_planes_drab != nullptr && pair_bytes <= cap_mb * (1LL << 20)) {
+            return BwdPlan{kPlanes, static_cast<uint64_t>(pair_bytes)};
+        }
+        const bool by_rule = many_tiles && (dmax > 128 || f->max_seq_len_k <= 1024 || f->total_q == batch * f->max_seq_len_q);
+        return (forced >= 1 || (forced < 0 && by_rule)) ? BwdPlan{kThreeLaunches, 0} : two;
     }
     const int64_t plane = batch * f->num_heads_q * f->max_seq_len_q * f->max_seq_len_k * 2;
     const bool three_fits = plane <= cap_mb * (1LL << 20);
@@ -614,6 +623,9 @@ static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
     if (forced == 1) {
         return three_fits ? three : two;
     }
+    if (dmax > 128) {
+        return (planes_fit && f->max_seq_len_k <= 4096) ? planes : (three_fits ? three : two);
+    }
     if (dmax <= 64 || f->max_seq_len_k > 2048) {
         return two;
     }
@@ -622,7 +634,7 @@ static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
     const double fill = static_cast<double>(f->total_q) / static_cast<double>(batch * f->max_seq_len_q);
     const double held = static_cast<double>(f->total_q) * fill * static_cast<double>(f->max_seq_len_k) * f->num_heads_q * 2.0 *
                         (f->mask_type == HSTU_MASK_TRIL ? 1.0 : 2.0);
-    if (planes_fit && (dmax > 128 || held <= 120e6)) {
+    if (planes_fit && held <= 120e6) {
         return planes;
     }
     return (three_fits && many_tiles) ? three : two;
@@ -750,10 +762,14 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
             a.drab = workspace;
         }
         if (plan.order == kPlanes) {
-            // the query-tile kernel with dS and P, then a dV-from-P and a dK-from-dS workgroup per key tile
+            // the query-tile kernel with dS and P (clearing the attn_bias gradient beside its work when there is one),
+            // then a dV-from-P and a dK-from-dS workgroup per key tile (the latter writing dS into that gradient)
             a.p_plane = workspace;
+            a.drab_clear_bytes = drab_bytes;
             hipLaunchKernelGGL(var->dq_ds_p, dim3(static_cast<unsigned>(grid_q)), dim3(256), 0, static_cast<hipStream_t>(stream), a);
-            hipLaunchKernelGGL(var->dv_dk_from_planes, dim3(static_cast<unsigned>(grid_kv)), dim3(hstu::kDkvThreads), 0,
+            a.drab_clear_bytes = 0;
+            hipLaunchKernelGGL(p->grad_attn_bias != nullptr ? var->dv_dk_from_planes_drab : var->dv_dk_from_planes,
+                               dim3(static_cast<unsigned>(grid_kv)), dim3(hstu::kDkvThreads), 0,
                                static_cast<hipStream_t>(stream), a);
             const hipError_t err2 = hipGetLastError();
             if (err2 != hipSuccess) {

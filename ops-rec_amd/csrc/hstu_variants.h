@@ -33,6 +33,7 @@ struct BwdVariant {
     // the order dQ storing dS and P / dV workgroups that read P beside dK workgroups that read dS
     void (*dq_ds_p)(const BwdArgs);
     void (*dv_dk_from_planes)(const BwdArgs);
+    void (*dv_dk_from_planes_drab)(const BwdArgs);  // the dK workgroups also write dS to the attn_bias gradient
 };
 
 // forward, 16-bit inputs: [rab: 0, 1][custom mask: 0, 1][dim slot: 32, 64, 128, 256]
