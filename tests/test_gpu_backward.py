@@ -112,10 +112,10 @@ def test_custom_mask_and_rab_alignment(max_len, monkeypatch):
 ], ids=lambda kw: "-".join(f"{k}{v}" for k, v in kw.items() if k != "dtype"))  # fmt: skip
 @pytest.mark.parametrize("custom_mask", [False, True], ids=["causal", "custom"])
 def test_attn_bias_gradient_handed_to_the_dk_workgroups(kw, custom_mask, monkeypatch):
-    """With the attn_bias gradient asked for and 16-byte aligned bias rows the library runs dV workgroups, the
-    query-tile kernel and then dK workgroups that read dS back from the attn_bias gradient;
-    HSTU_MI355_BWD_HANDOFF=0 keeps the order in which the dK workgroups recompute it.  dq, dv and the bias gradient
-    come from the same arithmetic in both orders (bit-identical), dk from dS rounded at the same point."""
+    """With the attn_bias gradient asked for and 16-byte aligned bias rows the library can hand dS (and P) from the
+    query-tile kernel to the workgroups that produce dK (and dV); HSTU_MI355_BWD_HANDOFF=0 keeps the order in which
+    they recompute them.  dq and the bias gradient come out bit-identical in every order, dv as well while P is
+    recomputed; what is computed from a stored dS or P agrees to rounding."""
     kw = dict(kw)
     w = make(batch=3, heads=kw.pop("heads", 2), seed=len(kw) + 50, rab_std=0.5, **kw)
     assert w.max_seq_len % 8 == 0
@@ -124,20 +124,27 @@ def test_attn_bias_gradient_handed_to_the_dk_workgroups(kw, custom_mask, monkeyp
         shape = (3, w.q.shape[1], w.max_seq_len, w.max_seq_len)
         mask = (torch.rand(shape, generator=g, device=DEV) < 0.7).to(w.q.dtype)
         w = dataclasses.replace(w, mask=mask, mask_type=3, num_context=None, num_target=None, target_group_size=0)
-    monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "1")  # (batches this small take two launches by the library's own rule)
-    check(w, monkeypatch)
+    tol = 1e-2 if w.q.dtype == torch.bfloat16 else 2e-3
     g = torch.Generator(device=DEV).manual_seed(6)
     grad_out = torch.randn(w.q.shape[0], w.q.shape[1], w.v.shape[2], generator=g, device=DEV).to(w.q.dtype)
-    monkeypatch.setenv("HSTU_MI355_GENERIC_BACKWARD", "0")
-    monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "0")
-    two = device_grads(w, grad_out)
-    monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "1")
-    three = device_grads(w, grad_out)
-    for name, i in (("dq", 0), ("dv", 2), ("dbias", 3)):
-        assert torch.equal(two[i], three[i]), name
-    scale = two[1].float().abs().max().item()
-    tol = 1e-2 if w.q.dtype == torch.bfloat16 else 2e-3
-    torch.testing.assert_close(three[1].float(), two[1].float(), atol=tol * scale, rtol=tol)
+    # 1: dV workgroups / query-tile kernel storing dS into the gradient / dK workgroups reading it;  2: query-tile
+    # kernel storing dS and P into a workspace and clearing the gradient / dV and dK workgroups reading them, the dK
+    # ones writing the gradient
+    for order in ("1", "2"):
+        monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", order)
+        monkeypatch.setenv("HSTU_MI355_POISON_WORKSPACE", "1")
+        check(w, monkeypatch)
+        monkeypatch.setenv("HSTU_MI355_GENERIC_BACKWARD", "0")
+        monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "0")
+        two = device_grads(w, grad_out)
+        monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", order)
+        other = device_grads(w, grad_out)
+        assert torch.equal(two[0], other[0]) and torch.equal(two[3], other[3])  # dq and the bias gradient: the same bits
+        if order == "1":
+            assert torch.equal(two[2], other[2])
+        for i in (1, 2):
+            scale = two[i].float().abs().max().item()
+            torch.testing.assert_close(other[i].float(), two[i].float(), atol=tol * scale, rtol=tol)
 
 
 @pytest.mark.parametrize("kw", [
