@@ -640,7 +640,7 @@ __global__ __launch_bounds__(256, bwd_dq_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void 
 // dK, dV
 // ---------------------------------------------------------------------------------------------------------
 
-// MODE 0: a dV and a dK workgroup per key tile (even / odd workgroups).  MODE 1 and 2 serve the three-launch order
+// MODE 0: a dV and a dK workgroup per key tile (8 apart in the grid, see below).  MODE 1 and 2 serve the three-launch order
 // dV / dQ / dK: all workgroups of a launch have one role, and the dK ones (MODE 2; rab and mask play no part in it)
 // take dS from the attn_bias gradient that the query-tile kernel wrote between the two launches.
 // MODE 4: launched after a query-tile kernel that stored dS and P: a workgroup that takes dV from P and one that
@@ -660,7 +660,7 @@ __global__ __launch_bounds__(kDkvThreads, (MODE == 2 || MODE >= 4) ? bwd_dk_from
     __shared__ __attribute__((aligned(1024))) uint16_t s_st2[kHalves * T::ELEMS];
     __shared__ __attribute__((aligned(1024))) uint16_t s_st3[kHalves * T::ELEMS];
     // a sub-tile is requested three steps ahead: the requests of two later steps may be outstanding at a step's start
-    // (plus, in MODE 2, the two loads of the next step's dS rows, issued between the two requests.  Reading rab / mask
+    // (plus, where dS / P rows are read, the two loads of the next step's rows, issued between the two requests.  Reading rab / mask
     // rows a step ahead in the same way was tried for the other modes: nothing for the dV-only launch, 277 -> 314 us
     // at C3 for the two-role one, which has no registers to spare at the head-dim slot 128.)
     constexpr int kAhead = (MODE == 2 || MODE >= 4) ? 2 : 0;  // (MODE 5's stores only make the wait stricter: the count must hold from the first step on)
