@@ -596,6 +596,12 @@ static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
     }
     const int64_t batch = f->n_offsets - 1;
     const int64_t dmax = f->head_dim_qk > f->head_dim_v ? f->head_dim_qk : f->head_dim_v;
+    // (one sequence's part of a plane sits behind a 32-bit descriptor)
+    const bool one_fits_32 = f->max_seq_len_q * f->max_seq_len_k * 2 < (1LL << 31);
+    const bool pair_fits_32 = f->max_seq_len_q * (64 * ((f->max_seq_len_k + 31) / 32)) * 2 < (1LL << 31);
+    if (!one_fits_32) {
+        return two;
+    }
     const int64_t n_ktiles = (f->max_seq_len_k + hstu::kBlockM - 1) / hstu::kBlockM;
     const bool many_tiles = n_ktiles * batch * f->num_heads_k >= 512;
     int64_t cap_mb = 4096;
@@ -604,7 +610,8 @@ static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
     }
     if (p->grad_attn_bias != nullptr) {
         const int64_t pair_bytes = batch * f->num_heads_q * f->max_seq_len_q * (64 * ((f->max_seq_len_k + 31) / 32)) * 2;
-        if ((forced == 2 || (forced < 0 && dmax > 128)) && var->dv_dk_from_planes_drab != nullptr && pair_bytes <= cap_mb * (1LL << 20)) {
+        if ((forced == 2 || (forced < 0 && dmax > 128)) && var->dv_dk_from_planes_drab != nullptr && pair_fits_32 &&
+            pair_bytes <= cap_mb * (1LL << 20)) {
             return BwdPlan{kPlanes, static_cast<uint64_t>(pair_bytes)};
         }
         const bool by_rule = many_tiles && (dmax > 128 || f->max_seq_len_k <= 1024 || f->total_q == batch * f->max_seq_len_q);
@@ -614,7 +621,7 @@ static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
     const bool three_fits = plane <= cap_mb * (1LL << 20);
     // (dS and P share rows of whole 32-key blocks, 64 elements each)
     const int64_t pair_plane = batch * f->num_heads_q * f->max_seq_len_q * (64 * ((f->max_seq_len_k + 31) / 32)) * 2;
-    const bool planes_fit = pair_plane <= cap_mb * (1LL << 20);
+    const bool planes_fit = pair_fits_32 && pair_plane <= cap_mb * (1LL << 20);
     const BwdPlan three = {kThreeLaunches, static_cast<uint64_t>(plane)};
     const BwdPlan planes = {kPlanes, static_cast<uint64_t>(pair_plane)};
     if (forced == 2) {

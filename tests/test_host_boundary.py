@@ -397,6 +397,53 @@ def test_backward_c_abi_validation_codes():
     assert lib.hstu_jagged_bwd(ctypes.byref(make(fwd=dict(mask_type=1))), None, 0, None) == 161002
 
 
+def test_backward_workspace_follows_the_launch_order(monkeypatch):
+    """hstu_jagged_bwd_workspace_size asks for the workspace of the launch order the library will take: a plane of
+    [batch, heads, max_q, max_k] elements for dS, one of 64 elements per 32-key block for dS and P together, or none
+    (the two-launch order; also whenever HSTU_MI355_BWD_HANDOFF=0)."""
+    lib = _native.load()
+    ws = ctypes.c_uint64(7)
+    fake = 0x1000
+
+    def size(grad_attn_bias=None, **fwd):
+        b = _native.new_bwd_params()
+        f = _valid_params()
+        for k, v in fwd.items():
+            setattr(f, k, v)
+        if grad_attn_bias is not None:
+            f.attn_bias = fake
+        _copy_fwd(b.fwd, f)
+        b.grad = b.grad_q = b.grad_k = b.grad_v = fake
+        b.grad_attn_bias = grad_attn_bias
+        assert lib.hstu_jagged_bwd_workspace_size(ctypes.byref(b), ctypes.byref(ws)) == 0, _native.last_error()
+        return ws.value
+
+    monkeypatch.delenv("HSTU_MI355_BWD_HANDOFF", raising=False)
+    monkeypatch.delenv("HSTU_MI355_BWD_WORKSPACE_MB", raising=False)
+    c2 = dict(n_offsets=33, num_heads_q=4, num_heads_k=4, total_q=20292, total_k=20292, max_seq_len_q=1024, max_seq_len_k=1024)
+    pair = 32 * 4 * 1024 * 64 * 32 * 2  # dS and P: 64 elements per 32-key block of every query row
+    one = 32 * 4 * 1024 * 1024 * 2
+    assert size(**c2) == pair  # a jagged batch whose planes stay in the memory-side cache: five products
+    assert size(**dict(c2, total_q=32 * 1024, total_k=32 * 1024)) == one  # the same without padding: three launches
+    assert size(**dict(c2, head_dim_qk=64, head_dim_v=64)) == 0  # head dims up to 64: two launches
+    assert size(**dict(c2, max_seq_len_q=1020, max_seq_len_k=1020)) == 0  # rows that are not multiples of 16 bytes
+    assert size(**dict(c2, head_dim_qk=256, head_dim_v=256, total_q=32 * 1024, total_k=32 * 1024)) == pair
+    assert size(**dict(c2, max_seq_len_q=4096, max_seq_len_k=4096)) == 0  # long rows at head dim 128
+    assert size(grad_attn_bias=fake, **c2) == 0  # dS goes through the gradient itself (or is recomputed)
+    assert size(grad_attn_bias=fake, **dict(c2, head_dim_qk=256, head_dim_v=256)) == pair
+    assert size(**dict(c2, dtype=_native.DT_FP32, out_dtype=_native.DT_FP32)) == 0  # the fp32 kernels have one order
+    monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "0")
+    assert size(**c2) == 0
+    monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "1")
+    assert size(**c2) == one and size(**dict(c2, head_dim_qk=64, head_dim_v=64)) == one
+    monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "2")
+    assert size(**c2) == pair
+    monkeypatch.setenv("HSTU_MI355_BWD_WORKSPACE_MB", "300")  # the limit of the workspace
+    assert size(**c2) == one
+    monkeypatch.setenv("HSTU_MI355_BWD_WORKSPACE_MB", "100")
+    assert size(**c2) == 0
+
+
 def test_paged_c_abi_validation_codes():
     lib = _native.load()
     ws = ctypes.c_uint64(7)
