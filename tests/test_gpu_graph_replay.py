@@ -1,5 +1,6 @@
-"""The operators under HIP graph capture: a captured chain (in_linear_silu -> hstu_jagged -> ln_mul, and a short-list
-forward that takes the split variant with its device-side counters) is replayed several times, with eager work and
+"""The operators under HIP graph capture: a captured chain (in_linear_silu -> hstu_jagged -> ln_mul, a short-list
+forward that takes the split variant with its device-side counters, and the backward in each of its launch orders) is
+replayed several times, with eager work and
 synchronisations of the program's own between the replays, and every replay is compared with the eager result bit for
 bit.  Nothing in these entry points allocates device memory behind torch's back or clears memory with a memset node:
 outputs and workspaces come from torch's allocator (its graph-private pool during capture), and the counter block at
@@ -84,3 +85,37 @@ def test_split_variant_replays():
     static = (ws[0].q.clone(), ws[0].k.clone(), ws[0].v.clone(), ws[0].seq_offset.clone())
     fresh = [(w.q, w.k, w.v, w.seq_offset) for w in ws[1:]] + [(ws[0].q, ws[0].k, ws[0].v, ws[0].seq_offset)]
     replay_and_compare(fwd, static, fresh)
+
+
+@pytest.mark.parametrize("order", ["0", "1", "2"], ids=["two_launches", "three_launches", "planes"])
+@pytest.mark.parametrize("rab", [False, True], ids=["norab", "rab"])
+def test_backward_replays_in_every_launch_order(order, rab, monkeypatch):
+    # the backward's launch orders under capture: fills are kernels, the workspace through which the query-tile kernel
+    # hands dS (and P) on comes from torch's graph-private pool and is never cleared; the gradients of every replay are
+    # compared with eager calls on the same values
+    monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", order)
+    max_len = 520
+
+    def make(seed):
+        return workloads.make("bwd", dtype=torch.bfloat16, device=DEV, seed=seed, batch=3, heads=2, dim=128, lo=100, hi=max_len,
+                              max_seq_len=max_len, std=0.5, silu_scale=1.0, rab_std=0.5 if rab else None)  # fmt: skip
+
+    ws = [make(s) for s in range(3)]
+    rows = max(w.q.shape[0] for w in ws)
+
+    def padded(t):  # (the same number of rows in every set: lengths differ between the seeds)
+        return torch.cat([t, torch.zeros(rows - t.shape[0], *t.shape[1:], dtype=t.dtype, device=DEV)])
+
+    def bwd(grad, q, k, v, bias, offsets):
+        got = ops_rec.ascendc.attention.hstu_jagged_backward(grad, q, k, v, None, bias, 0, max_len, max_len, 1.0, offsets,
+                                                             offsets, None, None, 0, 128**-0.5)  # fmt: skip
+        return torch.cat([g.float().flatten() for g in got if g is not None])
+
+    def inputs(w, seed):
+        g = torch.Generator(device=DEV).manual_seed(100 + seed)
+        grad = torch.randn(rows, 2, 128, generator=g, device=DEV).to(torch.bfloat16)
+        return (grad, padded(w.q), padded(w.k), padded(w.v), w.attn_bias, w.seq_offset)
+
+    sets = [inputs(w, i) for i, w in enumerate(ws)]
+    static = tuple(t.clone() if torch.is_tensor(t) else t for t in sets[0])
+    replay_and_compare(bwd, static, sets[1:] + [sets[0]])
