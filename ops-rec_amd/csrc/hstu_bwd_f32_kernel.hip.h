@@ -59,7 +59,10 @@ __device__ __forceinline__ void f32_load_row_keys(__amdgpu_buffer_rsrc_t rsrc, u
     }
 }
 
-template <int D, bool HAS_RAB, bool HAS_MASK>
+// PLANES: dS and P are stored as well, for a key-tile kernel that reads them back instead of computing them again: per
+// query row and 32-key block the 32 dS values followed by the 32 P values (a.p_plane; fp32; nothing in it is cleared:
+// the reading kernel reads what this one wrote).
+template <int D, bool HAS_RAB, bool HAS_MASK, bool PLANES = false>
 __global__ __launch_bounds__(256, 1) void hstu_bwd_f32_dq_kernel(const BwdArgs a)
 {
     constexpr int BN = 32;
@@ -164,6 +167,11 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_f32_dq_kernel(const BwdArgs a
     const bool want_drab = HAS_RAB && a.drab != nullptr;
     const __amdgpu_buffer_rsrc_t drab_rsrc =
         make_rsrc(want_drab ? static_cast<float*>(a.drab) + bias_plane : nullptr, want_drab ? bias_bytes : 0u);
+    const uint32_t pair_pitch = 64u * static_cast<uint32_t>((a.max_k + 31) / 32);  // elements per row of the dS / P plane
+    const __amdgpu_buffer_rsrc_t pair_rsrc = make_rsrc(
+        PLANES ? static_cast<float*>(a.p_plane) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(pair_pitch) : nullptr,
+        PLANES ? static_cast<uint32_t>(a.max_q) * pair_pitch * 4u : 0u);
+    const uint32_t pair_row_off = (wr0 + ln < sq) ? static_cast<uint32_t>(wr0 + ln) * pair_pitch * 4u : kOutOfRange;
     // rows past the sequence lie inside the plane but are not read or written: their offset leaves it
     const uint32_t bias_row_off =
         (wr0 + ln < sq) ? static_cast<uint32_t>(wr0 + ln) * static_cast<uint32_t>(a.max_k) * 4u : kOutOfRange;
@@ -226,8 +234,12 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_f32_dq_kernel(const BwdArgs a
             // dS^T, masked
             const bool full = !HAS_MASK && (c0 + 32 <= wb.lim_min) &&
                               !(wb.any_hole && c0 + 32 > si.hist_k && c0 < wb.hole_hi_max);
+            f32x16_t pv;  // P, when it is stored
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
+                if constexpr (PLANES) {
+                    pv[i] = score_p(s[i], sconst);
+                }
                 s[i] = score_ds(s[i], dp[i], sconst);
             }
             if (!full) {
@@ -236,10 +248,28 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_f32_dq_kernel(const BwdArgs a
                     const int jj = c0 + 8 * (i / 4) + 4 * lh + (i % 4);
                     const bool vis = (jj < lim) && !(jj >= hole_lo && jj < hole_hi);
                     float v = s[i];
+                    float pe = PLANES ? pv[i] : 0.f;
                     if constexpr (HAS_MASK) {
                         v *= mw[i];
+                        pe *= mw[i];
                     }
                     s[i] = vis ? v : 0.f;
+                    if constexpr (PLANES) {
+                        pv[i] = vis ? pe : 0.f;
+                    }
+                }
+            }
+            if constexpr (PLANES) {
+#pragma unroll
+                for (int g = 0; g < 4; ++g) {
+                    const int key = c0 + 8 * g + 4 * lh;
+                    const uint32_t off = pair_row_off + static_cast<uint32_t>(2 * c0 + 8 * g + 4 * lh) * 4u;
+                    const bwd_f32x4_t wd = {s[4 * g + 0], s[4 * g + 1], s[4 * g + 2], s[4 * g + 3]};
+                    const bwd_f32x4_t wp = {pv[4 * g + 0], pv[4 * g + 1], pv[4 * g + 2], pv[4 * g + 3]};
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, wd), pair_rsrc,
+                                                           static_cast<int>(key < sk ? off : kOutOfRange), 0, 0);
+                    __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4_t, wp), pair_rsrc,
+                                                           static_cast<int>(key < sk ? off + 128u : kOutOfRange), 0, 0);
                 }
             }
             if (want_drab) {
@@ -292,7 +322,9 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_f32_dq_kernel(const BwdArgs a
     }
 }
 
-template <int D, bool HAS_RAB, bool HAS_MASK>
+// PLANES: P and dS are read back from what the query-tile kernel stored (see there) instead of being computed: two
+// products per step instead of four, no score algebra, no rab / mask / K / V reads.
+template <int D, bool HAS_RAB, bool HAS_MASK, bool PLANES = false>
 __global__ __launch_bounds__(256, 1) void hstu_bwd_f32_dkv_kernel(const BwdArgs a)
 {
     constexpr int BN = 32;      // query rows per LDS tile
@@ -422,7 +454,27 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_f32_dkv_kernel(const BwdArgs 
                 }
                 active = active && cw0 < lim_max;
             }
-            if (active) {
+            float p[16], ds[16];
+            if constexpr (PLANES) {
+                if (active) {
+                    // only what the query-tile kernel wrote is read: the 32 x 32 blocks it swept (the blocks active
+                    // here), rows of the sequence, keys ahead of its last one
+                    const uint32_t pitch = 64u * static_cast<uint32_t>((a.max_k + 31) / 32);
+                    const __amdgpu_buffer_rsrc_t pair_rsrc = make_rsrc(
+                        static_cast<const float*>(a.p_plane) + (static_cast<int64_t>(b) * a.n_heads_q + hq) * a.max_q * static_cast<int64_t>(pitch),
+                        static_cast<uint32_t>(a.max_q) * pitch * 4u);
+#pragma unroll
+                    for (int i = 0; i < 16; ++i) {
+                        const int r = rq0 + 8 * (i / 4) + 4 * lh + (i % 4);
+                        const uint32_t off = (r < sq && key < sk)
+                                                 ? (static_cast<uint32_t>(r) * pitch + static_cast<uint32_t>(2 * cw0 + ln)) * 4u
+                                                 : kOutOfRange;
+                        ds[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(pair_rsrc, static_cast<int>(off), 0, 0));
+                        p[i] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(
+                                                             pair_rsrc, static_cast<int>(off == kOutOfRange ? kOutOfRange : off + 128u), 0, 0));
+                    }
+                }
+            } else if (active) {
                 f32x16_t s, dp;
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
@@ -441,7 +493,6 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_f32_dkv_kernel(const BwdArgs 
                         dp = __builtin_amdgcn_mfma_f32_32x32x2f32(gc[e], vf[j][e], dp, 0, 0, 0);
                     }
                 }
-                float p[16], ds[16];
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {
                     const int r = rq0 + 8 * (i / 4) + 4 * lh + (i % 4);
@@ -465,6 +516,8 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_f32_dkv_kernel(const BwdArgs 
                     p[i] = vis ? score_p(x_raw, sconst) * m : 0.f;
                     ds[i] = vis ? score_ds(x_raw, dp[i], sconst) * m : 0.f;
                 }
+            }
+            if (active) {
                 // dV^T += dO^T . P and dK^T += Q^T . dS: step i contracts the row pair {8 (i / 4) + i % 4, the same + 4}
 #pragma unroll
                 for (int i = 0; i < 16; ++i) {

@@ -55,7 +55,8 @@ const BwdVariant (*bwd_variants_generic())[3] { return kGenericBwd; }
 namespace {
 #define HSTU_F32_BWD_VARIANT(D, RAB, MASK)                                                                    \
     {"hstu_bwd_f32_d" #D "_rab" #RAB "_mask" #MASK, hstu_bwd_f32_dkv_kernel<D, RAB, MASK>, hstu_bwd_f32_dq_kernel<D, RAB, MASK>, \
-     hstu_bwd_f32_dq_kernel<D, RAB, MASK>}
+     hstu_bwd_f32_dq_kernel<D, RAB, MASK>, nullptr, nullptr, hstu_bwd_f32_dq_kernel<D, RAB, MASK, true>,                  \
+     hstu_bwd_f32_dkv_kernel<D, false, false, true>, hstu_bwd_f32_dkv_kernel<D, false, false, true>}
 #define HSTU_F32_BWD_DIMS(RAB, MASK) \
     {HSTU_F32_BWD_VARIANT(32, RAB, MASK), HSTU_F32_BWD_VARIANT(64, RAB, MASK), HSTU_F32_BWD_VARIANT(128, RAB, MASK)}
 const BwdVariant kF32Bwd[2][2][3] = {{HSTU_F32_BWD_DIMS(0, 0), HSTU_F32_BWD_DIMS(0, 1)},

@@ -591,7 +591,29 @@ static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
     const BwdPlan two = {kTwoLaunches, 0};
     const char* const env = getenv("HSTU_MI355_BWD_HANDOFF");
     const int forced = env == nullptr ? -1 : (env[0] == '0' ? 0 : (env[0] == '2' ? 2 : 1));
-    if (var->dk_from_ds == nullptr || forced == 0 || f->total_q == 0 || f->total_k == 0 || f->max_seq_len_k % 8 != 0) {
+    if (forced == 0 || f->total_q == 0 || f->total_k == 0) {
+        return two;
+    }
+    if (f->dtype == HSTU_DT_FP32) {
+        // the fp32 kernels know two orders: everything computed where it is used (7 products), or dS and P stored by the
+        // query-tile kernel in fp32 and read back by the key-tile kernel (5 products, 16 bytes of traffic per pair).
+        // The second is ahead wherever it was measured (recomputing -> planes): B16 H4 L100..1024 d32 245 -> 200 us,
+        // d64 382 -> 264 us, d128 595 -> 439 us; B32 H8 L1024 d64 1557 -> 1344 us, d128 2899 -> 2233 us; B4 H4 d128
+        // L300..700 405 -> 286 us; B2 H4 d128 L8192 4841 -> 4519 us -- the fp32 matrix instruction is slow enough for
+        // a product to cost more than its operands' trip through memory.  Taken whenever the workspace is within the limit.
+        if (var->dq_ds_p == nullptr) {
+            return two;
+        }
+        int64_t cap = 4096;
+        if (const char* const cap_env = getenv("HSTU_MI355_BWD_WORKSPACE_MB")) {
+            cap = atoll(cap_env);
+        }
+        const int64_t row = 64 * ((f->max_seq_len_k + 31) / 32);
+        const int64_t bytes = (f->n_offsets - 1) * f->num_heads_q * f->max_seq_len_q * row * 4;
+        const bool fits = f->max_seq_len_q * row * 4 < (1LL << 31) && bytes <= cap * (1LL << 20);
+        return fits ? BwdPlan{kPlanes, static_cast<uint64_t>(bytes)} : two;
+    }
+    if (var->dk_from_ds == nullptr || f->max_seq_len_k % 8 != 0) {
         return two;
     }
     const int64_t batch = f->n_offsets - 1;
@@ -759,8 +781,17 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
             launch_clear(p->grad_attn_bias, drab_bytes, stream);
         }
         if (f->total_k > 0 && f->total_q > 0 && grid_kv > 0 && grid_q > 0) {
-            hipLaunchKernelGGL(var->dkv, dim3(static_cast<unsigned>(grid_kv)), dim3(256), 0, static_cast<hipStream_t>(stream), a);
-            hipLaunchKernelGGL(var->dq, dim3(static_cast<unsigned>(grid_q)), dim3(256), 0, static_cast<hipStream_t>(stream), a);
+            if (plan.order == kPlanes && usable_workspace(workspace, workspace_bytes, plan.workspace_bytes) &&
+                reinterpret_cast<uintptr_t>(workspace) % 16 == 0) {
+                // (fp32) the query-tile kernel leaves dS and P in the workspace, the key-tile kernel reads them back
+                a.p_plane = workspace;
+                hipLaunchKernelGGL(var->dq_ds_p, dim3(static_cast<unsigned>(grid_q)), dim3(256), 0, static_cast<hipStream_t>(stream), a);
+                hipLaunchKernelGGL(var->dv_dk_from_planes, dim3(static_cast<unsigned>(grid_kv)), dim3(256), 0,
+                                   static_cast<hipStream_t>(stream), a);
+            } else {
+                hipLaunchKernelGGL(var->dkv, dim3(static_cast<unsigned>(grid_kv)), dim3(256), 0, static_cast<hipStream_t>(stream), a);
+                hipLaunchKernelGGL(var->dq, dim3(static_cast<unsigned>(grid_q)), dim3(256), 0, static_cast<hipStream_t>(stream), a);
+            }
         }
     } else if (f->total_k > 0 && grid_kv > 0 && f->total_q > 0 && grid_q > 0 && a.bias_vec_ok == 2 && plan.order != kTwoLaunches &&
                (plan.workspace_bytes == 0 || (usable_workspace(workspace, workspace_bytes, plan.workspace_bytes) &&

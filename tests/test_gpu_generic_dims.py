@@ -144,7 +144,13 @@ def test_backward_of_fp32_inputs_with_all_the_semantics(kw, generic, monkeypatch
     monkeypatch.setenv("HSTU_MI355_GENERIC_BACKWARD", generic)
     base = dict(seed=len(kw) + 23, batch=4, heads=2, dim=32, dim_v=48, lo=20, hi=160, dtype=torch.float32, std=0.5)
     base.update(kw)
-    check_backward(small_case(**base))
+    # the matrix-instruction kernels in both of their orders: everything computed where it is used, and dS and P handed
+    # from the query-tile kernel to the key-tile kernel through a workspace (filled with NaN here: nothing in it is
+    # cleared, the key-tile kernel reads what was written)
+    for order in (("0", "2") if generic == "0" else ("0",)):
+        monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", order)
+        monkeypatch.setenv("HSTU_MI355_POISON_WORKSPACE", "1")
+        check_backward(small_case(**base))
 
 
 @pytest.mark.parametrize("kw", [
@@ -152,7 +158,10 @@ def test_backward_of_fp32_inputs_with_all_the_semantics(kw, generic, monkeypatch
     dict(dim=128, dim_v=128, lo=0, hi=400, ctx=9, max_target=50, group=4), dict(dim=16, dim_v=16, lo=0, hi=260, delta=True, rab=True),
     dict(dim=8, dim_v=128, lo=127, hi=129, heads=6, heads_k=2, rab=True), dict(dim=104, dim_v=80, lo=255, hi=257, custom_mask=True),
 ], ids=lambda kw: "-".join(f"{k}{v}" for k, v in kw.items()))  # fmt: skip
-def test_backward_of_fp32_inputs_over_several_query_and_key_tiles(kw):
+@pytest.mark.parametrize("order", ["0", "2"], ids=["recompute", "planes"])
+def test_backward_of_fp32_inputs_over_several_query_and_key_tiles(kw, order, monkeypatch):
+    monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", order)
+    monkeypatch.setenv("HSTU_MI355_POISON_WORKSPACE", "1")
     base = dict(seed=len(kw) + 41, batch=3, heads=2, dtype=torch.float32, std=0.5)
     base.update(kw)
     check_backward(small_case(**base))

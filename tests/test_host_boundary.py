@@ -431,7 +431,9 @@ def test_backward_workspace_follows_the_launch_order(monkeypatch):
     assert size(**dict(c2, max_seq_len_q=4096, max_seq_len_k=4096)) == 0  # long rows at head dim 128
     assert size(grad_attn_bias=fake, **c2) == 0  # dS goes through the gradient itself (or is recomputed)
     assert size(grad_attn_bias=fake, **dict(c2, head_dim_qk=256, head_dim_v=256)) == pair
-    assert size(**dict(c2, dtype=_native.DT_FP32, out_dtype=_native.DT_FP32)) == 0  # the fp32 kernels have one order
+    # fp32: the matrix-instruction kernels (head dims up to 128) hand dS and P over in fp32; the generic ones do not
+    assert size(**dict(c2, dtype=_native.DT_FP32, out_dtype=_native.DT_FP32)) == 2 * pair
+    assert size(**dict(c2, dtype=_native.DT_FP32, out_dtype=_native.DT_FP32, head_dim_qk=256, head_dim_v=256)) == 0
     monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "0")
     assert size(**c2) == 0
     monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "1")
