@@ -182,7 +182,7 @@ HSTU_API uint64_t hstu_jagged_fwd_noalloc_max_workspace(void);
  * elements of the input type -- twice that (rounded up to whole 32-key blocks) for dS and P together --, which
  * hstu_jagged_bwd_workspace_size asks for where it was measured to pay (head dims above 64, max_seq_len_k a
  * multiple of 8, at most 4 GiB or HSTU_MI355_BWD_WORKSPACE_MB in the environment; at head dims above 128 also with
- * grad_attn_bias, for dS and P together).  Without the
+ * grad_attn_bias, for dS and P together; fp32 inputs with head dims up to 128: always, in fp32).  Without the
  * workspace, or with less than was asked for, the call still works: the kernels that produce grad_k then recompute
  * dS.  The workspace needs no clearing and holds nothing afterwards. */
 typedef struct hstu_jagged_bwd_params {
