@@ -564,17 +564,22 @@ HSTU_API int hstu_paged_fwd(const hstu_paged_fwd_params* p, void* workspace, uin
 //   L512..1024 203 -> 213 -> 139 us, B32 H4 d192 L256..1024 502 -> 402 -> 296 us); long rows included (no d rab: B4 H4
 //   d256 L1024..4096 885 -> 613 -> 465 us, B8 H4 d256 L4096 1845 -> 1257 -> 1135 us) up to max_seq_len_k 4096, three
 //   launches beyond (B2 H4 d256 L8192 1794 -> 1343 -> 1444 us);
-//   head dims 65 .. 128 without an attn_bias gradient, max_seq_len_k up to 2048:  planes when the plane holds at most
+//   head dims up to 128 without an attn_bias gradient, max_seq_len_k up to 2048:  planes when the plane holds at most
 //   about 120 MB (estimated from total_q, the batch and max_seq_len: C2 103 MB, B128 H4 L64..512 85 MB; B32 H8 L512
-//   unpadded 134 MB: 132 us with three launches, 141 us with planes); else three launches from 512 workgroups per
-//   launch on (key tiles x sequences x K/V heads: B8 H4 d128 L512..1024 and smaller lose with three); else two;
-//   head dims up to 128 with an attn_bias gradient: three launches from 512 workgroups per launch on when
+//   unpadded 134 MB: 132 us with three launches, 141 us with planes) -- at head dims up to 64 as well (B32 H4 d64
+//   L278..1004 102 -> 103 -> 92 us, B64 H4 d64 L64..512 65 -> 65 -> 52 us, B16 H4 d32 L128..512 40 -> 48 -> 33 us); else,
+//   above head dim 64, three launches from 512 workgroups per launch on (key tiles x sequences x K/V heads: B8 H4
+//   d128 L512..1024 and smaller lose with three); else two;
+//   head dims up to 128 with an attn_bias gradient: planes while that gradient is at most 160 MB, so that its clearing
+//   and the plane stay in the memory-side cache (B8 H4 d128 L512..1024 128 -> 136 -> 101 us, B16 H4 d96 L256..1024
+//   147 -> 152 -> 129 us, B16 H4 d64 L128..512 59 -> 70 -> 49 us; at 268 MB B32 H4 d64 L256..1024 176 -> 169 -> 203 us);
+//   else three launches from 512 workgroups per launch on when
 //   max_seq_len_k is at most 1024 (B64 H4 d128 L256..1024 431 -> 382 us, B128 H4 d64 L64..512 177 -> 146 us) or the
 //   batch has no padding, total_q = batch x max_seq_len_q (B32 H8 d128 L2048 2599 -> 2311 us, B32 H8 d32 L4096
 //   8013 -> 6810 us); not for long jagged batches, where the clearing of the gradient no longer hides behind the dV
 //   workgroups alone (B32 H4 d64 L100..1504 310 -> 341 us, B8 H8 d128 L1024..4096 1492 -> 1657 us; C3 396 -> 401 us,
 //   planes 408 us);
-//   everything else (head dims up to 64 without an attn_bias gradient, long rows at head dims up to 128): two launches.
+//   everything else (larger planes at head dims up to 64, long rows at head dims up to 128): two launches.
 // Also tried, not kept: the dV workgroups on a second stream beside the query-tile kernel (C2 143 -> 149 us), and the
 // query-tile kernel first with dV and dK-from-dS workgroups in one launch behind it (C2 160 us).
 // HSTU_MI355_BWD_HANDOFF in the environment overrides the rule: 0 = two launches, 1 = three wherever possible,
@@ -632,7 +637,9 @@ static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
     }
     if (p->grad_attn_bias != nullptr) {
         const int64_t pair_bytes = batch * f->num_heads_q * f->max_seq_len_q * (64 * ((f->max_seq_len_k + 31) / 32)) * 2;
-        if ((forced == 2 || (forced < 0 && dmax > 128)) && var->dv_dk_from_planes_drab != nullptr && pair_fits_32 &&
+        // (head dims up to 128: while the gradient is small enough for its clearing and the plane to stay in the cache)
+        const bool small_gradient = batch * f->num_heads_q * f->max_seq_len_q * f->max_seq_len_k * 2 <= 160LL * 1000 * 1000;
+        if ((forced == 2 || (forced < 0 && (dmax > 128 || small_gradient))) && var->dv_dk_from_planes_drab != nullptr && pair_fits_32 &&
             pair_bytes <= cap_mb * (1LL << 20)) {
             return BwdPlan{kPlanes, static_cast<uint64_t>(pair_bytes)};
         }
@@ -655,7 +662,7 @@ static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
     if (dmax > 128) {
         return (planes_fit && f->max_seq_len_k <= 4096) ? planes : (three_fits ? three : two);
     }
-    if (dmax <= 64 || f->max_seq_len_k > 2048) {
+    if (f->max_seq_len_k > 2048) {
         return two;
     }
     // what the plane holds under a causal mask, sum of L^2 / 2 pairs x 4 bytes per head, estimated from what the host
@@ -666,7 +673,7 @@ static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
     if (planes_fit && held <= 120e6) {
         return planes;
     }
-    return (three_fits && many_tiles) ? three : two;
+    return (dmax > 64 && three_fits && many_tiles) ? three : two;
 }
 
 HSTU_API int hstu_jagged_bwd_workspace_size(const hstu_jagged_bwd_params* params, uint64_t* workspace_bytes)

@@ -425,11 +425,13 @@ def test_backward_workspace_follows_the_launch_order(monkeypatch):
     one = 32 * 4 * 1024 * 1024 * 2
     assert size(**c2) == pair  # a jagged batch whose planes stay in the memory-side cache: five products
     assert size(**dict(c2, total_q=32 * 1024, total_k=32 * 1024)) == one  # the same without padding: three launches
-    assert size(**dict(c2, head_dim_qk=64, head_dim_v=64)) == 0  # head dims up to 64: two launches
+    assert size(**dict(c2, head_dim_qk=64, head_dim_v=64)) == pair  # small planes pay at every head dim
+    assert size(**dict(c2, head_dim_qk=64, head_dim_v=64, total_q=32 * 1024, total_k=32 * 1024)) == 0  # larger ones: two launches
     assert size(**dict(c2, max_seq_len_q=1020, max_seq_len_k=1020)) == 0  # rows that are not multiples of 16 bytes
     assert size(**dict(c2, head_dim_qk=256, head_dim_v=256, total_q=32 * 1024, total_k=32 * 1024)) == pair
     assert size(**dict(c2, max_seq_len_q=4096, max_seq_len_k=4096)) == 0  # long rows at head dim 128
     assert size(grad_attn_bias=fake, **c2) == 0  # dS goes through the gradient itself (or is recomputed)
+    assert size(grad_attn_bias=fake, **dict(c2, n_offsets=9, total_q=5000, total_k=5000)) == pair // 4  # a small gradient
     assert size(grad_attn_bias=fake, **dict(c2, head_dim_qk=256, head_dim_v=256)) == pair
     # fp32: the matrix-instruction kernels (head dims up to 128) hand dS and P over in fp32; the generic ones do not
     assert size(**dict(c2, dtype=_native.DT_FP32, out_dtype=_native.DT_FP32)) == 2 * pair
