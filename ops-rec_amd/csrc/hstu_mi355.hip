@@ -570,9 +570,11 @@ HSTU_API int hstu_paged_fwd(const hstu_paged_fwd_params* p, void* workspace, uin
 //   L278..1004 102 -> 103 -> 92 us, B64 H4 d64 L64..512 65 -> 65 -> 52 us, B16 H4 d32 L128..512 40 -> 48 -> 33 us); else,
 //   above head dim 64, three launches from 512 workgroups per launch on (key tiles x sequences x K/V heads: B8 H4
 //   d128 L512..1024 and smaller lose with three); else two;
-//   head dims up to 128 with an attn_bias gradient: planes while that gradient is at most 160 MB, so that its clearing
-//   and the plane stay in the memory-side cache (B8 H4 d128 L512..1024 128 -> 136 -> 101 us, B16 H4 d96 L256..1024
-//   147 -> 152 -> 129 us, B16 H4 d64 L128..512 59 -> 70 -> 49 us; at 268 MB B32 H4 d64 L256..1024 176 -> 169 -> 203 us);
+//   head dims up to 128 with an attn_bias gradient: planes while that gradient, weighted with the batch's fill
+//   (total_q / (batch x max_seq_len_q)), is at most 100 MB, so that its clearing and the plane stay in the memory-side
+//   cache (B8 H4 d128 L512..1024, 50 MB: 128 -> 136 -> 101 us; B16 H4 d96 L256..1024, 84 MB: 147 -> 152 -> 129 us; B16 H4
+//   d64 L128..512: 59 -> 70 -> 49 us; not B32 H8 d64 L512 unpadded, 134 MB: 157 with three launches, 174 with planes;
+//   nor B32 H4 d64 L256..1024, 168 MB: 176 -> 169 -> 203 us);
 //   else three launches from 512 workgroups per launch on when
 //   max_seq_len_k is at most 1024 (B64 H4 d128 L256..1024 431 -> 382 us, B128 H4 d64 L64..512 177 -> 146 us) or the
 //   batch has no padding, total_q = batch x max_seq_len_q (B32 H8 d128 L2048 2599 -> 2311 us, B32 H8 d32 L4096
@@ -638,7 +640,8 @@ static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
     if (p->grad_attn_bias != nullptr) {
         const int64_t pair_bytes = batch * f->num_heads_q * f->max_seq_len_q * (64 * ((f->max_seq_len_k + 31) / 32)) * 2;
         // (head dims up to 128: while the gradient is small enough for its clearing and the plane to stay in the cache)
-        const bool small_gradient = batch * f->num_heads_q * f->max_seq_len_q * f->max_seq_len_k * 2 <= 160LL * 1000 * 1000;
+        const double grad_bytes = static_cast<double>(batch * f->num_heads_q * f->max_seq_len_q * f->max_seq_len_k * 2);
+        const bool small_gradient = grad_bytes * static_cast<double>(f->total_q) / static_cast<double>(batch * f->max_seq_len_q) <= 100e6;
         if ((forced == 2 || (forced < 0 && (dmax > 128 || small_gradient))) && var->dv_dk_from_planes_drab != nullptr && pair_fits_32 &&
             pair_bytes <= cap_mb * (1LL << 20)) {
             return BwdPlan{kPlanes, static_cast<uint64_t>(pair_bytes)};
