@@ -181,7 +181,7 @@ HSTU_API uint64_t hstu_jagged_fwd_noalloc_max_workspace(void);
  * is dS) when that is asked for, otherwise in a workspace of [batch, num_heads_q, max_seq_len_q, max_seq_len_k]
  * elements of the input type -- twice that (rounded up to whole 32-key blocks) for dS and P together --, which
  * hstu_jagged_bwd_workspace_size asks for where it was measured to pay (head dims above 64, max_seq_len_k a
- * multiple of 8, at most 4 GiB or HSTU_MI355_BWD_WORKSPACE_MB in the environment; at head dims above 128 also with
+ * multiple of 8, at most 2 GiB or HSTU_MI355_BWD_WORKSPACE_MB in the environment; at head dims above 128 also with
  * grad_attn_bias, for dS and P together; fp32 inputs with head dims up to 128: always, in fp32).  Without the
  * workspace, or with less than was asked for, the call still works: the kernels that produce grad_k then recompute
  * dS.  The workspace needs no clearing and holds nothing afterwards. */
@@ -243,6 +243,12 @@ HSTU_API int hstu_paged_fwd(const hstu_paged_fwd_params* params, void* workspace
 /* replaces aclGetRecentErrMsg (ascendc/common/torch_plugin/pytorch_npu_helper.hpp:649,662):
  * text of the calling thread's most recent failure; never NULL. */
 HSTU_API const char* hstu_last_error(void);
+
+/* The library's process-wide switches (HSTU_MI355_SPLIT, HSTU_MI355_SHORT, HSTU_MI355_GENERIC_BACKWARD,
+ * HSTU_MI355_BWD_HANDOFF, HSTU_MI355_BWD_WORKSPACE_MB) are read from the environment once, at the first call that
+ * looks at one; this reads them again.  No counterpart in the reference: it is for a test or a tool that changes the
+ * environment after the library has been used.  Not safe against launches running at the same time in other threads. */
+HSTU_API void hstu_reload_switches(void);
 
 /* library version, (major << 16) | minor */
 HSTU_API int hstu_version(void);

@@ -22,6 +22,7 @@ constexpr int fwd_wgs_per_cu(int d, bool rab, bool mask)
 {
     return (!rab && !mask && d <= 64) ? (d <= 32 ? 4 : 3) : (d <= 32 && !(rab && mask)) ? 3 : (d <= 128 ? 2 : 1);
 }
+constexpr int kShortThreads = 512;  // threads of a workgroup of the forward kernel for short lists (eight wavefronts of 16 query rows)
 constexpr int kCounterBlockBytes = 16384;  // head of the workspace: device-side work counters (see the forward kernel)
 constexpr int kDkvThreads = 256;   // threads of a workgroup of the key-tile backward kernel
 constexpr int kGatherThreads = 128;
@@ -74,6 +75,7 @@ struct FwdArgs {
     int64_t num_pages;
     int64_t n_page_ids;
     int page_shift;  // log2(page_size); page_size is 32, 64, 128 or 256
+    int short_spread;  // kernel for short lists: the tiles of a (sequence, K/V head) alternate between two XCDs
 };
 
 struct BwdArgs {

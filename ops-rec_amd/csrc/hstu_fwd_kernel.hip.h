@@ -88,7 +88,7 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void* base, ui
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, static_cast<int>(bytes), kBufferFlags);
 }
 
-// Visibility bounds shared by the 32 query rows [wr0, min(wr0 + 32, sq)) of one wavefront under the
+// Visibility bounds shared by the `rows` (32, or 16 in the kernel for short lists) query rows [wr0, min(wr0 + rows, sq)) of one wavefront under the
 // built-in mask, in closed form (no cross-lane traffic).  A key j is visible to row i iff
 //   j < lim(i)  &&  !(hist_k <= j < hole_hi(i))
 // with lim(i) = clamp(i < n_ctx ? max(i + delta + 1, hist_k) : i + delta + 1, 0, sk), delta = sk - sq,
@@ -104,7 +104,7 @@ struct WaveBounds {
 };
 
 __device__ __forceinline__ WaveBounds wave_bounds(int mask_type, int wr0, int sq, int sk, int n_ctx, int n_tgt,
-                                                  int group, bool active)
+                                                  int group, bool active, int rows = kWaveM)
 {
     WaveBounds w;
     w.hole_hi_max = 0;
@@ -119,7 +119,7 @@ __device__ __forceinline__ WaveBounds wave_bounds(int mask_type, int wr0, int sq
         w.lim_max = sk;
         return w;
     }
-    const int wr1 = (wr0 + kWaveM < sq) ? wr0 + kWaveM : sq;
+    const int wr1 = (wr0 + rows < sq) ? wr0 + rows : sq;
     const int delta = sk - sq;
     const int hist_k = sk - n_tgt;
     int hi = wr1 + delta;  // lim of the last row

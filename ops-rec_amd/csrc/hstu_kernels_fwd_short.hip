@@ -1,0 +1,13 @@
+// forward kernels for short work lists (16-bit inputs, head-dim slot 128, no bias, no custom mask)
+#include "hstu_fwd_short_kernel.hip.h"
+#include "hstu_variants.h"
+
+namespace hstu {
+namespace {
+const ShortVariant kTable[2] = {
+    {"hstu_fwd_bf16_d128_short", hstu_fwd_short_kernel<bf16_tag, 128>},
+    {"hstu_fwd_f16_d128_short", hstu_fwd_short_kernel<f16_tag, 128>},
+};
+}
+const ShortVariant* fwd_variants_short() { return kTable; }
+}  // namespace hstu

@@ -72,6 +72,56 @@ int compute_units(int* out)
 }
 
 
+// Process-wide switches.  They are read from the environment once, at the first call that looks at one, and again
+// only when hstu_reload_switches() is called (a test that changes the environment calls it); a launch reads no
+// environment variable.  A value of -1 means "not set: the library's own rule applies".
+//   HSTU_MI355_SPLIT=0             forward: never cut long items into parts (the rows of a sequence are then the same bits
+//                                  whatever else is in the batch)
+//   HSTU_MI355_SHORT=0 / 1         forward: never / whenever possible the kernel for short lists
+//   HSTU_MI355_GENERIC_BACKWARD=1  backward: the generic kernels also where tuned ones exist (for comparisons)
+//   HSTU_MI355_BWD_HANDOFF=0/1/2   backward: force the launch order (two launches / three / planes)
+//   HSTU_MI355_BWD_WORKSPACE_MB=n  backward: the largest workspace the library asks for
+struct Switches {
+    int split;
+    int short_lists;
+    int generic_backward;
+    int bwd_handoff;
+    long long bwd_workspace_mb;
+};
+Switches g_switches = {-1, -1, -1, -1, -1};
+std::once_flag g_switches_once;
+
+int switch_digit(const char* name, int max_digit)
+{
+    const char* const v = getenv(name);
+    if (v == nullptr || v[0] < '0' || v[0] > '0' + max_digit || v[1] != '\0') {
+        return -1;  // unset, empty or not one of the values the switch knows: the library's own rule
+    }
+    return v[0] - '0';
+}
+void read_switches()
+{
+    g_switches.split = switch_digit("HSTU_MI355_SPLIT", 1);
+    g_switches.short_lists = switch_digit("HSTU_MI355_SHORT", 1);
+    g_switches.generic_backward = switch_digit("HSTU_MI355_GENERIC_BACKWARD", 1);
+    g_switches.bwd_handoff = switch_digit("HSTU_MI355_BWD_HANDOFF", 2);
+    const char* const mb = getenv("HSTU_MI355_BWD_WORKSPACE_MB");
+    g_switches.bwd_workspace_mb = (mb != nullptr && mb[0] >= '0' && mb[0] <= '9') ? atoll(mb) : -1;
+}
+const Switches& switches()
+{
+    std::call_once(g_switches_once, read_switches);
+    return g_switches;
+}
+// the largest backward workspace the library asks for, in MiB: 2 GiB unless HSTU_MI355_BWD_WORKSPACE_MB says otherwise
+// (a call whose planes would need more runs on the two-launch order, which needs none)
+int64_t workspace_cap_mb()
+{
+    const long long set = switches().bwd_workspace_mb;
+    return set >= 0 ? static_cast<int64_t>(set) : 2048;
+}
+
+
 int validate(const hstu_jagged_fwd_params* p, bool need_out = true)
 {
     if (p == nullptr) {
@@ -202,6 +252,45 @@ const Variant* select(const hstu_jagged_fwd_params* p)
     return &table[p->attn_bias != nullptr ? 1 : 0][p->mask_type == HSTU_MASK_CUSTOM ? 1 : 0][slot];
 }
 
+// The kernel for short work lists (hstu_fwd_short_kernel.hip.h) takes 16-bit inputs at the head-dim slot 128 without
+// bias or custom mask.  It is the faster one while the list -- at most n_blocks entries -- is a few items per
+// workgroup the persistent kernel would keep resident: there a launch lasts as long as its longest item, which the
+// short kernel's narrower wavefronts finish in about half the time; on longer lists the persistent kernel's
+// steady-state rate wins.  HSTU_MI355_SHORT in the environment overrides the rule: 0 = never, 1 = whenever the
+// kernel can take the call.
+const hstu::ShortVariant* short_variant(const Variant* var, const hstu_jagged_fwd_params* p)
+{
+    if ((p->dtype != HSTU_DT_BF16 && p->dtype != HSTU_DT_FP16) || p->attn_bias != nullptr ||
+        p->mask_type == HSTU_MASK_CUSTOM || var->d_pad != 128 || var->persistent_wgs_per_cu <= 0 ||
+        var->kernel_queues == nullptr) {
+        return nullptr;
+    }
+    const hstu::ShortVariant* const sv = &hstu::fwd_variants_short()[p->dtype == HSTU_DT_BF16 ? 0 : 1];
+    const int forced = switches().short_lists;
+    if (forced == 0) {
+        return nullptr;
+    }
+    if (forced == 1) {
+        return sv;
+    }
+    int cus = 0;
+    if (compute_units(&cus) != HSTU_OK) {
+        return nullptr;
+    }
+    // Measured on MI355X (bf16, head dim 128, persistent kernel -> this one): keys up to 1024 -- batch 32 x 4 heads
+    // lengths 256..1024 37.4 -> 33.6 us, 8 x 4 of 1024 32.9 -> 25.2, 64 x 4 of 512 43.1 -> 39.3, 256 x 4 of 256
+    // 68.2 -> 53.2, 2048 x 2 of 32 71.0 -> 40.0, 128 x 4 of 1024 220.9 -> 217.3 (even); keys up to 2048 with one to
+    // two slots per resident workgroup -- 8 x 8 of 1536 62.5 -> 52.5, 8 x 4 of 2048 57.4 -> 51.5, 16 x 4 of 2048 even;
+    // beyond that the persistent kernel's variants win: 32 x 4 lengths 512..2048 103.7 -> 107.9, 4 x 2 of 2048 36.7
+    // (split items) -> 41.4, 16 x 4 of 4096 291 -> 296, 1 x 4 of 8192 127 (split) -> 177.
+    const int64_t resident = static_cast<int64_t>(cus) * var->persistent_wgs_per_cu;
+    const int64_t n_qtiles = (p->max_seq_len_q + hstu::kBlockM - 1) / hstu::kBlockM;
+    const int64_t n_blocks = n_qtiles * (p->n_offsets - 1) * p->num_heads_q;
+    const bool short_keys = p->max_seq_len_k <= 1024;
+    const bool one_round = p->max_seq_len_k <= 2048 && n_blocks >= resident && n_blocks <= 2 * resident;
+    return (short_keys || one_round) ? sv : nullptr;
+}
+
 // persistent workgroups per CU of a launch: what the variant is compiled for, except that the slot-32 variants with a
 // bias or a custom mask, compiled for three, are launched two per CU when rows are longer than 2048 keys -- there the
 // bias stream is the bound and a third reader per CU costs 3 % (B32 H8 L4096 1351 -> 1391 us), where it is worth
@@ -248,10 +337,9 @@ bool may_take_split_variant(const Variant* var, const hstu_jagged_fwd_params* p,
     if (var->persistent_wgs_per_cu <= 0 || var->kernel_split == nullptr) {
         return false;
     }
-    // HSTU_MI355_SPLIT=0 in the environment (read at every call) turns splitting off: the rows of a sequence then
-    // come out bit for bit the same whatever else is in the batch (a split changes the order of the fp32 sums)
-    const char* const env = getenv("HSTU_MI355_SPLIT");
-    if (env != nullptr && env[0] == '0') {
+    // HSTU_MI355_SPLIT=0 turns splitting off: the rows of a sequence then come out bit for bit the same whatever
+    // else is in the batch (a split changes the order of the fp32 sums)
+    if (switches().split == 0) {
         return false;
     }
     int cus = 0;
@@ -283,6 +371,9 @@ uint64_t split_workspace_bytes(const Variant* var, const hstu_jagged_fwd_params*
 // split items, nothing for the lists in between (fixed schedule, no device counters)
 uint64_t forward_workspace_bytes(const Variant* var, const hstu_jagged_fwd_params* p)
 {
+    if (short_variant(var, p) != nullptr) {
+        return 0;
+    }
     if (takes_queue_variant(var, p, nullptr)) {
         return kCounterBytes;
     }
@@ -355,8 +446,7 @@ const BwdVariant* select_bwd(const hstu_jagged_bwd_params* p)
     const int64_t dmax = f->head_dim_qk > f->head_dim_v ? f->head_dim_qk : f->head_dim_v;
     const BwdVariant* generic = &hstu::bwd_variants_generic()[f->dtype == HSTU_DT_BF16 ? 0 : (f->dtype == HSTU_DT_FP16 ? 1 : 2)]
                                                              [dmax <= 128 ? 0 : (dmax <= 256 ? 1 : 2)];
-    const char* const env = getenv("HSTU_MI355_GENERIC_BACKWARD");
-    const bool force_generic = env != nullptr && env[0] == '1';
+    const bool force_generic = switches().generic_backward == 1;
     if (f->dtype == HSTU_DT_FP32 && dmax <= 128 && f->head_dim_qk % 8 == 0 && !force_generic) {
         // fp32 MFMA kernels: one sequence of one head group behind a 32-bit descriptor
         const int64_t sq4 = f->max_seq_len_q * f->num_heads_q * dmax * 4;
@@ -558,7 +648,7 @@ HSTU_API int hstu_paged_fwd(const hstu_paged_fwd_params* p, void* workspace, uin
 // 4 x head dim flops per pair each: it pays from the head-dim slot 128 on, and at 128 the second plane only while both
 // stay in the memory-side cache (256 MB) between the launches; few long sequences lose either way (each launch is
 // as long as its heaviest workgroup).  The rule:
-//   head dims above 128 (workspace within the limit: 4 GiB, or HSTU_MI355_BWD_WORKSPACE_MB in the environment): planes,
+//   head dims above 128 (workspace within the limit: 2 GiB, or HSTU_MI355_BWD_WORKSPACE_MB in the environment): planes,
 //   with or without an attn_bias gradient -- with one the query-tile kernel clears it beside its work and the dK
 //   workgroups write the dS pieces they read into it (B32 H8 d256 L1024 with d rab 1632 -> 1196 -> 1046 us, B8 H4 d256
 //   L512..1024 203 -> 213 -> 139 us, B32 H4 d192 L256..1024 502 -> 402 -> 296 us); long rows included (no d rab: B4 H4
@@ -596,8 +686,7 @@ static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
 {
     const hstu_jagged_fwd_params* f = &p->fwd;
     const BwdPlan two = {kTwoLaunches, 0};
-    const char* const env = getenv("HSTU_MI355_BWD_HANDOFF");
-    const int forced = env == nullptr ? -1 : (env[0] == '0' ? 0 : (env[0] == '2' ? 2 : 1));
+    const int forced = switches().bwd_handoff;
     if (forced == 0 || f->total_q == 0 || f->total_k == 0) {
         return two;
     }
@@ -611,10 +700,7 @@ static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
         if (var->dq_ds_p == nullptr) {
             return two;
         }
-        int64_t cap = 4096;
-        if (const char* const cap_env = getenv("HSTU_MI355_BWD_WORKSPACE_MB")) {
-            cap = atoll(cap_env);
-        }
+        const int64_t cap = workspace_cap_mb();
         const int64_t row = 64 * ((f->max_seq_len_k + 31) / 32);
         const int64_t bytes = (f->n_offsets - 1) * f->num_heads_q * f->max_seq_len_q * row * 4;
         const bool fits = f->max_seq_len_q * row * 4 < (1LL << 31) && bytes <= cap * (1LL << 20);
@@ -633,10 +719,7 @@ static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
     }
     const int64_t n_ktiles = (f->max_seq_len_k + hstu::kBlockM - 1) / hstu::kBlockM;
     const bool many_tiles = n_ktiles * batch * f->num_heads_k >= 512;
-    int64_t cap_mb = 4096;
-    if (const char* const cap_env = getenv("HSTU_MI355_BWD_WORKSPACE_MB")) {
-        cap_mb = atoll(cap_env);
-    }
+    const int64_t cap_mb = workspace_cap_mb();
     if (p->grad_attn_bias != nullptr) {
         const int64_t pair_bytes = batch * f->num_heads_q * f->max_seq_len_q * (64 * ((f->max_seq_len_k + 31) / 32)) * 2;
         // (head dims up to 128: while the gradient is small enough for its clearing and the plane to stay in the cache)
@@ -861,6 +944,12 @@ HSTU_API int hstu_version(void) { return (0 << 16) | 1; }
 
 HSTU_API const char* hstu_last_error(void) { return g_err; }
 
+HSTU_API void hstu_reload_switches(void)
+{
+    switches();  // (so that the one-time read cannot come after this one)
+    read_switches();
+}
+
 HSTU_API int hstu_jagged_fwd_workspace_size(const hstu_jagged_fwd_params* params, uint64_t* workspace_bytes)
 {
     if (workspace_bytes == nullptr) {
@@ -893,6 +982,9 @@ HSTU_API const char* hstu_jagged_fwd_kernel_name(const hstu_jagged_fwd_params* p
         return nullptr;
     }
     // (given the workspace asked for; without a usable device the plain name is reported)
+    if (const hstu::ShortVariant* const sv = short_variant(v, params)) {
+        return sv->name;
+    }
     if (takes_queue_variant(v, params, nullptr)) {
         return v->name_queues;
     }
@@ -976,6 +1068,27 @@ int launch_forward(const hstu_jagged_fwd_params* p, const hstu_paged_fwd_params*
     int64_t n_blocks = static_cast<int64_t>(a.n_qtiles) * a.bh;  // one per (query tile, sequence, head) slot
     if (n_blocks <= 0 || n_blocks > 0x7fffffffLL) {
         return fail(HSTU_ERR_INVALID, "grid of %lld workgroups is out of range", (long long)n_blocks);
+    }
+    if (const hstu::ShortVariant* const sv = (paged == nullptr) ? short_variant(var, p) : nullptr) {
+        // one workgroup per (query tile, K/V pair padded to a multiple of 8, query head of the pair) slot
+        const int64_t pairs_pad = (static_cast<int64_t>(a.n_batch) * a.n_heads_k + 7) & ~static_cast<int64_t>(7);
+        const int64_t slots = static_cast<int64_t>(a.n_qtiles) * pairs_pad * a.head_ratio;
+        if (slots > (1LL << 22)) {
+            return fail(HSTU_ERR_INVALID, "grid of %lld workgroups is out of range", (long long)slots);
+        }
+        a.short_spread = a.n_heads_k <= 4 ? 1 : 0;
+#ifdef HSTU_TIMELINE
+        if (const char* const t = getenv("HSTU_TIMELINE_BUFFER")) {
+            a.ws = reinterpret_cast<float*>(strtoull(t, nullptr, 0));  // development builds: where the workgroups leave their time stamps
+        }
+#endif
+        hipLaunchKernelGGL(sv->kernel, dim3(static_cast<unsigned>(slots)), dim3(hstu::kShortThreads), 0,
+                           static_cast<hipStream_t>(stream), a);
+        const hipError_t err_short = hipGetLastError();
+        if (err_short != hipSuccess) {
+            return fail(HSTU_ERR_RUNTIME, "launch of %s failed: %s", sv->name, hipGetErrorString(err_short));
+        }
+        return HSTU_OK;
     }
     void (*kernel)(const hstu::FwdArgs) = var->kernel;
     if (var->persistent_wgs_per_cu > 0) {

@@ -22,6 +22,13 @@ struct Variant {
     int persistent_wgs_per_cu;  // > 0: persistent kernel, this many workgroups per CU; 0: one workgroup per tile
 };
 
+// the forward kernel for short work lists (hstu_fwd_short_kernel.hip.h): one workgroup of `threads` per
+// (query tile, sequence, head) slot, no list, no workspace
+struct ShortVariant {
+    const char* name;
+    void (*kernel)(const FwdArgs);
+};
+
 struct BwdVariant {
     const char* name;
     void (*dkv)(const BwdArgs);
@@ -45,6 +52,8 @@ const Variant (*fwd_variants_f8())[2][2][3];
 const Variant (*fwd_variants_f32())[2][4];
 // forward, 16-bit inputs with head dims in (256, 512], q/k head dim a multiple of 8: [bf16, fp16][rab][custom mask]
 const Variant (*fwd_variants_wide())[2][2];
+// forward for short work lists, 16-bit inputs at the head-dim slot 128 without bias or custom mask: [bf16, fp16]
+const ShortVariant* fwd_variants_short();
 // forward, any head dims up to 512 (written for coverage, not speed): [bf16, fp16, fp32]
 const Variant* fwd_variants_generic();
 // backward: [rab][custom mask][dim slot: 64, 128, 256]

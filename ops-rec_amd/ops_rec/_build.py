@@ -22,6 +22,7 @@ SOURCES = [
     "hstu_kernels_fwd_f16.hip",
     "hstu_kernels_fwd_f8.hip",
     "hstu_kernels_fwd_f32.hip",
+    "hstu_kernels_fwd_short.hip",
     "hstu_kernels_bwd_bf16.hip",
     "hstu_kernels_bwd_f16.hip",
 ]

@@ -22,6 +22,7 @@ EXPORTED_SYMBOLS = (
     "hstu_jagged_fwd_noalloc",
     "hstu_jagged_fwd_noalloc_max_workspace",
     "hstu_last_error",
+    "hstu_reload_switches",
     "hstu_version",
     "hstu_jagged_fwd_kernel_name",
     "hstu_jagged_bwd_workspace_size",
@@ -202,6 +203,8 @@ def load() -> ctypes.CDLL:
     lib.hstu_jagged_fwd_noalloc_max_workspace.argtypes = []
     lib.hstu_last_error.restype = ctypes.c_char_p
     lib.hstu_last_error.argtypes = []
+    lib.hstu_reload_switches.restype = None
+    lib.hstu_reload_switches.argtypes = []
     lib.hstu_version.restype = ctypes.c_int
     lib.hstu_version.argtypes = []
     lib.hstu_jagged_fwd_kernel_name.restype = ctypes.c_char_p

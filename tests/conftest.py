@@ -28,3 +28,15 @@ def pytest_collection_modifyitems(config, items):
     for item in items:
         if "gpu" in item.keywords:
             item.add_marker(skip)
+
+
+@pytest.fixture(autouse=True)
+def _switches_follow_the_environment():
+    """A test that changes one of the library's ``HSTU_MI355_*`` switches (``helpers.set_switch``) leaves the library
+    holding that value; once the test's environment has been put back (this fixture is set up first, so it is torn
+    down last) the library reads its switches again."""
+    yield
+    from ops_rec import _native
+
+    if _native._lib is not None:
+        _native._lib.hstu_reload_switches()

@@ -8,6 +8,42 @@ import torch
 from ops_rec import workloads
 
 
+def set_switch(monkeypatch, name, value):
+    """Sets (``value`` a string) or unsets (None) one of the library's ``HSTU_MI355_*`` switches for the rest of the
+    test: the library reads its switches from the environment once per process, so it is told to read them again.
+    (``tests/conftest.py`` has it read them once more when the test's environment has been put back.)"""
+    from ops_rec import _native
+
+    if value is None:
+        monkeypatch.delenv(name, raising=False)
+    else:
+        monkeypatch.setenv(name, value)
+    _native.load().hstu_reload_switches()
+
+
+def poison_workspace(monkeypatch):
+    """The backward's workspace is handed out holding NaN in every element, so that a read of something never
+    written shows in the gradients."""
+    from ops_rec import _ops
+
+    plain = _ops._new_workspace
+
+    def poisoned(n_bytes, device):
+        ws = plain(n_bytes, device)
+        if ws is not None:
+            ws.fill_(0xFF)
+        return ws
+
+    monkeypatch.setattr(_ops, "_new_workspace", poisoned)
+
+
+def withhold_workspace(monkeypatch):
+    """The backward gets no workspace, as when the device has no room for it: the call must work without."""
+    from ops_rec import _ops
+
+    monkeypatch.setattr(_ops, "_new_workspace", lambda n_bytes, device: None)
+
+
 def small_case(seed=0, batch=3, heads=2, dim=32, lo=1, hi=40, dtype=torch.float32, std=1.0, rab=False, custom_mask=False,
                ctx=0, max_target=0, group=0, heads_k=None, dim_v=None, delta=False, index_dtype=torch.int32,
                alpha=None):  # fmt: skip

@@ -18,6 +18,7 @@ import torch
 import ops_rec
 from ops_rec import workloads
 from oracle import hstu_oracle as O
+import helpers
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -53,13 +54,13 @@ def device_grads(w, grad_out):
 def check(w, monkeypatch, seed=5):
     g = torch.Generator(device=DEV).manual_seed(seed)
     grad_out = torch.randn(w.q.shape[0], w.q.shape[1], w.v.shape[2], generator=g, device=DEV).to(w.q.dtype)
-    monkeypatch.setenv("HSTU_MI355_GENERIC_BACKWARD", "0")
+    helpers.set_switch(monkeypatch, "HSTU_MI355_GENERIC_BACKWARD", "0")
     # the workspace in which the query-tile kernel leaves dS for the dK workgroups is not cleared: filled with NaN
     # here, so that a read of an element that was never written would show in dk
-    monkeypatch.setenv("HSTU_MI355_POISON_WORKSPACE", "1")
+    helpers.poison_workspace(monkeypatch)
     got = device_grads(w, grad_out)
     assert torch.equal(device_grads(w, grad_out)[0], got[0])  # reproducible
-    monkeypatch.setenv("HSTU_MI355_GENERIC_BACKWARD", "1")
+    helpers.set_switch(monkeypatch, "HSTU_MI355_GENERIC_BACKWARD", "1")
     comp = device_grads(w, grad_out)
     ref = oracle_grads(w, grad_out)
     tol = 1e-2 if w.q.dtype == torch.bfloat16 else 2e-3
@@ -131,13 +132,13 @@ def test_attn_bias_gradient_handed_to_the_dk_workgroups(kw, custom_mask, monkeyp
     # kernel storing dS and P into a workspace and clearing the gradient / dV and dK workgroups reading them, the dK
     # ones writing the gradient
     for order in ("1", "2"):
-        monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", order)
-        monkeypatch.setenv("HSTU_MI355_POISON_WORKSPACE", "1")
+        helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", order)
+        helpers.poison_workspace(monkeypatch)
         check(w, monkeypatch)
-        monkeypatch.setenv("HSTU_MI355_GENERIC_BACKWARD", "0")
-        monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "0")
+        helpers.set_switch(monkeypatch, "HSTU_MI355_GENERIC_BACKWARD", "0")
+        helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", "0")
         two = device_grads(w, grad_out)
-        monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", order)
+        helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", order)
         other = device_grads(w, grad_out)
         assert torch.equal(two[0], other[0]) and torch.equal(two[3], other[3])  # dq and the bias gradient: the same bits
         if order == "1":
@@ -172,13 +173,13 @@ def test_ds_handed_to_the_dk_workgroups_through_a_workspace(kw, mask, monkeypatc
     g = torch.Generator(device=DEV).manual_seed(6)
     grad_out = torch.randn(w.q.shape[0], w.q.shape[1], w.v.shape[2], generator=g, device=DEV).to(w.q.dtype)
     for order in ("1", "2"):  # three launches (dS handed over) and the planes order (dS and P handed over)
-        monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", order)
-        monkeypatch.setenv("HSTU_MI355_POISON_WORKSPACE", "1")
+        helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", order)
+        helpers.poison_workspace(monkeypatch)
         check(w, monkeypatch)  # against the oracle and the generic kernels
-        monkeypatch.setenv("HSTU_MI355_GENERIC_BACKWARD", "0")
-        monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "0")
+        helpers.set_switch(monkeypatch, "HSTU_MI355_GENERIC_BACKWARD", "0")
+        helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", "0")
         two = device_grads(w, grad_out)
-        monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", order)
+        helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", order)
         other = device_grads(w, grad_out)
         assert torch.equal(two[0], other[0])  # dq: the same kernel arithmetic in every order
         if order == "1":
@@ -187,7 +188,7 @@ def test_ds_handed_to_the_dk_workgroups_through_a_workspace(kw, mask, monkeypatc
             scale = two[i].float().abs().max().item()
             torch.testing.assert_close(other[i].float(), two[i].float(), atol=tol * scale, rtol=tol)
         # a caller that does not bring the workspace the library asked for gets the two-launch order
-        monkeypatch.setenv("HSTU_MI355_POISON_WORKSPACE", "withhold")
+        helpers.withhold_workspace(monkeypatch)
         without = device_grads(w, grad_out)
         assert all(torch.equal(x, y) for x, y in zip(two[:3], without[:3]))
 
@@ -223,14 +224,14 @@ def test_ds_hand_over_with_more_keys_than_queries(rab, monkeypatch):
     w = workloads.Workload(name="delta", q=mk(sum(lq), 4, 128), k=mk(sum(lk), 2, 128), v=mk(sum(lk), 2, 128),
                            seq_offset=offs(lq), max_seq_len=200, silu_scale=1.0, alpha=0.09, seq_offset_k=offs(lk),
                            max_seq_len_k=376, attn_bias=bias, lengths=lq)  # fmt: skip
-    monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "1")
+    helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", "1")
     check(w, monkeypatch)
     g2 = torch.Generator(device=DEV).manual_seed(6)
     grad_out = torch.randn(w.q.shape[0], 4, 128, generator=g2, device=DEV).to(torch.bfloat16)
-    monkeypatch.setenv("HSTU_MI355_GENERIC_BACKWARD", "0")
-    monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "0")
+    helpers.set_switch(monkeypatch, "HSTU_MI355_GENERIC_BACKWARD", "0")
+    helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", "0")
     two = device_grads(w, grad_out)
-    monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "1")
+    helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", "1")
     three = device_grads(w, grad_out)
     assert torch.equal(two[0], three[0]) and torch.equal(two[2], three[2])
     if rab:
@@ -245,8 +246,8 @@ def test_random_shapes_in_both_launch_orders(monkeypatch):
     import random
 
     rnd = random.Random(5)
-    monkeypatch.setenv("HSTU_MI355_GENERIC_BACKWARD", "0")
-    monkeypatch.setenv("HSTU_MI355_POISON_WORKSPACE", "1")
+    helpers.set_switch(monkeypatch, "HSTU_MI355_GENERIC_BACKWARD", "0")
+    helpers.poison_workspace(monkeypatch)
     for case in range(60):
         d = rnd.choice([32, 64, 64, 128, 128, 128, 256, 80, 96, 48, 208])
         heads_k = rnd.choice([1, 2, 3])
@@ -269,12 +270,12 @@ def test_random_shapes_in_both_launch_orders(monkeypatch):
             w = dataclasses.replace(w, mask_type=2, num_context=None, num_target=None, target_group_size=0)
         g = torch.Generator(device=DEV).manual_seed(1000 + case)
         grad_out = torch.randn(w.q.shape[0], heads, w.v.shape[2], generator=g, device=DEV).to(w.q.dtype)
-        monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "0")
+        helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", "0")
         two = device_grads(w, grad_out)
         label = f"case {case}: {kw}, mask_type {mask_type}"
         tol = 1e-2 if w.q.dtype == torch.bfloat16 else 2e-3
         for order in ("1", "2"):  # (2: dS and P through the workspace; with an attn_bias gradient it is order 1 again)
-            monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", order)
+            helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", order)
             other = device_grads(w, grad_out)
             assert all(torch.isfinite(t).all() for t in other if t is not None), label
             assert torch.equal(two[0], other[0]), label
@@ -293,7 +294,7 @@ def test_long_sequences_and_rows_past_the_last_offset(monkeypatch):
     w = dataclasses.replace(w, q=pad(w.q), k=pad(w.k), v=pad(w.v))
     check(w, monkeypatch)
     grad_out = torch.ones(w.q.shape[0], 2, 128, dtype=torch.bfloat16, device=DEV)
-    monkeypatch.setenv("HSTU_MI355_GENERIC_BACKWARD", "0")
+    helpers.set_switch(monkeypatch, "HSTU_MI355_GENERIC_BACKWARD", "0")
     dq, dk, dv, _ = device_grads(w, grad_out)
     assert not dq[-40:].any() and not dk[-40:].any() and not dv[-40:].any()
 
@@ -304,7 +305,7 @@ def test_empty_sequences_and_trailing_repeated_offset(monkeypatch):
 
 
 def test_loss_backward_uses_the_kernels(monkeypatch):
-    monkeypatch.setenv("HSTU_MI355_GENERIC_BACKWARD", "0")
+    helpers.set_switch(monkeypatch, "HSTU_MI355_GENERIC_BACKWARD", "0")
     w = make(batch=2, heads=2, dim=64, lo=100, hi=200, seed=11, rab_std=0.3)
     q, k, v, bias = (t.clone().requires_grad_(True) for t in (w.q, w.k, w.v, w.attn_bias))
     args = list(w.op_args())
@@ -322,7 +323,7 @@ def test_loss_backward_uses_the_kernels(monkeypatch):
 def test_dense_layout_backward(dtype, dim, use_bias, monkeypatch):
     # hstu_dense / hstu_dense_backward: [B, S, N, D], alpha 1, every sequence of full length
     # (torch_extension/hstu_dense_plugin.cpp:41-151); loss.backward() through the registered autograd as well
-    monkeypatch.setenv("HSTU_MI355_GENERIC_BACKWARD", "0")
+    helpers.set_switch(monkeypatch, "HSTU_MI355_GENERIC_BACKWARD", "0")
     batch, seq, heads = 3, 200, 2
     g = torch.Generator().manual_seed(dim)
     mk = lambda *shape, std=0.5: (torch.randn(*shape, generator=g) * std).to(dtype)  # noqa: E731

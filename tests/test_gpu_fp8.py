@@ -14,6 +14,7 @@ import torch
 import ops_rec
 from ops_rec import workloads
 from oracle import hstu_oracle as O
+import helpers
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -207,7 +208,7 @@ def test_c5_full_size_properties(c5):
 
 
 def test_c5_sub_batch_matches_oracle(c5, monkeypatch):
-    monkeypatch.setenv("HSTU_MI355_SPLIT", "0")  # (bit-identity with the full batch needs the same order of fp32 sums)
+    helpers.set_switch(monkeypatch, "HSTU_MI355_SPLIT", "0")  # (bit-identity with the full batch needs the same order of fp32 sums)
     w, x8, sc, kw, out = c5
     order = sorted(range(len(w.lengths)), key=lambda b: w.lengths[b])
     seqs = sorted(order[:3] + [order[len(order) * 3 // 4]])  # three shortest and one of a few hundred rows

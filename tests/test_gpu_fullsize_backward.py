@@ -18,6 +18,7 @@ import ops_rec
 from ops_rec import workloads
 from oracle import hstu_oracle as O
 from test_gpu_fullsize import sub_batch
+import helpers
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -49,8 +50,8 @@ def config(request):
 def test_subbatch_matches_autograd_on_the_oracle(config, order, monkeypatch):
     name, w, grad_out = config
     if order != "library's choice":
-        monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", {"two launches": "0", "three launches": "1", "planes": "2"}[order])
-    monkeypatch.setenv("HSTU_MI355_POISON_WORKSPACE", "1")
+        helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", {"two launches": "0", "three launches": "1", "planes": "2"}[order])
+    helpers.poison_workspace(monkeypatch)
     dq, dk, dv, dbias = backward(w, grad_out)
     for t in (dq, dk, dv) + ((dbias,) if dbias is not None else ()):
         assert torch.isfinite(t).all()
@@ -86,11 +87,11 @@ def test_linear_in_grad_out_and_reproducible(config):
 
 def test_the_launch_orders_agree(config, monkeypatch):
     name, w, grad_out = config
-    monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "0")
+    helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", "0")
     two = backward(w, grad_out)
-    monkeypatch.setenv("HSTU_MI355_POISON_WORKSPACE", "1")
+    helpers.poison_workspace(monkeypatch)
     for order in ("1", "2"):
-        monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", order)
+        helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", order)
         other = backward(w, grad_out)
         assert torch.equal(two[0], other[0])
         if order == "1":

@@ -13,6 +13,7 @@ import ops_rec
 from ops_rec import _ops
 from oracle import hstu_oracle as O
 from helpers import small_case
+import helpers
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -141,15 +142,15 @@ def test_backward_at_head_dims_beyond_the_tuned_kernels(dtype, dim, dim_v):
 def test_backward_of_fp32_inputs_with_all_the_semantics(kw, generic, monkeypatch):
     # fp32 inputs with head dims up to 128 and a q/k head dim that is a multiple of 8 run on the fp32 matrix-instruction
     # backward kernels; HSTU_MI355_GENERIC_BACKWARD=1 sends the same cases through the generic kernels
-    monkeypatch.setenv("HSTU_MI355_GENERIC_BACKWARD", generic)
+    helpers.set_switch(monkeypatch, "HSTU_MI355_GENERIC_BACKWARD", generic)
     base = dict(seed=len(kw) + 23, batch=4, heads=2, dim=32, dim_v=48, lo=20, hi=160, dtype=torch.float32, std=0.5)
     base.update(kw)
     # the matrix-instruction kernels in both of their orders: everything computed where it is used, and dS and P handed
     # from the query-tile kernel to the key-tile kernel through a workspace (filled with NaN here: nothing in it is
     # cleared, the key-tile kernel reads what was written)
     for order in (("0", "2") if generic == "0" else ("0",)):
-        monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", order)
-        monkeypatch.setenv("HSTU_MI355_POISON_WORKSPACE", "1")
+        helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", order)
+        helpers.poison_workspace(monkeypatch)
         check_backward(small_case(**base))
 
 
@@ -160,8 +161,8 @@ def test_backward_of_fp32_inputs_with_all_the_semantics(kw, generic, monkeypatch
 ], ids=lambda kw: "-".join(f"{k}{v}" for k, v in kw.items()))  # fmt: skip
 @pytest.mark.parametrize("order", ["0", "2"], ids=["recompute", "planes"])
 def test_backward_of_fp32_inputs_over_several_query_and_key_tiles(kw, order, monkeypatch):
-    monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", order)
-    monkeypatch.setenv("HSTU_MI355_POISON_WORKSPACE", "1")
+    helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", order)
+    helpers.poison_workspace(monkeypatch)
     base = dict(seed=len(kw) + 41, batch=3, heads=2, dtype=torch.float32, std=0.5)
     base.update(kw)
     check_backward(small_case(**base))

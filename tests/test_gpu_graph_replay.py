@@ -11,6 +11,7 @@ import torch
 
 import ops_rec
 from ops_rec import workloads
+import helpers
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -93,7 +94,7 @@ def test_backward_replays_in_every_launch_order(order, rab, monkeypatch):
     # the backward's launch orders under capture: fills are kernels, the workspace through which the query-tile kernel
     # hands dS (and P) on comes from torch's graph-private pool and is never cleared; the gradients of every replay are
     # compared with eager calls on the same values
-    monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", order)
+    helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", order)
     max_len = 520
 
     def make(seed):

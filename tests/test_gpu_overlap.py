@@ -8,6 +8,7 @@ import pytest
 import torch
 
 import ops_rec
+import helpers
 from ops_rec import _ops, workloads
 
 pytestmark = pytest.mark.gpu
@@ -28,13 +29,16 @@ def cases():
         "queues": lambda s: mk("q", dtype=bf, device=DEV, seed=s, batch=48, heads=4, dim=128, lo=200, hi=2000),
         # two long sequences: split items (arrival counters and partial outputs in the workspace)
         "split": lambda s: mk("s", dtype=bf, device=DEV, seed=s, batch=2, heads=2, dim=128, lo=2500, hi=3000),
-        # a list in between: the plain variant, no counters
+        # a list in between: the plain variant, no counters (with the kernel for short lists switched off), and the
+        # same list on that kernel
         "plain": lambda s: mk("p", dtype=bf, device=DEV, seed=s, batch=24, heads=4, dim=128, lo=100, hi=900),
+        "short": lambda s: mk("p", dtype=bf, device=DEV, seed=s, batch=24, heads=4, dim=128, lo=100, hi=900),
     }
 
 
-@pytest.mark.parametrize("name", ["queues", "split", "plain"])
-def test_many_launches_in_flight_on_several_streams(name):
+@pytest.mark.parametrize("name", ["queues", "split", "plain", "short"])
+def test_many_launches_in_flight_on_several_streams(name, monkeypatch):
+    helpers.set_switch(monkeypatch, "HSTU_MI355_SHORT", None if name == "short" else "0")
     make = cases()[name]
     n_calls, n_streams = 72, 6  # more launches in flight than the 64 counter sets an earlier design shared
     inputs = [make(seed) for seed in range(4)]
@@ -42,6 +46,7 @@ def test_many_launches_in_flight_on_several_streams(name):
     for w in inputs:
         p = prepared(w)
         assert name in ("plain",) or name in p.kernel_name()
+        assert name != "plain" or p.kernel_name().endswith("maskfalse")
         serial.append(p.launch().clone())
     torch.cuda.synchronize()
     streams = [torch.cuda.Stream(device=DEV) for _ in range(n_streams)]

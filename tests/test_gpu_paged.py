@@ -10,6 +10,7 @@ import torch
 import ops_rec
 from helpers import paged_case
 from oracle import hstu_oracle as O
+import helpers
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -106,8 +107,8 @@ def test_long_cache_few_query_rows(monkeypatch):
     # sweeps: the key ranges are split over workgroups; without splitting the result is the same to the last rounding
     c = paged_case(hist=[40, 3], prev=[6000, 2500], targets=[16, 50], page_size=256, heads=4, heads_k=2, dim=128,
                    dtype=torch.bfloat16, std=0.3, seed=21)  # fmt: skip
-    monkeypatch.setenv("HSTU_MI355_SPLIT", "1")
+    helpers.set_switch(monkeypatch, "HSTU_MI355_SPLIT", "1")
     split = check(c, alpha=128**-0.5)
-    monkeypatch.setenv("HSTU_MI355_SPLIT", "0")
+    helpers.set_switch(monkeypatch, "HSTU_MI355_SPLIT", "0")
     whole = check(c, alpha=128**-0.5)
     torch.testing.assert_close(split.float(), whole.float(), atol=2e-7, rtol=2.0**-7)

@@ -13,6 +13,7 @@ import torch
 import ops_rec
 from ops_rec import workloads
 from oracle import hstu_oracle as O
+import helpers
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -55,7 +56,8 @@ CASES = {
 def test_schedule_does_not_change_results(name, monkeypatch):
     # (a sequence run on its own is a short list; without this, its long items would be split over workgroups,
     # which changes the order of the fp32 sums and with it the last bit of some outputs)
-    monkeypatch.setenv("HSTU_MI355_SPLIT", "0")
+    helpers.set_switch(monkeypatch, "HSTU_MI355_SPLIT", "0")
+    helpers.set_switch(monkeypatch, "HSTU_MI355_SHORT", "0")  # (keys up to 1024 would go to the kernel for short lists)
     w = workloads.make(name, dtype=torch.bfloat16, device=DEV, seed=5, **CASES[name])
     out = run(w)
     assert torch.isfinite(out.float()).all()
@@ -76,7 +78,7 @@ def test_schedule_does_not_change_results(name, monkeypatch):
 
 
 def test_fp8_long_list_matches_sequences_run_alone(monkeypatch):
-    monkeypatch.setenv("HSTU_MI355_SPLIT", "0")
+    helpers.set_switch(monkeypatch, "HSTU_MI355_SPLIT", "0")
     w = workloads.make("f8", dtype=torch.bfloat16, device=DEV, seed=7, batch=64, heads=8, heads_k=2, dim=128, lo=1,
                        hi=2048, max_seq_len=2048)  # fmt: skip
     (q8, qs), (k8, ks), (v8, vs) = (workloads.quantize_fp8(t) for t in (w.q, w.k, w.v))

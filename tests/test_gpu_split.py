@@ -17,6 +17,7 @@ import torch
 import ops_rec
 from ops_rec import _ops, workloads
 from oracle import hstu_oracle as O
+import helpers
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda:0"
@@ -36,11 +37,11 @@ def launch(p):
 
 
 def check_split(w, monkeypatch, atol=1e-2, rtol=1e-2):
-    monkeypatch.setenv("HSTU_MI355_SPLIT", "0")
+    helpers.set_switch(monkeypatch, "HSTU_MI355_SPLIT", "0")
     plain = prepare(w)
     assert plain.workspace_bytes == 0 and not plain.kernel_name().endswith("_split")
     want = launch(plain)
-    monkeypatch.setenv("HSTU_MI355_SPLIT", "1")
+    helpers.set_switch(monkeypatch, "HSTU_MI355_SPLIT", "1")
     split = prepare(w)
     assert split.workspace_bytes > 0 and split.kernel_name().endswith("_split"), split.kernel_name()
     got = launch(split)
@@ -113,9 +114,9 @@ def test_fp8_long_sequences(monkeypatch):
     w = workloads.make("f8", dtype=torch.bfloat16, device=DEV, seed=10, batch=2, heads=2, dim=128, lo=2000, hi=5000)
     (q8, qs), (k8, ks), (v8, vs) = (workloads.quantize_fp8(t) for t in (w.q, w.k, w.v))
     kw = dict(mask_type=0, max_seq_len=w.max_seq_len, silu_scale=w.silu_scale, alpha=w.alpha, seq_offset=w.seq_offset)
-    monkeypatch.setenv("HSTU_MI355_SPLIT", "0")
+    helpers.set_switch(monkeypatch, "HSTU_MI355_SPLIT", "0")
     want = ops_rec.hstu_jagged_fp8(q8, k8, v8, qs, ks, vs, **kw)
-    monkeypatch.setenv("HSTU_MI355_SPLIT", "1")
+    helpers.set_switch(monkeypatch, "HSTU_MI355_SPLIT", "1")
     got = ops_rec.hstu_jagged_fp8(q8, k8, v8, qs, ks, vs, **kw)
     torch.testing.assert_close(got.float(), want.float(), atol=2e-7, rtol=2.0**-7)
     assert torch.equal(ops_rec.hstu_jagged_fp8(q8, k8, v8, qs, ks, vs, **kw), got)

@@ -12,6 +12,7 @@ import torch
 import ops_rec
 from ops_rec import _native, _ops
 from ops_rec.autograd import hstu_v1_autograd as ag
+import helpers
 
 _ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
@@ -418,8 +419,8 @@ def test_backward_workspace_follows_the_launch_order(monkeypatch):
         assert lib.hstu_jagged_bwd_workspace_size(ctypes.byref(b), ctypes.byref(ws)) == 0, _native.last_error()
         return ws.value
 
-    monkeypatch.delenv("HSTU_MI355_BWD_HANDOFF", raising=False)
-    monkeypatch.delenv("HSTU_MI355_BWD_WORKSPACE_MB", raising=False)
+    helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", None)
+    helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_WORKSPACE_MB", None)
     c2 = dict(n_offsets=33, num_heads_q=4, num_heads_k=4, total_q=20292, total_k=20292, max_seq_len_q=1024, max_seq_len_k=1024)
     pair = 32 * 4 * 1024 * 64 * 32 * 2  # dS and P: 64 elements per 32-key block of every query row
     one = 32 * 4 * 1024 * 1024 * 2
@@ -436,15 +437,15 @@ def test_backward_workspace_follows_the_launch_order(monkeypatch):
     # fp32: the matrix-instruction kernels (head dims up to 128) hand dS and P over in fp32; the generic ones do not
     assert size(**dict(c2, dtype=_native.DT_FP32, out_dtype=_native.DT_FP32)) == 2 * pair
     assert size(**dict(c2, dtype=_native.DT_FP32, out_dtype=_native.DT_FP32, head_dim_qk=256, head_dim_v=256)) == 0
-    monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "0")
+    helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", "0")
     assert size(**c2) == 0
-    monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "1")
+    helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", "1")
     assert size(**c2) == one and size(**dict(c2, head_dim_qk=64, head_dim_v=64)) == one
-    monkeypatch.setenv("HSTU_MI355_BWD_HANDOFF", "2")
+    helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", "2")
     assert size(**c2) == pair
-    monkeypatch.setenv("HSTU_MI355_BWD_WORKSPACE_MB", "300")  # the limit of the workspace
+    helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_WORKSPACE_MB", "300")  # the limit of the workspace
     assert size(**c2) == one
-    monkeypatch.setenv("HSTU_MI355_BWD_WORKSPACE_MB", "100")
+    helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_WORKSPACE_MB", "100")
     assert size(**c2) == 0
 
 
