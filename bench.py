@@ -50,32 +50,37 @@ INFINITY_CACHE_BYTES = 256 << 20  # MI355X memory-side cache; a working set belo
 # the forward kernel's source at the time).  A figure whose hash no longer matches the source in the tree is stale
 # and is reported as null.
 MEASURED_TRAFFIC = {
-    "C2": (111_200_000, "profiles/hstu_fwd_bf16_d128_C2_trace_and_counters.md", "c3d9640e53904869"),
-    "C3": (298_900_000, "profiles/hstu_fwd_bf16_d128_rab_C3_trace_and_counters.md", "c3d9640e53904869"),
-    "C4": (1_608_700_000, "profiles/hstu_fwd_bf16_d128_rab_C4_trace_and_counters.md", "c3d9640e53904869"),
-    "C5": (842_000_000, "profiles/hstu_fwd_f8e4m3_d128_C5_trace_and_counters.md", "c3d9640e53904869"),
+    "C2": (99_200_000, "profiles/hstu_fwd_bf16_d128_C2_trace_and_counters.md", "1b3804d6e821f3ce"),
+    "C3": (298_700_000, "profiles/hstu_fwd_bf16_d128_rab_C3_trace_and_counters.md", "c6df3d201118c3e8"),
+    "C4": (1_606_400_000, "profiles/hstu_fwd_bf16_d128_rab_C4_trace_and_counters.md", "c6df3d201118c3e8"),
+    "C5": (839_600_000, "profiles/hstu_fwd_f8e4m3_d128_C5_trace_and_counters.md", "c6df3d201118c3e8"),
 }
-KERNEL_SOURCE = os.path.join(_ROOT, "ops-rec_amd", "csrc", "hstu_fwd_kernel.hip.h")
+_CSRC = os.path.join(_ROOT, "ops-rec_amd", "csrc")
+KERNEL_SOURCE = os.path.join(_CSRC, "hstu_fwd_kernel.hip.h")  # the persistent kernel (and the helpers the others share)
+SHORT_KERNEL_SOURCE = os.path.join(_CSRC, "hstu_fwd_short_kernel.hip.h")  # the kernel for short lists
 
 
-def kernel_source_hash() -> str:
-    """sha256[:16] of the forward kernel's code: its source with // comments, trailing blanks and empty lines removed,
-    so that a figure stays valid when only the comments change."""
+def kernel_source_hash(kernel_name: str = "") -> str:
+    """sha256[:16] of the code of the forward kernel that ran (by its name: the kernel for short lists includes the
+    persistent kernel's file for its helpers, so both files count for it): the sources with // comments, trailing
+    blanks and empty lines removed, so that a figure stays valid when only the comments change."""
     import hashlib
     import re
 
-    with open(KERNEL_SOURCE, "r", encoding="utf-8") as f:
-        lines = [re.sub(r"\s*//.*$", "", line.rstrip()) for line in f]
-    code = "\n".join(line for line in lines if line.strip())
-    return hashlib.sha256(code.encode()).hexdigest()[:16]
+    code = []
+    for path in (KERNEL_SOURCE, SHORT_KERNEL_SOURCE) if kernel_name.endswith("_short") else (KERNEL_SOURCE,):
+        with open(path, "r", encoding="utf-8") as f:
+            lines = [re.sub(r"\s*//.*$", "", line.rstrip()) for line in f]
+        code.append("\n".join(line for line in lines if line.strip()))
+    return hashlib.sha256("\n".join(code).encode()).hexdigest()[:16]
 
 
-def measured_traffic(workload: str):
+def measured_traffic(workload: str, kernel_name: str = ""):
     """(bytes or None, where the figure comes from)."""
     if workload not in MEASURED_TRAFFIC:
         return None, "not measured"
     nbytes, source, sha = MEASURED_TRAFFIC[workload]
-    now = kernel_source_hash()
+    now = kernel_source_hash(kernel_name)
     if sha != now:
         return None, f"stale: {source} was taken with kernel source {sha or '?'}, the tree has {now}"
     return nbytes, f"{source} (kernel source {sha})"
@@ -410,7 +415,6 @@ def main() -> int:
             "algorithmic_bytes_per_step": alg_bytes,
             "launch_path": "C ABI hstu_jagged_fwd, back-to-back on one stream",
         },
-        ("pct_of_fp8_mfma_peak" if fp8 else "pct_of_bf16_mfma_peak"): round(100.0 * tflops / peak, 2),
         "ms_per_step_cold": None if cold_ms is None else round(cold_ms, 6),
         "value_cold": None if cold_ms is None else round(flops / (cold_ms * 1e-3) / 1e12, 3),
         "cold_note": (f"{cold_sets} independent input / output sets of {alg_bytes / 1e6:.0f} MB take turns "
@@ -428,8 +432,11 @@ def main() -> int:
             "peak": peak,
             "unit": "TFLOP/s",
             "frac": round(kernel_tflops / peak, 4),
-            "traffic": None if args.drop_rab else measured_traffic(args.workload)[0],
-            "traffic_source": "not measured" if args.drop_rab else measured_traffic(args.workload)[1],
+            "traffic": None if args.drop_rab else measured_traffic(args.workload, kernel_name)[0],
+            "traffic_source": "not measured" if args.drop_rab else measured_traffic(args.workload, kernel_name)[1],
+            "kernel_source_hash": kernel_source_hash(kernel_name),
+            "clock": "HIP events on the launch stream around the timed launches (the fraction of the peak is quoted "
+                     "on this clock only; 'value' and 'ms_per_step' are the host's clock around the same launches)",
             "avg_launch_us": round(ev_ms * 1e3, 3),
             "hbm_achieved_GBs": round(alg_bytes / (ev_ms * 1e-3) / 1e9, 1),
             "hbm_peak_GBs": PEAK_HBM_GBS,

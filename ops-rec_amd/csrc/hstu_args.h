@@ -75,7 +75,6 @@ struct FwdArgs {
     int64_t num_pages;
     int64_t n_page_ids;
     int page_shift;  // log2(page_size); page_size is 32, 64, 128 or 256
-    int short_spread;  // kernel for short lists: the tiles of a (sequence, K/V head) alternate between two XCDs
 };
 
 struct BwdArgs {

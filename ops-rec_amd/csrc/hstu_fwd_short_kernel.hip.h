@@ -88,25 +88,23 @@ __device__ __forceinline__ uint32_t lds_address(const void* p)
 
 // The slot (position in the grid) of a workgroup -> level, (sequence, K/V head) pair and query head of the pair.
 // Pairs are padded to a multiple of 8 per level so that pair p lands on XCD p mod 8 at every level: the query tiles
-// that read the K / V rows of a pair find them in one L2.  With `spread` the tiles of a pair alternate between the
-// XCDs x and x ^ 4 from level to level: the rows are then fetched into two L2s, and the loads of the two XCDs, each a
-// sum over the few sequences whose pairs fall to it, even out (with 4 K/V heads XCD x holds head x mod 4 of every
-// other sequence: at batch 32 the two halves differ by a fifth of the work; measured on lengths 256..1024, batch 32,
-// 4 heads: 35.6 -> 32.3 us).  The host asks for it with up to 4 K/V heads; with 8 or more every XCD holds one head
-// of all sequences and is balanced as it is.
+// that read the K / V rows of a pair find them in one L2.  (Measured on lengths 256..1024, batch 32, 4 heads: letting
+// the tiles of a pair alternate between two XCDs evens out the XCDs' loads -- with 4 K/V heads XCD x holds head x mod 4
+// of every other sequence, and the two halves of a batch of 32 differ by a fifth of the work -- but fetches 135.4 MB
+// instead of 77.9 MB for the launch and is no faster once the inputs do not replay out of the memory-side cache.)
 struct ShortSlot {
     int level;
     int pair;
     int r;  // query head within the K/V head's group
 };
-__device__ __forceinline__ ShortSlot short_slot(int idx, int n_pairs, int ratio, int spread)
+__device__ __forceinline__ ShortSlot short_slot(int idx, int n_pairs, int ratio)
 {
     const int pairs_pad = (n_pairs + 7) & ~7;
     const int per_level = pairs_pad * ratio;
     ShortSlot s;
     s.level = div_small(idx, per_level);
     const int in_level = idx - s.level * per_level;
-    const int x = (in_level & 7) ^ ((spread != 0 && (s.level & 1)) ? 4 : 0);
+    const int x = in_level & 7;
     const int y = in_level >> 3;
     const int yq = div_small(y, ratio);
     s.r = y - yq * ratio;
@@ -158,7 +156,7 @@ __global__ __launch_bounds__(kShortThreads, kShortWavesPerSimd) void hstu_fwd_sh
     const int64_t last_offset = load_index_uniform(a.offs_q, a.n_batch, a.idx64);
 
     // ---- the item of this workgroup ----
-    const ShortSlot slot = short_slot(static_cast<int>(blockIdx.x), n_pairs, ratio, a.short_spread);
+    const ShortSlot slot = short_slot(static_cast<int>(blockIdx.x), n_pairs, ratio);
     bool live = slot.pair < n_pairs && slot.level < n_levels;
     int b = 0, hk = 0;
     if (live) {

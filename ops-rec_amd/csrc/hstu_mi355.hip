@@ -278,7 +278,7 @@ const hstu::ShortVariant* short_variant(const Variant* var, const hstu_jagged_fw
         return nullptr;
     }
     // Measured on MI355X (bf16, head dim 128, persistent kernel -> this one): keys up to 1024 -- batch 32 x 4 heads
-    // lengths 256..1024 37.4 -> 33.6 us, 8 x 4 of 1024 32.9 -> 25.2, 64 x 4 of 512 43.1 -> 39.3, 256 x 4 of 256
+    // lengths 256..1024 37.4 -> 35.0 us, 8 x 4 of 1024 32.9 -> 25.2, 64 x 4 of 512 43.1 -> 39.3, 256 x 4 of 256
     // 68.2 -> 53.2, 2048 x 2 of 32 71.0 -> 40.0, 128 x 4 of 1024 220.9 -> 217.3 (even); keys up to 2048 with one to
     // two slots per resident workgroup -- 8 x 8 of 1536 62.5 -> 52.5, 8 x 4 of 2048 57.4 -> 51.5, 16 x 4 of 2048 even;
     // beyond that the persistent kernel's variants win: 32 x 4 lengths 512..2048 103.7 -> 107.9, 4 x 2 of 2048 36.7
@@ -1076,7 +1076,6 @@ int launch_forward(const hstu_jagged_fwd_params* p, const hstu_paged_fwd_params*
         if (slots > (1LL << 22)) {
             return fail(HSTU_ERR_INVALID, "grid of %lld workgroups is out of range", (long long)slots);
         }
-        a.short_spread = a.n_heads_k <= 4 ? 1 : 0;
 #ifdef HSTU_TIMELINE
         if (const char* const t = getenv("HSTU_TIMELINE_BUFFER")) {
             a.ws = reinterpret_cast<float*>(strtoull(t, nullptr, 0));  // development builds: where the workgroups leave their time stamps

@@ -51,21 +51,23 @@ def _run(cmd: list[str], verbose: bool) -> None:
         raise RuntimeError(f"hipcc failed ({res.returncode}): {' '.join(cmd)}\n{res.stdout}")
 
 
-def build(verbose: bool = False, jobs: int | None = None) -> str:
-    """Compile ``csrc/*.hip`` into ``ops_rec/_lib/libhstu_mi355.so`` (always recompiles every source)."""
-    os.makedirs(LIB_DIR, exist_ok=True)
+def build(verbose: bool = False, jobs: int | None = None, extra_flags: tuple = (), lib_path: str | None = None) -> str:
+    """Compile ``csrc/*.hip`` into ``ops_rec/_lib/libhstu_mi355.so`` (always recompiles every source).
+    ``extra_flags`` / ``lib_path`` build a variant elsewhere (the timeline example builds one with ``-DHSTU_TIMELINE``)."""
+    target = lib_path or LIB_PATH
+    os.makedirs(os.path.dirname(target), exist_ok=True)
     hipcc = hipcc_path()
     jobs = jobs or max(1, min(len(SOURCES), os.cpu_count() or 1, int(os.environ.get("MAX_JOBS", "16"))))
     with tempfile.TemporaryDirectory(prefix="hstu_build_") as obj_dir:
         objects = [os.path.join(obj_dir, os.path.splitext(s)[0] + ".o") for s in SOURCES]
         with ThreadPoolExecutor(max_workers=jobs) as pool:
             jobs_done = [
-                pool.submit(_run, [hipcc, *HIPCC_FLAGS, "-c", os.path.join(CSRC, s), "-o", o], verbose)
+                pool.submit(_run, [hipcc, *HIPCC_FLAGS, *extra_flags, "-c", os.path.join(CSRC, s), "-o", o], verbose)
                 for s, o in zip(SOURCES, objects)
             ]
             for j in jobs_done:
                 j.result()
-        tmp = LIB_PATH + ".tmp"
+        tmp = target + ".tmp"
         _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objects], verbose)
-    os.replace(tmp, LIB_PATH)
-    return LIB_PATH
+    os.replace(tmp, target)
+    return target
