@@ -385,7 +385,7 @@ def main() -> int:
         op(*op_args)
     torch.cuda.synchronize()
     t0 = time.perf_counter()
-    n_py = max(10, args.steps // 4)
+    n_py = max(50, args.steps // 4)
     for _ in range(n_py):
         op(*op_args)
     torch.cuda.synchronize()

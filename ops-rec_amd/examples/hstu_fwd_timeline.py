@@ -46,7 +46,7 @@ def main() -> None:
     buf = torch.zeros(1 << 20, dtype=torch.int64, device=dev)  # 8 words per workgroup
     os.environ["HSTU_TIMELINE_BUFFER"] = str(buf.data_ptr())
     os.environ["HSTU_MI355_SHORT"] = "1"
-    _native.load().hstu_reload_switches()
+    _native.reload_switches()
     p = _ops.prepare_forward(w.q, w.k, w.v, None, None, w.mask_type, w.max_seq_len, w.max_seq_len, w.silu_scale,
                              w.seq_offset, w.seq_offset, w.num_context, w.num_target, w.target_group_size, w.alpha)  # fmt: skip
     if not p.kernel_name().endswith("_short"):

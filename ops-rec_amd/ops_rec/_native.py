@@ -181,6 +181,15 @@ def library_path() -> str:
     return _build.LIB_PATH
 
 
+def reload_switches() -> None:
+    """Has the library read its ``HSTU_MI355_*`` switches from the environment again (it reads them once per process
+    otherwise) and drops the call descriptions the Python side has cached, whose workspace sizes depend on them."""
+    load().hstu_reload_switches()
+    from . import _ops
+
+    _ops._PLAN_CACHE.clear()
+
+
 def load() -> ctypes.CDLL:
     """Load the HIP library; raises if it has not been built."""
     global _lib

@@ -137,6 +137,45 @@ class PreparedForward:
         return name.decode() if name else ""
 
 
+# Validated calls, by everything but the addresses: (shapes, dtypes, devices, scalars) -> (parameter block with the
+# scalar fields filled, workspace bytes).  A steady-state caller repeats one description with new tensors; on a hit
+# the checks below, the filling of the block and the workspace-size call are skipped and only the addresses are
+# patched in.  The library's answer depends on its switches too: ``_native.reload_switches()`` empties the cache.
+_PLAN_CACHE: dict = {}
+_PLAN_CACHE_MAX = 256
+
+
+def _meta(t: Optional[torch.Tensor]):
+    return None if t is None else (t.shape, t.dtype, t.device, t.is_contiguous())
+
+
+def _plan_key(q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max_seq_len_k, silu_scale, seq_offset, seq_offset_k,
+              num_context, num_target, target_group_size, alpha, deterministic, out_dtype, q_descale, k_descale,
+              v_descale, fp8_scaled_p):  # fmt: skip
+    return (_meta(q), _meta(k), _meta(v), _meta(mask), _meta(attn_bias), mask_type, max_seq_len_q, max_seq_len_k,
+            silu_scale, _meta(seq_offset), seq_offset_k is seq_offset or _meta(seq_offset_k), _meta(num_context),
+            _meta(num_target), target_group_size, alpha, deterministic, out_dtype, _meta(q_descale), _meta(k_descale),
+            _meta(v_descale), fp8_scaled_p)  # fmt: skip
+
+
+def _prepare_from_plan(plan, q, k, v, mask, attn_bias, seq_offset, seq_offset_k, num_context, num_target, scales):
+    """A cached description applied to new tensors (all of them contiguous and of the index type already: a
+    description is only cached when nothing had to be copied or converted)."""
+    template, ws_bytes, out_shape, out_dtype, use_mask = plan
+    p = _native.FwdParams.from_buffer_copy(template)
+    out = torch.empty(out_shape, dtype=out_dtype, device=q.device)
+    mask_c = mask if use_mask else None
+    p.q, p.k, p.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
+    p.mask, p.attn_bias = _ptr(mask_c), _ptr(attn_bias)
+    p.seq_offset_q, p.seq_offset_k = seq_offset.data_ptr(), seq_offset_k.data_ptr()
+    p.num_context, p.num_target = _ptr(num_context), _ptr(num_target)
+    p.out = out.data_ptr()
+    p.q_descale, p.k_descale, p.v_descale = (_ptr(t) for t in scales)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device) if ws_bytes else None
+    keep = (q, k, v, mask_c, attn_bias, seq_offset, seq_offset_k, num_context, num_target, *scales)
+    return PreparedForward(p, out, ws, ws_bytes, q.device, keep)
+
+
 def prepare_forward(
     q: torch.Tensor,
     k: torch.Tensor,
@@ -170,6 +209,15 @@ def prepare_forward(
     (hstu_forward_v1/test/pytest/test_hstu_jagged.py:183-195), and what a call through the reference's own
     entry point with e4m3 tensors gets; ``False`` quantises ``silu(X) * M`` and applies ``silu_scale`` to the
     fp32 output."""
+    key = None
+    if isinstance(q, torch.Tensor) and isinstance(seq_offset, torch.Tensor) and isinstance(seq_offset_k, torch.Tensor):
+        key = _plan_key(q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max_seq_len_k, silu_scale, seq_offset,
+                        seq_offset_k, num_context, num_target, target_group_size, alpha, deterministic, out_dtype,
+                        q_descale, k_descale, v_descale, fp8_scaled_p)  # fmt: skip
+        plan = _PLAN_CACHE.get(key)
+        if plan is not None:
+            return _prepare_from_plan(plan, q, k, v, mask, attn_bias, seq_offset, seq_offset_k, num_context,
+                                      num_target, (q_descale, k_descale, v_descale))  # fmt: skip
     _check(q.dim() == 3, "The q should be 3D in jagged layout")
     _check(seq_offset is not None and seq_offset_k is not None, "seq_offset is required")
     _check(seq_offset.dim() == 1 and seq_offset.size(0) >= 2,
@@ -271,6 +319,15 @@ def prepare_forward(
     ws = None
     if ws_bytes.value:
         ws = torch.empty(ws_bytes.value, dtype=torch.uint8, device=q_c.device)
+    # remember the description when the tensors went in as they came (nothing copied, nothing converted): the same
+    # description with other tensors then needs only their addresses
+    as_given = (q_c is q and k_c is k and v_c is v and offs_q is seq_offset and offs_k is seq_offset_k and ctx is num_context
+                and tgt is num_target and bias is attn_bias and (mask_c is None or mask_c is mask)
+                and all(t is g for t, g in zip(scales, (q_descale, k_descale, v_descale))))  # fmt: skip
+    if key is not None and as_given:
+        if len(_PLAN_CACHE) >= _PLAN_CACHE_MAX:
+            _PLAN_CACHE.clear()
+        _PLAN_CACHE[key] = (bytes(p), ws_bytes.value, tuple(out.shape), out_dtype, mask_c is not None)
     return PreparedForward(p, out, ws, ws_bytes.value, q_c.device, keep)
 
 

@@ -39,4 +39,4 @@ def _switches_follow_the_environment():
     from ops_rec import _native
 
     if _native._lib is not None:
-        _native._lib.hstu_reload_switches()
+        _native.reload_switches()

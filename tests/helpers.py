@@ -18,7 +18,7 @@ def set_switch(monkeypatch, name, value):
         monkeypatch.delenv(name, raising=False)
     else:
         monkeypatch.setenv(name, value)
-    _native.load().hstu_reload_switches()
+    _native.reload_switches()
 
 
 def poison_workspace(monkeypatch):

@@ -46,7 +46,7 @@ def test_many_launches_in_flight_on_several_streams(name, monkeypatch):
     for w in inputs:
         p = prepared(w)
         assert name in ("plain",) or name in p.kernel_name()
-        assert name != "plain" or p.kernel_name().endswith("maskfalse")
+        assert name != "plain" or not p.kernel_name().endswith(("_queues", "_short"))
         serial.append(p.launch().clone())
     torch.cuda.synchronize()
     streams = [torch.cuda.Stream(device=DEV) for _ in range(n_streams)]

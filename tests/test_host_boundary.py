@@ -533,3 +533,29 @@ def test_public_headers_are_plain_c(tmp_path):
     if gxx is not None:
         subprocess.run([gxx, "-std=c++11", "-Wall", "-Wextra", "-pedantic", "-Werror", "-fsyntax-only", "-x", "c++", "-I", inc,
                         str(src)], check=True)  # fmt: skip
+
+
+def test_forward_descriptions_are_cached_by_everything_but_the_addresses():
+    """``prepare_forward`` keeps a validated description and patches only addresses on a repeat; a description
+    that differs in any shape, type or scalar is validated afresh (the cache must never skip a check that would
+    fail), and the cache is emptied with the switches."""
+    from ops_rec import _ops
+
+    key = lambda **kw: _ops._plan_key(**{**base, **kw})  # noqa: E731
+    t = lambda *shape, dtype=torch.bfloat16: torch.zeros(*shape, dtype=dtype)  # noqa: E731
+    offs = torch.tensor([0, 3, 7], dtype=torch.int32)
+    base = dict(q=t(7, 2, 64), k=t(7, 2, 64), v=t(7, 2, 64), mask=None, attn_bias=None, mask_type=0, max_seq_len_q=8,
+                max_seq_len_k=8, silu_scale=0.0, seq_offset=offs, seq_offset_k=offs, num_context=None, num_target=None,
+                target_group_size=0, alpha=1.0, deterministic=False, out_dtype=None, q_descale=None, k_descale=None,
+                v_descale=None, fp8_scaled_p=False)  # fmt: skip
+    same = key(q=t(7, 2, 64), k=t(7, 2, 64), v=t(7, 2, 64))
+    assert same == key() and hash(same) == hash(key())
+    for change in (dict(q=t(8, 2, 64)), dict(v=t(7, 2, 32)), dict(k=t(7, 2, 64, dtype=torch.float16)), dict(mask_type=2),
+                   dict(max_seq_len_q=16), dict(silu_scale=0.5), dict(alpha=0.25), dict(target_group_size=2),
+                   dict(seq_offset_k=offs.clone()), dict(seq_offset=offs.long(), seq_offset_k=offs.long()),
+                   dict(attn_bias=t(2, 2, 8, 8)), dict(num_context=offs[:2]), dict(q=t(7, 4, 64)[:, ::2]),
+                   dict(deterministic=True)):  # fmt: skip
+        assert key(**change) != same, change
+    _ops._PLAN_CACHE["x"] = None
+    _native.reload_switches()
+    assert not _ops._PLAN_CACHE
