@@ -3,7 +3,7 @@
 // The reference accepts any q/k head dim in [1, 512] and any v head dim in [16, 512] in steps of 16
 // (ascendc/attention/hstu_v1/hstu_forward_v1/op_host/tiling_policy.cpp:68-93).  The MFMA kernels of this library
 // are built for head dims up to 256 with a q/k head dim that is a multiple of 8 (16-byte chunks).  This kernel
-// covers the rest -- head dims up to 512, any q/k head dim, bf16 / fp16 / fp32 -- so that every input the reference
+// covers the rest -- head dims up to 512, any q/k head dim, bf16 / fp16 / fp32 / fp8-e4m3 -- so that every input the reference
 // takes runs here too.  It is written for coverage, not for speed: plain fp32 arithmetic on the vector unit, the
 // same semantics (O = (silu(alpha (Q K^T + rab)) * silu_scale * M) V, masks, grouped heads, longer key sequences)
 // restated without any of the tuned kernels' machinery, one workgroup per 128-row query tile as in
@@ -21,15 +21,37 @@ namespace hstu {
 
 constexpr int kGenericMaxDim = 512;
 
+// fp8-e4m3 (OCP e4m3fn) elements, for the head dims the tuned fp8 kernels do not take (above 256, or a q/k head dim
+// that is not a multiple of 16).  Q, K, V, attn_bias and the custom mask are e4m3; the score is brought to its real
+// scale with the per-head dequantisation scales, P is rounded to e4m3 (nearest even, saturating at +-448) before or
+// after silu_scale is applied (FwdArgs::fp8_scaled_p, as in the tuned kernels), the second product and its sum are
+// fp32, and the V scale (and silu_scale in the second case) goes on the fp32 output, which is OutT (fp16 or bf16).
+struct f8e4m3_elem {
+    uint8_t bits;
+};
+
 template <typename T>
 __device__ __forceinline__ float generic_load(const void* p, int64_t i)
 {
     return static_cast<float>(static_cast<const T*>(p)[i]);
 }
+template <>
+__device__ __forceinline__ float generic_load<f8e4m3_elem>(const void* p, int64_t i)
+{
+    return __builtin_amdgcn_cvt_f32_fp8(static_cast<int>(static_cast<const uint8_t*>(p)[i]), 0);
+}
+// x rounded to e4m3 and back
+__device__ __forceinline__ float round_to_e4m3(float x)
+{
+    x = x > 448.0f ? 448.0f : (x < -448.0f ? -448.0f : x);  // (a NaN passes through)
+    const int packed = __builtin_amdgcn_cvt_pk_fp8_f32(x, 0.0f, 0, false);
+    return __builtin_amdgcn_cvt_f32_fp8(packed, 0);
+}
 
-template <typename T>
+template <typename T, typename OutT = T>
 __global__ __launch_bounds__(256) void hstu_fwd_generic_kernel(const FwdArgs a)
 {
+    constexpr bool F8 = std::is_same<T, f8e4m3_elem>::value;
     constexpr int kThreads = 256;
     constexpr int RB = 16;  // query rows per pass
     constexpr int KB = 16;  // keys per tile
@@ -60,15 +82,15 @@ __global__ __launch_bounds__(256) void hstu_fwd_generic_kernel(const FwdArgs a)
     sq = sq < a.max_q ? sq : a.max_q;
     sk = sk < a.max_k ? sk : a.max_k;
 
-    T* const out = static_cast<T*>(a.out);
+    OutT* const out = static_cast<OutT*>(a.out);
     const int64_t o_row_elems = static_cast<int64_t>(a.n_heads_q) * a.d_v;
     if (qt == 0) {  // rows past the last offset belong to no sequence: zero-fill them
         const int64_t last = load_index(a.offs_q, a.n_batch, a.idx64);
         const int64_t first_tail = last < 0 ? 0 : last;
         const int64_t n_tail = (a.total_q > first_tail ? a.total_q - first_tail : 0) * o_row_elems;
-        T* tail = out + first_tail * o_row_elems;
+        OutT* tail = out + first_tail * o_row_elems;
         for (int64_t e = static_cast<int64_t>(bhid) * kThreads + tid; e < n_tail; e += static_cast<int64_t>(a.bh) * kThreads) {
-            tail[e] = static_cast<T>(0.0f);
+            tail[e] = static_cast<OutT>(0.0f);
         }
     }
     const int r0 = qt * kBlockM;
@@ -92,6 +114,16 @@ __global__ __launch_bounds__(256) void hstu_fwd_generic_kernel(const FwdArgs a)
     const int64_t k_row_elems = static_cast<int64_t>(a.n_heads_k) * a.d_qk;
     const int64_t v_row_elems = static_cast<int64_t>(a.n_heads_k) * a.d_v;
     const int64_t bias_plane = (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k);
+    // fp8: raw score -> real score, what P is multiplied by before it is rounded, what the fp32 output is multiplied by
+    float score_scale = 1.0f, p_scale = a.silu_scale, out_scale = 1.0f;
+    if constexpr (F8) {
+        const float qs = a.q_descale ? a.q_descale[h] : 1.0f;
+        const float ks = a.k_descale ? a.k_descale[hk] : 1.0f;
+        const float vs = a.v_descale ? a.v_descale[hk] : 1.0f;
+        score_scale = qs * ks;
+        p_scale = a.fp8_scaled_p ? a.silu_scale : 1.0f;
+        out_scale = (a.fp8_scaled_p ? 1.0f : a.silu_scale) * vs;
+    }
     const int r = tid >> 4, c = tid & 15;
     constexpr int kMaxCols = kGenericMaxDim / 64;  // groups of 4 consecutive output columns per thread
     const int d_qk4 = (a.d_qk + 3) & ~3;                 // Q / K rows are staged zero-padded to a multiple of 4
@@ -165,15 +197,18 @@ __global__ __launch_bounds__(256) void hstu_fwd_generic_kernel(const FwdArgs a)
                 for (int dd = 0; dd < d_qk4 / 4; ++dd) {
                     s4 += qr[dd] * kr[dd];
                 }
-                float s = (s4[0] + s4[1]) + (s4[2] + s4[3]);
+                float s = ((s4[0] + s4[1]) + (s4[2] + s4[3])) * score_scale;
                 const int64_t at = bias_plane + static_cast<int64_t>(row) * a.max_k + key;
                 if (a.rab != nullptr) {
                     s += generic_load<T>(a.rab, at);
                 }
                 const float x = s * a.alpha;
-                p = x / (1.0f + __expf(-x)) * a.silu_scale;
+                p = x / (1.0f + __expf(-x)) * p_scale;
                 if (a.mask_type == 3) {
                     p *= generic_load<T>(a.mask, at);
+                }
+                if constexpr (F8) {
+                    p = round_to_e4m3(p);
                 }
             }
             s_p[r][c] = p;
@@ -203,7 +238,7 @@ __global__ __launch_bounds__(256) void hstu_fwd_generic_kernel(const FwdArgs a)
                 if (col < a.d_v) {
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        out[(q0 + row) * o_row_elems + static_cast<int64_t>(h) * a.d_v + col + e] = static_cast<T>(acc[jj][e]);
+                        out[(q0 + row) * o_row_elems + static_cast<int64_t>(h) * a.d_v + col + e] = static_cast<OutT>(acc[jj][e] * out_scale);
                     }
                 }
             }

@@ -25,8 +25,13 @@ const Variant (*fwd_variants_f32())[2][4] { return kTable; }
 namespace {
 #define HSTU_GENERIC_VARIANT(T, name) \
     {"hstu_fwd_generic_" name, nullptr, nullptr, hstu_fwd_generic_kernel<T>, nullptr, nullptr, nullptr, kGenericMaxDim, 256, 0}
-const Variant kGeneric[3] = {HSTU_GENERIC_VARIANT(__bf16, "bf16"), HSTU_GENERIC_VARIANT(_Float16, "f16"),
-                             HSTU_GENERIC_VARIANT(float, "f32")};
+#define HSTU_GENERIC_F8_VARIANT(OutT, name)                                                                           \
+    {"hstu_fwd_generic_f8e4m3_" name, nullptr, nullptr, hstu_fwd_generic_kernel<f8e4m3_elem, OutT>, nullptr, nullptr, nullptr, \
+     kGenericMaxDim, 256, 0}
+// [bf16, fp16, fp32, fp8-e4m3 with fp16 output, fp8-e4m3 with bf16 output]
+const Variant kGeneric[5] = {HSTU_GENERIC_VARIANT(__bf16, "bf16"), HSTU_GENERIC_VARIANT(_Float16, "f16"),
+                             HSTU_GENERIC_VARIANT(float, "f32"), HSTU_GENERIC_F8_VARIANT(_Float16, "f16"),
+                             HSTU_GENERIC_F8_VARIANT(__bf16, "bf16")};
 }  // namespace
 const Variant* fwd_variants_generic() { return kGeneric; }
 

@@ -204,10 +204,6 @@ const Variant* select(const hstu_jagged_fwd_params* p)
             fail(HSTU_ERR_UNSUPPORTED, "fp8 inputs produce fp16 (the reference's choice) or bf16 output");
             return nullptr;
         }
-        if (p->head_dim_qk % 16 != 0) {
-            fail(HSTU_ERR_UNSUPPORTED, "fp8 q/k head dim %lld is not a multiple of 16", (long long)p->head_dim_qk);
-            return nullptr;
-        }
     } else if (p->out_dtype != p->dtype) {
         fail(HSTU_ERR_UNSUPPORTED, "out_dtype must equal dtype for bf16 / fp16 / fp32 inputs");
         return nullptr;
@@ -233,10 +229,11 @@ const Variant* select(const hstu_jagged_fwd_params* p)
                                              [p->mask_type == HSTU_MASK_CUSTOM ? 1 : 0];
         }
     }
-    if (p->head_dim_qk % 8 != 0 || dmax > 256 || wide_span) {
+    // (the tuned fp8 kernels read 16-byte chunks of one-byte elements: a q/k head dim that is a multiple of 16)
+    const bool odd_f8 = p->dtype == HSTU_DT_FP8_E4M3 && p->head_dim_qk % 16 != 0;
+    if (p->head_dim_qk % 8 != 0 || dmax > 256 || wide_span || odd_f8) {
         if (p->dtype == HSTU_DT_FP8_E4M3) {
-            fail(HSTU_ERR_UNSUPPORTED, "fp8 inputs are built for head dims up to 256 (got %lld)", (long long)dmax);
-            return nullptr;
+            return &hstu::fwd_variants_generic()[p->out_dtype == HSTU_DT_FP16 ? 3 : 4];
         }
         return &hstu::fwd_variants_generic()[p->dtype == HSTU_DT_BF16 ? 0 : (p->dtype == HSTU_DT_FP16 ? 1 : 2)];
     }

@@ -54,7 +54,7 @@ const Variant (*fwd_variants_f32())[2][4];
 const Variant (*fwd_variants_wide())[2][2];
 // forward for short work lists, 16-bit inputs at the head-dim slot 128 without bias or custom mask: [bf16, fp16]
 const ShortVariant* fwd_variants_short();
-// forward, any head dims up to 512 (written for coverage, not speed): [bf16, fp16, fp32]
+// forward, any head dims up to 512 (written for coverage, not speed): [bf16, fp16, fp32, fp8-e4m3 -> fp16, fp8-e4m3 -> bf16]
 const Variant* fwd_variants_generic();
 // backward: [rab][custom mask][dim slot: 64, 128, 256]
 const BwdVariant (*bwd_variants_bf16())[2][3];

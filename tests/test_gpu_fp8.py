@@ -64,6 +64,46 @@ def test_fp8_forward_matrix(batch, heads, heads_k, d, dv, lo, hi, ctx, tgt, grou
     check(out, x8, sc, kw)
 
 
+@pytest.mark.parametrize("out_dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("ctx,tgt,group,mask_type", [(0, 0, 0, 0), (6, 30, 3, 0), (0, 0, 0, 2)])
+@pytest.mark.parametrize("batch,heads,heads_k,d,dv,lo,hi", [
+    (2, 2, 2, 512, 512, 60, 200), (2, 4, 2, 320, 272, 60, 200), (3, 2, 2, 24, 16, 1, 130), (2, 2, 1, 72, 80, 40, 200),
+    (2, 2, 2, 1, 16, 5, 40), (2, 2, 2, 264, 64, 100, 140),
+])  # fmt: skip
+def test_fp8_head_dims_beyond_the_tuned_kernels(batch, heads, heads_k, d, dv, lo, hi, ctx, tgt, group, mask_type, out_dtype):
+    """Everything the reference's tiling admits for its fp8 target -- any q/k head dim in [1, 512], v head dims up
+    to 512 in steps of 16 (op_host/tiling_policy.cpp:68-93, dtype list op_host/atlas950/op_def_arch.h:23-24) -- runs:
+    head dims above 256 and q/k head dims that are not multiples of 16 on the coverage kernel's e4m3 instantiation."""
+    w, x8, sc = make_case(batch, heads, heads_k, d, dv, lo, hi, seed=batch * 13 + d, extra_len=ctx + tgt)
+    nctx = torch.full((batch,), ctx, dtype=torch.int32) if ctx else None
+    ntgt = torch.full((batch,), tgt, dtype=torch.int32) if tgt else None
+    kw = dict(mask_type=mask_type, max_seq_len=w.max_seq_len, silu_scale=0.0, seq_offset=w.seq_offset,
+              num_context=nctx, num_target=ntgt, target_group_size=group, alpha=d**-0.5)  # fmt: skip
+    kwd = dict(kw, seq_offset=dev(w.seq_offset), num_context=dev(nctx), num_target=dev(ntgt))
+    out = ops_rec.hstu_jagged_fp8(*(dev(t) for t in x8), *(dev(t) for t in sc), out_dtype=out_dtype, **kwd)
+    assert out.dtype == out_dtype
+    check(out, x8, sc, kw)
+
+
+@pytest.mark.parametrize("d,dv", [(512, 512), (40, 48)])
+def test_fp8_beyond_the_tuned_kernels_reference_rounding_point_bias_and_mask(d, dv):
+    """The reference's entry point with e4m3 tensors (no scales, fp16 output, P rounded after silu_scale and the
+    mask) with an e4m3 attn_bias and custom mask, at head dims the coverage kernel takes."""
+    w, x8, _ = make_case(2, 2, 2, d, dv, 20, 90, seed=d, scales=False, std=1.0)
+    g = torch.Generator().manual_seed(d + 1)
+    shape = (2, 2, w.max_seq_len, w.max_seq_len)
+    bias = O.quantize_e4m3(torch.randn(shape, generator=g) * 0.5)
+    mask = O.quantize_e4m3(torch.randint(0, 2, shape, generator=g).float())
+    for mask_type, m in ((0, None), (3, mask)):
+        kw = dict(mask_type=mask_type, max_seq_len=w.max_seq_len, silu_scale=0.25, seq_offset=w.seq_offset, alpha=d**-0.5,
+                  attn_bias=bias, mask=m)  # fmt: skip
+        out = ops_rec.ascendc.attention.hstu_jagged(dev(x8[0]), dev(x8[1]), dev(x8[2]), dev(m), dev(bias), mask_type,
+                                                   w.max_seq_len, 0.25, dev(w.seq_offset), None, None, 0, d**-0.5)  # fmt: skip
+        assert out.dtype == torch.float16
+        want = O.hstu_jagged_forward_fp8(*x8, None, None, None, scaled_p=True, out_dtype=torch.float32, **kw)
+        torch.testing.assert_close(out.float().cpu(), want, atol=2e-3, rtol=1e-2)
+
+
 def test_reference_entry_point_with_e4m3_tensors_gives_half_output():
     # the reference's fp8 call: raw e4m3 tensors through hstu_jagged, no scales, fp16 out
     # (torch_extension/hstu_jagged_plugin.cpp:53-54); with silu_scale 1 the rounding point makes no difference
