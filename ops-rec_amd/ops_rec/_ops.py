@@ -280,8 +280,11 @@ def prepare_forward(
                    f"{name} must be a float32 tensor of {heads} per-head scales on the device of q")  # fmt: skip
             t = t.contiguous()
         scales.append(t)
-    # every row is written by the kernel (rows past the last offset are zero-filled there),
-    # so the zero-fill of the reference adapter (:56-59) is not repeated here
+    # Every row of a well-formed call is written by the kernel (rows past the last offset are zero-filled there), so
+    # the zero-fill of the reference adapter (:56-59) is not repeated here.  Well-formed: the first offset is 0 and no
+    # sequence is longer than max_seq_len; rows before a non-zero first offset and rows of a sequence past
+    # max_seq_len belong to no work item and keep what the allocator handed out, where the reference returns zeros
+    # (tests/test_gpu_output_rows.py pins which rows those are).
     out = torch.empty((q_c.size(0), q_c.size(1), v_c.size(2)), dtype=out_dtype, device=q_c.device)
     keep = (q_c, k_c, v_c, mask_c, bias, offs_q, offs_k, ctx, tgt, *scales)
     p = _native.new_params()

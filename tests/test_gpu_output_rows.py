@@ -149,3 +149,44 @@ def test_no_keys_at_all_still_clears_every_gradient(monkeypatch):
     torch.cuda.synchronize()
     assert dk.numel() == 0 and dv.numel() == 0
     assert float(dq.float().abs().max()) == 0.0 and float(dbias.float().abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("dim, short", [(64, None), (128, None), (128, "0")])
+def test_rows_that_belong_to_no_work_item_are_left_alone(dim, short, monkeypatch):
+    """The precondition of the C ABI, pinned: with a non-zero first offset or a sequence longer than ``max_seq_len``
+    the rows before the first offset and the rows of that sequence past ``max_seq_len`` are neither read nor written
+    (the reference's adapter hands out zeros there, torch_extension/hstu_jagged_plugin.cpp:56-59: a documented
+    difference); every other row is written exactly as in the well-formed call, rows past the last offset as zeros."""
+    import helpers
+
+    helpers.set_switch(monkeypatch, "HSTU_MI355_SHORT", short)  # (head dim 128: both forward kernels)
+    max_len, lead, trail = 150, 3, 5
+    lengths = [40, 190, 150, 7]  # the second one is 40 rows longer than max_seq_len
+    w = workloads.make("pre", dtype=torch.bfloat16, device=DEV, seed=31, batch=4, heads=2, dim=dim, lo=0, hi=0,
+                       lengths=lengths, max_seq_len=max_len)  # fmt: skip
+    total = sum(lengths)
+    pad = lambda t: torch.cat([torch.ones(lead, *t.shape[1:], dtype=t.dtype, device=DEV), t,
+                               torch.ones(trail, *t.shape[1:], dtype=t.dtype, device=DEV)])  # noqa: E731
+    q, k, v = pad(w.q), pad(w.k), pad(w.v)
+    offs = (w.seq_offset + lead).contiguous()
+    p = _ops.prepare_forward(q, k, v, None, None, 0, max_len, max_len, w.silu_scale, offs, offs, None, None, 0, w.alpha)
+    p.out.fill_(float("nan"))
+    out = p.launch()
+    torch.cuda.synchronize()
+    o = offs.cpu().tolist()
+    written = torch.zeros(lead + total + trail, dtype=torch.bool)
+    for b, n in enumerate(lengths):
+        written[o[b] : o[b] + min(n, max_len)] = True
+    written[o[-1] :] = True  # rows past the last offset: zero-filled
+    nan_rows = torch.isnan(out.float()).all(dim=(1, 2)).cpu()
+    finite_rows = torch.isfinite(out.float()).all(dim=(1, 2)).cpu()
+    assert torch.equal(nan_rows, ~written) and torch.equal(finite_rows, written)
+    assert (out[o[-1] :] == 0).all()
+    # the rows that are written equal those of the same sequences in a well-formed call (the long one cut to max_seq_len)
+    cut = [min(n, max_len) for n in lengths]
+    rows = torch.cat([torch.arange(o[b], o[b] + cut[b]) for b in range(4)]).to(DEV)
+    good = workloads.Workload(name="good", q=q[rows], k=k[rows], v=v[rows],
+                              seq_offset=torch.tensor([0] + list(torch.tensor(cut).cumsum(0)), dtype=offs.dtype, device=DEV),
+                              max_seq_len=max_len, silu_scale=w.silu_scale, alpha=w.alpha, lengths=cut)  # fmt: skip
+    want = ops_rec.ascendc.attention.hstu_jagged(*good.op_args())
+    assert torch.equal(out[rows], want)
