@@ -1,4 +1,6 @@
-// forward kernels for short work lists (16-bit inputs, head-dim slot 128, no bias, no custom mask)
+// kernels for short work lists / short rows (16-bit inputs, head-dim slot 128, no bias, no custom mask): the forward, and
+// the backward's query-tile kernel
+#include "hstu_bwd_dq_short_kernel.hip.h"
 #include "hstu_fwd_short_kernel.hip.h"
 #include "hstu_variants.h"
 
@@ -10,4 +12,12 @@ const ShortVariant kTable[2] = {
 };
 }
 const ShortVariant* fwd_variants_short() { return kTable; }
+
+namespace {
+const DqShortVariant kDqShort[2] = {
+    {hstu_bwd_dq_short_kernel<bf16_tag, 128, 0>, hstu_bwd_dq_short_kernel<bf16_tag, 128, 1>, hstu_bwd_dq_short_kernel<bf16_tag, 128, 2>},
+    {hstu_bwd_dq_short_kernel<f16_tag, 128, 0>, hstu_bwd_dq_short_kernel<f16_tag, 128, 1>, hstu_bwd_dq_short_kernel<f16_tag, 128, 2>},
+};
+}
+const DqShortVariant* bwd_variants_dq_short() { return kDqShort; }
 }  // namespace hstu

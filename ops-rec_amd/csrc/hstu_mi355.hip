@@ -759,6 +759,39 @@ static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
     return (dmax > 64 && three_fits && many_tiles) ? three : two;
 }
 
+// The query-tile kernel with 64-row tiles (hstu_bwd_dq_short_kernel.hip.h) where it is the faster one: 16-bit inputs at
+// the head-dim slot 128 without bias or custom mask, in launches whose 128-row tiles would leave compute units idle
+// (at most one (128-row tile, sequence, head) slot per compute unit: measured 9 to 16 % off the whole backward at
+// 4 x 1024 to 16 x 512 rows with 4 heads, level at 1.5 slots per unit, 4 to 9 % slower from 2 slots on, where its
+// 16-row matrix instructions cost more than the finer tiles bring).  HSTU_MI355_SHORT=0 / 1 overrides the rule.
+static const hstu::DqShortVariant* dq_short_variant(const hstu_jagged_bwd_params* p, const BwdVariant* var)
+{
+    const hstu_jagged_fwd_params* f = &p->fwd;
+    const int64_t dmax = f->head_dim_qk > f->head_dim_v ? f->head_dim_qk : f->head_dim_v;
+    if ((f->dtype != HSTU_DT_BF16 && f->dtype != HSTU_DT_FP16) || f->attn_bias != nullptr || f->mask_type == HSTU_MASK_CUSTOM ||
+        dmax <= 64 || dmax > 128 || f->head_dim_qk % 8 != 0 || is_generic_bwd(var) || var->dq_ds_p == nullptr) {
+        return nullptr;
+    }
+    const int forced = switches().short_lists;
+    if (forced == 0) {
+        return nullptr;
+    }
+    if (forced != 1) {
+        int cus = 0;
+        const int64_t slots = ((f->max_seq_len_q + 127) / 128) * (f->n_offsets - 1) * f->num_heads_q;
+        if (compute_units(&cus) != HSTU_OK || slots > cus) {
+            return nullptr;
+        }
+    }
+    return &hstu::bwd_variants_dq_short()[f->dtype == HSTU_DT_BF16 ? 0 : 1];
+}
+// grid of that kernel: one workgroup per (64-row tile, K/V pair padded to a multiple of 8, query head of the pair)
+static int64_t dq_short_grid(const hstu::BwdArgs& a)
+{
+    const int64_t pairs_pad = (static_cast<int64_t>(a.n_batch) * a.n_heads_k + 7) & ~static_cast<int64_t>(7);
+    return ((a.max_q + hstu::kDqShortRows - 1) / hstu::kDqShortRows) * pairs_pad * a.head_ratio;
+}
+
 HSTU_API int hstu_jagged_bwd_workspace_size(const hstu_jagged_bwd_params* params, uint64_t* workspace_bytes)
 {
     if (workspace_bytes == nullptr) {
@@ -859,6 +892,7 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
     // (with both roles in a launch: groups of 8 dV workgroups followed by their 8 dK workgroups, whole groups)
     const int64_t grid_kv = generic ? n_kv_slots : 16 * ((n_kv_slots + 7) / 8);
     const int64_t grid_q = static_cast<int64_t>(a.n_qtiles) * a.n_batch * a.n_heads_q;
+    const hstu::DqShortVariant* const dq_short = generic ? nullptr : dq_short_variant(p, var);
     if (grid_kv > 0x7fffffffLL || grid_q > 0x7fffffffLL) {
         return fail(HSTU_ERR_INVALID, "grid out of range");
     }
@@ -894,7 +928,12 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
             // then a dV-from-P and a dK-from-dS workgroup per key tile (the latter writing dS into that gradient)
             a.p_plane = workspace;
             a.drab_clear_bytes = drab_bytes;
-            hipLaunchKernelGGL(var->dq_ds_p, dim3(static_cast<unsigned>(grid_q)), dim3(256), 0, static_cast<hipStream_t>(stream), a);
+            if (dq_short != nullptr) {
+                hipLaunchKernelGGL(dq_short->dq_ds_p, dim3(static_cast<unsigned>(dq_short_grid(a))), dim3(hstu::kDqShortThreads), 0,
+                                   static_cast<hipStream_t>(stream), a);
+            } else {
+                hipLaunchKernelGGL(var->dq_ds_p, dim3(static_cast<unsigned>(grid_q)), dim3(256), 0, static_cast<hipStream_t>(stream), a);
+            }
             a.drab_clear_bytes = 0;
             hipLaunchKernelGGL(p->grad_attn_bias != nullptr ? var->dv_dk_from_planes_drab : var->dv_dk_from_planes,
                                dim3(static_cast<unsigned>(grid_kv)), dim3(hstu::kDkvThreads), 0,
@@ -911,7 +950,12 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
         hipLaunchKernelGGL(var->dv_only, dim3(static_cast<unsigned>(n_kv_slots)), dim3(hstu::kDkvThreads), 0,
                            static_cast<hipStream_t>(stream), a);
         a.drab_clear_bytes = 0;
-        hipLaunchKernelGGL(var->dq_drab, dim3(static_cast<unsigned>(grid_q)), dim3(256), 0, static_cast<hipStream_t>(stream), a);
+        if (dq_short != nullptr && p->grad_attn_bias == nullptr) {
+            hipLaunchKernelGGL(dq_short->dq_ds, dim3(static_cast<unsigned>(dq_short_grid(a))), dim3(hstu::kDqShortThreads), 0,
+                               static_cast<hipStream_t>(stream), a);
+        } else {
+            hipLaunchKernelGGL(var->dq_drab, dim3(static_cast<unsigned>(grid_q)), dim3(256), 0, static_cast<hipStream_t>(stream), a);
+        }
         hipLaunchKernelGGL(var->dk_from_ds, dim3(static_cast<unsigned>(n_kv_slots)), dim3(hstu::kDkvThreads), 0,
                            static_cast<hipStream_t>(stream), a);
         const hipError_t err3 = hipGetLastError();
@@ -927,8 +971,13 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
         launch_clear(p->grad_attn_bias, drab_bytes, stream);
     }
     if (!generic && f->total_q > 0 && grid_q > 0) {
-        hipLaunchKernelGGL(p->grad_attn_bias != nullptr ? var->dq_drab : var->dq, dim3(static_cast<unsigned>(grid_q)), dim3(256),
-                           0, static_cast<hipStream_t>(stream), a);
+        if (dq_short != nullptr && p->grad_attn_bias == nullptr) {
+            hipLaunchKernelGGL(dq_short->dq, dim3(static_cast<unsigned>(dq_short_grid(a))), dim3(hstu::kDqShortThreads), 0,
+                               static_cast<hipStream_t>(stream), a);
+        } else {
+            hipLaunchKernelGGL(p->grad_attn_bias != nullptr ? var->dq_drab : var->dq, dim3(static_cast<unsigned>(grid_q)), dim3(256),
+                               0, static_cast<hipStream_t>(stream), a);
+        }
     }
     const hipError_t err = hipGetLastError();
     if (err != hipSuccess) {

@@ -29,6 +29,14 @@ struct ShortVariant {
     void (*kernel)(const FwdArgs);
 };
 
+// the query-tile backward kernel for short rows (hstu_bwd_dq_short_kernel.hip.h): 16-bit inputs, head-dim slot 128,
+// no bias, no custom mask; one workgroup of `threads` per (64-row tile, sequence, head) slot
+struct DqShortVariant {
+    void (*dq)(const BwdArgs);       // dQ only
+    void (*dq_ds)(const BwdArgs);    // storing dS (bias layout) for dK workgroups that read it back
+    void (*dq_ds_p)(const BwdArgs);  // storing dS and P for the key-tile workgroups that read them back
+};
+
 struct BwdVariant {
     const char* name;
     void (*dkv)(const BwdArgs);
@@ -59,6 +67,8 @@ const Variant* fwd_variants_generic();
 // backward: [rab][custom mask][dim slot: 64, 128, 256]
 const BwdVariant (*bwd_variants_bf16())[2][3];
 const BwdVariant (*bwd_variants_f16())[2][3];
+// backward, query-tile kernel for short rows: [bf16, fp16]
+const DqShortVariant* bwd_variants_dq_short();
 // backward, fp32 inputs with head dims up to 128 (fp32 MFMA, one workgroup per key tile, the same kernel with and
 // without d rab; launched like the generic ones, behind fills of the outputs): [rab][custom mask][dim slot: 32, 64, 128]
 const BwdVariant (*bwd_variants_f32())[2][3];
