@@ -90,7 +90,11 @@ struct BwdArgs {
     void* dk;
     void* dv;
     void* drab;  // may be null
-    void* p_plane;  // where the query-tile kernel leaves P for dV workgroups that read it back (same shape as drab), or null
+    void* p_plane;  // where the query-tile kernel leaves dS and P for key-tile workgroups that read them back, or null
+    // layout of that plane in the 16-bit kernels (hstu_bwd_kernel.hip.h, pair plane): 128-byte lines per head, and whether
+    // the rows of a sequence's 32-row group G hold the blocks 0 .. G only
+    int64_t plane_head_lines;
+    int plane_tri;
     int64_t drab_clear_bytes;  // > 0: the key-tile kernel clears this many bytes at drab beside its work
     const void* offs_q;
     const void* offs_k;

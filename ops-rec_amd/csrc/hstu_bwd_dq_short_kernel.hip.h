@@ -190,12 +190,9 @@ __global__ __launch_bounds__(kDqShortThreads, kDqShortWavesPerSimd) void hstu_bw
     const int hole_lo_lane = hole_lo - 4 * g;
     const int hole_hi_lane = hole_hi - 4 * g;
 
-    const uint32_t pair_pitch = 64u * static_cast<uint32_t>((a.max_k + 31) / 32);  // elements per row of the plane
     const __amdgpu_buffer_rsrc_t p_rsrc =
-        make_rsrc(WANT_P ? static_cast<uint16_t*>(a.p_plane) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(pair_pitch)
-                         : nullptr,
-                  WANT_P ? static_cast<uint32_t>(a.max_q) * pair_pitch * 2u : 0u);
-    const uint32_t pair_row_off = (wr0 + n < sq) ? static_cast<uint32_t>(wr0 + n) * pair_pitch * 2u : kOutOfRange;
+        make_rsrc(WANT_P ? pair_plane_of(a, sq_info.q0, b, h) : nullptr, WANT_P ? pair_seq_bytes(a, sq) : 0u);
+    const uint32_t pair_row_off = (WANT_P && wr0 + n < sq) ? pair_row_offset(a, wr0 + n) : kOutOfRange;
 
     // STORE 1: dS in the bias layout
     const uint32_t bias_bytes = static_cast<uint32_t>(a.max_q) * static_cast<uint32_t>(a.max_k) * 2u;

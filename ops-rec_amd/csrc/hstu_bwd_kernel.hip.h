@@ -80,6 +80,37 @@ __device__ __forceinline__ SeqInfo load_seq(const BwdArgs& a, int b)
     return s;
 }
 
+// The pair plane of the 16-bit kernels: what the query-tile kernel hands to the key-tile workgroups of the next launch.
+// One 128-byte line per query row and 32-key block: the block's 32 dS values, then its 32 P values.  Lines are packed
+// per head by global query row (offs_q[b] + r; no room for rows that the batch does not have), the lines of a row side by
+// side -- all ceil(max_k / 32) blocks of it, or, for a causal mask over equal query and key offsets without context
+// rows (plane_tri; the host knows this much without reading the offsets), only the blocks 0 .. G that rows of the
+// sequence's 32-row group G can see.  The host sizes the triangular form without knowing the lengths: 32 rows of slack
+// per sequence make ((offs_q[b] + 32 b) (n_blk + 1) + 1) / 2 lines an upper bound of what the sequences ahead of b hold.
+__device__ __forceinline__ int64_t pair_lines_ahead(const BwdArgs& a, int64_t q0, int b)
+{
+    const int64_t n_blk = (a.max_k + 31) / 32;
+    return a.plane_tri ? ((q0 + 32 * static_cast<int64_t>(b)) * (n_blk + 1) + 1) / 2 : q0 * n_blk;
+}
+// first byte of sequence b's lines for head h, and their extent
+__device__ __forceinline__ uint8_t* pair_plane_of(const BwdArgs& a, int64_t q0, int b, int h)
+{
+    return static_cast<uint8_t*>(a.p_plane) + (static_cast<int64_t>(h) * a.plane_head_lines + pair_lines_ahead(a, q0, b)) * 128;
+}
+__device__ __forceinline__ uint32_t pair_seq_bytes(const BwdArgs& a, int sq)
+{
+    const uint32_t groups = static_cast<uint32_t>(sq + 31) >> 5;
+    const uint32_t n_blk = static_cast<uint32_t>(a.max_k + 31) >> 5;
+    return (a.plane_tri ? 16u * groups * (groups + 1u) : static_cast<uint32_t>(sq) * n_blk) * 128u;
+}
+// byte offset, from the sequence's first line, of row r's line for block 0
+__device__ __forceinline__ uint32_t pair_row_offset(const BwdArgs& a, int r)
+{
+    const uint32_t g = static_cast<uint32_t>(r) >> 5;
+    const uint32_t n_blk = static_cast<uint32_t>(a.max_k + 31) >> 5;
+    return (a.plane_tri ? 16u * g * (g + 1u) + (static_cast<uint32_t>(r) & 31u) * (g + 1u) : static_cast<uint32_t>(r) * n_blk) * 128u;
+}
+
 // rows past the last offset belong to no sequence: zero-fill them (all workgroups of a launch share the job)
 __device__ __forceinline__ void zero_tail_rows(void* out, const void* offs, int n_batch, int idx64, int64_t total,
                                                int64_t row_elems, int threads)
@@ -374,15 +405,11 @@ __global__ __launch_bounds__(256, bwd_dq_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void 
         make_rsrc(HAS_MASK ? static_cast<const uint16_t*>(a.mask) + bias_plane : nullptr, HAS_MASK ? bias_bytes : 0u);
     const __amdgpu_buffer_rsrc_t drab_rsrc =
         make_rsrc(WANT_DRAB ? static_cast<uint16_t*>(a.drab) + bias_plane : nullptr, WANT_DRAB ? bias_bytes : 0u);
-    // dS and P together (STORE 2) go to a plane of their own layout: per query row, the 32 dS values of a 32-key block
-    // followed by its 32 P values -- one whole 128-byte line per row and step, where two planes of the bias layout would
-    // each get half a line
-    const uint32_t pair_pitch = 64u * static_cast<uint32_t>((a.max_k + 31) / 32);  // elements per row
+    // dS and P together (STORE 2) go to the pair plane: one whole 128-byte line per row and step, where two planes of the
+    // bias layout would each get half a line
     const __amdgpu_buffer_rsrc_t p_rsrc =
-        make_rsrc(WANT_P ? static_cast<uint16_t*>(a.p_plane) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(pair_pitch)
-                         : nullptr,
-                  WANT_P ? static_cast<uint32_t>(a.max_q) * pair_pitch * 2u : 0u);
-    const uint32_t pair_row_off = (wr0 + ln < sq) ? static_cast<uint32_t>(wr0 + ln) * pair_pitch * 2u : kOutOfRange;
+        make_rsrc(WANT_P ? pair_plane_of(a, sq_info.q0, b, h) : nullptr, WANT_P ? pair_seq_bytes(a, sq) : 0u);
+    const uint32_t pair_row_off = (WANT_P && wr0 + ln < sq) ? pair_row_offset(a, wr0 + ln) : kOutOfRange;
     // rows past the sequence lie inside the plane but must stay untouched / unread: their offset leaves it
     const uint32_t bias_row_off =
         (wr0 + ln < sq) ? static_cast<uint32_t>(wr0 + ln) * static_cast<uint32_t>(a.max_k) * 2u : kOutOfRange;
@@ -881,17 +908,17 @@ __global__ __launch_bounds__(kDkvThreads, (MODE == 2 || MODE >= 4) ? bwd_dk_from
         ++ds_steps;
         // (MODE 4: dS and P share a plane of their own layout, see the query-tile kernel: per row and 32-key block, 32
         // dS values followed by 32 P values)
-        const uint32_t pitch = MODE >= 4 ? 64u * static_cast<uint32_t>((a.max_k + 31) / 32) : static_cast<uint32_t>(a.max_k);
-        const __amdgpu_buffer_rsrc_t ds_rsrc = make_rsrc(
-            static_cast<const uint16_t*>(MODE >= 4 ? a.p_plane : a.drab) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(pitch),
-            static_cast<uint32_t>(a.max_q) * pitch * 2u);
+        const uint32_t pitch = static_cast<uint32_t>(a.max_k);
+        const __amdgpu_buffer_rsrc_t ds_rsrc =
+            MODE >= 4 ? make_rsrc(pair_plane_of(a, si.q0, b, h), pair_seq_bytes(a, sq))
+                      : make_rsrc(static_cast<const uint16_t*>(a.drab) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(pitch),
+                                  static_cast<uint32_t>(a.max_q) * pitch * 2u);
+        const uint32_t row_off = MODE >= 4 ? pair_row_offset(a, rq0 + ln) : static_cast<uint32_t>(rq0 + ln) * pitch * 2u;
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int key0 = cw0 + 16 * j + 8 * lh;
             const uint32_t col = MODE >= 4 ? static_cast<uint32_t>(2 * cw0 + 16 * j + 8 * lh + (dk_role ? 0 : 32)) : static_cast<uint32_t>(key0);
-            const uint32_t off = (wanted && rq0 + ln < sq && key0 < sk)
-                                     ? (static_cast<uint32_t>(rq0 + ln) * pitch + col) * 2u
-                                     : kOutOfRange;
+            const uint32_t off = (wanted && rq0 + ln < sq && key0 < sk) ? row_off + col * 2u : kOutOfRange;
             ds_next[j] = __builtin_amdgcn_raw_buffer_load_b128(ds_rsrc, static_cast<int>(off), 0, 0);
         }
     };

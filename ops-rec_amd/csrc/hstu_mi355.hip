@@ -679,6 +679,30 @@ struct BwdPlan {
     uint64_t workspace_bytes;  // what the order needs (0: none)
 };
 
+// The pair plane of the 16-bit backward kernels (dS and P of every (row, 32-key block) the query-tile kernel sweeps, one
+// 128-byte line each; layout in hstu_bwd_kernel.hip.h): rows packed by global query row, and for a causal mask over equal
+// offsets without context rows only the blocks at or below the diagonal -- sized from what the host knows without reading
+// the offsets, total rows and the longest sequence allowed, with 32 rows of slack per sequence.
+struct PairPlane {
+    bool tri;
+    int64_t head_lines;
+    int64_t bytes;
+    bool fits_32;  // one sequence's lines sit behind a 32-bit descriptor
+};
+static PairPlane pair_plane(const hstu_jagged_fwd_params* f)
+{
+    PairPlane pp;
+    const int64_t batch = f->n_offsets - 1;
+    const int64_t n_blk = (f->max_seq_len_k + 31) / 32;
+    pp.tri = f->mask_type == HSTU_MASK_TRIL && f->num_context == nullptr && f->seq_offset_k == f->seq_offset_q &&
+             f->total_k == f->total_q;
+    const int64_t groups = ((f->max_seq_len_q < f->max_seq_len_k ? f->max_seq_len_q : f->max_seq_len_k) + 31) / 32;
+    pp.head_lines = pp.tri ? ((f->total_q + 32 * batch) * (n_blk + 1) + 1) / 2 : f->total_q * n_blk;
+    pp.bytes = f->num_heads_q * pp.head_lines * 128;
+    pp.fits_32 = (pp.tri ? 16 * groups * (groups + 1) : f->max_seq_len_q * n_blk) * 128 < (1LL << 31);
+    return pp;
+}
+
 static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
 {
     const hstu_jagged_fwd_params* f = &p->fwd;
@@ -710,7 +734,8 @@ static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
     const int64_t dmax = f->head_dim_qk > f->head_dim_v ? f->head_dim_qk : f->head_dim_v;
     // (one sequence's part of a plane sits behind a 32-bit descriptor)
     const bool one_fits_32 = f->max_seq_len_q * f->max_seq_len_k * 2 < (1LL << 31);
-    const bool pair_fits_32 = f->max_seq_len_q * (64 * ((f->max_seq_len_k + 31) / 32)) * 2 < (1LL << 31);
+    const PairPlane pp = pair_plane(f);
+    const bool pair_fits_32 = pp.fits_32;
     if (!one_fits_32) {
         return two;
     }
@@ -718,7 +743,7 @@ static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
     const bool many_tiles = n_ktiles * batch * f->num_heads_k >= 512;
     const int64_t cap_mb = workspace_cap_mb();
     if (p->grad_attn_bias != nullptr) {
-        const int64_t pair_bytes = batch * f->num_heads_q * f->max_seq_len_q * (64 * ((f->max_seq_len_k + 31) / 32)) * 2;
+        const int64_t pair_bytes = pp.bytes;
         // (head dims up to 128: while the gradient is small enough for its clearing and the plane to stay in the cache)
         const double grad_bytes = static_cast<double>(batch * f->num_heads_q * f->max_seq_len_q * f->max_seq_len_k * 2);
         const bool small_gradient = grad_bytes * static_cast<double>(f->total_q) / static_cast<double>(batch * f->max_seq_len_q) <= 100e6;
@@ -731,8 +756,7 @@ static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
     }
     const int64_t plane = batch * f->num_heads_q * f->max_seq_len_q * f->max_seq_len_k * 2;
     const bool three_fits = plane <= cap_mb * (1LL << 20);
-    // (dS and P share rows of whole 32-key blocks, 64 elements each)
-    const int64_t pair_plane = batch * f->num_heads_q * f->max_seq_len_q * (64 * ((f->max_seq_len_k + 31) / 32)) * 2;
+    const int64_t pair_plane = pp.bytes;
     const bool planes_fit = pair_fits_32 && pair_plane <= cap_mb * (1LL << 20);
     const BwdPlan three = {kThreeLaunches, static_cast<uint64_t>(plane)};
     const BwdPlan planes = {kPlanes, static_cast<uint64_t>(pair_plane)};
@@ -926,7 +950,10 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
         if (plan.order == kPlanes) {
             // the query-tile kernel with dS and P (clearing the attn_bias gradient beside its work when there is one),
             // then a dV-from-P and a dK-from-dS workgroup per key tile (the latter writing dS into that gradient)
+            const PairPlane pp = pair_plane(f);
             a.p_plane = workspace;
+            a.plane_head_lines = pp.head_lines;
+            a.plane_tri = pp.tri ? 1 : 0;
             a.drab_clear_bytes = drab_bytes;
             if (dq_short != nullptr) {
                 hipLaunchKernelGGL(dq_short->dq_ds_p, dim3(static_cast<unsigned>(dq_short_grid(a))), dim3(hstu::kDqShortThreads), 0,

@@ -399,8 +399,10 @@ def test_backward_c_abi_validation_codes():
 
 def test_backward_workspace_follows_the_launch_order(monkeypatch):
     """hstu_jagged_bwd_workspace_size asks for the workspace of the launch order the library will take: a plane of
-    [batch, heads, max_q, max_k] elements for dS, one of 64 elements per 32-key block for dS and P together, or none
-    (the two-launch order; also whenever HSTU_MI355_BWD_HANDOFF=0)."""
+    [batch, heads, max_q, max_k] elements for dS; for dS and P together one 128-byte line per query row of the batch
+    and 32-key block -- all blocks of a row, or, for a causal mask over equal offsets without context rows, those at or
+    below the diagonal only, bounded from the row count with 32 rows of slack per sequence; or none (the two-launch
+    order; also whenever HSTU_MI355_BWD_HANDOFF=0)."""
     lib = _native.load()
     ws = ctypes.c_uint64(7)
     fake = 0x1000
@@ -421,32 +423,44 @@ def test_backward_workspace_follows_the_launch_order(monkeypatch):
     helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", None)
     helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_WORKSPACE_MB", None)
     c2 = dict(n_offsets=33, num_heads_q=4, num_heads_k=4, total_q=20292, total_k=20292, max_seq_len_q=1024, max_seq_len_k=1024)
-    pair = 32 * 4 * 1024 * 64 * 32 * 2  # dS and P: 64 elements per 32-key block of every query row
+    def pair(rows=20292, batch=32, heads=4, blocks=32):  # causal, equal offsets, no context rows
+        return heads * (((rows + 32 * batch) * (blocks + 1) + 1) // 2) * 128
+
+    def pair_all_blocks(rows=20292, heads=4, blocks=32):
+        return heads * rows * blocks * 128
+
     one = 32 * 4 * 1024 * 1024 * 2
-    assert size(**c2) == pair  # a jagged batch whose planes stay in the memory-side cache: five products
-    assert size(**dict(c2, total_q=32 * 1024, total_k=32 * 1024)) == one  # the same without padding: three launches
-    assert size(**dict(c2, head_dim_qk=64, head_dim_v=64)) == pair  # small planes pay at every head dim
-    assert size(**dict(c2, head_dim_qk=64, head_dim_v=64, total_q=32 * 1024, total_k=32 * 1024)) == 0  # larger ones: two launches
+    full = 32 * 1024
+    assert size(**c2) == pair()  # a jagged batch whose planes stay in the memory-side cache: five products
+    assert pair() < 185e6 < 0.35 * (32 * 4 * 1024 * 32 * 128)  # a third of one line per (padded row, block)
+    assert size(**dict(c2, total_q=full, total_k=full)) == one  # the same without padding: three launches
+    assert size(**dict(c2, head_dim_qk=64, head_dim_v=64)) == pair()  # small planes pay at every head dim
+    assert size(**dict(c2, head_dim_qk=64, head_dim_v=64, total_q=full, total_k=full)) == 0  # larger ones: two launches
     assert size(**dict(c2, max_seq_len_q=1020, max_seq_len_k=1020)) == 0  # rows that are not multiples of 16 bytes
-    assert size(**dict(c2, head_dim_qk=256, head_dim_v=256, total_q=32 * 1024, total_k=32 * 1024)) == pair
+    assert size(**dict(c2, head_dim_qk=256, head_dim_v=256, total_q=full, total_k=full)) == pair(rows=full)
     assert size(**dict(c2, max_seq_len_q=4096, max_seq_len_k=4096)) == 0  # long rows at head dim 128
     assert size(grad_attn_bias=fake, **c2) == 0  # dS goes through the gradient itself (or is recomputed)
-    assert size(grad_attn_bias=fake, **dict(c2, n_offsets=9, total_q=5000, total_k=5000)) == pair // 4  # a small gradient
-    assert size(grad_attn_bias=fake, **dict(c2, head_dim_qk=256, head_dim_v=256)) == pair
-    # fp32: the matrix-instruction kernels (head dims up to 128) hand dS and P over in fp32; the generic ones do not
-    assert size(**dict(c2, dtype=_native.DT_FP32, out_dtype=_native.DT_FP32)) == 2 * pair
+    assert size(grad_attn_bias=fake, **dict(c2, n_offsets=9, total_q=5000, total_k=5000)) == pair(rows=5000, batch=8)  # a small gradient
+    assert size(grad_attn_bias=fake, **dict(c2, head_dim_qk=256, head_dim_v=256)) == pair()
+    # fp32: the matrix-instruction kernels (head dims up to 128) hand dS and P over in fp32, a plane per sequence; the
+    # generic ones do not
+    assert size(**dict(c2, dtype=_native.DT_FP32, out_dtype=_native.DT_FP32)) == 32 * 4 * 1024 * 64 * 32 * 4
     assert size(**dict(c2, dtype=_native.DT_FP32, out_dtype=_native.DT_FP32, head_dim_qk=256, head_dim_v=256)) == 0
     helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", "0")
     assert size(**c2) == 0
     helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", "1")
     assert size(**c2) == one and size(**dict(c2, head_dim_qk=64, head_dim_v=64)) == one
     helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", "2")
-    assert size(**c2) == pair
+    assert size(**c2) == pair()
+    # every block of a row where the host cannot tell that rows see no key past their own: no mask, context rows,
+    # key offsets of their own
+    assert size(**dict(c2, mask_type=2)) == pair_all_blocks()
+    assert size(**dict(c2, num_context=fake)) == pair_all_blocks()
+    assert size(**dict(c2, seq_offset_k=fake + 64)) == pair_all_blocks()
     helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_WORKSPACE_MB", "300")  # the limit of the workspace
-    assert size(**c2) == one
+    assert size(**dict(c2, mask_type=2)) == one
     helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_WORKSPACE_MB", "100")
     assert size(**c2) == 0
-
 
 def test_paged_c_abi_validation_codes():
     lib = _native.load()
