@@ -98,7 +98,7 @@ def algorithmic_bytes(w, out_element_size: int) -> int:
 # HBM bytes per ln_mul launch by rows (cols 512, bf16), from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE scaled by a plain
 # copy of known size (profiles/ln_mul_bf16_c512_trace_and_counters.md)
 # (m, n, k) -> bytes, same method (profiles/in_linear_silu_bf16_trace_and_counters.md)
-IN_LINEAR_SILU_MEASURED_TRAFFIC_BYTES = {(16384, 9216, 64): 623_800_000, (20292, 2048, 512): 338_000_000}
+IN_LINEAR_SILU_MEASURED_TRAFFIC_BYTES = {(16384, 9216, 64): 622_400_000, (20292, 2048, 512): 204_000_000}
 
 
 LN_MUL_MEASURED_TRAFFIC_BYTES = {20292: 62_457_000, 324672: 997_512_000}

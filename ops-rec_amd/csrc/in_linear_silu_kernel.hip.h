@@ -87,10 +87,12 @@ __global__ __launch_bounds__(kIlsThreads, ils_workgroups_per_cu(STAGES, WNB)) vo
     const int wave = uniform(threadIdx.x >> 6);
     const int n_tiles_n = (a.n + kIlsTileN - 1) / kIlsTileN;
     // Tile order.  Plain: n tiles fastest, so the workgroups in flight write whole output rows between them.  Grouped
-    // (a.xcd_groups, chosen by the host for weights far larger than the L2s): workgroup b runs on XCD b % 8, each with
-    // an L2 of its own; blocks are dealt in groups of 8 m tiles, XCD j taking all n tiles of the j-th m tile of the
-    // group, so that an x tile is fetched by one XCD only.  Measured at k = 8192, n = 32768: 7.8 -> 5.8 ms; at k <= 2048
-    // the plain order is 5-10 % faster.  The grid is padded to whole groups; workgroups past the end leave at once.
+    // (a.xcd_groups, chosen by the host for a weight matrix that every L2 can hold beside its streams): workgroup b runs
+    // on XCD b % 8, each with an L2 of its own; blocks are dealt in groups of 8 m tiles, XCD j taking all n tiles of the
+    // j-th m tile of the group, so that an x tile is fetched by one XCD only.  Measured at m = 20292 (plain -> grouped):
+    // n 2048, k 512: fetched bytes 169 -> 38 MB at the same 71 us; n 1024, k 256: 27.7 -> 24.2 us; n 2048, k 128: 41 -> 38 us;
+    // larger weights lose (n 8192, k 2048: 568 -> 661 us; n 32768, k 8192: 4.8 -> 6.1 ms), and so does k = 64 (110 -> 116 us).
+    // The grid is padded to whole groups; workgroups past the end leave at once.
     int tile_m, tile_n;
     if (a.xcd_groups) {
         const int group = blockIdx.x / (kIlsXcds * n_tiles_n);
@@ -294,8 +296,10 @@ __global__ __launch_bounds__(kIlsThreads, ils_workgroups_per_cu(STAGES, WNB)) vo
                 const u32x4_t lin = *reinterpret_cast<const u32x4_t*>(from);
                 const u32x4_t out = *reinterpret_cast<const u32x4_t*>(from + 32 * kEpiRowElems);
                 if (row < a.m && out_col < a.n) {
-                    *reinterpret_cast<u32x4_t*>(static_cast<uint16_t*>(a.linear_output) + row * a.n + out_col) = lin;
-                    *reinterpret_cast<u32x4_t*>(split_base + row * split_cols + split_col) = out;
+                    // (streaming stores: the outputs are not read again by this kernel, and kept out of the L2's way
+                    // they leave the weights and the x tiles there -- 3 to 15 % faster over k = 64 .. 1024)
+                    __builtin_nontemporal_store(lin, reinterpret_cast<u32x4_t*>(static_cast<uint16_t*>(a.linear_output) + row * a.n + out_col));
+                    __builtin_nontemporal_store(out, reinterpret_cast<u32x4_t*>(split_base + row * split_cols + split_col));
                 }
             }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");

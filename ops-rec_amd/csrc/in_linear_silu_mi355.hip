@@ -50,8 +50,12 @@ constexpr int64_t kMaxDim = 512 * 16;
 
 bool aligned16(const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) == 0; }
 
-// a weight matrix beyond what the eight L2s hold between them several times over: x tiles are kept to one XCD each
-bool xcd_groups(const in_linear_silu_params* p) { return p->n * p->k * 2 > (int64_t{64} << 20); }
+// x tiles kept to one XCD each (see the kernel): for a weight matrix of at most 2 MiB -- half an L2 -- with at most 16 n
+// tiles per m tile, rows long enough for the x tiles to weigh against the outputs, and at least four groups of m tiles
+bool xcd_groups(const in_linear_silu_params* p)
+{
+    return p->n * p->k * 2 <= (int64_t{2} << 20) && p->n <= 2048 && p->k >= 128 && p->m >= 4096;
+}
 
 // workgroups of a launch: m tiles (rounded up to whole groups of one per XCD in the grouped order) times n tiles
 int64_t grid_size(const in_linear_silu_params* p)

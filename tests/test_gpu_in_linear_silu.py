@@ -104,6 +104,8 @@ def test_reference_common_input(dtype):
     (200, 1024, 240 + 16, [256] * 4),
     (333, 4096, 1024, [1024, 1008, 1040, 1024]),  # 128 x 256 tiles: partial tiles in m, split edges inside a tile
     (130, 4096 + 64, 1040, [1040, 1040, 1040, 1040]),  # ... and a last n tile of 64 columns, k = 32.5 steps
+    (4100, 1024, 256, [256] * 4),  # m tiles dealt to the XCDs in groups of 8 (small weights, m >= 4096): 33 m tiles
+    (4230, 2048, 128, [512, 496, 528, 512]),
 ])  # fmt: skip
 def test_edges_and_long_k(m, n, k, split):
     g = torch.Generator().manual_seed(m + n + k)
