@@ -9,6 +9,7 @@
 #include <hip/hip_runtime.h>
 #include <stdlib.h>
 
+#include <algorithm>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -634,41 +635,23 @@ HSTU_API int hstu_paged_fwd(const hstu_paged_fwd_params* p, void* workspace, uin
 // Rows of 16 bytes are needed for the planes (max_seq_len_k a multiple of 8, 16-byte aligned pointers).  Nothing in a
 // workspace is cleared: the workgroups that read a plane read exactly the pieces the query-tile kernel wrote.
 //
-// Which order is taken follows what was measured (bf16, events through the operator, two launches -> three -> planes):
-//   C2 (B32 H4 d128 L278..1004)  161 -> 142 -> 109 us      B128 H4 d128 L64..512    166 -> 146 -> 123 us
-//   B8 H4 d128 L512..1024         85 ->  99 ->  65 us      B4 H4 d128 L300..700      64 ->  74 ->  49 us
-//   B16 H4 d256 L100..1504       396 -> 290 -> 213 us      B32 H8 d256 L1024       1258 -> 897 -> 792 us
-//   B64 H4 d128 L256..1024       254 -> 238 -> 235 us      B16 H4 d128 L512..2048   234 -> 219 -> 244 us
-//   B32 H8 d128 L1024            441 -> 430 -> 447 us      B32 H8 d64 L1024         257 -> 298 -> 359 us
-//   B4 H8 d128 L1024..4096       400 -> 503 -> 479 us      B2 H4 d128 L8192         743 -> 928 -> 1201 us
-// A plane costs 4 bytes of traffic per (query, key) pair, written and read back, against two products of
-// 4 x head dim flops per pair each: it pays from the head-dim slot 128 on, and at 128 the second plane only while both
-// stay in the memory-side cache (256 MB) between the launches; few long sequences lose either way (each launch is
-// as long as its heaviest workgroup).  The rule:
-//   head dims above 128 (workspace within the limit: 2 GiB, or HSTU_MI355_BWD_WORKSPACE_MB in the environment): planes,
-//   with or without an attn_bias gradient -- with one the query-tile kernel clears it beside its work and the dK
-//   workgroups write the dS pieces they read into it (B32 H8 d256 L1024 with d rab 1632 -> 1196 -> 1046 us, B8 H4 d256
-//   L512..1024 203 -> 213 -> 139 us, B32 H4 d192 L256..1024 502 -> 402 -> 296 us); long rows included (no d rab: B4 H4
-//   d256 L1024..4096 885 -> 613 -> 465 us, B8 H4 d256 L4096 1845 -> 1257 -> 1135 us) up to max_seq_len_k 4096, three
-//   launches beyond (B2 H4 d256 L8192 1794 -> 1343 -> 1444 us);
-//   head dims up to 128 without an attn_bias gradient, max_seq_len_k up to 2048:  planes when the plane holds at most
-//   about 120 MB (estimated from total_q, the batch and max_seq_len: C2 103 MB, B128 H4 L64..512 85 MB; B32 H8 L512
-//   unpadded 134 MB: 132 us with three launches, 141 us with planes) -- at head dims up to 64 as well (B32 H4 d64
-//   L278..1004 102 -> 103 -> 92 us, B64 H4 d64 L64..512 65 -> 65 -> 52 us, B16 H4 d32 L128..512 40 -> 48 -> 33 us); else,
-//   above head dim 64, three launches from 512 workgroups per launch on (key tiles x sequences x K/V heads: B8 H4
-//   d128 L512..1024 and smaller lose with three); else two;
-//   head dims up to 128 with an attn_bias gradient: planes while that gradient, weighted with the batch's fill
-//   (total_q / (batch x max_seq_len_q)), is at most 100 MB, so that its clearing and the plane stay in the memory-side
-//   cache (B8 H4 d128 L512..1024, 50 MB: 128 -> 136 -> 101 us; B16 H4 d96 L256..1024, 84 MB: 147 -> 152 -> 129 us; B16 H4
-//   d64 L128..512: 59 -> 70 -> 49 us; not B32 H8 d64 L512 unpadded, 134 MB: 157 with three launches, 174 with planes;
-//   nor B32 H4 d64 L256..1024, 168 MB: 176 -> 169 -> 203 us);
-//   else three launches from 512 workgroups per launch on when
-//   max_seq_len_k is at most 1024 (B64 H4 d128 L256..1024 431 -> 382 us, B128 H4 d64 L64..512 177 -> 146 us) or the
-//   batch has no padding, total_q = batch x max_seq_len_q (B32 H8 d128 L2048 2599 -> 2311 us, B32 H8 d32 L4096
-//   8013 -> 6810 us); not for long jagged batches, where the clearing of the gradient no longer hides behind the dV
-//   workgroups alone (B32 H4 d64 L100..1504 310 -> 341 us, B8 H8 d128 L1024..4096 1492 -> 1657 us; C3 396 -> 401 us,
-//   planes 408 us);
-//   everything else (larger planes at head dims up to 64, long rows at head dims up to 128): two launches.
+// Which order is taken follows an estimate of each order's time from what the host knows (batch, total rows, longest
+// sequence allowed, heads, head-dim slot, mask, attn_bias gradient or not), three terms per launch:
+//   products   (visible pairs + 400 per query row and head for the diagonal blocks, the fill and the drain of a tile)
+//              x products of the launch x the rate measured for that kernel family and head-dim slot with the machine
+//              full (us per 10^6 pairs and product, B128 H4 L1024: key-tile kernel 0.197 / 0.336 / 0.891 at slots 64 /
+//              128 / 256, query-tile kernel and the key-tile kernels fed from planes 0.111 / 0.216 / 0.554); the pairs
+//              are estimated as for lengths spread evenly between 2 x mean - max and max;
+//   planes     bytes written or read by the launch beyond its operands (dS 2 bytes per pair, dS and P 4, attn_bias 2, its
+//              gradient 2 and the clearing of the whole gradient) / 10 TB/s for the part of them within 120 MB, which stays
+//              in the memory-side cache between the launches, / 4.5 TB/s beyond (B128 H4 L1024: 537 MB of dS stored in
+//              125 us, 1.07 GB of dS and P in 236 us);
+//   tail       a launch lasts at least as long as its longest workgroup: (longest row / 32) steps (x query heads per K/V
+//              head for key tiles) x (0.3 us + 0.2 / 0.33 / 0.7 us per product of the workgroup).
+// A launch costs the larger of (products + planes) and tail, plus 2 us.  Checked on 34 shapes that none of the constants
+// was taken from (examples/hstu_bwd_order_sweep.py): the order picked is within 10 % of the fastest on 33 of them; with an
+// attn_bias gradient, on the 12 shapes of that example's set "bias", from which the slow-down of the variants that read
+// attn_bias (1.25) and the charge for the gradient's second writing in the planes order were taken.
 // Also tried, not kept: the dV workgroups on a second stream beside the query-tile kernel (C2 143 -> 149 us), and the
 // query-tile kernel first with dV and dK-from-dS workgroups in one launch behind it (C2 160 us).
 // HSTU_MI355_BWD_HANDOFF in the environment overrides the rule: 0 = two launches, 1 = three wherever possible,
@@ -703,6 +686,58 @@ static PairPlane pair_plane(const hstu_jagged_fwd_params* f)
     return pp;
 }
 
+// estimated microseconds of the three launch orders (see above)
+struct BwdCost {
+    double two, three, planes;
+};
+static BwdCost estimate_bwd(const hstu_jagged_fwd_params* f, bool bias_grad)
+{
+    static const double kRateKeyTile[3] = {0.197, 0.336, 0.891};  // us per 10^6 (pair x product), by head-dim slot
+    static const double kRateOther[3] = {0.111, 0.216, 0.554};
+    static const double kStepPerProduct[3] = {0.2, 0.33, 0.7};  // us per 32-key step of a workgroup
+    const double kStepFixed = 0.3, kRowOverhead = 400.0, kCacheBytes = 120e6, kCachedBw = 10.0e6, kMemoryBw = 4.5e6;  // (bytes per us)
+    const double kBiasSlowdown = 1.25;  // the variants that add attn_bias to the scores: fewer workgroups per CU
+    const int64_t dmax = f->head_dim_qk > f->head_dim_v ? f->head_dim_qk : f->head_dim_v;
+    const int slot = dmax <= 64 ? 0 : (dmax <= 128 ? 1 : 2);
+    const double batch = static_cast<double>(f->n_offsets - 1), heads = static_cast<double>(f->num_heads_q);
+    const double max_q = static_cast<double>(f->max_seq_len_q), max_k = static_cast<double>(f->max_seq_len_k);
+    const double mean_q = static_cast<double>(f->total_q) / batch, mean_k = static_cast<double>(f->total_k) / batch;
+    const bool causal = f->mask_type == HSTU_MASK_TRIL;
+    // sum over the sequences of (query rows x keys)
+    double area = batch * (mean_q * mean_k + (max_q > mean_q && max_k > mean_k ? (max_q - mean_q) * (max_k - mean_k) / 3.0 : 0.0));
+    area = std::min(area, static_cast<double>(f->total_q) * max_k);
+    const double pairs = heads * area * (causal ? 0.5 : 1.0);
+    const double mpairs = (pairs + (causal ? 1.0 : 0.4) * kRowOverhead * static_cast<double>(f->total_q) * heads) * 1e-6;
+    const double ratio = static_cast<double>(f->num_heads_q / f->num_heads_k);
+    const double dense = batch * heads * max_q * max_k * 2.0;  // the attn_bias gradient, cleared whole
+    const double bias = bias_grad ? 2.0 * pairs : 0.0;         // attn_bias as read by a launch that computes scores
+    auto launch = [&](int products, const double* rate, int products_per_wg, double bytes, bool key_tiles, bool scores) {
+        const double cached = bytes > kCacheBytes ? kCacheBytes / bytes : 1.0;
+        const double slow = (scores && bias_grad) ? kBiasSlowdown : 1.0;
+        const double work = mpairs * products * rate[slot] * slow + bytes * (cached / kCachedBw + (1.0 - cached) / kMemoryBw);
+        const double steps = (key_tiles ? max_q * ratio : max_k) / 32.0;
+        const double tail = steps * (kStepFixed + products_per_wg * kStepPerProduct[slot]) * slow;
+        return std::max(work, tail) + 2.0;
+    };
+    BwdCost c;
+    if (!bias_grad) {
+        c.two = launch(4, kRateKeyTile, 4, 0.0, true, true) + launch(3, kRateOther, 3, 0.0, false, true);
+        c.three = launch(2, kRateKeyTile, 2, 0.0, true, true) + launch(3, kRateOther, 3, 2.0 * pairs, false, true) +
+                  launch(1, kRateOther, 1, 2.0 * pairs, true, false);
+        c.planes = launch(3, kRateOther, 3, 4.0 * pairs, false, true) + launch(2, kRateOther, 1, 4.0 * pairs, true, false);
+    } else {
+        // (the gradient is cleared beside the first launch's work and written by the query-tile kernel, or, in the planes
+        // order, by the dK workgroups from the dS pieces they read)
+        c.two = launch(4, kRateKeyTile, 4, bias + dense, true, true) + launch(3, kRateOther, 3, bias + 2.0 * pairs, false, true);
+        c.three = launch(2, kRateKeyTile, 2, bias + dense, true, true) + launch(3, kRateOther, 3, bias + 2.0 * pairs, false, true) +
+                  launch(1, kRateOther, 1, 2.0 * pairs, true, false);
+        // (... in 16-byte pieces over lines cleared just before: charged as half the gradient once more, from memory)
+        c.planes = launch(3, kRateOther, 3, bias + 4.0 * pairs + dense, false, true) + launch(2, kRateOther, 1, 6.0 * pairs, true, false) +
+                   0.5 * dense / kMemoryBw;
+    }
+    return c;
+}
+
 static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
 {
     const hstu_jagged_fwd_params* f = &p->fwd;
@@ -731,56 +766,36 @@ static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
         return two;
     }
     const int64_t batch = f->n_offsets - 1;
-    const int64_t dmax = f->head_dim_qk > f->head_dim_v ? f->head_dim_qk : f->head_dim_v;
     // (one sequence's part of a plane sits behind a 32-bit descriptor)
-    const bool one_fits_32 = f->max_seq_len_q * f->max_seq_len_k * 2 < (1LL << 31);
-    const PairPlane pp = pair_plane(f);
-    const bool pair_fits_32 = pp.fits_32;
-    if (!one_fits_32) {
+    if (f->max_seq_len_q * f->max_seq_len_k * 2 >= (1LL << 31)) {
         return two;
     }
-    const int64_t n_ktiles = (f->max_seq_len_k + hstu::kBlockM - 1) / hstu::kBlockM;
-    const bool many_tiles = n_ktiles * batch * f->num_heads_k >= 512;
-    const int64_t cap_mb = workspace_cap_mb();
-    if (p->grad_attn_bias != nullptr) {
-        const int64_t pair_bytes = pp.bytes;
-        // (head dims up to 128: while the gradient is small enough for its clearing and the plane to stay in the cache)
-        const double grad_bytes = static_cast<double>(batch * f->num_heads_q * f->max_seq_len_q * f->max_seq_len_k * 2);
-        const bool small_gradient = grad_bytes * static_cast<double>(f->total_q) / static_cast<double>(batch * f->max_seq_len_q) <= 100e6;
-        if ((forced == 2 || (forced < 0 && (dmax > 128 || small_gradient))) && var->dv_dk_from_planes_drab != nullptr && pair_fits_32 &&
-            pair_bytes <= cap_mb * (1LL << 20)) {
-            return BwdPlan{kPlanes, static_cast<uint64_t>(pair_bytes)};
-        }
-        const bool by_rule = many_tiles && (dmax > 128 || f->max_seq_len_k <= 1024 || f->total_q == batch * f->max_seq_len_q);
-        return (forced >= 1 || (forced < 0 && by_rule)) ? BwdPlan{kThreeLaunches, 0} : two;
-    }
-    const int64_t plane = batch * f->num_heads_q * f->max_seq_len_q * f->max_seq_len_k * 2;
-    const bool three_fits = plane <= cap_mb * (1LL << 20);
-    const int64_t pair_plane = pp.bytes;
-    const bool planes_fit = pair_fits_32 && pair_plane <= cap_mb * (1LL << 20);
-    const BwdPlan three = {kThreeLaunches, static_cast<uint64_t>(plane)};
-    const BwdPlan planes = {kPlanes, static_cast<uint64_t>(pair_plane)};
+    const bool bias_grad = p->grad_attn_bias != nullptr;
+    const PairPlane pp = pair_plane(f);
+    const int64_t cap = workspace_cap_mb() * (1LL << 20);
+    // with an attn_bias gradient dS goes through the gradient itself in the three-launch order: no workspace
+    const int64_t ds_plane = bias_grad ? 0 : batch * f->num_heads_q * f->max_seq_len_q * f->max_seq_len_k * 2;
+    const bool three_fits = ds_plane <= cap;
+    const bool planes_fit = pp.fits_32 && pp.bytes <= cap && (!bias_grad || var->dv_dk_from_planes_drab != nullptr);
+    const BwdPlan three = {kThreeLaunches, static_cast<uint64_t>(ds_plane)};
+    const BwdPlan planes = {kPlanes, static_cast<uint64_t>(pp.bytes)};
     if (forced == 2) {
         return planes_fit ? planes : (three_fits ? three : two);
     }
     if (forced == 1) {
         return three_fits ? three : two;
     }
-    if (dmax > 128) {
-        return (planes_fit && f->max_seq_len_k <= 4096) ? planes : (three_fits ? three : two);
+    const BwdCost cost = estimate_bwd(f, bias_grad);
+    BwdPlan best = two;
+    double best_us = cost.two;
+    if (three_fits && cost.three < best_us) {
+        best = three;
+        best_us = cost.three;
     }
-    if (f->max_seq_len_k > 2048) {
-        return two;
+    if (planes_fit && cost.planes < best_us) {
+        best = planes;
     }
-    // what the plane holds under a causal mask, sum of L^2 / 2 pairs x 4 bytes per head, estimated from what the host
-    // knows as (mean L) x max_seq_len_k x batch with the mean taken twice for padded batches; doubled for other masks
-    const double fill = static_cast<double>(f->total_q) / static_cast<double>(batch * f->max_seq_len_q);
-    const double held = static_cast<double>(f->total_q) * fill * static_cast<double>(f->max_seq_len_k) * f->num_heads_q * 2.0 *
-                        (f->mask_type == HSTU_MASK_TRIL ? 1.0 : 2.0);
-    if (planes_fit && held <= 120e6) {
-        return planes;
-    }
-    return (dmax > 64 && three_fits && many_tiles) ? three : two;
+    return best;
 }
 
 // The query-tile kernel with 64-row tiles (hstu_bwd_dq_short_kernel.hip.h) where it is the faster one: 16-bit inputs at
