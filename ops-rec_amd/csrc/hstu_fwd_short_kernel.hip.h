@@ -21,7 +21,7 @@
 // one), which is why long lists stay on the persistent kernel.  Same arithmetic per element as that kernel:
 // p = s / (1 + exp2(-alpha log2e s)) rounded to the input type, alpha * silu_scale applied once to the fp32 output,
 // rows leave as whole 128-byte lines through LDS.  16-bit inputs, built-in mask (causal with context rows, target
-// rows and target groups) or no mask, no bias.
+// rows and target groups) or no mask, with or without attn_bias (added to the fp32 scores ahead of the SiLU).
 //
 // What this replaces in the reference (Ascend C): the same pieces as the persistent kernel, with the stream-K split
 // of ascendc/attention/hstu_v1/hstu_forward_v1/op_kernel/atlas950/hstu_split_core_policy.h:53-236 answered by
@@ -112,7 +112,25 @@ __device__ __forceinline__ ShortSlot short_slot(int idx, int n_pairs, int ratio)
     return s;
 }
 
-template <typename Tag, int D>
+// attn_bias values for the 16-row kernel, as assembly for the same reason as the tile requests: lane (n, g) asks for
+// the four values at keys 4 g .. 4 g + 3 of each 16-key half of a sub-tile of its row (8 bytes each, 32 bytes apart).
+// The registers named here are written when the data arrives; rab_wait() is where the kernel makes sure of that.
+__device__ __forceinline__ void request_rab(u32x2_t& lo, u32x2_t& hi, u32x4_t rsrc, uint32_t voffset, uint32_t soffset)
+{
+    asm volatile("buffer_load_dwordx2 %0, %2, %3, %4 offen\n\tbuffer_load_dwordx2 %1, %2, %3, %4 offen offset:32"
+                 : "=&v"(lo), "=&v"(hi)
+                 : "v"(voffset), "s"(rsrc), "s"(soffset));
+}
+// waits until at most `open` of this wavefront's memory requests are outstanding; the bias registers pass through
+// it so that nothing that reads them moves ahead of the wait
+template <int OPEN>
+__device__ __forceinline__ void rab_wait(u32x2_t& lo, u32x2_t& hi)
+{
+    static_assert(OPEN >= 0 && OPEN < 16, "vmcnt fits the low four bits here");
+    asm volatile("s_waitcnt vmcnt(%2)" : "+v"(lo), "+v"(hi) : "n"(OPEN));
+}
+
+template <typename Tag, int D, bool HAS_RAB = false>
 __global__ __launch_bounds__(kShortThreads, kShortWavesPerSimd) void hstu_fwd_short_kernel(const FwdArgs a)
 {
     static_assert(D == 128, "built for the head-dim slot 128");
@@ -122,7 +140,9 @@ __global__ __launch_bounds__(kShortThreads, kShortWavesPerSimd) void hstu_fwd_sh
     constexpr int MTILES = D / 16;          // 16-wide output tiles over the head dim (PV product)
     constexpr int SUB_KIB = 32 * D * 2 / 1024;  // 1 KiB load instructions per sub-tile: one per wavefront
     static_assert(SUB_KIB == kShortThreads / 64, "one load instruction per wavefront and sub-tile");
-    constexpr int kWaitTiles = (4 & 15) | (7 << 4) | (15 << 8);  // vmcnt(4): the requests of two steps may be open
+    // vmcnt(4): the tile requests of two steps may be open; with a bias the two bias requests of a step come on top
+    // (steps t - 1 and t: five pairs since the tile requests of sub-tile t + 1)
+    constexpr int kWaitTiles = ((HAS_RAB ? 10 : 4) & 15) | (7 << 4) | (15 << 8);
     constexpr uint32_t kPastEnd = 0x40000000u;
 
     // four slots each for K and V sub-tiles (sub-tile x in slot x mod 4); separate arrays so that the compiler can
@@ -349,6 +369,22 @@ __global__ __launch_bounds__(kShortThreads, kShortWavesPerSimd) void hstu_fwd_sh
         }
         const float c_exp = a.c_exp;
 
+        // ---- attn_bias: [batch, heads, max_q, max_k] in the input type; the values of sub-tile x are asked for two steps
+        // ahead into one of two register blocks (x & 1).  (Four steps ahead into four blocks: 3 to 8 % slower on every
+        // shape measured, 128 registers.)  Requests past the plane of this (sequence, head) read as zeros;
+        // those past the row or the sequence read values that the visibility test discards.
+        u32x4_t rab_rsrc = {0u, 0u, 0u, 0u};
+        uint32_t rab_voff = 0;
+        u32x2_t rab_lo0 = {0u, 0u}, rab_hi0 = {0u, 0u}, rab_lo1 = {0u, 0u}, rab_hi1 = {0u, 0u};
+        if constexpr (HAS_RAB) {
+            const int64_t plane = (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k);
+            rab_rsrc = make_rsrc_words(static_cast<const uint16_t*>(a.rab) + plane,
+                                       static_cast<uint32_t>(a.max_q) * static_cast<uint32_t>(a.max_k) * 2u);
+            rab_voff = static_cast<uint32_t>(wr0 + n) * static_cast<uint32_t>(a.max_k) * 2u + 8u * g;
+            request_rab(rab_lo0, rab_hi0, rab_rsrc, rab_voff, 0u);
+            request_rab(rab_lo1, rab_hi1, rab_rsrc, rab_voff, 64u);
+        }
+
         // one step over sub-tile t, which lies in slot S = t mod 4
         auto step = [&](auto sc, const int t) {
             constexpr int S = decltype(sc)::value;
@@ -367,6 +403,18 @@ __global__ __launch_bounds__(kShortThreads, kShortWavesPerSimd) void hstu_fwd_sh
                     const u32x4_t kb = *reinterpret_cast<const u32x4_t*>(kt + k_lane_off[js] + 16 * D);
                     s0 = mfma16<Tag>(ka, qf[js], s0);
                     s1 = mfma16<Tag>(kb, qf[js], s1);
+                }
+                if constexpr (HAS_RAB) {
+                    // the bias of this sub-tile is in: asked for two steps ago, and since then the tile requests and the
+                    // bias requests of one step and the tile requests of this one have gone out
+                    u32x2_t& lo = (S & 1) ? rab_lo1 : rab_lo0;
+                    u32x2_t& hi = (S & 1) ? rab_hi1 : rab_hi0;
+                    rab_wait<6>(lo, hi);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        s0[e] += (e & 1) ? hi_to_float<Tag>(lo[e >> 1]) : lo_to_float<Tag>(lo[e >> 1]);
+                        s1[e] += (e & 1) ? hi_to_float<Tag>(hi[e >> 1]) : lo_to_float<Tag>(hi[e >> 1]);
+                    }
                 }
                 // P^T = silu(S^T), masked, rounded: element (j, r) is key c0 + 16 j + 4 g + r of this lane's row
                 float p[8];
@@ -396,6 +444,16 @@ __global__ __launch_bounds__(kShortThreads, kShortWavesPerSimd) void hstu_fwd_sh
                     const u32x2_t hi = lds_read_tr16_b64(vp + 16 * D);
                     const u32x4_t va = {lo[0], lo[1], hi[0], hi[1]};
                     o_acc[mt] = mfma16<Tag>(va, pb, o_acc[mt]);
+                }
+            }
+            if constexpr (HAS_RAB) {
+                // the block of sub-tile t is free: ask for sub-tile t + 2 (every step, so that the count of open
+                // requests says the same thing in every wavefront)
+                __builtin_amdgcn_sched_barrier(0);
+                if constexpr (S & 1) {
+                    request_rab(rab_lo1, rab_hi1, rab_rsrc, rab_voff, static_cast<uint32_t>(t + 2) * 64u);
+                } else {
+                    request_rab(rab_lo0, rab_hi0, rab_rsrc, rab_voff, static_cast<uint32_t>(t + 2) * 64u);
                 }
             }
             // sub-tile t + 1 has landed: at most the requests of this step and of the one before are open (mine),
@@ -432,6 +490,11 @@ __global__ __launch_bounds__(kShortThreads, kShortWavesPerSimd) void hstu_fwd_sh
             step(ic3_t{}, t + 3);
         }
 
+        if constexpr (HAS_RAB) {
+            // the bias requests of the last two steps name registers that must stay theirs until they have landed
+            rab_wait<0>(rab_lo0, rab_hi0);
+            rab_wait<0>(rab_lo1, rab_hi1);
+        }
         HSTU_TL(3);
         // ---- store O: lane (n, g) holds dims 16 mt + 4 g + 0..3 of query row wr0 + n ----
         const float c_out = a.c_out;

@@ -1,14 +1,16 @@
-// kernels for short work lists / short rows (16-bit inputs, head-dim slot 128, no bias, no custom mask): the forward, and
-// the backward's query-tile kernel
+// kernels for short work lists / short rows (16-bit inputs, head-dim slot 128, no custom mask): the forward (with and
+// without attn_bias), and the backward's query-tile kernel (no bias)
 #include "hstu_bwd_dq_short_kernel.hip.h"
 #include "hstu_fwd_short_kernel.hip.h"
 #include "hstu_variants.h"
 
 namespace hstu {
 namespace {
-const ShortVariant kTable[2] = {
+const ShortVariant kTable[4] = {
     {"hstu_fwd_bf16_d128_short", hstu_fwd_short_kernel<bf16_tag, 128>},
     {"hstu_fwd_f16_d128_short", hstu_fwd_short_kernel<f16_tag, 128>},
+    {"hstu_fwd_bf16_d128_rab_short", hstu_fwd_short_kernel<bf16_tag, 128, true>},
+    {"hstu_fwd_f16_d128_rab_short", hstu_fwd_short_kernel<f16_tag, 128, true>},
 };
 }
 const ShortVariant* fwd_variants_short() { return kTable; }

@@ -258,12 +258,17 @@ const Variant* select(const hstu_jagged_fwd_params* p)
 // kernel can take the call.
 const hstu::ShortVariant* short_variant(const Variant* var, const hstu_jagged_fwd_params* p)
 {
-    if ((p->dtype != HSTU_DT_BF16 && p->dtype != HSTU_DT_FP16) || p->attn_bias != nullptr ||
-        p->mask_type == HSTU_MASK_CUSTOM || var->d_pad != 128 || var->persistent_wgs_per_cu <= 0 ||
-        var->kernel_queues == nullptr) {
+    if ((p->dtype != HSTU_DT_BF16 && p->dtype != HSTU_DT_FP16) || p->mask_type == HSTU_MASK_CUSTOM || var->d_pad != 128 ||
+        var->persistent_wgs_per_cu <= 0 || var->kernel_queues == nullptr) {
         return nullptr;
     }
-    const hstu::ShortVariant* const sv = &hstu::fwd_variants_short()[p->dtype == HSTU_DT_BF16 ? 0 : 1];
+    // (with a bias: rows of 8-byte pieces)
+    const bool bias = p->attn_bias != nullptr;
+    if (bias && (p->max_seq_len_k % 4 != 0 || reinterpret_cast<uintptr_t>(p->attn_bias) % 8 != 0 ||
+                 p->max_seq_len_q * p->max_seq_len_k * 2 >= (1LL << 32))) {
+        return nullptr;
+    }
+    const hstu::ShortVariant* const sv = &hstu::fwd_variants_short()[(bias ? 2 : 0) + (p->dtype == HSTU_DT_BF16 ? 0 : 1)];
     const int forced = switches().short_lists;
     if (forced == 0) {
         return nullptr;
@@ -284,6 +289,12 @@ const hstu::ShortVariant* short_variant(const Variant* var, const hstu_jagged_fw
     const int64_t resident = static_cast<int64_t>(cus) * var->persistent_wgs_per_cu;
     const int64_t n_qtiles = (p->max_seq_len_q + hstu::kBlockM - 1) / hstu::kBlockM;
     const int64_t n_blocks = n_qtiles * (p->n_offsets - 1) * p->num_heads_q;
+    if (bias) {
+        // with an attn_bias: keys up to 1024 and at most one slot per resident workgroup -- 8 x 4 of 1024 36.6 -> 27.6 us,
+        // 16 x 4 lengths 512..1024 45.0 -> 38.4; two slots per workgroup are even (32 x 4 lengths 256..1024, 64 x 4 of 512)
+        // and longer rows lose (16 x 4 lengths 512..2048 64 -> 84 us, 8 x 8 lengths 1024..2048 80 -> 98)
+        return (p->max_seq_len_k <= 1024 && n_blocks <= resident) ? sv : nullptr;
+    }
     const bool short_keys = p->max_seq_len_k <= 1024;
     const bool one_round = p->max_seq_len_k <= 2048 && n_blocks >= resident && n_blocks <= 2 * resident;
     return (short_keys || one_round) ? sv : nullptr;

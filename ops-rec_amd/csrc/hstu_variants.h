@@ -60,7 +60,8 @@ const Variant (*fwd_variants_f8())[2][2][3];
 const Variant (*fwd_variants_f32())[2][4];
 // forward, 16-bit inputs with head dims in (256, 512], q/k head dim a multiple of 8: [bf16, fp16][rab][custom mask]
 const Variant (*fwd_variants_wide())[2][2];
-// forward for short work lists, 16-bit inputs at the head-dim slot 128 without bias or custom mask: [bf16, fp16]
+// forward for short work lists, 16-bit inputs at the head-dim slot 128 without custom mask: [bf16, fp16, bf16 with
+// attn_bias, fp16 with attn_bias]
 const ShortVariant* fwd_variants_short();
 // forward, any head dims up to 512 (written for coverage, not speed): [bf16, fp16, fp32, fp8-e4m3 -> fp16, fp8-e4m3 -> bf16]
 const Variant* fwd_variants_generic();

@@ -1,4 +1,4 @@
-"""The forward kernel for short work lists (16-bit inputs, head-dim slot 128, no bias, no custom mask): one
+"""The forward kernel for short work lists (16-bit inputs, head-dim slot 128, no custom mask): one
 workgroup of eight 16-row wavefronts per (query tile, sequence, head) slot, no work list.
 
 Checked against the CPU oracle on the mask, layout and index variants it accepts (forced with HSTU_MI355_SHORT=1 so
@@ -60,6 +60,49 @@ def test_against_the_oracle(name, dtype, kernel, monkeypatch):
         torch.testing.assert_close(got, ref, atol=1e-2, rtol=1e-2)
         lo = O.hstu_jagged_forward(w.q, w.k, w.v, out_dtype=dtype, emulate_lowp=dtype, **w.oracle_kwargs()).float()
         assert O.mismatch_fraction(got, lo, 5e-3) < 5e-3
+
+
+BIAS_CASES = {
+    "plain": dict(batch=5, heads=2, dim=128, lo=1, hi=300, max_seq_len=304),
+    "context_targets_groups": dict(batch=4, heads=2, dim=128, lo=20, hi=400, max_seq_len=420, num_context=5, max_target=17,
+                                   target_group_size=3),
+    "grouped_heads_padded_dims": dict(batch=4, heads=4, heads_k=2, dim=96, dim_v=112, lo=1, hi=200, max_seq_len=200),
+    "long_rows": dict(batch=2, heads=1, dim=128, lo=900, hi=1500, max_seq_len=1500),
+    "one_sub_tile": dict(batch=6, heads=2, dim=128, lo=1, hi=31, max_seq_len=32),
+}
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("name", list(BIAS_CASES))
+def test_attn_bias_against_the_oracle(name, dtype, monkeypatch):
+    """With an attn_bias (rows of 8-byte pieces: max_seq_len_k a multiple of 4) the kernel adds it to the fp32 scores
+    ahead of the SiLU, like the persistent kernel; no-mask calls and rows whose last sub-tile runs past the row included."""
+    helpers.set_switch(monkeypatch, "HSTU_MI355_SHORT", "1")
+    for seed, mask_type in ((0, 0), (1, 0), (2, 2)):
+        w = workloads.make("bias", dtype=dtype, std=0.5, rab_std=0.5, seed=seed, **BIAS_CASES[name])
+        if mask_type == 2:
+            w.mask_type, w.num_context, w.num_target, w.target_group_size = 2, None, None, 0
+        wd = w.to(DEV)
+        assert kernel_name(wd).endswith("_d128_rab_short"), kernel_name(wd)
+        got = run(wd).float().cpu()
+        ref = O.hstu_jagged_forward(w.q, w.k, w.v, out_dtype=torch.float32, **w.oracle_kwargs())
+        torch.testing.assert_close(got, ref, atol=1e-2, rtol=1e-2)
+        lo = O.hstu_jagged_forward(w.q, w.k, w.v, out_dtype=dtype, emulate_lowp=dtype, **w.oracle_kwargs()).float()
+        assert O.mismatch_fraction(got, lo, 5e-3) < 5e-3
+        # the persistent kernel on the same inputs: the same sums in another order
+        helpers.set_switch(monkeypatch, "HSTU_MI355_SHORT", "0")
+        assert not kernel_name(wd).endswith("_short")
+        torch.testing.assert_close(run(wd).float().cpu(), got, atol=1e-2, rtol=1e-2)
+        helpers.set_switch(monkeypatch, "HSTU_MI355_SHORT", "1")
+
+
+def test_attn_bias_rows_that_are_not_8_byte_pieces_stay_on_the_persistent_kernel(monkeypatch):
+    helpers.set_switch(monkeypatch, "HSTU_MI355_SHORT", "1")
+    w = workloads.make("bias", dtype=torch.bfloat16, std=0.5, rab_std=0.5, batch=3, heads=2, dim=128, lo=1, hi=90, max_seq_len=90)
+    wd = w.to(DEV)
+    assert "_short" not in kernel_name(wd)
+    ref = O.hstu_jagged_forward(w.q, w.k, w.v, out_dtype=torch.float32, **w.oracle_kwargs())
+    torch.testing.assert_close(run(wd).float().cpu(), ref, atol=1e-2, rtol=1e-2)
 
 
 def test_no_mask_and_empty_sequences_and_rows_past_the_last_offset(monkeypatch):
@@ -134,7 +177,8 @@ def test_the_hosts_rule(monkeypatch):
     assert not name(max_seq_len=2048, batch=32).endswith("_short")  # four per resident workgroup
     assert not name(max_seq_len=2048, batch=2).endswith("_short")  # fewer than workgroups: split items
     assert not name(max_seq_len=4096, batch=4).endswith("_short")
-    assert not name(max_seq_len=1024, rab_std=0.1).endswith("_short")  # bias: persistent kernel
+    assert name(max_seq_len=1024, batch=8, rab_std=0.1).endswith("_rab_short")  # with a bias: up to a slot per workgroup
+    assert not name(max_seq_len=1024, batch=32, rab_std=0.1).endswith("_short")
     assert not name(max_seq_len=1024, dim=64).endswith("_short")  # other head-dim slots
     assert not name(max_seq_len=1024, dim=256).endswith("_short")
     w = workloads.make("m", batch=4, heads=2, dim=128, lo=8, hi=8, max_seq_len=64, dtype=torch.bfloat16, device=DEV)
