@@ -1,7 +1,8 @@
 // kernels for short work lists / short rows (16-bit inputs, head-dim slot 128, no custom mask): the forward (with and
-// without attn_bias), and the backward's query-tile kernel (no bias)
+// without attn_bias), the forward for batches of tiny sequences, and the backward's query-tile kernel (no bias)
 #include "hstu_bwd_dq_short_kernel.hip.h"
 #include "hstu_fwd_short_kernel.hip.h"
+#include "hstu_fwd_tiny_kernel.hip.h"
 #include "hstu_variants.h"
 
 namespace hstu {
@@ -14,6 +15,14 @@ const ShortVariant kTable[4] = {
 };
 }
 const ShortVariant* fwd_variants_short() { return kTable; }
+
+namespace {
+const ShortVariant kTiny[2][2] = {
+    {{"hstu_fwd_bf16_d128_tiny", hstu_fwd_tiny_kernel<bf16_tag, 128>}, {"hstu_fwd_bf16_d256_tiny", hstu_fwd_tiny_kernel<bf16_tag, 256>}},
+    {{"hstu_fwd_f16_d128_tiny", hstu_fwd_tiny_kernel<f16_tag, 128>}, {"hstu_fwd_f16_d256_tiny", hstu_fwd_tiny_kernel<f16_tag, 256>}},
+};
+}
+const ShortVariant (*fwd_variants_tiny())[2] { return kTiny; }
 
 namespace {
 const DqShortVariant kDqShort[2] = {

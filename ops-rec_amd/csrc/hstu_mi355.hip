@@ -250,6 +250,20 @@ const Variant* select(const hstu_jagged_fwd_params* p)
     return &table[p->attn_bias != nullptr ? 1 : 0][p->mask_type == HSTU_MASK_CUSTOM ? 1 : 0][slot];
 }
 
+// The kernel for batches of tiny sequences (hstu_fwd_tiny_kernel.hip.h): 16-bit inputs at the head-dim slots 128 and 256
+// without bias or custom mask, no sequence longer than 32 rows or keys.  Batch 2048 x 2 heads x 32 rows at head dim 256:
+// 135 us on the persistent kernel (a 128-row workgroup and its start-up per item).  HSTU_MI355_SHORT=0 switches it off with
+// the kernel for short lists.
+const hstu::ShortVariant* tiny_variant(const Variant* var, const hstu_jagged_fwd_params* p)
+{
+    if ((p->dtype != HSTU_DT_BF16 && p->dtype != HSTU_DT_FP16) || p->attn_bias != nullptr || p->mask_type == HSTU_MASK_CUSTOM ||
+        (var->d_pad != 128 && var->d_pad != 256) || var->persistent_wgs_per_cu <= 0 || p->max_seq_len_q > hstu::kTinyRows ||
+        p->max_seq_len_k > hstu::kTinyRows || switches().short_lists == 0) {
+        return nullptr;
+    }
+    return &hstu::fwd_variants_tiny()[p->dtype == HSTU_DT_BF16 ? 0 : 1][var->d_pad == 128 ? 0 : 1];
+}
+
 // The kernel for short work lists (hstu_fwd_short_kernel.hip.h) takes 16-bit inputs at the head-dim slot 128 without
 // bias or custom mask.  It is the faster one while the list -- at most n_blocks entries -- is a few items per
 // workgroup the persistent kernel would keep resident: there a launch lasts as long as its longest item, which the
@@ -260,6 +274,9 @@ const hstu::ShortVariant* short_variant(const Variant* var, const hstu_jagged_fw
 {
     if ((p->dtype != HSTU_DT_BF16 && p->dtype != HSTU_DT_FP16) || p->mask_type == HSTU_MASK_CUSTOM || var->d_pad != 128 ||
         var->persistent_wgs_per_cu <= 0 || var->kernel_queues == nullptr) {
+        return nullptr;
+    }
+    if (tiny_variant(var, p) != nullptr) {
         return nullptr;
     }
     // (with a bias: rows of 8-byte pieces)
@@ -380,7 +397,7 @@ uint64_t split_workspace_bytes(const Variant* var, const hstu_jagged_fwd_params*
 // split items, nothing for the lists in between (fixed schedule, no device counters)
 uint64_t forward_workspace_bytes(const Variant* var, const hstu_jagged_fwd_params* p)
 {
-    if (short_variant(var, p) != nullptr) {
+    if (short_variant(var, p) != nullptr || tiny_variant(var, p) != nullptr) {
         return 0;
     }
     if (takes_queue_variant(var, p, nullptr)) {
@@ -1081,6 +1098,9 @@ HSTU_API const char* hstu_jagged_fwd_kernel_name(const hstu_jagged_fwd_params* p
         return nullptr;
     }
     // (given the workspace asked for; without a usable device the plain name is reported)
+    if (const hstu::ShortVariant* const tv = tiny_variant(v, params)) {
+        return tv->name;
+    }
     if (const hstu::ShortVariant* const sv = short_variant(v, params)) {
         return sv->name;
     }
@@ -1167,6 +1187,15 @@ int launch_forward(const hstu_jagged_fwd_params* p, const hstu_paged_fwd_params*
     int64_t n_blocks = static_cast<int64_t>(a.n_qtiles) * a.bh;  // one per (query tile, sequence, head) slot
     if (n_blocks <= 0 || n_blocks > 0x7fffffffLL) {
         return fail(HSTU_ERR_INVALID, "grid of %lld workgroups is out of range", (long long)n_blocks);
+    }
+    if (const hstu::ShortVariant* const tv = (paged == nullptr) ? tiny_variant(var, p) : nullptr) {
+        // one workgroup per (sequence, query head)
+        hipLaunchKernelGGL(tv->kernel, dim3(static_cast<unsigned>(a.bh)), dim3(hstu::kTinyThreads), 0, static_cast<hipStream_t>(stream), a);
+        const hipError_t err_tiny = hipGetLastError();
+        if (err_tiny != hipSuccess) {
+            return fail(HSTU_ERR_RUNTIME, "launch of %s failed: %s", tv->name, hipGetErrorString(err_tiny));
+        }
+        return HSTU_OK;
     }
     if (const hstu::ShortVariant* const sv = (paged == nullptr) ? short_variant(var, p) : nullptr) {
         // one workgroup per (query tile, K/V pair padded to a multiple of 8, query head of the pair) slot

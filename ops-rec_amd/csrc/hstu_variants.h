@@ -63,6 +63,9 @@ const Variant (*fwd_variants_wide())[2][2];
 // forward for short work lists, 16-bit inputs at the head-dim slot 128 without custom mask: [bf16, fp16, bf16 with
 // attn_bias, fp16 with attn_bias]
 const ShortVariant* fwd_variants_short();
+// forward for batches of sequences of at most 32 rows and keys (hstu_fwd_tiny_kernel.hip.h; one workgroup of
+// kTinyThreads per (sequence, head)), no bias, no custom mask: [bf16, fp16][head-dim slot 128, 256]
+const ShortVariant (*fwd_variants_tiny())[2];
 // forward, any head dims up to 512 (written for coverage, not speed): [bf16, fp16, fp32, fp8-e4m3 -> fp16, fp8-e4m3 -> bf16]
 const Variant* fwd_variants_generic();
 // backward: [rab][custom mask][dim slot: 64, 128, 256]

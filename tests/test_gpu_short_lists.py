@@ -96,6 +96,60 @@ def test_attn_bias_against_the_oracle(name, dtype, monkeypatch):
         helpers.set_switch(monkeypatch, "HSTU_MI355_SHORT", "1")
 
 
+TINY_CASES = {
+    "dim256": dict(batch=40, heads=2, dim=256, lo=1, hi=32),
+    "dim128": dict(batch=40, heads=2, dim=128, lo=1, hi=32),
+    "all_32_rows": dict(batch=16, heads=3, dim=256, lo=32, hi=32),
+    "context_targets_groups": dict(batch=12, heads=2, dim=256, lo=12, hi=32, ctx=3, max_target=9, group=2),
+    "grouped_heads_more_keys": dict(batch=10, heads=4, heads_k=2, dim=256, lo=1, hi=24, delta=True),
+    "padded_head_dims": dict(batch=9, heads=2, dim=208, dim_v=144, lo=1, hi=30),
+    "padded_head_dims_128": dict(batch=9, heads=2, dim=80, dim_v=112, lo=1, hi=30),
+    "int64_offsets": dict(batch=7, heads=1, dim=256, lo=5, hi=20, index_dtype=torch.int64),
+}
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("name", list(TINY_CASES))
+def test_tiny_sequences_against_the_oracle(name, dtype, monkeypatch):
+    """Batches whose sequences are all at most 32 rows and keys long take the kernel with one two-wavefront workgroup
+    per (sequence, head); the same inputs on the persistent kernel (switch off) agree with it."""
+    for seed in range(2):
+        helpers.set_switch(monkeypatch, "HSTU_MI355_SHORT", None)
+        w = small_case(seed=seed, dtype=dtype, std=0.5, **TINY_CASES[name])
+        if seed == 1 and "ctx" not in TINY_CASES[name]:
+            w.mask_type = 2  # every key visible
+        wd = w.to(DEV)
+        assert kernel_name(wd).endswith("_tiny"), kernel_name(wd)
+        got = run(wd).float().cpu()
+        ref = O.hstu_jagged_forward(w.q, w.k, w.v, out_dtype=torch.float32, **w.oracle_kwargs())
+        torch.testing.assert_close(got, ref, atol=1e-2, rtol=1e-2)
+        lo = O.hstu_jagged_forward(w.q, w.k, w.v, out_dtype=dtype, emulate_lowp=dtype, **w.oracle_kwargs()).float()
+        assert O.mismatch_fraction(got, lo, 5e-3) < 5e-3
+        helpers.set_switch(monkeypatch, "HSTU_MI355_SHORT", "0")
+        assert "_tiny" not in kernel_name(wd) and "_short" not in kernel_name(wd)
+        torch.testing.assert_close(run(wd).float().cpu(), got, atol=1e-2, rtol=1e-2)
+
+
+def test_tiny_sequences_gaps_and_rows_past_the_last_offset():
+    lengths = [7, 0, 0, 32, 0, 31, 1]
+    w = workloads.make("gaps", batch=len(lengths), heads=2, dim=256, lo=0, hi=0, lengths=lengths, dtype=torch.bfloat16,
+                       std=0.5, max_seq_len=32)  # fmt: skip
+    extra = 9
+    pad = lambda t: torch.cat([t, torch.full((extra, *t.shape[1:]), 3.0, dtype=t.dtype)])  # noqa: E731
+    wd = workloads.Workload(**{**w.__dict__})
+    wd.q, wd.k, wd.v = pad(w.q), pad(w.k), pad(w.v)
+    wd.seq_offset = torch.cat([w.seq_offset, w.seq_offset[-1:]])
+    wd = wd.to(DEV)
+    assert kernel_name(wd).endswith("_d256_tiny")
+    got = run(wd).float().cpu()
+    ref = O.hstu_jagged_forward(w.q, w.k, w.v, out_dtype=torch.float32, **w.oracle_kwargs())
+    torch.testing.assert_close(got[: ref.shape[0]], ref, atol=1e-2, rtol=1e-2)
+    assert (got[ref.shape[0] :] == 0).all()
+    # one more key than the kernel takes: the other kernels
+    w33 = workloads.make("n", batch=4, heads=2, dim=256, lo=1, hi=33, dtype=torch.bfloat16, max_seq_len=33, device=DEV)
+    assert "_tiny" not in kernel_name(w33)
+
+
 def test_attn_bias_rows_that_are_not_8_byte_pieces_stay_on_the_persistent_kernel(monkeypatch):
     helpers.set_switch(monkeypatch, "HSTU_MI355_SHORT", "1")
     w = workloads.make("bias", dtype=torch.bfloat16, std=0.5, rab_std=0.5, batch=3, heads=2, dim=128, lo=1, hi=90, max_seq_len=90)
