@@ -97,6 +97,13 @@ struct BwdArgs {
     // the rows of a sequence's 32-row group G hold the blocks 0 .. G only
     int64_t plane_head_lines;
     int plane_tri;
+    // Head dims above 256 (hstu_bwd_kernel.hip.h, windows): the kernels of the slot 256 run on halves of the heads.
+    // win = 2: q / k / v / grad and the gradients are taken as 2 x heads of half the head dims (n_heads_q, n_heads_k, d_qk
+    // and d_v say so), head 2 h + w being window w of head h; planes and the attn_bias tensors are indexed by the real head.
+    // win_only >= 0: the launch covers that window only (its grid counts real heads).  Otherwise win = 1, win_only = -1.
+    int win;
+    int win_only;
+    float* partial;  // S and dP summed over the first window, fp32, for the launch that adds the second (or null)
     int64_t drab_clear_bytes;  // > 0: the key-tile kernel clears this many bytes at drab beside its work
     const void* offs_q;
     const void* offs_k;

@@ -111,6 +111,25 @@ __device__ __forceinline__ uint32_t pair_row_offset(const BwdArgs& a, int r)
     return (a.plane_tri ? 16u * g * (g + 1u) + (static_cast<uint32_t>(r) & 31u) * (g + 1u) : static_cast<uint32_t>(r) * n_blk) * 128u;
 }
 
+// Windows (head dims above 256 on the kernels of the slot 256): the real head of head h of a launch, its K/V head, and
+// the [max_q][max_k] plane of an attn_bias-shaped tensor for sequence b and head h, in elements
+__device__ __forceinline__ int real_head(const BwdArgs& a, int h) { return a.win == 2 ? h >> 1 : h; }
+__device__ __forceinline__ int kv_head_of(const BwdArgs& a, int h)
+{
+    return a.win == 2 ? ((h >> 1) / a.head_ratio) * 2 + (h & 1) : h / a.head_ratio;
+}
+__device__ __forceinline__ int64_t bias_plane_of(const BwdArgs& a, int b, int h)
+{
+    return (static_cast<int64_t>(b) * (a.n_heads_q / a.win) + real_head(a, h)) * a.max_q * static_cast<int64_t>(a.max_k);
+}
+// S and dP of the first window (PHASE 1 of the query-tile kernel writes, PHASE 2 reads): per real head, global query row,
+// 32-key block and half-wave the 16 + 16 fp32 accumulator values of the lane, 128 bytes
+__device__ __forceinline__ float* partial_of(const BwdArgs& a, int h, int64_t row, int x, int lh)
+{
+    const int64_t n_blk = (a.max_k + 31) / 32;
+    return a.partial + (((static_cast<int64_t>(real_head(a, h)) * a.total_q + row) * n_blk + x) * 2 + lh) * 32;
+}
+
 // rows past the last offset belong to no sequence: zero-fill them (all workgroups of a launch share the job)
 __device__ __forceinline__ void zero_tail_rows(void* out, const void* offs, int n_batch, int idx64, int64_t total,
                                                int64_t row_elems, int threads)
@@ -265,9 +284,16 @@ __device__ __forceinline__ void store_tile_rows(uint16_t* stage, const f32x16_t 
 // ---------------------------------------------------------------------------------------------------------
 // STORE: 0 = dQ only; 1 = dS stored as well (it is the attn_bias gradient; or into a workspace, for dK workgroups that
 // read it back); 2 = dS and P stored (P for dV workgroups that read it back: no product is then computed twice)
-template <typename Tag, int D, bool HAS_RAB, bool HAS_MASK, int STORE>
+// PHASE (head dims above 256, two windows per head): 0 = everything in one launch.  1 = first window: S and dP of the
+// window go to a.partial in fp32, nothing else is written.  2 = second window: S and dP start from a.partial, then as
+// PHASE 0 (the dQ written is that of this window).  3 = dQ of the first window from the dS that PHASE 2 stored in the pair
+// plane: no scores are computed.
+template <typename Tag, int D, bool HAS_RAB, bool HAS_MASK, int STORE, int PHASE = 0>
 __global__ __launch_bounds__(256, bwd_dq_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hstu_bwd_dq_kernel(const BwdArgs a)
 {
+    static_assert(PHASE == 0 || D == 256, "windows run on the kernels of the slot 256");
+    static_assert(PHASE != 1 || STORE == 0, "the first window stores its partial scores only");
+    static_assert(PHASE != 3 || STORE == 0, "dQ from the plane stores dQ only");
     constexpr bool WANT_DRAB = STORE >= 1;
     constexpr bool WANT_P = STORE == 2;
     typedef SubTile<D> T;
@@ -301,14 +327,18 @@ __global__ __launch_bounds__(256, bwd_dq_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void 
             clear_share(a.drab, a.drab_clear_bytes, blockIdx.x, gridDim.x, threadIdx.x, 256);
         }
     }
-    const int per_level = a.n_batch * a.n_heads_q;
+    const int grid_heads = a.win_only >= 0 ? a.n_heads_q / a.win : a.n_heads_q;
+    const int per_level = a.n_batch * grid_heads;
     const int lvl = static_cast<int>(blockIdx.x) / per_level;
     const int rem = static_cast<int>(blockIdx.x) - lvl * per_level;
     const int qt = a.n_qtiles - 1 - lvl;
-    const int b = rem / a.n_heads_q;
-    const int h = rem - b * a.n_heads_q;
-    const int hk = h / a.head_ratio;
-    zero_tail_rows(a.dq, a.offs_q, a.n_batch, a.idx64, a.total_q, static_cast<int64_t>(a.n_heads_q) * a.d_qk, 256);
+    const int b = rem / grid_heads;
+    const int h_grid = rem - b * grid_heads;
+    const int h = a.win_only >= 0 ? h_grid * a.win + a.win_only : h_grid;
+    const int hk = kv_head_of(a, h);
+    if constexpr (PHASE != 1) {
+        zero_tail_rows(a.dq, a.offs_q, a.n_batch, a.idx64, a.total_q, static_cast<int64_t>(a.n_heads_q) * a.d_qk, 256);
+    }
     const SeqInfo sq_info = load_seq(a, b);
     const int sq = sq_info.sq, sk = sq_info.sk;
     const int r0 = qt * kBlockM;
@@ -398,7 +428,7 @@ __global__ __launch_bounds__(256, bwd_dq_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void 
     const int nx_w = (wb.lim_max + 31) / 32;
 
     const uint32_t bias_bytes = static_cast<uint32_t>(a.max_q) * static_cast<uint32_t>(a.max_k) * 2u;
-    const int64_t bias_plane = (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k);
+    const int64_t bias_plane = bias_plane_of(a, b, h);
     const __amdgpu_buffer_rsrc_t rab_rsrc =
         make_rsrc(HAS_RAB ? static_cast<const uint16_t*>(a.rab) + bias_plane : nullptr, HAS_RAB ? bias_bytes : 0u);
     const __amdgpu_buffer_rsrc_t mask_rsrc =
@@ -408,8 +438,9 @@ __global__ __launch_bounds__(256, bwd_dq_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void 
     // dS and P together (STORE 2) go to the pair plane: one whole 128-byte line per row and step, where two planes of the
     // bias layout would each get half a line
     const __amdgpu_buffer_rsrc_t p_rsrc =
-        make_rsrc(WANT_P ? pair_plane_of(a, sq_info.q0, b, h) : nullptr, WANT_P ? pair_seq_bytes(a, sq) : 0u);
-    const uint32_t pair_row_off = (WANT_P && wr0 + ln < sq) ? pair_row_offset(a, wr0 + ln) : kOutOfRange;
+        make_rsrc((WANT_P || PHASE == 3) ? pair_plane_of(a, sq_info.q0, b, real_head(a, h)) : nullptr,
+                  (WANT_P || PHASE == 3) ? pair_seq_bytes(a, sq) : 0u);
+    const uint32_t pair_row_off = ((WANT_P || PHASE == 3) && wr0 + ln < sq) ? pair_row_offset(a, wr0 + ln) : kOutOfRange;
     // rows past the sequence lie inside the plane but must stay untouched / unread: their offset leaves it
     const uint32_t bias_row_off =
         (wr0 + ln < sq) ? static_cast<uint32_t>(wr0 + ln) * static_cast<uint32_t>(a.max_k) * 2u : kOutOfRange;
@@ -486,12 +517,51 @@ __global__ __launch_bounds__(256, bwd_dq_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void 
         // them then only waits for requests of earlier steps, not for the ones made now
         const int c0 = x * 32;
         uint32_t rw[8], mw[8];
+        f32x16_t s, dp;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            s[i] = 0.f;
+            dp[i] = 0.f;
+        }
+        uint32_t pk[8];
+        uint32_t pp[8];  // P, when it is stored
         if (x < nx_w) {
-            if constexpr (HAS_RAB) {
+            if constexpr (HAS_RAB && PHASE != 1 && PHASE != 3) {
                 load_words(rab_rsrc, c0, rw);
             }
-            if constexpr (HAS_MASK) {
+            if constexpr (HAS_MASK && PHASE != 1 && PHASE != 3) {
                 load_words(mask_rsrc, c0, mw);
+            }
+            if constexpr (PHASE == 2) {
+                // the sums over the first window: where the accumulators start
+                if (wr0 + ln < sq) {
+                    const float4* const from = reinterpret_cast<const float4*>(partial_of(a, h, sq_info.q0 + wr0 + ln, x, lh));
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float4 t = from[i], u = from[4 + i];
+                        s[4 * i + 0] = t.x, s[4 * i + 1] = t.y, s[4 * i + 2] = t.z, s[4 * i + 3] = t.w;
+                        dp[4 * i + 0] = u.x, dp[4 * i + 1] = u.y, dp[4 * i + 2] = u.z, dp[4 * i + 3] = u.w;
+                    }
+                }
+            }
+            if constexpr (PHASE == 3) {
+                // dS of this step as PHASE 2 stored it: the lane pair of a row holds 16-byte pieces (keys 16 h2 + 8 lh .. + 7)
+                // and trades halves back into accumulator order (the swap is its own inverse); pieces that start past the
+                // last key were not written and read as zeros
+                typedef __attribute__((ext_vector_type(2))) unsigned u2_t;
+#pragma unroll
+                for (int h2 = 0; h2 < 2; ++h2) {
+                    const int key = c0 + 16 * h2 + 8 * lh;
+                    const uint32_t off = pair_row_off + static_cast<uint32_t>(2 * c0 + 16 * h2 + 8 * lh) * 2u;
+                    const U32Quad wd = __builtin_bit_cast(
+                        U32Quad, __builtin_amdgcn_raw_buffer_load_b128(p_rsrc, static_cast<int>(key < sk ? off : kOutOfRange), 0, 0));
+                    const u2_t d0 = __builtin_amdgcn_permlane32_swap(wd.v[0], wd.v[2], false, false);
+                    const u2_t d1 = __builtin_amdgcn_permlane32_swap(wd.v[1], wd.v[3], false, false);
+                    pk[4 * h2 + 0] = d0[0];
+                    pk[4 * h2 + 2] = d0[1];
+                    pk[4 * h2 + 1] = d1[0];
+                    pk[4 * h2 + 3] = d1[1];
+                }
             }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -500,19 +570,25 @@ __global__ __launch_bounds__(256, bwd_dq_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void 
         if (x >= nx_w) {
             return;  // nothing of this sub-tile is visible to the rows of this wavefront
         }
-        f32x16_t s, dp;
+        if constexpr (PHASE != 3) {
 #pragma unroll
-        for (int i = 0; i < 16; ++i) {
-            s[i] = 0.f;
-            dp[i] = 0.f;
+            for (int js = 0; js < KSTEPS; ++js) {
+                s = mfma32<Tag>(read_n(kn, js), qf[js], s);
+                dp = mfma32<Tag>(read_n(vn, js), gf[js], dp);
+            }
         }
+        if constexpr (PHASE == 1) {
+            if (wr0 + ln < sq) {
+                float4* const to = reinterpret_cast<float4*>(partial_of(a, h, sq_info.q0 + wr0 + ln, x, lh));
 #pragma unroll
-        for (int js = 0; js < KSTEPS; ++js) {
-            s = mfma32<Tag>(read_n(kn, js), qf[js], s);
-            dp = mfma32<Tag>(read_n(vn, js), gf[js], dp);
+                for (int i = 0; i < 4; ++i) {
+                    to[i] = make_float4(s[4 * i + 0], s[4 * i + 1], s[4 * i + 2], s[4 * i + 3]);
+                    to[4 + i] = make_float4(dp[4 * i + 0], dp[4 * i + 1], dp[4 * i + 2], dp[4 * i + 3]);
+                }
+            }
+            return;
         }
-        uint32_t pk[8];
-        uint32_t pp[8];  // P, when it is stored
+        if constexpr (PHASE != 3) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             float ds2[2], p2[2];
@@ -559,6 +635,7 @@ __global__ __launch_bounds__(256, bwd_dq_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void 
                 }
             }
         }
+        }  // PHASE != 3
         if constexpr (WANT_P) {
             // the two lanes of a row trade halves (see below), then four 16-byte pieces per lane pair: dS, dS, P, P
             typedef __attribute__((ext_vector_type(2))) unsigned u2_t;
@@ -639,6 +716,9 @@ __global__ __launch_bounds__(256, bwd_dq_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void 
         }
     }
 
+    if constexpr (PHASE == 1) {
+        return;
+    }
     // store dQ: lane holds query row (wr0 + ln), dims 32*mt + 8*g + 4*lh + 0..3
     if (a.grad_vec_ok != 0) {
         // (every wavefront is done with the ring before anybody writes its rows into a stage)
@@ -838,8 +918,10 @@ __global__ __launch_bounds__(kDkvThreads, (MODE == 2 || MODE >= 4) ? bwd_dk_from
     }
 
     // head and sub-tile of iteration it, kept incrementally (no division in the loop)
-    int req_h = hk * a.head_ratio, req_x = x_first, req_it = 0;  // next request
-    int cur_h = hk * a.head_ratio, cur_x = x_first;              // current step
+    // (windows: K/V head hk is window hk % win of the real K/V head hk / win; its query heads follow win apart)
+    const int first_h = (hk / a.win) * a.head_ratio * a.win + (hk % a.win);
+    int req_h = first_h, req_x = x_first, req_it = 0;  // next request
+    int cur_h = first_h, cur_x = x_first;              // current step
     auto request = [&](uint16_t* stage) {
         const bool past = req_it >= n_iter;  // (sent out of range: moves no data, keeps the count per step constant)
         const __amdgpu_buffer_rsrc_t q_rsrc =
@@ -867,7 +949,7 @@ __global__ __launch_bounds__(kDkvThreads, (MODE == 2 || MODE >= 4) ? bwd_dk_from
         if (++req_x >= n_qsub) {
             req_x = x_first;
             if (!past && req_it < n_iter) {
-                ++req_h;
+                req_h += a.win;
             }
         }
     };
@@ -910,8 +992,8 @@ __global__ __launch_bounds__(kDkvThreads, (MODE == 2 || MODE >= 4) ? bwd_dk_from
         // dS values followed by 32 P values)
         const uint32_t pitch = static_cast<uint32_t>(a.max_k);
         const __amdgpu_buffer_rsrc_t ds_rsrc =
-            MODE >= 4 ? make_rsrc(pair_plane_of(a, si.q0, b, h), pair_seq_bytes(a, sq))
-                      : make_rsrc(static_cast<const uint16_t*>(a.drab) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(pitch),
+            MODE >= 4 ? make_rsrc(pair_plane_of(a, si.q0, b, real_head(a, h)), pair_seq_bytes(a, sq))
+                      : make_rsrc(static_cast<const uint16_t*>(a.drab) + bias_plane_of(a, b, h),
                                   static_cast<uint32_t>(a.max_q) * pitch * 2u);
         const uint32_t row_off = MODE >= 4 ? pair_row_offset(a, rq0 + ln) : static_cast<uint32_t>(rq0 + ln) * pitch * 2u;
 #pragma unroll
@@ -933,14 +1015,14 @@ __global__ __launch_bounds__(kDkvThreads, (MODE == 2 || MODE >= 4) ? bwd_dk_from
         const int rq0 = cur_x * 32;  // first query row of the sub-tile
         if (++cur_x >= n_qsub) {
             cur_x = x_first;
-            ++cur_h;
+            cur_h += a.win;
         }
         const bool active = block_active(rq0);
         const __amdgpu_buffer_rsrc_t rab_rsrc = make_rsrc(
-            HAS_RAB ? static_cast<const uint16_t*>(a.rab) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k) : nullptr,
+            HAS_RAB ? static_cast<const uint16_t*>(a.rab) + bias_plane_of(a, b, h) : nullptr,
             HAS_RAB ? bias_bytes : 0u);
         const __amdgpu_buffer_rsrc_t mask_rsrc = make_rsrc(
-            HAS_MASK ? static_cast<const uint16_t*>(a.mask) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k) : nullptr,
+            HAS_MASK ? static_cast<const uint16_t*>(a.mask) + bias_plane_of(a, b, h) : nullptr,
             HAS_MASK ? bias_bytes : 0u);
         // rab / mask rows of this step (16-byte path): lane (ln, lh) has row rq0 + ln, keys cw0 + 16 j + 8 lh .. + 7
         // (whole chunks are in or out of the row: max_seq_len_k is a multiple of 8 here)
@@ -977,7 +1059,7 @@ __global__ __launch_bounds__(kDkvThreads, (MODE == 2 || MODE >= 4) ? bwd_dk_from
             // step's loads, so that no load waits for them
             if (dk_role) {
                 const __amdgpu_buffer_rsrc_t drab_rsrc = make_rsrc(
-                    static_cast<uint16_t*>(a.drab) + (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k),
+                    static_cast<uint16_t*>(a.drab) + bias_plane_of(a, b, h),
                     bias_bytes);
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {

@@ -859,6 +859,51 @@ static int64_t dq_short_grid(const hstu::BwdArgs& a)
     return ((a.max_q + hstu::kDqShortRows - 1) / hstu::kDqShortRows) * pairs_pad * a.head_ratio;
 }
 
+// Head dims above 256 on the matrix pipe: 16-bit inputs whose head dims are multiples of 16 run as two windows per head
+// on the kernels of the slot 256 (heads taken as 2 x heads of half the dims): the query-tile kernel over the first window
+// (S and dP in fp32 to a partial plane), over the second (adds them up: dS and P to the pair plane, dQ of the second
+// window), once more for dQ of the first window from the stored dS, then the dV-from-P / dK-from-dS workgroups of all
+// windows.  Needs its workspace (partial plane: 256 bytes per query row, 32-key block and head; pair plane as in the planes
+// order): a call without it, or one whose planes pass the limit, runs on the generic kernels.  B8 H4 d512 L100..1024:
+// 37 ms on the generic kernels.  HSTU_MI355_GENERIC_BACKWARD=1 keeps the generic kernels.
+struct WindowPlan {
+    const BwdVariant* var;  // nullptr: not this path
+    PairPlane pair;
+    uint64_t partial_bytes;
+    uint64_t workspace_bytes;
+};
+static WindowPlan plan_windows(const hstu_jagged_bwd_params* p)
+{
+    WindowPlan w;
+    memset(&w, 0, sizeof(w));
+    const hstu_jagged_fwd_params* f = &p->fwd;
+    const int64_t dmax = f->head_dim_qk > f->head_dim_v ? f->head_dim_qk : f->head_dim_v;
+    if ((f->dtype != HSTU_DT_BF16 && f->dtype != HSTU_DT_FP16) || dmax <= 256 || dmax > 512 || f->head_dim_qk % 16 != 0 ||
+        f->head_dim_v % 16 != 0 || switches().generic_backward == 1 || f->total_q == 0 || f->total_k == 0 ||
+        f->max_seq_len_k % 8 != 0) {
+        return w;
+    }
+    // (16-byte rows of the planes and of the attn_bias tensors, spans behind 32-bit descriptors)
+    const uintptr_t ptrs = reinterpret_cast<uintptr_t>(f->attn_bias) | reinterpret_cast<uintptr_t>(f->mask) |
+                           reinterpret_cast<uintptr_t>(p->grad_attn_bias);
+    const int64_t span_q = f->max_seq_len_q * f->num_heads_q * dmax * 2;
+    const int64_t span_k = f->max_seq_len_k * f->num_heads_k * dmax * 2;
+    const int64_t span_b = f->max_seq_len_q * f->max_seq_len_k * 2;
+    if (ptrs % 16 != 0 || span_q >= (1LL << 30) || span_k >= (1LL << 30) || span_b >= (1LL << 31)) {
+        return w;
+    }
+    w.pair = pair_plane(f);
+    const int64_t n_blk = (f->max_seq_len_k + 31) / 32;
+    w.partial_bytes = static_cast<uint64_t>(f->num_heads_q * f->total_q * n_blk * 256);
+    w.workspace_bytes = static_cast<uint64_t>(w.pair.bytes) + w.partial_bytes;
+    if (!w.pair.fits_32 || w.workspace_bytes > static_cast<uint64_t>(workspace_cap_mb()) * (1ULL << 20)) {
+        return w;
+    }
+    const auto* table = f->dtype == HSTU_DT_BF16 ? hstu::bwd_variants_bf16() : hstu::bwd_variants_f16();
+    w.var = &table[f->attn_bias != nullptr ? 1 : 0][f->mask_type == HSTU_MASK_CUSTOM ? 1 : 0][2];
+    return w;
+}
+
 HSTU_API int hstu_jagged_bwd_workspace_size(const hstu_jagged_bwd_params* params, uint64_t* workspace_bytes)
 {
     if (workspace_bytes == nullptr) {
@@ -873,7 +918,8 @@ HSTU_API int hstu_jagged_bwd_workspace_size(const hstu_jagged_bwd_params* params
     if (var == nullptr) {
         return HSTU_ERR_UNSUPPORTED;
     }
-    *workspace_bytes = plan_bwd(params, var).workspace_bytes;
+    const WindowPlan windows = plan_windows(params);
+    *workspace_bytes = windows.var != nullptr ? windows.workspace_bytes : plan_bwd(params, var).workspace_bytes;
     return HSTU_OK;
 }
 
@@ -902,6 +948,8 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
     }
     hstu::BwdArgs a;
     memset(&a, 0, sizeof(a));
+    a.win = 1;
+    a.win_only = -1;
     a.q = f->q;
     a.k = f->k;
     a.v = f->v;
@@ -952,6 +1000,44 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
     a.alpha = static_cast<float>(f->alpha);
     a.scale = static_cast<float>((f->silu_scale == 0.0) ? 1.0 / static_cast<double>(f->max_seq_len_q) : f->silu_scale);
 
+    const WindowPlan windows = plan_windows(p);
+    if (windows.var != nullptr && usable_workspace(workspace, workspace_bytes, windows.workspace_bytes) &&
+        reinterpret_cast<uintptr_t>(workspace) % 16 == 0 && a.grad_vec_ok != 0) {
+        const BwdVariant* const wv = windows.var;
+        hstu::BwdArgs w = a;
+        w.win = 2;
+        w.d_qk = a.d_qk / 2;
+        w.d_v = a.d_v / 2;
+        w.n_heads_q = 2 * a.n_heads_q;
+        w.n_heads_k = 2 * a.n_heads_k;
+        w.bias_vec_ok = 2;
+        w.p_plane = workspace;
+        w.plane_head_lines = windows.pair.head_lines;
+        w.plane_tri = windows.pair.tri ? 1 : 0;
+        w.partial = reinterpret_cast<float*>(static_cast<uint8_t*>(workspace) + windows.pair.bytes);
+        const int64_t grid_q = static_cast<int64_t>(a.n_qtiles) * a.n_batch * a.n_heads_q;  // (real heads: one window per launch)
+        const int64_t kv_slots = static_cast<int64_t>(a.n_ktiles) * a.n_batch * w.n_heads_k;
+        const int64_t grid_kv = 16 * ((kv_slots + 7) / 8);
+        if (grid_kv > 0x7fffffffLL || grid_q > 0x7fffffffLL) {
+            return fail(HSTU_ERR_INVALID, "grid out of range");
+        }
+        w.win_only = 0;
+        hipLaunchKernelGGL(wv->dq_win_first, dim3(static_cast<unsigned>(grid_q)), dim3(256), 0, static_cast<hipStream_t>(stream), w);
+        w.win_only = 1;
+        w.drab_clear_bytes = drab_bytes;
+        hipLaunchKernelGGL(wv->dq_win_second_ds_p, dim3(static_cast<unsigned>(grid_q)), dim3(256), 0, static_cast<hipStream_t>(stream), w);
+        w.drab_clear_bytes = 0;
+        w.win_only = 0;
+        hipLaunchKernelGGL(wv->dq_win_from_plane, dim3(static_cast<unsigned>(grid_q)), dim3(256), 0, static_cast<hipStream_t>(stream), w);
+        w.win_only = -1;
+        hipLaunchKernelGGL(p->grad_attn_bias != nullptr ? wv->dv_dk_from_planes_drab : wv->dv_dk_from_planes,
+                           dim3(static_cast<unsigned>(grid_kv)), dim3(hstu::kDkvThreads), 0, static_cast<hipStream_t>(stream), w);
+        const hipError_t err_w = hipGetLastError();
+        if (err_w != hipSuccess) {
+            return fail(HSTU_ERR_RUNTIME, "launch of %s (two windows) failed: %s", wv->name, hipGetErrorString(err_w));
+        }
+        return HSTU_OK;
+    }
     const bool generic = is_generic_bwd(var);
     const BwdPlan plan = plan_bwd(p, var);
     // the tuned key-tile kernel runs a dV and a dK workgroup per tile, the generic one a workgroup per tile

@@ -49,6 +49,12 @@ struct BwdVariant {
     void (*dq_ds_p)(const BwdArgs);
     void (*dv_dk_from_planes)(const BwdArgs);
     void (*dv_dk_from_planes_drab)(const BwdArgs);  // the dK workgroups also write dS to the attn_bias gradient
+    // head dims above 256 as two windows per head on the kernels of the slot 256 (nullptr elsewhere): the query-tile kernel
+    // over the first window (S and dP to the fp32 partial plane), over the second (dS and P to the pair plane, dQ of that
+    // window), and dQ of the first window from the stored dS
+    void (*dq_win_first)(const BwdArgs);
+    void (*dq_win_second_ds_p)(const BwdArgs);
+    void (*dq_win_from_plane)(const BwdArgs);
 };
 
 // forward, 16-bit inputs: [rab: 0, 1][custom mask: 0, 1][dim slot: 32, 64, 128, 256]

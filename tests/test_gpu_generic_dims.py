@@ -187,3 +187,78 @@ def test_backward_runs_on_the_generic_kernels_for_these_dims():
     O.hstu_jagged_forward(qc, kc, vc, out_dtype=torch.float32, **c.oracle_kwargs()).sum().backward()
     for g, r in ((q.grad, qc.grad), (k.grad, kc.grad), (v.grad, vc.grad)):
         torch.testing.assert_close(g.float().cpu(), r, rtol=2e-2, atol=2e-2 * float(r.abs().max()))
+
+
+WINDOW_CASES = {
+    "plain_512": dict(batch=3, heads=2, dim=512, lo=1, hi=328, max_seq_len=328),
+    "dims_384_320": dict(batch=3, heads=2, dim=384, dim_v=320, lo=40, hi=200, max_seq_len=200),
+    "dims_64_512": dict(batch=2, heads=2, dim=64, dim_v=512, lo=1, hi=130, max_seq_len=136),
+    "dims_512_16": dict(batch=2, heads=2, dim=512, dim_v=16, lo=1, hi=130, max_seq_len=136),
+    "dims_272": dict(batch=2, heads=3, dim=272, lo=100, hi=300, max_seq_len=304),
+    "bias_and_its_gradient": dict(batch=3, heads=2, dim=512, lo=30, hi=264, max_seq_len=264, rab_std=0.5),
+    "context_targets_groups_bias": dict(batch=3, heads=2, dim=320, dim_v=384, lo=60, hi=264, max_seq_len=264, rab_std=0.5,
+                                        num_context=5, max_target=33, target_group_size=3),
+    "grouped_heads": dict(batch=3, heads=4, heads_k=2, dim=512, lo=1, hi=200, max_seq_len=200),
+    "one_kv_head_bias": dict(batch=2, heads=6, heads_k=1, dim=288, dim_v=512, lo=90, hi=160, max_seq_len=160, rab_std=0.5),
+    "int64_offsets": dict(batch=2, heads=2, dim=512, lo=33, hi=160, max_seq_len=160, index_dtype=torch.int64),
+}
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16], ids=["bf16", "f16"])
+@pytest.mark.parametrize("mask", ["builtin", "custom", "none"])
+@pytest.mark.parametrize("name", list(WINDOW_CASES))
+def test_backward_above_head_dim_256_as_two_windows(name, mask, dtype, monkeypatch):
+    """16-bit inputs with head dims in (256, 512] that are multiples of 16, rows of 16 bytes in the planes
+    (max_seq_len_k a multiple of 8): the kernels of the head-dim slot 256 over two windows per head, with the workspace
+    the library asks for -- the pair plane of the planes order plus 256 bytes per (query row, 32-key block, head) of
+    fp32 partial scores -- full of NaN.  Without the workspace, and with HSTU_MI355_GENERIC_BACKWARD=1, the generic
+    kernels take the call."""
+    from ops_rec import _ops, workloads
+
+    kw = dict(WINDOW_CASES[name])
+    if mask != "builtin" and "num_context" in kw:
+        pytest.skip("context and target rows belong to the built-in mask")
+    w = workloads.make("win", dtype=dtype, std=0.4, seed=len(name), **kw)
+    if mask == "custom":
+        g = torch.Generator().manual_seed(4)
+        shape = (len(w.lengths), w.q.shape[1], w.max_seq_len, w.max_seq_len)
+        w = dataclasses.replace(w, mask=(torch.rand(shape, generator=g) < 0.7).to(dtype), mask_type=3)
+    elif mask == "none":
+        w = dataclasses.replace(w, mask_type=2)
+    asked = []
+    plain = _ops._new_workspace
+
+    def poisoned(n_bytes, device):
+        asked.append(n_bytes)
+        ws = plain(n_bytes, device)
+        if ws is not None:
+            ws.fill_(0xFF)
+        return ws
+
+    monkeypatch.setattr(_ops, "_new_workspace", poisoned)
+    helpers.set_switch(monkeypatch, "HSTU_MI355_GENERIC_BACKWARD", None)
+    check_backward(w)
+    rows, heads, blocks = w.q.shape[0], w.q.shape[1], (w.max_seq_len + 31) // 32
+    partial = heads * rows * blocks * 256
+    assert asked and asked[-1] > partial and (asked[-1] - partial) % (128 * heads) == 0, (asked, partial)
+    # the generic kernels on the same inputs: no workspace
+    helpers.set_switch(monkeypatch, "HSTU_MI355_GENERIC_BACKWARD", "1")
+    check_backward(w)
+    assert asked[-1] == 0
+    helpers.set_switch(monkeypatch, "HSTU_MI355_GENERIC_BACKWARD", None)
+    helpers.withhold_workspace(monkeypatch)
+    check_backward(w)
+
+
+def test_backward_windows_do_not_take_rows_that_are_not_16_byte_pieces(monkeypatch):
+    from ops_rec import _ops, workloads
+
+    asked = []
+    plain = _ops._new_workspace
+    monkeypatch.setattr(_ops, "_new_workspace", lambda n, dev: (asked.append(n), plain(n, dev))[1])
+    w = workloads.make("win", dtype=torch.bfloat16, std=0.4, batch=2, heads=2, dim=512, lo=1, hi=90, max_seq_len=90)
+    check_backward(w)
+    assert asked[-1] == 0
+    w = workloads.make("win", dtype=torch.bfloat16, std=0.4, batch=2, heads=2, dim=264, dim_v=272, lo=1, hi=88, max_seq_len=88)
+    check_backward(w)  # a head dim that is not a multiple of 16
+    assert asked[-1] == 0
