@@ -132,6 +132,7 @@ def bench_ln_mul(attn_out, stream, args):
         p.epsilon = ln_mul_oracle.EPSILON
         raw = ctypes.c_void_p(stream.cuda_stream)
         n = max(50, args.steps)
+        settle(lambda: lib.ln_mul_fwd(ctypes.byref(p), raw), args.settle_ms)
         for _ in range(10):
             assert lib.ln_mul_fwd(ctypes.byref(p), raw) == 0, _native.last_error()
         torch.cuda.synchronize()
@@ -171,6 +172,20 @@ def bench_ln_mul(attn_out, stream, args):
             "cases": cases}  # fmt: skip
 
 
+def settle(launch, ms):
+    """Keeps the device busy with `launch` for about `ms` milliseconds (untimed), so that what is timed next starts with
+    the clocks where sustained work holds them."""
+    import torch
+
+    if ms <= 0:
+        return
+    t0 = time.perf_counter()
+    while (time.perf_counter() - t0) * 1e3 < ms:
+        for _ in range(32):
+            launch()
+        torch.cuda.synchronize()
+
+
 def bench_in_linear_silu(tokens, width, stream, args):
     """in_linear_silu through ``in_linear_silu_fwd`` of the C ABI, events on the launch stream.  Algorithmic bytes per
     launch: x, weight and bias read once, linear_output and the four splits written once =
@@ -204,6 +219,7 @@ def bench_in_linear_silu(tokens, width, stream, args):
         # (at least 100 launches behind 20 untimed ones: the layer shape is bound by the core clock, which takes a few
         # milliseconds of work to settle after the host-side gaps between the legs -- 25 launches show 86-90 us, 100 show 70-72)
         n_it = max(100, args.steps // 2)
+        settle(lambda: lib.in_linear_silu_fwd(ctypes.byref(p), raw), args.settle_ms)
         for _ in range(20):
             assert lib.in_linear_silu_fwd(ctypes.byref(p), raw) == 0, _native.last_error()
         torch.cuda.synchronize()
@@ -263,6 +279,8 @@ def main() -> int:
     ap.add_argument("--forward-only", action="store_true",
                     help="time the attention forward only; by default (none of --backward / --ln-mul / --in-linear-silu "
                     "given) the line also carries the 'backward', 'ln_mul' and 'in_linear_silu' objects")
+    ap.add_argument("--settle-ms", type=float, default=30.0,
+                    help="milliseconds of untimed launches ahead of each leg's warm-up launches (0: none)")
     ap.add_argument("--no-cold", action="store_true",
                     help="skip the cold-cache loop (profiler runs: every traced launch is then one of the timed loop's)")
     ap.add_argument("--drop-rab", action="store_true",
@@ -323,6 +341,9 @@ def main() -> int:
     raw_stream = stream.cuda_stream
 
     # ---- GPU: K launches through the C ABI, events on the launch stream ----
+    # (ahead of the W warm-up launches the device is kept busy for --settle-ms: the first millisecond or two of work
+    # after an idle period runs 4-5 % slower than the launches behind it, and K = 20 launches last under a millisecond)
+    settle(lambda: prepared.launch(raw_stream), args.settle_ms)
     for _ in range(args.warmup):
         prepared.launch(raw_stream)
     torch.cuda.synchronize()
@@ -403,6 +424,7 @@ def main() -> int:
         "n_gpus": 1,
         "steps": args.steps,
         "warmup": args.warmup,
+        "settle_ms": args.settle_ms,
         "ms_per_step": round(ms_per_step, 6),
         "higher_is_better": True,
         "scaling": "weak",
@@ -467,6 +489,7 @@ def main() -> int:
                     w.target_group_size, w.alpha)  # fmt: skip
         bwd = ops_rec.ascendc.attention.hstu_jagged_backward
         n_bwd = max(50, args.steps // 4)
+        settle(lambda: bwd(*bwd_args), args.settle_ms)
         for _ in range(10):
             bwd(*bwd_args)
         torch.cuda.synchronize()

@@ -574,3 +574,22 @@ def test_forward_descriptions_are_cached_by_everything_but_the_addresses():
     _ops._PLAN_CACHE["x"] = None
     _native.reload_switches()
     assert not _ops._PLAN_CACHE
+
+
+def test_backward_workspace_that_cannot_be_allocated_is_left_out(monkeypatch):
+    """The backward's workspace is optional scratch: when the allocator has no room for it the adapter passes none
+    (the library then takes an order that needs none) instead of failing a call the reference's backward would serve."""
+    from ops_rec import _ops
+
+    calls = []
+
+    def no_room(*args, **kwargs):
+        calls.append(args)
+        raise torch.cuda.OutOfMemoryError("HIP out of memory (test)")
+
+    assert _ops._new_workspace(0, torch.device("cpu")) is None  # nothing asked for, nothing allocated
+    monkeypatch.setattr(_ops.torch, "empty", no_room)
+    assert _ops._new_workspace(1 << 20, torch.device("cpu")) is None and len(calls) == 1
+    monkeypatch.undo()
+    ws = _ops._new_workspace(4096, torch.device("cpu"))
+    assert ws is not None and ws.numel() == 4096 and ws.dtype == torch.uint8
