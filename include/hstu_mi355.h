@@ -170,22 +170,25 @@ HSTU_API uint64_t hstu_jagged_fwd_noalloc_max_workspace(void);
  *
  * `fwd` describes q, k, v, mask, attn_bias, the offsets and the scalars exactly as for the forward (fwd.out is
  * not used and may be NULL).  bf16 / fp16 with head dims up to 256 and a q/k head dim that is a multiple of 8 run
- * on the tuned kernels; fp32 with head dims up to 128 and a q/k head dim that is a multiple of 8 runs on kernels
- * built on the fp32 matrix instruction; every other input the forward takes runs on generic fp32-arithmetic
+ * on the tuned kernels, and so do head dims in (256, 512] that are multiples of 16 (as two windows per head; this
+ * needs the workspace, see below); fp32 with head dims up to 128 and a q/k head dim that is a multiple of 8 runs on
+ * kernels built on the fp32 matrix instruction; every other input the forward takes runs on generic fp32-arithmetic
  * kernels (correct, slow).  fp8 inputs return HSTU_ERR_UNSUPPORTED.
  * grad_q / grad_k / grad_v: every row is written (rows past the last offset are zero-filled), so the caller
  * need not clear them.  grad_attn_bias (optional; requires attn_bias): written in full as well -- zeros outside
  * the part of a sequence's [S_q, S_k] corner that its query tiles sweep -- so the caller need not clear it either
- * (the kernel that produces grad_v clears it beside its work).
+ * (the first kernel of the call clears it beside its work).
  * Workspace (optional): the tuned kernels recompute nothing, or less, when the query-tile kernel's dS (and P) have
  * somewhere to stay until the kernels that produce grad_k (and grad_v) read them back: dS in grad_attn_bias (which
  * is dS) when that is asked for, otherwise in a workspace of [batch, num_heads_q, max_seq_len_q, max_seq_len_k]
- * elements of the input type -- twice that (rounded up to whole 32-key blocks) for dS and P together --, which
- * hstu_jagged_bwd_workspace_size asks for where it was measured to pay (head dims above 64, max_seq_len_k a
- * multiple of 8, at most 2 GiB or HSTU_MI355_BWD_WORKSPACE_MB in the environment; at head dims above 128 also with
- * grad_attn_bias, for dS and P together; fp32 inputs with head dims up to 128: always, in fp32).  Without the
- * workspace, or with less than was asked for, the call still works: the kernels that produce grad_k then recompute
- * dS.  The workspace needs no clearing and holds nothing afterwards. */
+ * elements of the input type; dS and P together in a workspace of one 128-byte line per head, query row of the batch
+ * and 32-key block (only the blocks at or below the diagonal for a causal mask over equal query and key offsets
+ * without context rows).  hstu_jagged_bwd_workspace_size asks for the workspace of the order it estimates to be the
+ * fastest (max_seq_len_k a multiple of 8; at most 2 GiB, or HSTU_MI355_BWD_WORKSPACE_MB in the environment; fp32
+ * inputs with head dims up to 128: dS and P in fp32 whenever that fits).  Head dims above 256 need, beside that line
+ * per row and block, 256 bytes per head, query row and block for the scores of the first window.  Without the workspace,
+ * or with less than was asked for, the call still works: the kernels that produce grad_k then recompute dS (head dims
+ * above 256: the generic kernels run).  The workspace needs no clearing and holds nothing afterwards. */
 typedef struct hstu_jagged_bwd_params {
     uint32_t struct_size; /* sizeof(hstu_jagged_bwd_params) */
     uint32_t reserved0;
