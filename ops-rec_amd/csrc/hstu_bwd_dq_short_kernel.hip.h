@@ -182,10 +182,7 @@ __global__ __launch_bounds__(kDqShortThreads, kDqShortWavesPerSimd) void hstu_bw
         wave_bounds(a.mask_type, wr0, sq, sk, sq_info.n_ctx, sq_info.n_tgt, a.target_group, wr0 < sq, kShortWaveM);
     const int nx_w = (wb.lim_max + 31) / 32;
     // the blocks the 32-row group of this wavefront's rows can see: what the readers of the plane take as written
-    const int wr0_32 = wr0 & ~31;
-    const WaveBounds wb32 =
-        wave_bounds(a.mask_type, wr0_32, sq, sk, sq_info.n_ctx, sq_info.n_tgt, a.target_group, wr0_32 < sq, kWaveM);
-    const int nx_store = (wb32.lim_max + 31) / 32;
+    const int nx_store = (swept_key_limit(a, sq_info, wr0 & ~31) + 31) / 32;
     const int lim_lane = lim - 4 * g;
     const int hole_lo_lane = hole_lo - 4 * g;
     const int hole_hi_lane = hole_hi - 4 * g;

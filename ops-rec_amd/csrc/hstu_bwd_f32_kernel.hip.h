@@ -201,7 +201,7 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_f32_dq_kernel(const BwdArgs a
         __syncthreads();
 
         const int c0 = kt * BN;
-        if (c0 < wb.lim_max) {
+        if (c0 < swept_key_limit(a, si, wr0)) {
             f32x16_t s, dp;
             if constexpr (HAS_RAB) {
                 f32_load_row_keys(rab_rsrc, bias_row_off, c0, lh, a.max_k, bias_vec, s);
@@ -446,14 +446,7 @@ __global__ __launch_bounds__(256, 1) void hstu_bwd_f32_dkv_kernel(const BwdArgs 
             __syncthreads();
 
             // whole block hidden from the keys of this wavefront?
-            bool active = cw0 < sk;
-            if (a.mask_type == 0) {
-                int lim_max = rq0 + 32 + si.delta;  // lim of the last row
-                if (rq0 < si.n_ctx) {
-                    lim_max = lim_max > si.hist_k ? lim_max : si.hist_k;
-                }
-                active = active && cw0 < lim_max;
-            }
+            const bool active = cw0 < swept_key_limit(a, si, rq0);
             float p[16], ds[16];
             if constexpr (PLANES) {
                 if (active) {

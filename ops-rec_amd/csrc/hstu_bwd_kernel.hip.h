@@ -130,6 +130,16 @@ __device__ __forceinline__ float* partial_of(const BwdArgs& a, int h, int64_t ro
     return a.partial + (((static_cast<int64_t>(real_head(a, h)) * a.total_q + row) * n_blk + x) * 2 + lh) * 32;
 }
 
+// The one statement of which 32-key blocks the query-tile kernels sweep for the 32 query rows from r0 on (r0 a multiple of
+// 32): those that start below this limit.  What such a kernel hands over through a workspace (dS, dS and P) it writes for
+// exactly these blocks, and the key-tile kernels read exactly these: both sides, 16-bit and fp32, take the limit from here,
+// so a workspace needs no clearing.  (The limit is that of the group's last row, or of its context rows; it never passes
+// the sequence's last key.  Rows and 16-byte pieces past the sequence are left out by both sides on top of it.)
+__device__ __forceinline__ int swept_key_limit(const BwdArgs& a, const SeqInfo& s, int r0)
+{
+    return wave_bounds(a.mask_type, r0, s.sq, s.sk, s.n_ctx, s.n_tgt, a.target_group, r0 < s.sq, kWaveM).lim_max;
+}
+
 // rows past the last offset belong to no sequence: zero-fill them (all workgroups of a launch share the job)
 __device__ __forceinline__ void zero_tail_rows(void* out, const void* offs, int n_batch, int idx64, int64_t total,
                                                int64_t row_elems, int threads)
@@ -425,7 +435,7 @@ __global__ __launch_bounds__(256, bwd_dq_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void 
     int lim, hole_lo, hole_hi;
     row_bounds(sq_info, a.mask_type, a.target_group, row, lim, hole_lo, hole_hi);
     const WaveBounds wb = wave_bounds(a.mask_type, wr0, sq, sk, sq_info.n_ctx, sq_info.n_tgt, a.target_group, wr0 < sq);
-    const int nx_w = (wb.lim_max + 31) / 32;
+    const int nx_w = (swept_key_limit(a, sq_info, wr0) + 31) / 32;  // (= wb.lim_max: a wavefront is a 32-row group here)
 
     const uint32_t bias_bytes = static_cast<uint32_t>(a.max_q) * static_cast<uint32_t>(a.max_k) * 2u;
     const int64_t bias_plane = bias_plane_of(a, b, h);
@@ -965,17 +975,7 @@ __global__ __launch_bounds__(kDkvThreads, (MODE == 2 || MODE >= 4) ? bwd_dk_from
     };
 
     // whole block hidden from the keys of this wavefront?  (rows rq0 .. rq0 + 31, keys cw0 .. cw0 + 31)
-    auto block_active = [&](int rq0) -> bool {
-        bool active = cw0 < sk;
-        if (a.mask_type == 0) {
-            int lim_max = rq0 + 32 + si.delta;  // lim of the last row
-            if (rq0 < si.n_ctx) {
-                lim_max = lim_max > si.hist_k ? lim_max : si.hist_k;
-            }
-            active = active && cw0 < lim_max;
-        }
-        return active;
-    };
+    auto block_active = [&](int rq0) -> bool { return cw0 < swept_key_limit(a, si, rq0); };
     // MODE 2 and 4: the dS (or P) rows of a step, as the query-tile kernel stored them (rounded to the input type, masked), are
     // read like rab rows -- lane (ln, lh) reads row rq0 + ln, keys cw0 + 16 j + 8 lh .. + 7 -- one step ahead of
     // their use, and transposed by the same routing products.  Only what that kernel wrote is read -- whole 16-byte

@@ -1413,7 +1413,8 @@ HSTU_API int hstu_jagged_fwd_noalloc(const hstu_jagged_fwd_params* p, void* stre
     if (rc_scratch != HSTU_OK) {
         return rc_scratch;
     }
-    return launch_forward(p, nullptr, ptr, kScratchBytes, stream);
+    // (the bytes hstu_jagged_fwd would be given for this description, so that both entry points split items alike)
+    return launch_forward(p, nullptr, ptr, need, stream);
 }
 
 }  // extern "C"

@@ -32,6 +32,8 @@ def noalloc(p):
     [
         # split items: counters and partial outputs in the scratch array; then a shorter sequence
         (dict(batch=2, heads=2, dim=128, lo=2800, hi=3000), dict(batch=1, heads=2, dim=128, lo=1500, hi=1500), "split"),
+        # the same at the head-dim slot 64 (three workgroups per CU resident: more parts than at 128)
+        (dict(batch=2, heads=2, dim=64, lo=2800, hi=3000), dict(batch=1, heads=2, dim=64, lo=1500, hi=1500), "split"),
         # per-XCD queues: counters in the scratch array; then a short plain list that needs none of it
         (dict(batch=48, heads=4, dim=128, lo=200, hi=2000), dict(batch=8, heads=4, dim=128, lo=100, hi=600), "queues"),
     ],
@@ -51,8 +53,17 @@ def test_noalloc_entry_point_matches_the_workspace_one(first, second, variant):
         assert torch.equal(p.out, want), f"{variant}, call {i}: the two entry points differ"
 
 
-def test_noalloc_entry_point_refuses_what_its_scratch_cannot_hold():
+def test_noalloc_entry_point_limits():
+    """The scratch array is sized for the largest request a description can make today (the counter block plus one
+    fp32 partial output of 128 x 128 per resident workgroup at two workgroups per CU), so the refusal with
+    HSTU_ERR_WORKSPACE guards variants to come and cannot be provoked from here; what can be checked from the host is
+    that a description is validated first and that the limit is what the header says."""
     lib = _native.load()
-    # head dim 512 is served by the coverage kernel, no workspace: accepted; a null description is refused
     assert lib.hstu_jagged_fwd_noalloc(None, None) == 161001
     assert lib.hstu_jagged_fwd_noalloc_max_workspace() == (32 << 20) + 16384
+    # the largest workspace any forward description asks for fits: long single sequences at every slot with split items
+    asked = []
+    for dim in (32, 64, 128, 256):
+        w = workloads.make("x", dtype=torch.bfloat16, device=DEV, batch=1, heads=1, dim=dim, lo=20480, hi=20480)
+        asked.append(prepared(w).workspace_bytes)
+    assert max(asked) == lib.hstu_jagged_fwd_noalloc_max_workspace(), asked
