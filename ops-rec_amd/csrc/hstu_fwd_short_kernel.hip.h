@@ -545,10 +545,10 @@ __global__ __launch_bounds__(kShortThreads, kShortWavesPerSimd) void hstu_fwd_sh
     }
 
 #ifdef HSTU_TIMELINE
-    if (a.ws != nullptr && tid == 0) {
+    if (a.counters != nullptr && tid == 0) {
         __builtin_amdgcn_s_waitcnt(0);
         HSTU_TL(4);
-        uint64_t* const rec = reinterpret_cast<uint64_t*>(a.ws) + static_cast<uint64_t>(blockIdx.x) * 8;
+        uint64_t* const rec = reinterpret_cast<uint64_t*>(a.counters) + static_cast<uint64_t>(blockIdx.x) * 8;
         for (int i = 0; i < 5; ++i) {
             rec[i] = tl[i];
         }

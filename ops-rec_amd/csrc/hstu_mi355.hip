@@ -1292,7 +1292,7 @@ int launch_forward(const hstu_jagged_fwd_params* p, const hstu_paged_fwd_params*
         }
 #ifdef HSTU_TIMELINE
         if (const char* const t = getenv("HSTU_TIMELINE_BUFFER")) {
-            a.ws = reinterpret_cast<float*>(strtoull(t, nullptr, 0));  // development builds: where the workgroups leave their time stamps
+            a.counters = reinterpret_cast<unsigned int*>(strtoull(t, nullptr, 0));  // development builds: where the workgroups leave their time stamps
         }
 #endif
         hipLaunchKernelGGL(sv->kernel, dim3(static_cast<unsigned>(slots)), dim3(hstu::kShortThreads), 0,

@@ -29,6 +29,8 @@ def main() -> None:
     ap = argparse.ArgumentParser()
     ap.add_argument("--build", action="store_true", help="compile the library with -DHSTU_TIMELINE and exit")
     ap.add_argument("--workload", default="C2")
+    ap.add_argument("--burst", type=int, default=1, help="launches back to back; the stamps are those of the last one")
+    ap.add_argument("--shape", default=None, help="batch,heads,shortest,longest at head dim 128 instead of a named workload")
     args = ap.parse_args()
     if args.build:
         print(_build.build(verbose=False, extra_flags=("-DHSTU_TIMELINE",), lib_path=TIMELINE_LIB))
@@ -42,7 +44,12 @@ def main() -> None:
     from ops_rec import _native, _ops, workloads
 
     dev = "cuda:0"
-    w = workloads.config(args.workload).to(dev)
+    if args.shape:
+        batch, heads, lo, hi = (int(v) for v in args.shape.split(","))
+        w = workloads.make("shape", dtype=torch.bfloat16, device=dev, dim=128, batch=batch, heads=heads, lo=lo, hi=hi)
+        args.workload = args.shape
+    else:
+        w = workloads.config(args.workload).to(dev)
     buf = torch.zeros(1 << 20, dtype=torch.int64, device=dev)  # 8 words per workgroup
     os.environ["HSTU_TIMELINE_BUFFER"] = str(buf.data_ptr())
     os.environ["HSTU_MI355_SHORT"] = "1"
@@ -56,7 +63,8 @@ def main() -> None:
     torch.cuda.synchronize()
     buf.zero_()
     torch.cuda.synchronize()
-    p.launch()
+    for _ in range(args.burst):  # (every launch overwrites the records: what is read back is the last one)
+        p.launch()
     torch.cuda.synchronize()
     r = buf.cpu().numpy().reshape(-1, 8)
     r = r[r[:, 0] != 0]
