@@ -188,7 +188,9 @@ HSTU_API uint64_t hstu_jagged_fwd_noalloc_max_workspace(void);
  * inputs with head dims up to 128: dS and P in fp32 whenever that fits).  Head dims above 256 need, beside that line
  * per row and block, 256 bytes per head, query row and block for the scores of the first window.  Without the workspace,
  * or with less than was asked for, the call still works: the kernels that produce grad_k then recompute dS (head dims
- * above 256: the generic kernels run).  The workspace needs no clearing and holds nothing afterwards. */
+ * above 256: the generic kernels run).  The workspace needs no clearing and holds nothing afterwards.  Batches of
+ * sequences of at most 32 rows and keys (bf16 / fp16, no attn_bias, no custom mask, head dims up to 256 in multiples
+ * of 8, 16-byte aligned tensors) run in one launch and ask for no workspace. */
 typedef struct hstu_jagged_bwd_params {
     uint32_t struct_size; /* sizeof(hstu_jagged_bwd_params) */
     uint32_t reserved0;

@@ -1,6 +1,8 @@
 // kernels for short work lists / short rows (16-bit inputs, head-dim slot 128, no custom mask): the forward (with and
-// without attn_bias), the forward for batches of tiny sequences, and the backward's query-tile kernel (no bias)
+// without attn_bias), the forward and the backward for batches of tiny sequences, and the backward's query-tile kernel
+// (no bias)
 #include "hstu_bwd_dq_short_kernel.hip.h"
+#include "hstu_bwd_tiny_kernel.hip.h"
 #include "hstu_fwd_short_kernel.hip.h"
 #include "hstu_fwd_tiny_kernel.hip.h"
 #include "hstu_variants.h"
@@ -31,4 +33,12 @@ const DqShortVariant kDqShort[2] = {
 };
 }
 const DqShortVariant* bwd_variants_dq_short() { return kDqShort; }
+
+namespace {
+const BwdTinyVariant kBwdTiny[2][2] = {
+    {{"hstu_bwd_bf16_d128_tiny", hstu_bwd_tiny_kernel<bf16_tag, 128>}, {"hstu_bwd_bf16_d256_tiny", hstu_bwd_tiny_kernel<bf16_tag, 256>}},
+    {{"hstu_bwd_f16_d128_tiny", hstu_bwd_tiny_kernel<f16_tag, 128>}, {"hstu_bwd_f16_d256_tiny", hstu_bwd_tiny_kernel<f16_tag, 256>}},
+};
+}
+const BwdTinyVariant (*bwd_variants_tiny())[2] { return kBwdTiny; }
 }  // namespace hstu

@@ -859,6 +859,26 @@ static int64_t dq_short_grid(const hstu::BwdArgs& a)
     return ((a.max_q + hstu::kDqShortRows - 1) / hstu::kDqShortRows) * pairs_pad * a.head_ratio;
 }
 
+// The whole backward in one launch for batches of tiny sequences (hstu_bwd_tiny_kernel.hip.h): 16-bit inputs with head
+// dims up to 256 in multiples of 8, no bias (nor its gradient), no custom mask, no sequence longer than 32 rows or keys,
+// every tensor on a 16-byte boundary.  No workspace.  Batch 2048 x 2 heads x 32 rows at head dim 256: 221 us on the tuned
+// kernels (a 128-row workgroup per item in each of two launches).  HSTU_MI355_SHORT=0 switches it off.
+static const hstu::BwdTinyVariant* bwd_tiny_variant(const hstu_jagged_bwd_params* p)
+{
+    const hstu_jagged_fwd_params* f = &p->fwd;
+    const int64_t dmax = f->head_dim_qk > f->head_dim_v ? f->head_dim_qk : f->head_dim_v;
+    const uintptr_t ptrs = reinterpret_cast<uintptr_t>(f->q) | reinterpret_cast<uintptr_t>(f->k) | reinterpret_cast<uintptr_t>(f->v) |
+                           reinterpret_cast<uintptr_t>(p->grad) | reinterpret_cast<uintptr_t>(p->grad_q) |
+                           reinterpret_cast<uintptr_t>(p->grad_k) | reinterpret_cast<uintptr_t>(p->grad_v);
+    if ((f->dtype != HSTU_DT_BF16 && f->dtype != HSTU_DT_FP16) || f->attn_bias != nullptr || p->grad_attn_bias != nullptr ||
+        f->mask_type == HSTU_MASK_CUSTOM || dmax > 256 || f->head_dim_qk % 8 != 0 || f->head_dim_v % 8 != 0 || ptrs % 16 != 0 ||
+        f->max_seq_len_q > hstu::kTinyRows || f->max_seq_len_k > hstu::kTinyRows || f->n_offsets < 2 ||
+        (f->n_offsets - 1) * f->num_heads_k > 0x7fffffffLL || switches().short_lists == 0 || switches().generic_backward == 1) {
+        return nullptr;
+    }
+    return &hstu::bwd_variants_tiny()[f->dtype == HSTU_DT_BF16 ? 0 : 1][dmax <= 128 ? 0 : 1];
+}
+
 // Head dims above 256 on the matrix pipe: 16-bit inputs whose head dims are multiples of 16 run as two windows per head
 // on the kernels of the slot 256 (heads taken as 2 x heads of half the dims): the query-tile kernel over the first window
 // (S and dP in fp32 to a partial plane), over the second (adds them up: dS and P to the pair plane, dQ of the second
@@ -917,6 +937,9 @@ HSTU_API int hstu_jagged_bwd_workspace_size(const hstu_jagged_bwd_params* params
     const BwdVariant* var = select_bwd(params);
     if (var == nullptr) {
         return HSTU_ERR_UNSUPPORTED;
+    }
+    if (bwd_tiny_variant(params) != nullptr) {
+        return HSTU_OK;
     }
     const WindowPlan windows = plan_windows(params);
     *workspace_bytes = windows.var != nullptr ? windows.workspace_bytes : plan_bwd(params, var).workspace_bytes;
@@ -1000,6 +1023,15 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
     a.alpha = static_cast<float>(f->alpha);
     a.scale = static_cast<float>((f->silu_scale == 0.0) ? 1.0 / static_cast<double>(f->max_seq_len_q) : f->silu_scale);
 
+    if (const hstu::BwdTinyVariant* const tv = bwd_tiny_variant(p)) {
+        hipLaunchKernelGGL(tv->kernel, dim3(static_cast<unsigned>(a.n_batch * a.n_heads_k)), dim3(hstu::kTinyThreads), 0,
+                           static_cast<hipStream_t>(stream), a);
+        const hipError_t err_tiny = hipGetLastError();
+        if (err_tiny != hipSuccess) {
+            return fail(HSTU_ERR_RUNTIME, "launch of %s failed: %s", tv->name, hipGetErrorString(err_tiny));
+        }
+        return HSTU_OK;
+    }
     const WindowPlan windows = plan_windows(p);
     if (windows.var != nullptr && usable_workspace(workspace, workspace_bytes, windows.workspace_bytes) &&
         reinterpret_cast<uintptr_t>(workspace) % 16 == 0 && a.grad_vec_ok != 0) {

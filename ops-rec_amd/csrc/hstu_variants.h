@@ -29,6 +29,12 @@ struct ShortVariant {
     void (*kernel)(const FwdArgs);
 };
 
+// the whole backward in one launch for batches of tiny sequences (hstu_bwd_tiny_kernel.hip.h)
+struct BwdTinyVariant {
+    const char* name;
+    void (*kernel)(const BwdArgs);
+};
+
 // the query-tile backward kernel for short rows (hstu_bwd_dq_short_kernel.hip.h): 16-bit inputs, head-dim slot 128,
 // no bias, no custom mask; one workgroup of `threads` per (64-row tile, sequence, head) slot
 struct DqShortVariant {
@@ -79,6 +85,9 @@ const BwdVariant (*bwd_variants_bf16())[2][3];
 const BwdVariant (*bwd_variants_f16())[2][3];
 // backward, query-tile kernel for short rows: [bf16, fp16]
 const DqShortVariant* bwd_variants_dq_short();
+// backward for batches of sequences of at most 32 rows and keys (one workgroup of kTinyThreads per (sequence, K/V head)),
+// no bias, no custom mask, head dims up to 256 in multiples of 8: [bf16, fp16][head-dim slot 128, 256]
+const BwdTinyVariant (*bwd_variants_tiny())[2];
 // backward, fp32 inputs with head dims up to 128 (fp32 MFMA, one workgroup per key tile, the same kernel with and
 // without d rab; launched like the generic ones, behind fills of the outputs): [rab][custom mask][dim slot: 32, 64, 128]
 const BwdVariant (*bwd_variants_f32())[2][3];

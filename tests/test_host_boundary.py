@@ -459,6 +459,17 @@ def test_backward_workspace_follows_the_launch_order(monkeypatch):
     assert size(**dict(c2, mask_type=2)) == pair_all_blocks()
     assert size(**dict(c2, num_context=fake)) == pair_all_blocks()
     assert size(**dict(c2, seq_offset_k=fake + 64)) == pair_all_blocks()
+    # batches of sequences of at most 32 rows and keys run in one launch that needs no workspace -- without bias or
+    # custom mask, head dims up to 256 in multiples of 8, 16-byte aligned tensors; HSTU_MI355_SHORT=0 switches it off
+    tiny = dict(c2, total_q=600, total_k=600, max_seq_len_q=32, max_seq_len_k=32)
+    tiny_pair = pair(rows=600, blocks=1)
+    assert size(**tiny) == 0 and size(**dict(tiny, head_dim_qk=256, head_dim_v=256)) == 0
+    assert size(**dict(tiny, max_seq_len_q=40, max_seq_len_k=40)) == pair(rows=600, blocks=2)
+    assert size(**dict(tiny, q=fake + 8)) == tiny_pair
+    assert size(grad_attn_bias=fake, **tiny) == tiny_pair
+    helpers.set_switch(monkeypatch, "HSTU_MI355_SHORT", "0")
+    assert size(**tiny) == tiny_pair
+    helpers.set_switch(monkeypatch, "HSTU_MI355_SHORT", None)
     helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_WORKSPACE_MB", "300")  # the limit of the workspace
     assert size(**dict(c2, mask_type=2)) == one
     helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_WORKSPACE_MB", "100")
