@@ -27,6 +27,8 @@ constexpr int kTinyThreads = 128;   // threads of a workgroup of the forward ker
 constexpr int kTinyRows = 32;       // the longest sequence (rows and keys) that kernel takes
 constexpr int kDqShortThreads = 256;  // threads of a workgroup of the backward's query-tile kernel for short rows (four wavefronts of 16 rows)
 constexpr int kDqShortRows = 64;      // query rows of its tile
+constexpr int kFewRowsThreads = 256;  // threads of a workgroup of the backward kernel for sequences of few query rows
+constexpr int kFewRows = 64;          // the most query rows of a sequence that kernel takes
 constexpr int kCounterBlockBytes = 16384;  // head of the workspace: device-side work counters (see the forward kernel)
 constexpr int kDkvThreads = 256;   // threads of a workgroup of the key-tile backward kernel
 constexpr int kGatherThreads = 128;

@@ -1,7 +1,8 @@
 // kernels for short work lists / short rows (16-bit inputs, head-dim slot 128, no custom mask): the forward (with and
-// without attn_bias), the forward and the backward for batches of tiny sequences, and the backward's query-tile kernel
-// (no bias)
+// without attn_bias), the forward and the backward for batches of tiny sequences, the backward for sequences of few query
+// rows, and the backward's query-tile kernel (no bias)
 #include "hstu_bwd_dq_short_kernel.hip.h"
+#include "hstu_bwd_few_rows_kernel.hip.h"
 #include "hstu_bwd_tiny_kernel.hip.h"
 #include "hstu_fwd_short_kernel.hip.h"
 #include "hstu_fwd_tiny_kernel.hip.h"
@@ -41,4 +42,12 @@ const BwdTinyVariant kBwdTiny[2][2] = {
 };
 }
 const BwdTinyVariant (*bwd_variants_tiny())[2] { return kBwdTiny; }
+
+namespace {
+const BwdTinyVariant kBwdFewRows[2] = {
+    {"hstu_bwd_bf16_d64_few_rows", hstu_bwd_few_rows_kernel<bf16_tag, 64>},
+    {"hstu_bwd_f16_d64_few_rows", hstu_bwd_few_rows_kernel<f16_tag, 64>},
+};
+}
+const BwdTinyVariant* bwd_variants_few_rows() { return kBwdFewRows; }
 }  // namespace hstu

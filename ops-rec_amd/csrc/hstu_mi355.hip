@@ -879,6 +879,37 @@ static const hstu::BwdTinyVariant* bwd_tiny_variant(const hstu_jagged_bwd_params
     return &hstu::bwd_variants_tiny()[f->dtype == HSTU_DT_BF16 ? 0 : 1][dmax <= 128 ? 0 : 1];
 }
 
+// The whole backward in one launch for sequences of few query rows (hstu_bwd_few_rows_kernel.hip.h): 16-bit inputs with
+// head dims up to 64 in multiples of 8, no bias (nor its gradient), no custom mask, no sequence of more than 64 query rows
+// (keys: any number), as many K/V heads as query heads, every tensor on a 16-byte boundary.  No workspace; K and V are
+// read once.  HSTU_MI355_SHORT=0 switches it off.
+static const hstu::BwdTinyVariant* bwd_few_rows_variant(const hstu_jagged_bwd_params* p)
+{
+    const hstu_jagged_fwd_params* f = &p->fwd;
+    const int64_t dmax = f->head_dim_qk > f->head_dim_v ? f->head_dim_qk : f->head_dim_v;
+    const uintptr_t ptrs = reinterpret_cast<uintptr_t>(f->q) | reinterpret_cast<uintptr_t>(f->k) | reinterpret_cast<uintptr_t>(f->v) |
+                           reinterpret_cast<uintptr_t>(p->grad) | reinterpret_cast<uintptr_t>(p->grad_q) |
+                           reinterpret_cast<uintptr_t>(p->grad_k) | reinterpret_cast<uintptr_t>(p->grad_v);
+    const int64_t span_k = f->max_seq_len_k * f->num_heads_k * dmax * 2;
+    if ((f->dtype != HSTU_DT_BF16 && f->dtype != HSTU_DT_FP16) || f->attn_bias != nullptr || p->grad_attn_bias != nullptr ||
+        f->mask_type == HSTU_MASK_CUSTOM || dmax > 64 || f->head_dim_qk % 8 != 0 || f->head_dim_v % 8 != 0 || ptrs % 16 != 0 ||
+        f->max_seq_len_q > hstu::kFewRows || f->num_heads_q != f->num_heads_k || f->n_offsets < 2 || span_k >= (1LL << 30) ||
+        (f->n_offsets - 1) * f->num_heads_k > 0x7fffffffLL || switches().short_lists == 0 || switches().generic_backward == 1) {
+        return nullptr;
+    }
+    return &hstu::bwd_variants_few_rows()[f->dtype == HSTU_DT_BF16 ? 0 : 1];
+}
+// the one-launch kernels: tiny sequences first (it takes grouped heads and head dims up to 256), then few query rows
+static const hstu::BwdTinyVariant* bwd_one_launch_variant(const hstu_jagged_bwd_params* p, unsigned* threads)
+{
+    if (const hstu::BwdTinyVariant* const tv = bwd_tiny_variant(p)) {
+        *threads = hstu::kTinyThreads;
+        return tv;
+    }
+    *threads = hstu::kFewRowsThreads;
+    return bwd_few_rows_variant(p);
+}
+
 // Head dims above 256 on the matrix pipe: 16-bit inputs whose head dims are multiples of 16 run as two windows per head
 // on the kernels of the slot 256 (heads taken as 2 x heads of half the dims): the query-tile kernel over the first window
 // (S and dP in fp32 to a partial plane), over the second (adds them up: dS and P to the pair plane, dQ of the second
@@ -938,7 +969,8 @@ HSTU_API int hstu_jagged_bwd_workspace_size(const hstu_jagged_bwd_params* params
     if (var == nullptr) {
         return HSTU_ERR_UNSUPPORTED;
     }
-    if (bwd_tiny_variant(params) != nullptr) {
+    unsigned one_launch_threads = 0;
+    if (bwd_one_launch_variant(params, &one_launch_threads) != nullptr) {
         return HSTU_OK;
     }
     const WindowPlan windows = plan_windows(params);
@@ -1023,8 +1055,9 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
     a.alpha = static_cast<float>(f->alpha);
     a.scale = static_cast<float>((f->silu_scale == 0.0) ? 1.0 / static_cast<double>(f->max_seq_len_q) : f->silu_scale);
 
-    if (const hstu::BwdTinyVariant* const tv = bwd_tiny_variant(p)) {
-        hipLaunchKernelGGL(tv->kernel, dim3(static_cast<unsigned>(a.n_batch * a.n_heads_k)), dim3(hstu::kTinyThreads), 0,
+    unsigned one_launch_threads = 0;
+    if (const hstu::BwdTinyVariant* const tv = bwd_one_launch_variant(p, &one_launch_threads)) {
+        hipLaunchKernelGGL(tv->kernel, dim3(static_cast<unsigned>(a.n_batch * a.n_heads_k)), dim3(one_launch_threads), 0,
                            static_cast<hipStream_t>(stream), a);
         const hipError_t err_tiny = hipGetLastError();
         if (err_tiny != hipSuccess) {

@@ -29,7 +29,8 @@ struct ShortVariant {
     void (*kernel)(const FwdArgs);
 };
 
-// the whole backward in one launch for batches of tiny sequences (hstu_bwd_tiny_kernel.hip.h)
+// the whole backward in one launch: for batches of tiny sequences (hstu_bwd_tiny_kernel.hip.h), for sequences of few query
+// rows (hstu_bwd_few_rows_kernel.hip.h)
 struct BwdTinyVariant {
     const char* name;
     void (*kernel)(const BwdArgs);
@@ -88,6 +89,9 @@ const DqShortVariant* bwd_variants_dq_short();
 // backward for batches of sequences of at most 32 rows and keys (one workgroup of kTinyThreads per (sequence, K/V head)),
 // no bias, no custom mask, head dims up to 256 in multiples of 8: [bf16, fp16][head-dim slot 128, 256]
 const BwdTinyVariant (*bwd_variants_tiny())[2];
+// backward for sequences of at most 64 query rows and any number of keys (one workgroup of kFewRowsThreads per (sequence,
+// head)), no bias, no custom mask, head dims up to 64 in multiples of 8, as many K/V heads as query heads: [bf16, fp16]
+const BwdTinyVariant* bwd_variants_few_rows();
 // backward, fp32 inputs with head dims up to 128 (fp32 MFMA, one workgroup per key tile, the same kernel with and
 // without d rab; launched like the generic ones, behind fills of the outputs): [rab][custom mask][dim slot: 32, 64, 128]
 const BwdVariant (*bwd_variants_f32())[2][3];

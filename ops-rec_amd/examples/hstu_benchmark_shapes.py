@@ -3,7 +3,7 @@
 (ascendc/attention/hstu_v2/test/pytest/test_backward_op_benchmark.py:183-197 "user case 1", :244-258 "user case 2":
 every sequence at the full length, causal mask, no context / targets), one JSON line per shape:
 
-    python hstu_benchmark_shapes.py [--case 1|2|all] [--budget-ms 300]
+    python hstu_benchmark_shapes.py [--case 1|2|all] [--only INDEX[,INDEX...]] [--budget-ms 300]
 
 The reference runs these under msprof and extracts the task duration per operator
 (hstu_v2/test/pytest/run_benchmark.sh:17-31, utils/perf_stats.py); here each operator call is timed with events on
@@ -93,9 +93,12 @@ def run(batch, heads, dims, lens, rab, dtype, budget_ms):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--case", default="all", choices=["1", "2", "all"])
+    ap.add_argument("--only", default="", help="positions in the chosen list, comma-separated (all when empty)")
     ap.add_argument("--budget-ms", type=float, default=300.0)
     args = ap.parse_args()
     shapes = (CASE_1 if args.case in ("1", "all") else []) + (CASE_2 if args.case in ("2", "all") else [])
+    if args.only:
+        shapes = [shapes[int(i)] for i in args.only.split(",")]
     for shape in shapes:
         try:
             print(json.dumps(run(*shape, args.budget_ms)), flush=True)
