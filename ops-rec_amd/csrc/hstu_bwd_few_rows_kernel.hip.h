@@ -42,7 +42,7 @@ __global__ __launch_bounds__(kFewRowsThreads, 2) void hstu_bwd_few_rows_kernel(c
     constexpr int NSTAGE = 3;
     constexpr int LPW = SUB_ELEMS * 2 / 1024 / 4;      // 1 KiB load instructions per wavefront and sub-tile (K, and again V)
     constexpr int QLOADS = ROWS * D * 2 / 1024 / 4;    // ... per wavefront for the Q tile (and again dO)
-    constexpr int STORES = MTILES;                     // store instructions per wavefront and step (dV or dK of 16 keys)
+    constexpr int STORES = MTILES / 2;                 // store instructions per wavefront and step (dV or dK of 16 keys)
     static_assert(LPW >= 1 && QLOADS >= 1, "whole load instructions per wavefront");
     // at the top of step x its sub-tile has landed when nothing older than this is open: the requests of step x + 1 and
     // the stores of two steps (vector memory operations complete in the order of issue)
@@ -266,24 +266,28 @@ __global__ __launch_bounds__(kFewRowsThreads, 2) void hstu_bwd_few_rows_kernel(c
                 const u32x2_t hi = lds_read_tr16_b64(xs + ks * 32 * 32 + 16 * 32);
                 bop[ks] = u32x4_t{lo[0], lo[1], hi[0], hi[1]};
             }
+            typedef __attribute__((ext_vector_type(2))) unsigned u2_t;
             const __amdgpu_buffer_rsrc_t out_rsrc = dk_role ? dk_rsrc : dv_rsrc;
             const uint32_t out_stride = dk_role ? k_stride : v_stride;
             const int out_dims = dk_role ? a.d_qk : a.d_v;
             const uint32_t row_off = static_cast<uint32_t>(c0 + 16 * kh + n) * out_stride;
 #pragma unroll
-            for (int mt = 0; mt < MTILES; ++mt) {
-                f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+            for (int mt = 0; mt < MTILES; mt += 2) {
+                f32x4_t acc0 = {0.f, 0.f, 0.f, 0.f}, acc1 = acc0;
 #pragma unroll
                 for (int ks = 0; ks < ROWS / 32; ++ks) {
-                    acc = mfma16<Tag>(read_t(rows + ks * 32 * D, mt), bop[ks], acc);
+                    acc0 = mfma16<Tag>(read_t(rows + ks * 32 * D, mt), bop[ks], acc0);
+                    acc1 = mfma16<Tag>(read_t(rows + ks * 32 * D, mt + 1), bop[ks], acc1);
                 }
-                // lane (n, g) holds dims 16 mt + 4 g + 0..3 of key c0 + 16 kh + n (keys past the sequence fall outside
-                // the descriptor)
-                const int d0 = 16 * mt + 4 * g;
-                u32x2_t w;
-                w[0] = pack2<Tag>(acc[0], acc[1]);
-                w[1] = pack2<Tag>(acc[2], acc[3]);
-                __builtin_amdgcn_raw_buffer_store_b64(w, out_rsrc, static_cast<int>(d0 < out_dims ? row_off + d0 * 2u : kOutOfRange), 0, 0);
+                // lane (n, g) holds dims 16 mt + 4 g + 0..3 of key c0 + 16 kh + n for both tiles; lanes 16 apart trade one
+                // of them (v_permlane16_swap: odd rows of the first operand against even rows of the second), after which
+                // a lane holds 8 dims in a row: of tile mt at 8 (g / 2) when g is even, of tile mt + 1 when it is odd
+                // (keys past the sequence fall outside the descriptor)
+                const u2_t lo = __builtin_amdgcn_permlane16_swap(pack2<Tag>(acc0[0], acc0[1]), pack2<Tag>(acc1[0], acc1[1]), false, false);
+                const u2_t hi = __builtin_amdgcn_permlane16_swap(pack2<Tag>(acc0[2], acc0[3]), pack2<Tag>(acc1[2], acc1[3]), false, false);
+                const u32x4_t piece = {lo[0], hi[0], lo[1], hi[1]};
+                const int d0 = 16 * (mt + (g & 1)) + 8 * (g >> 1);
+                __builtin_amdgcn_raw_buffer_store_b128(piece, out_rsrc, static_cast<int>(d0 < out_dims ? row_off + d0 * 2u : kOutOfRange), 0, 0);
             }
         }
         stage = stage + 1 < NSTAGE ? stage + 1 : 0;
