@@ -191,7 +191,7 @@ HSTU_API uint64_t hstu_jagged_fwd_noalloc_max_workspace(void);
  * above 256: the generic kernels run).  The workspace needs no clearing and holds nothing afterwards.  Batches of
  * sequences of at most 32 rows and keys (bf16 / fp16, no attn_bias, no custom mask, head dims up to 256 in multiples
  * of 8, 16-byte aligned tensors) run in one launch and ask for no workspace, and so do batches of sequences of at most
- * 64 query rows against keys of any length at head dims up to 64 with num_heads_k == num_heads_q. */
+ * 64 query rows against keys of any length at head dims up to 128 with num_heads_k == num_heads_q. */
 typedef struct hstu_jagged_bwd_params {
     uint32_t struct_size; /* sizeof(hstu_jagged_bwd_params) */
     uint32_t reserved0;

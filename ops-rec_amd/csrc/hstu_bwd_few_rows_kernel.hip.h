@@ -1,5 +1,5 @@
 // HSTU jagged attention backward for gfx950 (MI355X): the kernel for sequences of few query rows -- at most 64 -- against
-// keys of any length (candidates attending to a long history), head dims up to 64, one K/V head per query head.
+// keys of any length (candidates attending to a long history), head dims up to 128, one K/V head per query head.
 //
 // The tuned kernels give such a sequence one 128-row query tile, mostly empty, and a pair of workgroups per 128 keys,
 // each of which starts up (offsets, Q and dO rows) for a sweep of one or two steps: batch 2048 x 4 heads x 52 rows x
@@ -26,6 +26,17 @@ __device__ __forceinline__ int both_ways16_swizzle64(int row, int chunk)
     const int b1 = (row >> 1) & 1, b2 = (row >> 2) & 1, b3 = (row >> 3) & 1;
     return chunk ^ (b1 | (b2 << 1) | ((b1 ^ b3) << 2));
 }
+// the layout of the kernel's tiles by head-dim slot (rows of 128 elements: that of the query-tile kernel for short rows)
+template <int D>
+__device__ __forceinline__ int few_rows_swizzle(int row, int chunk)
+{
+    static_assert(D == 64 || D == 128, "head-dim slots 64 and 128");
+    if constexpr (D == 64) {
+        return both_ways16_swizzle64(row, chunk);
+    } else {
+        return both_ways16_swizzle<D>(row, chunk);
+    }
+}
 // The exchange buffer [64 rows][32 keys] in 8-byte chunks (4 keys): the query side writes a row's chunks g and 4 + g,
 // the key side reads 4-row x 16-key blocks transposing
 __device__ __forceinline__ int exchange_chunk(int row, int chunk) { return chunk ^ ((((row >> 2) & 1) << 2) | (((row >> 3) & 1) << 1)); }
@@ -33,19 +44,19 @@ __device__ __forceinline__ int exchange_chunk(int row, int chunk) { return chunk
 template <typename Tag, int D>
 __global__ __launch_bounds__(kFewRowsThreads, 2) void hstu_bwd_few_rows_kernel(const BwdArgs a)
 {
-    static_assert(D == 64, "built for the head-dim slot 64");
+    static_assert(D == 64 || D == 128, "built for the head-dim slots 64 and 128");
     constexpr int ROWS = kFewRows;
     constexpr int SUB_ELEMS = 32 * D;
     constexpr int CPR = D / 8;
     constexpr int KSTEPS = D / 32;
     constexpr int MTILES = D / 16;
-    constexpr int NSTAGE = 3;
+    constexpr int NSTAGE = D == 64 ? 3 : 2;  // (72 KiB of LDS at the slot 128: two workgroups per CU)
     constexpr int LPW = SUB_ELEMS * 2 / 1024 / 4;      // 1 KiB load instructions per wavefront and sub-tile (K, and again V)
     constexpr int QLOADS = ROWS * D * 2 / 1024 / 4;    // ... per wavefront for the Q tile (and again dO)
     constexpr int STORES = MTILES / 2;                 // store instructions per wavefront and step (dV or dK of 16 keys)
     static_assert(LPW >= 1 && QLOADS >= 1, "whole load instructions per wavefront");
-    // at the top of step x its sub-tile has landed when nothing older than this is open: the requests of step x + 1 and
-    // the stores of two steps (vector memory operations complete in the order of issue)
+    // at the top of step x its sub-tile has landed when nothing older than this is open: the requests of the steps after
+    // it and the stores of the steps since it was asked for (vector memory operations complete in the order of issue)
     constexpr int kOpen = (NSTAGE - 2) * 2 * LPW + (NSTAGE - 1) * STORES;
     static_assert(kOpen < 64, "6 bits of count");
     constexpr int kWaitStage = (kOpen & 15) | (7 << 4) | (15 << 8) | ((kOpen >> 4) << 14);
@@ -105,7 +116,7 @@ __global__ __launch_bounds__(kFewRowsThreads, 2) void hstu_bwd_few_rows_kernel(c
         const int instr = wave * QLOADS + i;
         const int piece = instr * 64 + lane;
         const int r = piece / CPR;
-        const int cs = both_ways16_swizzle64(r, piece % CPR);
+        const int cs = few_rows_swizzle<D>(r, piece % CPR);
         request_to_lds_b128(q_rsrc, lds_address(s_q) + instr * 1024u,
                             (cs * 8 < a.d_qk) ? static_cast<uint32_t>(r) * q_stride + cs * 16u : kOutOfRange);
         request_to_lds_b128(g_rsrc, lds_address(s_g) + instr * 1024u,
@@ -117,7 +128,7 @@ __global__ __launch_bounds__(kFewRowsThreads, 2) void hstu_bwd_few_rows_kernel(c
     for (int i = 0; i < LPW; ++i) {
         const int piece = (wave * LPW + i) * 64 + lane;
         const int r = piece / CPR;
-        const int cs = both_ways16_swizzle64(r, piece % CPR);
+        const int cs = few_rows_swizzle<D>(r, piece % CPR);
         k_src[i] = (cs * 8 < a.d_qk) ? static_cast<uint32_t>(r) * k_stride + cs * 16u : kOutOfRange;
         v_src[i] = (cs * 8 < a.d_v) ? static_cast<uint32_t>(r) * v_stride + cs * 16u : kOutOfRange;
     }
@@ -133,21 +144,23 @@ __global__ __launch_bounds__(kFewRowsThreads, 2) void hstu_bwd_few_rows_kernel(c
             request_to_lds_b128(v_rsrc, lds_address(s_v[stage]) + (wave * LPW + i) * 1024u, v_src[i] + vb);
         }
     };
-    request(0, 0);
-    request(1, 1);
+#pragma unroll
+    for (int i = 0; i < NSTAGE - 1; ++i) {
+        request(i, i);
+    }
 
     // LDS read offsets relative to a tile, in elements: plain read of row n (+ 16), MFMA step js; transposed read of rows
     // 4 g .. 4 g + 3 (+ 16), dims 16 mt .. + 15
     int n_lane_off[KSTEPS];
 #pragma unroll
     for (int js = 0; js < KSTEPS; ++js) {
-        n_lane_off[js] = n * D + both_ways16_swizzle64(n, 4 * js + g) * 8;
+        n_lane_off[js] = n * D + few_rows_swizzle<D>(n, 4 * js + g) * 8;
     }
     const int vr = 4 * g + (n >> 2);
     const int t_row_off = vr * D + 4 * (n & 1);
     const int t_chunk_lo = (n & 3) >> 1;
     auto read_t = [&](const uint16_t* tile, int mt) -> u32x4_t {
-        const uint16_t* const p = tile + t_row_off + both_ways16_swizzle64(vr, 2 * mt + t_chunk_lo) * 8;
+        const uint16_t* const p = tile + t_row_off + few_rows_swizzle<D>(vr, 2 * mt + t_chunk_lo) * 8;
         const u32x2_t lo = lds_read_tr16_b64(p);
         const u32x2_t hi = lds_read_tr16_b64(p + 16 * D);
         const u32x4_t r = {lo[0], lo[1], hi[0], hi[1]};
@@ -199,8 +212,8 @@ __global__ __launch_bounds__(kFewRowsThreads, 2) void hstu_bwd_few_rows_kernel(c
         __builtin_amdgcn_s_waitcnt(kWaitStage);
         __builtin_amdgcn_s_barrier();
         __builtin_amdgcn_sched_barrier(0);
-        const int ahead = stage >= 1 ? stage - 1 : NSTAGE - 1;  // (x + 2) mod 3
-        request(ahead, x + 2);
+        const int ahead = stage >= 1 ? stage - 1 : NSTAGE - 1;  // (x + NSTAGE - 1) mod NSTAGE
+        request(ahead, x + NSTAGE - 1);
         const uint16_t* const kn = s_k[stage];
         const uint16_t* const vn = s_v[stage];
         const int c0 = x * 32;

@@ -44,10 +44,10 @@ const BwdTinyVariant kBwdTiny[2][2] = {
 const BwdTinyVariant (*bwd_variants_tiny())[2] { return kBwdTiny; }
 
 namespace {
-const BwdTinyVariant kBwdFewRows[2] = {
-    {"hstu_bwd_bf16_d64_few_rows", hstu_bwd_few_rows_kernel<bf16_tag, 64>},
-    {"hstu_bwd_f16_d64_few_rows", hstu_bwd_few_rows_kernel<f16_tag, 64>},
+const BwdTinyVariant kBwdFewRows[2][2] = {
+    {{"hstu_bwd_bf16_d64_few_rows", hstu_bwd_few_rows_kernel<bf16_tag, 64>}, {"hstu_bwd_bf16_d128_few_rows", hstu_bwd_few_rows_kernel<bf16_tag, 128>}},
+    {{"hstu_bwd_f16_d64_few_rows", hstu_bwd_few_rows_kernel<f16_tag, 64>}, {"hstu_bwd_f16_d128_few_rows", hstu_bwd_few_rows_kernel<f16_tag, 128>}},
 };
 }
-const BwdTinyVariant* bwd_variants_few_rows() { return kBwdFewRows; }
+const BwdTinyVariant (*bwd_variants_few_rows())[2] { return kBwdFewRows; }
 }  // namespace hstu

@@ -880,7 +880,7 @@ static const hstu::BwdTinyVariant* bwd_tiny_variant(const hstu_jagged_bwd_params
 }
 
 // The whole backward in one launch for sequences of few query rows (hstu_bwd_few_rows_kernel.hip.h): 16-bit inputs with
-// head dims up to 64 in multiples of 8, no bias (nor its gradient), no custom mask, no sequence of more than 64 query rows
+// head dims up to 128 in multiples of 8, no bias (nor its gradient), no custom mask, no sequence of more than 64 query rows
 // (keys: any number), as many K/V heads as query heads, every tensor on a 16-byte boundary.  No workspace; K and V are
 // read once.  HSTU_MI355_SHORT=0 switches it off.
 static const hstu::BwdTinyVariant* bwd_few_rows_variant(const hstu_jagged_bwd_params* p)
@@ -892,12 +892,12 @@ static const hstu::BwdTinyVariant* bwd_few_rows_variant(const hstu_jagged_bwd_pa
                            reinterpret_cast<uintptr_t>(p->grad_k) | reinterpret_cast<uintptr_t>(p->grad_v);
     const int64_t span_k = f->max_seq_len_k * f->num_heads_k * dmax * 2;
     if ((f->dtype != HSTU_DT_BF16 && f->dtype != HSTU_DT_FP16) || f->attn_bias != nullptr || p->grad_attn_bias != nullptr ||
-        f->mask_type == HSTU_MASK_CUSTOM || dmax > 64 || f->head_dim_qk % 8 != 0 || f->head_dim_v % 8 != 0 || ptrs % 16 != 0 ||
+        f->mask_type == HSTU_MASK_CUSTOM || dmax > 128 || f->head_dim_qk % 8 != 0 || f->head_dim_v % 8 != 0 || ptrs % 16 != 0 ||
         f->max_seq_len_q > hstu::kFewRows || f->num_heads_q != f->num_heads_k || f->n_offsets < 2 || span_k >= (1LL << 30) ||
         (f->n_offsets - 1) * f->num_heads_k > 0x7fffffffLL || switches().short_lists == 0 || switches().generic_backward == 1) {
         return nullptr;
     }
-    return &hstu::bwd_variants_few_rows()[f->dtype == HSTU_DT_BF16 ? 0 : 1];
+    return &hstu::bwd_variants_few_rows()[f->dtype == HSTU_DT_BF16 ? 0 : 1][dmax <= 64 ? 0 : 1];
 }
 // the one-launch kernels: tiny sequences first (it takes grouped heads and head dims up to 256), then few query rows
 static const hstu::BwdTinyVariant* bwd_one_launch_variant(const hstu_jagged_bwd_params* p, unsigned* threads)

@@ -90,8 +90,9 @@ const DqShortVariant* bwd_variants_dq_short();
 // no bias, no custom mask, head dims up to 256 in multiples of 8: [bf16, fp16][head-dim slot 128, 256]
 const BwdTinyVariant (*bwd_variants_tiny())[2];
 // backward for sequences of at most 64 query rows and any number of keys (one workgroup of kFewRowsThreads per (sequence,
-// head)), no bias, no custom mask, head dims up to 64 in multiples of 8, as many K/V heads as query heads: [bf16, fp16]
-const BwdTinyVariant* bwd_variants_few_rows();
+// head)), no bias, no custom mask, head dims up to 128 in multiples of 8, as many K/V heads as query heads:
+// [bf16, fp16][head-dim slot 64, 128]
+const BwdTinyVariant (*bwd_variants_few_rows())[2];
 // backward, fp32 inputs with head dims up to 128 (fp32 MFMA, one workgroup per key tile, the same kernel with and
 // without d rab; launched like the generic ones, behind fills of the outputs): [rab][custom mask][dim slot: 32, 64, 128]
 const BwdVariant (*bwd_variants_f32())[2][3];

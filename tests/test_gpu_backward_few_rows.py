@@ -1,6 +1,6 @@
 """The backward for sequences of few query rows (hstu_bwd_few_rows_kernel.hip.h: one launch, a four-wavefront workgroup per
 (sequence, head) that keeps Q and dO in LDS, streams K and V once and finishes 32 keys per step; taken when no sequence
-has more than 64 query rows, head dims are at most 64 and every query head has its own K/V head): against torch autograd
+has more than 64 query rows, head dims are at most 128 and every query head has its own K/V head): against torch autograd
 on the CPU oracle and the library's generic kernels (the bars of test_gpu_backward.py), and against the tuned kernels on
 the same inputs (HSTU_MI355_SHORT=0).  Which calls take the kernel is the host's rule: test_host_boundary.py.
 """
@@ -49,6 +49,9 @@ DELTA_CASES = {
     "dims_8_64": dict(lq=[52, 3, 64, 17], lk=[499, 130, 64, 401], dim=8, dim_v=64),
     "dims_48_32": dict(lq=[32, 32, 32, 32, 32], lk=[499, 499, 499, 499, 499], dim=48, dim_v=32, heads=4),
     "three_heads": dict(lq=[50, 21, 64], lk=[257, 96, 65], heads=3),
+    "dim_128": dict(lq=[52, 7, 64, 33, 1], lk=[1000, 300, 64, 519, 77], dim=128),
+    "dims_72_128": dict(lq=[52, 3, 64, 17], lk=[499, 130, 64, 401], dim=72, dim_v=128),
+    "dims_128_96": dict(lq=[40, 64, 10, 0, 33], lk=[12, 200, 10, 50, 1], dim=128, dim_v=96, heads=3),
 }  # fmt: skip
 
 
@@ -70,6 +73,9 @@ SELF_CASES = {
     "targets": dict(batch=12, heads=3, dim=32, lo=34, hi=60, max_seq_len=60, max_target=30, target_group_size=1),
     "context_rows": dict(batch=9, heads=2, dim=64, dim_v=48, lo=33, hi=64, max_seq_len=64, num_context=40),
     "int64_offsets": dict(batch=7, heads=1, dim=64, lo=5, hi=50, max_seq_len=50, index_dtype=torch.int64),
+    "dim_128_up_to_64_rows": dict(batch=30, heads=2, dim=128, lo=1, hi=64, max_seq_len=64),
+    "dim_128_context_targets_groups": dict(batch=12, heads=2, dim=128, dim_v=112, lo=20, hi=64, max_seq_len=64, num_context=3,
+                                           max_target=9, target_group_size=2),
 }  # fmt: skip
 
 

@@ -464,14 +464,15 @@ def test_backward_workspace_follows_the_launch_order(monkeypatch):
     tiny = dict(c2, total_q=600, total_k=600, max_seq_len_q=32, max_seq_len_k=32)
     tiny_pair = pair(rows=600, blocks=1)
     assert size(**tiny) == 0 and size(**dict(tiny, head_dim_qk=256, head_dim_v=256)) == 0
-    assert size(**dict(tiny, max_seq_len_q=40, max_seq_len_k=40)) == pair(rows=600, blocks=2)
+    assert size(**dict(tiny, max_seq_len_q=40, max_seq_len_k=40)) == 0  # (the kernel for few query rows, below)
+    assert size(**dict(tiny, max_seq_len_q=72, max_seq_len_k=72)) == pair(rows=600, blocks=3)
     assert size(**dict(tiny, q=fake + 8)) == tiny_pair
     assert size(grad_attn_bias=fake, **tiny) == tiny_pair
-    # ... and so do sequences of at most 64 query rows against keys of any length at head dims up to 64 with as many
+    # ... and so do sequences of at most 64 query rows against keys of any length at head dims up to 128 with as many
     # K/V heads as query heads
     few = dict(c2, total_q=1500, max_seq_len_q=64, head_dim_qk=64, head_dim_v=48, seq_offset_k=fake + 64)
-    assert size(**few) == 0
-    for other in (dict(max_seq_len_q=72), dict(head_dim_qk=72), dict(num_heads_k=2), dict(k=fake + 8)):
+    assert size(**few) == 0 and size(**dict(few, head_dim_qk=128, head_dim_v=96)) == 0
+    for other in (dict(max_seq_len_q=72), dict(head_dim_qk=136), dict(num_heads_k=2), dict(k=fake + 8)):
         assert size(**dict(few, **other)) > 0
     assert size(grad_attn_bias=fake, **few) > 0
     helpers.set_switch(monkeypatch, "HSTU_MI355_SHORT", "0")
