@@ -29,6 +29,7 @@ constexpr int kDqShortThreads = 256;  // threads of a workgroup of the backward'
 constexpr int kDqShortRows = 64;      // query rows of its tile
 constexpr int kFewRowsThreads = 256;  // threads of a workgroup of the backward kernel for sequences of few query rows
 constexpr int kFewRows = 64;          // the most query rows of a sequence that kernel takes
+constexpr int kFwdFewRowsThreads = 512;  // threads of a workgroup of the forward kernel for few query rows (eight wavefronts over row groups and keys)
 constexpr int kCounterBlockBytes = 16384;  // head of the workspace: device-side work counters (see the forward kernel)
 constexpr int kDkvThreads = 256;   // threads of a workgroup of the key-tile backward kernel
 constexpr int kGatherThreads = 128;

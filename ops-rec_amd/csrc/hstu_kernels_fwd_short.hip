@@ -4,6 +4,7 @@
 #include "hstu_bwd_dq_short_kernel.hip.h"
 #include "hstu_bwd_few_rows_kernel.hip.h"
 #include "hstu_bwd_tiny_kernel.hip.h"
+#include "hstu_fwd_few_rows_kernel.hip.h"
 #include "hstu_fwd_short_kernel.hip.h"
 #include "hstu_fwd_tiny_kernel.hip.h"
 #include "hstu_variants.h"
@@ -26,6 +27,14 @@ const ShortVariant kTiny[2][2] = {
 };
 }
 const ShortVariant (*fwd_variants_tiny())[2] { return kTiny; }
+
+namespace {
+const ShortVariant kFwdFewRows[2][2] = {
+    {{"hstu_fwd_bf16_d64_few_rows", hstu_fwd_few_rows_kernel<bf16_tag, 64>}, {"hstu_fwd_bf16_d128_few_rows", hstu_fwd_few_rows_kernel<bf16_tag, 128>}},
+    {{"hstu_fwd_f16_d64_few_rows", hstu_fwd_few_rows_kernel<f16_tag, 64>}, {"hstu_fwd_f16_d128_few_rows", hstu_fwd_few_rows_kernel<f16_tag, 128>}},
+};
+}
+const ShortVariant (*fwd_variants_few_rows())[2] { return kFwdFewRows; }
 
 namespace {
 const DqShortVariant kDqShort[2] = {

@@ -264,6 +264,48 @@ const hstu::ShortVariant* tiny_variant(const Variant* var, const hstu_jagged_fwd
     return &hstu::fwd_variants_tiny()[p->dtype == HSTU_DT_BF16 ? 0 : 1][var->d_pad == 128 ? 0 : 1];
 }
 
+// The kernel for small launches of sequences with few query rows (hstu_fwd_few_rows_kernel.hip.h): 16-bit inputs with head
+// dims up to 128 (q/k head dim a multiple of 8), no bias, no custom mask, no sequence of more than 64 query rows (keys:
+// any number), 16-byte aligned tensors, and at most one (sequence, head) item per compute unit -- a launch then lasts
+// as long as one item, whose keys the kernel deals over the wavefronts of a workgroup; with more items the persistent
+// kernel, which streams K and V at the rate of memory, is the faster one.  HSTU_MI355_SHORT=0 switches it off.
+const hstu::ShortVariant* few_rows_variant(const Variant* var, const hstu_jagged_fwd_params* p)
+{
+    const int64_t dmax = p->head_dim_qk > p->head_dim_v ? p->head_dim_qk : p->head_dim_v;
+    const uintptr_t ptrs = reinterpret_cast<uintptr_t>(p->q) | reinterpret_cast<uintptr_t>(p->k) | reinterpret_cast<uintptr_t>(p->v);
+    const int64_t span_k = p->max_seq_len_k * p->num_heads_k * dmax * 2;
+    if ((p->dtype != HSTU_DT_BF16 && p->dtype != HSTU_DT_FP16) || p->attn_bias != nullptr || p->mask_type == HSTU_MASK_CUSTOM ||
+        dmax > 128 || p->head_dim_qk % 8 != 0 || p->head_dim_v % 8 != 0 || ptrs % 16 != 0 || var->persistent_wgs_per_cu <= 0 ||
+        p->max_seq_len_q > hstu::kFewRows || span_k >= (1LL << 30) || switches().short_lists == 0) {
+        return nullptr;
+    }
+    int cus = 0;
+    if (compute_units(&cus) != HSTU_OK || (p->n_offsets - 1) * p->num_heads_q > cus) {
+        return nullptr;
+    }
+    // ... and few sub-tiles per wavefront: the row groups of an item each fetch the item's K and V, which the persistent
+    // kernel shares through LDS (and long items it splits over workgroups).  Measured, fp16, this kernel against that one:
+    // 16 x 4 heads, 32 rows x 499 keys, d 64 / 32: 10.7 / 14.4 us; 16 rows x 1000 keys: 10.9 / 20.0; 32 x 8 heads, 10 x 500:
+    // 8.7 / 14.4; 256 x 1 head, 52 x 1000: 24.0 / 29.5; 8 x 8 heads, d 128, 32 x 2000 (16 sub-tiles per wavefront): 40.6 /
+    // 37.9; 64 x 4 heads, d 64, 64 x 4096 (64 per wavefront): 87.2 / 61.7
+    const int64_t splits = p->max_seq_len_q <= 16 ? 8 : (p->max_seq_len_q <= 32 ? 4 : 2);
+    const int64_t per_wavefront = ((p->max_seq_len_k + 31) / 32 + splits - 1) / splits;
+    if (per_wavefront > (dmax <= 64 ? 16 : 8)) {
+        return nullptr;
+    }
+    return &hstu::fwd_variants_few_rows()[p->dtype == HSTU_DT_BF16 ? 0 : 1][dmax <= 64 ? 0 : 1];
+}
+// the kernels with one workgroup per (sequence, head) item: tiny sequences first, then few query rows
+const hstu::ShortVariant* one_item_variant(const Variant* var, const hstu_jagged_fwd_params* p, unsigned* threads)
+{
+    if (const hstu::ShortVariant* const tv = tiny_variant(var, p)) {
+        *threads = hstu::kTinyThreads;
+        return tv;
+    }
+    *threads = hstu::kFwdFewRowsThreads;
+    return few_rows_variant(var, p);
+}
+
 // The kernel for short work lists (hstu_fwd_short_kernel.hip.h) takes 16-bit inputs at the head-dim slot 128 without
 // bias or custom mask.  It is the faster one while the list -- at most n_blocks entries -- is a few items per
 // workgroup the persistent kernel would keep resident: there a launch lasts as long as its longest item, which the
@@ -276,7 +318,8 @@ const hstu::ShortVariant* short_variant(const Variant* var, const hstu_jagged_fw
         var->persistent_wgs_per_cu <= 0 || var->kernel_queues == nullptr) {
         return nullptr;
     }
-    if (tiny_variant(var, p) != nullptr) {
+    unsigned one_item_threads = 0;
+    if (one_item_variant(var, p, &one_item_threads) != nullptr) {
         return nullptr;
     }
     // (with a bias: rows of 8-byte pieces)
@@ -397,7 +440,8 @@ uint64_t split_workspace_bytes(const Variant* var, const hstu_jagged_fwd_params*
 // split items, nothing for the lists in between (fixed schedule, no device counters)
 uint64_t forward_workspace_bytes(const Variant* var, const hstu_jagged_fwd_params* p)
 {
-    if (short_variant(var, p) != nullptr || tiny_variant(var, p) != nullptr) {
+    unsigned one_item_threads = 0;
+    if (short_variant(var, p) != nullptr || one_item_variant(var, p, &one_item_threads) != nullptr) {
         return 0;
     }
     if (takes_queue_variant(var, p, nullptr)) {
@@ -1249,7 +1293,8 @@ HSTU_API const char* hstu_jagged_fwd_kernel_name(const hstu_jagged_fwd_params* p
         return nullptr;
     }
     // (given the workspace asked for; without a usable device the plain name is reported)
-    if (const hstu::ShortVariant* const tv = tiny_variant(v, params)) {
+    unsigned one_item_threads = 0;
+    if (const hstu::ShortVariant* const tv = one_item_variant(v, params, &one_item_threads)) {
         return tv->name;
     }
     if (const hstu::ShortVariant* const sv = short_variant(v, params)) {
@@ -1339,9 +1384,10 @@ int launch_forward(const hstu_jagged_fwd_params* p, const hstu_paged_fwd_params*
     if (n_blocks <= 0 || n_blocks > 0x7fffffffLL) {
         return fail(HSTU_ERR_INVALID, "grid of %lld workgroups is out of range", (long long)n_blocks);
     }
-    if (const hstu::ShortVariant* const tv = (paged == nullptr) ? tiny_variant(var, p) : nullptr) {
+    unsigned one_item_threads = 0;
+    if (const hstu::ShortVariant* const tv = (paged == nullptr) ? one_item_variant(var, p, &one_item_threads) : nullptr) {
         // one workgroup per (sequence, query head)
-        hipLaunchKernelGGL(tv->kernel, dim3(static_cast<unsigned>(a.bh)), dim3(hstu::kTinyThreads), 0, static_cast<hipStream_t>(stream), a);
+        hipLaunchKernelGGL(tv->kernel, dim3(static_cast<unsigned>(a.bh)), dim3(one_item_threads), 0, static_cast<hipStream_t>(stream), a);
         const hipError_t err_tiny = hipGetLastError();
         if (err_tiny != hipSuccess) {
             return fail(HSTU_ERR_RUNTIME, "launch of %s failed: %s", tv->name, hipGetErrorString(err_tiny));

@@ -79,6 +79,9 @@ const ShortVariant* fwd_variants_short();
 // forward for batches of sequences of at most 32 rows and keys (hstu_fwd_tiny_kernel.hip.h; one workgroup of
 // kTinyThreads per (sequence, head)), no bias, no custom mask: [bf16, fp16][head-dim slot 128, 256]
 const ShortVariant (*fwd_variants_tiny())[2];
+// forward for small launches of sequences of at most 64 query rows against keys of any length (hstu_fwd_few_rows_kernel.hip.h;
+// one workgroup of kFwdFewRowsThreads per (sequence, head)), no bias, no custom mask: [bf16, fp16][head-dim slot 64, 128]
+const ShortVariant (*fwd_variants_few_rows())[2];
 // forward, any head dims up to 512 (written for coverage, not speed): [bf16, fp16, fp32, fp8-e4m3 -> fp16, fp8-e4m3 -> bf16]
 const Variant* fwd_variants_generic();
 // backward: [rab][custom mask][dim slot: 64, 128, 256]
