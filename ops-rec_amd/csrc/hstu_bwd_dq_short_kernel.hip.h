@@ -31,11 +31,12 @@ constexpr int kDqShortWavesPerSimd = 3;
 // K sub-tile in LDS, read plainly (A operand of S^T: 16 consecutive rows, one 16-byte chunk each) and transposed (A
 // operand of dQ^T: rows 4 g .. 4 g + 3 of two neighbouring groups, 32 bytes each): the XOR term is a bijection of the
 // low four row bits (the plain read hits 16 different chunks) whose upper three bits tell rows 0..7 apart (the eight
-// 32-byte pieces of a transposed read fall into different bank groups).  Adding 16 to the row leaves it alone.
+// 32-byte pieces of a transposed read fall into different bank groups).  Adding 16 to the row leaves it alone.  (Rows of
+// 256 elements: the same term over each half of the row's 32 chunks.)
 template <int D>
 __device__ __forceinline__ int both_ways16_swizzle(int row, int chunk)
 {
-    static_assert(D == 128, "built for the head-dim slot 128");
+    static_assert(D == 128 || D == 256, "16 or 32 chunks of 16 bytes per row");
     return chunk ^ (((row & 7) << 1) | ((row >> 3) & 1));
 }
 

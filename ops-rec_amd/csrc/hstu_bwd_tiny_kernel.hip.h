@@ -19,13 +19,6 @@
 
 namespace hstu {
 
-template <int D>
-__device__ __forceinline__ int both_ways16_wide_swizzle(int row, int chunk)
-{
-    static_assert(D >= 128, "16 or more 16-byte chunks per row");
-    return chunk ^ (((row & 7) << 1) | ((row >> 3) & 1));
-}
-
 template <typename Tag, int D>
 __global__ __launch_bounds__(kTinyThreads, 1) void hstu_bwd_tiny_kernel(const BwdArgs a)
 {
@@ -80,7 +73,7 @@ __global__ __launch_bounds__(kTinyThreads, 1) void hstu_bwd_tiny_kernel(const Bw
             const int instr = 2 * i + wave;
             const int piece = instr * 64 + lane;
             const int r = piece / CPR;
-            const int cs = both_ways16_wide_swizzle<D>(r, piece % CPR);
+            const int cs = both_ways16_swizzle<D>(r, piece % CPR);
             const uint32_t src = (cs * 8 < dims) ? static_cast<uint32_t>(r) * stride + cs * 16u : kOutOfRange;
             request_to_lds_b128(rsrc, lds_address(tile) + instr * 1024u, src);
         }
@@ -93,12 +86,12 @@ __global__ __launch_bounds__(kTinyThreads, 1) void hstu_bwd_tiny_kernel(const Bw
     int n_lane_off[KSTEPS];
 #pragma unroll
     for (int js = 0; js < KSTEPS; ++js) {
-        n_lane_off[js] = n * D + both_ways16_wide_swizzle<D>(n, 4 * js + g) * 8;
+        n_lane_off[js] = n * D + both_ways16_swizzle<D>(n, 4 * js + g) * 8;
     }
     const int vr = 4 * g + (n >> 2);
     const int t_row_off = vr * D + 4 * (n & 1);
     const int t_chunk_lo = (n & 3) >> 1;
-    auto t_lane_off = [&](int mt) -> int { return t_row_off + both_ways16_wide_swizzle<D>(vr, 2 * mt + t_chunk_lo) * 8; };
+    auto t_lane_off = [&](int mt) -> int { return t_row_off + both_ways16_swizzle<D>(vr, 2 * mt + t_chunk_lo) * 8; };
     auto read_t = [&](const uint16_t* tile, int mt) -> u32x4_t {
         const uint16_t* const p = tile + t_lane_off(mt);
         const u32x2_t lo = lds_read_tr16_b64(p);
