@@ -426,10 +426,42 @@ def _new_workspace(n_bytes: int, device) -> Optional[torch.Tensor]:
         return None
 
 
+def _launch_backward(p, ws_bytes: int, device) -> None:
+    ws = _new_workspace(ws_bytes, device)
+    stream = torch.cuda.current_stream(device).cuda_stream
+    rc = _native.load().hstu_jagged_bwd(ctypes.byref(p), _ptr(ws), ws.numel() if ws is not None else 0, ctypes.c_void_p(stream))
+    if rc != _native.HSTU_OK:
+        raise RuntimeError(f"hstu_jagged_bwd failed ({rc}): {_native.last_error()}")
+
+
+def _backward_from_plan(plan, grad, q, k, v, mask, attn_bias, seq_offset, seq_offset_k, num_context, num_target):
+    """A cached backward description applied to new tensors (all contiguous and of the index type already: a description
+    is only cached when nothing had to be copied or converted)."""
+    template, ws_bytes, use_mask = plan
+    p = _native.BwdParams.from_buffer_copy(template)
+    dq, dk, dv = _new_grad(q), _new_grad(k), _new_grad(v)
+    dbias = _new_grad(attn_bias) if attn_bias is not None else None
+    f = p.fwd
+    f.q, f.k, f.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
+    f.mask, f.attn_bias = _ptr(mask if use_mask else None), _ptr(attn_bias)
+    f.seq_offset_q, f.seq_offset_k = seq_offset.data_ptr(), seq_offset_k.data_ptr()
+    f.num_context, f.num_target = _ptr(num_context), _ptr(num_target)
+    p.grad, p.grad_q, p.grad_k, p.grad_v, p.grad_attn_bias = grad.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), _ptr(dbias)
+    _launch_backward(p, ws_bytes, q.device)
+    return dq, dk, dv, dbias
+
+
 def _backward_hip(grad, q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max_seq_len_k, silu_scale, seq_offset,
                   seq_offset_k, num_context, num_target, group, alpha):  # fmt: skip
-    """The backward through the C ABI (``hstu_jagged_bwd``): two or three kernels on the current stream, the latter
-    with the workspace the library asks for (dS handed from the query-tile kernel to the dK workgroups)."""
+    """The backward through the C ABI (``hstu_jagged_bwd``): one to four kernels on the current stream, with the
+    workspace the library asks for (dS, or dS and P, handed from the query-tile kernel to the key-tile workgroups).
+    Validated calls are cached like the forward's, by everything but the addresses."""
+    key = ("bwd", _meta(grad), _meta(q), _meta(k), _meta(v), _meta(mask), _meta(attn_bias), mask_type, max_seq_len_q,
+           max_seq_len_k, silu_scale, _meta(seq_offset), seq_offset_k is seq_offset or _meta(seq_offset_k),
+           _meta(num_context), _meta(num_target), group, alpha)  # fmt: skip
+    plan = _PLAN_CACHE.get(key)
+    if plan is not None:
+        return _backward_from_plan(plan, grad, q, k, v, mask, attn_bias, seq_offset, seq_offset_k, num_context, num_target)
     _check(q.device.type == "cuda", f"q must be a GPU tensor, but it is on {q.device}")
     _check_devices(q.device, (("grad", grad), ("k", k), ("v", v), ("mask", mask), ("attn_bias", attn_bias),
                               ("seq_offset", seq_offset), ("seq_offset_k", seq_offset_k), ("num_context", num_context),
@@ -481,11 +513,15 @@ def _backward_hip(grad, q, k, v, mask, attn_bias, mask_type, max_seq_len_q, max_
     rc = lib.hstu_jagged_bwd_workspace_size(ctypes.byref(p), ctypes.byref(ws_bytes))
     if rc != _native.HSTU_OK:
         raise RuntimeError(f"hstu_jagged_bwd_workspace_size failed ({rc}): {_native.last_error()}")
-    ws = _new_workspace(ws_bytes.value, q_c.device)
-    stream = torch.cuda.current_stream(q_c.device).cuda_stream
-    rc = lib.hstu_jagged_bwd(ctypes.byref(p), _ptr(ws), ws.numel() if ws is not None else 0, ctypes.c_void_p(stream))
-    if rc != _native.HSTU_OK:
-        raise RuntimeError(f"hstu_jagged_bwd failed ({rc}): {_native.last_error()}")
+    _launch_backward(p, ws_bytes.value, q_c.device)
+    # (cached when every tensor was taken as it came: the next call with this description only patches addresses in)
+    same = (q_c is q and k_c is k and v_c is v and g_c is grad and offs_q is seq_offset and
+            (offs_k is seq_offset_k or seq_offset_k is seq_offset) and ctx is num_context and tgt is num_target and
+            bias is attn_bias and (mask_c is None or mask_c is mask))  # fmt: skip
+    if same:
+        if len(_PLAN_CACHE) >= _PLAN_CACHE_MAX:
+            _PLAN_CACHE.clear()
+        _PLAN_CACHE[key] = (bytes(p), ws_bytes.value, mask_c is not None)
     return dq, dk, dv, dbias
 
 
