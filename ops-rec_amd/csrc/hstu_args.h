@@ -23,8 +23,8 @@ constexpr int fwd_wgs_per_cu(int d, bool rab, bool mask)
     return (!rab && !mask && d <= 64) ? (d <= 32 ? 4 : 3) : (d <= 32 && !(rab && mask)) ? 3 : (d <= 128 ? 2 : 1);
 }
 constexpr int kShortThreads = 512;  // threads of a workgroup of the forward kernel for short lists (eight wavefronts of 16 query rows)
-constexpr int kTinyThreads = 128;   // threads of a workgroup of the forward kernel for tiny sequences (two wavefronts of 16 query rows)
-constexpr int kTinyRows = 32;       // the longest sequence (rows and keys) that kernel takes
+constexpr int kTinyThreads = 128;   // threads of a workgroup of the backward kernel for tiny sequences (two wavefronts of 16 query rows)
+constexpr int kTinyRows = 32;       // the longest sequence (rows and keys) that kernel takes; the forward one: 32 or 64, four threads per row
 constexpr int kDqShortThreads = 256;  // threads of a workgroup of the backward's query-tile kernel for short rows (four wavefronts of 16 rows)
 constexpr int kDqShortRows = 64;      // query rows of its tile
 constexpr int kFewRowsThreads = 256;  // threads of a workgroup of the backward kernel for sequences of few query rows

@@ -21,12 +21,17 @@ const ShortVariant kTable[4] = {
 const ShortVariant* fwd_variants_short() { return kTable; }
 
 namespace {
-const ShortVariant kTiny[2][2] = {
-    {{"hstu_fwd_bf16_d128_tiny", hstu_fwd_tiny_kernel<bf16_tag, 128>}, {"hstu_fwd_bf16_d256_tiny", hstu_fwd_tiny_kernel<bf16_tag, 256>}},
-    {{"hstu_fwd_f16_d128_tiny", hstu_fwd_tiny_kernel<f16_tag, 128>}, {"hstu_fwd_f16_d256_tiny", hstu_fwd_tiny_kernel<f16_tag, 256>}},
+#define HSTU_TINY(tag, tagname, D, R) {"hstu_fwd_" tagname "_d" #D "_tiny" #R, hstu_fwd_tiny_kernel<tag, D, R>}
+const ShortVariant kTiny[2][3][2] = {
+    {{HSTU_TINY(bf16_tag, "bf16", 64, 32), HSTU_TINY(bf16_tag, "bf16", 64, 64)},
+     {HSTU_TINY(bf16_tag, "bf16", 128, 32), HSTU_TINY(bf16_tag, "bf16", 128, 64)},
+     {HSTU_TINY(bf16_tag, "bf16", 256, 32), HSTU_TINY(bf16_tag, "bf16", 256, 64)}},
+    {{HSTU_TINY(f16_tag, "f16", 64, 32), HSTU_TINY(f16_tag, "f16", 64, 64)},
+     {HSTU_TINY(f16_tag, "f16", 128, 32), HSTU_TINY(f16_tag, "f16", 128, 64)},
+     {HSTU_TINY(f16_tag, "f16", 256, 32), HSTU_TINY(f16_tag, "f16", 256, 64)}},
 };
 }
-const ShortVariant (*fwd_variants_tiny())[2] { return kTiny; }
+const ShortVariant (*fwd_variants_tiny())[3][2] { return kTiny; }
 
 namespace {
 const ShortVariant kFwdFewRows[2][2] = {

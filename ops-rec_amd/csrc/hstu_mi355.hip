@@ -250,18 +250,23 @@ const Variant* select(const hstu_jagged_fwd_params* p)
     return &table[p->attn_bias != nullptr ? 1 : 0][p->mask_type == HSTU_MASK_CUSTOM ? 1 : 0][slot];
 }
 
-// The kernel for batches of tiny sequences (hstu_fwd_tiny_kernel.hip.h): 16-bit inputs at the head-dim slots 128 and 256
-// without bias or custom mask, no sequence longer than 32 rows or keys.  Batch 2048 x 2 heads x 32 rows at head dim 256:
-// 135 us on the persistent kernel (a 128-row workgroup and its start-up per item).  HSTU_MI355_SHORT=0 switches it off with
-// the kernel for short lists.
-const hstu::ShortVariant* tiny_variant(const Variant* var, const hstu_jagged_fwd_params* p)
+// The kernel for batches of tiny sequences (hstu_fwd_tiny_kernel.hip.h): 16-bit inputs with head dims up to 256 (q/k head
+// dim a multiple of 8) without bias or custom mask, no sequence longer than 64 rows or keys, 16-byte aligned tensors.
+// Batch 2048 x 2 heads x 32 rows at head dim 256: 135 us on the persistent kernel (a 128-row workgroup and its start-up
+// per item); batch 2048 x 4 heads x 48 rows at head dim 64: 118 us.  HSTU_MI355_SHORT=0 switches it off with the kernel
+// for short lists.
+const hstu::ShortVariant* tiny_variant(const Variant* var, const hstu_jagged_fwd_params* p, unsigned* threads)
 {
+    const int64_t dmax = p->head_dim_qk > p->head_dim_v ? p->head_dim_qk : p->head_dim_v;
+    const uintptr_t ptrs = reinterpret_cast<uintptr_t>(p->q) | reinterpret_cast<uintptr_t>(p->k) | reinterpret_cast<uintptr_t>(p->v);
     if ((p->dtype != HSTU_DT_BF16 && p->dtype != HSTU_DT_FP16) || p->attn_bias != nullptr || p->mask_type == HSTU_MASK_CUSTOM ||
-        (var->d_pad != 128 && var->d_pad != 256) || var->persistent_wgs_per_cu <= 0 || p->max_seq_len_q > hstu::kTinyRows ||
-        p->max_seq_len_k > hstu::kTinyRows || switches().short_lists == 0) {
+        dmax > 256 || p->head_dim_qk % 8 != 0 || p->head_dim_v % 8 != 0 || ptrs % 16 != 0 || var->persistent_wgs_per_cu <= 0 ||
+        p->max_seq_len_q > 64 || p->max_seq_len_k > 64 || switches().short_lists == 0) {
         return nullptr;
     }
-    return &hstu::fwd_variants_tiny()[p->dtype == HSTU_DT_BF16 ? 0 : 1][var->d_pad == 128 ? 0 : 1];
+    const int rows64 = (p->max_seq_len_q > 32 || p->max_seq_len_k > 32) ? 1 : 0;
+    *threads = rows64 ? 256u : 128u;
+    return &hstu::fwd_variants_tiny()[p->dtype == HSTU_DT_BF16 ? 0 : 1][dmax <= 64 ? 0 : (dmax <= 128 ? 1 : 2)][rows64];
 }
 
 // The kernel for small launches of sequences with few query rows (hstu_fwd_few_rows_kernel.hip.h): 16-bit inputs with head
@@ -298,8 +303,7 @@ const hstu::ShortVariant* few_rows_variant(const Variant* var, const hstu_jagged
 // the kernels with one workgroup per (sequence, head) item: tiny sequences first, then few query rows
 const hstu::ShortVariant* one_item_variant(const Variant* var, const hstu_jagged_fwd_params* p, unsigned* threads)
 {
-    if (const hstu::ShortVariant* const tv = tiny_variant(var, p)) {
-        *threads = hstu::kTinyThreads;
+    if (const hstu::ShortVariant* const tv = tiny_variant(var, p, threads)) {
         return tv;
     }
     *threads = hstu::kFwdFewRowsThreads;

@@ -76,9 +76,9 @@ const Variant (*fwd_variants_wide())[2][2];
 // forward for short work lists, 16-bit inputs at the head-dim slot 128 without custom mask: [bf16, fp16, bf16 with
 // attn_bias, fp16 with attn_bias]
 const ShortVariant* fwd_variants_short();
-// forward for batches of sequences of at most 32 rows and keys (hstu_fwd_tiny_kernel.hip.h; one workgroup of
-// kTinyThreads per (sequence, head)), no bias, no custom mask: [bf16, fp16][head-dim slot 128, 256]
-const ShortVariant (*fwd_variants_tiny())[2];
+// forward for batches of sequences of at most 32 or 64 rows and keys (hstu_fwd_tiny_kernel.hip.h; one workgroup of four
+// threads per row per (sequence, head)), no bias, no custom mask: [bf16, fp16][head-dim slot 64, 128, 256][32, 64 rows]
+const ShortVariant (*fwd_variants_tiny())[3][2];
 // forward for small launches of sequences of at most 64 query rows against keys of any length (hstu_fwd_few_rows_kernel.hip.h;
 // one workgroup of kFwdFewRowsThreads per (sequence, head)), no bias, no custom mask: [bf16, fp16][head-dim slot 64, 128]
 const ShortVariant (*fwd_variants_few_rows())[2];

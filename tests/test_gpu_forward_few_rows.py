@@ -1,6 +1,7 @@
 """The forward kernel for small launches of sequences with few query rows (hstu_fwd_few_rows_kernel.hip.h: one workgroup per
 (sequence, head) whose eight wavefronts are dealt over the 16-row groups and over the keys; taken when no sequence has more
-than 64 query rows, head dims are at most 128 and there is at most one item per compute unit): against the CPU oracle, and
+than 64 query rows, some sequence has more than 64 keys (else the kernel for tiny sequences runs), head dims are at most 128
+and there is at most one item per compute unit): against the CPU oracle, and
 against the persistent kernel on the same inputs (HSTU_MI355_SHORT=0).
 """
 
@@ -40,10 +41,10 @@ def kernel_name(w):
     return p.kernel_name()
 
 
-def check(w, monkeypatch, dtype):
+def check(w, monkeypatch, dtype, kernel="_few_rows"):
     helpers.set_switch(monkeypatch, "HSTU_MI355_SHORT", None)
     wd = w.to(DEV)
-    assert kernel_name(wd).endswith("_few_rows"), kernel_name(wd)
+    assert kernel_name(wd).endswith(kernel), kernel_name(wd)
     got = run(wd).float().cpu()
     assert torch.equal(run(wd).float().cpu(), got)  # the partial outputs are added in a fixed order
     ref = O.hstu_jagged_forward(w.q, w.k, w.v, out_dtype=torch.float32, **w.oracle_kwargs())
@@ -51,7 +52,7 @@ def check(w, monkeypatch, dtype):
     lo = O.hstu_jagged_forward(w.q, w.k, w.v, out_dtype=dtype, emulate_lowp=dtype, **w.oracle_kwargs()).float()
     assert O.mismatch_fraction(got, lo, 5e-3) < 5e-3
     helpers.set_switch(monkeypatch, "HSTU_MI355_SHORT", "0")
-    assert "_few_rows" not in kernel_name(wd)
+    assert not kernel_name(wd).endswith(kernel)
     torch.testing.assert_close(run(wd).float().cpu(), got, atol=1e-2, rtol=1e-2)
     helpers.set_switch(monkeypatch, "HSTU_MI355_SHORT", None)
 
@@ -61,7 +62,7 @@ CASES = {
     "one_row_group": dict(lq=[7, 16, 1, 12], lk=[300, 1000, 33, 257]),
     "two_row_groups": dict(lq=[17, 32, 20], lk=[300, 64, 700]),
     "three_and_four_row_groups": dict(lq=[33, 48, 49, 64, 40], lk=[519, 48, 1001, 64, 130]),
-    "fewer_keys_than_rows": dict(lq=[40, 64, 10, 33], lk=[12, 40, 10, 1]),
+    "fewer_keys_than_rows": dict(lq=[40, 64, 10, 33, 20], lk=[12, 40, 10, 1, 70]),
     "sequences_without_rows_or_keys": dict(lq=[0, 30, 5, 0, 64, 9], lk=[40, 0, 77, 0, 200, 9]),
     "dims_32_16": dict(lq=[52, 3, 64, 17], lk=[499, 130, 64, 401], dim=32, dim_v=16),
     "dims_8_64": dict(lq=[52, 3, 64, 17], lk=[499, 130, 64, 401], dim=8, dim_v=64),
@@ -92,14 +93,15 @@ def test_few_query_rows_context_rows_and_targets(monkeypatch):
             check(w, monkeypatch, torch.bfloat16)
 
 
-def test_few_query_rows_over_equal_offsets_and_rows_past_the_last_offset(monkeypatch):
-    w = workloads.make("self", batch=30, heads=2, dim=64, lo=0, hi=64, max_seq_len=64, dtype=torch.bfloat16, std=0.5, seed=3)
+def test_few_query_rows_and_rows_past_the_last_offset(monkeypatch):
+    w = case([7, 0, 64, 31], [100, 40, 64, 500])
     check(w, monkeypatch, torch.bfloat16)
     extra = 9
     pad = lambda t: torch.cat([t, torch.full((extra, *t.shape[1:]), 3.0, dtype=t.dtype)])  # noqa: E731
     wd = workloads.Workload(**{**w.__dict__})
     wd.q, wd.k, wd.v = pad(w.q), pad(w.k), pad(w.v)
     wd.seq_offset = torch.cat([w.seq_offset, w.seq_offset[-1:]])
+    wd.seq_offset_k = torch.cat([w.seq_offset_k, w.seq_offset_k[-1:]])
     wd = wd.to(DEV)
     assert kernel_name(wd).endswith("_few_rows")
     got = run(wd).float().cpu()
@@ -116,7 +118,7 @@ def test_the_hosts_rule_for_few_query_rows(monkeypatch):
     assert kernel_name(case([30] * 8, [200] * 8, dim=96).to(DEV)).endswith("_d128_few_rows")
     assert "_few_rows" not in kernel_name(case([65] + [30] * 7, [200] * 8).to(DEV))  # 65 query rows
     assert "_few_rows" not in kernel_name(case([30] * 8, [200] * 8, dim=136, dim_v=144).to(DEV))  # head dims above 128
-    many = case([8] * (cus // 2 + 1), [40] * (cus // 2 + 1), heads=2).to(DEV)  # more items than compute units
+    many = case([8] * (cus // 2 + 1), [100] * (cus // 2 + 1), heads=2).to(DEV)  # more items than compute units
     assert "_few_rows" not in kernel_name(many)
     assert "_few_rows" not in kernel_name(case([30] * 8, [2100] * 8).to(DEV))  # 17 sub-tiles per wavefront
     assert kernel_name(case([16] * 8, [4096] * 8).to(DEV)).endswith("_few_rows")  # 16 rows: eight wavefronts over the keys

@@ -105,6 +105,15 @@ TINY_CASES = {
     "padded_head_dims": dict(batch=9, heads=2, dim=208, dim_v=144, lo=1, hi=30),
     "padded_head_dims_128": dict(batch=9, heads=2, dim=80, dim_v=112, lo=1, hi=30),
     "int64_offsets": dict(batch=7, heads=1, dim=256, lo=5, hi=20, index_dtype=torch.int64),
+    "dim64": dict(batch=40, heads=3, dim=64, lo=1, hi=32),
+    "dims_8_16": dict(batch=12, heads=2, dim=8, dim_v=16, lo=1, hi=30),
+    "up_to_64_rows_dim64": dict(batch=40, heads=2, dim=64, lo=1, hi=64),
+    "up_to_64_rows_dim128": dict(batch=30, heads=2, dim=128, lo=20, hi=64),
+    "up_to_64_rows_dim256": dict(batch=20, heads=2, dim=256, lo=33, hi=64),
+    "all_64_rows": dict(batch=9, heads=3, dim=128, lo=64, hi=64),
+    "64_rows_context_targets_groups": dict(batch=12, heads=2, dim=64, dim_v=48, lo=24, hi=64, ctx=5, max_target=20, group=3),
+    "64_rows_grouped_heads_more_keys": dict(batch=10, heads=4, heads_k=2, dim=128, lo=1, hi=55, delta=True),
+    "64_rows_padded_head_dims": dict(batch=9, heads=2, dim=208, dim_v=144, lo=1, hi=60),
 }
 
 
@@ -119,7 +128,8 @@ def test_tiny_sequences_against_the_oracle(name, dtype, monkeypatch):
         if seed == 1 and "ctx" not in TINY_CASES[name]:
             w.mask_type = 2  # every key visible
         wd = w.to(DEV)
-        assert kernel_name(wd).endswith("_tiny"), kernel_name(wd)
+        longest = max(wd.max_seq_len, wd.max_seq_len_k or 0)
+        assert kernel_name(wd).endswith("_tiny32" if longest <= 32 else "_tiny64"), kernel_name(wd)
         got = run(wd).float().cpu()
         ref = O.hstu_jagged_forward(w.q, w.k, w.v, out_dtype=torch.float32, **w.oracle_kwargs())
         torch.testing.assert_close(got, ref, atol=1e-2, rtol=1e-2)
@@ -140,14 +150,16 @@ def test_tiny_sequences_gaps_and_rows_past_the_last_offset():
     wd.q, wd.k, wd.v = pad(w.q), pad(w.k), pad(w.v)
     wd.seq_offset = torch.cat([w.seq_offset, w.seq_offset[-1:]])
     wd = wd.to(DEV)
-    assert kernel_name(wd).endswith("_d256_tiny")
+    assert kernel_name(wd).endswith("_d256_tiny32")
     got = run(wd).float().cpu()
     ref = O.hstu_jagged_forward(w.q, w.k, w.v, out_dtype=torch.float32, **w.oracle_kwargs())
     torch.testing.assert_close(got[: ref.shape[0]], ref, atol=1e-2, rtol=1e-2)
     assert (got[ref.shape[0] :] == 0).all()
-    # one more key than the kernel takes: the other kernels
+    # one more key than the kernel for 32 rows takes: the one for 64; one more than that takes: the other kernels
     w33 = workloads.make("n", batch=4, heads=2, dim=256, lo=1, hi=33, dtype=torch.bfloat16, max_seq_len=33, device=DEV)
-    assert "_tiny" not in kernel_name(w33)
+    assert kernel_name(w33).endswith("_d256_tiny64")
+    w65 = workloads.make("n", batch=4, heads=2, dim=256, lo=1, hi=65, dtype=torch.bfloat16, max_seq_len=65, device=DEV)
+    assert "_tiny" not in kernel_name(w65)
 
 
 def test_attn_bias_rows_that_are_not_8_byte_pieces_stay_on_the_persistent_kernel(monkeypatch):
