@@ -294,10 +294,16 @@ def test_kernel_variant_selection():
         n = lib.hstu_jagged_fwd_kernel_name(ctypes.byref(p))
         return n.decode() if n else None
 
-    assert "_d32_" in name(head_dim_qk=16, head_dim_v=16)
-    assert "_d64_" in name(head_dim_qk=64, head_dim_v=48)
-    assert "_d128_" in name(head_dim_qk=64, head_dim_v=128)
-    assert "_d256_" in name(head_dim_qk=256, head_dim_v=256)
+    long = dict(max_seq_len_q=100, max_seq_len_k=100)
+    assert "_d32_" in name(head_dim_qk=16, head_dim_v=16, **long)
+    assert "_d64_" in name(head_dim_qk=64, head_dim_v=48, **long)
+    assert "_d128_" in name(head_dim_qk=64, head_dim_v=128, **long)
+    assert "_d256_" in name(head_dim_qk=256, head_dim_v=256, **long)
+    # sequences of at most 32 / 64 rows and keys: the kernel for tiny sequences, head-dim slots 64, 128, 256
+    assert name(head_dim_qk=16, head_dim_v=16) == "hstu_fwd_bf16_d64_tiny32"
+    assert name(head_dim_qk=64, head_dim_v=128, max_seq_len_q=33) == "hstu_fwd_bf16_d128_tiny64"
+    assert name(head_dim_qk=256, head_dim_v=256, max_seq_len_k=64) == "hstu_fwd_bf16_d256_tiny64"
+    assert "_tiny" not in name(max_seq_len_k=65) and "_tiny" not in name(q=0x1008)
     assert "rabtrue" in name(attn_bias=0x2000)
     assert "masktrue" in name(mask=0x2000, mask_type=3)
     assert "f16" in name(dtype=_native.DT_FP16, out_dtype=_native.DT_FP16)
