@@ -93,20 +93,25 @@ def test_linear_in_v(config):
 
 def test_zero_bias_equals_no_bias(config, monkeypatch):
     name, w, out = config
-    if name != "C2":
-        pytest.skip("covered at C2 size: the rab tensors of C3 / C4 are already in use")
-    # (bit for bit on one kernel: with a bias the call runs on the persistent kernel, without one a list of this shape
+    # (bit for bit on one kernel: with a bias the call runs on the persistent kernel, without one a list of C2's shape
     # would take the kernel for short lists, whose fp32 sums are taken in pieces of another size)
     helpers.set_switch(monkeypatch, "HSTU_MI355_SHORT", "0")
-    w2 = workloads.Workload(**{**w.__dict__})
-    w2.attn_bias = torch.zeros(len(w.lengths), w.q.shape[1], w.max_seq_len, w.max_seq_len, dtype=w.q.dtype, device=DEV)
-    assert torch.equal(launch(w2), launch(w))
+    bare = workloads.Workload(**{**w.__dict__})
+    bare.attn_bias = None
+    expected = launch(bare)
+    zeroed = workloads.Workload(**{**w.__dict__})
+    zeroed.attn_bias = torch.zeros(len(w.lengths), w.q.shape[1], w.max_seq_len, w.max_seq_len, dtype=w.q.dtype, device=DEV)
+    got = launch(zeroed)
+    del zeroed
+    torch.cuda.empty_cache()
+    assert torch.equal(got, expected)
+    if w.attn_bias is not None:
+        # and the configuration's own bias does change the rows (the comparison above is not between two calls that ignore it)
+        assert not torch.equal(out, expected)
 
 
 def test_sequence_permutation(config):
     name, w, out = config
-    if name == "C4":
-        pytest.skip("a permuted copy of the 4 GiB rab is not worth the memory; covered at C2 / C3 size")
     offs = w.seq_offset.cpu().tolist()
     order = list(reversed(range(len(w.lengths))))
     rows = torch.cat([torch.arange(offs[b], offs[b + 1]) for b in order]).to(DEV)
@@ -120,7 +125,10 @@ def test_sequence_permutation(config):
     w2.attn_bias = None if w.attn_bias is None else w.attn_bias[idx]
     w2.num_context = None if w.num_context is None else w.num_context[idx]
     w2.num_target = None if w.num_target is None else w.num_target[idx]
-    assert torch.equal(launch(w2), out[rows])
+    got = launch(w2)
+    del w2  # (C4: the permuted copy of the bias is 4 GiB)
+    torch.cuda.empty_cache()
+    assert torch.equal(got, out[rows])
 
 
 def test_flop_model_matches_expectation():
