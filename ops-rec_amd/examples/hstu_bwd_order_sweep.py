@@ -2,6 +2,8 @@
 times, the order the library's rule takes and how far that is from the best (markdown table on stdout).
 
     python ops-rec_amd/examples/hstu_bwd_order_sweep.py [--set heldout|fit|bias] [--launches 10]
+    python ops-rec_amd/examples/hstu_bwd_order_sweep.py --shape 1,4,4,128,1024,1024,causal --only planes   # one shape, one
+                                                        # order: what a kernel trace or a counter run of a launch order wants
 
 Orders (forced with HSTU_MI355_BWD_HANDOFF = 0 / 1 / 2, read once per process, hence ``reload_switches``):
   two     key-tile kernel (S, dP, dV, dK) + query-tile kernel (S, dP, dQ): 7 products, no workspace
@@ -77,6 +79,9 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--set", default="heldout", choices=["heldout", "fit", "bias"])
     ap.add_argument("--launches", type=int, default=10)
+    ap.add_argument("--shape", action="append", default=[],
+                    help="batch,heads,kv_heads,dim,shortest,longest,causal|none (repeatable); instead of --set")
+    ap.add_argument("--only", choices=sorted(NAMES.values()), help="run this launch order only and print its time")
     args = ap.parse_args()
     bwd = ops_rec.ascendc.attention.hstu_jagged_backward
     asked = []
@@ -86,6 +91,8 @@ def main():
     print("|---|---|---|---|---|---|")
     worst, within = 0.0, 0
     shapes = {"heldout": HELDOUT, "fit": FIT, "bias": BIAS}[args.set]
+    if args.shape:
+        shapes = [tuple(int(v) for v in t.split(",")[:6]) + (t.split(",")[6],) for t in args.shape]
     for batch, heads, heads_k, dim, lo, hi, mask in shapes:
         max_len = (hi + 7) // 8 * 8
         w = workloads.make("sweep", dtype=torch.bfloat16, device="cuda", batch=batch, heads=heads, heads_k=heads_k, dim=dim,
@@ -96,6 +103,12 @@ def main():
             rab = (torch.randn(batch, heads, max_len, max_len, device="cuda") * 0.1).to(torch.bfloat16)
         call = (grad, w.q, w.k, w.v, None, rab, 0 if mask == "causal" else 2, max_len, w.silu_scale, w.seq_offset, None, None, 0, w.alpha)
         times = {}
+        if args.only:
+            os.environ["HSTU_MI355_BWD_HANDOFF"] = {v: k for k, v in NAMES.items()}[args.only]
+            _native.reload_switches()
+            print(f"| {batch}, {heads} ({heads_k}), {dim}, {lo}..{hi}, {mask} | {args.only} only: "
+                  f"{time_us(lambda: bwd(*call), args.launches):.1f} us |", flush=True)  # fmt: skip
+            continue
         for order in ("0", "1", "2", None):
             if order is None:
                 os.environ.pop("HSTU_MI355_BWD_HANDOFF", None)
@@ -119,6 +132,8 @@ def main():
         worst, within = max(worst, ratio), within + (ratio <= 1.10)
         print(f"| {batch}, {heads} ({heads_k}), {dim}, {lo}..{hi}, {mask} | {times['0']:.1f} | {times['1']:.1f} | {times['2']:.1f} | "
               f"{pick} ({times[None]:.1f}) | {ratio:.2f} |", flush=True)  # fmt: skip
+    if args.only:
+        return
     print(f"\nrule within 10 % of the best order on {within} of {len(shapes)} shapes; worst {worst:.2f}x")
 
 
