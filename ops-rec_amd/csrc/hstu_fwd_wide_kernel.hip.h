@@ -3,16 +3,17 @@
 // The reference takes head dims up to 512 (ascendc/attention/hstu_v1/hstu_forward_v1/op_host/tiling_policy.cpp:68-93,
 // blockK up to 512 in op_host/atlas950/tiling_policy_arch.cpp:173-177).  The tuned kernel stops at 256: 128 output
 // registers per 32 rows, and two four-slot LDS rings of 16 KB sub-tiles.  This kernel carries the same arithmetic to
-// 512 on the matrix pipe with the plain structure of hstu_fwd_f32_kernel -- one workgroup per 128-row query tile,
-// one 32-key sub-tile of K and V in LDS at a time, load / barrier / products / barrier -- and the tuned kernel's
-// operand layouts: S^T = K . Q^T with v_mfma_f32_32x32x16 (the Q rows of a lane in 128 registers, K rows read from
+// 512 on the matrix pipe with a plain structure -- one workgroup per 128-row query tile and window of 256 output dims
+// (blockIdx.y: a head dim of v above 256 takes two workgroups per tile, each computing the scores for itself), 32-key
+// sub-tiles of K and V in two LDS stages, the next sub-tile on its way while the products of this one run -- and the
+// tuned kernel's operand layouts: S^T = K . Q^T with v_mfma_f32_32x32x16 (the Q rows of a lane in 128 registers, K rows read from
 // LDS 16 bytes at a time), P^T packed in registers as the B operand of O^T += V^T . P^T, V^T taken from the row-major
 // V sub-tile by transposed LDS reads.  LDS rows are padded instead of swizzled (K rows by 16 bytes: the 16 rows an
 // operand read takes together fall into different bank groups; V rows by 64 bytes: the four rows of a transposed read
 // likewise), so that every LDS address is one per-lane base plus a compile-time offset -- with 384 registers already
-// spoken for there is no room for a table of swizzled addresses.  A wavefront holds 256 output, 128 Q and 32 score registers: one wavefront
-// per SIMD, no overlap of loads with products -- a hundred times the rate of the vector-unit kernel this replaces for
-// these head dims, a fraction of the tuned kernel's.  Head dims are padded to 512 (chunks past the real dims read
+// spoken for there is no room for a table of swizzled addresses.  A wavefront holds 128 output, 128 Q and 32 score registers: one wavefront
+// per SIMD.  (With all 512 output dims in one wavefront -- 256 output registers -- the compiler kept 156 registers of Q
+// rows in scratch memory and a sub-tile's loads were waited for in the open: 89 .. 121 TFLOP/s.)  Head dims are padded to 512 (chunks past the real dims read
 // as zeros); a q/k head dim that is not a multiple of 8 stays with the generic kernel.
 #pragma once
 #include "hstu_fwd_kernel.hip.h"
@@ -33,8 +34,14 @@ __global__ __launch_bounds__(256, 1) void hstu_fwd_wide_kernel(const FwdArgs a)
     constexpr int KSTEPS = D / 16;
     constexpr int MTILES = D / 32;
 
-    __shared__ __attribute__((aligned(16))) uint16_t s_k[BN * K_ROW];
-    __shared__ __attribute__((aligned(16))) uint16_t s_v[BN * V_ROW];
+    constexpr int OW = 256;             // output dims per workgroup
+    constexpr int MT_O = OW / 32;
+    // two stages (separate arrays, so that the compiler can tell the one being filled from the one being read); a V row
+    // keeps the pitch of 512 dims, of which the window's 256 are filled
+    __shared__ __attribute__((aligned(16))) uint16_t s_k0[BN * K_ROW];
+    __shared__ __attribute__((aligned(16))) uint16_t s_k1[BN * K_ROW];
+    __shared__ __attribute__((aligned(16))) uint16_t s_v0[BN * V_ROW];
+    __shared__ __attribute__((aligned(16))) uint16_t s_v1[BN * V_ROW];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -48,6 +55,7 @@ __global__ __launch_bounds__(256, 1) void hstu_fwd_wide_kernel(const FwdArgs a)
     const int b = bhid / a.n_heads_q;
     const int h = bhid - b * a.n_heads_q;
     const int hk = h / a.head_ratio;
+    const int ow0 = static_cast<int>(blockIdx.y) * OW;  // first output dim of this workgroup
 
     int64_t q0 = load_index(a.offs_q, b, a.idx64);
     int64_t q1 = load_index(a.offs_q, b + 1, a.idx64);
@@ -63,7 +71,7 @@ __global__ __launch_bounds__(256, 1) void hstu_fwd_wide_kernel(const FwdArgs a)
     sk = uniform(sk < a.max_k ? sk : a.max_k);
 
     uint16_t* const out16 = static_cast<uint16_t*>(a.out);
-    if (qt == 0) {  // rows past the last offset belong to no sequence: zero-fill them
+    if (qt == 0 && ow0 == 0) {  // rows past the last offset belong to no sequence: zero-fill them
         const int64_t last = load_index(a.offs_q, a.n_batch, a.idx64);
         const int64_t first_tail = last < 0 ? 0 : last;
         const int64_t row_elems = static_cast<int64_t>(a.n_heads_q) * a.d_v;
@@ -165,11 +173,12 @@ __global__ __launch_bounds__(256, 1) void hstu_fwd_wide_kernel(const FwdArgs a)
 
     // load instruction i of this wavefront fills row wave * LPW + i of a tile: lane l brings the 16-byte chunk l
     const uint32_t k_lane_src = (lane * 8 < a.d_qk) ? static_cast<uint32_t>(lane) * 16u : kOutOfRange;
-    const uint32_t v_lane_src = (lane * 8 < a.d_v) ? static_cast<uint32_t>(lane) * 16u : kOutOfRange;
+    const uint32_t v_lane_src =
+        (lane < OW / 8 && ow0 + lane * 8 < a.d_v) ? static_cast<uint32_t>(ow0 + lane * 8) * 2u : kOutOfRange;
     // per-lane bases of the operand reads: K row ln, chunk lh (+ 2 js chunks per MFMA step); V rows vr0 (+ 8, + 16 j2),
     // dims 16 ((lane / 16) % 2) + 4 (lane % 4) (+ 32 mt)
-    const uint16_t* const k_read = s_k + ln * K_ROW + 8 * lh;
-    const uint16_t* const v_read = s_v + (4 * lh + ((lane & 15) >> 2)) * V_ROW + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+    const int k_read_off = ln * K_ROW + 8 * lh;
+    const int v_read_off = (4 * lh + ((lane & 15) >> 2)) * V_ROW + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
 
     const uint32_t bias_bytes = static_cast<uint32_t>(a.max_q) * static_cast<uint32_t>(a.max_k) * 2u;
     const int64_t bias_plane = (static_cast<int64_t>(b) * a.n_heads_q + h) * a.max_q * static_cast<int64_t>(a.max_k);
@@ -204,9 +213,9 @@ __global__ __launch_bounds__(256, 1) void hstu_fwd_wide_kernel(const FwdArgs a)
         }
     };
 
-    f32x16_t o_acc[MTILES];
+    f32x16_t o_acc[MT_O];
 #pragma unroll
-    for (int mt = 0; mt < MTILES; ++mt) {
+    for (int mt = 0; mt < MT_O; ++mt) {
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             o_acc[mt][i] = 0.f;
@@ -214,18 +223,26 @@ __global__ __launch_bounds__(256, 1) void hstu_fwd_wide_kernel(const FwdArgs a)
     }
     const float c_exp = a.c_exp;
 
-    for (int kt = 0; kt < n_kt; ++kt) {
+    // sub-tile kt into a stage (requests past the last sub-tile move nothing)
+    auto request = [&](uint16_t* sk_to, uint16_t* sv_to, int kt) {
+        const bool past = kt >= n_kt;
         const uint32_t kb = static_cast<uint32_t>(kt * BN) * k_stride;
         const uint32_t vb = static_cast<uint32_t>(kt * BN) * v_stride;
 #pragma unroll
         for (int i = 0; i < LPW; ++i) {
             const int r = wave * LPW + i;
-            load_to_lds_b128(k_rsrc, s_k + r * K_ROW, k_lane_src + kb + static_cast<uint32_t>(r) * k_stride);
-            load_to_lds_b128(v_rsrc, s_v + r * V_ROW, v_lane_src + vb + static_cast<uint32_t>(r) * v_stride);
+            load_to_lds_b128(k_rsrc, sk_to + r * K_ROW, past ? kOutOfRange : k_lane_src + kb + static_cast<uint32_t>(r) * k_stride);
+            load_to_lds_b128(v_rsrc, sv_to + r * V_ROW, past ? kOutOfRange : v_lane_src + vb + static_cast<uint32_t>(r) * v_stride);
         }
+    };
+    // one step: sub-tile kt has landed in (sk, sv) -- mine, then everybody's -- and everybody is done with the other stage,
+    // which the next sub-tile may now fill while the products of this one run
+    auto step = [&](const uint16_t* sk, const uint16_t* sv, uint16_t* sk_next, uint16_t* sv_next, int kt) {
         __builtin_amdgcn_s_waitcnt(0);
         __syncthreads();
-
+        request(sk_next, sv_next, kt + 1);
+        const uint16_t* const k_read = sk + k_read_off;
+        const uint16_t* const v_read = sv + v_read_off;
         const int c0 = kt * BN;
         if (c0 < wb.lim_max) {
             f32x16_t s;
@@ -251,9 +268,9 @@ __global__ __launch_bounds__(256, 1) void hstu_fwd_wide_kernel(const FwdArgs a)
                               !(wb.any_hole && c0 + 32 > hist_k && c0 < wb.hole_hi_max);
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                const float sv = s[i];
-                const float ex = __builtin_amdgcn_exp2f(sv * c_exp);
-                s[i] = sv * __builtin_amdgcn_rcpf(1.0f + ex);
+                const float sv_ = s[i];
+                const float ex = __builtin_amdgcn_exp2f(sv_ * c_exp);
+                s[i] = sv_ * __builtin_amdgcn_rcpf(1.0f + ex);
             }
             if (!full) {
                 f32x16_t mw;
@@ -276,9 +293,9 @@ __global__ __launch_bounds__(256, 1) void hstu_fwd_wide_kernel(const FwdArgs a)
             for (int i = 0; i < 8; ++i) {
                 pk[i] = pack2<Tag>(s[2 * i], s[2 * i + 1]);
             }
-            // O^T += V^T . P^T: chunk (mt, j2) contracts the 16 keys of half j2 into output tile mt
+            // O^T += V^T . P^T: chunk (mt, j2) contracts the 16 keys of half j2 into output tile mt of the window
 #pragma unroll
-            for (int mt = 0; mt < MTILES; ++mt) {
+            for (int mt = 0; mt < MT_O; ++mt) {
 #pragma unroll
                 for (int j2 = 0; j2 < 2; ++j2) {
                     const u32x2_t lo = lds_read_tr16_b64(v_read + 32 * mt + 16 * j2 * V_ROW);
@@ -290,18 +307,29 @@ __global__ __launch_bounds__(256, 1) void hstu_fwd_wide_kernel(const FwdArgs a)
                 __builtin_amdgcn_sched_barrier(0);
             }
         }
-        __syncthreads();
+    };
+    if (n_kt > 0) {
+        request(s_k0, s_v0, 0);
+        for (int kt = 0; kt < n_kt; kt += 2) {
+            step(s_k0, s_v0, s_k1, s_v1, kt);
+            if (kt + 1 >= n_kt) {
+                break;
+            }
+            step(s_k1, s_v1, s_k0, s_v0, kt + 1);
+        }
+        // (the request past the last sub-tile names a stage: it has moved nothing, and is waited for before the kernel ends)
+        __builtin_amdgcn_s_waitcnt(0);
     }
 
-    // store O: lane holds query row (wr0 + ln), dims 32 mt + 8 g + 4 lh + 0..3 (d_v is a multiple of 16)
+    // store O: lane holds query row (wr0 + ln), dims ow0 + 32 mt + 8 g + 4 lh + 0..3 (d_v is a multiple of 16)
     {
         const float c_out = a.c_out;
         const uint32_t row_off = static_cast<uint32_t>(wr0 + ln) * o_stride;
 #pragma unroll
-        for (int mt = 0; mt < MTILES; ++mt) {
+        for (int mt = 0; mt < MT_O; ++mt) {
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                const int d0 = 32 * mt + 8 * g + 4 * lh;
+                const int d0 = ow0 + 32 * mt + 8 * g + 4 * lh;
                 const uint32_t off = (d0 < a.d_v) ? row_off + d0 * 2u : kOutOfRange;
                 u32x2_t w;
                 w[0] = pack2<Tag>(o_acc[mt][4 * g + 0] * c_out, o_acc[mt][4 * g + 1] * c_out);

@@ -838,7 +838,13 @@ static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
         const bool fits = f->max_seq_len_q * row * 4 < (1LL << 31) && bytes <= cap * (1LL << 20);
         return fits ? BwdPlan{kPlanes, static_cast<uint64_t>(bytes)} : two;
     }
-    if (var->dk_from_ds == nullptr || f->max_seq_len_k % 8 != 0) {
+    // Rows of the [max_q][max_k] tensors -- attn_bias, custom mask, the attn_bias gradient, a dense dS plane -- start at
+    // multiples of 16 bytes only when max_seq_len_k is a multiple of 8: the kernels that read or write such rows 16 bytes
+    // per lane need that.  The pair plane has a layout of its own: a call with none of those tensors can take the planes
+    // order whatever max_seq_len_k is (max_seq_len 1004 instead of 1024 must not cost the two-launch order's 7 products).
+    const bool rows16 = f->max_seq_len_k % 8 == 0;
+    const bool no_bias_tensors = f->attn_bias == nullptr && f->mask == nullptr && p->grad_attn_bias == nullptr;
+    if (var->dk_from_ds == nullptr || (!rows16 && !no_bias_tensors)) {
         return two;
     }
     const int64_t batch = f->n_offsets - 1;
@@ -851,7 +857,7 @@ static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
     const int64_t cap = workspace_cap_mb() * (1LL << 20);
     // with an attn_bias gradient dS goes through the gradient itself in the three-launch order: no workspace
     const int64_t ds_plane = bias_grad ? 0 : batch * f->num_heads_q * f->max_seq_len_q * f->max_seq_len_k * 2;
-    const bool three_fits = ds_plane <= cap;
+    const bool three_fits = rows16 && ds_plane <= cap;
     const bool planes_fit = pp.fits_32 && pp.bytes <= cap && (!bias_grad || var->dv_dk_from_planes_drab != nullptr);
     const BwdPlan three = {kThreeLaunches, static_cast<uint64_t>(ds_plane)};
     const BwdPlan planes = {kPlanes, static_cast<uint64_t>(pp.bytes)};
@@ -978,8 +984,12 @@ static WindowPlan plan_windows(const hstu_jagged_bwd_params* p)
     const hstu_jagged_fwd_params* f = &p->fwd;
     const int64_t dmax = f->head_dim_qk > f->head_dim_v ? f->head_dim_qk : f->head_dim_v;
     if ((f->dtype != HSTU_DT_BF16 && f->dtype != HSTU_DT_FP16) || dmax <= 256 || dmax > 512 || f->head_dim_qk % 16 != 0 ||
-        f->head_dim_v % 16 != 0 || switches().generic_backward == 1 || f->total_q == 0 || f->total_k == 0 ||
-        f->max_seq_len_k % 8 != 0) {
+        f->head_dim_v % 16 != 0 || switches().generic_backward == 1 || f->total_q == 0 || f->total_k == 0) {
+        return w;
+    }
+    // (rows of attn_bias, custom mask and the gradient are read and written 16 bytes per lane: see plan_bwd)
+    const bool no_bias_tensors = f->attn_bias == nullptr && f->mask == nullptr && p->grad_attn_bias == nullptr;
+    if (f->max_seq_len_k % 8 != 0 && !no_bias_tensors) {
         return w;
     }
     // (16-byte rows of the planes and of the attn_bias tensors, spans behind 32-bit descriptors)
@@ -1183,7 +1193,8 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
                 hipLaunchKernelGGL(var->dq, dim3(static_cast<unsigned>(grid_q)), dim3(256), 0, static_cast<hipStream_t>(stream), a);
             }
         }
-    } else if (f->total_k > 0 && grid_kv > 0 && f->total_q > 0 && grid_q > 0 && a.bias_vec_ok == 2 && plan.order != kTwoLaunches &&
+    } else if (f->total_k > 0 && grid_kv > 0 && f->total_q > 0 && grid_q > 0 && plan.order != kTwoLaunches &&
+               (a.bias_vec_ok == 2 || (plan.order == kPlanes && f->attn_bias == nullptr && f->mask == nullptr && p->grad_attn_bias == nullptr)) &&
                (plan.workspace_bytes == 0 || (usable_workspace(workspace, workspace_bytes, plan.workspace_bytes) &&
                                               reinterpret_cast<uintptr_t>(workspace) % 16 == 0))) {
         if (p->grad_attn_bias == nullptr) {
@@ -1452,7 +1463,10 @@ int launch_forward(const hstu_jagged_fwd_params* p, const hstu_paged_fwd_params*
             launch_clear(a.counters, static_cast<int64_t>(kCounterBytes), stream);
         }
     }
-    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(n_blocks)), dim3(static_cast<unsigned>(var->threads)), 0,
+    // (the kernel for head dims above 256 takes a workgroup per window of 256 output dims)
+    const Variant* const wide0 = &hstu::fwd_variants_wide()[0][0][0];
+    const unsigned out_windows = (var >= wide0 && var < wide0 + 8 && p->head_dim_v > 256) ? 2u : 1u;
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(n_blocks), out_windows), dim3(static_cast<unsigned>(var->threads)), 0,
                        static_cast<hipStream_t>(stream), a);
     const hipError_t err = hipGetLastError();
     if (err != hipSuccess) {

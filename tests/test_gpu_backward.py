@@ -193,6 +193,34 @@ def test_ds_handed_to_the_dk_workgroups_through_a_workspace(kw, mask, monkeypatc
         assert all(torch.equal(x, y) for x, y in zip(two[:3], without[:3]))
 
 
+@pytest.mark.parametrize("kw", [
+    dict(dim=128, lo=200, hi=1004, max_seq_len=1004, heads=4), dict(dim=64, lo=1, hi=331, max_seq_len=331),
+    dict(dim=256, lo=100, hi=261, max_seq_len=261), dict(dim=512, lo=60, hi=301, max_seq_len=301),
+    dict(dim=384, dim_v=320, lo=1, hi=203, max_seq_len=203, heads=4, heads_k=2),
+], ids=lambda kw: "-".join(f"{k}{v}" for k, v in kw.items()))  # fmt: skip
+@pytest.mark.parametrize("mask_type", [0, 2], ids=["causal", "none"])
+def test_planes_with_a_max_seq_len_that_is_not_a_multiple_of_8(kw, mask_type, monkeypatch):
+    """The pair plane has a layout of its own, so a call without attn_bias, custom mask or attn_bias gradient takes the
+    planes order (and, above head dim 256, the two windows) whatever max_seq_len_k is: the library asks for the
+    workspace, and the gradients come out right with it full of NaN.  (Rows of [max_q][max_k] tensors start at multiples
+    of 16 bytes only when max_seq_len_k is a multiple of 8: with such a tensor in the call the same shapes run in two
+    launches, or on the generic kernels.)"""
+    from ops_rec import _ops
+
+    kw = dict(kw)
+    w = dataclasses.replace(make(batch=3, heads=kw.pop("heads", 2), seed=77, **kw), mask_type=mask_type)
+    asked = []
+    plain = _ops._new_workspace
+    monkeypatch.setattr(_ops, "_new_workspace", lambda n, dev: (asked.append(n), plain(n, dev))[1])
+    helpers.set_switch(monkeypatch, "HSTU_MI355_GENERIC_BACKWARD", "0")
+    helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", "2")
+    g = torch.Generator(device=DEV).manual_seed(6)
+    grad_out = torch.randn(w.q.shape[0], w.q.shape[1], w.v.shape[2], generator=g, device=DEV).to(w.q.dtype)
+    device_grads(w, grad_out)
+    assert asked and asked[-1] > 0  # the planes (and, for the windows, the partial scores)
+    check(w, monkeypatch)  # with the workspace full of NaN, against the oracle and the generic kernels
+
+
 def test_no_mask(monkeypatch):
     check(dataclasses.replace(make(batch=2, heads=2, dim=128, lo=100, hi=300, seed=9), mask_type=2), monkeypatch)
 

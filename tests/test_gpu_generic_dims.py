@@ -252,15 +252,21 @@ def test_backward_above_head_dim_256_as_two_windows(name, mask, dtype, monkeypat
     check_backward(w)
 
 
-def test_backward_windows_do_not_take_rows_that_are_not_16_byte_pieces(monkeypatch):
+def test_backward_windows_and_rows_that_are_not_16_byte_pieces(monkeypatch):
+    """Rows of [max_q][max_k] tensors are 16-byte pieces only when max_seq_len_k is a multiple of 8: a call with an
+    attn_bias at another max_seq_len_k stays on the generic kernels (no workspace), one without such tensors takes the
+    windows all the same; a head dim that is not a multiple of 16 stays on the generic kernels either way."""
     from ops_rec import _ops, workloads
 
     asked = []
     plain = _ops._new_workspace
     monkeypatch.setattr(_ops, "_new_workspace", lambda n, dev: (asked.append(n), plain(n, dev))[1])
-    w = workloads.make("win", dtype=torch.bfloat16, std=0.4, batch=2, heads=2, dim=512, lo=1, hi=90, max_seq_len=90)
+    w = workloads.make("win", dtype=torch.bfloat16, std=0.4, batch=2, heads=2, dim=512, lo=1, hi=90, max_seq_len=90, rab_std=0.5)
     check_backward(w)
     assert asked[-1] == 0
+    w = workloads.make("win", dtype=torch.bfloat16, std=0.4, batch=2, heads=2, dim=512, lo=1, hi=90, max_seq_len=90)
+    check_backward(w)
+    assert asked[-1] > 0
     w = workloads.make("win", dtype=torch.bfloat16, std=0.4, batch=2, heads=2, dim=264, dim_v=272, lo=1, hi=88, max_seq_len=88)
     check_backward(w)  # a head dim that is not a multiple of 16
     assert asked[-1] == 0

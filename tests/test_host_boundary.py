@@ -442,7 +442,10 @@ def test_backward_workspace_follows_the_launch_order(monkeypatch):
     assert size(**dict(c2, total_q=full, total_k=full)) == one  # the same without padding: three launches
     assert size(**dict(c2, head_dim_qk=64, head_dim_v=64)) == pair()  # small planes pay at every head dim
     assert size(**dict(c2, head_dim_qk=64, head_dim_v=64, num_heads_q=8, num_heads_k=8, total_q=full, total_k=full)) == 0  # larger ones: two launches
-    assert size(**dict(c2, max_seq_len_q=1020, max_seq_len_k=1020)) == 0  # rows that are not multiples of 16 bytes
+    # rows of [max_q][max_k] tensors that are not multiples of 16 bytes: the pair plane has its own layout and is taken all
+    # the same when the call has no such tensor; with an attn_bias and its gradient the call runs in two launches
+    assert size(**dict(c2, max_seq_len_q=1020, max_seq_len_k=1020)) == pair()
+    assert size(grad_attn_bias=fake, **dict(c2, max_seq_len_q=1020, max_seq_len_k=1020)) == 0
     assert size(**dict(c2, head_dim_qk=256, head_dim_v=256, total_q=full, total_k=full)) == pair(rows=full)
     assert size(**dict(c2, max_seq_len_q=4096, max_seq_len_k=4096)) == 0  # long rows at head dim 128
     # with an attn_bias gradient dS goes through the gradient itself in the three-launch order: planes or nothing
