@@ -185,8 +185,9 @@ HSTU_API uint64_t hstu_jagged_fwd_noalloc_max_workspace(void);
  * and 32-key block (only the blocks at or below the diagonal for a causal mask over equal query and key offsets
  * without context rows).  hstu_jagged_bwd_workspace_size asks for the workspace of the order it estimates to be the
  * fastest (at most 2 GiB, or HSTU_MI355_BWD_WORKSPACE_MB in the environment; with an attn_bias, a custom mask or an
- * attn_bias gradient, or for the [batch, ...] plane of dS alone, max_seq_len_k must be a multiple of 8 -- rows of such
- * tensors are read and written 16 bytes per lane -- while the workspace for dS and P together has its own layout; fp32
+ * attn_bias gradient, or for the [batch, ...] plane of dS alone, max_seq_len_k must be a multiple of 4 -- rows of such
+ * tensors are read and written in pieces of 8 keys, one 16-byte access when max_seq_len_k is a multiple of 8, two
+ * 8-byte ones otherwise -- while the workspace for dS and P together has its own layout; fp32
  * inputs with head dims up to 128: dS and P in fp32 whenever that fits).  Head dims above 256 need, beside that line
  * per row and block, 256 bytes per head, query row and block for the scores of the first window.  Without the workspace,
  * or with less than was asked for, the call still works: the kernels that produce grad_k then recompute dS (head dims

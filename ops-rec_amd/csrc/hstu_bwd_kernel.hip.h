@@ -913,7 +913,20 @@ __global__ __launch_bounds__(kDkvThreads, (MODE == 2 || MODE >= 4) ? bwd_dk_from
     // row, 8 consecutive keys per 16-byte load) as the A operand of two MFMAs whose B operand is a constant 0/1
     // matrix that routes k-slot (half lh, element e) of MFMA j to key column 16 j + 8 lh + e: the matrix pipe does
     // the transposition (exactly: every product is a value times 1 or 0), and rab lands in the S accumulators.
+    // With rows that start at multiples of 8 bytes only (max_seq_len_k a multiple of 4, not of 8) a piece of 8 keys is
+    // two 8-byte loads, and its second half is asked for only when it starts inside the row (inside the sequence's keys,
+    // for values that another kernel wrote piece by piece): past it lies the next row.
     const bool vec16 = a.bias_vec_ok == 2;
+    const bool vec8 = a.bias_vec_ok != 0;
+    auto load_piece = [&](const __amdgpu_buffer_rsrc_t rsrc, uint32_t off, bool second_half) -> u32x4_t {
+        if (vec16) {
+            return __builtin_amdgcn_raw_buffer_load_b128(rsrc, static_cast<int>(off), 0, 0);
+        }
+        const u32x2_t lo = __builtin_amdgcn_raw_buffer_load_b64(rsrc, static_cast<int>(off), 0, 0);
+        const u32x2_t hi = __builtin_amdgcn_raw_buffer_load_b64(rsrc, static_cast<int>(second_half ? off + 8u : kOutOfRange), 0, 0);
+        const u32x4_t r = {lo[0], lo[1], hi[0], hi[1]};
+        return r;
+    };
     u32x4_t route[2] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
     if constexpr (HAS_RAB || HAS_MASK || from_plane) {
         const uint32_t one = std::is_same<Tag, bf16_tag>::value ? 0x3f80u : 0x3c00u;  // 1.0 in the input type
@@ -1001,7 +1014,11 @@ __global__ __launch_bounds__(kDkvThreads, (MODE == 2 || MODE >= 4) ? bwd_dk_from
             const int key0 = cw0 + 16 * j + 8 * lh;
             const uint32_t col = MODE >= 4 ? static_cast<uint32_t>(2 * cw0 + 16 * j + 8 * lh + (dk_role ? 0 : 32)) : static_cast<uint32_t>(key0);
             const uint32_t off = (wanted && rq0 + ln < sq && key0 < sk) ? row_off + col * 2u : kOutOfRange;
-            ds_next[j] = __builtin_amdgcn_raw_buffer_load_b128(ds_rsrc, static_cast<int>(off), 0, 0);
+            if constexpr (MODE >= 4) {  // (the pair plane: 16-byte pieces whatever max_seq_len_k is)
+                ds_next[j] = __builtin_amdgcn_raw_buffer_load_b128(ds_rsrc, static_cast<int>(off), 0, 0);
+            } else {
+                ds_next[j] = load_piece(ds_rsrc, off, key0 + 4 < sk);
+            }
         }
     };
 
@@ -1035,7 +1052,7 @@ __global__ __launch_bounds__(kDkvThreads, (MODE == 2 || MODE >= 4) ? bwd_dk_from
         } else if constexpr (HAS_RAB || HAS_MASK) {
             // (ahead of the tile requests: loads return in order, so waiting for them then only waits for requests
             // of earlier steps)
-            if (vec16 && active) {
+            if (vec8 && active) {
 #pragma unroll
                 for (int j = 0; j < 2; ++j) {
                     const int key0 = cw0 + 16 * j + 8 * lh;
@@ -1043,10 +1060,10 @@ __global__ __launch_bounds__(kDkvThreads, (MODE == 2 || MODE >= 4) ? bwd_dk_from
                                              ? (static_cast<uint32_t>(rq0 + ln) * static_cast<uint32_t>(a.max_k) + static_cast<uint32_t>(key0)) * 2u
                                              : kOutOfRange;
                     if constexpr (HAS_RAB) {
-                        ra[j] = __builtin_amdgcn_raw_buffer_load_b128(rab_rsrc, static_cast<int>(off), 0, 0);
+                        ra[j] = load_piece(rab_rsrc, off, key0 + 4 < a.max_k);
                     }
                     if constexpr (HAS_MASK) {
-                        ma[j] = __builtin_amdgcn_raw_buffer_load_b128(mask_rsrc, static_cast<int>(off), 0, 0);
+                        ma[j] = load_piece(mask_rsrc, off, key0 + 4 < a.max_k);
                     }
                 }
             }
@@ -1067,7 +1084,13 @@ __global__ __launch_bounds__(kDkvThreads, (MODE == 2 || MODE >= 4) ? bwd_dk_from
                     const uint32_t off = (active && rq0 + ln < sq && key0 < sk)
                                              ? (static_cast<uint32_t>(rq0 + ln) * static_cast<uint32_t>(a.max_k) + static_cast<uint32_t>(key0)) * 2u
                                              : kOutOfRange;
-                    __builtin_amdgcn_raw_buffer_store_b128(ra[j], drab_rsrc, static_cast<int>(off), 0, 0);
+                    if (vec16) {
+                        __builtin_amdgcn_raw_buffer_store_b128(ra[j], drab_rsrc, static_cast<int>(off), 0, 0);
+                    } else {  // (8-byte pieces; the second one only when it starts inside the sequence's keys)
+                        const u32x2_t lo = {ra[j][0], ra[j][1]}, hi = {ra[j][2], ra[j][3]};
+                        __builtin_amdgcn_raw_buffer_store_b64(lo, drab_rsrc, static_cast<int>(off), 0, 0);
+                        __builtin_amdgcn_raw_buffer_store_b64(hi, drab_rsrc, static_cast<int>(key0 + 4 < sk ? off + 8u : kOutOfRange), 0, 0);
+                    }
                 }
             } else {
                 // (the dV workgroups keep the same count of requests in flight)
@@ -1133,7 +1156,7 @@ __global__ __launch_bounds__(kDkvThreads, (MODE == 2 || MODE >= 4) ? bwd_dk_from
             float xs[16], ms[16];
             f32x16_t mt16;  // custom mask tile, transposed by the matrix pipe
             if constexpr (HAS_RAB || HAS_MASK) {
-                if (vec16) {
+                if (vec8) {
                     if constexpr (HAS_RAB) {
                         s = mfma32<Tag>(ra[0], route[0], s);
                         s = mfma32<Tag>(ra[1], route[1], s);
@@ -1154,12 +1177,12 @@ __global__ __launch_bounds__(kDkvThreads, (MODE == 2 || MODE >= 4) ? bwd_dk_from
                 xs[e] = s[e];
                 ms[e] = 1.0f;
                 if constexpr (HAS_MASK) {
-                    if (vec16) {
+                    if (vec8) {
                         ms[e] = mt16[e];
                     }
                 }
                 if constexpr (HAS_RAB || HAS_MASK) {
-                    if (!vec16) {
+                    if (!vec8) {
                     const uint32_t boff = (r < sq && key < a.max_k)
                                               ? (static_cast<uint32_t>(r) * static_cast<uint32_t>(a.max_k) + static_cast<uint32_t>(key)) * 2u
                                               : kOutOfRange;

@@ -838,13 +838,14 @@ static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
         const bool fits = f->max_seq_len_q * row * 4 < (1LL << 31) && bytes <= cap * (1LL << 20);
         return fits ? BwdPlan{kPlanes, static_cast<uint64_t>(bytes)} : two;
     }
-    // Rows of the [max_q][max_k] tensors -- attn_bias, custom mask, the attn_bias gradient, a dense dS plane -- start at
-    // multiples of 16 bytes only when max_seq_len_k is a multiple of 8: the kernels that read or write such rows 16 bytes
-    // per lane need that.  The pair plane has a layout of its own: a call with none of those tensors can take the planes
-    // order whatever max_seq_len_k is (max_seq_len 1004 instead of 1024 must not cost the two-launch order's 7 products).
-    const bool rows16 = f->max_seq_len_k % 8 == 0;
+    // Rows of the [max_q][max_k] tensors -- attn_bias, custom mask, the attn_bias gradient, a dense dS plane -- are read
+    // and written by the key-tile kernels in pieces of 8 keys: one 16-byte access when max_seq_len_k is a multiple of 8,
+    // two 8-byte ones when it is a multiple of 4; otherwise the call runs in two launches that take such rows element by
+    // element.  The pair plane has a layout of its own: a call with none of those tensors can take the planes order
+    // whatever max_seq_len_k is (max_seq_len 1004 instead of 1024 must not cost the two-launch order's 7 products).
+    const bool rows8 = f->max_seq_len_k % 4 == 0;
     const bool no_bias_tensors = f->attn_bias == nullptr && f->mask == nullptr && p->grad_attn_bias == nullptr;
-    if (var->dk_from_ds == nullptr || (!rows16 && !no_bias_tensors)) {
+    if (var->dk_from_ds == nullptr || (!rows8 && !no_bias_tensors)) {
         return two;
     }
     const int64_t batch = f->n_offsets - 1;
@@ -857,7 +858,7 @@ static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
     const int64_t cap = workspace_cap_mb() * (1LL << 20);
     // with an attn_bias gradient dS goes through the gradient itself in the three-launch order: no workspace
     const int64_t ds_plane = bias_grad ? 0 : batch * f->num_heads_q * f->max_seq_len_q * f->max_seq_len_k * 2;
-    const bool three_fits = rows16 && ds_plane <= cap;
+    const bool three_fits = rows8 && ds_plane <= cap;
     const bool planes_fit = pp.fits_32 && pp.bytes <= cap && (!bias_grad || var->dv_dk_from_planes_drab != nullptr);
     const BwdPlan three = {kThreeLaunches, static_cast<uint64_t>(ds_plane)};
     const BwdPlan planes = {kPlanes, static_cast<uint64_t>(pp.bytes)};
@@ -987,9 +988,9 @@ static WindowPlan plan_windows(const hstu_jagged_bwd_params* p)
         f->head_dim_v % 16 != 0 || switches().generic_backward == 1 || f->total_q == 0 || f->total_k == 0) {
         return w;
     }
-    // (rows of attn_bias, custom mask and the gradient are read and written 16 bytes per lane: see plan_bwd)
+    // (rows of attn_bias, custom mask and the gradient are read and written in pieces of 8 or 16 bytes: see plan_bwd)
     const bool no_bias_tensors = f->attn_bias == nullptr && f->mask == nullptr && p->grad_attn_bias == nullptr;
-    if (f->max_seq_len_k % 8 != 0 && !no_bias_tensors) {
+    if (f->max_seq_len_k % 4 != 0 && !no_bias_tensors) {
         return w;
     }
     // (16-byte rows of the planes and of the attn_bias tensors, spans behind 32-bit descriptors)
@@ -1133,7 +1134,7 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
         w.d_v = a.d_v / 2;
         w.n_heads_q = 2 * a.n_heads_q;
         w.n_heads_k = 2 * a.n_heads_k;
-        w.bias_vec_ok = 2;
+        w.bias_vec_ok = f->max_seq_len_k % 8 == 0 ? 2 : 1;  // (pointers are 16-byte aligned here; rows of 16 or of 8 bytes)
         w.p_plane = workspace;
         w.plane_head_lines = windows.pair.head_lines;
         w.plane_tri = windows.pair.tri ? 1 : 0;
@@ -1194,7 +1195,7 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
             }
         }
     } else if (f->total_k > 0 && grid_kv > 0 && f->total_q > 0 && grid_q > 0 && plan.order != kTwoLaunches &&
-               (a.bias_vec_ok == 2 || (plan.order == kPlanes && f->attn_bias == nullptr && f->mask == nullptr && p->grad_attn_bias == nullptr)) &&
+               (a.bias_vec_ok != 0 || (plan.order == kPlanes && f->attn_bias == nullptr && f->mask == nullptr && p->grad_attn_bias == nullptr)) &&
                (plan.workspace_bytes == 0 || (usable_workspace(workspace, workspace_bytes, plan.workspace_bytes) &&
                                               reinterpret_cast<uintptr_t>(workspace) % 16 == 0))) {
         if (p->grad_attn_bias == nullptr) {
@@ -1230,7 +1231,7 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
         hipLaunchKernelGGL(var->dv_only, dim3(static_cast<unsigned>(n_kv_slots)), dim3(hstu::kDkvThreads), 0,
                            static_cast<hipStream_t>(stream), a);
         a.drab_clear_bytes = 0;
-        if (dq_short != nullptr && p->grad_attn_bias == nullptr) {
+        if (dq_short != nullptr && p->grad_attn_bias == nullptr && a.bias_vec_ok == 2) {  // (its dS pieces assume 16-byte rows)
             hipLaunchKernelGGL(dq_short->dq_ds, dim3(static_cast<unsigned>(dq_short_grid(a))), dim3(hstu::kDqShortThreads), 0,
                                static_cast<hipStream_t>(stream), a);
         } else {

@@ -221,6 +221,31 @@ def test_planes_with_a_max_seq_len_that_is_not_a_multiple_of_8(kw, mask_type, mo
     check(w, monkeypatch)  # with the workspace full of NaN, against the oracle and the generic kernels
 
 
+@pytest.mark.parametrize("dim,max_len", [(64, 300), (128, 420), (256, 268), (384, 132)])
+@pytest.mark.parametrize("custom_mask", [False, True], ids=["builtin", "custom"])
+@pytest.mark.parametrize("want_drab", [False, True], ids=["nodrab", "drab"])
+def test_rows_of_8_byte_pieces_in_every_order(dim, max_len, custom_mask, want_drab, monkeypatch):
+    """max_seq_len_k a multiple of 4 but not of 8: rows of attn_bias, custom mask, the attn_bias gradient and the dense dS
+    plane start at multiples of 8 bytes only.  The key-tile kernels then take a piece of 8 keys as two 8-byte accesses, the
+    second only when it starts inside the row (the sequence's keys): sequences that end at, one short of and three short
+    of max_seq_len_k put the next row right behind such a piece.  Every launch order, the workspace full of NaN, against
+    the oracle and the generic kernels."""
+    lengths = [max_len, max_len - 1, max_len - 3, max_len // 2, 37]
+    w = make(batch=len(lengths), heads=2, dim=dim, lo=0, hi=0, lengths=lengths, max_seq_len=max_len, seed=dim + max_len,
+             rab_std=0.5)  # fmt: skip
+    if custom_mask:
+        g = torch.Generator(device=DEV).manual_seed(1)
+        m = (torch.rand(len(lengths), 2, max_len, max_len, generator=g, device=DEV) < 0.6).to(w.q.dtype)
+        w = dataclasses.replace(w, mask=m, mask_type=3)
+    if not want_drab:
+        # (the operator returns the gradient of every attn_bias it is given: the case without one keeps the custom mask
+        # or, failing that, runs without bias tensors at all -- the planes order with a layout of its own)
+        w = dataclasses.replace(w, attn_bias=None)
+    for order in ("0", "1", "2"):
+        helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", order)
+        check(w, monkeypatch)
+
+
 def test_no_mask(monkeypatch):
     check(dataclasses.replace(make(batch=2, heads=2, dim=128, lo=100, hi=300, seed=9), mask_type=2), monkeypatch)
 
