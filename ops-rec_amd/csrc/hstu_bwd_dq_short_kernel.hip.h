@@ -81,7 +81,8 @@ __global__ __launch_bounds__(kDqShortThreads, kDqShortWavesPerSimd) void hstu_bw
     const int b = div_small(slot.pair, a.n_heads_k);
     const int hk = slot.pair - b * a.n_heads_k;
     const int h = hk * a.head_ratio + slot.r;
-    const int qt = n_levels - 1 - slot.level;
+    // (heaviest tiles first; with context rows the first tile of a sequence sweeps all of its history keys and goes ahead)
+    const int qt = (a.mask_type == 0 && a.num_ctx != nullptr) ? (slot.level == 0 ? 0 : n_levels - slot.level) : n_levels - 1 - slot.level;
     const SeqInfo sq_info = load_seq(a, b);
     const int sq = sq_info.sq, sk = sq_info.sk;
     const int r0 = qt * kDqShortRows;

@@ -341,7 +341,8 @@ __global__ __launch_bounds__(256, bwd_dq_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void 
     const int per_level = a.n_batch * grid_heads;
     const int lvl = static_cast<int>(blockIdx.x) / per_level;
     const int rem = static_cast<int>(blockIdx.x) - lvl * per_level;
-    const int qt = a.n_qtiles - 1 - lvl;
+    // (heaviest tiles first; with context rows the first tile of a sequence sweeps all of its history keys and goes ahead)
+    const int qt = (a.mask_type == 0 && a.num_ctx != nullptr) ? (lvl == 0 ? 0 : a.n_qtiles - lvl) : a.n_qtiles - 1 - lvl;
     const int b = rem / grid_heads;
     const int h_grid = rem - b * grid_heads;
     const int h = a.win_only >= 0 ? h_grid * a.win + a.win_only : h_grid;
@@ -888,13 +889,25 @@ __global__ __launch_bounds__(kDkvThreads, (MODE == 2 || MODE >= 4) ? bwd_dk_from
     }
 
     // query sub-tiles that can see a key of this tile
+    // (causal: from the sub-tile of the first row that sees key c0 on; with context rows ahead of that, which see every history
+    // key: their sub-tiles first, then the same -- the sub-tiles in between see nothing of this tile and are skipped)
     const int n_qsub = (sq + 31) / 32;
     int x_first = 0;
-    if (a.mask_type == 0 && !(si.n_ctx > 0 && c0 < si.hist_k)) {
+    int x_skip_from = -1, x_skip_to = -1;
+    if (a.mask_type == 0) {
         const int first_row = c0 - si.delta;  // the first row that sees key c0
-        x_first = first_row > 0 ? first_row / 32 : 0;
+        const int x_causal = first_row > 0 ? first_row / 32 : 0;
+        if (si.n_ctx > 0 && c0 < si.hist_k) {
+            const int ctx_end = ((si.n_ctx < sq ? si.n_ctx : sq) + 31) / 32;  // sub-tiles that hold context rows
+            if (x_causal > ctx_end) {
+                x_skip_from = ctx_end;
+                x_skip_to = x_causal < n_qsub ? x_causal : n_qsub;
+            }
+        } else {
+            x_first = x_causal;
+        }
     }
-    const int nx = n_qsub > x_first ? n_qsub - x_first : 0;
+    const int nx = (n_qsub > x_first ? n_qsub - x_first : 0) - (x_skip_to - x_skip_from);
     const int n_iter = nx * a.head_ratio;  // (query head of the group, query sub-tile), head-major
 
     f32x16_t acc[MTILES];  // dK^T or dV^T of this wavefront's keys, by role
@@ -969,7 +982,10 @@ __global__ __launch_bounds__(kDkvThreads, (MODE == 2 || MODE >= 4) ? bwd_dk_from
             }
         }
         ++req_it;
-        if (++req_x >= n_qsub) {
+        if (++req_x == x_skip_from) {
+            req_x = x_skip_to;
+        }
+        if (req_x >= n_qsub) {
             req_x = x_first;
             if (!past && req_it < n_iter) {
                 req_h += a.win;
@@ -1030,7 +1046,10 @@ __global__ __launch_bounds__(kDkvThreads, (MODE == 2 || MODE >= 4) ? bwd_dk_from
         __builtin_amdgcn_sched_barrier(0);
         const int h = cur_h;
         const int rq0 = cur_x * 32;  // first query row of the sub-tile
-        if (++cur_x >= n_qsub) {
+        if (++cur_x == x_skip_from) {
+            cur_x = x_skip_to;
+        }
+        if (cur_x >= n_qsub) {
             cur_x = x_first;
             cur_h += a.win;
         }

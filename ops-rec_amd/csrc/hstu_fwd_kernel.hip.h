@@ -905,6 +905,11 @@ __global__ __launch_bounds__(256, fwd_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hst
             const int rem_item = j_item - m_item * per_pair;
             const int t_item = div_small(rem_item, ratio);
             qt = nt_item - 1 - t_item;
+            if (a.mask_type == 0 && a.num_ctx != nullptr) {
+                // with context rows the first tile of a sequence sweeps all of its history keys: it goes ahead of the pair's
+                // other tiles instead of last, where it would end the launch with one long item per queue
+                qt = t_item == 0 ? 0 : nt_item - t_item;
+            }
             r_item = rem_item - t_item * ratio;
             const int p_first = static_cast<int>(s_rank_start[nt_item]) * n_heads_k;
             p_item = p_first + ((fq_queue + kQueues - (p_first & (kQueues - 1))) & (kQueues - 1)) + m_item * kQueues;

@@ -184,7 +184,10 @@ __global__ __launch_bounds__(kShortThreads, kShortWavesPerSimd) void hstu_fwd_sh
         hk = slot.pair - b * a.n_heads_k;
     }
     const int h = hk * ratio + slot.r;
-    const int qt = n_levels - 1 - slot.level;
+    // heaviest tiles first; with context rows the first tile of a sequence sweeps all of its history keys, so it goes ahead
+    // of the others instead of last
+    const bool ctx_first = a.mask_type == 0 && a.num_ctx != nullptr;
+    const int qt = ctx_first ? (slot.level == 0 ? 0 : n_levels - slot.level) : n_levels - 1 - slot.level;
     int64_t q0 = 0, q1 = 0, k0 = 0, k1 = 0;
     int n_ctx = 0, n_tgt = 0;
     if (live) {
