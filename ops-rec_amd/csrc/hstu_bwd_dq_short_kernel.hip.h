@@ -72,7 +72,8 @@ __global__ __launch_bounds__(kDqShortThreads, kDqShortWavesPerSimd) void hstu_bw
 
     zero_tail_rows(a.dq, a.offs_q, a.n_batch, a.idx64, a.total_q, static_cast<int64_t>(a.n_heads_q) * a.d_qk, kDqShortThreads);
 
-    const int n_levels = (a.max_q + kDqShortRows - 1) / kDqShortRows;
+    // (the levels that exist in the batch, at most those the host sized the grid for: see batch_max_rows)
+    const int n_levels = live_levels(a, lane, kDqShortRows, (a.max_q + kDqShortRows - 1) / kDqShortRows);
     const int n_pairs = a.n_batch * a.n_heads_k;
     const ShortSlot slot = short_slot(static_cast<int>(blockIdx.x), n_pairs, a.head_ratio);
     if (slot.pair >= n_pairs || slot.level >= n_levels) {

@@ -80,6 +80,36 @@ __device__ __forceinline__ SeqInfo load_seq(const BwdArgs& a, int b)
     return s;
 }
 
+// The longest sequence of the batch in query rows, clamped as load_seq clamps: one pass of the wavefront over the offsets.
+// The host sizes the grids of the query-tile kernels from max_seq_len_q, a bound that callers often set far above their
+// sequences (a configuration constant); the kernels take the number of tile levels that exist from here, so that the
+// workgroups of levels no sequence has come last in the grid instead of first and the heaviest tiles start at once.
+__device__ __forceinline__ int batch_max_rows(const BwdArgs& a, int lane)
+{
+    int longest = 0;
+    for (int b = lane; b < a.n_batch; b += 64) {
+        int64_t q0 = load_index(a.offs_q, b, a.idx64);
+        int64_t q1 = load_index(a.offs_q, b + 1, a.idx64);
+        q1 = q1 < a.total_q ? q1 : a.total_q;
+        q0 = q0 < 0 ? 0 : q0;
+        const int sq = static_cast<int>(q1 > q0 ? q1 - q0 : 0);
+        longest = sq > longest ? sq : longest;
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) {
+        const int other = __shfl_xor(longest, m, 64);
+        longest = other > longest ? other : longest;
+    }
+    longest = uniform(longest);
+    return longest < a.max_q ? longest : a.max_q;
+}
+// tile levels (of `rows` query rows each) that some sequence of the batch has: at most the host's count, at least one
+__device__ __forceinline__ int live_levels(const BwdArgs& a, int lane, int rows, int host_levels)
+{
+    const int n = (batch_max_rows(a, lane) + rows - 1) / rows;
+    return n < 1 ? 1 : (n < host_levels ? n : host_levels);
+}
+
 // The pair plane of the 16-bit kernels: what the query-tile kernel hands to the key-tile workgroups of the next launch.
 // One 128-byte line per query row and 32-key block: the block's 32 dS values, then its 32 P values.  Lines are packed
 // per head by global query row (offs_q[b] + r; no room for rows that the batch does not have), the lines of a row side by
@@ -341,14 +371,19 @@ __global__ __launch_bounds__(256, bwd_dq_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void 
     const int per_level = a.n_batch * grid_heads;
     const int lvl = static_cast<int>(blockIdx.x) / per_level;
     const int rem = static_cast<int>(blockIdx.x) - lvl * per_level;
-    // (heaviest tiles first; with context rows the first tile of a sequence sweeps all of its history keys and goes ahead)
-    const int qt = (a.mask_type == 0 && a.num_ctx != nullptr) ? (lvl == 0 ? 0 : a.n_qtiles - lvl) : a.n_qtiles - 1 - lvl;
+    // (heaviest tiles first, counted from the highest level that exists in the batch; with context rows the first tile of a
+    // sequence sweeps all of its history keys and goes ahead)
+    const int n_levels = live_levels(a, lane, kBlockM, a.n_qtiles);
+    const int qt = (a.mask_type == 0 && a.num_ctx != nullptr) ? (lvl == 0 ? 0 : n_levels - lvl) : n_levels - 1 - lvl;
     const int b = rem / grid_heads;
     const int h_grid = rem - b * grid_heads;
     const int h = a.win_only >= 0 ? h_grid * a.win + a.win_only : h_grid;
     const int hk = kv_head_of(a, h);
     if constexpr (PHASE != 1) {
         zero_tail_rows(a.dq, a.offs_q, a.n_batch, a.idx64, a.total_q, static_cast<int64_t>(a.n_heads_q) * a.d_qk, 256);
+    }
+    if (lvl >= n_levels) {
+        return;  // a level that no sequence of the batch has
     }
     const SeqInfo sq_info = load_seq(a, b);
     const int sq = sq_info.sq, sk = sq_info.sk;

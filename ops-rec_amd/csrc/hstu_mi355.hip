@@ -776,8 +776,13 @@ static BwdCost estimate_bwd(const hstu_jagged_fwd_params* f, bool bias_grad)
     const int64_t dmax = f->head_dim_qk > f->head_dim_v ? f->head_dim_qk : f->head_dim_v;
     const int slot = dmax <= 64 ? 0 : (dmax <= 128 ? 1 : 2);
     const double batch = static_cast<double>(f->n_offsets - 1), heads = static_cast<double>(f->num_heads_q);
-    const double max_q = static_cast<double>(f->max_seq_len_q), max_k = static_cast<double>(f->max_seq_len_k);
     const double mean_q = static_cast<double>(f->total_q) / batch, mean_k = static_cast<double>(f->total_k) / batch;
+    // max_seq_len is a bound, and callers often pass a configuration constant far above their sequences: lengths spread
+    // evenly up to a longest one have a mean of half of it, so twice the mean stands in for a bound beyond that (a batch
+    // of 32 sequences of 256..1024 rows under max_seq_len 8192 is then priced like the same batch under 1024: planes,
+    // 174 -> 117 us, where the bound priced every order by one 8192-row tail and picked the two launches)
+    const double max_q = std::max(mean_q, std::min(static_cast<double>(f->max_seq_len_q), 2.0 * mean_q));
+    const double max_k = std::max(mean_k, std::min(static_cast<double>(f->max_seq_len_k), 2.0 * mean_k));
     const bool causal = f->mask_type == HSTU_MASK_TRIL;
     // sum over the sequences of (query rows x keys)
     double area = batch * (mean_q * mean_k + (max_q > mean_q && max_k > mean_k ? (max_q - mean_q) * (max_k - mean_k) / 3.0 : 0.0));
@@ -785,7 +790,7 @@ static BwdCost estimate_bwd(const hstu_jagged_fwd_params* f, bool bias_grad)
     const double pairs = heads * area * (causal ? 0.5 : 1.0);
     const double mpairs = (pairs + (causal ? 1.0 : 0.4) * kRowOverhead * static_cast<double>(f->total_q) * heads) * 1e-6;
     const double ratio = static_cast<double>(f->num_heads_q / f->num_heads_k);
-    const double dense = batch * heads * max_q * max_k * 2.0;  // the attn_bias gradient, cleared whole
+    const double dense = batch * heads * static_cast<double>(f->max_seq_len_q) * static_cast<double>(f->max_seq_len_k) * 2.0;  // the attn_bias gradient, cleared whole
     const double bias = bias_grad ? 2.0 * pairs : 0.0;         // attn_bias as read by a launch that computes scores
     auto launch = [&](int products, const double* rate, int products_per_wg, double bytes, bool key_tiles, bool scores) {
         const double cached = bytes > kCacheBytes ? kCacheBytes / bytes : 1.0;
