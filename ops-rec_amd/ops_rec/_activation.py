@@ -28,6 +28,35 @@ LN_MUL_EPSILON = 1e-5
 _lib_def.define("ln_mul(Tensor x, Tensor u, Tensor gamma, Tensor beta) -> Tensor")
 
 
+# Validated calls, by everything but the addresses: (shapes, dtypes, devices, contiguity) -> the parameter block with its
+# scalar fields filled.  A layer repeats one description per step with new tensors; on a hit the checks and the filling of
+# the block are skipped and only the addresses are set (the checks cost more host time than the kernels of a small layer
+# take: [20292, 512] bf16 ln_mul 18.7 us per call for a 10.4 us kernel before, in_linear_silu 30 us for small shapes).
+_CALL_CACHE: dict = {}
+_CALL_CACHE_MAX = 256
+
+
+def _tensor_key(t: Optional[torch.Tensor]):
+    return None if t is None else (tuple(t.shape), t.dtype, t.device, t.is_contiguous())
+
+
+def _remember(key, params) -> None:
+    if len(_CALL_CACHE) >= _CALL_CACHE_MAX:
+        _CALL_CACHE.clear()
+    _CALL_CACHE[key] = bytes(params)
+
+
+def _launch(fn, params, device: torch.device, what: str) -> None:
+    """``fn(params, stream)`` of the C ABI on the current stream of ``device``."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        rc = fn(ctypes.byref(params), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    else:
+        with torch.cuda.device(device):
+            rc = fn(ctypes.byref(params), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    if rc != 0:
+        raise RuntimeError(f"{what} failed ({rc}): {_native.last_error()}")
+
+
 def _non_empty(t: torch.Tensor, name: str) -> None:
     # check_tensor_non_empty (ascendc/common/torch_plugin/common_utils.h:34-39)
     _check(t is not None, f"{name} tensor must be defined")
@@ -44,6 +73,14 @@ def _ln_mul_shapes(x, u, gamma, beta) -> None:
 
 
 def ln_mul(x, u, gamma, beta):
+    key = ("ln_mul", _tensor_key(x), _tensor_key(u), _tensor_key(gamma), _tensor_key(beta))
+    cached = _CALL_CACHE.get(key)
+    if cached is not None and key[1][3] and key[2][3] and key[3][3] and key[4][3]:  # (contiguous tensors: used as they are)
+        out = torch.empty_like(x)
+        p = _native.LnMulParams.from_buffer_copy(cached)
+        p.x, p.u, p.gamma, p.beta, p.out = x.data_ptr(), u.data_ptr(), gamma.data_ptr(), beta.data_ptr(), out.data_ptr()
+        _launch(_native.load().ln_mul_fwd, p, x.device, "ln_mul")
+        return out
     for t, name in ((x, "x"), (u, "u"), (gamma, "gamma"), (beta, "beta")):
         _non_empty(t, name)
     for t, name in ((x, "x"), (u, "u"), (gamma, "gamma"), (beta, "beta")):
@@ -62,11 +99,8 @@ def ln_mul(x, u, gamma, beta):
     p.rows, p.cols = x_c.size(0), x_c.size(1)
     p.dtype, p.affine_dtype = _DTYPE_CODE[x_c.dtype], _DTYPE_CODE[g_c.dtype]
     p.epsilon = LN_MUL_EPSILON
-    lib = _native.load()
-    with torch.cuda.device(x_c.device):
-        rc = lib.ln_mul_fwd(ctypes.byref(p), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
-    if rc != 0:
-        raise RuntimeError(f"ln_mul failed ({rc}): {_native.last_error()}")
+    _launch(_native.load().ln_mul_fwd, p, x_c.device, "ln_mul")
+    _remember(key, p)  # (the library took the description)
     return out
 
 
@@ -119,6 +153,18 @@ def _in_linear_silu_shapes(x, weight, bias, split: List[int]) -> None:
 
 def distance_in_linear_silu(x, weight, bias, attr_dict):
     split = [int(s) for s in attr_dict]
+    key = ("in_linear_silu", _tensor_key(x), _tensor_key(weight), _tensor_key(bias), tuple(split))
+    cached = _CALL_CACHE.get(key)
+    if cached is not None and key[1][3] and key[2][3] and (bias is None or key[3][3]):
+        m, n = x.size(0), weight.size(0)
+        outs = [torch.empty((m, s_), dtype=x.dtype, device=x.device) for s_ in split]
+        linear_output = torch.empty((m, n), dtype=x.dtype, device=x.device)
+        p = _native.InLinearSiluParams.from_buffer_copy(cached)
+        p.x, p.weight, p.bias = x.data_ptr(), weight.data_ptr(), (bias.data_ptr() if bias is not None else None)
+        p.user, p.value, p.query, p.key = (t.data_ptr() for t in outs)
+        p.linear_output = linear_output.data_ptr()
+        _launch(_native.load().in_linear_silu_fwd, p, x.device, "in_linear_silu")
+        return outs[0], outs[1], outs[2], outs[3], linear_output
     _in_linear_silu_shapes(x, weight, bias, split)
     _check(x.dtype in (torch.bfloat16, torch.float16), f"x must be float16 or bfloat16, got {x.dtype}")
     _check(weight.dtype == x.dtype, "weight must have the dtype of x")
@@ -140,11 +186,8 @@ def distance_in_linear_silu(x, weight, bias, attr_dict):
     for i, s in enumerate(split):
         p.split[i] = s
     p.dtype = _DTYPE_CODE[x.dtype]
-    lib = _native.load()
-    with torch.cuda.device(x.device):
-        rc = lib.in_linear_silu_fwd(ctypes.byref(p), ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
-    if rc != 0:
-        raise RuntimeError(f"in_linear_silu failed ({rc}): {_native.last_error()}")
+    _launch(_native.load().in_linear_silu_fwd, p, x.device, "in_linear_silu")
+    _remember(key, p)  # (the library took the description)
     return outs[0], outs[1], outs[2], outs[3], linear_output
 
 
