@@ -655,7 +655,7 @@ HSTU_API int hstu_paged_fwd(const hstu_paged_fwd_params* p, void* workspace, uin
         }
         return launch_forward(&g, p, workspace, workspace_bytes, stream);
     }
-    // no paged kernel for this combination (fp32, head dims above 128): gather the rows, then the plain forward
+    // no paged kernel for this combination (fp32, head dims up to 32 or above 256): gather the rows, then the plain forward
     if (p->fwd.total_k > 0) {
         if (workspace == nullptr || workspace_bytes < 2 * region || reinterpret_cast<uintptr_t>(workspace) % 16 != 0) {
             return fail(HSTU_ERR_WORKSPACE, "the paged forward needs a 16-byte aligned workspace of at least %llu bytes",

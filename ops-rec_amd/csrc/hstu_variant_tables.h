@@ -28,7 +28,7 @@ constexpr auto split_kernel() -> void (*)(const FwdArgs)
 template <typename Tag, typename OutTag, int D, bool RAB, bool MASK>
 constexpr auto paged_kernel() -> void (*)(const FwdArgs)
 {
-    if constexpr (D == 64 || D == 128) {
+    if constexpr (D == 64 || D == 128 || D == 256) {
         return hstu_fwd_kernel<Tag, OutTag, D, RAB, MASK, false, true, true>;
     } else {
         return nullptr;

@@ -7,8 +7,8 @@
 
 namespace hstu {
 
-// kernel variants with the per-XCD work queues, with split items and with paged keys exist for the head-dim slots
-// 64 and 128 (nullptr elsewhere)
+// kernel variants with the per-XCD work queues and with split items exist for the head-dim slots 64 and 128, the one
+// with paged keys for 64, 128 and 256 (nullptr elsewhere)
 struct Variant {
     const char* name;
     const char* name_queues;

@@ -62,6 +62,21 @@ def test_rows_cached_before_the_request_and_target_groups(group):
     check(c, group=group, alpha=128**-0.5)
 
 
+@pytest.mark.parametrize("dim,page_size", [(256, 128), (192, 32), (256, 256), (160, 64)])
+@pytest.mark.parametrize("with_bias", [False, True], ids=["plain", "bias"])
+def test_head_dims_of_the_slot_256_read_the_pages_themselves(dim, page_size, with_bias):
+    """Head dims above 128 have a paged kernel variant as well (they were gathered into contiguous rows first): rows cached
+    before the request, partial last pages, grouped heads, with and without attn_bias on the paged keys."""
+    c = paged_case(hist=[140, 64, 33], prev=[700, 0, 130], targets=[12, 7, 40], page_size=page_size, heads=4, heads_k=2,
+                   dim=dim, dtype=torch.bfloat16, std=0.3, seed=dim + page_size)  # fmt: skip
+    if with_bias:
+        g = torch.Generator().manual_seed(3)
+        bias = (torch.randn(3, 4, c["max_seq_len"], c["max_seq_len_k"], generator=g) * 0.3).to(torch.bfloat16)
+        check(c, attn_bias=bias.to(DEV), alpha=dim**-0.5)
+    else:
+        check(c, alpha=dim**-0.5)
+
+
 def test_attn_bias_and_custom_mask_on_paged_keys():
     c = paged_case(hist=[90, 150], prev=[40, 0], targets=[5, 9], page_size=32, heads=2, dim=64, dtype=torch.float16,
                    std=0.5, seed=9)  # fmt: skip
