@@ -8,6 +8,8 @@ namespace hstu {
 template <typename Tag, typename OutTag, int D, bool RAB, bool MASK>
 constexpr auto queues_kernel() -> void (*)(const FwdArgs)
 {
+    // (at the slot 256, one workgroup per CU, the queues and the split items were measured level with the plain list:
+    // -5 .. +5 % and -12 .. +16 % over ten shapes)
     if constexpr (D == 64 || D == 128) {
         return hstu_fwd_kernel<Tag, OutTag, D, RAB, MASK, true>;
     } else {
