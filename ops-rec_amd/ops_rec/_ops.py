@@ -574,6 +574,22 @@ def hstu_jagged_backward_delta_meta(grad, q, k, v, mask=None, attn_bias=None, ma
     return _backward_meta(grad, q, k, v, attn_bias)
 
 
+_DENSE_OFFSETS: dict = {}
+
+
+def _dense_offsets(batch: int, s_len: int, dev) -> torch.Tensor:
+    """``0, S, 2S, ..`` (batch + 1 values, int32) on ``dev``: the offsets of a dense batch, built once per shape (a
+    layer calls with one shape step after step; the tensor is only ever read)."""
+    key = (batch, s_len, dev)
+    offs = _DENSE_OFFSETS.get(key)
+    if offs is None:
+        if len(_DENSE_OFFSETS) >= 64:
+            _DENSE_OFFSETS.clear()
+        offs = torch.arange(0, (batch + 1) * max(s_len, 1), max(s_len, 1), dtype=torch.int32, device=dev)[: batch + 1]
+        _DENSE_OFFSETS[key] = offs
+    return offs
+
+
 def hstu_dense(q, k, v, mask=None, attn_bias=None, mask_type=0, max_seq_len=0, silu_scale=0.0):
     """Dense ``[B, S, N, D]`` forward (torch_extension/hstu_dense_plugin.cpp:19-40): every sequence has the full
     length S, no alpha (1.0), no context / target arguments.  Served by the jagged kernel on a view
@@ -587,8 +603,8 @@ def hstu_dense(q, k, v, mask=None, attn_bias=None, mask_type=0, max_seq_len=0, s
     real_scale = (1.0 / float(max_seq_len)) if float(silu_scale) == 0.0 else float(silu_scale)
     qc, kc, vc = q.contiguous(), k.contiguous(), v.contiguous()
     dev = qc.device
-    offs_q = torch.arange(0, (batch + 1) * s_q, max(s_q, 1), dtype=torch.int32, device=dev)[: batch + 1]
-    offs_k = offs_q if s_k == s_q else torch.arange(0, (batch + 1) * s_k, max(s_k, 1), dtype=torch.int32, device=dev)[: batch + 1]
+    offs_q = _dense_offsets(batch, s_q, dev)
+    offs_k = offs_q if s_k == s_q else _dense_offsets(batch, s_k, dev)
     if batch == 0 or s_q == 0:
         return torch.empty((batch, s_q, q.size(2), v.size(3)), dtype=_out_dtype(qc), device=dev)
     out = _forward_impl(qc.view(batch * s_q, q.size(2), q.size(3)), kc.view(batch * s_k, k.size(2), k.size(3)),
@@ -695,7 +711,7 @@ def hstu_dense_backward(grad, q, k, v, mask, attn_bias, mask_type=0, max_seq_len
             _check(t.dtype == grad.dtype, f"{name} dtype should be the same as grad dtype, but got {name}: {t.dtype} and grad: {grad.dtype}")
     _check(s_len == int(max_seq_len), "seqLen must be equal to maxSeqLen")
     dev = grad.device
-    offs = torch.arange(0, (batch + 1) * s_len, s_len, dtype=torch.int32, device=dev)[: batch + 1]
+    offs = _dense_offsets(batch, s_len, dev)
     flat = lambda t: t.contiguous().view(batch * s_len, heads, dim)  # noqa: E731
     dq, dk, dv, dbias = _backward_impl(flat(grad), flat(q), flat(k), flat(v), mask, attn_bias, mask_type, s_len, s_len,
                                        silu_scale, offs, offs, None, None, 0, 1.0)  # fmt: skip
