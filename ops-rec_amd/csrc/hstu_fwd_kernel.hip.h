@@ -392,7 +392,7 @@ struct U32Quad {
 // these are two 16-byte reads of a K row (and the matching two pieces of the Q fragment: k index (half, byte) =
 // dim 16 (2p + half) + byte of piece p); PV contracts over the 64 keys of a pair of sub-tiles, its V^T operand
 // being four 8-bit transposed reads (16 keys x 32 dims each) in the order in which P^T holds the keys.  rab and the
-// custom mask are e4m3 tensors like q (plain list only).
+// custom mask are e4m3 tensors like q (the plain list and the per-XCD queues; items are not split).
 //
 // QUEUES: build the per-XCD queue machinery (see "Work queues" below).  It pays on long, jagged batches with many
 // items per workgroup; its code is on the path of every item, so launches that cannot profit (the host decides by
@@ -415,7 +415,7 @@ __global__ __launch_bounds__(256, fwd_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hst
         fp8_saturating_conversions();  // P^T beyond +-448 becomes +-448, not NaN (an fp16 output saturates likewise)
     }
     constexpr uint32_t ES = elem_traits<Tag>::kBytes;  // bytes per input element
-    static_assert(!F8 || !(HAS_RAB || HAS_MASK) || !(QUEUES || SPLIT), "fp8 with rab / custom mask: plain list only");
+    static_assert(!F8 || !(HAS_RAB || HAS_MASK) || !SPLIT, "fp8 with rab / custom mask: whole items only");
     static_assert(!F8 || D >= 64, "fp8 rows are at least 64 bytes");
     static_assert(!(QUEUES && SPLIT), "one list policy per variant");
     static_assert(!PAGED || (SPLIT && !F8), "the paged variant builds on the split variant, 16-bit inputs");

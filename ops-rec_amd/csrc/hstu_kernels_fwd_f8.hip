@@ -8,10 +8,12 @@
      hstu::hstu_fwd_kernel<hstu::f8_tag, hstu::otag, D, false, false>,                          \
      hstu::queues_kernel<hstu::f8_tag, hstu::otag, D, false, false>(),                          \
      hstu::split_kernel<hstu::f8_tag, hstu::otag, D, false, false>(), nullptr, D, 256, hstu::fwd_wgs_per_cu(D, false, false)}
-// with rab and / or a custom mask (e4m3 tensors like q): the plain list only
+// with rab and / or a custom mask (e4m3 tensors like q): the plain list, and the per-XCD queues for long lists
 #define HSTU_F8_BIASED(otag, oname, D, RAB, MASK, WGS)                                          \
-    {"hstu_fwd_f8e4m3_" oname "_d" #D "_rab" #RAB "_mask" #MASK, nullptr, nullptr,              \
-     hstu::hstu_fwd_kernel<hstu::f8_tag, hstu::otag, D, RAB, MASK>, nullptr, nullptr, nullptr, D, 256, hstu::fwd_wgs_per_cu(D, RAB, MASK)}
+    {"hstu_fwd_f8e4m3_" oname "_d" #D "_rab" #RAB "_mask" #MASK,                                \
+     "hstu_fwd_f8e4m3_" oname "_d" #D "_rab" #RAB "_mask" #MASK "_queues", nullptr,             \
+     hstu::hstu_fwd_kernel<hstu::f8_tag, hstu::otag, D, RAB, MASK>,                             \
+     hstu::queues_kernel<hstu::f8_tag, hstu::otag, D, RAB, MASK>(), nullptr, nullptr, D, 256, hstu::fwd_wgs_per_cu(D, RAB, MASK)}
 #define HSTU_F8_DIMS(otag, oname)                                                                \
     {{{HSTU_F8_VARIANT(otag, oname, 64, 2), HSTU_F8_VARIANT(otag, oname, 128, 2), HSTU_F8_VARIANT(otag, oname, 256, 1)},   \
       {HSTU_F8_BIASED(otag, oname, 64, false, true, 2), HSTU_F8_BIASED(otag, oname, 128, false, true, 2),                  \

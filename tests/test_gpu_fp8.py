@@ -200,6 +200,45 @@ def test_fp8_with_attn_bias_and_custom_mask(batch, heads, heads_k, d, dv, max_le
     check(out, x8, sc, kw)
 
 
+@pytest.mark.parametrize("d,enable_bias,mask_type", [(128, True, 0), (64, True, 3), (128, False, 3)])
+def test_fp8_long_list_with_attn_bias_takes_the_queues(d, enable_bias, mask_type):
+    """A list of several items per resident workgroup with an e4m3 attn_bias and / or custom mask runs on the variant with
+    per-XCD queues, like one without them.  Sequences are independent: a few of them cut out and run alone (a short
+    list: the plain variant) give the same bits, and those rows are compared with the oracle."""
+    from ops_rec import _ops
+
+    batch, heads, max_len = 48, 8, 1024
+    g = torch.Generator(device=DEV).manual_seed(d + mask_type)
+    lengths = torch.randint(300, max_len + 1, (batch,), generator=torch.Generator().manual_seed(d)).tolist()
+    offs = torch.tensor([0] + list(torch.tensor(lengths).cumsum(0)), dtype=torch.int32)
+    total = int(offs[-1])
+    x = [torch.randn(total, heads, d, generator=g, device=DEV) * 0.5 for _ in range(3)]
+    x8, sc = zip(*(workloads.quantize_fp8(t) for t in x))
+    shape = (batch, heads, max_len, max_len)
+    bias = (torch.randn(shape, generator=g, device=DEV) * 0.5).to(torch.float8_e4m3fn) if enable_bias else None
+    mask = (torch.rand(shape, generator=g, device=DEV) < 0.7).float().to(torch.float8_e4m3fn) if mask_type == 3 else None
+    kw = dict(mask=mask, attn_bias=bias, mask_type=mask_type, max_seq_len=max_len, silu_scale=0.0, seq_offset=offs.to(DEV),
+              alpha=d**-0.5)  # fmt: skip
+    prepared = _ops.prepare_forward(*x8, mask, bias, mask_type, max_len, max_len, 0.0, kw["seq_offset"], kw["seq_offset"], None,
+                                    None, 0, kw["alpha"], out_dtype=torch.bfloat16, q_descale=sc[0], k_descale=sc[1],
+                                    v_descale=sc[2])  # fmt: skip
+    assert prepared.kernel_name().endswith("_queues"), prepared.kernel_name()
+    out = ops_rec.hstu_jagged_fp8(*x8, *sc, **kw)
+    assert torch.equal(out, ops_rec.hstu_jagged_fp8(*x8, *sc, **kw))  # reproducible
+    seqs = [0, 17, 40]
+    o = offs.tolist()
+    rows = torch.cat([torch.arange(o[b], o[b + 1]) for b in seqs]).to(DEV)
+    sub_offs = torch.tensor([0] + list(torch.tensor([lengths[b] for b in seqs]).cumsum(0)), dtype=torch.int32)
+    pick = lambda t: None if t is None else t[torch.tensor(seqs, device=DEV)]  # noqa: E731
+    sub8 = tuple(t[rows] for t in x8)
+    subkw = dict(kw, mask=pick(mask), attn_bias=pick(bias), seq_offset=sub_offs.to(DEV))
+    alone = ops_rec.hstu_jagged_fp8(*sub8, *sc, **subkw)
+    assert torch.equal(alone, out[rows])
+    cpu = lambda t: None if t is None else t.cpu()  # noqa: E731
+    check(alone, tuple(t.cpu() for t in sub8), tuple(t.cpu() for t in sc),
+          dict(subkw, mask=cpu(subkw["mask"]), attn_bias=cpu(subkw["attn_bias"]), seq_offset=sub_offs))
+
+
 @pytest.mark.parametrize("silu_scale", [0.0, 0.25])
 def test_reference_entry_point_keeps_the_reference_rounding_point(silu_scale):
     # through hstu_jagged with raw e4m3 tensors P is quantised AFTER silu_scale and the mask, as the reference's golden
