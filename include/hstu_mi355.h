@@ -115,7 +115,7 @@ typedef struct hstu_jagged_fwd_params {
      * e4m3 (round to nearest even), P.V accumulates in fp32, the output is fp16 (the reference's choice,
      * torch_extension/hstu_jagged_plugin.cpp:53-54) or bf16.  attn_bias and a custom mask, when given, are e4m3
      * tensors as well (they follow q's type, op_host/hstu_jagged_forward.cpp:65-66) and are used in fp32; such calls
-     * run on the fixed schedule (no per-XCD queues, no split items).  Head dims above 256 and a head_dim_qk that is
+     * run on the fixed schedule or, for long lists, on the per-XCD queues (their items are not split).  Head dims above 256 and a head_dim_qk that is
      * not a multiple of 16 run on the coverage kernel (vector unit, same semantics).  Where
      * silu_scale is applied relative to the rounding of P is chosen by fp8_scaled_p above.
      * Extension with no counterpart in the reference (its fp8 path is unscaled): per-head dequantisation
