@@ -266,6 +266,26 @@ def test_more_keys_than_queries(monkeypatch):
     check(w, monkeypatch)
 
 
+@pytest.mark.parametrize("n_ctx", [3, 40, 130, 700])
+@pytest.mark.parametrize("order", ["0", "1", "2"])
+def test_context_rows_with_grouped_heads_and_more_keys_than_queries(n_ctx, order, monkeypatch):
+    """Context rows see every history key: the first query tile of a sequence runs ahead of the others, and a key tile's
+    workgroup sweeps the sub-tiles of the context rows, skips those that see nothing of it and goes on at the first causal
+    row -- for every query head of its group.  Context rows within one sub-tile, over several, past the first query tile
+    and longer than a sequence; key ranges longer than the query ranges; every launch order."""
+    lq, lk = [600, 333, 64, 1, 190], [900, 333, 264, 129, 200]
+    g = torch.Generator(device=DEV).manual_seed(n_ctx)
+    mk = lambda n, h, d: (torch.randn(n, h, d, generator=g, device=DEV) * 0.5).to(torch.bfloat16)  # noqa: E731
+    offs = lambda ls: torch.tensor([0] + list(torch.tensor(ls).cumsum(0)), dtype=torch.int32, device=DEV)  # noqa: E731
+    w = workloads.Workload(name="ctx", q=mk(sum(lq), 4, 128), k=mk(sum(lk), 2, 128), v=mk(sum(lk), 2, 128),
+                           seq_offset=offs(lq), max_seq_len=600, silu_scale=1.0, alpha=0.09, seq_offset_k=offs(lk),
+                           max_seq_len_k=904, lengths=lq,
+                           num_context=torch.tensor([n_ctx, n_ctx, 5, 0, n_ctx], dtype=torch.int32, device=DEV),
+                           num_target=torch.tensor([30, 0, 7, 1, 64], dtype=torch.int32, device=DEV), target_group_size=3)  # fmt: skip
+    helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", order)
+    check(w, monkeypatch)
+
+
 @pytest.mark.parametrize("rab", [False, True], ids=["workspace", "bias_gradient"])
 def test_ds_hand_over_with_more_keys_than_queries(rab, monkeypatch):
     # the three-launch order on key ranges longer than the query ranges (delta), grouped heads, 16-byte aligned rows
