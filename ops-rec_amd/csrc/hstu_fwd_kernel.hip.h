@@ -474,6 +474,11 @@ __global__ __launch_bounds__(256, fwd_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hst
     uint16_t* const out16 = static_cast<uint16_t*>(a.out);
     const int n_levels = a.n_qtiles;
     const int n_heads = a.n_heads_q;
+    // Lists by tile: level l holds query tile n_levels - 1 - l (longest sweeps first).  With context rows under the
+    // built-in mask the first tile of a sequence sweeps all of its history keys, so it is the longest item of all and
+    // goes first: level 0 = tile 0, level l >= 1 = tile n_levels - l.
+    const bool ctx_first = a.mask_type == 0 && a.num_ctx != nullptr;
+    auto tile_of_level = [&](int l) -> int { return ctx_first ? (l == 0 ? 0 : n_levels - l) : n_levels - 1 - l; };
 
     // rows past the last offset belong to no sequence and are zero-filled when the workgroup leaves (all workgroups
     // share the job); the offset is requested here, so that nothing waits for it
@@ -502,17 +507,23 @@ __global__ __launch_bounds__(256, fwd_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hst
     // 161 levels the extra additions cost nothing).  In the same pass it gets the first item of list level l = nt
     // of the plain list (one queue, by tile, nothing split): level l' holds the items of query tile
     // n_levels - 1 - l', i.e. n_heads per sequence with more tiles than that, so the levels before l hold
-    // n_heads * sum over nt' of count[nt'] * max(0, nt' - (n_levels - l)) items.
+    // n_heads * sum over nt' of count[nt'] * max(0, nt' - (n_levels - l)) items.  (With tile 0 in level 0, level
+    // l >= 1 starts after all sequences that have a tile at all plus what stood before level l - 1.)
     static_assert(kMaxLevels + 2 <= kThreads, "one thread per level");
     {
         uint32_t above = 0;
         uint32_t items_before = 0;
         if (tid <= n_levels) {
-            const int floor_tiles = n_levels - tid;
+            const int floor_tiles = n_levels - tid + (ctx_first ? 1 : 0);
+            uint32_t with_tiles = 0;
             for (int nt = n_levels; nt >= 1; --nt) {
                 const uint32_t c = s_bucket[nt];
                 above += nt > tid ? c : 0u;
+                with_tiles += c;
                 items_before += nt > floor_tiles ? c * static_cast<uint32_t>(nt - floor_tiles) : 0u;
+            }
+            if (ctx_first) {
+                items_before = tid == 0 ? 0u : items_before + with_tiles;
             }
         }
         __syncthreads();  // the counts have been read by everybody
@@ -537,7 +548,7 @@ __global__ __launch_bounds__(256, fwd_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hst
     //   by tile  - the heaviest (highest) query tile of all its pairs first, then the next tile down, ...: longest
     //              items first.  With a handful of items per workgroup and item lengths between 1 and
     //              max_seq_len / 32 steps this is what keeps the end of the launch short.  Level l of the queue =
-    //              query tile n_levels - 1 - l of its pairs that have it (the sequences at sorted positions
+    //              query tile tile_of_level(l) of its pairs that have it (the sequences at sorted positions
     //              [0, s_rank_start[qt]) have more than qt tiles).
     //   by pair  - pair after pair (most tiles first), the tiles of a pair together, heaviest first: the
     //              workgroups of the XCD sweep the K / V rows of few pairs at a time, and each row is fetched
@@ -570,8 +581,9 @@ __global__ __launch_bounds__(256, fwd_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hst
         }
         const int ratio = a.head_ratio;
         const int n_heads_k = a.n_heads_k;
-        // Splitting long items.  Level l holds the items of query tile qt = n_levels - 1 - l; under the built-in
-        // mask such an item sweeps about 4 (qt + 1) sub-tiles, otherwise all of max_seq_len_k.  With `target` = the
+        // Splitting long items.  Level l holds the items of query tile qt = tile_of_level(l); under the built-in
+        // mask such an item sweeps about 4 (qt + 1) sub-tiles (tile 0 with context rows: all), otherwise all of
+        // max_seq_len_k.  With `target` = the
         // mean number of time steps per workgroup (3 steps of start-up per item included, never below 8), the items
         // of a level whose nominal length exceeds it are listed as m = ceil(nominal / target) entries (at most
         // kMaxParts), one per part of the key range, next to each other in the list.  Part i sweeps the sub-tiles
@@ -590,7 +602,7 @@ __global__ __launch_bounds__(256, fwd_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hst
         uint32_t split_items = 0, split_bufs = 0;
         auto nominal_steps = [&](int qt) -> uint32_t {
             const int all = (a.max_k + 31) / 32;
-            if (a.mask_type != 0) {
+            if (a.mask_type != 0 || (ctx_first && qt == 0)) {
                 return static_cast<uint32_t>(all);
             }
             const int causal = 4 * (qt + 1) + (a.max_k > a.max_q ? (a.max_k - a.max_q) / 32 : 0);
@@ -599,8 +611,8 @@ __global__ __launch_bounds__(256, fwd_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hst
         if constexpr (SPLIT) {
             uint32_t steps = 0, items = 0;
             for (int l = 0; l < n_levels; ++l) {
-                const uint32_t cnt = s_rank_start[n_levels - 1 - l] * static_cast<uint32_t>(n_heads);
-                steps += cnt * (nominal_steps(n_levels - 1 - l) + 3u);
+                const uint32_t cnt = s_rank_start[tile_of_level(l)] * static_cast<uint32_t>(n_heads);
+                steps += cnt * (nominal_steps(tile_of_level(l)) + 3u);
                 items += cnt;
             }
             split_target = steps / gridDim.x;
@@ -616,8 +628,8 @@ __global__ __launch_bounds__(256, fwd_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hst
                 uint32_t entries = 0;
                 const float inv_target = 1.0f / static_cast<float>(split_target);
                 for (int l = 0; l < n_levels; ++l) {
-                    const uint32_t cnt = s_rank_start[n_levels - 1 - l] * static_cast<uint32_t>(n_heads);
-                    const uint32_t m = static_cast<uint32_t>(static_cast<float>(nominal_steps(n_levels - 1 - l)) * inv_target + 0.999f);
+                    const uint32_t cnt = s_rank_start[tile_of_level(l)] * static_cast<uint32_t>(n_heads);
+                    const uint32_t m = static_cast<uint32_t>(static_cast<float>(nominal_steps(tile_of_level(l))) * inv_target + 0.999f);
                     entries += cnt * (m > static_cast<uint32_t>(kMaxParts) ? static_cast<uint32_t>(kMaxParts) : (m < 1u ? 1u : m));
                 }
                 if (entries > gridDim.x) {
@@ -631,8 +643,8 @@ __global__ __launch_bounds__(256, fwd_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hst
         for (int l = 0; l < n_levels; ++l) {
             s_queue_start[tid][l] = acc;
             if constexpr (SPLIT) {
-                const uint32_t cnt = s_rank_start[n_levels - 1 - l] * static_cast<uint32_t>(n_heads);
-                uint32_t m = (nominal_steps(n_levels - 1 - l) + split_target - 1u) / split_target;
+                const uint32_t cnt = s_rank_start[tile_of_level(l)] * static_cast<uint32_t>(n_heads);
+                uint32_t m = (nominal_steps(tile_of_level(l)) + split_target - 1u) / split_target;
                 m = m > static_cast<uint32_t>(kMaxParts) ? static_cast<uint32_t>(kMaxParts) : m;
                 if (m > 1u && (split_items + cnt > static_cast<uint32_t>(kMaxSplitItems) || split_bufs + cnt * m > a.ws_parts)) {
                     m = 1u;
@@ -655,7 +667,7 @@ __global__ __launch_bounds__(256, fwd_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hst
                 const uint32_t mine = (p1 + kQueues - 1 - tid) / kQueues - (p0 + kQueues - 1 - tid) / kQueues;
                 acc += mine * static_cast<uint32_t>(nt * ratio);
             } else if (tid == 0) {
-                acc += s_rank_start[n_levels - 1 - l] * static_cast<uint32_t>(n_heads);  // every pair that has this tile
+                acc += s_rank_start[tile_of_level(l)] * static_cast<uint32_t>(n_heads);  // every pair that has this tile
             }
         }
         s_queue_start[tid][n_levels] = acc;
@@ -915,7 +927,7 @@ __global__ __launch_bounds__(256, fwd_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hst
             p_item = p_first + ((fq_queue + kQueues - (p_first & (kQueues - 1))) & (kQueues - 1)) + m_item * kQueues;
         } else {
             // item j of level lvl (query tile qt) = pair j / ratio, query head (kv head) * ratio + j % ratio
-            qt = n_levels - 1 - lvl;
+            qt = tile_of_level(lvl);
             int j_whole = j_item;
             if constexpr (SPLIT) {
                 // entry j of a split level = part j % m of item j / m
@@ -989,7 +1001,7 @@ __global__ __launch_bounds__(256, fwd_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hst
             }
         }
         if (lane == 0) {
-            rec[1] = static_cast<uint32_t>(n_levels - 1 - lvl);
+            rec[1] = static_cast<uint32_t>(tile_of_level(lvl));
             rec[2] = static_cast<uint32_t>(seq);
             rec[3] = static_cast<uint32_t>(hk_item * a.head_ratio + r_item);
             rec[4] = static_cast<uint32_t>(hk_item);
@@ -1302,6 +1314,21 @@ __global__ __launch_bounds__(256, fwd_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hst
         const bool any_hole = wb.any_hole;
         const int nx_all = (wb.lim_max + 31) / 32;  // sub-tiles this wavefront's rows can see (<= n_sub)
         const int nx_w = (SPLIT && x_end < nx_all) ? x_end : nx_all;  // ... and the end of what it works on in this part
+        // Context rows: the sub-tiles [rows_only_from, rows_only_to) of this wavefront lie past the limit of every row
+        // of its that is not a context row and wholly below the limit of every context row (and before the target keys,
+        // when target rows carve holes): a row sees such a sub-tile whole or not at all, and its visibility is one
+        // comparison per lane instead of one per score.  These are nearly all steps of a sequence's first query tile.
+        int rows_only_from = 0, rows_only_to = 0;
+        if (a.mask_type == 0 && wave_active && wr0 < n_ctx) {
+            const int wr1 = (wr0 + kWaveM < sq) ? wr0 + kWaveM : sq;
+            int other_hi = n_ctx < wr1 ? wr1 + delta : 0;  // limit of the last row that is not a context row
+            other_hi = other_hi < 0 ? 0 : (other_hi > sk ? sk : other_hi);
+            int ctx_lo = wr0 + delta + 1 > hist_k ? wr0 + delta + 1 : hist_k;  // limit of the first context row
+            ctx_lo = (any_hole && ctx_lo > hist_k) ? hist_k : ctx_lo;
+            ctx_lo = ctx_lo < 0 ? 0 : (ctx_lo > sk ? sk : ctx_lo);
+            rows_only_from = (other_hi + 31) >> 5;
+            rows_only_to = ctx_lo >> 5;
+        }
         // per-lane bounds relative to the lane's first key of a sub-tile (key = c0 + 4*lh + kk)
         const int lim_lane = lim - 4 * lh;
         const int hole_lo_lane = hole_lo - 4 * lh;
@@ -1847,7 +1874,13 @@ __global__ __launch_bounds__(256, fwd_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hst
                 }
             }
             // visibility: key c0 + 8*(e/4) + 4*lh + e%4 of element e is hidden at or past lim and inside the hole
-            if (do_silu && !full) {
+            if (do_silu && !full && t >= rows_only_from && t < rows_only_to) {
+                const uint32_t keep = lim >= c0 + 32 ? 0xffffffffu : 0u;
+#pragma unroll
+                for (int w = 0; w < (F8 ? 4 : 8); ++w) {
+                    pk_cur[w] &= keep;
+                }
+            } else if (do_silu && !full) {
                 constexpr int EPW = F8 ? 4 : 2;  // packed elements per word
 #pragma unroll
                 for (int w = 0; w < 16 / EPW; ++w) {

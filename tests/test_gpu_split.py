@@ -69,6 +69,16 @@ def test_few_sequences_rab_context_targets(monkeypatch):
     check_split(w, monkeypatch)
 
 
+@pytest.mark.parametrize("n_ctx,max_target,group,dim", [(40, 0, 0, 128), (8, 30, 2, 128), (33, 70, 1, 64)])
+def test_context_rows_first_tile_sweeps_all_history(n_ctx, max_target, group, dim, monkeypatch):
+    # with context rows the first query tile of a sequence is its longest item: it stands first in the list (and is
+    # split like the top tile), and nearly all of its steps see a sub-tile whole from the context rows and not at
+    # all from the others (the contexts end in the first or the second wavefront of the tile)
+    w = workloads.make("ctx", dtype=torch.bfloat16, device=DEV, seed=12, batch=3, heads=2, dim=dim, lo=900, hi=2600,
+                       max_seq_len=2600, num_context=n_ctx, max_target=max_target, target_group_size=group)  # fmt: skip
+    check_split(w, monkeypatch)
+
+
 def test_custom_mask_f16_grouped_heads(monkeypatch):
     w = workloads.make("mask", dtype=torch.float16, device=DEV, seed=5, batch=2, heads=4, heads_k=2, dim=64, lo=700,
                        hi=1800, max_seq_len=1800)  # fmt: skip
