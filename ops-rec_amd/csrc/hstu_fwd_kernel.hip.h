@@ -1329,6 +1329,8 @@ __global__ __launch_bounds__(256, fwd_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hst
             rows_only_from = (other_hi + 31) >> 5;
             rows_only_to = ctx_lo >> 5;
         }
+        // (one scalar register: the d = 128 variants have none to spare)
+        const uint32_t rows_only = static_cast<uint32_t>(uniform(rows_only_from | (rows_only_to << 16)));
         // per-lane bounds relative to the lane's first key of a sub-tile (key = c0 + 4*lh + kk)
         const int lim_lane = lim - 4 * lh;
         const int hole_lo_lane = hole_lo - 4 * lh;
@@ -1874,8 +1876,9 @@ __global__ __launch_bounds__(256, fwd_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hst
                 }
             }
             // visibility: key c0 + 8*(e/4) + 4*lh + e%4 of element e is hidden at or past lim and inside the hole
-            if (do_silu && !full && t >= rows_only_from && t < rows_only_to) {
-                const uint32_t keep = lim >= c0 + 32 ? 0xffffffffu : 0u;
+            if (do_silu && !full && t >= static_cast<int>(rows_only & 0xffffu) && t < static_cast<int>(rows_only >> 16)) {
+                // (a context row's limit lies at or past the end of the sub-tile, any other row's at or before its start)
+                const uint32_t keep = lim_lane > c0 ? 0xffffffffu : 0u;
 #pragma unroll
                 for (int w = 0; w < (F8 ? 4 : 8); ++w) {
                     pk_cur[w] &= keep;
