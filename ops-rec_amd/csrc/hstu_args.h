@@ -22,6 +22,11 @@ constexpr int fwd_wgs_per_cu(int d, bool rab, bool mask)
 {
     return (!rab && !mask && d <= 64) ? (d <= 32 ? 4 : 3) : (d <= 32 && !(rab && mask)) ? 3 : (d <= 128 ? 2 : 1);
 }
+// Lines per query row of the pair plane in its full form (every 32-key block of the row): odd, so that the 32 lines
+// one store instruction of a wavefront writes -- the same block of 32 consecutive rows -- fall on different memory
+// channels.  With max_seq_len_k 8192 the plain count, 256 lines = 32 KiB, put them all on one (measured on MI355X, 2
+// sequences x 4 heads of 4096 .. 8192 rows: query-tile kernel 445 us, 298 us with the odd pitch).
+constexpr int64_t pair_full_pitch_lines(int64_t max_k) { return ((max_k + 31) / 32) | 1; }
 constexpr int kShortThreads = 512;  // threads of a workgroup of the forward kernel for short lists (eight wavefronts of 16 query rows)
 constexpr int kTinyThreads = 128;   // threads of a workgroup of the backward kernel for tiny sequences (two wavefronts of 16 query rows)
 constexpr int kTinyRows = 32;       // the longest sequence (rows and keys) that kernel takes; the forward one: 32 or 64, four threads per row

@@ -113,14 +113,14 @@ __device__ __forceinline__ int live_levels(const BwdArgs& a, int lane, int rows,
 // The pair plane of the 16-bit kernels: what the query-tile kernel hands to the key-tile workgroups of the next launch.
 // One 128-byte line per query row and 32-key block: the block's 32 dS values, then its 32 P values.  Lines are packed
 // per head by global query row (offs_q[b] + r; no room for rows that the batch does not have), the lines of a row side by
-// side -- all ceil(max_k / 32) blocks of it, or, for a causal mask over equal query and key offsets without context
+// side -- all ceil(max_k / 32) blocks of it (at a pitch of pair_full_pitch_lines() lines), or, for a causal mask over equal query and key offsets without context
 // rows (plane_tri; the host knows this much without reading the offsets), only the blocks 0 .. G that rows of the
 // sequence's 32-row group G can see.  The host sizes the triangular form without knowing the lengths: 32 rows of slack
 // per sequence make ((offs_q[b] + 32 b) (n_blk + 1) + 1) / 2 lines an upper bound of what the sequences ahead of b hold.
 __device__ __forceinline__ int64_t pair_lines_ahead(const BwdArgs& a, int64_t q0, int b)
 {
     const int64_t n_blk = (a.max_k + 31) / 32;
-    return a.plane_tri ? ((q0 + 32 * static_cast<int64_t>(b)) * (n_blk + 1) + 1) / 2 : q0 * n_blk;
+    return a.plane_tri ? ((q0 + 32 * static_cast<int64_t>(b)) * (n_blk + 1) + 1) / 2 : q0 * pair_full_pitch_lines(a.max_k);
 }
 // first byte of sequence b's lines for head h, and their extent
 __device__ __forceinline__ uint8_t* pair_plane_of(const BwdArgs& a, int64_t q0, int b, int h)
@@ -130,15 +130,15 @@ __device__ __forceinline__ uint8_t* pair_plane_of(const BwdArgs& a, int64_t q0, 
 __device__ __forceinline__ uint32_t pair_seq_bytes(const BwdArgs& a, int sq)
 {
     const uint32_t groups = static_cast<uint32_t>(sq + 31) >> 5;
-    const uint32_t n_blk = static_cast<uint32_t>(a.max_k + 31) >> 5;
-    return (a.plane_tri ? 16u * groups * (groups + 1u) : static_cast<uint32_t>(sq) * n_blk) * 128u;
+    const uint32_t pitch = static_cast<uint32_t>(pair_full_pitch_lines(a.max_k));
+    return (a.plane_tri ? 16u * groups * (groups + 1u) : static_cast<uint32_t>(sq) * pitch) * 128u;
 }
 // byte offset, from the sequence's first line, of row r's line for block 0
 __device__ __forceinline__ uint32_t pair_row_offset(const BwdArgs& a, int r)
 {
     const uint32_t g = static_cast<uint32_t>(r) >> 5;
-    const uint32_t n_blk = static_cast<uint32_t>(a.max_k + 31) >> 5;
-    return (a.plane_tri ? 16u * g * (g + 1u) + (static_cast<uint32_t>(r) & 31u) * (g + 1u) : static_cast<uint32_t>(r) * n_blk) * 128u;
+    const uint32_t pitch = static_cast<uint32_t>(pair_full_pitch_lines(a.max_k));
+    return (a.plane_tri ? 16u * g * (g + 1u) + (static_cast<uint32_t>(r) & 31u) * (g + 1u) : static_cast<uint32_t>(r) * pitch) * 128u;
 }
 
 // Windows (head dims above 256 on the kernels of the slot 256): the real head of head h of a launch, its K/V head, and
@@ -472,6 +472,20 @@ __global__ __launch_bounds__(256, bwd_dq_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void 
     row_bounds(sq_info, a.mask_type, a.target_group, row, lim, hole_lo, hole_hi);
     const WaveBounds wb = wave_bounds(a.mask_type, wr0, sq, sk, sq_info.n_ctx, sq_info.n_tgt, a.target_group, wr0 < sq);
     const int nx_w = (swept_key_limit(a, sq_info, wr0) + 31) / 32;  // (= wb.lim_max: a wavefront is a 32-row group here)
+    // Context rows: the keys [row_only_lo, row_only_hi) lie past the limit of every row of this wavefront that is not a
+    // context row and below the limit of each of its context rows (and before the target keys, when target rows carve
+    // holes): a row sees a sub-tile in that range whole or not at all -- nearly every step of a sequence's first tile.
+    int row_only_lo = 0, row_only_hi = 0;
+    if (a.mask_type == 0 && wr0 < sq && wr0 < sq_info.n_ctx) {
+        const int wr1 = (wr0 + kWaveM < sq) ? wr0 + kWaveM : sq;
+        int other_hi = sq_info.n_ctx < wr1 ? wr1 + sq_info.delta : 0;
+        other_hi = other_hi < 0 ? 0 : (other_hi > sk ? sk : other_hi);
+        int ctx_lo = wr0 + sq_info.delta + 1 > sq_info.hist_k ? wr0 + sq_info.delta + 1 : sq_info.hist_k;
+        ctx_lo = (wb.any_hole && ctx_lo > sq_info.hist_k) ? sq_info.hist_k : ctx_lo;
+        ctx_lo = ctx_lo < 0 ? 0 : (ctx_lo > sk ? sk : ctx_lo);
+        row_only_lo = uniform(other_hi);
+        row_only_hi = uniform(ctx_lo);
+    }
 
     const uint32_t bias_bytes = static_cast<uint32_t>(a.max_q) * static_cast<uint32_t>(a.max_k) * 2u;
     const int64_t bias_plane = bias_plane_of(a, b, h);
@@ -664,7 +678,16 @@ __global__ __launch_bounds__(256, bwd_dq_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void 
         // wavefront's rows (as in the forward): key c0 + 8 (e / 4) + 4 lh + e % 4 of element e is hidden at or past
         // lim and inside the hole
         const bool full = (c0 + 32 <= wb.lim_min) && !(wb.any_hole && c0 + 32 > sq_info.hist_k && c0 < wb.hole_hi_max);
-        if (!full) {
+        if (!full && c0 >= row_only_lo && c0 + 32 <= row_only_hi) {
+            const uint32_t keep = lim > c0 ? 0xffffffffu : 0u;  // (a context row's limit is at or past c0 + 32, any other row's at or before c0)
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                pk[i] &= keep;
+                if constexpr (WANT_P) {
+                    pp[i] &= keep;
+                }
+            }
+        } else if (!full) {
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 uint32_t keep = 0;

@@ -756,9 +756,10 @@ static PairPlane pair_plane(const hstu_jagged_fwd_params* f)
     pp.tri = f->mask_type == HSTU_MASK_TRIL && f->num_context == nullptr && f->seq_offset_k == f->seq_offset_q &&
              f->total_k == f->total_q;
     const int64_t groups = ((f->max_seq_len_q < f->max_seq_len_k ? f->max_seq_len_q : f->max_seq_len_k) + 31) / 32;
-    pp.head_lines = pp.tri ? ((f->total_q + 32 * batch) * (n_blk + 1) + 1) / 2 : f->total_q * n_blk;
+    const int64_t pitch = hstu::pair_full_pitch_lines(f->max_seq_len_k);
+    pp.head_lines = pp.tri ? ((f->total_q + 32 * batch) * (n_blk + 1) + 1) / 2 : f->total_q * pitch;
     pp.bytes = f->num_heads_q * pp.head_lines * 128;
-    pp.fits_32 = (pp.tri ? 16 * groups * (groups + 1) : f->max_seq_len_q * n_blk) * 128 < (1LL << 31);
+    pp.fits_32 = (pp.tri ? 16 * groups * (groups + 1) : f->max_seq_len_q * pitch) * 128 < (1LL << 31);
     return pp;
 }
 

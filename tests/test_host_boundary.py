@@ -433,7 +433,8 @@ def test_backward_workspace_follows_the_launch_order(monkeypatch):
         return heads * (((rows + 32 * batch) * (blocks + 1) + 1) // 2) * 128
 
     def pair_all_blocks(rows=20292, heads=4, blocks=32):
-        return heads * rows * blocks * 128
+        # (an odd number of lines per row: the lines of a block's 32 rows then fall on different memory channels)
+        return heads * rows * (blocks | 1) * 128
 
     one = 32 * 4 * 1024 * 1024 * 2
     full = 32 * 1024
