@@ -2,7 +2,7 @@
 times, the order the library's rule takes and how far that is from the best (markdown table on stdout).
 
     python ops-rec_amd/examples/hstu_bwd_order_sweep.py [--set heldout|fit|bias] [--launches 10]
-    python ops-rec_amd/examples/hstu_bwd_order_sweep.py --shape 1,4,4,128,1024,1024,causal --only planes   # one shape, one
+    python ops-rec_amd/examples/hstu_bwd_order_sweep.py --shape 1,4,4,128,1024,1024,causal [--bias] --only planes   # one shape, one
                                                         # order: what a kernel trace or a counter run of a launch order wants
 
 Orders (forced with HSTU_MI355_BWD_HANDOFF = 0 / 1 / 2, read once per process, hence ``reload_switches``):
@@ -81,6 +81,7 @@ def main():
     ap.add_argument("--launches", type=int, default=10)
     ap.add_argument("--shape", action="append", default=[],
                     help="batch,heads,kv_heads,dim,shortest,longest,causal|none (repeatable); instead of --set")
+    ap.add_argument("--bias", action="store_true", help="run the shapes of --shape with an attn_bias and its gradient")
     ap.add_argument("--only", choices=sorted(NAMES.values()), help="run this launch order only and print its time")
     args = ap.parse_args()
     bwd = ops_rec.ascendc.attention.hstu_jagged_backward
@@ -99,7 +100,7 @@ def main():
                            lo=lo, hi=hi, max_seq_len=max_len, seed=batch + hi)  # fmt: skip
         grad = (torch.randn(w.q.shape[0], heads, dim, device="cuda") * 0.1).to(torch.bfloat16)
         rab = None
-        if args.set == "bias":
+        if args.bias if args.shape else args.set == "bias":
             rab = (torch.randn(batch, heads, max_len, max_len, device="cuda") * 0.1).to(torch.bfloat16)
         call = (grad, w.q, w.k, w.v, None, rab, 0 if mask == "causal" else 2, max_len, w.silu_scale, w.seq_offset, None, None, 0, w.alpha)
         times = {}
