@@ -255,7 +255,7 @@ HSTU_API int hstu_paged_fwd(const hstu_paged_fwd_params* params, void* workspace
 HSTU_API const char* hstu_last_error(void);
 
 /* The library's process-wide switches (HSTU_MI355_SPLIT, HSTU_MI355_SHORT, HSTU_MI355_GENERIC_BACKWARD,
- * HSTU_MI355_BWD_HANDOFF, HSTU_MI355_BWD_WORKSPACE_MB) are read from the environment once, at the first call that
+ * HSTU_MI355_BWD_HANDOFF, HSTU_MI355_BWD_WORKSPACE_MB, HSTU_MI355_BWD_PAIR_MAJOR) are read from the environment once, at the first call that
  * looks at one; this reads them again.  No counterpart in the reference: it is for a test or a tool that changes the
  * environment after the library has been used.  Not safe against launches running at the same time in other threads. */
 HSTU_API void hstu_reload_switches(void);

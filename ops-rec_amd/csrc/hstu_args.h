@@ -111,6 +111,9 @@ struct BwdArgs {
     // win_only >= 0: the launch covers that window only (its grid counts real heads).  Otherwise win = 1, win_only = -1.
     int win;
     int win_only;
+    // Order of the (tile level, pair) slots in the grids of the tuned 16-bit kernels (hstu_bwd_kernel.hip.h, slot_of):
+    // 0 = level after level (heaviest tiles of all pairs first), 1 = pair after pair, the pairs dealt to the 8 XCDs.
+    int pair_major;
     float* partial;  // S and dP summed over the first window, fp32, for the launch that adds the second (or null)
     int64_t drab_clear_bytes;  // > 0: the key-tile kernel clears this many bytes at drab beside its work
     const void* offs_q;

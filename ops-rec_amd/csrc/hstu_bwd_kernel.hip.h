@@ -110,6 +110,27 @@ __device__ __forceinline__ int live_levels(const BwdArgs& a, int lane, int rows,
     return n < 1 ? 1 : (n < host_levels ? n : host_levels);
 }
 
+// Slot `slot` of a grid over (tile level, pair) -> its level and pair (`pair` may come out at or past n_pairs: a slot of
+// the rounded-up grid that has no work).  Level after level, all pairs of the heaviest level first, keeps the end of a
+// launch short -- but the workgroups resident at any time then belong to as many pairs as there are, and once the K / V (or
+// Q / dO) rows of all pairs together no longer fit the caches every one of them streams its rows from memory.  Pair after
+// pair (a.pair_major; the host's choice for launches of many items over more rows than the caches hold): workgroups go to
+// the 8 XCDs in turn, so slot i belongs to XCD i mod 8; XCD x takes the pairs x, x + 8, ... one after the other, the levels
+// of a pair next to each other, heaviest first, so that the tiles of a pair run side by side on one XCD and find its rows
+// in that XCD's L2.  (The host sizes such a grid as n_levels x 8 x ceil(n_pairs / 8) slots.)
+__device__ __forceinline__ void slot_of(const BwdArgs& a, int slot, int n_levels, int n_pairs, int& lvl, int& pair)
+{
+    if (a.pair_major == 0) {
+        lvl = slot / n_pairs;
+        pair = slot - lvl * n_pairs;
+        return;
+    }
+    const int j = slot >> 3;
+    const int turn = j / n_levels;
+    lvl = j - turn * n_levels;
+    pair = turn * 8 + (slot & 7);
+}
+
 // The pair plane of the 16-bit kernels: what the query-tile kernel hands to the key-tile workgroups of the next launch.
 // One 128-byte line per query row and 32-key block: the block's 32 dS values, then its 32 P values.  Lines are packed
 // per head by global query row (offs_q[b] + r; no room for rows that the batch does not have), the lines of a row side by
@@ -369,8 +390,8 @@ __global__ __launch_bounds__(256, bwd_dq_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void 
     }
     const int grid_heads = a.win_only >= 0 ? a.n_heads_q / a.win : a.n_heads_q;
     const int per_level = a.n_batch * grid_heads;
-    const int lvl = static_cast<int>(blockIdx.x) / per_level;
-    const int rem = static_cast<int>(blockIdx.x) - lvl * per_level;
+    int lvl, rem;
+    slot_of(a, static_cast<int>(blockIdx.x), a.n_qtiles, per_level, lvl, rem);
     // (heaviest tiles first, counted from the highest level that exists in the batch; with context rows the first tile of a
     // sequence sweeps all of its history keys and goes ahead)
     const int n_levels = live_levels(a, lane, kBlockM, a.n_qtiles);
@@ -382,8 +403,8 @@ __global__ __launch_bounds__(256, bwd_dq_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void 
     if constexpr (PHASE != 1) {
         zero_tail_rows(a.dq, a.offs_q, a.n_batch, a.idx64, a.total_q, static_cast<int64_t>(a.n_heads_q) * a.d_qk, 256);
     }
-    if (lvl >= n_levels) {
-        return;  // a level that no sequence of the batch has
+    if (lvl >= n_levels || rem >= per_level) {
+        return;  // a level that no sequence of the batch has, or a slot past the last pair
     }
     const SeqInfo sq_info = load_seq(a, b);
     const int sq = sq_info.sq, sk = sq_info.sk;
@@ -861,8 +882,8 @@ __global__ __launch_bounds__(kDkvThreads, (MODE == 2 || MODE >= 4) ? bwd_dk_from
     // key tile 0 is seen by the most query rows: heaviest first
     const int per_level = a.n_batch * a.n_heads_k;
     const int tile_slot = static_cast<int>(paired ? (blockIdx.x >> 4) * 8 + (blockIdx.x & 7) : blockIdx.x);
-    const int kt_idx = tile_slot / per_level;
-    const int rem = tile_slot - kt_idx * per_level;
+    int kt_idx, rem;
+    slot_of(a, tile_slot, a.n_ktiles, per_level, kt_idx, rem);
     const int b = rem / a.n_heads_k;
     const int hk = rem - b * a.n_heads_k;
     if constexpr (MODE != 1) {
@@ -877,6 +898,9 @@ __global__ __launch_bounds__(kDkvThreads, (MODE == 2 || MODE >= 4) ? bwd_dk_from
         // steps of the sweep instead, a few stores per thread and step, was measured slower: stores and tile
         // requests retire through one in-order counter.)
         clear_share(a.drab, a.drab_clear_bytes, blockIdx.x, gridDim.x, tid, kDkvThreads);
+    }
+    if (rem >= per_level) {
+        return;  // (pair after pair: a slot past the last pair)
     }
     const SeqInfo si = load_seq(a, b);
     const int sq = si.sq, sk = si.sk;

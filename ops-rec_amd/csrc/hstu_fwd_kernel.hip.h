@@ -557,7 +557,10 @@ __global__ __launch_bounds__(256, fwd_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hst
     // "By pair" starts the heavy tiles of late pairs late; that is harmless when there are many items per
     // workgroup and the late pairs are short (a jagged batch), and costly when all sequences are equally long.
     // It is chosen when the list has at least 4 items per workgroup and the mean tile count of the sequences is
-    // at most 0.7 of the largest.
+    // at most 0.7 of the largest, and whatever the lengths from 6 items per workgroup on: by tile, the resident workgroups
+    // of a long list all work on different pairs, and every item streams its keys from memory (128 x 4 heads of 7621
+    // rows, d 128: 61 GB in 11.05 ms by tile, 7.21 ms by pair; 64 x 4 of 4096 rows 1.39 -> 1.14 ms; level at 8 items per
+    // workgroup of 1024 or 512 rows).
     // "By tile" runs as ONE queue shared by all workgroups (the order that matters there is global), "by pair" as
     // one queue per XCD.
     if ((QUEUES || SPLIT) && tid < (QUEUES ? kQueues : 1)) {
@@ -573,8 +576,8 @@ __global__ __launch_bounds__(256, fwd_wgs_per_cu(D, HAS_RAB, HAS_MASK)) void hst
                 seqs += c;
                 nt_max = c != 0 ? nt : nt_max;
             }
-            by_pair = tiles * static_cast<uint32_t>(n_heads) >= 4u * gridDim.x &&
-                      10u * tiles <= 7u * seqs * static_cast<uint32_t>(nt_max);
+            const uint32_t items = tiles * static_cast<uint32_t>(n_heads);
+            by_pair = (items >= 4u * gridDim.x && 10u * tiles <= 7u * seqs * static_cast<uint32_t>(nt_max)) || items >= 6u * gridDim.x;
         }
         if (tid == 0) {
             s_item[4] = by_pair ? 1u : 0u;

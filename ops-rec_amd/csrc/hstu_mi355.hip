@@ -82,14 +82,16 @@ int compute_units(int* out)
 //   HSTU_MI355_GENERIC_BACKWARD=1  backward: the generic kernels also where tuned ones exist (for comparisons)
 //   HSTU_MI355_BWD_HANDOFF=0/1/2   backward: force the launch order (two launches / three / planes)
 //   HSTU_MI355_BWD_WORKSPACE_MB=n  backward: the largest workspace the library asks for
+//   HSTU_MI355_BWD_PAIR_MAJOR=0/1  backward: the grids of the tuned 16-bit kernels level after level / pair after pair
 struct Switches {
     int split;
     int short_lists;
     int generic_backward;
     int bwd_handoff;
     long long bwd_workspace_mb;
+    int bwd_pair_major;
 };
-Switches g_switches = {-1, -1, -1, -1, -1};
+Switches g_switches = {-1, -1, -1, -1, -1, -1};
 std::once_flag g_switches_once;
 
 int switch_digit(const char* name, int max_digit)
@@ -108,6 +110,7 @@ void read_switches()
     g_switches.bwd_handoff = switch_digit("HSTU_MI355_BWD_HANDOFF", 2);
     const char* const mb = getenv("HSTU_MI355_BWD_WORKSPACE_MB");
     g_switches.bwd_workspace_mb = (mb != nullptr && mb[0] >= '0' && mb[0] <= '9') ? atoll(mb) : -1;
+    g_switches.bwd_pair_major = switch_digit("HSTU_MI355_BWD_PAIR_MAJOR", 1);
 }
 const Switches& switches()
 {
@@ -1170,12 +1173,33 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
     }
     const bool generic = is_generic_bwd(var);
     const BwdPlan plan = plan_bwd(p, var);
+    const hstu::DqShortVariant* const dq_short = generic ? nullptr : dq_short_variant(p, var);
+    // The order of the slots in the grids of the tuned kernels (slot_of in hstu_bwd_kernel.hip.h): pair after pair, on one
+    // XCD each, where level after level would have every resident workgroup stream another pair's rows from memory --
+    // K, V, Q and dO of the call together beyond the 256 MB memory-side cache, at the head-dim slots that run two workgroups
+    // per CU (at the slot 256 a step takes twice as long per byte it streams, and memory keeps up: 96 x 2 heads of 3072 rows
+    // 6.59 ms level after level, 6.90 ms pair after pair) -- and the launch is long enough for the pairs left at its end not to
+    // matter (8 tiles per workgroup that fits the machine, by the mean length).  Measured, bf16 d 128, 4 heads: 128 x 7621 rows
+    // 40.5 -> 32.9 ms, 64 x 4096 rows 5.83 -> 5.04 ms, 64 x 1024..4096 rows 2.92 -> 2.58 ms, 256 x 1024 rows level.
+    if (!generic && dq_short == nullptr) {
+        int cus = 0;
+        if (compute_units(&cus) != HSTU_OK) {
+            return HSTU_ERR_RUNTIME;
+        }
+        const int64_t row_bytes = (f->head_dim_qk + f->head_dim_v) * es;
+        const int64_t streamed = f->total_k * f->num_heads_k * row_bytes + f->total_q * f->num_heads_q * row_bytes;
+        const int64_t tiles = (f->total_q / hstu::kBlockM) * f->num_heads_q;
+        const int64_t dmax = f->head_dim_qk > f->head_dim_v ? f->head_dim_qk : f->head_dim_v;
+        const bool long_launch = dmax <= 128 && streamed >= (512LL << 20) && tiles >= 16LL * cus;
+        const int forced = switches().bwd_pair_major;
+        a.pair_major = forced >= 0 ? forced : (long_launch ? 1 : 0);
+    }
+    const int64_t pairs_q = static_cast<int64_t>(a.n_batch) * a.n_heads_q, pairs_k = static_cast<int64_t>(a.n_batch) * a.n_heads_k;
     // the tuned key-tile kernel runs a dV and a dK workgroup per tile, the generic one a workgroup per tile
-    const int64_t n_kv_slots = static_cast<int64_t>(a.n_ktiles) * a.n_batch * a.n_heads_k;
+    const int64_t n_kv_slots = static_cast<int64_t>(a.n_ktiles) * (a.pair_major ? 8 * ((pairs_k + 7) / 8) : pairs_k);
     // (with both roles in a launch: groups of 8 dV workgroups followed by their 8 dK workgroups, whole groups)
     const int64_t grid_kv = generic ? n_kv_slots : 16 * ((n_kv_slots + 7) / 8);
-    const int64_t grid_q = static_cast<int64_t>(a.n_qtiles) * a.n_batch * a.n_heads_q;
-    const hstu::DqShortVariant* const dq_short = generic ? nullptr : dq_short_variant(p, var);
+    const int64_t grid_q = static_cast<int64_t>(a.n_qtiles) * (a.pair_major ? 8 * ((pairs_q + 7) / 8) : pairs_q);
     if (grid_kv > 0x7fffffffLL || grid_q > 0x7fffffffLL) {
         return fail(HSTU_ERR_INVALID, "grid out of range");
     }

@@ -286,6 +286,38 @@ def test_context_rows_with_grouped_heads_and_more_keys_than_queries(n_ctx, order
     check(w, monkeypatch)
 
 
+@pytest.mark.parametrize("order", ["0", "1", "2"])
+@pytest.mark.parametrize("rab", [False, True], ids=["plain", "bias_gradient"])
+def test_grids_pair_after_pair_give_the_same_bits(order, rab, monkeypatch):
+    """Long launches over more rows than the caches hold run their grids pair after pair, the pairs dealt to the XCDs,
+    instead of level after level (HSTU_MI355_BWD_PAIR_MAJOR forces either): the same workgroups in another order, so every
+    gradient must come out bit for bit the same -- here with 30 (query) and 15 (key) pairs, neither a multiple of 8, so that
+    the rounded-up grids have slots without a pair, with empty and one-row sequences, context rows, targets, and more keys
+    than queries, in every launch order; the level-after-level result is checked against the oracle as usual."""
+    lq, lk = [600, 333, 0, 1, 190], [900, 333, 0, 129, 200]
+    g = torch.Generator(device=DEV).manual_seed(77)
+    mk = lambda n, h, d: (torch.randn(n, h, d, generator=g, device=DEV) * 0.5).to(torch.bfloat16)  # noqa: E731
+    offs = lambda ls: torch.tensor([0] + list(torch.tensor(ls).cumsum(0)), dtype=torch.int32, device=DEV)  # noqa: E731
+    bias = (torch.randn(5, 6, 600, 904, generator=g, device=DEV) * 0.5).to(torch.bfloat16) if rab else None
+    w = workloads.Workload(name="pairs", q=mk(sum(lq), 6, 128), k=mk(sum(lk), 3, 128), v=mk(sum(lk), 3, 128),
+                           seq_offset=offs(lq), max_seq_len=600, silu_scale=1.0, alpha=0.09, seq_offset_k=offs(lk),
+                           max_seq_len_k=904, attn_bias=bias, lengths=lq,
+                           num_context=torch.tensor([3, 40, 0, 0, 5], dtype=torch.int32, device=DEV),
+                           num_target=torch.tensor([30, 0, 0, 1, 64], dtype=torch.int32, device=DEV), target_group_size=3)  # fmt: skip
+    helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", order)
+    helpers.set_switch(monkeypatch, "HSTU_MI355_SHORT", "0")  # (the 64-row query-tile kernel has a grid of its own)
+    helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_PAIR_MAJOR", "0")
+    check(w, monkeypatch)
+    grad_out = torch.randn(w.q.shape[0], 6, 128, generator=g, device=DEV).to(torch.bfloat16)
+    by_level = device_grads(w, grad_out)
+    helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_PAIR_MAJOR", "1")
+    by_pair = device_grads(w, grad_out)
+    for name, a, b in zip(("dq", "dk", "dv", "d_attn_bias"), by_level, by_pair):
+        assert (a is None) == (b is None), name
+        if a is not None:
+            assert torch.equal(a, b), name
+
+
 @pytest.mark.parametrize("rab", [False, True], ids=["workspace", "bias_gradient"])
 def test_ds_hand_over_with_more_keys_than_queries(rab, monkeypatch):
     # the three-launch order on key ranges longer than the query ranges (delta), grouped heads, 16-byte aligned rows

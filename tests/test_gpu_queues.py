@@ -49,6 +49,8 @@ CASES = {
     # context rows and grouped targets with the per-pair order
     "jagged_targets": dict(batch=48, heads=8, heads_k=8, dim=128, lo=64, hi=2048, max_seq_len=2048, num_context=6,
                            max_target=40, target_group_size=3),
+    # all sequences equally long and six items per workgroup: per-pair order all the same
+    "uniform_many": dict(batch=48, heads=8, heads_k=8, dim=128, lo=1024, hi=1024, max_seq_len=1024),
     # context rows with the per-tile order: the first tile of every pair stands ahead of the top tiles
     "uniform_contexts": dict(batch=32, heads=8, heads_k=8, dim=128, lo=1024, hi=1024, max_seq_len=1024, num_context=9),
 }  # fmt: skip
