@@ -50,10 +50,10 @@ INFINITY_CACHE_BYTES = 256 << 20  # MI355X memory-side cache; a working set belo
 # the forward kernel's source at the time).  A figure whose hash no longer matches the source in the tree is stale
 # and is reported as null.
 MEASURED_TRAFFIC = {
-    "C2": (99_300_000, "profiles/hstu_fwd_bf16_d128_C2_trace_and_counters.md", "4472f325a667df50"),
-    "C3": (301_200_000, "profiles/hstu_fwd_bf16_d128_rab_C3_trace_and_counters.md", "c69c75c3656b8c0d"),
-    "C4": (1_498_200_000, "profiles/hstu_fwd_bf16_d128_rab_C4_trace_and_counters.md", "c69c75c3656b8c0d"),
-    "C5": (842_300_000, "profiles/hstu_fwd_f8e4m3_d128_C5_trace_and_counters.md", "c69c75c3656b8c0d"),
+    "C2": (98_400_000, "profiles/hstu_fwd_bf16_d128_C2_trace_and_counters.md", "e5fd7490210191fc"),
+    "C3": (301_300_000, "profiles/hstu_fwd_bf16_d128_rab_C3_trace_and_counters.md", "53b56a23cf722f67"),
+    "C4": (1_498_000_000, "profiles/hstu_fwd_bf16_d128_rab_C4_trace_and_counters.md", "53b56a23cf722f67"),
+    "C5": (846_100_000, "profiles/hstu_fwd_f8e4m3_d128_C5_trace_and_counters.md", "53b56a23cf722f67"),
 }
 _CSRC = os.path.join(_ROOT, "ops-rec_amd", "csrc")
 KERNEL_SOURCE = os.path.join(_CSRC, "hstu_fwd_kernel.hip.h")  # the persistent kernel (and the helpers the others share)
