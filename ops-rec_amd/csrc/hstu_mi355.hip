@@ -362,6 +362,17 @@ const hstu::ShortVariant* short_variant(const Variant* var, const hstu_jagged_fw
         // and longer rows lose (16 x 4 lengths 512..2048 64 -> 84 us, 8 x 8 lengths 1024..2048 80 -> 98)
         return (p->max_seq_len_k <= 1024 && n_blocks <= resident) ? sv : nullptr;
     }
+    // Long lists over more K / V rows than the caches hold go to the persistent kernel's queues, which take the items pair
+    // after pair on one XCD each: this kernel's grid runs level after level, so that every resident workgroup then streams
+    // another pair's keys from memory.  (This kernel -> the queues, 4 heads, lengths 256..1024: batch 128 112 -> 117 us, 256
+    // 237 -> 232, 384 431 -> 370, 512 629 -> 449; 256 x 1024 rows 557 -> 398, 512 x 512 rows 371 -> 288, 1024 x 64..512 rows
+    // 408 -> 335; sequences of a tile or two have nothing to share: 2048 x 16..256 rows 282 -> 299.)
+    const int64_t batch = p->n_offsets - 1;
+    const int64_t items = (p->total_q / hstu::kBlockM + batch / 2) * p->num_heads_q;  // (by the mean length)
+    const int64_t kv_bytes = p->total_k * p->num_heads_k * (p->head_dim_qk + p->head_dim_v) * 2;
+    if (items >= 6 * resident && kv_bytes >= (256LL << 20) && p->total_q >= 256 * batch) {
+        return nullptr;
+    }
     const bool short_keys = p->max_seq_len_k <= 1024;
     const bool one_round = p->max_seq_len_k <= 2048 && n_blocks >= resident && n_blocks <= 2 * resident;
     return (short_keys || one_round) ? sv : nullptr;

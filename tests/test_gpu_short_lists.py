@@ -239,6 +239,10 @@ def test_the_hosts_rule(monkeypatch):
     assert name(max_seq_len=1024).endswith("_short")  # the headline shape: keys up to 1024
     assert name(max_seq_len=1024, dtype=torch.float16).endswith("_short")
     assert name(max_seq_len=1024, batch=512).endswith("_short")  # long list, short keys
+    # long lists over more K / V rows than the caches hold: the queues (pair after pair on one XCD each)
+    assert name(max_seq_len=1024, batch=384, lo=700, hi=700).endswith("_queues")
+    assert name(max_seq_len=1024, batch=128, lo=700, hi=700).endswith("_short")  # under six items per resident workgroup
+    assert name(max_seq_len=256, batch=2048, lo=136, hi=136).endswith("_short")  # sequences of a tile or two share nothing
     assert name(max_seq_len=2048, batch=8).endswith("_short")  # keys up to 2048, one slot per resident workgroup
     assert not name(max_seq_len=2048, batch=32).endswith("_short")  # four per resident workgroup
     assert not name(max_seq_len=2048, batch=2).endswith("_short")  # fewer than workgroups: split items
