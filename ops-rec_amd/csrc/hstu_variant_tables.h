@@ -8,9 +8,9 @@ namespace hstu {
 template <typename Tag, typename OutTag, int D, bool RAB, bool MASK>
 constexpr auto queues_kernel() -> void (*)(const FwdArgs)
 {
-    // (at the slot 256, one workgroup per CU, the queues and the split items were measured level with the plain list:
-    // -5 .. +5 % and -12 .. +16 % over ten shapes)
-    if constexpr (D == 64 || D == 128) {
+    // (at the slot 256, one workgroup per CU: plain list -> queues 32 x 8 heads of 4096 rows 3.12 -> 2.47 ms, 64 x 4 of
+    // 1024..4096 rows 1.43 -> 1.23 ms, 256 x 4 of 256..1024 rows 575 -> 502 us, 32 x 4 of 512..2048 rows 199 -> 188 us)
+    if constexpr (D == 64 || D == 128 || D == 256) {
         return hstu_fwd_kernel<Tag, OutTag, D, RAB, MASK, true>;
     } else {
         return nullptr;
@@ -20,6 +20,7 @@ constexpr auto queues_kernel() -> void (*)(const FwdArgs)
 template <typename Tag, typename OutTag, int D, bool RAB, bool MASK>
 constexpr auto split_kernel() -> void (*)(const FwdArgs)
 {
+    // (at the slot 256 split items were measured level with the plain list: -12 .. +16 % over ten shapes)
     if constexpr (D == 64 || D == 128) {
         return hstu_fwd_kernel<Tag, OutTag, D, RAB, MASK, false, true>;
     } else {

@@ -51,6 +51,9 @@ CASES = {
                            max_target=40, target_group_size=3),
     # all sequences equally long and six items per workgroup: per-pair order all the same
     "uniform_many": dict(batch=48, heads=8, heads_k=8, dim=128, lo=1024, hi=1024, max_seq_len=1024),
+    # the head-dim slot 256 (one workgroup per CU): jagged with a bias, and equally long sequences
+    "jagged_d256_rab": dict(batch=40, heads=4, heads_k=2, dim=256, lo=1, hi=2048, max_seq_len=2048, rab_std=0.2),
+    "uniform_d256": dict(batch=32, heads=8, heads_k=8, dim=256, lo=1024, hi=1024, max_seq_len=1024),
     # context rows with the per-tile order: the first tile of every pair stands ahead of the top tiles
     "uniform_contexts": dict(batch=32, heads=8, heads_k=8, dim=128, lo=1024, hi=1024, max_seq_len=1024, num_context=9),
 }  # fmt: skip
@@ -81,9 +84,10 @@ def test_schedule_does_not_change_results(name, monkeypatch):
     assert torch.equal(run(w), out)  # and the same bits again
 
 
-def test_fp8_long_list_matches_sequences_run_alone(monkeypatch):
+@pytest.mark.parametrize("dim", [128, 256])
+def test_fp8_long_list_matches_sequences_run_alone(dim, monkeypatch):
     helpers.set_switch(monkeypatch, "HSTU_MI355_SPLIT", "0")
-    w = workloads.make("f8", dtype=torch.bfloat16, device=DEV, seed=7, batch=64, heads=8, heads_k=2, dim=128, lo=1,
+    w = workloads.make("f8", dtype=torch.bfloat16, device=DEV, seed=7, batch=64, heads=8, heads_k=2, dim=dim, lo=1,
                        hi=2048, max_seq_len=2048)  # fmt: skip
     (q8, qs), (k8, ks), (v8, vs) = (workloads.quantize_fp8(t) for t in (w.q, w.k, w.v))
     kw = dict(mask_type=0, max_seq_len=w.max_seq_len, silu_scale=w.silu_scale, alpha=w.alpha)
