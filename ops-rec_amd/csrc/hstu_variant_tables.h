@@ -8,9 +8,11 @@ namespace hstu {
 template <typename Tag, typename OutTag, int D, bool RAB, bool MASK>
 constexpr auto queues_kernel() -> void (*)(const FwdArgs)
 {
+    // (at the slot 32, four workgroups per CU and the fewest flops per byte streamed: plain list -> queues 128 x 8 heads of
+    // 4096 rows 2.96 -> 2.19 ms, 512 x 8 of 1024 rows 933 -> 760 us, 1024 x 4 of 256..1024 rows 506 -> 399 us)
     // (at the slot 256, one workgroup per CU: plain list -> queues 32 x 8 heads of 4096 rows 3.12 -> 2.47 ms, 64 x 4 of
     // 1024..4096 rows 1.43 -> 1.23 ms, 256 x 4 of 256..1024 rows 575 -> 502 us, 32 x 4 of 512..2048 rows 199 -> 188 us)
-    if constexpr (D == 64 || D == 128 || D == 256) {
+    if constexpr (D == 32 || D == 64 || D == 128 || D == 256) {
         return hstu_fwd_kernel<Tag, OutTag, D, RAB, MASK, true>;
     } else {
         return nullptr;

@@ -51,6 +51,8 @@ CASES = {
                            max_target=40, target_group_size=3),
     # all sequences equally long and six items per workgroup: per-pair order all the same
     "uniform_many": dict(batch=48, heads=8, heads_k=8, dim=128, lo=1024, hi=1024, max_seq_len=1024),
+    # the head-dim slot 32 (four workgroups per CU)
+    "jagged_d32": dict(batch=64, heads=8, heads_k=4, dim=32, lo=1, hi=2048, max_seq_len=2048),
     # the head-dim slot 256 (one workgroup per CU): jagged with a bias, and equally long sequences
     "jagged_d256_rab": dict(batch=40, heads=4, heads_k=2, dim=256, lo=1, hi=2048, max_seq_len=2048, rab_std=0.2),
     "uniform_d256": dict(batch=32, heads=8, heads_k=8, dim=256, lo=1024, hi=1024, max_seq_len=1024),
