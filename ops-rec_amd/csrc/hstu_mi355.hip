@@ -117,12 +117,14 @@ const Switches& switches()
     std::call_once(g_switches_once, read_switches);
     return g_switches;
 }
-// the largest backward workspace the library asks for, in MiB: 2 GiB unless HSTU_MI355_BWD_WORKSPACE_MB says otherwise
-// (a call whose planes would need more runs on the two-launch order, which needs none)
+// the largest backward workspace the library asks for, in MiB: 16 GiB (of the 288 GB of an MI355X) unless
+// HSTU_MI355_BWD_WORKSPACE_MB says otherwise (a call whose planes would need more runs on the two-launch order, which needs
+// none).  With the 2 GiB this limit used to be, large calls at the head-dim slot 256 paid the two-launch order's seven
+// products: 32 x 8 heads of 4096 rows 15.5 -> 11.0 ms (8.7 GB of planes), 64 x 4 heads of 1024..4096 rows 7.9 -> 4.7 ms.
 int64_t workspace_cap_mb()
 {
     const long long set = switches().bwd_workspace_mb;
-    return set >= 0 ? static_cast<int64_t>(set) : 2048;
+    return set >= 0 ? static_cast<int64_t>(set) : 16384;
 }
 
 

@@ -23,18 +23,21 @@ def set_switch(monkeypatch, name, value):
 
 def poison_workspace(monkeypatch):
     """The backward's workspace is handed out holding NaN in every element, so that a read of something never
-    written shows in the gradients."""
+    written shows in the gradients.  Returns the list to which the sizes asked for are appended."""
     from ops_rec import _ops
 
     plain = _ops._new_workspace
+    asked = []
 
     def poisoned(n_bytes, device):
+        asked.append(n_bytes)
         ws = plain(n_bytes, device)
         if ws is not None:
             ws.fill_(0xFF)
         return ws
 
     monkeypatch.setattr(_ops, "_new_workspace", poisoned)
+    return asked
 
 
 def withhold_workspace(monkeypatch):

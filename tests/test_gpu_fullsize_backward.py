@@ -101,3 +101,25 @@ def test_the_launch_orders_agree(config, monkeypatch):
         for i in (1, 2):
             scale = two[i].float().abs().max().item()
             torch.testing.assert_close(other[i].float(), two[i].float(), atol=1e-2 * scale, rtol=1e-2)
+
+
+def test_planes_beyond_4_gib_agree_with_the_two_launch_order(monkeypatch):
+    """A call whose pair plane passes 4 GiB (64 sequences x 4 heads of 1024 .. 4096 rows at head dim 256: 5.5 GB, within the
+    library's limit of 16 GiB): offsets into the plane are 64-bit sums of 32-bit parts per sequence.  The workspace is
+    filled with NaN beforehand; dq must match the two-launch order bit for bit, dk and dv to rounding."""
+    helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_WORKSPACE_MB", None)
+    w = workloads.make("big", dtype=torch.bfloat16, device=DEV, seed=21, batch=64, heads=4, dim=256, lo=1024, hi=4096,
+                       max_seq_len=4096, std=0.5)  # fmt: skip
+    g = torch.Generator(device=DEV).manual_seed(3)
+    grad_out = torch.randn(w.q.shape, generator=g, device=DEV).to(torch.bfloat16)
+    helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", "0")
+    two = backward(w, grad_out)
+    asked = helpers.poison_workspace(monkeypatch)
+    helpers.set_switch(monkeypatch, "HSTU_MI355_BWD_HANDOFF", "2")
+    planes = backward(w, grad_out)
+    assert asked and asked[-1] > (4 << 30), asked
+    assert torch.equal(two[0], planes[0])
+    for i in (1, 2):
+        assert torch.isfinite(planes[i].float()).all()
+        scale = two[i].float().abs().max().item()
+        torch.testing.assert_close(planes[i].float(), two[i].float(), atol=1e-2 * scale, rtol=1e-2)
