@@ -184,7 +184,7 @@ HSTU_API uint64_t hstu_jagged_fwd_noalloc_max_workspace(void);
  * elements of the input type; dS and P together in a workspace of one 128-byte line per head, query row of the batch
  * and 32-key block (only the blocks at or below the diagonal for a causal mask over equal query and key offsets
  * without context rows; otherwise ceil(max_seq_len_k / 32) | 1 lines per row).  hstu_jagged_bwd_workspace_size asks for the workspace of the order it estimates to be the
- * fastest (at most 16 GiB, or HSTU_MI355_BWD_WORKSPACE_MB in the environment; with an attn_bias, a custom mask or an
+ * fastest (at most 2 GiB -- 16 GiB at head dims above 128, where it saves a good part of the call -- or HSTU_MI355_BWD_WORKSPACE_MB in the environment; with an attn_bias, a custom mask or an
  * attn_bias gradient, or for the [batch, ...] plane of dS alone, max_seq_len_k must be a multiple of 4 -- rows of such
  * tensors are read and written in pieces of 8 keys, one 16-byte access when max_seq_len_k is a multiple of 8, two
  * 8-byte ones otherwise -- while the workspace for dS and P together has its own layout; fp32

@@ -117,14 +117,16 @@ const Switches& switches()
     std::call_once(g_switches_once, read_switches);
     return g_switches;
 }
-// the largest backward workspace the library asks for, in MiB: 16 GiB (of the 288 GB of an MI355X) unless
-// HSTU_MI355_BWD_WORKSPACE_MB says otherwise (a call whose planes would need more runs on the two-launch order, which needs
-// none).  With the 2 GiB this limit used to be, large calls at the head-dim slot 256 paid the two-launch order's seven
-// products: 32 x 8 heads of 4096 rows 15.5 -> 11.0 ms (8.7 GB of planes), 64 x 4 heads of 1024..4096 rows 7.9 -> 4.7 ms.
-int64_t workspace_cap_mb()
+// The largest backward workspace the library asks for, in MiB.  HSTU_MI355_BWD_WORKSPACE_MB sets it for every call.
+// Otherwise 2 GiB -- a training step has better uses for its memory than the last few per cent of this operator, and a
+// call whose planes would need more runs on the two-launch order, which needs none -- except where more buys a good part
+// of the call (`large`: 16-bit inputs at head dims above 128, where a product is dearest; plan_bwd takes more than the
+// 2 GiB only for an estimated tenth of the time): 16 GiB of an MI355X's 288 GB.  With 2 GiB everywhere, 32 x 8 heads of
+// 4096 rows at d 256 took 15.5 ms, 11.0 ms with their 8.7 GB of planes; 64 x 4 heads of 1024..4096 rows 7.9 -> 4.7 ms.
+int64_t workspace_cap_mb(bool large = false)
 {
     const long long set = switches().bwd_workspace_mb;
-    return set >= 0 ? static_cast<int64_t>(set) : 16384;
+    return set >= 0 ? static_cast<int64_t>(set) : (large ? 16384 : 2048);
 }
 
 
@@ -877,7 +879,9 @@ static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
     }
     const bool bias_grad = p->grad_attn_bias != nullptr;
     const PairPlane pp = pair_plane(f);
-    const int64_t cap = workspace_cap_mb() * (1LL << 20);
+    const int64_t dmax = f->head_dim_qk > f->head_dim_v ? f->head_dim_qk : f->head_dim_v;
+    const int64_t cap_small = workspace_cap_mb() * (1LL << 20);
+    const int64_t cap = workspace_cap_mb(dmax > 128) * (1LL << 20);
     // with an attn_bias gradient dS goes through the gradient itself in the three-launch order: no workspace
     const int64_t ds_plane = bias_grad ? 0 : batch * f->num_heads_q * f->max_seq_len_q * f->max_seq_len_k * 2;
     const bool three_fits = rows8 && ds_plane <= cap;
@@ -891,14 +895,23 @@ static BwdPlan plan_bwd(const hstu_jagged_bwd_params* p, const BwdVariant* var)
         return three_fits ? three : two;
     }
     const BwdCost cost = estimate_bwd(f, bias_grad);
-    BwdPlan best = two;
-    double best_us = cost.two;
-    if (three_fits && cost.three < best_us) {
-        best = three;
-        best_us = cost.three;
-    }
-    if (planes_fit && cost.planes < best_us) {
-        best = planes;
+    // the best order within the small limit, then the best of all: more than the small limit only for a tenth of the time
+    BwdPlan best = two, best_small = two;
+    double best_us = cost.two, best_small_us = cost.two;
+    auto consider = [&](bool fits, const BwdPlan& plan, double us) {
+        if (fits && us < best_us) {
+            best = plan;
+            best_us = us;
+        }
+        if (fits && static_cast<int64_t>(plan.workspace_bytes) <= cap_small && us < best_small_us) {
+            best_small = plan;
+            best_small_us = us;
+        }
+    };
+    consider(three_fits, three, cost.three);
+    consider(planes_fit, planes, cost.planes);
+    if (static_cast<int64_t>(best.workspace_bytes) > cap_small && best_us > 0.9 * best_small_us) {
+        return best_small;
     }
     return best;
 }
@@ -1028,7 +1041,8 @@ static WindowPlan plan_windows(const hstu_jagged_bwd_params* p)
     const int64_t n_blk = (f->max_seq_len_k + 31) / 32;
     w.partial_bytes = static_cast<uint64_t>(f->num_heads_q * f->total_q * n_blk * 256);
     w.workspace_bytes = static_cast<uint64_t>(w.pair.bytes) + w.partial_bytes;
-    if (!w.pair.fits_32 || w.workspace_bytes > static_cast<uint64_t>(workspace_cap_mb()) * (1ULL << 20)) {
+    // (without the workspace these head dims run on the generic kernels: the larger limit)
+    if (!w.pair.fits_32 || w.workspace_bytes > static_cast<uint64_t>(workspace_cap_mb(true)) * (1ULL << 20)) {
         return w;
     }
     const auto* table = f->dtype == HSTU_DT_BF16 ? hstu::bwd_variants_bf16() : hstu::bwd_variants_f16();
