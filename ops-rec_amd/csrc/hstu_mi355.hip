@@ -1219,7 +1219,10 @@ HSTU_API int hstu_jagged_bwd(const hstu_jagged_bwd_params* p, void* workspace, u
         const int64_t dmax = f->head_dim_qk > f->head_dim_v ? f->head_dim_qk : f->head_dim_v;
         // (the slot 256: jagged batches only -- 64 x 4 heads of 1024..4096 rows 8.87 -> 7.91 ms, 256 x 4 of 256..1024 rows 1.93 -> 1.68 ms)
         const bool jagged = 10 * f->total_q <= 7 * (f->n_offsets - 1) * f->max_seq_len_q;
-        const bool long_launch = (dmax <= 128 || jagged) && streamed >= (512LL << 20) && tiles >= 16LL * cus;
+        // (jagged batches from half of that on: 16 x 8 heads of 1024..4096 rows 1.35 -> 1.19 ms, 64 x 4 of 512..2048 rows 813 -> 774 us;
+        // equally long sequences lose there: 32 x 8 of 1024 rows 436 -> 512 us)
+        const bool long_launch = ((dmax <= 128 || jagged) && streamed >= (512LL << 20) && tiles >= 16LL * cus) ||
+                                 (dmax <= 128 && jagged && streamed >= (256LL << 20) && tiles >= 8LL * cus);
         const int forced = switches().bwd_pair_major;
         a.pair_major = forced >= 0 ? forced : (long_launch ? 1 : 0);
     }
