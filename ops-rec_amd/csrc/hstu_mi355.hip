@@ -323,7 +323,7 @@ const hstu::ShortVariant* one_item_variant(const Variant* var, const hstu_jagged
 // short kernel's narrower wavefronts finish in about half the time; on longer lists the persistent kernel's
 // steady-state rate wins.  HSTU_MI355_SHORT in the environment overrides the rule: 0 = never, 1 = whenever the
 // kernel can take the call.
-const hstu::ShortVariant* short_variant(const Variant* var, const hstu_jagged_fwd_params* p)
+const hstu::ShortVariant* short_variant(const Variant* var, const hstu_jagged_fwd_params* p, bool have_counters = true)
 {
     if ((p->dtype != HSTU_DT_BF16 && p->dtype != HSTU_DT_FP16) || p->mask_type == HSTU_MASK_CUSTOM || var->d_pad != 128 ||
         var->persistent_wgs_per_cu <= 0 || var->kernel_queues == nullptr) {
@@ -374,7 +374,8 @@ const hstu::ShortVariant* short_variant(const Variant* var, const hstu_jagged_fw
     const int64_t batch = p->n_offsets - 1;
     const int64_t items = (p->total_q / hstu::kBlockM + batch / 2) * p->num_heads_q;  // (by the mean length)
     const int64_t kv_bytes = p->total_k * p->num_heads_k * (p->head_dim_qk + p->head_dim_v) * 2;
-    if (items >= 6 * resident && kv_bytes >= (256LL << 20) && p->total_q >= 256 * batch) {
+    // (a caller that brings no room for the queues' counters keeps this kernel: the plain list runs level after level too)
+    if (have_counters && items >= 6 * resident && kv_bytes >= (256LL << 20) && p->total_q >= 256 * batch) {
         return nullptr;
     }
     const bool short_keys = p->max_seq_len_k <= 1024;
@@ -1472,7 +1473,8 @@ int launch_forward(const hstu_jagged_fwd_params* p, const hstu_paged_fwd_params*
         }
         return HSTU_OK;
     }
-    if (const hstu::ShortVariant* const sv = (paged == nullptr) ? short_variant(var, p) : nullptr) {
+    if (const hstu::ShortVariant* const sv =
+            (paged == nullptr) ? short_variant(var, p, usable_workspace(workspace, workspace_bytes, kCounterBytes)) : nullptr) {
         // one workgroup per (query tile, K/V pair padded to a multiple of 8, query head of the pair) slot
         const int64_t pairs_pad = (static_cast<int64_t>(a.n_batch) * a.n_heads_k + 7) & ~static_cast<int64_t>(7);
         const int64_t slots = static_cast<int64_t>(a.n_qtiles) * pairs_pad * a.head_ratio;
